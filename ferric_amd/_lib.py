@@ -1,0 +1,110 @@
+"""Loads libferric_hip.so (the C-ABI library of include/ferric_hip.h) through ctypes.
+
+There is no CPU fallback: if the library has not been built, or no gfx950 device can be
+initialised, every entry point of this package raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "libferric_hip.so")
+
+OK, ERR_UNSUPPORTED_TYPE, ERR_SHAPE, ERR_HIP, ERR_ARG = 0, -1, -2, -3, -4
+
+_vp = C.c_void_p
+_sz = C.c_size_t
+_u32 = C.c_uint32
+
+# name -> (restype, argtypes); exactly the symbols include/ferric_hip.h declares
+SYMBOLS = {
+    "fhip_init": (C.c_int, [C.c_int]),
+    "fhip_last_error": (C.c_char_p, []),
+    "fhip_device_cus": (C.c_int, []),
+    "fhip_type_size": (_sz, [_u32, _sz]),
+    "fhip_block_bytes": (C.c_int, [_u32, C.POINTER(_sz), C.POINTER(_sz)]),
+    "fhip_malloc": (C.c_int, [C.POINTER(_vp), _sz]),
+    "fhip_free": (C.c_int, [_vp]),
+    "fhip_memcpy_h2d": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fhip_memcpy_d2h": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fhip_memcpy_d2d": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fhip_memset": (C.c_int, [_vp, C.c_int, _sz, _vp]),
+    "fhip_stream_create": (C.c_int, [C.POINTER(_vp)]),
+    "fhip_stream_destroy": (C.c_int, [_vp]),
+    "fhip_stream_sync": (C.c_int, [_vp]),
+    "fhip_event_create": (C.c_int, [C.POINTER(_vp)]),
+    "fhip_event_destroy": (C.c_int, [_vp]),
+    "fhip_event_record": (C.c_int, [_vp, _vp]),
+    "fhip_event_sync": (C.c_int, [_vp]),
+    "fhip_event_elapsed_ms": (C.c_int, [_vp, _vp, C.POINTER(C.c_float)]),
+    "fhip_graph_capture_begin": (C.c_int, [_vp]),
+    "fhip_graph_capture_end": (C.c_int, [_vp, C.POINTER(_vp)]),
+    "fhip_graph_launch": (C.c_int, [_vp, _vp]),
+    "fhip_graph_destroy": (C.c_int, [_vp]),
+    "fhip_weight_create": (C.c_int, [_u32, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "fhip_weight_wrap_device": (C.c_int, [_u32, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "fhip_weight_destroy": (None, [_vp]),
+    "fhip_weight_rows": (_sz, [_vp]),
+    "fhip_weight_cols": (_sz, [_vp]),
+    "fhip_weight_nbytes": (_sz, [_vp]),
+    "fhip_weight_type": (_u32, [_vp]),
+    "fhip_f16_to_f32": (C.c_int, [_vp, _sz, _vp, _vp]),
+    "fhip_dequant_rows": (C.c_int, [_vp, _sz, _sz, _vp, _vp]),
+    "fhip_deq_raw": (C.c_int, [_vp, _sz, _sz, _u32, _vp, C.POINTER(_sz)]),
+    "fhip_matmul_q": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
+    "fhip_matmul_q_swiglu": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
+    "fhip_swiglu": (C.c_int, [_vp, _sz, _sz, _vp, _vp]),
+    "fhip_ffn": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _vp, _vp]),
+    "fhip_gemm_q_bf16": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
+    "fhip_matvec_q8_0_host": (C.c_int, [_vp, _vp, _sz, _sz, _sz, _vp]),
+}
+
+_lib = None
+_inited = False
+
+
+class FerricHipError(RuntimeError):
+    """A HIP runtime failure or an unusable argument reported by the library."""
+
+
+def load():
+    """dlopen the library and bind every declared symbol (no device is touched)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(SO_PATH):
+            raise ImportError(f"{SO_PATH} is missing: build it with `python -m ferric_amd.build` (needs hipcc); "
+                              "there is no CPU fallback")
+        lib = C.CDLL(SO_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(lib, name)  # AttributeError if the library does not export it
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def last_error():
+    return load().fhip_last_error().decode("utf-8", "replace")
+
+
+def check(rc):
+    """Map a return code to the exception the reference's behaviour calls for:
+    unsupported type -> ValueError (reference: Err(String)); shape violation -> AssertionError
+    (reference: assert!/assert_eq! panic); anything else -> FerricHipError."""
+    if rc == OK:
+        return
+    msg = last_error()
+    if rc == ERR_UNSUPPORTED_TYPE:
+        raise ValueError(msg)
+    if rc == ERR_SHAPE:
+        raise AssertionError(msg)
+    raise FerricHipError(f"[{rc}] {msg}")
+
+
+def init(device=0):
+    """Initialise the device once per process; raises if there is no usable gfx950 GPU."""
+    global _inited
+    lib = load()
+    if not _inited:
+        check(lib.fhip_init(device))
+        _inited = True
+    return lib

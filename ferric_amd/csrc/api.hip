@@ -1,0 +1,368 @@
+// The extern "C" surface of libferric_hip (declared in include/ferric_hip.h): argument checks with
+// the reference's error behaviour, weight handles, and thin dispatch into the kernel launchers.
+#include "common.hpp"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace {
+
+thread_local char g_err[512] = "";
+int g_device = -1;
+int g_cus = 0;
+
+bool block_info(uint32_t ty, size_t& vals, size_t& bytes) {
+    switch (ty) {
+        case FHIP_Q8_0: vals = 32; bytes = 34; return true;
+        case FHIP_Q4_K: vals = 256; bytes = 144; return true;
+        case FHIP_Q6_K: vals = 256; bytes = 210; return true;
+        default: return false;
+    }
+}
+
+const char* type_name(uint32_t ty) { return ty == FHIP_Q8_0 ? "Q8_0" : ty == FHIP_Q4_K ? "Q4_K" : ty == FHIP_Q6_K ? "Q6_K" : "?"; }
+
+int need_init() {
+    if (g_device < 0) return fhip::set_error(FHIP_ERR_ARG, "fhip_init has not been called");
+    return FHIP_OK;
+}
+
+// Shape checks of the per-format constructors: crates/ferric-tensor/src/dtype.rs:1271-1272 (Q8_0),
+// :1389-1390 (Q4_K), :1148-1149 (Q6_K) -- `assert_eq!(cols % blk, 0)` and exact byte length.
+int make_weight(uint32_t ty, size_t nbytes, size_t rows, size_t cols, fhip_weight& w) {
+    size_t vals, bytes;
+    if (!block_info(ty, vals, bytes)) return fhip::set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", ty);
+    if (cols % vals != 0) return fhip::set_error(FHIP_ERR_SHAPE, "%s cols must be a multiple of %zu", type_name(ty), vals);
+    size_t row_bytes = cols / vals * bytes;
+    if (nbytes != rows * row_bytes) return fhip::set_error(FHIP_ERR_SHAPE, "unexpected %s byte length", type_name(ty));
+    if (rows > 0x7FFFFFFFull || cols > 0x7FFFFFFFull) return fhip::set_error(FHIP_ERR_SHAPE, "weight dimensions exceed 2^31");
+    w.type = ty; w.rows = rows; w.cols = cols; w.row_bytes = row_bytes; w.nbytes = nbytes; w.d_raw = nullptr; w.owns = false;
+    return FHIP_OK;
+}
+
+}  // namespace
+
+namespace fhip {
+
+int set_error(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return FHIP_OK;
+    return set_error(FHIP_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int device_cus() { return g_cus; }
+
+}  // namespace fhip
+
+using fhip::check_hip;
+using fhip::set_error;
+
+extern "C" {
+
+int fhip_init(int device) {
+    int n = 0;
+    int rc = check_hip(hipGetDeviceCount(&n), "hipGetDeviceCount");
+    if (rc) return rc;
+    if (device < 0 || device >= n) return set_error(FHIP_ERR_ARG, "device %d out of range (%d visible)", device, n);
+    if ((rc = check_hip(hipSetDevice(device), "hipSetDevice"))) return rc;
+    hipDeviceProp_t prop;
+    if ((rc = check_hip(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties"))) return rc;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return set_error(FHIP_ERR_HIP, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    g_cus = prop.multiProcessorCount;
+    g_device = device;
+    return FHIP_OK;
+}
+
+const char* fhip_last_error(void) { return g_err; }
+int fhip_device_cus(void) { return g_cus; }
+
+size_t fhip_type_size(uint32_t ty, size_t n) {
+    size_t vals, bytes;
+    if (!block_info(ty, vals, bytes)) { set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", ty); return 0; }
+    return n / vals * bytes;
+}
+
+int fhip_block_bytes(uint32_t ty, size_t* values, size_t* bytes) {
+    size_t v, b;
+    if (!values || !bytes) return set_error(FHIP_ERR_ARG, "fhip_block_bytes: NULL output");
+    if (!block_info(ty, v, b)) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", ty);
+    *values = v; *bytes = b;
+    return FHIP_OK;
+}
+
+// ---- plumbing -------------------------------------------------------------------------------
+
+int fhip_malloc(void** d_ptr, size_t nbytes) {
+    if (!d_ptr) return set_error(FHIP_ERR_ARG, "fhip_malloc: NULL output");
+    int rc = need_init();
+    if (rc) return rc;
+    *d_ptr = nullptr;
+    return check_hip(hipMalloc(d_ptr, nbytes ? nbytes : 1), "hipMalloc");
+}
+int fhip_free(void* d_ptr) { return d_ptr ? check_hip(hipFree(d_ptr), "hipFree") : FHIP_OK; }
+int fhip_memcpy_h2d(void* d, const void* h, size_t n, void* s) {
+    if (n == 0) return FHIP_OK;
+    if (!d || !h) return set_error(FHIP_ERR_ARG, "fhip_memcpy_h2d: NULL pointer");
+    return check_hip(hipMemcpyAsync(d, h, n, hipMemcpyHostToDevice, (hipStream_t)s), "hipMemcpyAsync H2D");
+}
+int fhip_memcpy_d2h(void* h, const void* d, size_t n, void* s) {
+    if (n == 0) return FHIP_OK;
+    if (!d || !h) return set_error(FHIP_ERR_ARG, "fhip_memcpy_d2h: NULL pointer");
+    int rc = check_hip(hipMemcpyAsync(h, d, n, hipMemcpyDeviceToHost, (hipStream_t)s), "hipMemcpyAsync D2H");
+    if (rc) return rc;
+    return check_hip(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize");
+}
+int fhip_memcpy_d2d(void* dst, const void* src, size_t n, void* s) {
+    if (n == 0) return FHIP_OK;
+    if (!dst || !src) return set_error(FHIP_ERR_ARG, "fhip_memcpy_d2d: NULL pointer");
+    return check_hip(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, (hipStream_t)s), "hipMemcpyAsync D2D");
+}
+int fhip_memset(void* d, int byte, size_t n, void* s) {
+    if (n == 0) return FHIP_OK;
+    if (!d) return set_error(FHIP_ERR_ARG, "fhip_memset: NULL pointer");
+    return check_hip(hipMemsetAsync(d, byte, n, (hipStream_t)s), "hipMemsetAsync");
+}
+int fhip_stream_create(void** s) {
+    if (!s) return set_error(FHIP_ERR_ARG, "fhip_stream_create: NULL output");
+    int rc = need_init();
+    if (rc) return rc;
+    hipStream_t st;
+    rc = check_hip(hipStreamCreateWithFlags(&st, hipStreamNonBlocking), "hipStreamCreate");
+    *s = rc ? nullptr : (void*)st;
+    return rc;
+}
+int fhip_stream_destroy(void* s) { return s ? check_hip(hipStreamDestroy((hipStream_t)s), "hipStreamDestroy") : FHIP_OK; }
+int fhip_stream_sync(void* s) { return check_hip(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize"); }
+int fhip_event_create(void** e) {
+    if (!e) return set_error(FHIP_ERR_ARG, "fhip_event_create: NULL output");
+    int rc = need_init();
+    if (rc) return rc;
+    hipEvent_t ev;
+    rc = check_hip(hipEventCreate(&ev), "hipEventCreate");
+    *e = rc ? nullptr : (void*)ev;
+    return rc;
+}
+int fhip_event_destroy(void* e) { return e ? check_hip(hipEventDestroy((hipEvent_t)e), "hipEventDestroy") : FHIP_OK; }
+int fhip_event_record(void* e, void* s) { return check_hip(hipEventRecord((hipEvent_t)e, (hipStream_t)s), "hipEventRecord"); }
+int fhip_event_sync(void* e) { return check_hip(hipEventSynchronize((hipEvent_t)e), "hipEventSynchronize"); }
+int fhip_event_elapsed_ms(void* a, void* b, float* ms) {
+    if (!ms) return set_error(FHIP_ERR_ARG, "fhip_event_elapsed_ms: NULL output");
+    return check_hip(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b), "hipEventElapsedTime");
+}
+
+int fhip_graph_capture_begin(void* s) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!s) return set_error(FHIP_ERR_ARG, "fhip_graph_capture_begin: needs a stream from fhip_stream_create");
+    return check_hip(hipStreamBeginCapture((hipStream_t)s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+}
+int fhip_graph_capture_end(void* s, void** graph_exec) {
+    if (!s || !graph_exec) return set_error(FHIP_ERR_ARG, "fhip_graph_capture_end: NULL argument");
+    *graph_exec = nullptr;
+    hipGraph_t g = nullptr;
+    int rc = check_hip(hipStreamEndCapture((hipStream_t)s, &g), "hipStreamEndCapture");
+    if (rc) return rc;
+    hipGraphExec_t ge = nullptr;
+    rc = check_hip(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0), "hipGraphInstantiate");
+    (void)hipGraphDestroy(g);
+    if (!rc) *graph_exec = (void*)ge;
+    return rc;
+}
+int fhip_graph_launch(void* ge, void* s) {
+    if (!ge) return set_error(FHIP_ERR_ARG, "fhip_graph_launch: NULL graph");
+    return check_hip(hipGraphLaunch((hipGraphExec_t)ge, (hipStream_t)s), "hipGraphLaunch");
+}
+int fhip_graph_destroy(void* ge) { return ge ? check_hip(hipGraphExecDestroy((hipGraphExec_t)ge), "hipGraphExecDestroy") : FHIP_OK; }
+
+// ---- weights --------------------------------------------------------------------------------
+
+int fhip_weight_create(uint32_t ty, const uint8_t* h_raw, size_t nbytes, size_t rows, size_t cols, fhip_weight** out) {
+    if (!out) return set_error(FHIP_ERR_ARG, "fhip_weight_create: NULL output");
+    *out = nullptr;
+    int rc = need_init();
+    if (rc) return rc;
+    fhip_weight w;
+    if ((rc = make_weight(ty, nbytes, rows, cols, w))) return rc;
+    if (nbytes && !h_raw) return set_error(FHIP_ERR_ARG, "fhip_weight_create: NULL bytes");
+    void* d = nullptr;
+    // 256 bytes of slack past the stream: wide loads of lanes that are masked out stay inside the allocation.
+    if ((rc = check_hip(hipMalloc(&d, nbytes + 256), "hipMalloc(weight)"))) return rc;
+    if (nbytes && (rc = check_hip(hipMemcpy(d, h_raw, nbytes, hipMemcpyHostToDevice), "hipMemcpy(weight)"))) { (void)hipFree(d); return rc; }
+    if ((rc = check_hip(hipMemset((uint8_t*)d + nbytes, 0, 256), "hipMemset(weight tail)"))) { (void)hipFree(d); return rc; }
+    w.d_raw = (const uint8_t*)d;
+    w.owns = true;
+    *out = new fhip_weight(w);
+    return FHIP_OK;
+}
+
+int fhip_weight_wrap_device(uint32_t ty, const uint8_t* d_raw, size_t nbytes, size_t rows, size_t cols, fhip_weight** out) {
+    if (!out) return set_error(FHIP_ERR_ARG, "fhip_weight_wrap_device: NULL output");
+    *out = nullptr;
+    int rc = need_init();
+    if (rc) return rc;
+    fhip_weight w;
+    if ((rc = make_weight(ty, nbytes, rows, cols, w))) return rc;
+    if (nbytes && !d_raw) return set_error(FHIP_ERR_ARG, "fhip_weight_wrap_device: NULL bytes");
+    if (((uintptr_t)d_raw & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_weight_wrap_device: bytes must be 16-byte aligned");
+    w.d_raw = d_raw;
+    w.owns = false;
+    *out = new fhip_weight(w);
+    return FHIP_OK;
+}
+
+void fhip_weight_destroy(fhip_weight* w) {
+    if (!w) return;
+    if (w->owns && w->d_raw) (void)hipFree((void*)w->d_raw);
+    delete w;
+}
+
+size_t fhip_weight_rows(const fhip_weight* w) { return w ? w->rows : 0; }
+size_t fhip_weight_cols(const fhip_weight* w) { return w ? w->cols : 0; }
+size_t fhip_weight_nbytes(const fhip_weight* w) { return w ? w->nbytes : 0; }
+uint32_t fhip_weight_type(const fhip_weight* w) { return w ? w->type : 0; }
+
+// ---- unpackers ------------------------------------------------------------------------------
+
+int fhip_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (n && (!d_bits || !d_out)) return set_error(FHIP_ERR_ARG, "fhip_f16_to_f32: NULL pointer");
+    return fhip::launch_f16_to_f32(d_bits, n, d_out, (hipStream_t)stream);
+}
+
+int fhip_dequant_rows(const fhip_weight* w, size_t row0, size_t nrows, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!w) return set_error(FHIP_ERR_ARG, "fhip_dequant_rows: NULL weight");
+    if (row0 > w->rows || nrows > w->rows - row0) return set_error(FHIP_ERR_SHAPE, "fhip_dequant_rows: rows [%zu, %zu) outside [0, %zu)", row0, row0 + nrows, w->rows);
+    if (nrows == 0 || w->cols == 0) return FHIP_OK;
+    if (!d_out) return set_error(FHIP_ERR_ARG, "fhip_dequant_rows: NULL output");
+    size_t vals, bytes;
+    block_info(w->type, vals, bytes);
+    return fhip::launch_dequant(w->type, w->d_raw + row0 * w->row_bytes, nrows * (w->cols / vals), d_out, (hipStream_t)stream);
+}
+
+int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ty, float* h_out, size_t* n_written) {
+    int rc = need_init();
+    if (rc) return rc;
+    size_t vals, bytes;
+    if (!block_info(ty, vals, bytes)) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", ty);
+    if (n && !h_out) return set_error(FHIP_ERR_ARG, "fhip_deq_raw: NULL output");
+    size_t nb = n / vals;
+    if (nbytes / bytes < nb) nb = nbytes / bytes;  // chunks_exact(..).take(n / blk)
+    if (nb && !h_raw) return set_error(FHIP_ERR_ARG, "fhip_deq_raw: NULL bytes");
+    // The K-quant dequantizers pre-size the output to n zeros (lib.rs:794, :722); Q8_0 pushes whole
+    // blocks only and so returns a shorter vector (lib.rs:609-614).
+    size_t produced = ty == FHIP_Q8_0 ? nb * vals : n;
+    if (n_written) *n_written = produced;
+    if (nb) {
+        void *d_in = nullptr, *d_out = nullptr;
+        if ((rc = check_hip(hipMalloc(&d_in, nb * bytes), "hipMalloc"))) return rc;
+        if ((rc = check_hip(hipMalloc(&d_out, nb * vals * sizeof(float)), "hipMalloc"))) { (void)hipFree(d_in); return rc; }
+        rc = check_hip(hipMemcpy(d_in, h_raw, nb * bytes, hipMemcpyHostToDevice), "hipMemcpy H2D");
+        if (!rc) rc = fhip::launch_dequant(ty, (const uint8_t*)d_in, nb, (float*)d_out, nullptr);
+        if (!rc) rc = check_hip(hipMemcpy(h_out, d_out, nb * vals * sizeof(float), hipMemcpyDeviceToHost), "hipMemcpy D2H");
+        (void)hipFree(d_in);
+        (void)hipFree(d_out);
+        if (rc) return rc;
+    }
+    for (size_t i = nb * vals; i < produced; i++) h_out[i] = 0.0f;
+    return FHIP_OK;
+}
+
+// ---- matmuls --------------------------------------------------------------------------------
+
+int fhip_matmul_q(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!w) return set_error(FHIP_ERR_ARG, "fhip_matmul_q: NULL weight");
+    if (rows_x == 0 || w->rows == 0) return FHIP_OK;
+    if (!d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_matmul_q: NULL pointer");
+    if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q: x must be 16-byte aligned");
+    return fhip::launch_gemv(w, d_x, rows_x, d_y, 0, (hipStream_t)stream);
+}
+
+int fhip_matmul_q_swiglu(const fhip_weight* gu, const float* d_x, size_t rows_x, float* d_y, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!gu) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu: NULL weight");
+    if (gu->type == FHIP_Q8_0) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "try_matmul_swiglu: no fused kernel for Q8_0");
+    if (gu->rows % 2 != 0) return set_error(FHIP_ERR_SHAPE, "matmul_swiglu: gate_up rows must be even");
+    if (rows_x == 0 || gu->rows == 0) return FHIP_OK;
+    if (!d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu: NULL pointer");
+    if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu: x must be 16-byte aligned");
+    return fhip::launch_gemv(gu, d_x, rows_x, d_y, gu->rows / 2, (hipStream_t)stream);
+}
+
+int fhip_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (t * d == 0) return FHIP_OK;
+    if (!d_gu || !d_out) return set_error(FHIP_ERR_ARG, "fhip_swiglu: NULL pointer");
+    return fhip::launch_swiglu(d_gu, t, d, d_out, (hipStream_t)stream);
+}
+
+int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y, float* d_ws, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!gu || !down) return set_error(FHIP_ERR_ARG, "fhip_ffn: NULL weight");
+    if (gu->rows % 2 != 0) return set_error(FHIP_ERR_SHAPE, "ffn: gate_up rows must be even");
+    size_t n_ff = gu->rows / 2;
+    // crates/ferric-tensor/src/dtype.rs:979-981: down in dim must equal n_ff, down out dim is the model width.
+    if (down->cols != n_ff) return set_error(FHIP_ERR_SHAPE, "down in dim must equal n_ff");
+    if (rows_x == 0) return FHIP_OK;
+    if (!d_x || !d_y || !d_ws) return set_error(FHIP_ERR_ARG, "fhip_ffn: NULL pointer");
+    if (gu->type == FHIP_Q8_0) {
+        // no fused gate/up kernel for this format: matmul_q then swiglu, as the reference's callers
+        // do when try_matmul_swiglu returns None (crates/ferric-llama/src/qwen3.rs:219-227). The
+        // [rows_x, 2 n_ff] intermediate then also lives in d_ws, which this path needs 3x larger.
+        return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "fhip_ffn: gate_up must be Q4_K or Q6_K");
+    }
+    if ((rc = fhip::launch_gemv(gu, d_x, rows_x, d_ws, n_ff, (hipStream_t)stream))) return rc;
+    return fhip::launch_gemv(down, d_ws, rows_x, d_y, 0, (hipStream_t)stream);
+}
+
+int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!w) return set_error(FHIP_ERR_ARG, "fhip_gemm_q_bf16: NULL weight");
+    if (t == 0 || w->rows == 0) return FHIP_OK;
+    if (!d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_gemm_q_bf16: NULL pointer");
+    return fhip::launch_gemm_bf16(w, d_x, t, d_y, (hipStream_t)stream);
+}
+
+int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, size_t rows, size_t cols, float* h_y) {
+    int rc = need_init();
+    if (rc) return rc;
+    // asserts of crates/ferric-tensor/src/cpu_simd.rs:80-83
+    if (cols % 32 != 0) return set_error(FHIP_ERR_SHAPE, "Q8_0 cols must be a multiple of 32");
+    if (w_len != rows * (cols / 32) * 34) return set_error(FHIP_ERR_SHAPE, "unexpected Q8_0 byte length");
+    if (rows == 0) return FHIP_OK;
+    if (!h_x || !h_w || !h_y) return set_error(FHIP_ERR_ARG, "fhip_matvec_q8_0_host: NULL pointer");
+    fhip_weight* w = nullptr;
+    if ((rc = fhip_weight_create(FHIP_Q8_0, h_w, w_len, rows, cols, &w))) return rc;
+    void *d_x = nullptr, *d_y = nullptr;
+    rc = check_hip(hipMalloc(&d_x, (cols ? cols : 1) * sizeof(float)), "hipMalloc");
+    if (!rc) rc = check_hip(hipMalloc(&d_y, rows * sizeof(float)), "hipMalloc");
+    if (!rc && cols) rc = check_hip(hipMemcpy(d_x, h_x, cols * sizeof(float), hipMemcpyHostToDevice), "hipMemcpy H2D");
+    if (!rc) {
+        if (cols == 0) rc = check_hip(hipMemset(d_y, 0, rows * sizeof(float)), "hipMemset");
+        else rc = fhip::launch_gemv(w, (const float*)d_x, 1, (float*)d_y, 0, nullptr);
+    }
+    if (!rc) rc = check_hip(hipMemcpy(h_y, d_y, rows * sizeof(float), hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    if (d_x) (void)hipFree(d_x);
+    if (d_y) (void)hipFree(d_y);
+    fhip_weight_destroy(w);
+    return rc;
+}
+
+}  // extern "C"

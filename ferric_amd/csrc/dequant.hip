@@ -1,0 +1,135 @@
+// Bit-exact block unpackers for Q8_0 / Q4_K / Q6_K on gfx950.
+//
+// The reference CPU dequantizers round every f32 operation separately (Rust never fuses a*b+c):
+//   Q8_0  y = f32(q) * d                       crates/ferric-gguf/src/lib.rs:608-615
+//   Q4_K  y = (d*sc)*q - (dmin*m)              crates/ferric-gguf/src/lib.rs:793-825
+//   Q6_K  y = (d*sc)*q                         crates/ferric-gguf/src/lib.rs:721-746
+// so this file is compiled with -ffp-contract=off AND spells every operation with the
+// round-to-nearest intrinsics, which the compiler never contracts.
+//
+// These kernels are write-bound (4 B out per 0.53-1.06 B in): one lane produces 4 consecutive
+// outputs and stores them as one 16-byte vector, so a wave writes 1 KiB contiguous per store.
+#include "common.hpp"
+
+#include <hip/hip_fp16.h>
+
+namespace {
+
+__device__ __forceinline__ float f16_bits(uint32_t b) {
+    // v_cvt_f32_f16: exact for every finite / subnormal / infinite pattern.
+    return __half2float(__ushort_as_half((unsigned short)b));
+}
+
+// 4 bytes from a 2-byte-aligned address (Q8_0 and Q6_K blocks are only 2-byte aligned).
+__device__ __forceinline__ uint32_t ld4_a2(const uint8_t* p) {
+    const uint16_t* h = (const uint16_t*)p;
+    return (uint32_t)h[0] | ((uint32_t)h[1] << 16);
+}
+
+__global__ void f16_to_f32_kernel(const uint16_t* __restrict__ in, size_t n, float* __restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = f16_bits(in[i]);
+}
+
+// ---- Q8_0: 34 B = [f16 d][i8 q[32]] ------------------------------------------------------------
+__global__ void deq_q8_0_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane = 4 values
+    if (t >= nquads) return;
+    size_t blk = t >> 3;
+    int j = (int)(t & 7) * 4;
+    const uint8_t* b = raw + blk * 34;
+    float d = f16_bits(*(const uint16_t*)b);
+    uint32_t q = ld4_a2(b + 2 + j);
+    float4 o;
+    o.x = __fmul_rn((float)(int8_t)(q & 0xFF), d);
+    o.y = __fmul_rn((float)(int8_t)((q >> 8) & 0xFF), d);
+    o.z = __fmul_rn((float)(int8_t)((q >> 16) & 0xFF), d);
+    o.w = __fmul_rn((float)(int8_t)(q >> 24), d);
+    *(float4*)(out + t * 4) = o;
+}
+
+// ---- Q4_K: 144 B = [f16 d][f16 dmin][u8 s[12]][u8 qs[128]] --------------------------------------
+// 6-bit (scale, min) of sub-block j -- get_sc_min, crates/ferric-gguf/src/lib.rs:795-804.
+__device__ __forceinline__ void q4k_sc_min(const uint8_t* s, int j, uint32_t& sc, uint32_t& m) {
+    if (j < 4) {
+        sc = s[j] & 63u;
+        m = s[j + 4] & 63u;
+    } else {
+        sc = (s[j + 4] & 0x0Fu) | ((uint32_t)(s[j - 4] >> 6) << 4);
+        m = (uint32_t)(s[j + 4] >> 4) | ((uint32_t)(s[j] >> 6) << 4);
+    }
+}
+
+__global__ void deq_q4_k_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane = 4 values, 64 lanes = one block
+    if (t >= nquads) return;
+    size_t blk = t >> 6;
+    int v = (int)(t & 63) * 4;
+    int sb = v >> 5, l = v & 31;
+    const uint8_t* b = raw + blk * 144;  // 16-byte aligned
+    uint32_t hd = *(const uint32_t*)b;
+    float d = f16_bits(hd & 0xFFFFu), dmin = f16_bits(hd >> 16);
+    uint32_t sc, m;
+    q4k_sc_min(b + 4, sb, sc, m);
+    uint32_t q = *(const uint32_t*)(b + 16 + 32 * (sb >> 1) + l);
+    if (sb & 1) q >>= 4;
+    q &= 0x0F0F0F0Fu;
+    float d1 = __fmul_rn(d, (float)sc), mm = __fmul_rn(dmin, (float)m);
+    float4 o;
+    o.x = __fsub_rn(__fmul_rn(d1, (float)(q & 0xFF)), mm);
+    o.y = __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xFF)), mm);
+    o.z = __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xFF)), mm);
+    o.w = __fsub_rn(__fmul_rn(d1, (float)(q >> 24)), mm);
+    *(float4*)(out + t * 4) = o;
+}
+
+// ---- Q6_K: 210 B = [u8 ql[128]][u8 qh[64]][i8 sc[16]][f16 d] ------------------------------------
+__global__ void deq_q6_k_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= nquads) return;
+    size_t blk = t >> 6;
+    int v = (int)(t & 63) * 4;
+    int hf = v >> 7, w = v & 127, g = w >> 5, l = w & 31, is = l >> 4;
+    const uint8_t* b = raw + blk * 210;  // 2-byte aligned
+    float d = f16_bits(*(const uint16_t*)(b + 208));
+    float sc = (float)(int8_t)b[192 + 8 * hf + is + 2 * g];
+    uint32_t ql = ld4_a2(b + 64 * hf + 32 * (g & 1) + l);
+    uint32_t qh = ld4_a2(b + 128 + 32 * hf + l);
+    uint32_t nib = (g >= 2 ? (ql >> 4) : ql) & 0x0F0F0F0Fu;
+    uint32_t q = nib | (((qh >> (2 * g)) & 0x03030303u) << 4);
+    float ds = __fmul_rn(d, sc);
+    float4 o;
+    o.x = __fmul_rn(ds, (float)((int)(q & 0xFF) - 32));
+    o.y = __fmul_rn(ds, (float)((int)((q >> 8) & 0xFF) - 32));
+    o.z = __fmul_rn(ds, (float)((int)((q >> 16) & 0xFF) - 32));
+    o.w = __fmul_rn(ds, (float)((int)(q >> 24) - 32));
+    *(float4*)(out + t * 4) = o;
+}
+
+}  // namespace
+
+namespace fhip {
+
+int launch_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_t s) {
+    if (n == 0) return FHIP_OK;
+    unsigned grid = (unsigned)((n + 255) / 256);
+    hipLaunchKernelGGL(f16_to_f32_kernel, dim3(grid), dim3(256), 0, s, d_bits, n, d_out);
+    return check_hip(hipGetLastError(), "f16_to_f32 launch");
+}
+
+int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d_out, hipStream_t s) {
+    if (nblocks == 0) return FHIP_OK;
+    size_t vals = type == FHIP_Q8_0 ? 32 : 256;
+    size_t nquads = nblocks * vals / 4;
+    size_t grid = (nquads + 255) / 256;
+    if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_ARG, "dequant: %zu blocks exceed one launch", nblocks);
+    switch (type) {
+        case FHIP_Q8_0: hipLaunchKernelGGL(deq_q8_0_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_Q4_K: hipLaunchKernelGGL(deq_q4_k_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_Q6_K: hipLaunchKernelGGL(deq_q6_k_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", type);
+    }
+    return check_hip(hipGetLastError(), "dequant launch");
+}
+
+}  // namespace fhip

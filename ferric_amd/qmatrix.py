@@ -1,0 +1,352 @@
+"""Host-side mirror of the reference's quantized-linear interface, over the C ABI.
+
+Names, argument meaning and error behaviour follow the reference (paths relative to its checkout):
+
+    type_size / deq_raw                       crates/ferric-gguf/src/lib.rs:471 / :497
+    QMatrix.block_bytes / from_bytes / ...    crates/ferric-tensor/src/dtype.rs:873-931
+    Q8_0Weights / Q4_KWeights / Q6_KWeights   crates/ferric-tensor/src/dtype.rs:1261 / 1374 / 1138
+    Tensor.matmul_q / try_matmul_swiglu / ... crates/ferric-tensor/src/dtype.rs:935-959
+    Tensor.swiglu                             crates/ferric-tensor/src/lib.rs:728
+    matvec_q8_0 / _threaded / _span           crates/ferric-tensor/src/cpu_simd.rs:79-122
+
+`Err(String)` becomes ValueError, an `assert!` panic becomes AssertionError. Everything computes on
+the GPU through libferric_hip.so; nothing here does arithmetic on the host.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+
+
+def _vp(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class Stream:
+    """One HIP stream; ops enqueue on it and return (ordering = submission order, as on the
+    reference's single wgpu queue). None means the default stream."""
+
+    def __init__(self):
+        lib = _lib.init()
+        h = C.c_void_p()
+        _lib.check(lib.fhip_stream_create(C.byref(h)))
+        self.handle = h
+
+    def synchronize(self):
+        _lib.check(_lib.load().fhip_stream_sync(self.handle))
+
+    def __del__(self):
+        try:
+            if self.handle:
+                _lib.load().fhip_stream_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+class Graph:
+    """Calls recorded on a stream between Graph.begin(stream) and .end(), replayed with launch():
+    the counterpart of the reference's batch(ctx, ..) single-submission recorder (lib.rs:1802)."""
+
+    def __init__(self, stream):
+        self.stream, self.handle = stream, None
+
+    @staticmethod
+    def begin(stream):
+        g = Graph(stream)
+        _lib.check(_lib.load().fhip_graph_capture_begin(stream.handle))
+        return g
+
+    def end(self):
+        h = C.c_void_p()
+        _lib.check(_lib.load().fhip_graph_capture_end(self.stream.handle, C.byref(h)))
+        self.handle = h
+        return self
+
+    def launch(self, stream=None):
+        _lib.check(_lib.load().fhip_graph_launch(self.handle, (stream or self.stream).handle))
+
+    def __del__(self):
+        try:
+            if self.handle:
+                _lib.load().fhip_graph_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def _stream_handle(stream):
+    return stream.handle if stream is not None else None
+
+
+class DeviceBuffer:
+    """nbytes of device memory, freed with the object."""
+
+    def __init__(self, nbytes):
+        lib = _lib.init()
+        p = C.c_void_p()
+        _lib.check(lib.fhip_malloc(C.byref(p), nbytes))
+        self.ptr, self.nbytes = p, nbytes
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                _lib.load().fhip_free(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+class Tensor:
+    """A contiguous row-major device tensor (f32 unless made with from_bf16_bits)."""
+
+    def __init__(self, buf, shape, dtype=np.float32):
+        self.buf, self.shape, self.dtype = buf, tuple(int(s) for s in shape), np.dtype(dtype)
+
+    # -- construction / readback (crates/ferric-tensor/src/lib.rs: Tensor::from_vec, to_vec) --
+    @staticmethod
+    def from_vec(data, shape, stream=None):
+        a = np.ascontiguousarray(data, dtype=np.float32)
+        assert a.size == int(np.prod(shape)), "from_vec: data does not match shape"
+        t = Tensor(DeviceBuffer(a.nbytes), shape)
+        _lib.check(_lib.load().fhip_memcpy_h2d(t.buf.ptr, _vp(a), a.nbytes, _stream_handle(stream)))
+        if stream is None:
+            _lib.check(_lib.load().fhip_stream_sync(None))
+        else:
+            stream.synchronize()  # the host array may go away
+        return t
+
+    @staticmethod
+    def from_bf16_bits(bits, shape):
+        a = np.ascontiguousarray(bits, dtype=np.uint16)
+        assert a.size == int(np.prod(shape))
+        t = Tensor(DeviceBuffer(a.nbytes), shape, np.uint16)
+        _lib.check(_lib.load().fhip_memcpy_h2d(t.buf.ptr, _vp(a), a.nbytes, None))
+        _lib.check(_lib.load().fhip_stream_sync(None))
+        return t
+
+    @staticmethod
+    def empty(shape, dtype=np.float32):
+        n = int(np.prod(shape))
+        return Tensor(DeviceBuffer(n * np.dtype(dtype).itemsize), shape, dtype)
+
+    def numel(self):
+        return int(np.prod(self.shape))
+
+    def to_vec(self, stream=None):
+        """Device -> host; the only synchronising call (the reference's readback)."""
+        out = np.empty(self.numel(), dtype=self.dtype)
+        _lib.check(_lib.load().fhip_memcpy_d2h(_vp(out), self.buf.ptr, out.nbytes, _stream_handle(stream)))
+        return out
+
+    # -- quantized matmuls --------------------------------------------------------------------
+    def _rows_inner(self):
+        assert len(self.shape) == 2, "matmul_q expects a [rows, in] tensor"
+        return self.shape
+
+    def matmul_q(self, w, stream=None):
+        """y = x . W^T for a packed weight of any supported format -- dtype.rs:935."""
+        rows, inn = self._rows_inner()
+        assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
+        out = Tensor.empty((rows, w.rows()))
+        _lib.check(_lib.load().fhip_matmul_q(w.handle, self.buf.ptr, rows, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def _matmul_typed(self, w, ty, stream):
+        assert w.ggml_type == ty, f"weight is ggml type {w.ggml_type}, not {ty}"
+        return self.matmul_q(w, stream)
+
+    def matmul_q8_0(self, w, stream=None):  # dtype.rs:1292
+        return self._matmul_typed(w, Q8_0, stream)
+
+    def matmul_q4_k(self, w, stream=None):  # dtype.rs:1426
+        return self._matmul_typed(w, Q4_K, stream)
+
+    def matmul_q6_k(self, w, stream=None):  # dtype.rs:1172
+        return self._matmul_typed(w, Q6_K, stream)
+
+    def try_matmul_swiglu(self, w, stream=None):
+        """Fused gate/up + SwiGLU -- dtype.rs:949. None when the format has no fused kernel
+        (Q8_0); the caller then runs matmul_q(w).swiglu(n_ff)."""
+        if w.ggml_type not in (Q4_K, Q6_K):
+            return None
+        rows, inn = self._rows_inner()
+        assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
+        out = Tensor.empty((rows, w.rows() // 2))
+        _lib.check(_lib.load().fhip_matmul_q_swiglu(w.handle, self.buf.ptr, rows, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def matmul_q4_k_swiglu(self, w, stream=None):  # dtype.rs:1551
+        assert w.ggml_type == Q4_K
+        return self.try_matmul_swiglu(w, stream)
+
+    def matmul_q6_k_swiglu(self, w, stream=None):  # dtype.rs:1802
+        assert w.ggml_type == Q6_K
+        return self.try_matmul_swiglu(w, stream)
+
+    def swiglu(self, d, stream=None):
+        """self is [t, 2d] = [gate | up]; returns silu(gate) * up as [t, d] -- lib.rs:728."""
+        t = self.numel() // (2 * d)
+        out = Tensor.empty((t, d))
+        _lib.check(_lib.load().fhip_swiglu(self.buf.ptr, t, d, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def ffn(self, gate_up, down, stream=None):
+        """down(swiglu(gate_up(x))) -- the FFN of crates/ferric-llama/src/qwen3.rs:944-964."""
+        rows, inn = self._rows_inner()
+        assert inn == gate_up.cols(), "gate_up in dim mismatch"
+        n_ff = gate_up.rows() // 2
+        ws = Tensor.empty((rows, n_ff))
+        out = Tensor.empty((rows, down.rows()))
+        _lib.check(_lib.load().fhip_ffn(gate_up.handle, down.handle, self.buf.ptr, rows, out.buf.ptr, ws.buf.ptr,
+                                        _stream_handle(stream)))
+        out._keepalive = ws  # scratch must outlive the enqueued work
+        return out
+
+    def gemm_q_bf16(self, w, stream=None):
+        """Prefill: self holds bf16 bit patterns [t, in]; y f32 [t, out] via the matrix cores -- dtype.rs:1818."""
+        assert self.dtype == np.uint16, "gemm_q_bf16 expects bf16 bit patterns"
+        t, inn = self._rows_inner()
+        assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
+        out = Tensor.empty((t, w.rows()))
+        _lib.check(_lib.load().fhip_gemm_q_bf16(w.handle, self.buf.ptr, t, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+
+class QMatrix:
+    """A packed-quant weight [rows = out, cols = in] resident in HBM as the raw GGUF block stream."""
+
+    def __init__(self, handle, ggml_type, keepalive=None):
+        self.handle, self.ggml_type, self._keepalive = handle, ggml_type, keepalive
+
+    @staticmethod
+    def block_bytes(ggml_type):
+        """(values per block, bytes per block) or None -- dtype.rs:873."""
+        v, b = C.c_size_t(), C.c_size_t()
+        rc = _lib.load().fhip_block_bytes(ggml_type, C.byref(v), C.byref(b))
+        return (v.value, b.value) if rc == _lib.OK else None
+
+    @staticmethod
+    def from_bytes(data, ggml_type, rows, cols):
+        """dtype.rs:893. Unknown type -> ValueError; cols not a block multiple or a wrong byte
+        length -> AssertionError (the per-format constructors' asserts)."""
+        lib = _lib.init()
+        a = np.ascontiguousarray(np.frombuffer(data, dtype=np.uint8) if isinstance(data, (bytes, bytearray, memoryview)) else data,
+                                 dtype=np.uint8)
+        h = C.c_void_p()
+        _lib.check(lib.fhip_weight_create(ggml_type, _vp(a), a.size, rows, cols, C.byref(h)))
+        return QMatrix(h, ggml_type)
+
+    @staticmethod
+    def wrap_device(buf, nbytes, ggml_type, rows, cols, offset=0):
+        """Adopt block bytes already in HBM (buf: DeviceBuffer), no copy."""
+        lib = _lib.init()
+        h = C.c_void_p()
+        _lib.check(lib.fhip_weight_wrap_device(ggml_type, C.c_void_p(buf.ptr.value + offset), nbytes, rows, cols, C.byref(h)))
+        return QMatrix(h, ggml_type, keepalive=buf)
+
+    def rows(self):
+        return _lib.load().fhip_weight_rows(self.handle)
+
+    def cols(self):
+        return _lib.load().fhip_weight_cols(self.handle)
+
+    def nbytes(self):
+        return _lib.load().fhip_weight_nbytes(self.handle)
+
+    def n_shards(self):
+        return 1  # one HBM allocation holds any size; the reference shards only for WebGPU binding limits
+
+    def dequant_rows(self, row0, nrows, stream=None):
+        """Rows [row0, row0+nrows) dequantized on the GPU, bit-exact with deq_raw."""
+        out = Tensor.empty((nrows, self.cols()))
+        _lib.check(_lib.load().fhip_dequant_rows(self.handle, row0, nrows, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def dequant(self, stream=None):
+        return self.dequant_rows(0, self.rows(), stream)
+
+    def __del__(self):
+        try:
+            if self.handle:
+                _lib.load().fhip_weight_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def _typed(ty, name):
+    class _W:
+        """Per-format constructor, same asserts as the reference's `from_bytes`."""
+
+        @staticmethod
+        def from_bytes(data, rows, cols):
+            return QMatrix.from_bytes(data, ty, rows, cols)
+
+    _W.__name__ = name
+    return _W
+
+
+Q8_0Weights = _typed(Q8_0, "Q8_0Weights")
+Q4_KWeights = _typed(Q4_K, "Q4_KWeights")
+Q6_KWeights = _typed(Q6_K, "Q6_KWeights")
+
+
+def type_size(ty, n):
+    """Bytes of n elements of ggml type ty -- lib.rs:471; unknown type -> ValueError."""
+    if QMatrix.block_bytes(ty) is None:
+        raise ValueError(f"unsupported ggml type {ty}")
+    return int(_lib.load().fhip_type_size(ty, n))
+
+
+def deq_raw(raw, n, ty):
+    """Dequantize n elements out of raw block bytes on the GPU -- lib.rs:497. Same edge behaviour:
+    K-quants return n values with a ragged tail left 0.0, Q8_0 returns whole blocks only."""
+    lib = _lib.init()
+    a = np.ascontiguousarray(raw, dtype=np.uint8)
+    out = np.empty(n, dtype=np.float32)
+    got = C.c_size_t()
+    _lib.check(lib.fhip_deq_raw(_vp(a), a.size, n, ty, _vp(out), C.byref(got)))
+    return out[: got.value]
+
+
+def f16_to_f32(bits):
+    """IEEE binary16 patterns -> f32 on the GPU -- lib.rs:605 rd_f16."""
+    lib = _lib.init()
+    a = np.ascontiguousarray(bits, dtype=np.uint16)
+    din, dout = DeviceBuffer(a.nbytes), DeviceBuffer(a.size * 4)
+    _lib.check(lib.fhip_memcpy_h2d(din.ptr, _vp(a), a.nbytes, None))
+    _lib.check(lib.fhip_f16_to_f32(din.ptr, a.size, dout.ptr, None))
+    out = np.empty(a.size, dtype=np.float32)
+    _lib.check(lib.fhip_memcpy_d2h(_vp(out), dout.ptr, out.nbytes, None))
+    return out
+
+
+def matvec_q8_0(x, w, rows, cols):
+    """y = x . W^T, W raw Q8_0 bytes [rows, cols], host arrays in and out -- cpu_simd.rs:79."""
+    lib = _lib.init()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    assert cols % 32 == 0, "Q8_0 cols must be a multiple of 32"
+    assert x.size == cols, "activation length must equal cols"
+    y = np.empty(rows, dtype=np.float32)
+    _lib.check(lib.fhip_matvec_q8_0_host(_vp(x), _vp(w), w.size, rows, cols, _vp(y)))
+    return y
+
+
+def matvec_q8_0_threaded(x, w, rows, cols, threads):
+    """cpu_simd.rs:92. The thread count only partitions rows on the CPU; on the GPU every
+    partition gives the same result, so it is accepted and ignored."""
+    del threads
+    return matvec_q8_0(x, w, rows, cols)
+
+
+def matvec_q8_0_span(x, w, cols, lo, hi, threads=1):
+    """Rows [lo, hi) only -- cpu_simd.rs:118."""
+    assert lo <= hi, "empty or inverted span"
+    row_bytes = cols // 32 * 34
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    return matvec_q8_0_threaded(x, w[lo * row_bytes: hi * row_bytes], hi - lo, cols, threads)

@@ -1,0 +1,174 @@
+/*
+ * ferric_hip.h -- C ABI of the MI355X (gfx950) quantized-GGUF matmul path.
+ *
+ * One shared library, libferric_hip.so, exports exactly these symbols. They are the functions a
+ * `ferric-hip` backend crate binds (extern "C") to stand in for the reference's quantized-linear
+ * entry points; each declaration cites the reference interface it replaces (paths are relative to
+ * the reference checkout).
+ *
+ * Conventions
+ *   - Weights are [rows = out, cols = in], row-major, as the RAW GGUF block byte stream
+ *     (Q8_0 34 B / 32 values, Q4_K 144 B / 256, Q6_K 210 B / 256). No repack is needed or done.
+ *   - Activations x are f32 [rows_x, cols] contiguous, outputs y are f32 [rows_x, rows] contiguous,
+ *     both in device memory owned by the caller.
+ *   - Every compute call only enqueues work on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream) and returns; there is no hidden synchronisation or allocation in them.
+ *   - Return value: FHIP_OK (0) or a negative FHIP_ERR_* code; the text is available from
+ *     fhip_last_error() (thread-local). Nothing in this library aborts the process: shape
+ *     violations that the reference turns into `assert!` panics come back as FHIP_ERR_SHAPE so the
+ *     binding can re-raise them on its own side.
+ *   - Handles are immutable after creation and may be shared read-only between threads; one host
+ *     thread drives one stream.
+ */
+#ifndef FERRIC_HIP_H
+#define FERRIC_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type ids of the supported formats (crates/ferric-gguf/src/lib.rs:471-494). */
+#define FHIP_Q8_0 8u
+#define FHIP_Q4_K 12u
+#define FHIP_Q6_K 14u
+
+#define FHIP_OK 0
+#define FHIP_ERR_UNSUPPORTED_TYPE (-1) /* reference: Err("unsupported ggml type N") / Err("QMatrix: no native matmul ...") */
+#define FHIP_ERR_SHAPE (-2)            /* reference: assert!/assert_eq! panic on cols % block, byte length, inner dim */
+#define FHIP_ERR_HIP (-3)              /* a HIP runtime call failed */
+#define FHIP_ERR_ARG (-4)              /* NULL pointer or otherwise unusable argument */
+
+typedef struct fhip_weight fhip_weight; /* opaque: one packed weight resident in HBM */
+
+/* ---- library / device ---------------------------------------------------------------------- */
+
+/* Select the device and probe it. Stands where the reference creates its device context
+ * (crates/ferric-core/src/lib.rs:109 Context::new). Must be called once before anything else. */
+int fhip_init(int device);
+
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char* fhip_last_error(void);
+
+/* Number of compute units of the initialised device (0 before fhip_init). */
+int fhip_device_cus(void);
+
+/* ---- sizes --------------------------------------------------------------------------------- */
+
+/* crates/ferric-gguf/src/lib.rs:471 type_size(ty, n): bytes of n elements; 0 = unsupported type
+ * (the reference returns Err). Integer division truncates as in the reference (n/32*34 ...). */
+size_t fhip_type_size(uint32_t ggml_type, size_t n);
+
+/* crates/ferric-tensor/src/dtype.rs:873 QMatrix::block_bytes: (values, bytes) of one block.
+ * Returns FHIP_OK or FHIP_ERR_UNSUPPORTED_TYPE (reference: None). */
+int fhip_block_bytes(uint32_t ggml_type, size_t* values, size_t* bytes);
+
+/* ---- device memory, streams, events (plumbing the binding needs to own tensors) ------------- */
+/* These stand where the reference's Tensor creates/reads wgpu buffers
+ * (crates/ferric-tensor/src/lib.rs:1481 empty(), :141 to_vec(), :1816 readback). */
+int fhip_malloc(void** d_ptr, size_t nbytes);
+int fhip_free(void* d_ptr);
+int fhip_memcpy_h2d(void* d_dst, const void* h_src, size_t nbytes, void* stream); /* async on stream */
+int fhip_memcpy_d2h(void* h_dst, const void* d_src, size_t nbytes, void* stream); /* synchronises stream before returning */
+int fhip_memcpy_d2d(void* d_dst, const void* d_src, size_t nbytes, void* stream);
+int fhip_memset(void* d_dst, int byte, size_t nbytes, void* stream);
+int fhip_stream_create(void** stream);
+int fhip_stream_destroy(void* stream);
+int fhip_stream_sync(void* stream);
+int fhip_event_create(void** event);
+int fhip_event_destroy(void* event);
+int fhip_event_record(void* event, void* stream);
+int fhip_event_sync(void* event);
+int fhip_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* Record-then-replay of a sequence of calls on one stream, standing for the reference's
+ * batch(ctx, ..) recorder that encodes every dispatch of a decode step into one submission
+ * (crates/ferric-tensor/src/lib.rs:1802). Between begin and end, compute calls on `stream` (which
+ * must come from fhip_stream_create) are captured into a HIP graph instead of executed; the
+ * returned executable graph replays them with one launch. Buffers used by the captured calls must
+ * stay alive and in place while the graph exists. */
+int fhip_graph_capture_begin(void* stream);
+int fhip_graph_capture_end(void* stream, void** graph_exec);
+int fhip_graph_launch(void* graph_exec, void* stream);
+int fhip_graph_destroy(void* graph_exec);
+
+/* ---- packed weights ------------------------------------------------------------------------ */
+
+/* crates/ferric-tensor/src/dtype.rs:893 QMatrix::from_bytes(ctx, bytes, ggml_type, rows, cols) and the
+ * per-format constructors Q8_0Weights/Q4_KWeights/Q6_KWeights::from_bytes (dtype.rs:1270/1388/1147).
+ * Copies `nbytes` host bytes into HBM (the caller keeps nothing alive). The device layout IS the
+ * GGUF byte stream; one allocation holds any size, so there is no row-sharding.
+ * Errors: unsupported type -> FHIP_ERR_UNSUPPORTED_TYPE; cols % block_values != 0 or
+ * nbytes != rows*(cols/block_values)*block_bytes -> FHIP_ERR_SHAPE. */
+int fhip_weight_create(uint32_t ggml_type, const uint8_t* h_raw, size_t nbytes, size_t rows, size_t cols,
+                       fhip_weight** out);
+
+/* Same, but adopts block bytes that are already in device memory (no copy; the caller keeps the
+ * buffer alive until fhip_weight_destroy). Used when a loader streams a file straight into HBM. */
+int fhip_weight_wrap_device(uint32_t ggml_type, const uint8_t* d_raw, size_t nbytes, size_t rows, size_t cols,
+                            fhip_weight** out);
+
+void fhip_weight_destroy(fhip_weight* w);
+
+/* dtype.rs:927-930 QMatrix::{rows, cols, nbytes}; ggml type of the handle. */
+size_t fhip_weight_rows(const fhip_weight* w);
+size_t fhip_weight_cols(const fhip_weight* w);
+size_t fhip_weight_nbytes(const fhip_weight* w);
+uint32_t fhip_weight_type(const fhip_weight* w);
+
+/* ---- unpackers (bit-exact with the reference CPU dequantizers) ------------------------------- */
+
+/* crates/ferric-gguf/src/lib.rs:605 rd_f16 / crates/ferric-tensor/src/cpu_simd.rs:29 f16:
+ * n IEEE binary16 patterns (device) -> f32 (device), exact incl. subnormal / inf / nan. */
+int fhip_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, void* stream);
+
+/* crates/ferric-gguf/src/lib.rs:608 deq_q8_0, :793 deq_q4_k, :721 deq_q6_k applied to rows
+ * [row0, row0+nrows) of a resident weight: d_out receives nrows*cols f32, row-major.
+ * (The callers dequantize embedding rows this way: crates/ferric-llama/src/qwen3.rs:749.) */
+int fhip_dequant_rows(const fhip_weight* w, size_t row0, size_t nrows, float* d_out, void* stream);
+
+/* crates/ferric-gguf/src/lib.rs:497 deq_raw(raw, n, ty) with host buffers on both sides: uploads,
+ * dequantizes on the GPU, downloads, synchronises. h_out must hold n f32. *n_written receives what
+ * the reference's Vec would hold: n for the K-quants (a ragged tail stays 0.0), whole blocks only
+ * for Q8_0. Only min(n / block_values, nbytes / block_bytes) whole blocks are read. */
+int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ggml_type, float* h_out, size_t* n_written);
+
+/* ---- matmuls ------------------------------------------------------------------------------- */
+
+/* crates/ferric-tensor/src/dtype.rs:935 Tensor::matmul_q (and :1292 matmul_q8_0, :1426 matmul_q4_k,
+ * :1172 matmul_q6_k): y[rows_x, rows] = x[rows_x, cols] * W^T, f32 in, f32 accumulate, f32 out.
+ * rows_x = 1 is the decode GEMV; any rows_x >= 1 is accepted. */
+int fhip_matmul_q(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, void* stream);
+
+/* crates/ferric-tensor/src/dtype.rs:949 try_matmul_swiglu / :1551 matmul_q4_k_swiglu / :1802
+ * matmul_q6_k_swiglu: `gate_up` stacks gate rows [0, n_ff) then up rows [n_ff, 2 n_ff);
+ * y[rows_x, n_ff] = silu(x*gate^T) * (x*up^T), silu(g) = g / (1 + exp(-g)).
+ * Errors: odd row count -> FHIP_ERR_SHAPE; Q8_0 -> FHIP_ERR_UNSUPPORTED_TYPE (reference: None,
+ * the caller then runs matmul_q + swiglu). */
+int fhip_matmul_q_swiglu(const fhip_weight* gate_up, const float* d_x, size_t rows_x, float* d_y, void* stream);
+
+/* crates/ferric-tensor/src/lib.rs:728 Tensor::swiglu(d): gu is [t, 2d] = [gate | up] per row,
+ * out[t, d] = silu(gate) * up. */
+int fhip_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, void* stream);
+
+/* The FFN block of crates/ferric-llama/src/qwen3.rs:944-964: y = down( swiglu( gate_up(x) ) ).
+ * d_ws is caller-provided scratch of at least rows_x * n_ff f32 (n_ff = gate_up rows / 2). */
+int fhip_ffn(const fhip_weight* gate_up, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y,
+             float* d_ws, void* stream);
+
+/* Prefill dequant-GEMM, stands for crates/ferric-tensor/src/dtype.rs:1818 matmul_q4_k_coop (:1199
+ * Q6_K, :1316 Q8_0): x is bf16 [t, cols] (raw 16-bit patterns), y f32 [t, rows]; weights are
+ * dequantized tile by tile into LDS as bf16 and contracted on the matrix cores, f32 accumulate. */
+int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x_bf16, size_t t, float* d_y, void* stream);
+
+/* crates/ferric-tensor/src/cpu_simd.rs:79 matvec_q8_0(x, w, rows, cols) with HOST buffers on both
+ * sides (upload, GEMV, download, synchronise) -- the drop-in for the CPU mat-vec call.
+ * Errors as the reference's asserts: cols % 32, w_len != rows * cols/32*34 -> FHIP_ERR_SHAPE. */
+int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, size_t rows, size_t cols, float* h_y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FERRIC_HIP_H */

@@ -1,0 +1,256 @@
+"""GPU mat-vec / small-batch matmul / fused SwiGLU / FFN vs the CPU oracle, through the C ABI.
+
+Tolerances (written where used):
+  * north-star bound: |y - y64| <= 1e-3 * ||w_row||_2 * ||x||_2 against the f64-accumulated product of
+    the oracle-dequantized weights;
+  * the reference examples' own bar for scalar kernels: max|y - ref| / max(|ref|, 1e-3) < 1e-5
+    (crates/ferric-tensor/examples/q4_k.rs:54, q6_k.rs:33, q8_0.rs:21, ffn_fuse.rs:106).
+"""
+import numpy as np
+import pytest
+
+from conftest import bits
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+
+
+def check_matmul(F, O, w, ty, rows, cols, x, what=""):
+    """Run y = x W^T on the GPU and hold it to both tolerances; returns the GPU result [m, rows]."""
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, cols)
+    qm = F.QMatrix.from_bytes(w, ty, rows, cols)
+    assert (qm.rows(), qm.cols(), qm.nbytes(), qm.n_shards()) == (rows, cols, w.size, 1)
+    y = F.Tensor.from_vec(x, x.shape).matmul_q(qm).to_vec().reshape(x.shape[0], rows)
+    y64, wn = O.matmul_f64(x, w, ty, rows, cols)
+    err = np.abs(y - y64)
+    bound = 1e-3 * wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None]
+    assert (err <= bound + 1e-30).all(), f"{what}: north-star bound violated by {np.max(err / (bound + 1e-30)):.3g}x"
+    rel = err.max() / max(1e-3, np.abs(y64).max())
+    assert rel < 1e-5, f"{what}: max|d|/max|ref| = {rel:.2e}"
+    return y
+
+
+def cosx(m, cols):
+    return np.cos(np.arange(m * cols, dtype=np.float32) * np.float32(0.013)).astype(np.float32).reshape(m, cols)
+
+
+# ---------------------------------------------------------------- the reference examples, same inputs
+
+@pytest.mark.parametrize("rows,cols,m", [(8, 256, 4), (13, 512, 1), (4096, 2048, 1)])
+def test_q4_k_example(F, O, rows, cols, m):          # crates/ferric-tensor/examples/q4_k.rs:43-56
+    check_matmul(F, O, O.gen_kquant_matrix(Q4_K, rows, cols), Q4_K, rows, cols, cosx(m, cols), "q4_k.rs")
+
+
+@pytest.mark.parametrize("rows,cols,m", [(8, 256, 4), (7, 512, 1), (2048, 1024, 1)])
+def test_q6_k_example(F, O, rows, cols, m):          # crates/ferric-tensor/examples/q6_k.rs:22-35
+    check_matmul(F, O, O.gen_kquant_matrix(Q6_K, rows, cols), Q6_K, rows, cols, cosx(m, cols), "q6_k.rs")
+
+
+@pytest.mark.parametrize("rows,cols,m", [(8, 256, 4), (13, 128, 1), (4096, 2048, 1)])
+def test_q8_0_example(F, O, rows, cols, m):          # crates/ferric-tensor/examples/q8_0.rs:10-23
+    wf = (np.sin(np.arange(rows * cols, dtype=np.float32) * np.float32(0.021)) * np.float32(0.7)).astype(np.float32)
+    check_matmul(F, O, O.quant_q8_0(wf), Q8_0, rows, cols, cosx(m, cols), "q8_0.rs")
+
+
+def test_golden_gemv_vectors(F, golden):
+    x = golden["gemv_x"]
+    for name, ty in (("q4k", Q4_K), ("q6k", Q6_K), ("q8_0", Q8_0)):
+        qm = F.QMatrix.from_bytes(golden[f"gemv_{name}_w"], ty, 8, 256)
+        y = F.Tensor.from_vec(x, (1, 256)).matmul_q(qm).to_vec()
+        want = golden[f"gemv_{name}_y64"]
+        assert np.abs(y - want).max() / max(1e-3, np.abs(want).max()) < 1e-5, name
+        assert (np.abs(y - want) <= 1e-3 * golden[f"gemv_{name}_wnorm"] * np.linalg.norm(x.astype(np.float64))).all(), name
+
+
+# ---------------------------------------------------------------- cpu_simd.rs tests against the drop-in host entry
+
+def test_matvec_matches_the_dequantised_reference(F, O):      # cpu_simd.rs:162-173
+    for rows, cols in [(1, 32), (8, 64), (17, 256), (64, 512)]:
+        raw, vals = O.gen_q8_0_synth(rows, cols, rows * 13 + cols)
+        x = ((np.arange(cols) * 37 % 101).astype(np.float32) - 50.0) / np.float32(50.0)
+        got = F.matvec_q8_0(x, raw, rows, cols)
+        want = (vals.reshape(rows, cols).astype(np.float64) * x).sum(1)
+        assert np.abs(got - want).max() / max(1e-6, np.abs(want).max()) < 1e-5
+        cpu = O.matvec_q8_0(x, raw, rows, cols)                # GPU vs the CPU mat-vec itself: fabric_split.rs:54 bar
+        assert np.abs(got - cpu).max() / max(1e-6, np.abs(cpu).max()) < 1e-4
+
+
+def test_partitioning_changes_nothing_about_the_answer(F, O):  # cpu_simd.rs:175-200
+    raw, _ = O.gen_q8_0_synth(64, 256, 7)
+    x = np.sin(np.arange(256, dtype=np.float32) * np.float32(0.01))
+    one = F.matvec_q8_0(x, raw, 64, 256)
+    for t in (2, 3, 8, 64, 128):
+        assert np.array_equal(bits(one), bits(F.matvec_q8_0_threaded(x, raw, 64, 256, t)))
+    raw, _ = O.gen_q8_0_synth(40, 128, 3)
+    x = (np.arange(128) % 7).astype(np.float32) - 3.0
+    whole = F.matvec_q8_0(x, raw, 40, 128)
+    for cut in (0, 1, 17, 39, 40):
+        joined = np.concatenate([F.matvec_q8_0_span(x, raw, 128, 0, cut), F.matvec_q8_0_span(x, raw, 128, cut, 40)])
+        assert np.array_equal(bits(whole), bits(joined)), cut
+
+
+# ---------------------------------------------------------------- benchmark configurations at full size
+
+def test_config1_q8_0_4096(F, O):
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(Q8_0, 4096, 4096, 0)
+    x = np.random.default_rng(0).standard_normal(4096).astype(np.float32)       # seed 0, as the config says
+    y = check_matmul(F, O, w, Q8_0, 4096, 4096, x, "C1")
+    cpu = O.matmul_cpu(x, w, Q8_0, 4096, 4096, threads=8, direct_q8=True)        # the repo's CPU reference dequant-dot
+    assert np.abs(y - cpu).max() / np.abs(cpu).max() < 1e-4
+
+
+def test_config2_q4_k_5120(F, O):
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(Q4_K, 5120, 5120, 1)
+    x = np.random.default_rng(2).standard_normal(5120).astype(np.float32)
+    y = check_matmul(F, O, w, Q4_K, 5120, 5120, x, "C2")
+    cpu = O.matmul_cpu(x, w, Q4_K, 5120, 5120, threads=8)
+    assert np.abs(y - cpu).max() / np.abs(cpu).max() < 1e-4
+
+
+@pytest.mark.parametrize("batch", [1, 4, 8])
+def test_config3_ffn_block(F, O, batch):
+    # gate|up 2 x (5120 -> 17408) Q4_K stacked gate-first, down 17408 -> 5120 Q6_K, SwiGLU between
+    from ferric_amd.synth import synth_weights
+    n_embd, n_ff = 5120, 17408
+    gu = synth_weights(Q4_K, 2 * n_ff, n_embd, 3)
+    dn = synth_weights(Q6_K, n_embd, n_ff, 4)
+    x = np.random.default_rng(5).standard_normal((batch, n_embd)).astype(np.float32)
+    wgu = F.QMatrix.from_bytes(gu, Q4_K, 2 * n_ff, n_embd)
+    wdn = F.QMatrix.from_bytes(dn, Q6_K, n_embd, n_ff)
+    xt = F.Tensor.from_vec(x, x.shape)
+    # stage 1: fused gate/up + SwiGLU vs f64
+    h = xt.try_matmul_swiglu(wgu).to_vec().reshape(batch, n_ff)
+    g64, wn = O.matmul_f64(x, gu, Q4_K, 2 * n_ff, n_embd)
+    g, u = g64[:, :n_ff], g64[:, n_ff:]
+    h64 = g / (1.0 + np.exp(-g)) * u
+    assert np.abs(h - h64).max() / np.abs(h64).max() < 1e-5
+    # stage 2: down projection of the GPU's own h (so the check isolates the Q6_K matmul)
+    y = F.Tensor.from_vec(h, h.shape).matmul_q(wdn).to_vec().reshape(batch, n_embd)
+    y64, wn = O.matmul_f64(h, dn, Q6_K, n_embd, n_ff)
+    err = np.abs(y - y64)
+    assert (err <= 1e-3 * wn[None, :] * np.linalg.norm(h.astype(np.float64), axis=1)[:, None]).all()
+    assert err.max() / np.abs(y64).max() < 1e-5
+    # the one-call FFN gives the same bits as the two stages
+    y2 = xt.ffn(wgu, wdn).to_vec().reshape(batch, n_embd)
+    assert np.array_equal(bits(y2), bits(y))
+
+
+# ---------------------------------------------------------------- invariants
+
+@pytest.mark.parametrize("ty,rows,cols", [(Q4_K, 96, 5120), (Q6_K, 70, 2048), (Q8_0, 130, 1024), (Q6_K, 40, 17408)])
+def test_batch_rows_are_independent(F, O, ty, rows, cols):
+    # row r of a batch-m result is bit-identical to the batch-1 result for x_r
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(ty, rows, cols, 7)
+    qm = F.QMatrix.from_bytes(w, ty, rows, cols)
+    x = np.random.default_rng(8).standard_normal((11, cols)).astype(np.float32)
+    singles = np.stack([F.Tensor.from_vec(x[i], (1, cols)).matmul_q(qm).to_vec() for i in range(11)])
+    for m in (2, 3, 4, 5, 8, 11):
+        y = check_matmul(F, O, w, ty, rows, cols, x[:m], f"batch {m}")
+        assert np.array_equal(bits(y), bits(singles[:m])), m
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+def test_row_partition_invariance_and_odd_shapes(F, O, ty):
+    # any split of the output rows gives identical bits (the property QMatrix sharding and the
+    # CPU/GPU fabric split rely on: dtype.rs:936-943, cpu_simd.rs:114-122); shapes that do not fill
+    # a wave, a workgroup or the grid evenly
+    from ferric_amd.synth import synth_weights
+    vals, nbytes = O.BLOCK[ty]
+    for rows, cols in [(1, 256), (3, 256), (257, 768), (1000, 2304), (33, 8192), (5, 32768 if ty != Q8_0 else 4096)]:
+        w = synth_weights(ty, rows, cols, rows)
+        x = np.random.default_rng(rows).standard_normal(cols).astype(np.float32)
+        whole = check_matmul(F, O, w, ty, rows, cols, x, f"{rows}x{cols}")[0]
+        rb = cols // vals * nbytes
+        cut = rows // 3
+        parts = []
+        for lo, hi in ((0, cut), (cut, rows)):
+            if hi > lo:
+                qm = F.QMatrix.from_bytes(w[lo * rb: hi * rb], ty, hi - lo, cols)
+                parts.append(F.Tensor.from_vec(x, (1, cols)).matmul_q(qm).to_vec())
+        assert np.array_equal(bits(np.concatenate(parts)), bits(whole))
+
+
+def test_q8_0_cols_multiple_of_32_only(F, O):
+    from ferric_amd.synth import synth_weights
+    for rows, cols in [(9, 32), (4, 96), (17, 1056)]:
+        w = synth_weights(Q8_0, rows, cols, 3)
+        check_matmul(F, O, w, Q8_0, rows, cols, np.random.default_rng(1).standard_normal((3, cols)), f"{rows}x{cols}")
+
+
+def test_zero_inputs_give_exact_zeros(F, O):
+    from ferric_amd.synth import synth_weights
+    for ty in (Q4_K, Q6_K, Q8_0):
+        w = synth_weights(ty, 64, 1024, 1)
+        qm = F.QMatrix.from_bytes(w, ty, 64, 1024)
+        y = F.Tensor.from_vec(np.zeros((2, 1024), np.float32), (2, 1024)).matmul_q(qm).to_vec()
+        assert not y.any()
+        vals, nbytes = O.BLOCK[ty]
+        qz = F.QMatrix.from_bytes(np.zeros(64 * 1024 // vals * nbytes, np.uint8), ty, 64, 1024)
+        y = F.Tensor.from_vec(np.random.default_rng(0).standard_normal((2, 1024)).astype(np.float32), (2, 1024)).matmul_q(qz).to_vec()
+        assert not y.any()
+
+
+# ---------------------------------------------------------------- fused SwiGLU
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [1, 8])
+def test_fused_swiglu_matches_unfused(F, O, ty, t):
+    # crates/ferric-tensor/examples/ffn_fuse.rs:66-108: n_ff 3072, n_embd 1024, h = cos(0.017 i) * 0.3
+    n_ff, n_embd = 3072, 1024
+    w = O.gen_kquant_matrix(ty, 2 * n_ff, n_embd)
+    qm = F.QMatrix.from_bytes(w, ty, 2 * n_ff, n_embd)
+    h = (np.cos(np.arange(t * n_embd, dtype=np.float32) * np.float32(0.017)) * np.float32(0.3)).astype(np.float32).reshape(t, n_embd)
+    ht = F.Tensor.from_vec(h, h.shape)
+    fused = ht.try_matmul_swiglu(qm).to_vec()
+    unfused = ht.matmul_q(qm).swiglu(n_ff).to_vec()
+    scale = max(1e-3, np.abs(unfused).max())
+    assert np.abs(fused - unfused).max() / scale < 1e-5
+    g64, _ = O.matmul_f64(h, w, ty, 2 * n_ff, n_embd)
+    want = (g64[:, :n_ff] / (1 + np.exp(-g64[:, :n_ff])) * g64[:, n_ff:]).reshape(-1)
+    assert np.abs(fused - want).max() / max(1e-3, np.abs(want).max()) < 1e-5
+    assert np.abs(O.swiglu(ht.matmul_q(qm).to_vec().reshape(t, -1), n_ff).reshape(-1) - unfused).max() / scale < 1e-6
+
+
+def test_swiglu_unsupported_for_q8_0(F, O):
+    from ferric_amd.synth import synth_weights
+    qm = F.QMatrix.from_bytes(synth_weights(Q8_0, 64, 256, 1), Q8_0, 64, 256)
+    x = F.Tensor.from_vec(np.ones((1, 256), np.float32), (1, 256))
+    assert x.try_matmul_swiglu(qm) is None                                  # dtype.rs:949-959 returns None -> caller un-fuses
+    y = x.matmul_q(qm).swiglu(32).to_vec()
+    assert y.shape == (32,)
+
+
+# ---------------------------------------------------------------- error behaviour of the boundary
+
+def test_constructor_errors_match_the_reference(F):
+    z = np.zeros(144 * 4, np.uint8)
+    with pytest.raises(ValueError, match="no native matmul for ggml type 13"):         # dtype.rs:855
+        F.QMatrix.from_bytes(z, 13, 1, 256)
+    with pytest.raises(AssertionError, match="Q4_K cols must be a multiple of 256"):    # dtype.rs:1389
+        F.Q4_KWeights.from_bytes(z, 1, 300)
+    with pytest.raises(AssertionError, match="unexpected Q4_K byte length"):            # dtype.rs:1390
+        F.Q4_KWeights.from_bytes(z, 5, 256)
+    with pytest.raises(AssertionError, match="Q6_K cols must be a multiple of 256"):    # dtype.rs:1148
+        F.Q6_KWeights.from_bytes(z, 1, 128)
+    with pytest.raises(AssertionError, match="unexpected Q8_0 byte length"):            # dtype.rs:1272
+        F.Q8_0Weights.from_bytes(z, 2, 64)
+    qm = F.Q4_KWeights.from_bytes(z, 4, 256)
+    with pytest.raises(AssertionError, match="inner dim mismatch"):                     # dtype.rs:1429
+        F.Tensor.from_vec(np.zeros(512, np.float32), (1, 512)).matmul_q(qm)
+    with pytest.raises(AssertionError):                                                 # cpu_simd.rs:80-83
+        F.matvec_q8_0(np.zeros(33, np.float32), np.zeros(34, np.uint8), 1, 33)
+    with pytest.raises(AssertionError, match="unexpected Q8_0 byte length"):
+        F.matvec_q8_0(np.zeros(32, np.float32), np.zeros(35, np.uint8), 1, 32)
+
+
+def test_empty_shapes(F):
+    qm = F.QMatrix.from_bytes(np.zeros(0, np.uint8), Q4_K, 0, 256)
+    assert F.Tensor.from_vec(np.zeros(256, np.float32), (1, 256)).matmul_q(qm).to_vec().size == 0
+    qm = F.QMatrix.from_bytes(np.zeros(144 * 3, np.uint8), Q4_K, 3, 256)
+    assert F.Tensor.from_vec(np.zeros(0, np.float32), (0, 256)).matmul_q(qm).to_vec().size == 0
+    assert F.matvec_q8_0(np.zeros(0, np.float32), np.zeros(0, np.uint8), 0, 0).size == 0
+    y = F.matvec_q8_0(np.zeros(0, np.float32), np.zeros(0, np.uint8), 5, 0)
+    assert y.shape == (5,) and not y.any()
