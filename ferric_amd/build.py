@@ -22,6 +22,7 @@ UNITS = {
     "api.hip": [],
     "dequant.hip": ["-ffp-contract=off"],
     "gemv.hip": [],
+    "gemv_generic.hip": [],
     "gemm_mfma.hip": [],
 }
 

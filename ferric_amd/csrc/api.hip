@@ -11,6 +11,7 @@ namespace {
 thread_local char g_err[512] = "";
 int g_device = -1;
 int g_cus = 0;
+size_t g_lds = 64 * 1024;
 
 bool block_info(uint32_t ty, size_t& vals, size_t& bytes) {
     switch (ty) {
@@ -59,6 +60,7 @@ int check_hip(hipError_t e, const char* what) {
 }
 
 int device_cus() { return g_cus; }
+size_t device_lds_bytes() { return g_lds; }
 
 }  // namespace fhip
 
@@ -78,6 +80,8 @@ int fhip_init(int device) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return set_error(FHIP_ERR_HIP, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
     g_cus = prop.multiProcessorCount;
+    g_lds = prop.sharedMemPerBlockOptin > prop.sharedMemPerBlock ? prop.sharedMemPerBlockOptin : prop.sharedMemPerBlock;
+    if (g_lds < 64 * 1024) g_lds = 64 * 1024;
     g_device = device;
     return FHIP_OK;
 }

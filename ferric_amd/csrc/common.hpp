@@ -21,6 +21,7 @@ namespace fhip {
 int set_error(int code, const char* fmt, ...);
 int check_hip(hipError_t e, const char* what);
 int device_cus();
+size_t device_lds_bytes();  // LDS one workgroup may use
 
 // dequant.hip
 int launch_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_t s);
@@ -30,6 +31,8 @@ int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d
 // y[rows_x, out_rows] = x * W^T; when n_ff > 0 the weight stacks gate|up (2*n_ff rows) and
 // y[rows_x, n_ff] = silu(gate.x) * (up.x).
 int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
+// gemv_generic.hip: same contract, any cols the format allows (up to 32768)
+int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s);
 
 // gemm_mfma.hip

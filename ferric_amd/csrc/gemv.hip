@@ -1,23 +1,31 @@
-// Decode-shape mat-vec (and small-batch mat-mat) on the raw GGUF block stream, gfx950.
+// Decode mat-vec (and batch <= 4 per pass) streaming the raw GGUF block bytes once, gfx950.
 //
-//   y[m, o] = sum_k x[m, k] * dequant(W[o, k])        f32 activations, f32 accumulate
+//   y[m, o] = sum_k x[m, k] * dequant(W[o, k])
 //
 // Replaces the reference's split-K / flat WGSL kernels (crates/ferric-tensor/src/dtype.rs:2995-3051
 // Q4_K, :3423-3469 Q6_K, :3473-3529 Q8_0) and the fused gate/up SwiGLU kernels (:2372-2410, :2734-2775).
 //
-// Work decomposition (memory-bound design, one pass over the weight bytes):
-//   * The unit of lane work is 32 weights of one row ("unit"): a 16-byte quant chunk of a Q4_K
-//     block, an (8+8+8)-byte ql/ql/qh triple of a Q6_K block, or one whole 34-byte Q8_0 block.
-//     A row has cols/32 units, for every format.
-//   * A wave owns 64 consecutive units of the row (a K-slice) and keeps the matching 32 activation
-//     values per lane in REGISTERS for its whole life: the lane -> column mapping is the same for
-//     every row, so x is read once per wave (staged through LDS once per workgroup) and never again.
-//   * S = ceil(units/64) waves cover one row (K split across waves); G such wave-sets ("row groups")
-//     share a workgroup and walk disjoint contiguous row spans, streaming the weight bytes with
-//     16-/8-byte loads straight from the GGUF layout, U rows in flight per wave.
-//   * Per row each wave reduces its 64 partial sums with DPP (no LDS traffic) and parks one float
-//     in LDS; after one barrier the S partials of each row are added in a fixed order, so the result
-//     does not depend on scheduling.
+// Why it looks the way it does. At 8 TB/s a CU gets ~13 weight bytes per clock, i.e. ~23 Q4_K weights,
+// while it can issue 64 lane-instructions per clock: under 3 instructions per weight all-in. A plain
+// "unpack nibble, convert, f32 multiply-add" loop costs ~4.7, so it is instruction-bound at about a
+// third of the memory roofline. This kernel gets below 2 by
+//   * holding the activations as 24-bit block fixed point (three signed byte planes per run of 32 or
+//     16 columns, one f32 scale per run: the same significand width as f32 at the run maximum) and
+//     doing the inner products with v_dot4_i32_i8 -- four weights per instruction and plane, exact
+//     integer sums, converted once per sub-block and from there on accumulated in f32;
+//   * giving a lane 64 weights that share one scale header (two nibble chunks of one Q4_K group, one
+//     ql/ql/qh triple of a Q6_K half), so the 6-bit scale decode is paid once per 64 weights;
+//   * keeping the lane -> column mapping fixed for the life of a wave, so the activation planes sit in
+//     registers (quantised once per workgroup through LDS) and are never re-read.
+//
+// Tiling. 16 lanes ("slot") cover 16 units = 1024 weights (512 for Q8_0) of one row; a row is NG slots.
+// Waves 0..NG/4-1 of a row group take 4 consecutive slots of the same row; the NG%4 left-over slots
+// go to one tail wave that works on 4 (or 2) rows at once, so no lane idles for K = 5120 or 17408.
+// Each slot reduces its 16 lanes with DPP and parks one float per row in LDS; after one barrier the
+// NG partials of a row are added in a fixed order (results do not depend on scheduling or on how rows
+// are partitioned over workgroups). Row groups walk contiguous row spans with U rows of 16-byte
+// loads in flight per wave; weight loads for the first rows are issued before the activations are
+// touched, so the two latencies overlap.
 #include "common.hpp"
 
 #include <hip/hip_fp16.h>
@@ -27,166 +35,190 @@ namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-// Q6_K / Q8_0 blocks are only 2-byte aligned in the GGUF stream; gfx950 global loads accept that.
 struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };
 struct __attribute__((packed, aligned(2))) U2A2 { u32x2 v; };
 
 __device__ __forceinline__ float f16_bits(uint32_t b) { return __half2float(__ushort_as_half((unsigned short)b)); }
-__device__ __forceinline__ float ub(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }  // v_cvt_f32_ubyteK
+__device__ __forceinline__ float ub(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ float sb(uint32_t v, int k) { return (float)(int8_t)((v >> (8 * k)) & 0xFFu); }
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 
-// Pins a loaded dword in a VGPR at the point of use. Without it the optimizer unpacks the bytes of
-// a prefetched row the moment the load returns and carries 32 unpacked values per row in flight,
-// which spills; with it the rows in flight stay as the packed dwords that were loaded.
+// Keeps a prefetched row as the packed dwords that were loaded (otherwise the optimizer unpacks
+// bytes as soon as a load returns and carries the unpacked values across the pipeline, which spills).
 __device__ __forceinline__ void pin(uint32_t& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void pin(u32x2& v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void pin(u32x4& v) { asm volatile("" : "+v"(v)); }
 
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_add(float v) {
-    int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
-    return v + __int_as_float(t);
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
-// Sum over the 64 lanes of a wave; the total lands in lane 63.
-__device__ __forceinline__ float wave_sum_to_lane63(float v) {
-    v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
-    v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
-    v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
-    v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane of a 16-lane row holds the row sum
-    v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
-    v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+// All-reduce over the 16 lanes of a DPP row.
+__device__ __forceinline__ float slot_sum(float v) {
+    v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f<0x141>(v);  // row_half_mirror
+    v += dpp_f<0x140>(v);  // row_mirror
     return v;
 }
 
+// Three signed byte planes of a 24-bit fixed-point value: v = a*65536 + b*256 + c, a,b,c in [-127,127]
+// for |v| <= QMAX.
+constexpr float QMAX = 8355711.0f;  // 127*65536 + 127*256 + 127
+
+// exact integer plane sums -> f32 (the only rounding is the final add, 2^-24 relative)
+__device__ __forceinline__ float planes_to_f32(int a, int b, int c) { return fmaf((float)a, 65536.0f, (float)((b << 8) + c)); }
+
 // ------------------------------------------------------------------------------------------------
-// Per-format lane work. `setup` maps unit u of a row to byte offsets inside the row and to the four
-// runs of 8 activation columns the lane needs (x[m][8*j + i] = x[m, xo[j] + i]). `dot` returns the
-// lane's share of the dot product for M activation rows. sx[m][j] = sum_i x[m][8*j+i].
+// Per-format lane work. A unit is WPL weights of one row; RUN is the activation run that shares one
+// fixed-point scale (the format's own sub-block length); a lane needs NRUN runs.
+//   setup(u)  -> byte offsets of unit u inside a row and the indices of its activation runs
+//   load      -> the raw bytes of the unit for one row (16-/8-byte loads, 2-byte aligned where the
+//                GGUF layout is)
+//   dot<M>    -> the lane's share of the M dot products
+// xp[m][j][p][i]: plane p, dword i of run j;  xs[m][j]: scale of run j;  xsum[m][j]: sum of x over run j.
 // ------------------------------------------------------------------------------------------------
 
 struct Q4K {
-    // 144 B = [f16 d][f16 dmin][12 B packed 6-bit scales/mins][128 B nibbles]; every piece 16-byte aligned.
+    static constexpr int WPL = 64, RUN = 32, NRUN = 2, BLOCK_VALUES = 256;
     struct Lane { uint32_t off_h, off_q, sh; bool high; };
-    struct Data { u32x4 h, q; __device__ __forceinline__ void pin_all() { pin(h); pin(q); } };
-    static __device__ __forceinline__ void setup(int u, Lane& L, int (&xo)[4]) {
-        int b = u >> 3, p = u & 7, g = p >> 1, hf = p & 1;
+    struct Data {
+        u32x4 h, q0, q1;
+        __device__ __forceinline__ void pin_all() { pin(h); pin(q0); pin(q1); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        int b = u >> 2, g = u & 3;             // unit = group g of block b: qs[32g, 32g+32)
         L.off_h = b * 144;
-        L.off_q = b * 144 + 16 + 16 * p;  // qs[16p, 16p+16): group g, l in [16hf, 16hf+16)
+        L.off_q = b * 144 + 16 + 32 * g;
         L.sh = 16 * (g & 1);
         L.high = g >= 2;
-        int base = 256 * b + 64 * g + 16 * hf;
-        xo[0] = base; xo[1] = base + 8; xo[2] = base + 32; xo[3] = base + 40;  // low nibbles, then high nibbles
+        run[0] = 2 * u;                        // low nibbles  -> sub-block 2g   = columns [64u, 64u+32)
+        run[1] = 2 * u + 1;                    // high nibbles -> sub-block 2g+1 = columns [64u+32, 64u+64)
     }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
         Data d;
         d.h = *(const u32x4*)(row + L.off_h);
-        d.q = *(const u32x4*)(row + L.off_q);
+        d.q0 = *(const u32x4*)(row + L.off_q);
+        d.q1 = *(const u32x4*)(row + L.off_q + 16);
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const float (&x)[M][32], const float (&sx)[M][4],
-                                               float (&out)[M]) {
-        // (sc, m) of sub-blocks 2g and 2g+1 as two packed bytes each -- get_sc_min,
-        // crates/ferric-gguf/src/lib.rs:795-804, evaluated for a byte pair at once.
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
+        // 6-bit (scale, min) of sub-blocks 2g and 2g+1, two packed bytes each: get_sc_min,
+        // crates/ferric-gguf/src/lib.rs:795-804, for a byte pair at once
         uint32_t a = D.h[1] >> L.sh, b = D.h[2] >> L.sh, c = D.h[3] >> L.sh;
         uint32_t scp = L.high ? ((c & 0x0F0Fu) | ((a >> 2) & 0x3030u)) : (a & 0x3F3Fu);
         uint32_t mp = L.high ? (((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u)) : (b & 0x3F3Fu);
         float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
-        float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1) * 0.0625f;  // high nibbles are used as 16*n
-        float m0 = dmin * ub(mp, 0), m1 = dmin * ub(mp, 1);
-        float lo[M], hi[M];
-#pragma unroll
-        for (int m = 0; m < M; m++) { lo[m] = 0.f; hi[m] = 0.f; }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            uint32_t ql = D.q[i] & 0x0F0F0F0Fu, qh = D.q[i] & 0xF0F0F0F0u;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                float fl = ub(ql, k), fh = ub(qh, k);
-#pragma unroll
-                for (int m = 0; m < M; m++) {
-                    lo[m] = fmaf(x[m][4 * i + k], fl, lo[m]);
-                    hi[m] = fmaf(x[m][16 + 4 * i + k], fh, hi[m]);
-                }
-            }
-        }
+        float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1), m0 = dmin * ub(mp, 0), m1 = dmin * ub(mp, 1);
+        int acc[M][2][3];
 #pragma unroll
         for (int m = 0; m < M; m++)
-            out[m] = d0 * lo[m] - m0 * (sx[m][0] + sx[m][1]) + (d1 * hi[m] - m1 * (sx[m][2] + sx[m][3]));
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int p = 0; p < 3; p++) acc[m][j][p] = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t w = i < 4 ? D.q0[i] : D.q1[i - 4];
+            uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int p = 0; p < 3; p++) {
+                    acc[m][0][p] = dot4(xp[m][0][p][i], lo, acc[m][0][p]);
+                    acc[m][1][p] = dot4(xp[m][1][p][i], hi, acc[m][1][p]);
+                }
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            float f0 = xs[m][0] * planes_to_f32(acc[m][0][0], acc[m][0][1], acc[m][0][2]);
+            float f1 = xs[m][1] * planes_to_f32(acc[m][1][0], acc[m][1][1], acc[m][1][2]);
+            // sum_l x_l (d*sc*q_l - dmin*m) = d*sc * sum x_l q_l - dmin*m * sum x_l
+            out[m] = (d0 * f0 - m0 * xsum[m][0]) + (d1 * f1 - m1 * xsum[m][1]);
+        }
     }
 };
 
 struct Q6K {
-    // 210 B = [ql 128][qh 64][i8 sc 16][f16 d]; unit (hf, t): l in [8t, 8t+8) of half hf.
+    static constexpr int WPL = 64, RUN = 16, NRUN = 4, BLOCK_VALUES = 256;
     struct Lane { uint32_t off_a, off_h, off_s, off_d, ssh; };
-    struct Data { u32x2 a, b, h, s; uint32_t d; __device__ __forceinline__ void pin_all() { pin(a); pin(b); pin(h); pin(s); pin(d); } };
-    static __device__ __forceinline__ void setup(int u, Lane& L, int (&xo)[4]) {
-        int b = u >> 3, r = u & 7, hf = r >> 2, t = r & 3;
-        L.off_a = b * 210 + 64 * hf + 8 * t;
-        L.off_h = b * 210 + 128 + 32 * hf + 8 * t;
+    struct Data {
+        u32x4 a, b, h; u32x2 s; uint32_t d;
+        __device__ __forceinline__ void pin_all() { pin(a); pin(b); pin(h); pin(s); pin(d); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        int b = u >> 2, hf = (u >> 1) & 1, t = u & 1;   // unit: l in [16t, 16t+16) of half hf of block b
+        L.off_a = b * 210 + 64 * hf + 16 * t;           // ql[l], and ql[l+32] at +32
+        L.off_h = b * 210 + 128 + 32 * hf + 16 * t;
         L.off_s = b * 210 + 192 + 8 * hf;
         L.off_d = b * 210 + 208;
-        L.ssh = 8 * (t >> 1);  // is = l / 16
-        int base = 256 * b + 128 * hf + 8 * t;
-        xo[0] = base; xo[1] = base + 32; xo[2] = base + 64; xo[3] = base + 96;
+        L.ssh = 8 * t;                                  // is = l / 16 = t
+#pragma unroll
+        for (int g = 0; g < 4; g++) run[g] = 16 * b + 8 * hf + t + 2 * g;   // columns 256b + 128hf + 32g + 16t + [0,16)
     }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
         Data d;
-        d.a = ((const U2A2*)(row + L.off_a))->v;
-        d.b = ((const U2A2*)(row + L.off_a + 32))->v;
-        d.h = ((const U2A2*)(row + L.off_h))->v;
+        d.a = ((const U4A2*)(row + L.off_a))->v;
+        d.b = ((const U4A2*)(row + L.off_a + 32))->v;
+        d.h = ((const U4A2*)(row + L.off_h))->v;
         d.s = ((const U2A2*)(row + L.off_s))->v;
         d.d = *(const uint16_t*)(row + L.off_d);
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const float (&x)[M][32], const float (&sx)[M][4],
-                                               float (&out)[M]) {
-        float acc[M][4];
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
+        int acc[M][4][3];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) acc[m][j] = 0.f;
+            for (int g = 0; g < 4; g++)
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+                for (int p = 0; p < 3; p++) acc[m][g][p] = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
             uint32_t A = D.a[i], B = D.b[i], H = D.h[i];
-            // the four 6-bit quants that share byte l -- crates/ferric-gguf/src/lib.rs:733-736, four bytes at a time
+            // the four 6-bit quants that share byte l (crates/ferric-gguf/src/lib.rs:733-736), 4 bytes at a time, as 0..63
             uint32_t q[4];
             q[0] = (A & 0x0F0F0F0Fu) | ((H & 0x03030303u) << 4);
             q[1] = (B & 0x0F0F0F0Fu) | ((H & 0x0C0C0C0Cu) << 2);
             q[2] = ((A >> 4) & 0x0F0F0F0Fu) | (H & 0x30303030u);
             q[3] = ((B >> 4) & 0x0F0F0F0Fu) | ((H >> 2) & 0x30303030u);
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+            for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    float f = ub(q[j], k);
+                for (int g = 0; g < 4; g++)
 #pragma unroll
-                    for (int m = 0; m < M; m++) acc[m][j] = fmaf(x[m][8 * j + 4 * i + k], f, acc[m][j]);
-                }
+                    for (int p = 0; p < 3; p++) acc[m][g][p] = dot4(xp[m][g][p][i], q[g], acc[m][g][p]);
         }
         uint32_t s0 = D.s[0] >> L.ssh, s1 = D.s[1] >> L.ssh;  // sc[is], sc[is+2] | sc[is+4], sc[is+6]
-        float c0 = sb(s0, 0), c1 = sb(s0, 2), c2 = sb(s1, 0), c3 = sb(s1, 2);
+        float c[4] = {sb(s0, 0), sb(s0, 2), sb(s1, 0), sb(s1, 2)};
         float d = f16_bits(D.d);
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            // sum_l x*(q-32) = sum_l x*q - 32*sum_l x
-            float t = c0 * fmaf(-32.f, sx[m][0], acc[m][0]);
-            t = fmaf(c1, fmaf(-32.f, sx[m][1], acc[m][1]), t);
-            t = fmaf(c2, fmaf(-32.f, sx[m][2], acc[m][2]), t);
-            t = fmaf(c3, fmaf(-32.f, sx[m][3], acc[m][3]), t);
+            float t = 0.f;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float f = xs[m][g] * planes_to_f32(acc[m][g][0], acc[m][g][1], acc[m][g][2]);
+                t = fmaf(c[g], fmaf(-32.f, xsum[m][g], f), t);   // sum x*(q-32) = sum x*q - 32*sum x
+            }
             out[m] = d * t;
         }
     }
 };
 
 struct Q80 {
-    // 34 B = [f16 d][i8 q[32]]; one unit = one block.
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32;
     struct Lane { uint32_t off; };
-    struct Data { u32x4 q0, q1; uint32_t d; __device__ __forceinline__ void pin_all() { pin(q0); pin(q1); pin(d); } };
-    static __device__ __forceinline__ void setup(int u, Lane& L, int (&xo)[4]) {
+    struct Data {
+        u32x4 q0, q1; uint32_t d;
+        __device__ __forceinline__ void pin_all() { pin(q0); pin(q1); pin(d); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
         L.off = u * 34;
-        xo[0] = 32 * u; xo[1] = 32 * u + 8; xo[2] = 32 * u + 16; xo[3] = 32 * u + 24;
+        run[0] = u;
     }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
         Data d;
@@ -196,25 +228,25 @@ struct Q80 {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const float (&x)[M][32], const float (&)[M][4],
-                                               float (&out)[M]) {
-        float acc[M];
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&)[M][NRUN], float (&out)[M]) {
+        int acc[M][3];
 #pragma unroll
-        for (int m = 0; m < M; m++) acc[m] = 0.f;
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int p = 0; p < 3; p++) acc[m][p] = 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             uint32_t w = i < 4 ? D.q0[i] : D.q1[i - 4];
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                float f = sb(w, k);
+            for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int m = 0; m < M; m++) acc[m] = fmaf(x[m][4 * i + k], f, acc[m]);
-            }
+                for (int p = 0; p < 3; p++) acc[m][p] = dot4(xp[m][0][p][i], w, acc[m][p]);
         }
         float d = f16_bits(D.d);
         // per block: part = sum x*q, then part*d -- crates/ferric-tensor/src/cpu_simd.rs:66-70
 #pragma unroll
-        for (int m = 0; m < M; m++) out[m] = acc[m] * d;
+        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])) * d;
     }
 };
 
@@ -226,115 +258,183 @@ struct GemvParams {
     int cols;
     size_t row_bytes;
     size_t pair_bytes;   // fused SwiGLU: byte distance from gate row r to up row r (= n_ff * row_bytes)
-    int S, G, rpg;       // waves per row, row groups per workgroup, output rows per row group
-    int stage;           // 1: x staged through LDS once per workgroup
+    int NG;              // 16-lane slots per row = cols / (16 * WPL)
+    int RF;              // replicas of the full-wave set, each taking every RF-th row (balances them against the tail wave)
+    int G;               // row groups per workgroup
+    int rpg;             // output rows per row group
 };
 
-// Threads per workgroup allowed for M activation rows: the 32*M resident activation registers per
-// lane must fit the VGPR budget the launch bound implies (1024 threads -> 128, 768 -> 168, 512 -> 256).
-constexpr int max_threads(int M) { return M == 1 ? 1024 : M == 2 ? 768 : 512; }
-// Rows in flight per wave: 4 at batch 1, 2 when the batch already fills the register file.
-constexpr int rows_in_flight(int M) { return M == 1 ? 4 : 2; }
+// Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 768 -> 168, 512 -> 256).
+constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
+// Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit that budget.
+template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? (F::WPL == 64 ? (F::RUN == 16 ? 2 : 3) : 4) : 2; }
+// Activation rows one pass can hold in registers (48 plane dwords per row for the 64-weight units, 24 for Q8_0).
+template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
 
 template <class F, int M, int U, bool SWIGLU>
-__global__ void __launch_bounds__(max_threads(M)) gemv_kernel(GemvParams p) {
-    extern __shared__ float smem[];
-    constexpr int VPR = SWIGLU ? 2 : 1;  // weight rows walked per output row
+__global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int VPR = SWIGLU ? 2 : 1;       // weight rows walked per output row
+    constexpr int RUN = F::RUN, NRUN = F::NRUN, RD = RUN / 4;
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps row pointers and loop control scalar
-    const int ks = wave % p.S, rg = wave / p.S;
-    float* part = smem + (p.stage ? M * p.cols : 0);  // [G][rpg*VPR][S][M]
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int NGF = p.NG >> 2, NT = p.NG & 3, NFW = NGF * p.RF, WPR = NFW + (NT ? 1 : 0);
+    const int wr = wave % WPR, rg = wave / WPR;          // wave within row group, row group within workgroup
+    const bool tail = wr == NFW;                         // wave-uniform
+    const int RT = tail ? (NT == 1 ? 4 : NT == 2 ? 2 : 1) : 1;   // rows this wave works on at once
+    // iteration i of this wave works on virtual row v_start + i * v_step (+ row_off per lane in a tail wave)
+    const int v_start = tail ? 0 : wr / NGF, v_step = tail ? RT : p.RF;
 
-    const int units = p.cols >> 5;
-    const int u = ks * 64 + lane;
-    const bool valid = u < units;
+    // LDS: activation planes [M][cols/RUN][3][RUN] bytes | scales [M][cols/RUN] | sums [M][cols/RUN] | partials
+    const int nrun = p.cols / RUN;
+    uint8_t* planes = smem;
+    float* scales = (float*)(smem + (size_t)M * p.cols * 3);
+    float* sums = scales + (size_t)M * nrun;
+    float* part = sums + (size_t)M * nrun;               // [G][rpg*VPR][NG][M]
+
+    // ---- which unit of which row this lane works on
+    const int slot = lane >> 4, l16 = lane & 15;
+    int group, row_off;
+    bool lane_ok = true;
+    if (!tail) { group = 4 * (wr % NGF) + slot; row_off = 0; }
+    else if (NT == 3) { lane_ok = slot < 3; group = 4 * NGF + (lane_ok ? slot : 0); row_off = 0; }
+    else { group = 4 * NGF + (NT == 2 ? (slot & 1) : 0); row_off = NT == 2 ? (slot >> 1) : slot; }
     typename F::Lane L;
-    int xo[4];
-    F::setup(valid ? u : 0, L, xo);
+    int run[NRUN];
+    F::setup(group * 16 + l16, L, run);
 
-    // ---- activations: 32 columns per lane, resident in registers for the life of the wave
-    float x[M][32], sx[M][4];
-    if (p.stage) {
-        for (int i = tid * 4; i < M * p.cols; i += blockDim.x * 4) *(float4*)(smem + i) = *(const float4*)(p.x + i);
-        __syncthreads();
-#pragma unroll
-        for (int m = 0; m < M; m++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                float4 a = *(const float4*)(smem + m * p.cols + xo[j]), b = *(const float4*)(smem + m * p.cols + xo[j] + 4);
-                x[m][8 * j + 0] = a.x; x[m][8 * j + 1] = a.y; x[m][8 * j + 2] = a.z; x[m][8 * j + 3] = a.w;
-                x[m][8 * j + 4] = b.x; x[m][8 * j + 5] = b.y; x[m][8 * j + 6] = b.z; x[m][8 * j + 7] = b.w;
-            }
-    } else {
-#pragma unroll
-        for (int m = 0; m < M; m++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                float4 a = *(const float4*)(p.x + (size_t)m * p.cols + xo[j]), b = *(const float4*)(p.x + (size_t)m * p.cols + xo[j] + 4);
-                x[m][8 * j + 0] = a.x; x[m][8 * j + 1] = a.y; x[m][8 * j + 2] = a.z; x[m][8 * j + 3] = a.w;
-                x[m][8 * j + 4] = b.x; x[m][8 * j + 5] = b.y; x[m][8 * j + 6] = b.z; x[m][8 * j + 7] = b.w;
-            }
-    }
-#pragma unroll
-    for (int m = 0; m < M; m++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float s = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) s += x[m][8 * j + i];
-            sx[m][j] = s;
-        }
-
-    // ---- stream the rows of this row group: virtual row v -> weight row r0 + v/VPR (+ pair for odd v)
     const int r0 = (blockIdx.x * p.G + rg) * p.rpg;
     int nrows = p.out_rows - r0;
     nrows = nrows < 0 ? 0 : (nrows > p.rpg ? p.rpg : nrows);
-    const int nv = nrows * VPR;
+    const int nv = nrows * VPR;                          // virtual rows: v -> weight row r0 + v/VPR (+ pair for odd v)
     const uint8_t* base = p.W + (size_t)r0 * p.row_bytes;
-    auto row_ptr = [&](int v) -> const uint8_t* {
+    const int n_it = nv > v_start ? (nv - v_start + v_step - 1) / v_step : 0;
+    auto row_ptr = [&](int it) -> const uint8_t* {
+        int v = v_start + it * v_step + row_off;
+        v = v < nv ? v : nv - 1;                         // lanes past the end re-read the last row; they are masked below
         return SWIGLU ? base + (size_t)(v >> 1) * p.row_bytes + (size_t)(v & 1) * p.pair_bytes : base + (size_t)v * p.row_bytes;
     };
-    float* mypart = part + ((size_t)rg * p.rpg * VPR * p.S + ks) * M;
 
+    // ---- weight bytes of the first U iterations go in flight before the activations are touched
     typename F::Data buf[U];
 #pragma unroll
     for (int j = 0; j < U; j++)
-        if (j < nv) buf[j] = F::load(row_ptr(j), L);
-#pragma unroll 1
-    for (int v = 0; v < nv; v += U) {
-#pragma unroll
-        for (int j = 0; j < U; j++) {
-            if (v + j < nv) {
-                typename F::Data cur = buf[j];
-                if (v + j + U < nv) buf[j] = F::load(row_ptr(v + j + U), L);
-                cur.pin_all();
-                float acc[M];
-                F::template dot<M>(cur, L, x, sx, acc);
-#pragma unroll
-                for (int m = 0; m < M; m++) {
-                    float t = wave_sum_to_lane63(valid ? acc[m] : 0.f);
-                    if (lane == 63) mypart[(size_t)(v + j) * p.S * M + m] = t;
-                }
-            }
+        if (j < n_it) buf[j] = F::load(row_ptr(j), L);
+
+    // ---- activations -> 24-bit block fixed point, once per workgroup, through LDS
+    for (int e = tid * 8; e < M * p.cols; e += blockDim.x * 8) {
+        float4 a = *(const float4*)(p.x + e), b = *(const float4*)(p.x + e + 4);
+        float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        float amax = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
+                           fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
+        float sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+        amax = fmaxf(amax, dpp_f<0xB1>(amax));           // the 2 (RUN 16) or 4 (RUN 32) lanes of a run sit in one quad
+        sum += dpp_f<0xB1>(sum);
+        if (RUN == 32) {
+            amax = fmaxf(amax, dpp_f<0x4E>(amax));
+            sum += dpp_f<0x4E>(sum);
         }
+        float inv = amax > 0.f ? QMAX / amax : 0.f;
+        uint32_t pl[3][2] = {{0, 0}, {0, 0}, {0, 0}};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            int q = __float2int_rn(v[i] * inv);
+            q = q > (int)QMAX ? (int)QMAX : (q < -(int)QMAX ? -(int)QMAX : q);   // rounding of v*inv may overshoot by one
+            int c = (q << 24) >> 24;
+            int q1 = (q - c) >> 8;
+            int b8 = (q1 << 24) >> 24;
+            int a8 = (q1 - b8) >> 8;
+            pl[0][i >> 2] |= (uint32_t)(a8 & 0xFF) << (8 * (i & 3));
+            pl[1][i >> 2] |= (uint32_t)(b8 & 0xFF) << (8 * (i & 3));
+            pl[2][i >> 2] |= (uint32_t)(c & 0xFF) << (8 * (i & 3));
+        }
+        int r = e / RUN, within = e % RUN;               // run index counts across the M activation rows
+#pragma unroll
+        for (int pp = 0; pp < 3; pp++) *(u32x2*)(planes + ((size_t)r * 3 + pp) * RUN + within) = u32x2{pl[pp][0], pl[pp][1]};
+        if (within == 0) { scales[r] = amax / QMAX; sums[r] = sum; }
     }
     __syncthreads();
 
-    // ---- combine the S partials of each output in a fixed order, apply SwiGLU, store
+    uint32_t xp[M][NRUN][3][RD];
+    float xs[M][NRUN], xsum[M][NRUN];
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int j = 0; j < NRUN; j++) {
+            int r = m * nrun + run[j];
+            xs[m][j] = scales[r];
+            xsum[m][j] = sums[r];
+#pragma unroll
+            for (int pp = 0; pp < 3; pp++)
+#pragma unroll
+                for (int i = 0; i < RD; i += 4) {
+                    u32x4 t = *(const u32x4*)(planes + ((size_t)r * 3 + pp) * RUN + 4 * i);
+                    xp[m][j][pp][i] = t[0]; xp[m][j][pp][i + 1] = t[1]; xp[m][j][pp][i + 2] = t[2]; xp[m][j][pp][i + 3] = t[3];
+                }
+        }
+
+    // ---- stream the rows. Software pipeline over the U row buffers, written so that the steady-state
+    // loop has no conditional reload: a reload under a condition makes the loop-carried buffers phi
+    // nodes whose copies wait for every outstanding load at the back edge, which serialises the stream.
+    float* mypart = part + (size_t)rg * p.rpg * VPR * p.NG * M;
+    auto consume = [&](typename F::Data& cur, int it) {
+        cur.pin_all();
+        float acc[M];
+        F::template dot<M>(cur, L, xp, xs, xsum, acc);
+        const int v = v_start + it * v_step + row_off;
+        const bool ok = lane_ok && v < nv;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            float t = slot_sum(acc[m]);
+            if (ok && l16 == 0) mypart[((size_t)v * p.NG + group) * M + m] = t;
+        }
+    };
+    int i0 = 0;
+    // All prologue loads have landed by now (they overlapped the activation quantisation). Saying so
+    // explicitly gives the compiler's wait-count tracking a clean state at the loop head; without it the
+    // merge of the prologue's load order with the loop's makes every iteration wait for vmcnt(0).
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt/lgkmcnt untouched
+#pragma unroll 1
+    for (; i0 + 2 * U <= n_it; i0 += U) {        // every row of this step and of the next one exists
+#pragma unroll
+        for (int j = 0; j < U; j++) {
+            // consume, then refill the same registers: the old bytes are dead when the new load is issued,
+            // so the loop-carried buffer needs no copy (and no wait) at the back edge
+            consume(buf[j], i0 + j);
+            buf[j] = F::load(row_ptr(i0 + j + U), L);
+        }
+    }
+    // drain, step A: iterations [i0, i0+U) that exist, reloading what is left of the step after it
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+        const int it = i0 + j;
+        if (it < n_it) {
+            consume(buf[j], it);
+            if (it + U < n_it) buf[j] = F::load(row_ptr(it + U), L);
+        }
+    }
+    // drain, step B: iterations [i0+U, n_it)
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+        const int it = i0 + U + j;
+        if (it < n_it) consume(buf[j], it);
+    }
+    __syncthreads();
+
+    // ---- add the NG slot partials of each output in a fixed order, apply SwiGLU, store
     const int per_wg = p.G * p.rpg;
     for (int i = tid; i < per_wg * M; i += blockDim.x) {
-        int m = i / per_wg, rr = i % per_wg;  // consecutive threads -> consecutive output rows
+        int m = i / per_wg, rr = i % per_wg;             // consecutive threads -> consecutive output rows
         int g = rr / p.rpg, rl = rr % p.rpg;
         int r = (blockIdx.x * p.G + g) * p.rpg + rl;
         if (r >= p.out_rows) continue;
-        const float* q = part + (((size_t)g * p.rpg + rl) * VPR * p.S) * M + m;
+        const float* q = part + (((size_t)g * p.rpg + rl) * VPR * p.NG) * M + m;
         float a = 0.f;
-        for (int s = 0; s < p.S; s++) a += q[s * M];
+        for (int s = 0; s < p.NG; s++) a += q[s * M];
         if (SWIGLU) {
             float b = 0.f;
-            for (int s = 0; s < p.S; s++) b += q[(p.S + s) * M];
-            // silu(g) * u, crates/ferric-tensor/src/dtype.rs:2408
-            a = (a / (1.0f + expf(-a))) * b;
+            for (int s = 0; s < p.NG; s++) b += q[(p.NG + s) * M];
+            a = (a / (1.0f + expf(-a))) * b;             // silu(gate) * up, crates/ferric-tensor/src/dtype.rs:2408
         }
         p.y[(size_t)m * p.out_rows + r] = a;
     }
@@ -359,56 +459,98 @@ int env_int(const char* name, int dflt) {
     return v && *v ? atoi(v) : dflt;
 }
 
+// The tail wave of a row group works on 4 (NG%4 == 1) or 2 (NG%4 == 2) rows per iteration while a full
+// wave works on one; replicating the full-wave set RF times, each replica taking every RF-th row, evens
+// the iteration counts out (K = 5120: 4 full waves + 1 tail wave, one iteration each per 4 rows).
+int full_wave_replicas(int NG, int maxw) {
+    const int NGF = NG / 4, NT = NG % 4;
+    if (NGF == 0 || NT == 0 || NT == 3) return 1;
+    int rf = NT == 1 ? 4 : 2;
+    while (rf > 1 && NGF * rf + 1 > maxw) rf /= 2;
+    return rf;
+}
+int waves_per_row_group(int NG, int maxw) { return (NG / 4) * full_wave_replicas(NG, maxw) + (NG % 4 ? 1 : 0); }
+
+template <class F, int M, bool SWIGLU>
+size_t lds_bytes(size_t cols, int NG, int G, int rpg) {
+    return M * cols * 3 + 2 * M * (cols / F::RUN) * sizeof(float) + (size_t)G * rpg * (SWIGLU ? 2 : 1) * NG * M * sizeof(float);
+}
+
 template <class F, int M, bool SWIGLU>
 int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s) {
-    static const int tune_g = env_int("FHIP_GEMV_G", 0), tune_rpg = env_int("FHIP_GEMV_RPG", 0), tune_u = env_int("FHIP_GEMV_U", 0);
+    static const int tune_g = env_int("FHIP_GEMV_G", 0), tune_rpg = env_int("FHIP_GEMV_RPG", 0);
+    constexpr int U = rows_in_flight<F>(M);
+    auto kernel = gemv_stream_kernel<F, M, U, SWIGLU>;
+    static bool lds_raised = false;
+    if (!lds_raised) {  // workgroups may use more than the default 64 KiB of the CU's 160 KiB
+        (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fhip::device_lds_bytes());
+        (void)hipGetLastError();
+        lds_raised = true;
+    }
     GemvParams p;
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
     p.pair_bytes = SWIGLU ? out_rows * w->row_bytes : 0;
-    const int units = (int)(w->cols / 32);
-    p.S = (units + 63) / 64;
+    p.NG = (int)(w->cols / (16 * F::WPL));
     constexpr int MAXW = max_threads(M) / 64;
-    if (p.S > MAXW) return fhip::set_error(FHIP_ERR_SHAPE, "matmul_q: cols %zu exceeds the %d this kernel covers", w->cols, MAXW * 2048);
-    // Row groups per workgroup: fill the workgroup with waves.
-    int G = tune_g > 0 ? tune_g : MAXW / p.S;
-    if (G < 1) G = 1;
-    while (G > 1 && p.S * G > MAXW) G--;
-    p.stage = (size_t)M * w->cols * 4 <= 48 * 1024 ? 1 : 0;
-    p.G = G;
-    // Rows per row group: enough workgroups to spread over every CU several times, but at least a
-    // few rows per wave so the one-time activation load is amortised.
+    p.RF = full_wave_replicas(p.NG, MAXW);
+    const int WPR = waves_per_row_group(p.NG, MAXW);
+    // Rows per row group (rpg) and row groups per workgroup (G). A CU holds Gcap row groups at once
+    // (one workgroup of MAXW waves), the chip cus*Gcap; row groups of rpg rows are dealt out in rounds,
+    // so the run takes about rounds*rpg row times: minimise that, preferring more rows per activation
+    // load on a tie. With a single, partly filled round the row groups are spread over all CUs.
     const int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    int rpg = tune_rpg > 0 ? tune_rpg : (int)((out_rows + (size_t)cus * G - 1) / ((size_t)cus * G));
-    if (tune_rpg <= 0) {
-        if (rpg > 32) rpg = 32;
-        if (rpg < 1) rpg = 1;
+    int Gcap = MAXW / WPR;
+    if (Gcap < 1) Gcap = 1;
+    int rpg = 1;
+    size_t best = ~(size_t)0;
+    for (int r = 1; r <= 32; r++) {
+        size_t nrg = (out_rows + r - 1) / r;
+        size_t rounds = (nrg + (size_t)cus * Gcap - 1) / ((size_t)cus * Gcap);
+        if (rounds * r <= best) { best = rounds * r; rpg = r; }
     }
-    p.rpg = rpg;
+    const size_t nrg = (out_rows + rpg - 1) / rpg;
+    int G = nrg >= (size_t)cus * Gcap ? Gcap : (int)((nrg + cus - 1) / cus);
+    if (tune_g > 0) G = tune_g;
+    if (tune_rpg > 0) rpg = tune_rpg;
+    p.G = G; p.rpg = rpg;
     const size_t per_wg = (size_t)G * rpg;
     const size_t grid = (out_rows + per_wg - 1) / per_wg;
-    const size_t lds = ((p.stage ? (size_t)M * w->cols : 0) + per_wg * (SWIGLU ? 2 : 1) * p.S * M) * sizeof(float);
-    if (lds > 64 * 1024) return fhip::set_error(FHIP_ERR_SHAPE, "matmul_q: LDS budget exceeded (%zu B)", lds);
-    dim3 block(64 * p.S * G);
-    constexpr int U = rows_in_flight(M);
-    if (tune_u == 2 && U != 2) hipLaunchKernelGGL((gemv_kernel<F, M, 2, SWIGLU>), dim3((unsigned)grid), block, lds, s, p);
-    else hipLaunchKernelGGL((gemv_kernel<F, M, U, SWIGLU>), dim3((unsigned)grid), block, lds, s, p);
+    const size_t lds = lds_bytes<F, M, SWIGLU>(w->cols, p.NG, G, rpg);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * WPR * G), lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
 }
 
+// Largest batch width (4, 2, 1, or 0 = shape not covered) whose workgroup fits the wave and LDS limits.
 template <class F, bool SWIGLU>
-int launch_fmt(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t out_rows, hipStream_t s) {
+int max_batch(const fhip_weight* w, size_t left) {
+    if (w->cols % (16 * F::WPL) != 0) return 0;
+    const int NG = (int)(w->cols / (16 * F::WPL));
+    auto WPRm = [&](int m) { return waves_per_row_group(NG, max_threads(m) / 64); };
+    const size_t cap = fhip::device_lds_bytes();
+    if (left >= 4 && max_m<F>() >= 4 && WPRm(4) * 64 <= max_threads(4) && lds_bytes<F, 4, SWIGLU>(w->cols, NG, 1, 32) <= cap) return 4;
+    if (left >= 2 && WPRm(2) * 64 <= max_threads(2) && lds_bytes<F, 2, SWIGLU>(w->cols, NG, 1, 32) <= cap) return 2;
+    if (WPRm(1) * 64 <= max_threads(1) && lds_bytes<F, 1, SWIGLU>(w->cols, NG, 1, 32) <= cap) return 1;
+    return 0;
+}
+
+template <class F, bool SWIGLU>
+int launch_fmt(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t out_rows, size_t n_ff, hipStream_t s) {
+    // The kernel choice depends on the weight's shape only, never on the batch, so a row of a batch
+    // result is bit-identical to the same row computed alone.
+    if (max_batch<F, SWIGLU>(w, 1) == 0) return fhip::launch_gemv_generic(w, d_x, rows_x, d_y, n_ff, s);
     size_t m0 = 0;
     while (m0 < rows_x) {
-        size_t left = rows_x - m0;
         const float* x = d_x + m0 * w->cols;
         float* y = d_y + m0 * out_rows;
-        int rc;
-        const size_t waves_per_row = (w->cols / 32 + 63) / 64;
-        if (left >= 4 && waves_per_row * 64 <= (size_t)max_threads(4)) { rc = launch_one<F, 4, SWIGLU>(w, x, y, out_rows, s); m0 += 4; }
-        else if (left >= 2 && waves_per_row * 64 <= (size_t)max_threads(2)) { rc = launch_one<F, 2, SWIGLU>(w, x, y, out_rows, s); m0 += 2; }
-        else { rc = launch_one<F, 1, SWIGLU>(w, x, y, out_rows, s); m0 += 1; }
+        int mb = max_batch<F, SWIGLU>(w, rows_x - m0), rc;
+        if constexpr (max_m<F>() >= 4) {
+            if (mb == 4) { rc = launch_one<F, 4, SWIGLU>(w, x, y, out_rows, s); if (rc != FHIP_OK) return rc; m0 += 4; continue; }
+        }
+        if (mb == 2) rc = launch_one<F, 2, SWIGLU>(w, x, y, out_rows, s);
+        else rc = launch_one<F, 1, SWIGLU>(w, x, y, out_rows, s);
         if (rc != FHIP_OK) return rc;
+        m0 += mb;
     }
     return FHIP_OK;
 }
@@ -419,21 +561,19 @@ namespace fhip {
 
 int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s) {
     if (w->rows == 0 || rows_x == 0) return FHIP_OK;
+    const size_t out_rows = n_ff ? n_ff : w->rows;
     if (w->cols == 0) {  // empty inner dimension: every dot product is 0 (and silu(0)*0 = 0)
-        size_t n = rows_x * (n_ff ? n_ff : w->rows);
+        size_t n = rows_x * out_rows;
         hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
         return check_hip(hipGetLastError(), "zero launch");
     }
-    // NOTE: y rows of different activation rows are written by different launches when rows_x > 4;
-    // each launch writes its own [m0, m0+M) slice of y with row stride out_rows.
-    const size_t out_rows = n_ff ? n_ff : w->rows;
-    // y is [rows_x, out_rows]: a batch slice starting at m0 is contiguous, so slicing by pointer is exact.
+    // y is [rows_x, out_rows]: a batch slice starting at row m0 is contiguous, so slicing by pointer is exact.
     switch (w->type) {
-        case FHIP_Q4_K: return n_ff ? launch_fmt<Q4K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_fmt<Q4K, false>(w, d_x, rows_x, d_y, out_rows, s);
-        case FHIP_Q6_K: return n_ff ? launch_fmt<Q6K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_fmt<Q6K, false>(w, d_x, rows_x, d_y, out_rows, s);
+        case FHIP_Q4_K: return n_ff ? launch_fmt<Q4K, true>(w, d_x, rows_x, d_y, out_rows, n_ff, s) : launch_fmt<Q4K, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+        case FHIP_Q6_K: return n_ff ? launch_fmt<Q6K, true>(w, d_x, rows_x, d_y, out_rows, n_ff, s) : launch_fmt<Q6K, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
         case FHIP_Q8_0:
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for Q8_0");
-            return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, s);
+            return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }
