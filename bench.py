@@ -155,6 +155,29 @@ def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
                       "ops still execute in stream order"}
 
 
+def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
+    """configs[3]: W 5120x5120 Q4_K, X [T, 5120] bf16 -> f32 [T, 5120] on the matrix cores."""
+    from ferric_amd.synth import synth_weights
+    n = k = 5120
+    qm = F.QMatrix.from_bytes(synth_weights(Q4_K, n, k, 1), Q4_K, n, k)
+    res = {}
+    for t in ts:
+        xf = np.random.default_rng(7).standard_normal((t, k)).astype(np.float32)
+        u = xf.view(np.uint32).astype(np.uint64)
+        xb = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+        x = F.Tensor.from_bf16_bits(xb, (t, k))
+        y = F.Tensor.empty((t, n))
+        g = F.Graph.begin(stream)
+        for _ in range(reps):
+            check(lib.fhip_gemm_q_bf16(qm.handle, x.buf.ptr, t, y.buf.ptr, stream.handle))
+        g.end()
+        g.launch()
+        ms = timer.time_ms(g.launch) / reps
+        tf = 2.0 * t * n * k / (ms * 1e-3) / 1e12
+        res[str(t)] = {"ms": ms, "TFLOPs": tf, "frac_of_bf16_mfma_peak": tf / 2500.0}
+    return res
+
+
 def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
     """The reference's CPU route for Q4_K (deq_raw then a sequential f32 dot per row, rows split in
     contiguous spans over threads), timed through the C oracle on this host's cores."""
@@ -188,6 +211,7 @@ def main():
     ap.add_argument("--no-ffn", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-q8", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, not code")
@@ -228,6 +252,9 @@ def main():
         log("[bench] Q4_K_M FFN block, batch 1/4/8 ...")
         ffn, wb = bench_ffn(F, lib, check, stream, timer, (1, 4, 8))
         line["ffn_q4k_q6k"] = {"weight_bytes": wb, "batch": ffn}
+    if not args.no_prefill:
+        log("[bench] prefill dequant-GEMM, T = 128/512/2048 ...")
+        line["prefill_q4k_5120_bf16_mfma"] = bench_prefill(F, lib, check, stream, timer)
     if not args.no_sweep:
         log("[bench] 64-layer decode weight sweep (14.0 GB) ...")
         line["decode_sweep"] = bench_sweep(F, lib, check, stream, timer)
