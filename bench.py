@@ -26,6 +26,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+# HBM bytes per launch of the headline kernel from hardware counters (FETCH_SIZE * 1.99976 + WRITE_SIZE * 1.0, both
+# calibrated on a 256 MiB copy); source and commands: profiles/gemv_hbm_traffic_pmc.txt
+Q4K_5120_TRAFFIC_BYTES = 15098461
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 
 
@@ -79,7 +82,7 @@ def gemv_graph(F, lib, check, stream, weights, x, y, steps, swiglu=False):
     return g.end()
 
 
-def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed, x_seed, ncopy):
+def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed, x_seed, ncopy, cold_only=False):
     from ferric_amd.synth import synth_weights
     nbytes = weight_bytes(ty, rows, cols)
     host = synth_weights(ty, rows, cols, seed)
@@ -89,7 +92,7 @@ def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed
     y = F.Tensor.empty((1, rows))
     alg = nbytes + 4 * cols + 4 * rows
     out = {}
-    for name, wl in (("cold", ws), ("warm", ws[:1])):
+    for name, wl in ((("cold", ws),) if cold_only else (("cold", ws), ("warm", ws[:1]))):
         gw = gemv_graph(F, lib, check, stream, wl, x, y, max(warmup, 1))
         g = gemv_graph(F, lib, check, stream, wl, x, y, steps)
         gw.launch()
@@ -178,6 +181,31 @@ def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
     return res
 
 
+def probe(F, lib, check):
+    """Work for a hardware-counter run: a copy of known size to calibrate FETCH_SIZE / WRITE_SIZE, then the
+    kernels of interest on weights no earlier launch has touched."""
+    from ferric_amd.synth import synth_weights
+    n = 256 << 20
+    src, dst = F.DeviceBuffer(n), F.DeviceBuffer(n)
+    check(lib.fhip_memset(src.ptr, 1, n, None))
+    check(lib.fhip_stream_sync(None))
+    check(lib.fhip_memcpy_d2d(dst.ptr, src.ptr, n, None))          # calibration dispatch: reads n, writes n
+    check(lib.fhip_stream_sync(None))
+    host = synth_weights(Q4_K, 5120, 5120, 1)
+    buf = replicate(F, lib, check, host, 48)
+    ws = [F.QMatrix.wrap_device(buf, host.size, Q4_K, 5120, 5120, offset=i * host.size) for i in range(48)]
+    x = F.Tensor.from_vec(np.random.default_rng(2).standard_normal(5120).astype(np.float32), (1, 5120))
+    y = F.Tensor.empty((1, 34816))
+    for i in range(32, 48):                                         # the last copies written are the least likely to sit in a cache
+        check(lib.fhip_matmul_q(ws[i].handle, x.buf.ptr, 1, y.buf.ptr, None))
+    gu = F.QMatrix.from_bytes(synth_weights(Q4_K, 34816, 5120, 3), Q4_K, 34816, 5120)
+    dn = F.QMatrix.from_bytes(synth_weights(Q6_K, 5120, 17408, 4), Q6_K, 5120, 17408)
+    h = F.Tensor.from_vec(np.random.default_rng(3).standard_normal(17408).astype(np.float32), (1, 17408))
+    check(lib.fhip_matmul_q_swiglu(gu.handle, x.buf.ptr, 1, y.buf.ptr, None))
+    check(lib.fhip_matmul_q(dn.handle, h.buf.ptr, 1, y.buf.ptr, None))
+    check(lib.fhip_stream_sync(None))
+
+
 def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
     """The reference's CPU route for Q4_K (deq_raw then a sequential f32 dot per row, rows split in
     contiguous spans over threads), timed through the C oracle on this host's cores."""
@@ -212,6 +240,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-q8", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="only the cold-rotation Q4_K 5120x5120 GEMV loop (what `value` is computed from); for profiling")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter probe for rocprofv3 --pmc: one 256 MiB device copy (calibration), then 16 cold Q4_K 5120x5120 "
+                         "GEMVs, one fused gate|up 34816x5120 and one Q6_K 5120x17408 GEMV; prints nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, not code")
@@ -224,8 +257,15 @@ def main():
     timer = Timer(lib, check, stream)
 
     rows = cols = 5120
+    if args.probe:
+        probe(F, lib, check)
+        return
     log("[bench] Q4_K GEMV 5120x5120 ...")
-    c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64)
+    c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
+                                 cold_only=args.headline_only)
+    if args.headline_only:
+        args.no_q8 = args.no_ffn = args.no_prefill = args.no_sweep = args.no_cpu = True
+        c2["warm"] = None
     ms_step = c2["cold"]["ms_per_step"]
     value = c2["cold"]["GBps"]
     line = {
@@ -239,8 +279,8 @@ def main():
         "pct_of_peak": 100.0 * value / HBM_PEAK_GBPS,
         "warm_single_copy": c2["warm"],
         "roofline": {"bound": "hbm", "achieved": alg / (ms_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
-                     "kernel": "gemv_kernel<Q4K, M=1>", "algorithmic_bytes_per_launch": alg,
+                     "frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": Q4K_5120_TRAFFIC_BYTES,
+                     "kernel": "gemv_stream_kernel<Q4K, M=1, U=3>", "algorithmic_bytes_per_launch": alg,
                      "launch_us": ms_step * 1e3},
     }
     if not args.no_q8:

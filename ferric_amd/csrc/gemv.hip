@@ -42,6 +42,13 @@ __device__ __forceinline__ float f16_bits(uint32_t b) { return __half2float(__us
 __device__ __forceinline__ float ub(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ float sb(uint32_t v, int k) { return (float)(int8_t)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
+__device__ __forceinline__ int udot4(uint32_t a, uint32_t b, int c) { return (int)__builtin_amdgcn_udot4(a, b, (uint32_t)c, false); }
+// Plane p of a run times 4 weight bytes. Plane 0 holds signed digits. Planes 1 and 2 hold unsigned bytes
+// when the weights are non-negative codes (K-quants) and signed balanced digits when they are int8 (Q8_0).
+template <bool SIGNED_W>
+__device__ __forceinline__ int pdot(int p, uint32_t x, uint32_t w, int acc) {
+    return (SIGNED_W || p == 0) ? dot4(x, w, acc) : udot4(x, w, acc);
+}
 
 // Keeps a prefetched row as the packed dwords that were loaded (otherwise the optimizer unpacks
 // bytes as soon as a load returns and carries the unpacked values across the pipeline, which spills).
@@ -62,9 +69,10 @@ __device__ __forceinline__ float slot_sum(float v) {
     return v;
 }
 
-// Three signed byte planes of a 24-bit fixed-point value: v = a*65536 + b*256 + c, a,b,c in [-127,127]
-// for |v| <= QMAX.
-constexpr float QMAX = 8355711.0f;  // 127*65536 + 127*256 + 127
+// A 24-bit fixed-point value v = a*65536 + b*256 + c as three byte planes, in one of two digit systems:
+//   unsigned low digits: a = v >> 16 (signed), b, c = the low bytes of v, |v| <= 2^23 - 1   (weights >= 0)
+//   balanced digits:     a, b, c in [-127, 127], |v| <= 127*65536 + 127*256 + 127             (int8 weights)
+constexpr float QMAX_U = 8388607.0f, QMAX_S = 8355711.0f;
 
 // exact integer plane sums -> f32 (the only rounding is the final add, 2^-24 relative)
 __device__ __forceinline__ float planes_to_f32(int a, int b, int c) { return fmaf((float)a, 65536.0f, (float)((b << 8) + c)); }
@@ -81,7 +89,8 @@ __device__ __forceinline__ float planes_to_f32(int a, int b, int c) { return fma
 
 struct Q4K {
     static constexpr int WPL = 64, RUN = 32, NRUN = 2, BLOCK_VALUES = 256;
-    struct Lane { uint32_t off_h, off_q, sh; bool high; };
+    static constexpr bool SIGNED_W = false;
+    struct Lane { uint32_t off_h, off_q, sh, m1, m2, m3; };
     struct Data {
         u32x4 h, q0, q1;
         __device__ __forceinline__ void pin_all() { pin(h); pin(q0); pin(q1); }
@@ -91,25 +100,28 @@ struct Q4K {
         L.off_h = b * 144;
         L.off_q = b * 144 + 16 + 32 * g;
         L.sh = 16 * (g & 1);
-        L.high = g >= 2;
+        // get_sc_min (crates/ferric-gguf/src/lib.rs:795-804) for the byte pair (2g, 2g+1), as masks so both
+        // branches are one expression: g < 2 -> s & 63; g >= 2 -> (s' & 15) | ((s >> 6) << 4)
+        L.m1 = g >= 2 ? 0u : 0x3F3Fu;
+        L.m2 = g >= 2 ? 0x0F0Fu : 0u;
+        L.m3 = g >= 2 ? 0x3030u : 0u;
         run[0] = 2 * u;                        // low nibbles  -> sub-block 2g   = columns [64u, 64u+32)
         run[1] = 2 * u + 1;                    // high nibbles -> sub-block 2g+1 = columns [64u+32, 64u+64)
     }
-    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
-        d.h = *(const u32x4*)(row + L.off_h);
-        d.q0 = *(const u32x4*)(row + L.off_q);
-        d.q1 = *(const u32x4*)(row + L.off_q + 16);
+        d.h = *(const u32x4*)(row + (L.off_h + eo));
+        d.q0 = *(const u32x4*)(row + (L.off_q + eo));
+        d.q1 = *(const u32x4*)(row + (L.off_q + eo) + 16);
         return d;
     }
     template <int M>
     static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
                                                const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
-        // 6-bit (scale, min) of sub-blocks 2g and 2g+1, two packed bytes each: get_sc_min,
-        // crates/ferric-gguf/src/lib.rs:795-804, for a byte pair at once
+        // 6-bit (scale, min) of sub-blocks 2g and 2g+1, two packed bytes each
         uint32_t a = D.h[1] >> L.sh, b = D.h[2] >> L.sh, c = D.h[3] >> L.sh;
-        uint32_t scp = L.high ? ((c & 0x0F0Fu) | ((a >> 2) & 0x3030u)) : (a & 0x3F3Fu);
-        uint32_t mp = L.high ? (((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u)) : (b & 0x3F3Fu);
+        uint32_t scp = (a & L.m1) | (c & L.m2) | ((a >> 2) & L.m3);
+        uint32_t mp = (b & L.m1) | ((c >> 4) & L.m2) | ((b >> 2) & L.m3);
         float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
         float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1), m0 = dmin * ub(mp, 0), m1 = dmin * ub(mp, 1);
         int acc[M][2][3];
@@ -127,8 +139,8 @@ struct Q4K {
             for (int m = 0; m < M; m++)
 #pragma unroll
                 for (int p = 0; p < 3; p++) {
-                    acc[m][0][p] = dot4(xp[m][0][p][i], lo, acc[m][0][p]);
-                    acc[m][1][p] = dot4(xp[m][1][p][i], hi, acc[m][1][p]);
+                    acc[m][0][p] = pdot<false>(p, xp[m][0][p][i], lo, acc[m][0][p]);
+                    acc[m][1][p] = pdot<false>(p, xp[m][1][p][i], hi, acc[m][1][p]);
                 }
         }
 #pragma unroll
@@ -143,6 +155,7 @@ struct Q4K {
 
 struct Q6K {
     static constexpr int WPL = 64, RUN = 16, NRUN = 4, BLOCK_VALUES = 256;
+    static constexpr bool SIGNED_W = false;
     struct Lane { uint32_t off_a, off_h, off_s, off_d, ssh; };
     struct Data {
         u32x4 a, b, h; u32x2 s; uint32_t d;
@@ -158,13 +171,13 @@ struct Q6K {
 #pragma unroll
         for (int g = 0; g < 4; g++) run[g] = 16 * b + 8 * hf + t + 2 * g;   // columns 256b + 128hf + 32g + 16t + [0,16)
     }
-    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
-        d.a = ((const U4A2*)(row + L.off_a))->v;
-        d.b = ((const U4A2*)(row + L.off_a + 32))->v;
-        d.h = ((const U4A2*)(row + L.off_h))->v;
-        d.s = ((const U2A2*)(row + L.off_s))->v;
-        d.d = *(const uint16_t*)(row + L.off_d);
+        d.a = ((const U4A2*)(row + (L.off_a + eo)))->v;
+        d.b = ((const U4A2*)(row + (L.off_a + eo) + 32))->v;
+        d.h = ((const U4A2*)(row + (L.off_h + eo)))->v;
+        d.s = ((const U2A2*)(row + (L.off_s + eo)))->v;
+        d.d = *(const uint16_t*)(row + (L.off_d + eo));
         return d;
     }
     template <int M>
@@ -191,7 +204,7 @@ struct Q6K {
 #pragma unroll
                 for (int g = 0; g < 4; g++)
 #pragma unroll
-                    for (int p = 0; p < 3; p++) acc[m][g][p] = dot4(xp[m][g][p][i], q[g], acc[m][g][p]);
+                    for (int p = 0; p < 3; p++) acc[m][g][p] = pdot<false>(p, xp[m][g][p][i], q[g], acc[m][g][p]);
         }
         uint32_t s0 = D.s[0] >> L.ssh, s1 = D.s[1] >> L.ssh;  // sc[is], sc[is+2] | sc[is+4], sc[is+6]
         float c[4] = {sb(s0, 0), sb(s0, 2), sb(s1, 0), sb(s1, 2)};
@@ -211,6 +224,7 @@ struct Q6K {
 
 struct Q80 {
     static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32;
+    static constexpr bool SIGNED_W = true;
     struct Lane { uint32_t off; };
     struct Data {
         u32x4 q0, q1; uint32_t d;
@@ -220,11 +234,11 @@ struct Q80 {
         L.off = u * 34;
         run[0] = u;
     }
-    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
-        d.d = *(const uint16_t*)(row + L.off);
-        d.q0 = ((const U4A2*)(row + L.off + 2))->v;
-        d.q1 = ((const U4A2*)(row + L.off + 18))->v;
+        d.d = *(const uint16_t*)(row + (L.off + eo));
+        d.q0 = ((const U4A2*)(row + (L.off + eo) + 2))->v;
+        d.q1 = ((const U4A2*)(row + (L.off + eo) + 18))->v;
         return d;
     }
     template <int M>
@@ -267,6 +281,9 @@ struct GemvParams {
 // Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 768 -> 168, 512 -> 256).
 constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
 // Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit that budget.
+// Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit 128 VGPRs
+// at batch 1 (16 waves per CU). Measured: 16 waves with 3 rows in flight beat 12 waves with 6-8 in flight
+// on every shape but the 638 MB head, and there by 6 % only.
 template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? (F::WPL == 64 ? (F::RUN == 16 ? 2 : 3) : 4) : 2; }
 // Activation rows one pass can hold in registers (48 plane dwords per row for the 64-weight units, 24 for Q8_0).
 template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
@@ -309,19 +326,26 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     const int nv = nrows * VPR;                          // virtual rows: v -> weight row r0 + v/VPR (+ pair for odd v)
     const uint8_t* base = p.W + (size_t)r0 * p.row_bytes;
     const int n_it = nv > v_start ? (nv - v_start + v_step - 1) / v_step : 0;
-    auto row_ptr = [&](int it) -> const uint8_t* {
-        int v = v_start + it * v_step + row_off;
-        v = v < nv ? v : nv - 1;                         // lanes past the end re-read the last row; they are masked below
+    // Address of iteration `it`: a wave-uniform row base (scalar registers) plus a 32-bit lane offset. A tail
+    // wave's lanes sit row_off rows further (v_start + it*v_step is a multiple of RT there, so with fused
+    // SwiGLU the gate/up split of row_off is fixed); lanes past the last row read the uniform row instead
+    // and are masked when the partial is written.
+    const uint32_t lane_extra = SWIGLU ? (uint32_t)((size_t)(row_off >> 1) * p.row_bytes + (size_t)(row_off & 1) * p.pair_bytes)
+                                       : (uint32_t)((size_t)row_off * p.row_bytes);
+    auto row_base = [&](int it) -> const uint8_t* {
+        const int v = v_start + it * v_step;             // wave-uniform
         return SWIGLU ? base + (size_t)(v >> 1) * p.row_bytes + (size_t)(v & 1) * p.pair_bytes : base + (size_t)v * p.row_bytes;
     };
+    auto fetch = [&](int it) { return F::load(row_base(it), L, (v_start + it * v_step + row_off < nv) ? lane_extra : 0u); };
 
     // ---- weight bytes of the first U iterations go in flight before the activations are touched
     typename F::Data buf[U];
 #pragma unroll
     for (int j = 0; j < U; j++)
-        if (j < n_it) buf[j] = F::load(row_ptr(j), L);
+        if (j < n_it) buf[j] = fetch(j);
 
     // ---- activations -> 24-bit block fixed point, once per workgroup, through LDS
+    constexpr float QMAX = F::SIGNED_W ? QMAX_S : QMAX_U;
     for (int e = tid * 8; e < M * p.cols; e += blockDim.x * 8) {
         float4 a = *(const float4*)(p.x + e), b = *(const float4*)(p.x + e + 4);
         float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -335,18 +359,36 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
             sum += dpp_f<0x4E>(sum);
         }
         float inv = amax > 0.f ? QMAX / amax : 0.f;
-        uint32_t pl[3][2] = {{0, 0}, {0, 0}, {0, 0}};
+        int q[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            int q = __float2int_rn(v[i] * inv);
-            q = q > (int)QMAX ? (int)QMAX : (q < -(int)QMAX ? -(int)QMAX : q);   // rounding of v*inv may overshoot by one
-            int c = (q << 24) >> 24;
-            int q1 = (q - c) >> 8;
-            int b8 = (q1 << 24) >> 24;
-            int a8 = (q1 - b8) >> 8;
-            pl[0][i >> 2] |= (uint32_t)(a8 & 0xFF) << (8 * (i & 3));
-            pl[1][i >> 2] |= (uint32_t)(b8 & 0xFF) << (8 * (i & 3));
-            pl[2][i >> 2] |= (uint32_t)(c & 0xFF) << (8 * (i & 3));
+            q[i] = __float2int_rn(v[i] * inv);
+            q[i] = q[i] > (int)QMAX ? (int)QMAX : (q[i] < -(int)QMAX ? -(int)QMAX : q[i]);   // rounding of v*inv may overshoot by one
+        }
+        uint32_t pl[3][2];
+        if (F::SIGNED_W) {
+#pragma unroll
+            for (int pp = 0; pp < 3; pp++) pl[pp][0] = pl[pp][1] = 0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {                // balanced digits
+                int c = (q[i] << 24) >> 24;
+                int q1 = (q[i] - c) >> 8;
+                int b8 = (q1 << 24) >> 24;
+                int a8 = (q1 - b8) >> 8;
+                pl[0][i >> 2] |= (uint32_t)(a8 & 0xFF) << (8 * (i & 3));
+                pl[1][i >> 2] |= (uint32_t)(b8 & 0xFF) << (8 * (i & 3));
+                pl[2][i >> 2] |= (uint32_t)(c & 0xFF) << (8 * (i & 3));
+            }
+        } else {
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {             // planes = byte lanes 2, 1, 0 of the two's complement integers
+                uint32_t q0 = q[4 * hh], q1 = q[4 * hh + 1], q2 = q[4 * hh + 2], q3 = q[4 * hh + 3];
+                uint32_t t01 = __builtin_amdgcn_perm(q1, q0, 0x05010400u), t23 = __builtin_amdgcn_perm(q3, q2, 0x05010400u);
+                uint32_t u01 = __builtin_amdgcn_perm(q1, q0, 0x00000602u), u23 = __builtin_amdgcn_perm(q3, q2, 0x00000602u);
+                pl[2][hh] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);   // bytes 0
+                pl[1][hh] = __builtin_amdgcn_perm(t23, t01, 0x07060302u);   // bytes 1
+                pl[0][hh] = __builtin_amdgcn_perm(u23, u01, 0x05040100u);   // bytes 2 (sign carried by the arithmetic shift)
+            }
         }
         int r = e / RUN, within = e % RUN;               // run index counts across the M activation rows
 #pragma unroll
@@ -401,7 +443,7 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
             // consume, then refill the same registers: the old bytes are dead when the new load is issued,
             // so the loop-carried buffer needs no copy (and no wait) at the back edge
             consume(buf[j], i0 + j);
-            buf[j] = F::load(row_ptr(i0 + j + U), L);
+            buf[j] = fetch(i0 + j + U);
         }
     }
     // drain, step A: iterations [i0, i0+U) that exist, reloading what is left of the step after it
@@ -410,7 +452,7 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
         const int it = i0 + j;
         if (it < n_it) {
             consume(buf[j], it);
-            if (it + U < n_it) buf[j] = F::load(row_ptr(it + U), L);
+            if (it + U < n_it) buf[j] = fetch(it + U);
         }
     }
     // drain, step B: iterations [i0+U, n_it)
@@ -495,22 +537,21 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     constexpr int MAXW = max_threads(M) / 64;
     p.RF = full_wave_replicas(p.NG, MAXW);
     const int WPR = waves_per_row_group(p.NG, MAXW);
-    // Rows per row group (rpg) and row groups per workgroup (G). A CU holds Gcap row groups at once
-    // (one workgroup of MAXW waves), the chip cus*Gcap; row groups of rpg rows are dealt out in rounds,
-    // so the run takes about rounds*rpg row times: minimise that, preferring more rows per activation
-    // load on a tie. With a single, partly filled round the row groups are spread over all CUs.
+    // Rows per row group (rpg) and row groups per workgroup (G). A CU holds Gcap row groups at once (one
+    // workgroup of MAXW waves). Every workgroup pays a fixed few microseconds (activation quantisation,
+    // pipeline fill and drain), so the rows are dealt out in as few rounds as possible: one workgroup per
+    // CU with up to RPG_MAX rows per row group, more rounds of equal size only beyond that. With a
+    // partly filled single round the row groups are spread over all CUs.
+    constexpr int RPG_MAX = 256;
     const int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     int Gcap = MAXW / WPR;
     if (Gcap < 1) Gcap = 1;
-    int rpg = 1;
-    size_t best = ~(size_t)0;
-    for (int r = 1; r <= 32; r++) {
-        size_t nrg = (out_rows + r - 1) / r;
-        size_t rounds = (nrg + (size_t)cus * Gcap - 1) / ((size_t)cus * Gcap);
-        if (rounds * r <= best) { best = rounds * r; rpg = r; }
-    }
+    const size_t slots = (size_t)cus * Gcap;
+    const size_t rounds = (out_rows + slots * RPG_MAX - 1) / (slots * RPG_MAX);
+    int rpg = (int)((out_rows + slots * rounds - 1) / (slots * rounds));
+    if (rpg < 1) rpg = 1;
     const size_t nrg = (out_rows + rpg - 1) / rpg;
-    int G = nrg >= (size_t)cus * Gcap ? Gcap : (int)((nrg + cus - 1) / cus);
+    int G = nrg >= slots ? Gcap : (int)((nrg + cus - 1) / cus);
     if (tune_g > 0) G = tune_g;
     if (tune_rpg > 0) rpg = tune_rpg;
     p.G = G; p.rpg = rpg;
@@ -528,9 +569,9 @@ int max_batch(const fhip_weight* w, size_t left) {
     const int NG = (int)(w->cols / (16 * F::WPL));
     auto WPRm = [&](int m) { return waves_per_row_group(NG, max_threads(m) / 64); };
     const size_t cap = fhip::device_lds_bytes();
-    if (left >= 4 && max_m<F>() >= 4 && WPRm(4) * 64 <= max_threads(4) && lds_bytes<F, 4, SWIGLU>(w->cols, NG, 1, 32) <= cap) return 4;
-    if (left >= 2 && WPRm(2) * 64 <= max_threads(2) && lds_bytes<F, 2, SWIGLU>(w->cols, NG, 1, 32) <= cap) return 2;
-    if (WPRm(1) * 64 <= max_threads(1) && lds_bytes<F, 1, SWIGLU>(w->cols, NG, 1, 32) <= cap) return 1;
+    if (left >= 4 && max_m<F>() >= 4 && WPRm(4) * 64 <= max_threads(4) && lds_bytes<F, 4, SWIGLU>(w->cols, NG, max_threads(4) / 64 / WPRm(4), 256) <= cap) return 4;
+    if (left >= 2 && WPRm(2) * 64 <= max_threads(2) && lds_bytes<F, 2, SWIGLU>(w->cols, NG, max_threads(2) / 64 / WPRm(2), 256) <= cap) return 2;
+    if (WPRm(1) * 64 <= max_threads(1) && lds_bytes<F, 1, SWIGLU>(w->cols, NG, max_threads(1) / 64 / WPRm(1), 256) <= cap) return 1;
     return 0;
 }
 
