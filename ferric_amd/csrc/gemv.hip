@@ -324,7 +324,7 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     int nrows = p.out_rows - r0;
     nrows = nrows < 0 ? 0 : (nrows > p.rpg ? p.rpg : nrows);
     const int nv = nrows * VPR;                          // virtual rows: v -> weight row r0 + v/VPR (+ pair for odd v)
-    const uint8_t* base = p.W + (size_t)r0 * p.row_bytes;
+    const uint8_t* base = p.W + (size_t)(nrows > 0 ? r0 : 0) * p.row_bytes;   // a row group past the end points at row 0
     const int n_it = nv > v_start ? (nv - v_start + v_step - 1) / v_step : 0;
     // Address of iteration `it`: a wave-uniform row base (scalar registers) plus a 32-bit lane offset. A tail
     // wave's lanes sit row_off rows further (v_start + it*v_step is a multiple of RT there, so with fused
@@ -338,7 +338,13 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     };
     auto fetch = [&](int it) { return F::load(row_base(it), L, (v_start + it * v_step + row_off < nv) ? lane_extra : 0u); };
 
-    // ---- weight bytes of the first U iterations go in flight before the activations are touched
+    // ---- the (cache-resident) activation loads go out first, then the weight bytes of the first U iterations.
+    // (Loads return in issue order. Issuing exactly U row loads unconditionally would let the wait for the
+    // activations be a counted one instead of a drain, but the dummy loads of waves with fewer than U rows
+    // cost more than that saves: measured +40 % on the 4096x4096 Q8_0 GEMV.)
+    const int e0 = tid * 8;
+    float4 xa0 = {0, 0, 0, 0}, xb0 = {0, 0, 0, 0};
+    if (e0 < M * p.cols) { xa0 = *(const float4*)(p.x + e0); xb0 = *(const float4*)(p.x + e0 + 4); }
     typename F::Data buf[U];
 #pragma unroll
     for (int j = 0; j < U; j++)
@@ -346,8 +352,9 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
 
     // ---- activations -> 24-bit block fixed point, once per workgroup, through LDS
     constexpr float QMAX = F::SIGNED_W ? QMAX_S : QMAX_U;
-    for (int e = tid * 8; e < M * p.cols; e += blockDim.x * 8) {
-        float4 a = *(const float4*)(p.x + e), b = *(const float4*)(p.x + e + 4);
+    for (int e = e0; e < M * p.cols; e += blockDim.x * 8) {
+        float4 a = xa0, b = xb0;
+        if (e != e0) { a = *(const float4*)(p.x + e); b = *(const float4*)(p.x + e + 4); }
         float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
         float amax = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
                            fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
@@ -463,23 +470,25 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     }
     __syncthreads();
 
-    // ---- add the NG slot partials of each output in a fixed order, apply SwiGLU, store
+    // ---- add the NG slot partials of each output in a fixed order, apply SwiGLU, store.
+    // Local row rr = g*rpg + rl is output row blockIdx.x*G*rpg + rr, and its partials start at rr*VPR*NG.
     const int per_wg = p.G * p.rpg;
-    for (int i = tid; i < per_wg * M; i += blockDim.x) {
-        int m = i / per_wg, rr = i % per_wg;             // consecutive threads -> consecutive output rows
-        int g = rr / p.rpg, rl = rr % p.rpg;
-        int r = (blockIdx.x * p.G + g) * p.rpg + rl;
-        if (r >= p.out_rows) continue;
-        const float* q = part + (((size_t)g * p.rpg + rl) * VPR * p.NG) * M + m;
-        float a = 0.f;
-        for (int s = 0; s < p.NG; s++) a += q[s * M];
-        if (SWIGLU) {
-            float b = 0.f;
-            for (int s = 0; s < p.NG; s++) b += q[(p.NG + s) * M];
-            a = (a / (1.0f + expf(-a))) * b;             // silu(gate) * up, crates/ferric-tensor/src/dtype.rs:2408
+    const int row0 = blockIdx.x * per_wg;
+#pragma unroll
+    for (int m = 0; m < M; m++)
+        for (int rr = tid; rr < per_wg; rr += blockDim.x) {   // consecutive threads -> consecutive output rows
+            const int r = row0 + rr;
+            if (r >= p.out_rows) break;
+            const float* q = part + ((size_t)rr * VPR * p.NG) * M + m;
+            float a = 0.f;
+            for (int s = 0; s < p.NG; s++) a += q[s * M];
+            if (SWIGLU) {
+                float b = 0.f;
+                for (int s = 0; s < p.NG; s++) b += q[(p.NG + s) * M];
+                a = (a / (1.0f + expf(-a))) * b;             // silu(gate) * up, crates/ferric-tensor/src/dtype.rs:2408
+            }
+            p.y[(size_t)m * p.out_rows + r] = a;
         }
-        p.y[(size_t)m * p.out_rows + r] = a;
-    }
 }
 
 // Un-fused SwiGLU, crates/ferric-tensor/src/lib.rs:2603-2618: gu [t, 2d] = [gate | up] per row.
