@@ -6,22 +6,29 @@
 // feed an 8x8 f32 matrix unit. Here the unit is v_mfma_f32_32x32x16_bf16.
 //
 // Shape of the kernel. The reference found this path bound by the unpack arithmetic, not the matrix
-// unit (crates/ferric-core/src/lib.rs:90-101), and the same holds here: a Q4_K weight costs ~3 VALU
+// unit (crates/ferric-core/src/lib.rs:90-101), and the same holds here: a weight costs ~3 VALU
 // operations to turn into bf16, an MFMA retires 16K multiply-adds in 32 cycles. So
 //   * each lane dequantizes straight into the B-operand registers of the MFMA it feeds (the B fragment of
 //     a 32x32x16 MFMA is 8 consecutive k of one weight row per lane, which is 8 consecutive quants of the
 //     GGUF stream: no LDS round trip, no transposition for the weights);
 //   * a dequantized fragment is reused for every 32-row slab of the activation tile the wave owns
-//     (MI slabs), so unpack cost is amortised over BM = 32*MI activation rows;
+//     (MI slabs, up to 8), so unpack cost is amortised over BM = 32*MI activation rows;
+//   * the fragments of step s+1 are produced while the MFMAs of step s run: the two instruction streams
+//     are independent, and the matrix pipe executes an issued MFMA while the wave goes on issuing VALU work;
 //   * the activation tile, which all 4 waves of a workgroup share, is staged through LDS (padded rows,
 //     16-byte reads) and each fragment read feeds NI MFMAs;
 //   * the 16 k of one MFMA are chosen inside ONE scale sub-block (the k order inside an MFMA is free as
-//     long as both operands agree), so a fragment needs a single (scale, min) pair.
-// One k-step is 64 columns = 4 MFMA slices. Dequantized values are exactly the f32 the CPU dequantizer
-// produces, rounded to bf16 (RNE) by v_cvt_pk_bf16_f32.
+//     long as both operands agree), so a fragment needs a single (scale, min) pair;
+//   * weight bytes are fetched a whole 256-column chunk ahead into the registers the previous chunk has
+//     just vacated (consume, then refill), so no load is waited for in the steady state.
+// One k-step is 64 columns = 4 MFMA slices; a chunk is 4 steps = one K-quant super-block or 8 Q8_0 blocks.
+// Dequantized values are exactly the f32 the CPU dequantizer produces, rounded to bf16 (RNE) by
+// v_cvt_pk_bf16_f32.
 #include "common.hpp"
 
 #include <hip/hip_fp16.h>
+
+#include <type_traits>
 
 namespace {
 
@@ -30,13 +37,10 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };
-struct __attribute__((packed, aligned(2))) U2A2 { u32x2 v; };
 
 __device__ __forceinline__ float f16_bits(uint32_t b) { return __half2float(__ushort_as_half((unsigned short)b)); }
 __device__ __forceinline__ float ub(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
-__device__ __forceinline__ float sb(uint32_t v, int k) { return (float)(int8_t)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ uint32_t pk_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){a, b}, bf16x2));
 }
@@ -51,100 +55,177 @@ __device__ __forceinline__ bf16x8 frag8(uint32_t q0, uint32_t q1, float s, float
 }
 
 constexpr int KSTEP = 64;            // columns per k-step: 4 MFMA slices of 16
+constexpr int CHUNK = 256;           // columns per chunk: 4 steps
 constexpr int LDS_ROW = KSTEP + 8;   // bf16 per staged activation row (+16 B pad: conflict-free 16-byte reads)
 
+// Column of the 8 consecutive k that lane half h (= lane / 32) holds in slice t of a step, for both
+// operands and every format: sub-block (t >> 1) of the step, elements 16h + 8(t & 1) + [0, 8).
+__device__ __forceinline__ constexpr int kcol(int t, int h) { return 32 * (t >> 1) + 16 * h + 8 * (t & 1); }
+
 // ------------------------------------------------------------------------------------------------
-// Per-format fragment builders. For k-step s of row `row` and lane half h (= lane / 32), produce the four
-// B fragments; slice t of the step covers, for lane half h, the 8 columns
-//     k0 + koff(t) + 8h' ... with the per-format column map given by `kcol`, which the activation side uses
-// to fetch the matching 8 columns.
+// Per-format weight streams. `Raw` is the per-lane register image of one chunk of one weight row (the
+// half h of it this lane unpacks). prime() loads chunk c whole. For step G of a chunk, begin<G>() derives
+// the step's scales into a `Ctx`, frag<G, T>() builds the B fragment of slice T, and refill<G>() reloads
+// the registers step G has just read with the same bytes of chunk `nc` (the following chunk, clamped by
+// the caller to one that exists).
 // ------------------------------------------------------------------------------------------------
 
 struct Q4K {
-    // step = group g of block b: slice t -> sub-block 2g + (t>>1), elements 16h + 8(t&1) + [0,8)
-    static __device__ __forceinline__ int kcol(int t, int h) { return 32 * (t >> 1) + 16 * h + 8 * (t & 1); }
-    struct Raw { u32x4 hd, q; };
-    static __device__ __forceinline__ Raw load(const uint8_t* row, int step, int h) {
-        const uint8_t* blk = row + (size_t)(step >> 2) * 144;
-        Raw r;
+    static constexpr int BLOCK = 144;
+    static constexpr bool PARTIAL = false;
+    static __host__ __device__ int chunks(int K) { return K / 256; }
+    struct Raw { u32x4 hd, hdn, q[4]; };
+    struct Ctx { float d0, o0, d1, o1; };
+    static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int h, int) {
+        const uint8_t* blk = row + (size_t)c * BLOCK;
         r.hd = *(const u32x4*)blk;
-        r.q = *(const u32x4*)(blk + 16 + 32 * (step & 3) + 16 * h);
-        return r;
+        r.hdn = r.hd;
+#pragma unroll
+        for (int g = 0; g < 4; g++) r.q[g] = *(const u32x4*)(blk + 16 + 32 * g + 16 * h);
     }
-    static __device__ __forceinline__ void frags(const Raw& r, int step, int, bf16x8 (&b)[4]) {
-        const int g = step & 3;
-        // get_sc_min for sub-blocks 2g, 2g+1 (crates/ferric-gguf/src/lib.rs:795-804), two packed bytes each
-        const int sh = 16 * (g & 1);
-        uint32_t a = r.hd[1] >> sh, bb = r.hd[2] >> sh, c = r.hd[3] >> sh;
-        uint32_t scp = g >= 2 ? ((c & 0x0F0Fu) | ((a >> 2) & 0x3030u)) : (a & 0x3F3Fu);
-        uint32_t mp = g >= 2 ? (((c >> 4) & 0x0F0Fu) | ((bb >> 2) & 0x3030u)) : (bb & 0x3F3Fu);
-        float d = f16_bits(r.hd[0] & 0xFFFFu), dmin = f16_bits(r.hd[0] >> 16);
-        // y = (d*sc)*q - (dmin*m): the product is exact in f32, so the fused form rounds identically
-        float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1), m0 = -(dmin * ub(mp, 0)), m1 = -(dmin * ub(mp, 1));
-        const uint32_t M = 0x0F0F0F0Fu;
-        b[0] = frag8(r.q[0] & M, r.q[1] & M, d0, m0);
-        b[1] = frag8(r.q[2] & M, r.q[3] & M, d0, m0);
-        b[2] = frag8((r.q[0] >> 4) & M, (r.q[1] >> 4) & M, d1, m1);
-        b[3] = frag8((r.q[2] >> 4) & M, (r.q[3] >> 4) & M, d1, m1);
+    // get_sc_min (crates/ferric-gguf/src/lib.rs:795-804) for sub-block j (a compile-time constant after inlining)
+    static __device__ __forceinline__ void sc_min(const u32x4& hd, int j, float& sc, float& mn) {
+        const uint32_t a = hd[1], b = hd[2], c = hd[3];
+        if (j < 4) {
+            sc = (float)((a >> (8 * j)) & 63u);
+            mn = (float)((b >> (8 * j)) & 63u);
+        } else {
+            const int i = j - 4;
+            sc = (float)(((c >> (8 * i)) & 0xFu) | (((a >> (8 * i + 6)) & 3u) << 4));
+            mn = (float)(((c >> (8 * i + 4)) & 0xFu) | (((b >> (8 * i + 6)) & 3u) << 4));
+        }
+    }
+    template <int G>
+    static __device__ __forceinline__ void begin(Raw& r, int, int, int, Ctx& x) {
+        if (G == 0) r.hd = r.hdn;
+        const float d = f16_bits(r.hd[0] & 0xFFFFu), dmin = f16_bits(r.hd[0] >> 16);
+        float s0, m0, s1, m1;
+        sc_min(r.hd, 2 * G, s0, m0);
+        sc_min(r.hd, 2 * G + 1, s1, m1);
+        // y = (d*sc)*q - (dmin*m): the product is exact in f32, so the fused form rounds identically.
+        // The high nibbles stay in place (q * 16) and their scale carries the 1/16, an exact power of two.
+        x.d0 = d * s0; x.o0 = -(dmin * m0); x.d1 = (d * s1) * 0.0625f; x.o1 = -(dmin * m1);
+    }
+    // slice T: sub-block 2G + (T >> 1) = low (T < 2) or high nibbles of bytes 32G + 16h + 8(T & 1) + [0, 8)
+    template <int G, int T>
+    static __device__ __forceinline__ bf16x8 frag(const Raw& r, const Ctx& x) {
+        constexpr uint32_t M = T < 2 ? 0x0F0F0F0Fu : 0xF0F0F0F0u;
+        return frag8(r.q[G][2 * (T & 1)] & M, r.q[G][2 * (T & 1) + 1] & M, T < 2 ? x.d0 : x.d1, T < 2 ? x.o0 : x.o1);
+    }
+    template <int G>
+    static __device__ __forceinline__ void refill(Raw& r, const uint8_t* row, int nc, int h, int) {
+        const uint8_t* nb = row + (size_t)nc * BLOCK;
+        r.q[G] = *(const u32x4*)(nb + 16 + 32 * G + 16 * h);
+        if (G == 1) r.hdn = *(const u32x4*)nb;
     }
 };
 
 struct Q6K {
-    // step = 64 columns of half hf: groups g0 = 2*(step&1), g0+1; slice t -> group g0 + (t>>1),
-    // l = 16(t&1) + 8h + [0,8)  (one scale per slice: sc[8hf + 2g + l/16])
-    static __device__ __forceinline__ int kcol(int t, int h) { return 32 * (t >> 1) + 16 * (t & 1) + 8 * h; }
-    struct Raw { u32x2 ql[4], qh[2], sc8; uint32_t d; };
-    static __device__ __forceinline__ Raw load(const uint8_t* row, int step, int h) {
-        const uint8_t* blk = row + (size_t)(step >> 2) * 210;
-        const int hf = (step >> 1) & 1;
-        Raw r;
-        r.d = *(const uint16_t*)(blk + 208);
-        r.sc8 = ((const U2A2*)(blk + 192 + 8 * hf))->v;               // sc[8hf .. 8hf+8)
+    // Step G covers half hf = G >> 1 of the super-block and its groups g0 = 2(G & 1), g0 + 1 (low nibbles of
+    // ql for G even, high nibbles for G odd); slice T is group g = g0 + (T >> 1), l = 16h + 8(T & 1) + [0, 8),
+    // whose scale is sc[8hf + 2g + h]  (crates/ferric-gguf/src/lib.rs:833-851).
+    static constexpr int BLOCK = 210;
+    static constexpr bool PARTIAL = false;
+    static __host__ __device__ int chunks(int K) { return K / 256; }
+    struct Raw { u32x4 ql[2][2], qh[2], sc, scn; uint32_t d, dn; };
+    struct Ctx { float d; };
+    static __device__ __forceinline__ u32x4 ld16(const uint8_t* p) { return ((const U4A2*)p)->v; }
+    static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int h, int) {
+        const uint8_t* blk = row + (size_t)c * BLOCK;
 #pragma unroll
-        for (int t = 0; t < 4; t++)                                   // group parity (t>>1), l = 16(t&1) + 8h
-            r.ql[t] = ((const U2A2*)(blk + 64 * hf + 32 * (t >> 1) + 16 * (t & 1) + 8 * h))->v;
-#pragma unroll
-        for (int u = 0; u < 2; u++) r.qh[u] = ((const U2A2*)(blk + 128 + 32 * hf + 16 * u + 8 * h))->v;
-        return r;
+        for (int hf = 0; hf < 2; hf++) {
+            r.ql[hf][0] = ld16(blk + 64 * hf + 16 * h);
+            r.ql[hf][1] = ld16(blk + 64 * hf + 32 + 16 * h);
+            r.qh[hf] = ld16(blk + 128 + 32 * hf + 16 * h);
+        }
+        r.scn = ld16(blk + 192);
+        r.dn = *(const uint16_t*)(blk + 208);
+        r.sc = r.scn;
+        r.d = r.dn;
     }
-    static __device__ __forceinline__ void frags(const Raw& r, int step, int, bf16x8 (&b)[4]) {
-        const int g0 = 2 * (step & 1);                                // groups g0 (t = 0,1) and g0+1 (t = 2,3)
-        float d = f16_bits(r.d);
-        uint32_t scw = g0 ? r.sc8[1] : r.sc8[0];                      // sc[8hf + 2g0 + t], t = 0..3
+    template <int G>
+    static __device__ __forceinline__ void begin(Raw& r, int, int h, int, Ctx& x) {
+        if (G == 0) {
+            // byte h of every 16-bit pair is this lane half's scale: shift it down once per chunk
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const int g = g0 + (t >> 1);                              // ql byte parity g&1 = t>>1, nibble = g>=2 = (g0 != 0)
-            uint32_t n0 = (g0 ? r.ql[t][0] >> 4 : r.ql[t][0]) & 0x0F0F0F0Fu, n1 = (g0 ? r.ql[t][1] >> 4 : r.ql[t][1]) & 0x0F0F0F0Fu;
-            uint32_t h0 = ((r.qh[t & 1][0] >> (2 * g)) & 0x03030303u) << 4, h1 = ((r.qh[t & 1][1] >> (2 * g)) & 0x03030303u) << 4;
-            float ds = d * sb(scw, t);
-            // (d*sc)*(q-32) = ds*q - 32*ds, every term exact in f32
-            b[t] = frag8(n0 | h0, n1 | h1, ds, -32.0f * ds);
+            for (int w = 0; w < 4; w++) r.sc[w] = r.scn[w] >> (8 * h);
+            r.d = r.dn;
+        }
+        x.d = f16_bits(r.d);
+    }
+    template <int G, int T>
+    static __device__ __forceinline__ bf16x8 frag(const Raw& r, const Ctx& x) {
+        constexpr int hf = G >> 1, g = 2 * (G & 1) + (T >> 1), par = T >> 1, w = 2 * (T & 1);
+        const uint32_t l0 = r.ql[hf][par][w], l1 = r.ql[hf][par][w + 1];
+        const uint32_t h0 = r.qh[hf][w], h1 = r.qh[hf][w + 1];
+        uint32_t n0, n1, u0, u1;
+        if (G & 1) { n0 = (l0 >> 4) & 0x0F0F0F0Fu; n1 = (l1 >> 4) & 0x0F0F0F0Fu; }
+        else       { n0 = l0 & 0x0F0F0F0Fu;        n1 = l1 & 0x0F0F0F0Fu; }
+        if (g < 2) { u0 = (h0 << (g < 2 ? 4 - 2 * g : 0)) & 0x30303030u; u1 = (h1 << (g < 2 ? 4 - 2 * g : 0)) & 0x30303030u; }
+        else       { u0 = (h0 >> (g < 2 ? 0 : 2 * g - 4)) & 0x30303030u; u1 = (h1 >> (g < 2 ? 0 : 2 * g - 4)) & 0x30303030u; }
+        const uint32_t scw = r.sc[2 * hf + (g >> 1)];
+        const float ds = x.d * (float)(int8_t)((scw >> (16 * (g & 1))) & 0xFFu);
+        // (d*sc)*(q-32) = ds*q - 32*ds, every term exact in f32
+        return frag8(n0 | u0, n1 | u1, ds, -32.0f * ds);
+    }
+    template <int G>
+    static __device__ __forceinline__ void refill(Raw& r, const uint8_t* row, int nc, int h, int) {
+        constexpr int hf = G >> 1;
+        const uint8_t* nb = row + (size_t)nc * BLOCK;
+        if (G & 1) {   // both nibble planes of this half are spent
+            r.ql[hf][0] = ld16(nb + 64 * hf + 16 * h);
+            r.ql[hf][1] = ld16(nb + 64 * hf + 32 + 16 * h);
+            r.qh[hf] = ld16(nb + 128 + 32 * hf + 16 * h);
+        }
+        if (G == 1) {
+            r.scn = ld16(nb + 192);
+            r.dn = *(const uint16_t*)(nb + 208);
         }
     }
 };
 
 struct Q80 {
-    // step = blocks 2s, 2s+1: slice t -> block 2s + (t>>1), elements 16(t&1) + 8h + [0,8)
-    static __device__ __forceinline__ int kcol(int t, int h) { return 32 * (t >> 1) + 16 * (t & 1) + 8 * h; }
-    struct Raw { u32x2 q[4]; uint32_t d[2]; };
-    static __device__ __forceinline__ Raw load(const uint8_t* row, int step, int h) {
-        Raw r;
-#pragma unroll
-        for (int u = 0; u < 2; u++) r.d[u] = *(const uint16_t*)(row + (size_t)(2 * step + u) * 34);
-#pragma unroll
-        for (int t = 0; t < 4; t++) r.q[t] = ((const U2A2*)(row + (size_t)(2 * step + (t >> 1)) * 34 + 2 + 16 * (t & 1) + 8 * h))->v;
-        return r;
+    // A chunk is 8 blocks of 34 bytes; step G covers blocks 2G, 2G+1; slice T is block 2G + (T >> 1),
+    // elements 16h + 8(T & 1) + [0, 8). A trailing partial chunk is allowed: blocks past the row's end are
+    // read from the last valid block's address and given scale 0 (their activations are staged as 0 too).
+    static constexpr int BLOCK = 34;
+    static constexpr bool PARTIAL = true;   // a row may end inside a chunk
+    static __host__ __device__ int chunks(int K) { return (K + 255) / 256; }
+    struct Raw { u32x4 q[4][2]; uint32_t d[4][2]; };
+    struct Ctx { float d[2]; };
+    static __device__ __forceinline__ const uint8_t* blk(const uint8_t* row, int c, int i, int nblk) {
+        int bi = 8 * c + i;
+        bi = bi < nblk ? bi : nblk - 1;
+        return row + (size_t)bi * BLOCK;
     }
-    static __device__ __forceinline__ void frags(const Raw& r, int, int, bf16x8 (&b)[4]) {
+    static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int h, int nblk) {
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-            float d = f16_bits(r.d[t >> 1]);
-            u32x4 o;
-            o[0] = pk_bf16(sb(r.q[t][0], 0) * d, sb(r.q[t][0], 1) * d);
-            o[1] = pk_bf16(sb(r.q[t][0], 2) * d, sb(r.q[t][0], 3) * d);
-            o[2] = pk_bf16(sb(r.q[t][1], 0) * d, sb(r.q[t][1], 1) * d);
-            o[3] = pk_bf16(sb(r.q[t][1], 2) * d, sb(r.q[t][1], 3) * d);
-            b[t] = __builtin_bit_cast(bf16x8, o);
+        for (int g = 0; g < 4; g++)
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const uint8_t* p = blk(row, c, 2 * g + u, nblk);
+                r.d[g][u] = *(const uint16_t*)p;
+                r.q[g][u] = ((const U4A2*)(p + 2 + 16 * h))->v;
+            }
+    }
+    template <int G>
+    static __device__ __forceinline__ void begin(Raw& r, int c, int, int nblk, Ctx& x) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) x.d[u] = (8 * c + 2 * G + u) < nblk ? f16_bits(r.d[G][u]) : 0.0f;
+    }
+    template <int G, int T>
+    static __device__ __forceinline__ bf16x8 frag(const Raw& r, const Ctx& x) {
+        // q = (q ^ 0x80) - 128 with the biased byte unsigned: d*q = d*u - 128*d, every term exact in f32
+        const float d = x.d[T >> 1];
+        return frag8(r.q[G][T >> 1][2 * (T & 1)] ^ 0x80808080u, r.q[G][T >> 1][2 * (T & 1) + 1] ^ 0x80808080u, d, -128.0f * d);
+    }
+    template <int G>
+    static __device__ __forceinline__ void refill(Raw& r, const uint8_t* row, int nc, int h, int nblk) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const uint8_t* p = blk(row, nc, 2 * G + u, nblk);
+            r.d[G][u] = *(const uint16_t*)p;
+            r.q[G][u] = ((const U4A2*)(p + 2 + 16 * h))->v;
         }
     }
 };
@@ -154,10 +235,19 @@ struct GemmParams {
     const uint16_t* X;   // bf16 bits [T, K]
     float* Y;            // [T, N]
     int T, N, K;
+    int nblk;            // blocks per weight row
     size_t row_bytes;
-    int steps_per_split; // k-steps each grid.z slice walks
+    int chunks_per_split; // chunks each grid.z slice walks
     int atomic;          // 1: several k-splits add into a zeroed Y
 };
+
+template <int I, int N, class Fn>
+__device__ __forceinline__ void static_for(Fn&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
 
 // Workgroup = 4 waves side by side along N; wave tile = (32*MI) x (32*NI); workgroup tile = (32*MI) x (128*NI).
 template <class F, int MI, int NI>
@@ -168,9 +258,11 @@ __global__ void __launch_bounds__(256) gemm_q_bf16_kernel(GemmParams p) {
     const int h = lane >> 5, c = lane & 31;
     const int t0 = blockIdx.y * BM;
     const int n0 = blockIdx.x * (128 * NI) + wave * (32 * NI);
-    const int nsteps = p.K / KSTEP;
-    const int s_begin = blockIdx.z * p.steps_per_split;
-    const int s_end = s_begin + p.steps_per_split < nsteps ? s_begin + p.steps_per_split : nsteps;
+    const int nchunks = F::chunks(p.K);
+    const int c_begin = blockIdx.z * p.chunks_per_split;
+    const int c_end = c_begin + p.chunks_per_split < nchunks ? c_begin + p.chunks_per_split : nchunks;
+    if (c_begin >= c_end) return;
+    const int c_last = c_end - 1;
 
     // weight row of each of this lane's NI fragments (clamped: rows past N are computed but not stored)
     const uint8_t* wrow[NI];
@@ -188,56 +280,123 @@ __global__ void __launch_bounds__(256) gemm_q_bf16_kernel(GemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // activation staging: BM rows x 64 bf16 = BM * 128 B per step; each thread moves 16 B pieces
-    constexpr int PIECES = BM * 8 / 256;  // 16-byte pieces per thread per step
-    u32x4 stage[PIECES];
-    auto load_a = [&](int s) {
+    // Activation staging: BM rows x 64 bf16 per step; thread `tid` moves the 16-byte piece (tid & 7) of rows
+    // (tid >> 3) + 32q, q < MI. Rows past T are read from row T-1 (their outputs are never stored); columns
+    // past K (a partial last chunk) are staged as zeros.
+    const int a_col = (tid & 7) * 8;
+    const uint16_t* a_src[MI];
 #pragma unroll
-        for (int q = 0; q < PIECES; q++) {
-            int piece = tid + 256 * q, r = piece >> 3, col = (piece & 7) * 8;
-            int t = t0 + r;
-            if (t < p.T) stage[q] = *(const u32x4*)(p.X + (size_t)t * p.K + (size_t)s * KSTEP + col);
-            else stage[q] = (u32x4){0, 0, 0, 0};
+    for (int q = 0; q < MI; q++) {
+        int t = t0 + (tid >> 3) + 32 * q;
+        a_src[q] = p.X + (size_t)(t < p.T ? t : p.T - 1) * p.K + a_col;
+    }
+    const int a_dst = (tid >> 3) * LDS_ROW + a_col;
+    u32x4 stage[MI];
+    auto load_a = [&](int s) {   // s = absolute step index (64 columns each)
+        if constexpr (F::PARTIAL) {
+            const bool ok = s * KSTEP + a_col < p.K;
+            const int off = ok ? s * KSTEP : 0;
+            const uint32_t keep = ok ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+            for (int q = 0; q < MI; q++) {
+                u32x4 v = *(const u32x4*)(a_src[q] + off);
+                stage[q] = (u32x4){v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
+            }
+        } else {
+            const int off = s * KSTEP < p.K ? s * KSTEP : 0;   // past the end: any valid address, the tile is never read
+#pragma unroll
+            for (int q = 0; q < MI; q++) stage[q] = *(const u32x4*)(a_src[q] + off);
         }
     };
     auto store_a = [&](int buf) {
 #pragma unroll
-        for (int q = 0; q < PIECES; q++) {
-            int piece = tid + 256 * q, r = piece >> 3, col = (piece & 7) * 8;
-            *(u32x4*)(&As[buf][r * LDS_ROW + col]) = stage[q];
-        }
+        for (int q = 0; q < MI; q++) *(u32x4*)(&As[buf][a_dst + 32 * q * LDS_ROW]) = stage[q];
     };
+    const int a_rd = c * LDS_ROW + 16 * h;   // + 32*i rows, + kcol(t, 0)
 
     typename F::Raw raw[NI];
-    if (s_begin < s_end) {
-        load_a(s_begin);
+    bf16x8 bA[NI][4], bB[NI][4];
 #pragma unroll
-        for (int j = 0; j < NI; j++) raw[j] = F::load(wrow[j], s_begin, h);
-        store_a(0);
+    for (int j = 0; j < NI; j++) F::prime(raw[j], wrow[j], c_begin, h, p.nblk);
+    load_a(4 * c_begin);
+    {
+        const int nc = c_begin + 1 < c_last ? c_begin + 1 : c_last;
+#pragma unroll
+        for (int j = 0; j < NI; j++) {
+            typename F::Ctx x;
+            F::template begin<0>(raw[j], c_begin, h, p.nblk, x);
+            static_for<0, 4>([&](auto T) { bA[j][T.value] = F::template frag<0, T.value>(raw[j], x); });
+            F::template refill<0>(raw[j], wrow[j], nc, h, p.nblk);
+        }
     }
+    store_a(0);
     __syncthreads();
-    for (int s = s_begin; s < s_end; s++) {
-        const int buf = (s - s_begin) & 1;
-        bf16x8 b[NI][4];
+
+    // One k-step: the MFMAs of step (chunk ck, G) from `cur` and LDS buffer G & 1, while the fragments of
+    // the following step are produced into `nxt` and its activations travel global -> registers -> LDS.
+    // The step is cut into segments of SA activation fragments (SA*NI MFMAs); each segment first reads the
+    // next segment's fragments from LDS, then alternates one MFMA with its share of the unpack arithmetic,
+    // so that the matrix pipe and the VALU both stay busy from this one wave. Nothing moves between segments.
+    constexpr int SA = MI < 4 ? MI : 4;
+    constexpr int NSEG = 4 * MI / SA;
+    constexpr int FPS = 4 * NI / NSEG;                          // fragments produced per segment
+    static_assert(FPS * NSEG == 4 * NI, "fragments must divide over the segments");
+    constexpr int VPM = (26 * FPS + SA * NI - 1) / (SA * NI);   // VALU instructions issued behind each MFMA
+    auto step = [&](auto Gc, int ck, bf16x8 (&cur)[NI][4], bf16x8 (&nxt)[NI][4]) {
+        constexpr int G = decltype(Gc)::value;
+        constexpr int GN = (G + 1) & 3;
+        constexpr int buf = G & 1;
+        // fragments of step G+1 of this chunk, or of step 0 of the next one
+        const int pc = G == 3 ? (ck + 1 < c_last ? ck + 1 : c_last) : ck;
+        const int nc = pc + 1 < c_last ? pc + 1 : c_last;
+        typename F::Ctx ctx[NI];
+        bf16x8 a[2][SA];
+        auto read_a = [&](int sg, bf16x8 (&dst)[SA]) {
 #pragma unroll
-        for (int j = 0; j < NI; j++) F::frags(raw[j], s, h, b[j]);
-        if (s + 1 < s_end) {                         // next step's activations and weight bytes in flight during the MFMAs
-            load_a(s + 1);
-#pragma unroll
-            for (int j = 0; j < NI; j++) raw[j] = F::load(wrow[j], s + 1, h);
-        }
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            const int kc = F::kcol(t, h);
-#pragma unroll
-            for (int i = 0; i < MI; i++) {
-                bf16x8 a = *(const bf16x8*)(&As[buf][(32 * i + c) * LDS_ROW + kc]);
-#pragma unroll
-                for (int j = 0; j < NI; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[j][t], acc[i][j], 0, 0, 0);
+            for (int u = 0; u < SA; u++) {
+                const int m = sg * SA + u, t = m / MI, i = m % MI;
+                dst[u] = *(const bf16x8*)(&As[buf][a_rd + 32 * i * LDS_ROW + kcol(t, 0)]);
             }
-        }
-        if (s + 1 < s_end) store_a(buf ^ 1);
+        };
+        read_a(0, a[0]);
+        load_a(4 * ck + G + 1);
+#pragma unroll
+        for (int j = 0; j < NI; j++) F::template begin<GN>(raw[j], pc, h, p.nblk, ctx[j]);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<0, NSEG>([&](auto S) {
+            constexpr int sg = decltype(S)::value;
+            if constexpr (sg + 1 < NSEG) read_a(sg + 1, a[(sg + 1) & 1]);
+#pragma unroll
+            for (int u = 0; u < SA; u++) {
+                const int m = sg * SA + u, t = m / MI, i = m % MI;
+#pragma unroll
+                for (int j = 0; j < NI; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[sg & 1][u], cur[j][t], acc[i][j], 0, 0, 0);
+            }
+            static_for<0, FPS>([&](auto Kc) {
+                constexpr int f = sg * FPS + decltype(Kc)::value, j = f / 4, T = f % 4;
+                nxt[j][T] = F::template frag<GN, T>(raw[j], ctx[j]);
+            });
+            if constexpr (sg + 1 < NSEG) __builtin_amdgcn_sched_group_barrier(0x100, SA, 0);
+#pragma unroll
+            for (int u = 0; u < SA * NI; u++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+#pragma unroll
+        for (int j = 0; j < NI; j++) F::template refill<GN>(raw[j], wrow[j], nc, h, p.nblk);
+        store_a(buf ^ 1);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    for (int ck = c_begin; ck < c_end; ck++) {
+        step(std::integral_constant<int, 0>{}, ck, bA, bB);
+        step(std::integral_constant<int, 1>{}, ck, bB, bA);
+        step(std::integral_constant<int, 2>{}, ck, bA, bB);
+        step(std::integral_constant<int, 3>{}, ck, bB, bA);
     }
 
     // D layout of the 32x32 MFMA: register r of lane (h, c) is row 8*(r/4) + 4*h + (r%4), column c
@@ -269,19 +428,27 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     GemmParams p;
     p.W = w->d_raw; p.X = d_x; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
-    const int nsteps = p.K / KSTEP;
+    p.nblk = (int)(w->row_bytes / F::BLOCK);
+    const int nchunks = F::chunks(p.K);
     dim3 grid((unsigned)((w->rows + 128 * NI - 1) / (128 * NI)), (unsigned)((t + 32 * MI - 1) / (32 * MI)), 1);
-    // Too few output tiles to occupy the CUs: split K over grid.z and add the slices into a zeroed Y.
+    // Workgroups run in rounds of `slots` (one per CU for the 256-row tile, whose accumulators take a SIMD's
+    // whole register file; two otherwise). When the output tiles do not fill the rounds evenly, split K over
+    // grid.z and add the slices into a zeroed Y: pick the split with the least (rounds x chunks per slice),
+    // charging every slice two chunks for its prologue, epilogue and atomic traffic.
     const int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    int split = 1;
+    const size_t slots = (size_t)cus * (MI >= 8 ? 1 : 2);
     const size_t tiles = (size_t)grid.x * grid.y;
-    if (tiles < (size_t)cus) {
-        split = (int)((cus + tiles - 1) / tiles);
-        if (split > nsteps) split = nsteps;
-        if (split > 16) split = 16;
+    int split = 1;
+    size_t best = 0;
+    for (int sp = 1; sp <= 16 && sp <= nchunks; sp++) {
+        const int cps = (nchunks + sp - 1) / sp;
+        const int z = (nchunks + cps - 1) / cps;
+        const size_t rounds = (tiles * z + slots - 1) / slots;
+        const size_t cost = rounds * (size_t)(cps + (z > 1 ? 2 : 0));
+        if (best == 0 || cost < best) { best = cost; split = sp; }
     }
-    p.steps_per_split = (nsteps + split - 1) / split;
-    grid.z = (unsigned)((nsteps + p.steps_per_split - 1) / p.steps_per_split);
+    p.chunks_per_split = (nchunks + split - 1) / split;
+    grid.z = (unsigned)((nchunks + p.chunks_per_split - 1) / p.chunks_per_split);
     p.atomic = grid.z > 1;
     if (p.atomic) {
         size_t n = t * w->rows;
@@ -293,7 +460,8 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
 
 template <class F>
 int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
-    if (t > 64) return launch_cfg<F, 4, 2>(w, d_x, t, d_y, s);   // 128 x 256 workgroup tile
+    if (t > 128) return launch_cfg<F, 8, 2>(w, d_x, t, d_y, s);  // 256 x 256 workgroup tile
+    if (t > 64) return launch_cfg<F, 4, 2>(w, d_x, t, d_y, s);
     if (t > 32) return launch_cfg<F, 2, 2>(w, d_x, t, d_y, s);
     return launch_cfg<F, 1, 2>(w, d_x, t, d_y, s);
 }
@@ -303,8 +471,7 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
 namespace fhip {
 
 int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
-    if (w->cols % KSTEP != 0)
-        return set_error(FHIP_ERR_SHAPE, "gemm_q_bf16: cols must be a multiple of %d (got %zu)", KSTEP, w->cols);
+    if (t == 0 || w->rows == 0) return FHIP_OK;
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "gemm_q_bf16: x must be 16-byte aligned");
     switch (w->type) {
         case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s);
