@@ -237,8 +237,11 @@ struct GemmParams {
     int T, N, K;
     int nblk;            // blocks per weight row
     size_t row_bytes;
-    int chunks_per_split; // chunks each grid.z slice walks
-    int atomic;          // 1: several k-splits add into a zeroed Y
+    int tiles_n;         // workgroup tiles along N
+    int nchunks;         // chunks per weight row
+    int whole_rounds;    // rounds of whole tiles every workgroup computes first: tile = round * gridDim.x + blockIdx.x
+    long long units;     // the remaining tiles' (tile, chunk) work units, chunk fastest
+    int per;             // of those, units per workgroup
 };
 
 template <int I, int N, class Fn>
@@ -249,28 +252,61 @@ __device__ __forceinline__ void static_for(Fn&& f) {
     }
 }
 
-// Workgroup = 4 waves side by side along N; wave tile = (32*MI) x (32*NI); workgroup tile = (32*MI) x (128*NI).
-template <class F, int MI, int NI>
-__global__ void __launch_bounds__(256) gemm_q_bf16_kernel(GemmParams p) {
-    constexpr int BM = 32 * MI;
+// Workgroup = 8 waves, 2 along T x 4 along N; wave tile = (32*MI) x 64; workgroup tile = (64*MI) x 256.
+// Two waves per SIMD: a wave issues one VALU instruction per ~6 cycles and one 16-byte LDS read per ~16, so
+// a single wave cannot feed its own MFMAs and unpack at the same time; two can.
+// The two waves of a T-pair need the same 64 weight rows. Each unpacks 32 of them (all four slices of a
+// step) and publishes the fragments in LDS in MFMA operand order (lane L's 16 bytes at L*16), where both
+// read them back: unpack work per MFMA halves, and a wave carries the raw bytes of one row only.
+//
+// Work distribution. One workgroup per CU. Every workgroup first computes `whole_rounds` whole tiles (tile =
+// round * gridDim.x + blockIdx.x, so the workgroups running side by side share activation rows in L2). The
+// tiles left over, fewer than one per workgroup, are cut along K: their (tile, chunk) units are dealt out in
+// equal contiguous runs of `per`, so every CU does the same amount of MFMA work whatever the tile count (no
+// partial last round). A run may start and end inside a tile: a segment that covers its tile's whole K stores
+// the tile, any other adds it atomically into a Y that zero_split_tiles_kernel cleared beforehand.
+template <class F, int MI>
+__global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
+    constexpr int NI = 2;
+    constexpr int BM = 64 * MI;
+    constexpr int FRAG = 512;                                   // bf16 per published fragment (64 lanes x 8)
     __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_ROW];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][32 * FRAG];   // [n-block 0..7][slice 0..3]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave & 3, wm = wave >> 2;
     const int h = lane >> 5, c = lane & 31;
-    const int t0 = blockIdx.y * BM;
-    const int n0 = blockIdx.x * (128 * NI) + wave * (32 * NI);
-    const int nchunks = F::chunks(p.K);
-    const int c_begin = blockIdx.z * p.chunks_per_split;
-    const int c_end = c_begin + p.chunks_per_split < nchunks ? c_begin + p.chunks_per_split : nchunks;
-    if (c_begin >= c_end) return;
+    const int nchunks = p.nchunks;
+    long long u = (long long)blockIdx.x * p.per;
+    const long long u_end = u + p.per < p.units ? u + p.per : p.units;
+  for (int round = 0;; round++) {
+    int tile, c_begin, c_end;
+    if (round < p.whole_rounds) {
+        tile = round * gridDim.x + blockIdx.x;
+        c_begin = 0;
+        c_end = nchunks;
+    } else {
+        if (u >= u_end) break;
+        const int rt = (int)(u / nchunks);
+        tile = p.whole_rounds * gridDim.x + rt;
+        c_begin = (int)(u - (long long)rt * nchunks);
+        c_end = (long long)(nchunks - c_begin) < u_end - u ? nchunks : c_begin + (int)(u_end - u);
+        u += c_end - c_begin;
+    }
+    const bool whole = c_begin == 0 && c_end == nchunks;
+    const int tile_y = tile / p.tiles_n, tile_x = tile - tile_y * p.tiles_n;
+    const int t0 = tile_y * BM + wm * (32 * MI);
+    const int n0 = tile_x * 256 + wn * 64;
     const int c_last = c_end - 1;
 
-    // weight row of each of this lane's NI fragments (clamped: rows past N are computed but not stored)
-    const uint8_t* wrow[NI];
-#pragma unroll
-    for (int j = 0; j < NI; j++) {
-        int n = n0 + 32 * j + c;
-        wrow[j] = p.W + (size_t)(n < p.N ? n : p.N - 1) * p.row_bytes;
+    // the weight row this lane unpacks: n-block 2*wn + wm of the workgroup tile (clamped: rows past N are
+    // computed but not stored)
+    const uint8_t* wrow;
+    {
+        int n = n0 + 32 * wm + c;
+        wrow = p.W + (size_t)(n < p.N ? n : p.N - 1) * p.row_bytes;
     }
+    const int b_wr = ((2 * wn + wm) * 4) * FRAG + lane * 8;    // + t * FRAG
+    const int b_rd = ((2 * wn) * 4) * FRAG + lane * 8;         // + (4 * j + t) * FRAG
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -281,14 +317,14 @@ __global__ void __launch_bounds__(256) gemm_q_bf16_kernel(GemmParams p) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     // Activation staging: BM rows x 64 bf16 per step; thread `tid` moves the 16-byte piece (tid & 7) of rows
-    // (tid >> 3) + 32q, q < MI. Rows past T are read from row T-1 (their outputs are never stored); columns
+    // (tid >> 3) + 64q, q < MI. Rows past T are read from row T-1 (their outputs are never stored); columns
     // past K (a partial last chunk) are staged as zeros.
     const int a_col = (tid & 7) * 8;
-    const uint16_t* a_src[MI];
+    uint32_t a_src[MI];   // element offsets into X (the launcher checks T*K fits 31 bits)
 #pragma unroll
     for (int q = 0; q < MI; q++) {
-        int t = t0 + (tid >> 3) + 32 * q;
-        a_src[q] = p.X + (size_t)(t < p.T ? t : p.T - 1) * p.K + a_col;
+        int t = tile_y * BM + (tid >> 3) + 64 * q;
+        a_src[q] = (uint32_t)(t < p.T ? t : p.T - 1) * (uint32_t)p.K + a_col;
     }
     const int a_dst = (tid >> 3) * LDS_ROW + a_col;
     u32x4 stage[MI];
@@ -299,104 +335,89 @@ __global__ void __launch_bounds__(256) gemm_q_bf16_kernel(GemmParams p) {
             const uint32_t keep = ok ? 0xFFFFFFFFu : 0u;
 #pragma unroll
             for (int q = 0; q < MI; q++) {
-                u32x4 v = *(const u32x4*)(a_src[q] + off);
+                u32x4 v = *(const u32x4*)(p.X + (a_src[q] + off));
                 stage[q] = (u32x4){v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
             }
         } else {
             const int off = s * KSTEP < p.K ? s * KSTEP : 0;   // past the end: any valid address, the tile is never read
 #pragma unroll
-            for (int q = 0; q < MI; q++) stage[q] = *(const u32x4*)(a_src[q] + off);
+            for (int q = 0; q < MI; q++) stage[q] = *(const u32x4*)(p.X + (a_src[q] + off));
         }
     };
     auto store_a = [&](int buf) {
 #pragma unroll
-        for (int q = 0; q < MI; q++) *(u32x4*)(&As[buf][a_dst + 32 * q * LDS_ROW]) = stage[q];
+        for (int q = 0; q < MI; q++) *(u32x4*)(&As[buf][a_dst + 64 * q * LDS_ROW]) = stage[q];
     };
-    const int a_rd = c * LDS_ROW + 16 * h;   // + 32*i rows, + kcol(t, 0)
-
-    typename F::Raw raw[NI];
-    bf16x8 bA[NI][4], bB[NI][4];
-#pragma unroll
-    for (int j = 0; j < NI; j++) F::prime(raw[j], wrow[j], c_begin, h, p.nblk);
+    const int a_rd = (wm * 32 * MI + c) * LDS_ROW + 16 * h;   // + 32*i rows, + kcol(t, 0)
+    typename F::Raw raw;
+    F::prime(raw, wrow, c_begin, h, p.nblk);
     load_a(4 * c_begin);
     {
         const int nc = c_begin + 1 < c_last ? c_begin + 1 : c_last;
-#pragma unroll
-        for (int j = 0; j < NI; j++) {
-            typename F::Ctx x;
-            F::template begin<0>(raw[j], c_begin, h, p.nblk, x);
-            static_for<0, 4>([&](auto T) { bA[j][T.value] = F::template frag<0, T.value>(raw[j], x); });
-            F::template refill<0>(raw[j], wrow[j], nc, h, p.nblk);
-        }
+        typename F::Ctx x;
+        F::template begin<0>(raw, c_begin, h, p.nblk, x);
+        static_for<0, 4>([&](auto T) {
+            *(bf16x8*)(&Bs[0][b_wr + T.value * FRAG]) = F::template frag<0, T.value>(raw, x);
+        });
+        F::template refill<0>(raw, wrow, nc, h, p.nblk);
     }
     store_a(0);
     __syncthreads();
 
-    // One k-step: the MFMAs of step (chunk ck, G) from `cur` and LDS buffer G & 1, while the fragments of
-    // the following step are produced into `nxt` and its activations travel global -> registers -> LDS.
-    // The step is cut into segments of SA activation fragments (SA*NI MFMAs); each segment first reads the
-    // next segment's fragments from LDS, then alternates one MFMA with its share of the unpack arithmetic,
-    // so that the matrix pipe and the VALU both stay busy from this one wave. Nothing moves between segments.
-    constexpr int SA = MI < 4 ? MI : 4;
-    constexpr int NSEG = 4 * MI / SA;
-    constexpr int FPS = 4 * NI / NSEG;                          // fragments produced per segment
-    static_assert(FPS * NSEG == 4 * NI, "fragments must divide over the segments");
-    constexpr int VPM = (26 * FPS + SA * NI - 1) / (SA * NI);   // VALU instructions issued behind each MFMA
-    auto step = [&](auto Gc, int ck, bf16x8 (&cur)[NI][4], bf16x8 (&nxt)[NI][4]) {
+    // One k-step: the MFMAs of step (chunk ck, G) from LDS buffers G & 1, while this wave's fragments of the
+    // following step are unpacked and published into the other B buffer and the following activations
+    // travel global -> registers -> LDS. The step is cut into its four slices; each slice first reads the
+    // next slice's operands from LDS, then alternates one MFMA with its share of the unpack arithmetic.
+    // Nothing moves between slices.
+    constexpr int VPM = (26 + MI * NI - 1) / (MI * NI);   // VALU instructions issued behind each MFMA
+    auto step = [&](auto Gc, int ck) {
         constexpr int G = decltype(Gc)::value;
         constexpr int GN = (G + 1) & 3;
         constexpr int buf = G & 1;
         // fragments of step G+1 of this chunk, or of step 0 of the next one
         const int pc = G == 3 ? (ck + 1 < c_last ? ck + 1 : c_last) : ck;
         const int nc = pc + 1 < c_last ? pc + 1 : c_last;
-        typename F::Ctx ctx[NI];
-        bf16x8 a[2][SA];
-        auto read_a = [&](int sg, bf16x8 (&dst)[SA]) {
+        typename F::Ctx ctx;
+        bf16x8 a[2][MI], b[2][NI];
+        auto read_ops = [&](int t, bf16x8 (&da)[MI], bf16x8 (&db)[NI]) {
 #pragma unroll
-            for (int u = 0; u < SA; u++) {
-                const int m = sg * SA + u, t = m / MI, i = m % MI;
-                dst[u] = *(const bf16x8*)(&As[buf][a_rd + 32 * i * LDS_ROW + kcol(t, 0)]);
-            }
+            for (int i = 0; i < MI; i++) da[i] = *(const bf16x8*)(&As[buf][a_rd + 32 * i * LDS_ROW + kcol(t, 0)]);
+#pragma unroll
+            for (int j = 0; j < NI; j++) db[j] = *(const bf16x8*)(&Bs[buf][b_rd + (4 * j + t) * FRAG]);
         };
-        read_a(0, a[0]);
+        read_ops(0, a[0], b[0]);
         load_a(4 * ck + G + 1);
-#pragma unroll
-        for (int j = 0; j < NI; j++) F::template begin<GN>(raw[j], pc, h, p.nblk, ctx[j]);
+        F::template begin<GN>(raw, pc, h, p.nblk, ctx);
         __builtin_amdgcn_sched_barrier(0);
-        static_for<0, NSEG>([&](auto S) {
-            constexpr int sg = decltype(S)::value;
-            if constexpr (sg + 1 < NSEG) read_a(sg + 1, a[(sg + 1) & 1]);
+        static_for<0, 4>([&](auto S) {
+            constexpr int t = decltype(S)::value;
+            if constexpr (t < 3) read_ops(t + 1, a[(t + 1) & 1], b[(t + 1) & 1]);
 #pragma unroll
-            for (int u = 0; u < SA; u++) {
-                const int m = sg * SA + u, t = m / MI, i = m % MI;
+            for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < NI; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[sg & 1][u], cur[j][t], acc[i][j], 0, 0, 0);
-            }
-            static_for<0, FPS>([&](auto Kc) {
-                constexpr int f = sg * FPS + decltype(Kc)::value, j = f / 4, T = f % 4;
-                nxt[j][T] = F::template frag<GN, T>(raw[j], ctx[j]);
-            });
-            if constexpr (sg + 1 < NSEG) __builtin_amdgcn_sched_group_barrier(0x100, SA, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t & 1][i], b[t & 1][j], acc[i][j], 0, 0, 0);
+            *(bf16x8*)(&Bs[buf ^ 1][b_wr + t * FRAG]) = F::template frag<GN, t>(raw, ctx);
+            if constexpr (t < 3) __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
 #pragma unroll
-            for (int u = 0; u < SA * NI; u++) {
+            for (int u = 0; u < MI * NI; u++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);
             }
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
             __builtin_amdgcn_sched_barrier(0);
         });
-#pragma unroll
-        for (int j = 0; j < NI; j++) F::template refill<GN>(raw[j], wrow[j], nc, h, p.nblk);
+        F::template refill<GN>(raw, wrow, nc, h, p.nblk);
         store_a(buf ^ 1);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     };
 
     for (int ck = c_begin; ck < c_end; ck++) {
-        step(std::integral_constant<int, 0>{}, ck, bA, bB);
-        step(std::integral_constant<int, 1>{}, ck, bB, bA);
-        step(std::integral_constant<int, 2>{}, ck, bA, bB);
-        step(std::integral_constant<int, 3>{}, ck, bB, bA);
+        step(std::integral_constant<int, 0>{}, ck);
+        step(std::integral_constant<int, 1>{}, ck);
+        step(std::integral_constant<int, 2>{}, ck);
+        step(std::integral_constant<int, 3>{}, ck);
     }
 
     // D layout of the 32x32 MFMA: register r of lane (h, c) is row 8*(r/4) + 4*h + (r%4), column c
@@ -411,59 +432,61 @@ __global__ void __launch_bounds__(256) gemm_q_bf16_kernel(GemmParams p) {
                 const int t = t0 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
                 if (t < p.T) {
                     float* y = p.Y + (size_t)t * p.N + n;
-                    if (p.atomic) unsafeAtomicAdd(y, acc[i][j][r]);
-                    else *y = acc[i][j][r];
+                    if (whole) *y = acc[i][j][r];
+                    else unsafeAtomicAdd(y, acc[i][j][r]);
                 }
             }
         }
+  }
 }
 
-__global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = 0.f;
+// Clears the output tiles that more than one workgroup contributes to (left-over tile `blockIdx.x` is split iff its first
+// and last chunk fall into different runs).
+__global__ void __launch_bounds__(256) zero_split_tiles_kernel(float* __restrict__ Y, int T, int N, int BM, int tiles_n,
+                                                             int nchunks, int per, int first_tile) {
+    const int tile = first_tile + blockIdx.x;
+    const long long u0 = (long long)blockIdx.x * nchunks;
+    if (u0 / per == (u0 + nchunks - 1) / per) return;
+    const int tile_y = tile / tiles_n, tile_x = tile - tile_y * tiles_n;
+    const int col = tile_x * 256 + threadIdx.x;
+    if (col >= N) return;
+    const int t_end = (tile_y + 1) * BM < T ? (tile_y + 1) * BM : T;
+    for (int t = tile_y * BM; t < t_end; t++) Y[(size_t)t * N + col] = 0.f;
 }
 
-template <class F, int MI, int NI>
+template <class F, int MI>
 int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
     GemmParams p;
     p.W = w->d_raw; p.X = d_x; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
     p.nblk = (int)(w->row_bytes / F::BLOCK);
-    const int nchunks = F::chunks(p.K);
-    dim3 grid((unsigned)((w->rows + 128 * NI - 1) / (128 * NI)), (unsigned)((t + 32 * MI - 1) / (32 * MI)), 1);
-    // Workgroups run in rounds of `slots` (one per CU for the 256-row tile, whose accumulators take a SIMD's
-    // whole register file; two otherwise). When the output tiles do not fill the rounds evenly, split K over
-    // grid.z and add the slices into a zeroed Y: pick the split with the least (rounds x chunks per slice),
-    // charging every slice two chunks for its prologue, epilogue and atomic traffic.
-    const int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    const size_t slots = (size_t)cus * (MI >= 8 ? 1 : 2);
-    const size_t tiles = (size_t)grid.x * grid.y;
-    int split = 1;
-    size_t best = 0;
-    for (int sp = 1; sp <= 16 && sp <= nchunks; sp++) {
-        const int cps = (nchunks + sp - 1) / sp;
-        const int z = (nchunks + cps - 1) / cps;
-        const size_t rounds = (tiles * z + slots - 1) / slots;
-        const size_t cost = rounds * (size_t)(cps + (z > 1 ? 2 : 0));
-        if (best == 0 || cost < best) { best = cost; split = sp; }
-    }
-    p.chunks_per_split = (nchunks + split - 1) / split;
-    grid.z = (unsigned)((nchunks + p.chunks_per_split - 1) / p.chunks_per_split);
-    p.atomic = grid.z > 1;
-    if (p.atomic) {
-        size_t n = t * w->rows;
-        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
-    }
-    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI, NI>), grid, dim3(256), 0, s, p);
+    p.nchunks = F::chunks(p.K);
+    p.tiles_n = (int)((w->rows + 255) / 256);
+    const int tiles_t = (int)((t + 64 * MI - 1) / (64 * MI));
+    const long long tiles = (long long)p.tiles_n * tiles_t;
+    // one workgroup per CU (its LDS tiles take most of a CU's 160 KB)
+    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    p.whole_rounds = (int)(tiles / cus);
+    const long long left = tiles - p.whole_rounds * cus;
+    p.units = left * p.nchunks;
+    long long per = (p.units + cus - 1) / cus;
+    // a run shorter than a tile's K that is close to it is rounded up to whole tiles: no atomics, no clearing
+    if (per * 4 >= (long long)p.nchunks * 3) per = p.nchunks;
+    if (per < 1) per = 1;
+    p.per = (int)per;
+    const unsigned grid = p.whole_rounds > 0 ? (unsigned)cus : (unsigned)((p.units + per - 1) / per);
+    if (left > 0 && per % p.nchunks != 0)
+        hipLaunchKernelGGL(zero_split_tiles_kernel, dim3((unsigned)left), dim3(256), 0, s, d_y, p.T, p.N, 64 * MI,
+                           p.tiles_n, p.nchunks, p.per, (int)(p.whole_rounds * cus));
+    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(grid), dim3(512), 0, s, p);
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
 template <class F>
 int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
-    if (t > 128) return launch_cfg<F, 8, 2>(w, d_x, t, d_y, s);  // 256 x 256 workgroup tile
-    if (t > 64) return launch_cfg<F, 4, 2>(w, d_x, t, d_y, s);
-    if (t > 32) return launch_cfg<F, 2, 2>(w, d_x, t, d_y, s);
-    return launch_cfg<F, 1, 2>(w, d_x, t, d_y, s);
+    if (t > 128) return launch_cfg<F, 4>(w, d_x, t, d_y, s);  // 256 x 256 workgroup tile
+    if (t > 64) return launch_cfg<F, 2>(w, d_x, t, d_y, s);
+    return launch_cfg<F, 1>(w, d_x, t, d_y, s);
 }
 
 }  // namespace
@@ -473,6 +496,8 @@ namespace fhip {
 int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
     if (t == 0 || w->rows == 0) return FHIP_OK;
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "gemm_q_bf16: x must be 16-byte aligned");
+    if ((unsigned long long)t * w->cols >= (1ull << 31))
+        return set_error(FHIP_ERR_SHAPE, "gemm_q_bf16: t * cols must be below 2^31 (got %zu x %zu)", t, w->cols);
     switch (w->type) {
         case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s);
         case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s);
