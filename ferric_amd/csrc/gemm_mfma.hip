@@ -8,19 +8,18 @@
 // Shape of the kernel. The reference found this path bound by the unpack arithmetic, not the matrix
 // unit (crates/ferric-core/src/lib.rs:90-101), and the same holds here: a weight costs ~3 VALU
 // operations to turn into bf16, an MFMA retires 16K multiply-adds in 32 cycles. So
-//   * each lane dequantizes straight into the B-operand registers of the MFMA it feeds (the B fragment of
-//     a 32x32x16 MFMA is 8 consecutive k of one weight row per lane, which is 8 consecutive quants of the
-//     GGUF stream: no LDS round trip, no transposition for the weights);
-//   * a dequantized fragment is reused for every 32-row slab of the activation tile the wave owns
-//     (MI slabs, up to 8), so unpack cost is amortised over BM = 32*MI activation rows;
-//   * the fragments of step s+1 are produced while the MFMAs of step s run: the two instruction streams
-//     are independent, and the matrix pipe executes an issued MFMA while the wave goes on issuing VALU work;
-//   * the activation tile, which all 4 waves of a workgroup share, is staged through LDS (padded rows,
-//     16-byte reads) and each fragment read feeds NI MFMAs;
+//   * each lane dequantizes 8 consecutive quants of one weight row, which is exactly the B fragment a lane
+//     holds in a 32x32x16 MFMA: no transposition for the weights;
+//   * a dequantized fragment is published once in LDS and used by both waves of a T-pair for every 32-row
+//     slab they own, so unpack cost is amortised over the workgroup's 64*MI activation rows;
+//   * the fragments of step s+1 are produced while the MFMAs of step s run, one MFMA alternating with its
+//     share of the unpack arithmetic, with two waves per SIMD to fill each other's issue gaps;
+//   * the activation tile, which all 8 waves of a workgroup share, is staged through LDS (padded rows,
+//     16-byte reads);
 //   * the 16 k of one MFMA are chosen inside ONE scale sub-block (the k order inside an MFMA is free as
 //     long as both operands agree), so a fragment needs a single (scale, min) pair;
 //   * weight bytes are fetched a whole 256-column chunk ahead into the registers the previous chunk has
-//     just vacated (consume, then refill), so no load is waited for in the steady state.
+//     just vacated (consume, then refill), so no weight load is waited for in the steady state.
 // One k-step is 64 columns = 4 MFMA slices; a chunk is 4 steps = one K-quant super-block or 8 Q8_0 blocks.
 // Dequantized values are exactly the f32 the CPU dequantizer produces, rounded to bf16 (RNE) by
 // v_cvt_pk_bf16_f32.
@@ -28,6 +27,7 @@
 
 #include <hip/hip_fp16.h>
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -46,6 +46,11 @@ __device__ __forceinline__ uint32_t pk_bf16(float a, float b) {
 }
 // 8 weights w_i = fma(s, q_i, o) from the bytes of two dwords -> one MFMA operand (8 bf16)
 __device__ __forceinline__ bf16x8 frag8(uint32_t q0, uint32_t q1, float s, float o) {
+    // Hide from the optimiser which bits of the bytes are known zero: with that knowledge it narrows every
+    // byte extraction to a bit-field extract and adds one instruction per weight in front of the byte-lane
+    // conversions v_cvt_f32_ubyte0..3, which take the byte lane as it is.
+    asm("" : "+v"(q0));
+    asm("" : "+v"(q1));
     u32x4 r;
     r[0] = pk_bf16(fmaf(s, ub(q0, 0), o), fmaf(s, ub(q0, 1), o));
     r[1] = pk_bf16(fmaf(s, ub(q0, 2), o), fmaf(s, ub(q0, 3), o));
@@ -454,6 +459,172 @@ __global__ void __launch_bounds__(256) zero_split_tiles_kernel(float* __restrict
     for (int t = tile_y * BM; t < t_end; t++) Y[(size_t)t * N + col] = 0.f;
 }
 
+// ------------------------------------------------------------------------------------------------
+// T <= 32 (batched decode, short prompts): one 32-row MFMA slab of activations, so the kernel is bound by
+// the weight stream and its unpack arithmetic, not by the matrix pipe. A workgroup is 4 waves on 4 adjacent
+// 32-row weight blocks; each wave unpacks its own block straight into its B operand (no LDS for weights)
+// with the weight bytes one chunk ahead, the same register image and refill order as the tiled kernel. The
+// activations of a chunk (TP rows x 256 columns, TP = 8 or 32) are staged once per workgroup in LDS, double
+// buffered, one barrier per chunk. The (128-row group, chunk) units, chunk fastest, are dealt to the
+// workgroups in equal contiguous runs, two to four workgroups per CU; a segment that covers its group's whole K
+// stores its tile, any other adds it atomically into a Y cleared beforehand.
+// ------------------------------------------------------------------------------------------------
+struct SkinnyParams {
+    const uint8_t* W;
+    const uint16_t* X;
+    float* Y;
+    int T, N, K;
+    int nblk;
+    size_t row_bytes;
+    int nchunks;
+    long long units;   // 128-row groups * nchunks
+    int per;           // units per workgroup
+};
+
+constexpr int XROW = CHUNK + 8;   // bf16 per staged activation row of a chunk (+16 B pad)
+
+template <class F, int TP>
+__global__ void __launch_bounds__(256, TP == 8 ? 4 : 2) gemm_q_bf16_skinny_kernel(SkinnyParams p) {
+    __shared__ __attribute__((aligned(16))) uint16_t Xs[2][TP * XROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5, c = lane & 31;
+    const int nchunks = p.nchunks;
+    long long u = (long long)blockIdx.x * p.per;
+    const long long u_end = u + p.per < p.units ? u + p.per : p.units;
+    // staging: thread `tid` moves the 16-byte piece (tid & 31) of rows (tid >> 5) + 8q, q < TP / 8; rows past T
+    // repeat row T-1 (their outputs are never stored)
+    constexpr int NQ = TP / 8;
+    const int s_col = (tid & 31) * 8;
+    uint32_t s_src[NQ];
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+        int t = (tid >> 5) + 8 * q;
+        s_src[q] = (uint32_t)(t < p.T ? t : p.T - 1) * (uint32_t)p.K;
+    }
+    const int s_dst = (tid >> 5) * XROW + s_col;
+    const int k_last = p.K - 8;   // a partial last chunk reads earlier columns of the same row (their weights are 0)
+    u32x4 stage[NQ];
+    auto load_x = [&](int ck) {
+        int col = ck * CHUNK + s_col;
+        col = col < k_last ? col : k_last;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) stage[q] = *(const u32x4*)(p.X + (s_src[q] + col));
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < NQ; q++) *(u32x4*)(&Xs[buf][s_dst + 8 * q * XROW]) = stage[q];
+    };
+    const int a_rd = (c & (TP - 1)) * XROW + 16 * h;   // + 64 * step + kcol(t, 0)
+
+    for (int seg = 0; u < u_end; seg++) {
+        const int grp = (int)(u / nchunks);
+        const int c_begin = (int)(u - (long long)grp * nchunks);
+        const int c_end = (long long)(nchunks - c_begin) < u_end - u ? nchunks : c_begin + (int)(u_end - u);
+        u += c_end - c_begin;
+        const bool whole = c_begin == 0 && c_end == nchunks;
+        const int c_last = c_end - 1;
+        const int n = grp * 128 + wave * 32 + c;
+        const uint8_t* wrow = p.W + (size_t)(n < p.N ? n : p.N - 1) * p.row_bytes;
+
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.f;
+        // Weight bytes: the whole next chunk is requested at the top of a chunk, all its loads back to back, so
+        // the two or three cache lines a row's block spans are fetched from L2 once (loads of one block spread
+        // over the chunk's steps would find the line evicted from L1 each time and refetch it).
+        typename F::Raw raw, nxt;
+        bf16x8 a[4], b[4];   // both operands of the step in flight; each slice is replaced as soon as its MFMA has issued
+        F::prime(raw, wrow, c_begin, h, p.nblk);
+        load_x(c_begin);
+        if (seg > 0) __syncthreads();   // the previous segment's last reads of buffer 0 are done
+        store_x(0);
+        {
+            typename F::Ctx x;
+            F::template begin<0>(raw, c_begin, h, p.nblk, x);
+            static_for<0, 4>([&](auto T) { b[T.value] = F::template frag<0, T.value>(raw, x); });
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < 4; t++) a[t] = *(const bf16x8*)(&Xs[0][a_rd + kcol(t, 0)]);
+
+        for (int ck = c_begin; ck < c_end; ck++) {
+            const int buf = (ck - c_begin) & 1;
+            const int cn = ck + 1 < c_end ? ck + 1 : ck;
+            F::prime(nxt, wrow, cn, h, p.nblk);
+            load_x(cn);
+            static_for<0, 4>([&](auto Gc) {
+                constexpr int G = decltype(Gc)::value;
+                constexpr int GN = (G + 1) & 3;
+                typename F::Ctx x;
+                if constexpr (G == 3) {
+                    F::template begin<0>(nxt, cn, h, p.nblk, x);
+                    static_for<0, 4>([&](auto T) {
+                        constexpr int t = decltype(T)::value;
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t], b[t], acc, 0, 0, 0);
+                        b[t] = F::template frag<0, t>(nxt, x);
+                    });
+                    store_x(buf ^ 1);
+                    __syncthreads();
+#pragma unroll
+                    for (int t = 0; t < 4; t++) a[t] = *(const bf16x8*)(&Xs[buf ^ 1][a_rd + kcol(t, 0)]);
+                } else {
+                    F::template begin<GN>(raw, ck, h, p.nblk, x);
+                    static_for<0, 4>([&](auto T) {
+                        constexpr int t = decltype(T)::value;
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t], b[t], acc, 0, 0, 0);
+                        a[t] = *(const bf16x8*)(&Xs[buf][a_rd + KSTEP * (G + 1) + kcol(t, 0)]);
+                        b[t] = F::template frag<GN, t>(raw, x);
+                    });
+                }
+            });
+            raw = nxt;
+        }
+        if (n < p.N) {
+#pragma unroll
+            for (int r = 0; r < (TP == 8 ? 4 : 16); r++) {
+                const int t = 8 * (r >> 2) + 4 * h + (r & 3);
+                if (t < p.T) {
+                    float* y = p.Y + (size_t)t * p.N + n;
+                    if (whole) *y = acc[r];
+                    else unsafeAtomicAdd(y, acc[r]);
+                }
+            }
+        }
+    }
+}
+
+__global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = 0.f;
+}
+
+template <class F>
+int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
+    SkinnyParams p;
+    p.W = w->d_raw; p.X = d_x; p.Y = d_y;
+    p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
+    p.nblk = (int)(w->row_bytes / F::BLOCK);
+    p.nchunks = F::chunks(p.K);
+    const long long groups = ((long long)w->rows + 127) / 128;
+    p.units = groups * p.nchunks;
+    // workgroups per CU as the register budget allows: four with 8 activation rows staged, two with 32
+    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    const long long wgs = cus * (t <= 8 ? 4 : 2);
+    long long per = (p.units + wgs - 1) / wgs;
+    if (per * 4 >= (long long)p.nchunks * 3 && per < p.nchunks) per = p.nchunks;   // nearly whole groups: make them whole
+    if (per < 1) per = 1;
+    if (const char* e = getenv("FHIP_SKINNY_PER")) per = atoi(e) > 0 ? atoi(e) : per;
+    p.per = (int)per;
+    const unsigned grid = (unsigned)((p.units + per - 1) / per);
+    if (per % p.nchunks != 0) {
+        const size_t n = t * w->rows;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
+    }
+    if (t <= 8) hipLaunchKernelGGL((gemm_q_bf16_skinny_kernel<F, 8>), dim3(grid), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((gemm_q_bf16_skinny_kernel<F, 32>), dim3(grid), dim3(256), 0, s, p);
+    return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
+}
+
 template <class F, int MI>
 int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
     GemmParams p;
@@ -484,6 +655,7 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
 
 template <class F>
 int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
+    if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s);
     if (t > 128) return launch_cfg<F, 4>(w, d_x, t, d_y, s);  // 256 x 256 workgroup tile
     if (t > 64) return launch_cfg<F, 2>(w, d_x, t, d_y, s);
     return launch_cfg<F, 1>(w, d_x, t, d_y, s);
