@@ -118,6 +118,16 @@ def bench_ffn(F, lib, check, stream, timer, batches, reps=20):
         g.launch()
         ms = timer.time_ms(g.launch) / reps
         res[str(b)] = {"ms": ms, "weight_GBps": wbytes / (ms * 1e-3) / 1e9, "tokens_per_s": b / (ms * 1e-3)}
+        # the same block through the matrix-core entry point (bf16 operands, f32 accumulate): one pass over
+        # the weights for the whole batch
+        wsb = F.DeviceBuffer(max(256, lib.fhip_ffn_coop_ws_bytes(gu.handle, dn.handle, b)))
+        g = F.Graph.begin(stream)
+        for _ in range(reps):
+            check(lib.fhip_ffn_coop(gu.handle, dn.handle, x.buf.ptr, b, y.buf.ptr, wsb.ptr, stream.handle))
+        g.end()
+        g.launch()
+        ms = timer.time_ms(g.launch) / reps
+        res[str(b)]["matrix_core_path"] = {"ms": ms, "weight_GBps": wbytes / (ms * 1e-3) / 1e9, "tokens_per_s": b / (ms * 1e-3)}
     return res, wbytes
 
 
@@ -159,25 +169,28 @@ def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
 
 
 def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
-    """configs[3]: W 5120x5120 Q4_K, X [T, 5120] bf16 -> f32 [T, 5120] on the matrix cores."""
+    """configs[3]: W 5120x5120 Q4_K, X [T, 5120] bf16 -> f32 [T, 5120] on the matrix cores; and the same on the
+    layer's largest projection (fused gate|up, 34816x5120), where the launch has enough tiles to fill the chip."""
     from ferric_amd.synth import synth_weights
-    n = k = 5120
-    qm = F.QMatrix.from_bytes(synth_weights(Q4_K, n, k, 1), Q4_K, n, k)
     res = {}
-    for t in ts:
-        xf = np.random.default_rng(7).standard_normal((t, k)).astype(np.float32)
-        u = xf.view(np.uint32).astype(np.uint64)
-        xb = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
-        x = F.Tensor.from_bf16_bits(xb, (t, k))
-        y = F.Tensor.empty((t, n))
-        g = F.Graph.begin(stream)
-        for _ in range(reps):
-            check(lib.fhip_gemm_q_bf16(qm.handle, x.buf.ptr, t, y.buf.ptr, stream.handle))
-        g.end()
-        g.launch()
-        ms = timer.time_ms(g.launch) / reps
-        tf = 2.0 * t * n * k / (ms * 1e-3) / 1e12
-        res[str(t)] = {"ms": ms, "TFLOPs": tf, "frac_of_bf16_mfma_peak": tf / 2500.0}
+    for name, n, k in (("5120x5120", 5120, 5120), ("34816x5120", 34816, 5120)):
+        qm = F.QMatrix.from_bytes(synth_weights(Q4_K, n, k, 1), Q4_K, n, k)
+        out = {}
+        for t in ts:
+            xf = np.random.default_rng(7).standard_normal((t, k)).astype(np.float32)
+            u = xf.view(np.uint32).astype(np.uint64)
+            xb = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+            x = F.Tensor.from_bf16_bits(xb, (t, k))
+            y = F.Tensor.empty((t, n))
+            g = F.Graph.begin(stream)
+            for _ in range(reps):
+                check(lib.fhip_gemm_q_bf16(qm.handle, x.buf.ptr, t, y.buf.ptr, stream.handle))
+            g.end()
+            g.launch()
+            ms = timer.time_ms(g.launch) / reps
+            tf = 2.0 * t * n * k / (ms * 1e-3) / 1e12
+            out[str(t)] = {"ms": ms, "TFLOPs": tf, "frac_of_bf16_mfma_peak": tf / 2500.0}
+        res[name] = out
     return res
 
 
@@ -294,7 +307,7 @@ def main():
         line["ffn_q4k_q6k"] = {"weight_bytes": wb, "batch": ffn}
     if not args.no_prefill:
         log("[bench] prefill dequant-GEMM, T = 128/512/2048 ...")
-        line["prefill_q4k_5120_bf16_mfma"] = bench_prefill(F, lib, check, stream, timer)
+        line["prefill_q4k_bf16_mfma"] = bench_prefill(F, lib, check, stream, timer)
     if not args.no_sweep:
         log("[bench] 64-layer decode weight sweep (14.0 GB) ...")
         line["decode_sweep"] = bench_sweep(F, lib, check, stream, timer)

@@ -344,6 +344,53 @@ int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float*
     return fhip::launch_gemm_bf16(w, d_x, t, d_y, (hipStream_t)stream);
 }
 
+int fhip_cvt_f32_bf16(const float* d_x, size_t n, uint16_t* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (n == 0) return FHIP_OK;
+    if (!d_x || !d_out) return set_error(FHIP_ERR_ARG, "fhip_cvt_f32_bf16: NULL pointer");
+    return fhip::launch_cvt_bf16(d_x, n, d_out, (hipStream_t)stream);
+}
+
+int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, uint16_t* d_ws_bf16, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!w) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL weight");
+    if (rows_x == 0 || w->rows == 0) return FHIP_OK;
+    if (!d_x || !d_y || !d_ws_bf16) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL pointer");
+    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * w->cols, d_ws_bf16, (hipStream_t)stream))) return rc;
+    return fhip::launch_gemm_bf16(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream);
+}
+
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+size_t fhip_ffn_coop_ws_bytes(const fhip_weight* gu, const fhip_weight* down, size_t rows_x) {
+    if (!gu || !down) return 0;
+    return align256(rows_x * gu->cols * 2) + align256(rows_x * gu->rows * 4) + align256(rows_x * down->cols * 2);
+}
+
+int fhip_ffn_coop(const fhip_weight* gu, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y,
+                  void* d_ws, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!gu || !down) return set_error(FHIP_ERR_ARG, "fhip_ffn_coop: NULL weight");
+    if (gu->rows % 2 != 0) return set_error(FHIP_ERR_SHAPE, "fhip_ffn_coop: gate_up rows must be even");
+    const size_t n_ff = gu->rows / 2;
+    if (down->cols != n_ff) return set_error(FHIP_ERR_SHAPE, "down in dim must equal n_ff");
+    if (rows_x == 0) return FHIP_OK;
+    if (!d_x || !d_y || !d_ws) return set_error(FHIP_ERR_ARG, "fhip_ffn_coop: NULL pointer");
+    if (((uintptr_t)d_ws & 255) != 0) return set_error(FHIP_ERR_ARG, "fhip_ffn_coop: workspace must be 256-byte aligned");
+    uint8_t* ws = (uint8_t*)d_ws;
+    uint16_t* xb = (uint16_t*)ws;
+    float* g = (float*)(ws + align256(rows_x * gu->cols * 2));
+    uint16_t* hb = (uint16_t*)((uint8_t*)g + align256(rows_x * gu->rows * 4));
+    hipStream_t s = (hipStream_t)stream;
+    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * gu->cols, xb, s))) return rc;
+    if ((rc = fhip::launch_gemm_bf16(gu, xb, rows_x, g, s))) return rc;
+    if ((rc = fhip::launch_swiglu_bf16(g, rows_x, n_ff, hb, s))) return rc;
+    return fhip::launch_gemm_bf16(down, hb, rows_x, d_y, s);
+}
+
 int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, size_t rows, size_t cols, float* h_y) {
     int rc = need_init();
     if (rc) return rc;

@@ -37,5 +37,7 @@ int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream
 
 // gemm_mfma.hip
 int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s);
+int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s);
+int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s);
 
 }  // namespace fhip

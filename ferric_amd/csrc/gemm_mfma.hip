@@ -661,9 +661,45 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     return launch_cfg<F, 1>(w, d_x, t, d_y, s);
 }
 
+// f32 -> bf16 (round to nearest even), 8 values per thread; `n8` full groups of 8, the tail one by one
+__global__ void __launch_bounds__(256) cvt_f32_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, size_t n) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i + 8 <= n) {
+        const float4 a = *(const float4*)(x + i), b = *(const float4*)(x + i + 4);
+        u32x4 r = {pk_bf16(a.x, a.y), pk_bf16(a.z, a.w), pk_bf16(b.x, b.y), pk_bf16(b.z, b.w)};
+        *(u32x4*)(out + i) = r;
+    } else {
+        for (size_t k = i; k < n; k++) out[k] = (uint16_t)(pk_bf16(x[k], 0.f) & 0xFFFFu);
+    }
+}
+
+// SwiGLU of a [t, 2d] = [gate | up] f32 matrix, written as bf16 [t, d] for the down projection's A operand.
+// Same arithmetic as the un-fused f32 op (crates/ferric-tensor/src/lib.rs:2603-2618), then one RNE rounding.
+__global__ void __launch_bounds__(256) swiglu_bf16_kernel(const float* __restrict__ gu, size_t n, size_t d, uint16_t* __restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t row = i / d, col = i % d;
+    const float g = gu[row * 2 * d + col], u = gu[row * 2 * d + d + col];
+    out[i] = (uint16_t)(pk_bf16((g / (1.0f + expf(-g))) * u, 0.f) & 0xFFFFu);
+}
+
 }  // namespace
 
 namespace fhip {
+
+int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s) {
+    const size_t n = t * d;
+    if (n == 0) return FHIP_OK;
+    hipLaunchKernelGGL(swiglu_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gu, n, d, d_out);
+    return check_hip(hipGetLastError(), "swiglu_bf16 launch");
+}
+
+int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s) {
+    if (n == 0) return FHIP_OK;
+    if ((((uintptr_t)d_x | (uintptr_t)d_out) & 15) != 0) return set_error(FHIP_ERR_ARG, "cvt_f32_bf16: pointers must be 16-byte aligned");
+    hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s, d_x, d_out, n);
+    return check_hip(hipGetLastError(), "cvt_f32_bf16 launch");
+}
 
 int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
     if (t == 0 || w->rows == 0) return FHIP_OK;

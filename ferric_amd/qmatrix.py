@@ -206,6 +206,55 @@ class Tensor:
         out._keepalive = ws  # scratch must outlive the enqueued work
         return out
 
+    def cvt_bf16(self, stream=None):
+        """f32 -> bf16 bit patterns (round to nearest even), same shape."""
+        assert self.dtype == np.float32
+        n = self.numel()
+        out = Tensor(DeviceBuffer(max(16, 2 * n)), self.shape, np.uint16)
+        _lib.check(_lib.load().fhip_cvt_f32_bf16(self.buf.ptr, n, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def matmul_q_coop(self, w, stream=None):
+        """f32 x [rows, in] @ W^T on the matrix cores -- dtype.rs:1818 matmul_q4_k_coop / :1199 / :1316."""
+        assert self.dtype == np.float32, "matmul_q_coop expects f32 activations"
+        rows, inn = self._rows_inner()
+        assert inn == w.cols(), "inner dim mismatch"
+        assert w.rows() % 8 == 0, "matmul_q_coop needs N (out) a multiple of 8"   # dtype.rs:1822
+        out = Tensor.empty((rows, w.rows()))
+        ws = DeviceBuffer(max(16, rows * inn * 2))
+        _lib.check(_lib.load().fhip_matmul_q_coop(w.handle, self.buf.ptr, rows, out.buf.ptr, ws.ptr, _stream_handle(stream)))
+        if stream is not None:
+            stream.synchronize()      # ws is freed on return
+        else:
+            _lib.check(_lib.load().fhip_stream_sync(None))
+        return out
+
+    def matmul_q4_k_coop(self, w, stream=None):
+        assert w.ggml_type == 12
+        return self.matmul_q_coop(w, stream)
+
+    def matmul_q6_k_coop(self, w, stream=None):
+        assert w.ggml_type == 14
+        return self.matmul_q_coop(w, stream)
+
+    def matmul_q8_0_coop(self, w, stream=None):
+        assert w.ggml_type == 8
+        return self.matmul_q_coop(w, stream)
+
+    def ffn_coop(self, gate_up, down, stream=None):
+        """down(swiglu(gate_up(x))) on the matrix cores, for a batch of rows -- qwen3.rs:944-964 over dtype.rs:1818."""
+        rows, inn = self._rows_inner()
+        assert inn == gate_up.cols(), "inner dim mismatch"
+        lib = _lib.load()
+        ws = DeviceBuffer(max(256, lib.fhip_ffn_coop_ws_bytes(gate_up.handle, down.handle, rows)))
+        out = Tensor.empty((rows, down.rows()))
+        _lib.check(lib.fhip_ffn_coop(gate_up.handle, down.handle, self.buf.ptr, rows, out.buf.ptr, ws.ptr, _stream_handle(stream)))
+        if stream is not None:
+            stream.synchronize()      # ws is freed on return
+        else:
+            _lib.check(lib.fhip_stream_sync(None))
+        return out
+
     def gemm_q_bf16(self, w, stream=None):
         """Prefill: self holds bf16 bit patterns [t, in]; y f32 [t, out] via the matrix cores -- dtype.rs:1818."""
         assert self.dtype == np.uint16, "gemm_q_bf16 expects bf16 bit patterns"

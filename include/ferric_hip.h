@@ -163,6 +163,26 @@ int fhip_ffn(const fhip_weight* gate_up, const fhip_weight* down, const float* d
  * dequantized tile by tile into LDS as bf16 and contracted on the matrix cores, f32 accumulate. */
 int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x_bf16, size_t t, float* d_y, void* stream);
 
+/* f32 -> bf16 bit patterns, round to nearest even, n values (both pointers 16-byte aligned). The reference's
+ * matrix-unit kernels read f32 activations (crates/ferric-tensor/src/dtype.rs:1824-1830, `xp.buf`); the
+ * matrix cores here take bf16, so this is the conversion in front of fhip_gemm_q_bf16. */
+int fhip_cvt_f32_bf16(const float* d_x, size_t n, uint16_t* d_out_bf16, void* stream);
+
+/* crates/ferric-tensor/src/dtype.rs:1818 Tensor::matmul_q4_k_coop(w) (:1199 matmul_q6_k_coop, :1316
+ * matmul_q8_0_coop) with the reference's own operand types: x f32 [rows_x, cols] -> y f32 [rows_x, rows].
+ * Converts x into the caller's scratch d_ws_bf16 (rows_x * cols 16-bit values, 16-byte aligned) and runs
+ * fhip_gemm_q_bf16 on it. Any rows_x (no padding to 8 as at dtype.rs:1823: the kernel masks). */
+int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, uint16_t* d_ws_bf16,
+                       void* stream);
+
+/* The FFN block of crates/ferric-llama/src/qwen3.rs:944-964 built from the matrix-unit matmuls
+ * (crates/ferric-tensor/src/dtype.rs:1818, :1199, :1316) for a batch of rows: x f32 -> bf16, gate_up GEMM,
+ * SwiGLU rounded to bf16, down GEMM, y f32 [rows_x, down rows]. d_ws: caller-provided scratch of
+ * fhip_ffn_coop_ws_bytes(...) bytes, 256-byte aligned. Any of the three formats for either weight. */
+size_t fhip_ffn_coop_ws_bytes(const fhip_weight* gate_up, const fhip_weight* down, size_t rows_x);
+int fhip_ffn_coop(const fhip_weight* gate_up, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y,
+                  void* d_ws, void* stream);
+
 /* crates/ferric-tensor/src/cpu_simd.rs:79 matvec_q8_0(x, w, rows, cols) with HOST buffers on both
  * sides (upload, GEMV, download, synchronise) -- the drop-in for the CPU mat-vec call.
  * Errors as the reference's asserts: cols % 32, w_len != rows * cols/32*34 -> FHIP_ERR_SHAPE. */

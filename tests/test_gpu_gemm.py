@@ -89,6 +89,58 @@ def test_q8_0_rows_ending_inside_a_chunk(F, O):
         run_case(F, O, Q8_0, t, n, k, 40 + i)
 
 
+def test_coop_entry_takes_f32_activations(F, O):
+    # dtype.rs:1818 matmul_q4_k_coop reads f32 x; here x is rounded to bf16 (RNE) on the device first. The
+    # rounding is checked bit for bit, the product against the bf16 entry point fed host-rounded activations
+    # (equal up to the order in which K slices are added when the launch splits K).
+    from ferric_amd.synth import synth_weights
+    for ty, name, (t, n, k) in [(Q4_K, "matmul_q4_k_coop", (8, 512, 1024)), (Q6_K, "matmul_q6_k_coop", (4, 256, 512)),
+                                (Q8_0, "matmul_q8_0_coop", (21, 264, 416)), (Q4_K, "matmul_q4_k_coop", (150, 384, 768))]:
+        w = synth_weights(ty, n, k, 60)
+        qm = F.QMatrix.from_bytes(w, ty, n, k)
+        x = (np.random.default_rng(61).standard_normal((t, k)) * 3).astype(np.float32)
+        x[0, :4] = [0.0, -0.0, 1.00390625, 1.01171875]   # exact ties, to even both ways
+        xb, _ = bf16_round(x)
+        xt = F.Tensor.from_vec(x.reshape(-1), (t, k))
+        assert np.array_equal(xt.cvt_bf16().to_vec().reshape(t, k), xb)
+        want = F.Tensor.from_bf16_bits(xb, (t, k)).gemm_q_bf16(qm).to_vec()
+        got = getattr(xt, name)(qm).to_vec()
+        assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max(), name
+    odd = np.arange(13, dtype=np.float32) * 1.001      # a length that is not a multiple of 8: the scalar tail
+    odd[:5] = [3.0e38, -3.3895314e38, 1e-40, -65280.0, np.inf]   # near and past the largest bf16, a denormal
+    assert np.array_equal(F.Tensor.from_vec(odd, (1, 13)).cvt_bf16().to_vec(), bf16_round(odd)[0])
+    with pytest.raises(AssertionError, match="multiple of 8"):
+        qm = F.QMatrix.from_bytes(synth_weights(Q4_K, 12, 256, 1), Q4_K, 12, 256)
+        F.Tensor.from_vec(np.zeros(256, np.float32), (1, 256)).matmul_q4_k_coop(qm)
+
+
+def test_batched_decode_ffn_on_the_matrix_cores(F, O):
+    # FFN block at batch 4 and 8 through the coop entry points: gate_up -> swiglu -> down, against f64 on
+    # oracle-dequantized weights, to the north-star bound applied to each matmul
+    from ferric_amd.synth import synth_weights
+    d, n_ff = 1024, 2816
+    gu = synth_weights(Q4_K, 2 * n_ff, d, 70)
+    dn = synth_weights(Q6_K, d, n_ff, 71)
+    qgu, qdn = F.QMatrix.from_bytes(gu, Q4_K, 2 * n_ff, d), F.QMatrix.from_bytes(dn, Q6_K, d, n_ff)
+    wgu = O.deq_raw(gu, 2 * n_ff * d, Q4_K).reshape(2 * n_ff, d).astype(np.float64)
+    wdn = O.deq_raw(dn, d * n_ff, Q6_K).reshape(d, n_ff).astype(np.float64)
+    for b in (4, 8):
+        x = np.random.default_rng(72 + b).standard_normal((b, d)).astype(np.float32)
+        g = F.Tensor.from_vec(x.reshape(-1), (b, d)).matmul_q4_k_coop(qgu)
+        g64 = x.astype(np.float64) @ wgu.T
+        bound = 1e-3 * np.linalg.norm(wgu, axis=1)[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None]
+        assert (np.abs(g.to_vec().reshape(b, -1) - g64) <= bound).all()
+        hid = g.swiglu(n_ff)
+        hv = hid.to_vec().reshape(b, n_ff)
+        y = hid.matmul_q6_k_coop(qdn).to_vec().reshape(b, d)
+        y64 = hv.astype(np.float64) @ wdn.T
+        bound = 1e-3 * np.linalg.norm(wdn, axis=1)[None, :] * np.linalg.norm(hv.astype(np.float64), axis=1)[:, None]
+        assert (np.abs(y - y64) <= bound).all()
+        # the one-call block does the same steps (the SwiGLU output is rounded to bf16 either way)
+        y1 = F.Tensor.from_vec(x.reshape(-1), (b, d)).ffn_coop(qgu, qdn).to_vec().reshape(b, d)
+        assert np.abs(y1 - y).max() <= 2e-5 * np.abs(y).max()
+
+
 def test_gemm_errors(F):
     qm = F.QMatrix.from_bytes(np.zeros(144, np.uint8), Q4_K, 1, 256)
     with pytest.raises(AssertionError, match="inner dim mismatch"):
