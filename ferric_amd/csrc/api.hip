@@ -358,8 +358,10 @@ int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, fl
     if (!w) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL weight");
     if (rows_x == 0 || w->rows == 0) return FHIP_OK;
     if (!d_x || !d_y || !d_ws_bf16) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL pointer");
-    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * w->cols, d_ws_bf16, (hipStream_t)stream))) return rc;
-    return fhip::launch_gemm_bf16(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream);
+    const bool clr = fhip::gemm_bf16_adds_into_y(rows_x);
+    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * w->cols, d_ws_bf16, (hipStream_t)stream, clr ? d_y : nullptr, clr ? rows_x * w->rows : 0)))
+        return rc;
+    return fhip::launch_gemm_bf16(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream, clr);
 }
 
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -385,10 +387,11 @@ int fhip_ffn_coop(const fhip_weight* gu, const fhip_weight* down, const float* d
     float* g = (float*)(ws + align256(rows_x * gu->cols * 2));
     uint16_t* hb = (uint16_t*)((uint8_t*)g + align256(rows_x * gu->rows * 4));
     hipStream_t s = (hipStream_t)stream;
-    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * gu->cols, xb, s))) return rc;
-    if ((rc = fhip::launch_gemm_bf16(gu, xb, rows_x, g, s))) return rc;
-    if ((rc = fhip::launch_swiglu_bf16(g, rows_x, n_ff, hb, s))) return rc;
-    return fhip::launch_gemm_bf16(down, hb, rows_x, d_y, s);
+    const bool clr = fhip::gemm_bf16_adds_into_y(rows_x);   // then each conversion clears the next GEMM's output on the side
+    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * gu->cols, xb, s, clr ? g : nullptr, clr ? rows_x * gu->rows : 0))) return rc;
+    if ((rc = fhip::launch_gemm_bf16(gu, xb, rows_x, g, s, clr))) return rc;
+    if ((rc = fhip::launch_swiglu_bf16(g, rows_x, n_ff, hb, s, clr ? d_y : nullptr, clr ? rows_x * down->rows : 0))) return rc;
+    return fhip::launch_gemm_bf16(down, hb, rows_x, d_y, s, clr);
 }
 
 int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, size_t rows, size_t cols, float* h_y) {

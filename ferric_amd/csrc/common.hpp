@@ -36,8 +36,12 @@ int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, f
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s);
 
 // gemm_mfma.hip
-int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s);
-int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s);
-int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s);
+// y_cleared: the caller has zeroed y on this stream already (see gemm_bf16_adds_into_y)
+int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared = false);
+bool gemm_bf16_adds_into_y(size_t t);   // true: a launch for t rows may add into y, so a cleared y saves it a launch
+// conversions in front of the GEMM; each can also clear `zero_n` floats at `zero`
+int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s, float* zero = nullptr, size_t zero_n = 0);
+int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s, float* zero = nullptr,
+                       size_t zero_n = 0);
 
 }  // namespace fhip

@@ -599,7 +599,7 @@ __global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
 }
 
 template <class F>
-int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
+int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
     SkinnyParams p;
     p.W = w->d_raw; p.X = d_x; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
@@ -616,7 +616,7 @@ int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_
     if (const char* e = getenv("FHIP_SKINNY_PER")) per = atoi(e) > 0 ? atoi(e) : per;
     p.per = (int)per;
     const unsigned grid = (unsigned)((p.units + per - 1) / per);
-    if (per % p.nchunks != 0) {
+    if (per % p.nchunks != 0 && !y_cleared) {
         const size_t n = t * w->rows;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
     }
@@ -654,16 +654,25 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
 }
 
 template <class F>
-int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
-    if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s);
+int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+    if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, y_cleared);
     if (t > 128) return launch_cfg<F, 4>(w, d_x, t, d_y, s);  // 256 x 256 workgroup tile
     if (t > 64) return launch_cfg<F, 2>(w, d_x, t, d_y, s);
     return launch_cfg<F, 1>(w, d_x, t, d_y, s);
 }
 
 // f32 -> bf16 (round to nearest even), 8 values per thread; `n8` full groups of 8, the tail one by one
-__global__ void __launch_bounds__(256) cvt_f32_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, size_t n) {
+// Both conversion kernels can clear a f32 region on the side (`zero`, `zero_n` values): the output of the
+// T <= 32 GEMM that follows, which adds K slices atomically, so that it needs no clearing launch of its own.
+__device__ __forceinline__ void zero_on_the_side(float* __restrict__ zero, size_t zero_n) {
+    for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < zero_n; k += (size_t)gridDim.x * blockDim.x) zero[k] = 0.f;
+}
+
+__global__ void __launch_bounds__(256) cvt_f32_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, size_t n,
+                                                         float* __restrict__ zero, size_t zero_n) {
+    zero_on_the_side(zero, zero_n);
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i >= n) return;
     if (i + 8 <= n) {
         const float4 a = *(const float4*)(x + i), b = *(const float4*)(x + i + 4);
         u32x4 r = {pk_bf16(a.x, a.y), pk_bf16(a.z, a.w), pk_bf16(b.x, b.y), pk_bf16(b.z, b.w)};
@@ -675,7 +684,9 @@ __global__ void __launch_bounds__(256) cvt_f32_bf16_kernel(const float* __restri
 
 // SwiGLU of a [t, 2d] = [gate | up] f32 matrix, written as bf16 [t, d] for the down projection's A operand.
 // Same arithmetic as the un-fused f32 op (crates/ferric-tensor/src/lib.rs:2603-2618), then one RNE rounding.
-__global__ void __launch_bounds__(256) swiglu_bf16_kernel(const float* __restrict__ gu, size_t n, size_t d, uint16_t* __restrict__ out) {
+__global__ void __launch_bounds__(256) swiglu_bf16_kernel(const float* __restrict__ gu, size_t n, size_t d, uint16_t* __restrict__ out,
+                                                        float* __restrict__ zero, size_t zero_n) {
+    zero_on_the_side(zero, zero_n);
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const size_t row = i / d, col = i % d;
@@ -687,29 +698,31 @@ __global__ void __launch_bounds__(256) swiglu_bf16_kernel(const float* __restric
 
 namespace fhip {
 
-int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s) {
+int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s, float* zero, size_t zero_n) {
     const size_t n = t * d;
     if (n == 0) return FHIP_OK;
-    hipLaunchKernelGGL(swiglu_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gu, n, d, d_out);
+    hipLaunchKernelGGL(swiglu_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gu, n, d, d_out, zero, zero_n);
     return check_hip(hipGetLastError(), "swiglu_bf16 launch");
 }
 
-int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s) {
+int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s, float* zero, size_t zero_n) {
     if (n == 0) return FHIP_OK;
     if ((((uintptr_t)d_x | (uintptr_t)d_out) & 15) != 0) return set_error(FHIP_ERR_ARG, "cvt_f32_bf16: pointers must be 16-byte aligned");
-    hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s, d_x, d_out, n);
+    hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s, d_x, d_out, n, zero, zero_n);
     return check_hip(hipGetLastError(), "cvt_f32_bf16 launch");
 }
 
-int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
+bool gemm_bf16_adds_into_y(size_t t) { return t <= 32; }
+
+int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
     if (t == 0 || w->rows == 0) return FHIP_OK;
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "gemm_q_bf16: x must be 16-byte aligned");
     if ((unsigned long long)t * w->cols >= (1ull << 31))
         return set_error(FHIP_ERR_SHAPE, "gemm_q_bf16: t * cols must be below 2^31 (got %zu x %zu)", t, w->cols);
     switch (w->type) {
-        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s);
-        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s);
-        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_x, t, d_y, s);
+        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s, y_cleared);
+        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s, y_cleared);
+        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_x, t, d_y, s, y_cleared);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }
