@@ -219,6 +219,21 @@ def probe(F, lib, check):
     check(lib.fhip_stream_sync(None))
 
 
+def probe_prefill(F, lib, check):
+    """Work for a profiler run of the matrix-core kernels: Q4_K 5120x5120 and 34816x5120 at T = 2048 (tiled kernel),
+    T = 128 (tiled, K split) and T = 8 (the T <= 32 kernel), 5 launches each."""
+    from ferric_amd.synth import synth_weights
+    for n, k in ((5120, 5120), (34816, 5120)):
+        qm = F.QMatrix.from_bytes(synth_weights(Q4_K, n, k, 1), Q4_K, n, k)
+        for t in (2048, 128, 8):
+            xb = (np.random.default_rng(7).standard_normal((t, k)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+            x = F.Tensor.from_bf16_bits(xb, (t, k))
+            y = F.Tensor.empty((t, n))
+            for _ in range(5):
+                check(lib.fhip_gemm_q_bf16(qm.handle, x.buf.ptr, t, y.buf.ptr, None))
+            check(lib.fhip_stream_sync(None))
+
+
 def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
     """The reference's CPU route for Q4_K (deq_raw then a sequential f32 dot per row, rows split in
     contiguous spans over threads), timed through the C oracle on this host's cores."""
@@ -258,6 +273,9 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for rocprofv3 --pmc: one 256 MiB device copy (calibration), then 16 cold Q4_K 5120x5120 "
                          "GEMVs, one fused gate|up 34816x5120 and one Q6_K 5120x17408 GEMV; prints nothing else")
+    ap.add_argument("--probe-prefill", action="store_true",
+                    help="profiler probe for the matrix-core GEMM: Q4_K 5120x5120 and 34816x5120 at T = 2048, 128 and 8, "
+                         "5 launches each; prints nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, not code")
@@ -272,6 +290,9 @@ def main():
     rows = cols = 5120
     if args.probe:
         probe(F, lib, check)
+        return
+    if args.probe_prefill:
+        probe_prefill(F, lib, check)
         return
     log("[bench] Q4_K GEMV 5120x5120 ...")
     c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
