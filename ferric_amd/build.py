@@ -24,6 +24,7 @@ UNITS = {
     "gemv.hip": [],
     "gemv_generic.hip": [],
     "gemm_mfma.hip": [],
+    "moe.hip": [],
 }
 
 

@@ -344,6 +344,69 @@ int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float*
     return fhip::launch_gemm_bf16(w, d_x, t, d_y, (hipStream_t)stream);
 }
 
+// ---- mixture-of-experts entry points (crates/ferric-tensor/src/dtype.rs:1582-1780) ----------------------
+
+int fhip_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t n_expert, size_t k, int sigmoid, float scale, int norm,
+                  float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (k < 1 || k > 8) return set_error(FHIP_ERR_SHAPE, "k must be 1..=8");                                   // dtype.rs:1599
+    if (n_expert > 1024) return set_error(FHIP_ERR_SHAPE, "moe_topk: n_expert <= 1024 (single-thread scan)");   // dtype.rs:1600
+    if (n_expert == 0) return set_error(FHIP_ERR_SHAPE, "moe_topk: n_expert must be positive");
+    if (t == 0) return FHIP_OK;
+    if (!d_logits || !d_out) return set_error(FHIP_ERR_ARG, "fhip_moe_topk: NULL pointer");
+    return fhip::launch_moe_topk(d_logits, d_bias, t, n_expert, (int)k, sigmoid != 0, scale, norm != 0, d_out, (hipStream_t)stream);
+}
+
+static int sel_checks(const char* who, const fhip_weight* w, size_t k, size_t expert_rows, fhip::SelParams* sel) {
+    if (!w) return set_error(FHIP_ERR_ARG, "%s: NULL weight", who);
+    if (k < 1 || k > 8) return set_error(FHIP_ERR_SHAPE, "k must be 1..=8");
+    if (expert_rows == 0 || w->rows % expert_rows != 0)
+        return set_error(FHIP_ERR_SHAPE, "%s: weight rows %zu are not a whole number of experts of %zu rows", who, w->rows, expert_rows);
+    sel->k = (int)k;
+    sel->n_expert = (int)(w->rows / expert_rows);
+    sel->expert_rows = expert_rows;
+    return FHIP_OK;
+}
+
+int fhip_matmul_q_swiglu_id(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t eff, float* d_y,
+                            void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    fhip::SelParams sel{};
+    if ((rc = sel_checks("matmul_q_swiglu_id", w, k, 2 * eff, &sel))) return rc;
+    if (t == 0) return FHIP_OK;
+    if (!d_x || !d_selw || !d_y) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu_id: NULL pointer");
+    if (((uintptr_t)d_x & 15) != 0 || (w->cols * 4) % 16 != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu_id: x rows must be 16-byte aligned");
+    sel.selw = d_selw; sel.x_per_pair = 0; sel.y_stride = eff; sel.npairs = (int)(t * k);
+    return fhip::launch_gemv_sel(w, d_x, d_y, eff, true, sel, (hipStream_t)stream);
+}
+
+int fhip_matmul_q_id(const fhip_weight* w, const float* d_x, const float* d_selw, size_t k, size_t out_pe, float* d_y, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    fhip::SelParams sel{};
+    if ((rc = sel_checks("matmul_q_id", w, k, out_pe, &sel))) return rc;
+    if (!d_x || !d_selw || !d_y) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_id: NULL pointer");
+    if (((uintptr_t)d_x & 15) != 0 || (w->cols * 4) % 16 != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_id: x rows must be 16-byte aligned");
+    sel.selw = d_selw; sel.x_per_pair = 1; sel.y_stride = out_pe; sel.npairs = (int)k;
+    return fhip::launch_gemv_sel(w, d_x, d_y, out_pe, false, sel, (hipStream_t)stream);
+}
+
+int fhip_matmul_q_id_wsum(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t out_pe, float* d_y,
+                          float* d_ws, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    fhip::SelParams sel{};
+    if ((rc = sel_checks("matmul_q_id_wsum", w, k, out_pe, &sel))) return rc;
+    if (t == 0) return FHIP_OK;
+    if (!d_x || !d_selw || !d_y || !d_ws) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_id_wsum: NULL pointer");
+    if (((uintptr_t)d_x & 15) != 0 || (w->cols * 4) % 16 != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_id_wsum: x rows must be 16-byte aligned");
+    sel.selw = d_selw; sel.x_per_pair = 1; sel.y_stride = out_pe; sel.npairs = (int)(t * k);
+    if ((rc = fhip::launch_gemv_sel(w, d_x, d_ws, out_pe, false, sel, (hipStream_t)stream))) return rc;
+    return fhip::launch_moe_wsum(d_ws, d_selw, t, (int)k, out_pe, d_y, (hipStream_t)stream);
+}
+
 int fhip_cvt_f32_bf16(const float* d_x, size_t n, uint16_t* d_out, void* stream) {
     int rc = need_init();
     if (rc) return rc;

@@ -18,6 +18,33 @@ struct fhip_weight {
 
 namespace fhip {
 
+// Expert selection for the mixture-of-experts "_id" matmuls (crates/ferric-tensor/src/dtype.rs:2463-2700).
+// The weight is a slab of n_expert experts of `expert_rows` rows each. The launch is replicated over `npairs`
+// (token, slot) pairs along grid.y; pair p = ti * k + s uses expert e = selw[ti*2k + k + s] (the index half of a
+// moe_topk row, stored as f32), activation row (x_per_pair ? p : ti) and writes at y + p * y_stride.
+// selw == nullptr: a plain launch.
+struct SelParams {
+    const float* selw;
+    int k, n_expert;
+    size_t expert_rows;
+    int x_per_pair;
+    size_t y_stride;
+    int npairs;
+};
+// applied at the top of a kernel: moves the three base pointers to this y-slice's expert / row / output
+template <class P>
+__device__ __forceinline__ void apply_selection(P& p) {
+    if (p.sel.selw) {
+        const int pair = blockIdx.y, ti = pair / p.sel.k, s = pair - ti * p.sel.k;
+        int e = (int)p.sel.selw[(size_t)ti * 2 * p.sel.k + p.sel.k + s];
+        e = e < 0 ? 0 : (e >= p.sel.n_expert ? p.sel.n_expert - 1 : e);   // a corrupt index must not leave the slab
+        e = __builtin_amdgcn_readfirstlane(e);
+        p.W += (size_t)e * p.sel.expert_rows * p.row_bytes;
+        p.x += (size_t)(p.sel.x_per_pair ? pair : ti) * p.cols;
+        p.y += (size_t)pair * p.sel.y_stride;
+    }
+}
+
 int set_error(int code, const char* fmt, ...);
 int check_hip(hipError_t e, const char* what);
 int device_cus();
@@ -34,6 +61,17 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
 // gemv_generic.hip: same contract, any cols the format allows (up to 32768)
 int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s);
+// One batch-1 GEMV per (token, slot) pair on the selected expert's `out_rows` rows (fused SwiGLU over its
+// gate|up halves when swiglu: then expert_rows = 2 * out_rows). Both files provide it, same contract as above.
+int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel,
+                    hipStream_t s);
+int launch_gemv_generic_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu,
+                            const SelParams& sel, hipStream_t s);
+
+// moe.hip
+int launch_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t ne, int k, int sigmoid, float scale, int norm,
+                    float* d_out, hipStream_t s);
+int launch_moe_wsum(const float* d_parts, const float* d_selw, size_t t, int k, size_t out_pe, float* d_y, hipStream_t s);
 
 // gemm_mfma.hip
 // y_cleared: the caller has zeroed y on this stream already (see gemm_bf16_adds_into_y)

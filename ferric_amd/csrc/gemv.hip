@@ -276,6 +276,7 @@ struct GemvParams {
     int RF;              // replicas of the full-wave set, each taking every RF-th row (balances them against the tail wave)
     int G;               // row groups per workgroup
     int rpg;             // output rows per row group
+    fhip::SelParams sel; // expert selection (selw == nullptr: none)
 };
 
 // Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 768 -> 168, 512 -> 256).
@@ -291,6 +292,7 @@ template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
 template <class F, int M, int U, bool SWIGLU>
 __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    fhip::apply_selection(p);
     constexpr int VPR = SWIGLU ? 2 : 1;       // weight rows walked per output row
     constexpr int RUN = F::RUN, NRUN = F::NRUN, RD = RUN / 4;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -528,7 +530,7 @@ size_t lds_bytes(size_t cols, int NG, int G, int rpg) {
 }
 
 template <class F, int M, bool SWIGLU>
-int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s) {
+int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr) {
     static const int tune_g = env_int("FHIP_GEMV_G", 0), tune_rpg = env_int("FHIP_GEMV_RPG", 0);
     constexpr int U = rows_in_flight<F>(M);
     auto kernel = gemv_stream_kernel<F, M, U, SWIGLU>;
@@ -542,6 +544,7 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
     p.pair_bytes = SWIGLU ? out_rows * w->row_bytes : 0;
+    p.sel = sel ? *sel : fhip::SelParams{nullptr, 0, 0, 0, 0, 0, 1};
     p.NG = (int)(w->cols / (16 * F::WPL));
     constexpr int MAXW = max_threads(M) / 64;
     p.RF = full_wave_replicas(p.NG, MAXW);
@@ -552,7 +555,8 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     // CU with up to RPG_MAX rows per row group, more rounds of equal size only beyond that. With a
     // partly filled single round the row groups are spread over all CUs.
     constexpr int RPG_MAX = 256;
-    const int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    if (p.sel.npairs > 1) cus = cus / p.sel.npairs > 0 ? cus / p.sel.npairs : 1;   // the pairs of an "_id" launch share the chip
     int Gcap = MAXW / WPR;
     if (Gcap < 1) Gcap = 1;
     const size_t slots = (size_t)cus * Gcap;
@@ -567,7 +571,7 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     const size_t per_wg = (size_t)G * rpg;
     const size_t grid = (out_rows + per_wg - 1) / per_wg;
     const size_t lds = lds_bytes<F, M, SWIGLU>(w->cols, p.NG, G, rpg);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(64 * WPR * G), lds, s, p);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid, (unsigned)p.sel.npairs), dim3(64 * WPR * G), lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
 }
 
@@ -624,6 +628,24 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
         case FHIP_Q8_0:
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for Q8_0");
             return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+        default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
+    }
+}
+
+template <class F>
+int launch_sel_fmt(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel, hipStream_t s) {
+    const bool covered = swiglu ? max_batch<F, true>(w, 1) != 0 : max_batch<F, false>(w, 1) != 0;
+    if (!covered) return launch_gemv_generic_sel(w, d_x, d_y, out_rows, swiglu, sel, s);
+    return swiglu ? launch_one<F, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<F, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+}
+
+int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel,
+                    hipStream_t s) {
+    if (sel.npairs == 0 || out_rows == 0) return FHIP_OK;
+    switch (w->type) {
+        case FHIP_Q4_K: return launch_sel_fmt<Q4K>(w, d_x, d_y, out_rows, swiglu, sel, s);
+        case FHIP_Q6_K: return launch_sel_fmt<Q6K>(w, d_x, d_y, out_rows, swiglu, sel, s);
+        case FHIP_Q8_0: return launch_sel_fmt<Q80>(w, d_x, d_y, out_rows, swiglu, sel, s);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

@@ -231,6 +231,7 @@ struct GemvParams {
     size_t pair_bytes;   // fused SwiGLU: byte distance from gate row r to up row r (= n_ff * row_bytes)
     int S, G, rpg;       // waves per row, row groups per workgroup, output rows per row group
     int stage;           // 1: x staged through LDS once per workgroup
+    fhip::SelParams sel; // expert selection (selw == nullptr: none)
 };
 
 // Threads per workgroup allowed for M activation rows: the 32*M resident activation registers per
@@ -242,6 +243,7 @@ constexpr int rows_in_flight(int M) { return M == 1 ? 4 : 2; }
 template <class F, int M, int U, bool SWIGLU>
 __global__ void __launch_bounds__(max_threads(M)) gemv_kernel(GemvParams p) {
     extern __shared__ float smem[];
+    fhip::apply_selection(p);
     constexpr int VPR = SWIGLU ? 2 : 1;  // weight rows walked per output row
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps row pointers and loop control scalar
@@ -349,12 +351,13 @@ int env_int(const char* name, int dflt) {
 }
 
 template <class F, int M, bool SWIGLU>
-int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s) {
+int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr) {
     static const int tune_g = env_int("FHIP_GEMV_G", 0), tune_rpg = env_int("FHIP_GEMV_RPG", 0), tune_u = env_int("FHIP_GEMV_U", 0);
     GemvParams p;
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
     p.pair_bytes = SWIGLU ? out_rows * w->row_bytes : 0;
+    p.sel = sel ? *sel : fhip::SelParams{nullptr, 0, 0, 0, 0, 0, 1};
     const int units = (int)(w->cols / 32);
     p.S = (units + 63) / 64;
     constexpr int MAXW = max_threads(M) / 64;
@@ -367,7 +370,8 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     p.G = G;
     // Rows per row group: enough workgroups to spread over every CU several times, but at least a
     // few rows per wave so the one-time activation load is amortised.
-    const int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    if (p.sel.npairs > 1) cus = cus / p.sel.npairs > 0 ? cus / p.sel.npairs : 1;   // the pairs of an "_id" launch share the chip
     int rpg = tune_rpg > 0 ? tune_rpg : (int)((out_rows + (size_t)cus * G - 1) / ((size_t)cus * G));
     if (tune_rpg <= 0) {
         if (rpg > 32) rpg = 32;
@@ -380,8 +384,9 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     if (lds > 64 * 1024) return fhip::set_error(FHIP_ERR_SHAPE, "matmul_q: LDS budget exceeded (%zu B)", lds);
     dim3 block(64 * p.S * G);
     constexpr int U = rows_in_flight(M);
-    if (tune_u == 2 && U != 2) hipLaunchKernelGGL((gemv_kernel<F, M, 2, SWIGLU>), dim3((unsigned)grid), block, lds, s, p);
-    else hipLaunchKernelGGL((gemv_kernel<F, M, U, SWIGLU>), dim3((unsigned)grid), block, lds, s, p);
+    const dim3 g3((unsigned)grid, (unsigned)p.sel.npairs);
+    if (tune_u == 2 && U != 2) hipLaunchKernelGGL((gemv_kernel<F, M, 2, SWIGLU>), g3, block, lds, s, p);
+    else hipLaunchKernelGGL((gemv_kernel<F, M, U, SWIGLU>), g3, block, lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
 }
 
@@ -415,6 +420,17 @@ int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, f
         case FHIP_Q8_0:
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for Q8_0");
             return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, s);
+        default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
+    }
+}
+
+int launch_gemv_generic_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu,
+                            const SelParams& sel, hipStream_t s) {
+    if (sel.npairs == 0 || out_rows == 0) return FHIP_OK;
+    switch (w->type) {
+        case FHIP_Q4_K: return swiglu ? launch_one<Q4K, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q4K, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_Q6_K: return swiglu ? launch_one<Q6K, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q6K, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_Q8_0: return swiglu ? launch_one<Q80, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q80, 1, false>(w, d_x, d_y, out_rows, s, &sel);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

@@ -206,6 +206,77 @@ class Tensor:
         out._keepalive = ws  # scratch must outlive the enqueued work
         return out
 
+    # -- mixture-of-experts decode (dtype.rs:1582-1780) -----------------------------------------
+    def moe_topk(self, bias, k, sigmoid, scale, stream=None):
+        """Router top-k on the device -- dtype.rs:1582. self = logits [T, n_expert]; returns [T, 2k] = [w | idx]."""
+        return self.moe_topk_ex(bias, k, sigmoid, scale, True, stream)
+
+    def moe_topk_ex(self, bias, k, sigmoid, scale, norm, stream=None):
+        """moe_topk with explicit control over renormalisation -- dtype.rs:1596."""
+        t, ne = (self.shape[0], self.shape[1]) if len(self.shape) == 2 else (1, self.numel())
+        assert 1 <= k <= 8, "k must be 1..=8"
+        assert ne <= 1024, "moe_topk: n_expert <= 1024 (single-thread scan)"
+        out = Tensor.empty((t, 2 * k))
+        _lib.check(_lib.load().fhip_moe_topk(self.buf.ptr, bias.buf.ptr if bias is not None else None, t, ne, k, int(bool(sigmoid)),
+                                             float(scale), int(bool(norm)), out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def _swiglu_id(self, w, selw, k, eff, stream):
+        t, inn = self._rows_inner()
+        assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
+        assert 1 <= k <= 8, "k must be 1..=8"
+        out = Tensor.empty((t, k, eff))
+        _lib.check(_lib.load().fhip_matmul_q_swiglu_id(w.handle, self.buf.ptr, t, selw.buf.ptr, k, eff, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def matmul_q4_k_swiglu_id(self, w, selw, k, eff, stream=None):
+        """Selected experts' gate|up + SwiGLU for every (token, slot): [T, in] -> [T, k, eff] -- dtype.rs:1620."""
+        assert w.ggml_type == Q4_K
+        return self._swiglu_id(w, selw, k, eff, stream)
+
+    def matmul_q8_0_swiglu_id(self, w, selw, k, eff, stream=None):
+        """dtype.rs:1731."""
+        assert w.ggml_type == Q8_0
+        return self._swiglu_id(w, selw, k, eff, stream)
+
+    def matmul_q6_k_id(self, w, selw, out_pe, stream=None):
+        """Selected experts' down projection, one row per slot: [k, in] -> [k, out_pe] -- dtype.rs:1640."""
+        k, inn = self._rows_inner()
+        assert 1 <= k <= 8, "k must be 1..=8"
+        assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
+        out = Tensor.empty((k, out_pe))
+        _lib.check(_lib.load().fhip_matmul_q_id(w.handle, self.buf.ptr, selw.buf.ptr, k, out_pe, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def _id_wsum(self, w, selw, out_pe, stream):
+        t, k, inn = self.shape if len(self.shape) == 3 else (1, self.shape[0], self.shape[1])
+        assert 1 <= k <= 8, "k must be 1..=8"
+        assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
+        out = Tensor.empty((t, out_pe))
+        ws = Tensor.empty((t * k, out_pe))
+        _lib.check(_lib.load().fhip_matmul_q_id_wsum(w.handle, self.buf.ptr, t, selw.buf.ptr, k, out_pe, out.buf.ptr, ws.buf.ptr,
+                                                     _stream_handle(stream)))
+        if stream is not None:
+            stream.synchronize()      # ws is freed on return
+        else:
+            _lib.check(_lib.load().fhip_stream_sync(None))
+        return out
+
+    def matmul_q6_k_id_wsum(self, w, selw, out_pe, stream=None):
+        """Down projection with the weighted sum over slots fused: [T, k, in] -> [T, out_pe] -- dtype.rs:1662."""
+        assert w.ggml_type == Q6_K
+        return self._id_wsum(w, selw, out_pe, stream)
+
+    def matmul_q4_k_id_wsum(self, w, selw, out_pe, stream=None):
+        """dtype.rs:1765."""
+        assert w.ggml_type == Q4_K
+        return self._id_wsum(w, selw, out_pe, stream)
+
+    def matmul_q8_0_id_wsum(self, w, selw, out_pe, stream=None):
+        """dtype.rs:1748."""
+        assert w.ggml_type == Q8_0
+        return self._id_wsum(w, selw, out_pe, stream)
+
     def cvt_bf16(self, stream=None):
         """f32 -> bf16 bit patterns (round to nearest even), same shape."""
         assert self.dtype == np.float32

@@ -163,6 +163,33 @@ int fhip_ffn(const fhip_weight* gate_up, const fhip_weight* down, const float* d
  * dequantized tile by tile into LDS as bf16 and contracted on the matrix cores, f32 accumulate. */
 int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x_bf16, size_t t, float* d_y, void* stream);
 
+/* ---- mixture-of-experts decode: the "_id" variants that sit behind the same matmul entry points ---------- */
+
+/* crates/ferric-tensor/src/dtype.rs:1582 Tensor::moe_topk / :1596 moe_topk_ex (kernel :2415-2461). logits
+ * [t, n_expert] f32, bias n_expert f32 or NULL; out [t, 2k] = [w_0..w_{k-1} | idx_0..idx_{k-1}], indices as f32.
+ * Scores: softmax over all experts, or sigmoid; selection by score + bias, ties to the lowest index; weights =
+ * selected scores (without bias), / their sum when norm, * scale. k not in 1..=8 or n_expert > 1024 ->
+ * FHIP_ERR_SHAPE (the reference's asserts, dtype.rs:1599-1600). */
+int fhip_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t n_expert, size_t k, int sigmoid, float scale, int norm,
+                  float* d_out, void* stream);
+
+/* dtype.rs:1620 matmul_q4_k_swiglu_id / :1731 matmul_q8_0_swiglu_id (kernels :2463, :2618): x [t, cols], w packs all
+ * experts' fused gate|up rows expert-major (rows = n_expert * 2 * eff: gate rows, then up rows, per expert), selw the
+ * [t, 2k] moe_topk output; y [t, k, eff] = silu(gate_e . x_t) * (up_e . x_t) for every (token, selected expert).
+ * Any of the three formats. An index outside the slab is clamped into it. */
+int fhip_matmul_q_swiglu_id(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t eff, float* d_y,
+                            void* stream);
+
+/* dtype.rs:1640 matmul_q6_k_id (kernel :2509): x [k, cols] (row s = slot s's SwiGLU output), w packs all experts' down
+ * rows expert-major (rows = n_expert * out_pe), selw one moe_topk row [2k]; y [k, out_pe]. Any of the three formats. */
+int fhip_matmul_q_id(const fhip_weight* w, const float* d_x, const float* d_selw, size_t k, size_t out_pe, float* d_y, void* stream);
+
+/* dtype.rs:1662 matmul_q6_k_id_wsum / :1765 matmul_q4_k_id_wsum / :1748 matmul_q8_0_id_wsum (kernels :2538, :2571,
+ * :2654): x [t, k, cols]; y [t, out_pe], row t = sum_s w_{t,s} * down_{e_{t,s}}(x_{t,s}), slots added in order.
+ * d_ws: caller-provided scratch of t * k * out_pe f32 (the per-slot projections before the weighted sum). */
+int fhip_matmul_q_id_wsum(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t out_pe, float* d_y,
+                          float* d_ws, void* stream);
+
 /* f32 -> bf16 bit patterns, round to nearest even, n values (both pointers 16-byte aligned). The reference's
  * matrix-unit kernels read f32 activations (crates/ferric-tensor/src/dtype.rs:1824-1830, `xp.buf`); the
  * matrix cores here take bf16, so this is the conversion in front of fhip_gemm_q_bf16. */

@@ -197,6 +197,109 @@ def swiglu(gu, n_ff):
     return out
 
 
+# ---------------------------------------------------------------- mixture-of-experts ops (numpy restatements)
+def moe_topk(logits, bias, k, sigmoid, scale, norm=True):
+    """MOE_TOPK_WGSL, crates/ferric-tensor/src/dtype.rs:2415-2461, statement by statement in f32: per token the
+    scores (softmax with a sequential f32 sum, or sigmoid), k rounds of a first-maximum scan over the not yet
+    picked experts on score + bias, weights = picked scores / (their sequential sum if norm) * scale.
+    Returns [T, 2k] f32 = [w | idx]."""
+    f = np.float32
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    logits = logits.reshape(1, -1) if logits.ndim == 1 else logits
+    t, ne = logits.shape
+    assert 1 <= k <= 8, "k must be 1..=8"
+    assert ne <= 1024, "moe_topk: n_expert <= 1024 (single-thread scan)"
+    out = np.zeros((t, 2 * k), dtype=np.float32)
+    for ti in range(t):
+        l = logits[ti]
+        maxl, ssum = f(-3.4e38), f(0.0)
+        if not sigmoid:
+            for i in range(ne):
+                maxl = max(maxl, l[i])
+            for i in range(ne):
+                ssum = f(ssum + np.exp(f(l[i] - maxl), dtype=np.float32))
+
+        def score(i):
+            if sigmoid:
+                return f(f(1.0) / f(f(1.0) + np.exp(f(-l[i]), dtype=np.float32)))
+            return f(np.exp(f(l[i] - maxl), dtype=np.float32) / ssum)
+
+        picked, wsum = set(), f(0.0)
+        with np.errstate(all="ignore"):
+            for s in range(k):
+                bi, bv = 0, f(-3.4e38)
+                for i in range(ne):
+                    if i in picked:
+                        continue
+                    m = score(i)
+                    if bias is not None:
+                        m = f(m + f(bias[i]))
+                    if m > bv:
+                        bv, bi = m, i
+                picked.add(bi)
+                sc = score(bi)
+                out[ti, s], out[ti, k + s] = sc, f(bi)
+                wsum = f(wsum + sc)
+            den = wsum if norm else f(1.0)
+            for s in range(k):
+                out[ti, s] = f(f(out[ti, s] / den) * f(scale))
+    return out
+
+
+def matmul_swiglu_id_f64(x, w, ty, selw, k, eff, cols):
+    """MATMUL_Q4_K_SWIGLU_ID_WGSL / MATMUL_Q8_0_SWIGLU_ID_WGSL (dtype.rs:2463-2507, :2618-2652) in f64 on the
+    dequantized expert slab: out[ti, s, o] = silu(g) * u with g, u the dots of token ti's row with rows
+    e*2eff + o and e*2eff + eff + o, e = selw[ti, k + s]. Also returns (|g| bound terms) the per-row weight norms."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, cols)
+    w, _ = _u8(w)
+    rows = w.size // (cols // BLOCK[ty][0] * BLOCK[ty][1])
+    wd = deq_raw(w, rows * cols, ty).reshape(rows, cols).astype(np.float64)
+    selw = np.asarray(selw, dtype=np.float32).reshape(x.shape[0], 2 * k)
+    out = np.zeros((x.shape[0], k, eff))
+    for ti in range(x.shape[0]):
+        for s in range(k):
+            base = int(selw[ti, k + s]) * 2 * eff
+            g = wd[base:base + eff] @ x[ti].astype(np.float64)
+            u = wd[base + eff:base + 2 * eff] @ x[ti].astype(np.float64)
+            out[ti, s] = g / (1.0 + np.exp(-g)) * u
+    return out
+
+
+def matmul_id_f64(x, w, ty, selw, k, out_pe, cols):
+    """MATMUL_Q6_K_ID_WGSL (dtype.rs:2509-2536) in f64: out[s, o] = x[s] . W[e_s*out_pe + o], plus the weight norms."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(k, cols)
+    w, _ = _u8(w)
+    rows = w.size // (cols // BLOCK[ty][0] * BLOCK[ty][1])
+    wd = deq_raw(w, rows * cols, ty).reshape(rows, cols).astype(np.float64)
+    selw = np.asarray(selw, dtype=np.float32).reshape(-1)
+    out = np.zeros((k, out_pe))
+    wn = np.zeros((k, out_pe))
+    for s in range(k):
+        blk = wd[int(selw[k + s]) * out_pe:][:out_pe]
+        out[s] = blk @ x[s].astype(np.float64)
+        wn[s] = np.linalg.norm(blk, axis=1)
+    return out, wn
+
+
+def matmul_id_wsum_f64(x, w, ty, selw, k, out_pe, cols):
+    """MATMUL_{Q6_K,Q4_K,Q8_0}_ID_WSUM_WGSL (dtype.rs:2538-2700) in f64: out[ti, o] = sum_s w[ti, s] * x[ti, s] .
+    W[e*out_pe + o]; also returns sum_s |w| * ||W row|| * ||x[ti, s]||, the scale of the tolerance bound."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k, cols)
+    w, _ = _u8(w)
+    rows = w.size // (cols // BLOCK[ty][0] * BLOCK[ty][1])
+    wd = deq_raw(w, rows * cols, ty).reshape(rows, cols).astype(np.float64)
+    selw = np.asarray(selw, dtype=np.float32).reshape(x.shape[0], 2 * k)
+    out = np.zeros((x.shape[0], out_pe))
+    bound = np.zeros((x.shape[0], out_pe))
+    for ti in range(x.shape[0]):
+        for s in range(k):
+            blk = wd[int(selw[ti, k + s]) * out_pe:][:out_pe]
+            xv = x[ti, s].astype(np.float64)
+            out[ti] += float(selw[ti, s]) * (blk @ xv)
+            bound[ti] += abs(float(selw[ti, s])) * np.linalg.norm(blk, axis=1) * np.linalg.norm(xv)
+    return out, bound
+
+
 # ---------------------------------------------------------------- reference test-data generators
 
 def gen_q4k_block(seed):
