@@ -131,6 +131,38 @@ def bench_ffn(F, lib, check, stream, timer, batches, reps=20):
     return res, wbytes
 
 
+def bench_moe(F, lib, check, stream, timer, reps=64):
+    """The routed-expert block of a mixture-of-experts decode layer (the callers of the "_id" entry points,
+    crates/ferric-llama/src/qwen35.rs:862-871) at Qwen3-30B-A3B's shape: hidden 2048, 128 experts, 8 used, expert FFN
+    768; gate|up slab Q4_K [128*1536, 2048] (226 MB), down slab Q6_K [128*2048, 768] (165 MB). One step = router
+    top-k on given logits, selected gate|up + SwiGLU, selected down + weighted sum. Each of the `reps` steps in the
+    graph uses its own random logits, so different experts are read from step to step (391 MB of slabs)."""
+    from ferric_amd.synth import synth_weights
+    d, ne, k, eff = 2048, 128, 8, 768
+    def slab(ty, rows_pe, cols, seed):   # 8 distinct experts' bytes tiled 16 times: the values do not matter for timing
+        one = synth_weights(ty, 8 * rows_pe, cols, seed)
+        return F.QMatrix.from_bytes(np.tile(one, ne // 8), ty, ne * rows_pe, cols)
+    gu, dn = slab(Q4_K, 2 * eff, d, 60), slab(Q6_K, d, eff, 61)
+    res = {}
+    for t in (1, 4):
+        rng = np.random.default_rng(62 + t)
+        x = F.Tensor.from_vec(rng.standard_normal((t, d)).astype(np.float32), (t, d))
+        logits = [F.Tensor.from_vec(rng.standard_normal((t, ne)).astype(np.float32) * 2, (t, ne)) for _ in range(reps)]
+        selw, mid = F.Tensor.empty((t, 2 * k)), F.Tensor.empty((t, k, eff))
+        y, ws = F.Tensor.empty((t, d)), F.Tensor.empty((t * k, d))
+        g = F.Graph.begin(stream)
+        for i in range(reps):
+            check(lib.fhip_moe_topk(logits[i].buf.ptr, None, t, ne, k, 0, 1.0, 1, selw.buf.ptr, stream.handle))
+            check(lib.fhip_matmul_q_swiglu_id(gu.handle, x.buf.ptr, t, selw.buf.ptr, k, eff, mid.buf.ptr, stream.handle))
+            check(lib.fhip_matmul_q_id_wsum(dn.handle, mid.buf.ptr, t, selw.buf.ptr, k, d, y.buf.ptr, ws.buf.ptr, stream.handle))
+        g.end()
+        g.launch()
+        ms = min(timer.time_ms(g.launch) for _ in range(3)) / reps
+        wbytes = t * k * (weight_bytes(Q4_K, 2 * eff, d) + weight_bytes(Q6_K, d, eff))
+        res[str(t)] = {"ms": ms, "expert_weight_bytes_read": wbytes, "weight_GBps": wbytes / (ms * 1e-3) / 1e9, "launches": 4}
+    return res
+
+
 def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
     """configs[4]: per layer fused QKV 5120->7168, O 5120->5120, fused gate+up 5120->34816 (+SwiGLU), all Q4_K,
     down 17408->5120 Q6_K; lm_head 5120->151936 Q6_K. One stream, one graph of layers*4+1 launches."""
@@ -268,6 +300,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-q8", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-moe", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the cold-rotation Q4_K 5120x5120 GEMV loop (what `value` is computed from); for profiling")
     ap.add_argument("--probe", action="store_true",
@@ -298,7 +331,7 @@ def main():
     c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
                                  cold_only=args.headline_only)
     if args.headline_only:
-        args.no_q8 = args.no_ffn = args.no_prefill = args.no_sweep = args.no_cpu = True
+        args.no_q8 = args.no_ffn = args.no_prefill = args.no_moe = args.no_sweep = args.no_cpu = True
         c2["warm"] = None
     ms_step = c2["cold"]["ms_per_step"]
     value = c2["cold"]["GBps"]
@@ -329,6 +362,9 @@ def main():
     if not args.no_prefill:
         log("[bench] prefill dequant-GEMM, T = 128/512/2048 ...")
         line["prefill_q4k_bf16_mfma"] = bench_prefill(F, lib, check, stream, timer)
+    if not args.no_moe:
+        log("[bench] routed-expert block of an MoE decode layer ...")
+        line["moe_routed_experts_q4k_q6k"] = bench_moe(F, lib, check, stream, timer)
     if not args.no_sweep:
         log("[bench] 64-layer decode weight sweep (14.0 GB) ...")
         line["decode_sweep"] = bench_sweep(F, lib, check, stream, timer)

@@ -11,29 +11,41 @@
 
 namespace {
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// All-lanes maximum / sum without LDS traffic: four DPP steps make every lane of a 16-lane row hold its row's
+// result, the four rows are then combined through scalar reads of one lane each.
+__device__ __forceinline__ float lane_f(float v, int ln) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), ln));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, dpp_f<0xB1>(v));    // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_f<0x4E>(v));    // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_f<0x141>(v));   // row_half_mirror
+    v = fmaxf(v, dpp_f<0x140>(v));   // row_mirror
+    return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x141>(v);
+    v += dpp_f<0x140>(v);
+    return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
 }
 
-constexpr int PER_LANE = 16;   // n_expert <= 64 * 16
-
+// PL = experts per lane (n_expert <= 64 * PL); expert i lives in lane i % 64, register i / 64
+template <int PL>
 __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int t, int ne,
                                                        int k, int sigmoid, float scale, int norm, float* __restrict__ out) {
     const int ti = blockIdx.x, lane = threadIdx.x;
     if (ti >= t) return;
     const float* l = logits + (size_t)ti * ne;
-    // expert i lives in lane i % 64, register i / 64
-    float sc[PER_LANE], key[PER_LANE];
+    float sc[PL], key[PL];
     float maxl = -3.4e38f;
 #pragma unroll
-    for (int j = 0; j < PER_LANE; j++) {
+    for (int j = 0; j < PL; j++) {
         const int i = j * 64 + lane;
         sc[j] = i < ne ? l[i] : 0.f;
         if (i < ne && !sigmoid) maxl = fmaxf(maxl, sc[j]);
@@ -42,7 +54,7 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
     if (!sigmoid) {
         maxl = wave_max(maxl);
 #pragma unroll
-        for (int j = 0; j < PER_LANE; j++) {
+        for (int j = 0; j < PL; j++) {
             const int i = j * 64 + lane;
             sc[j] = i < ne ? expf(sc[j] - maxl) : 0.f;
             ssum += sc[j];
@@ -50,7 +62,7 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
         ssum = wave_sum(ssum);
     }
 #pragma unroll
-    for (int j = 0; j < PER_LANE; j++) {
+    for (int j = 0; j < PL; j++) {
         const int i = j * 64 + lane;
         if (i < ne) {
             sc[j] = sigmoid ? 1.0f / (1.0f + expf(-sc[j])) : sc[j] / ssum;
@@ -62,32 +74,36 @@ __global__ void __launch_bounds__(64) moe_topk_kernel(const float* __restrict__ 
     float wsum = 0.f, myw = 0.f, myi = 0.f;   // lane s keeps slot s
     for (int s = 0; s < k; s++) {
         // best of this lane: larger key first, then lower index; a key must exceed -3.4e38 to count at all
-        float bv = -3.4e38f;
+        float bv = -3.4e38f, bs = 0.f;
         int bi = 0x7fffffff;
-        float bs = 0.f;
 #pragma unroll
-        for (int j = 0; j < PER_LANE; j++) {
+        for (int j = 0; j < PL; j++) {
             if (key[j] > bv) { bv = key[j]; bi = j * 64 + lane; bs = sc[j]; }
         }
+        // the wave's best value, then among the lanes that hold it the lowest expert index (usually one lane)
+        const float vmax = wave_max(bv);
+        unsigned long long m = __ballot(bv == vmax && bi != 0x7fffffff);
+        int win = 0, owner = 0;
+        float ws = 0.f;
+        if (m == 0) {   // nothing selectable (all NaN, or already taken): the reference's scan leaves index 0
+            ws = lane_f(sc[0], 0);
+        } else {
+            win = 0x7fffffff;
+            while (m) {
+                const int ln = __builtin_ctzll(m);
+                const int i = __builtin_amdgcn_readlane(bi, ln);
+                if (i < win) { win = i; owner = ln; }
+                m &= m - 1;
+            }
+            ws = lane_f(bs, owner);
+            if (lane == owner) {   // retire the winner
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-            const float ov = __shfl_xor(bv, o, 64);
-            const int oi = __shfl_xor(bi, o, 64);
-            const float os = __shfl_xor(bs, o, 64);
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; bs = os; }
+                for (int j = 0; j < PL; j++)
+                    if (j == (win >> 6)) key[j] = -__builtin_inff();
+            }
         }
-        if (bi == 0x7fffffff) {   // nothing selectable (all NaN or already taken): the reference's scan leaves index 0
-            bi = 0;
-            bs = __shfl(sc[0], 0, 64);
-        }
-        // retire the winner
-        if ((bi & 63) == lane) {
-#pragma unroll
-            for (int j = 0; j < PER_LANE; j++)
-                if (j == (bi >> 6)) key[j] = -__builtin_inff();
-        }
-        wsum += bs;
-        if (lane == s) { myw = bs; myi = (float)bi; }
+        wsum += ws;
+        if (lane == s) { myw = ws; myi = (float)win; }
     }
     const float den = norm ? wsum : 1.0f;
     if (lane < k) {
@@ -114,7 +130,14 @@ namespace fhip {
 int launch_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t ne, int k, int sigmoid, float scale, int norm,
                     float* d_out, hipStream_t s) {
     if (t == 0) return FHIP_OK;
-    hipLaunchKernelGGL(moe_topk_kernel, dim3((unsigned)t), dim3(64), 0, s, d_logits, d_bias, (int)t, (int)ne, k, sigmoid, scale, norm, d_out);
+    auto go = [&](auto kern) {
+        hipLaunchKernelGGL(kern, dim3((unsigned)t), dim3(64), 0, s, d_logits, d_bias, (int)t, (int)ne, k, sigmoid, scale, norm, d_out);
+    };
+    if (ne <= 64) go(moe_topk_kernel<1>);
+    else if (ne <= 128) go(moe_topk_kernel<2>);
+    else if (ne <= 256) go(moe_topk_kernel<4>);
+    else if (ne <= 512) go(moe_topk_kernel<8>);
+    else go(moe_topk_kernel<16>);
     return check_hip(hipGetLastError(), "moe_topk launch");
 }
 
