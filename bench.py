@@ -163,6 +163,41 @@ def bench_moe(F, lib, check, stream, timer, reps=64):
     return res
 
 
+def bench_gguf(F, lib, check, n_tensors=8, rows=11008, cols=5120):
+    """GGUF ingest: a synthetic file of n_tensors Q4_K [rows, cols] tensors (31.7 MB each) written to a temporary
+    file, then opened (mmap + header parse + stride check) and every tensor uploaded straight from the mapping.
+    Host-side I/O and PCIe: reported for the record, never part of `value`."""
+    import struct
+    import tempfile
+    from ferric_amd.synth import synth_weights
+    one = synth_weights(Q4_K, rows, cols, 70).tobytes()
+    head = bytearray(b"GGUF" + struct.pack("<IQQ", 3, n_tensors, 0))
+    for i in range(n_tensors):
+        name = f"blk.{i}.ffn_down.weight".encode()
+        head += struct.pack("<Q", len(name)) + name + struct.pack("<IQQIQ", 2, cols, rows, Q4_K, i * len(one))
+    head.extend(b"\0" * (-len(head) % 32))
+    with tempfile.NamedTemporaryFile(suffix=".gguf") as f:
+        f.write(head)
+        for _ in range(n_tensors):
+            f.write(one)
+        f.flush()
+        t0 = time.perf_counter()
+        g = F.GgufFile.open(f.name)
+        t_open = time.perf_counter() - t0
+        best = None
+        for _ in range(3):
+            t0 = time.perf_counter()
+            ws = [g.qmatrix(t.name) for t in g.tensors]
+            check(lib.fhip_stream_sync(None))
+            dt = time.perf_counter() - t0
+            best = dt if best is None or dt < best else best
+            del ws
+        g.close()
+    total = n_tensors * len(one)
+    return {"file_bytes": total + len(head), "open_parse_ms": t_open * 1e3, "upload_ms": best * 1e3, "upload_GBps": total / best / 1e9,
+            "note": "page-cache-resident file, pageable mapping -> hipMemcpy; host I/O and PCIe bound"}
+
+
 def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
     """configs[4]: per layer fused QKV 5120->7168, O 5120->5120, fused gate+up 5120->34816 (+SwiGLU), all Q4_K,
     down 17408->5120 Q6_K; lm_head 5120->151936 Q6_K. One stream, one graph of layers*4+1 launches."""
@@ -365,6 +400,9 @@ def main():
     if not args.no_moe:
         log("[bench] routed-expert block of an MoE decode layer ...")
         line["moe_routed_experts_q4k_q6k"] = bench_moe(F, lib, check, stream, timer)
+    if not args.no_moe:
+        log("[bench] GGUF ingest ...")
+        line["gguf_ingest"] = bench_gguf(F, lib, check)
     if not args.no_sweep:
         log("[bench] 64-layer decode weight sweep (14.0 GB) ...")
         line["decode_sweep"] = bench_sweep(F, lib, check, stream, timer)

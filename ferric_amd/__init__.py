@@ -5,6 +5,8 @@ mirror of the reference's quantized-linear interface on top of it.
 """
 from .qmatrix import (Q4_K, Q6_K, Q8_0, DeviceBuffer, Graph, Q4_KWeights, Q6_KWeights, Q8_0Weights, QMatrix, Stream, Tensor,
                       deq_raw, f16_to_f32, matvec_q8_0, matvec_q8_0_span, matvec_q8_0_threaded, type_size)
+from .gguf import Gguf, GgufFile, TensorInfo
 
 __all__ = ["Q4_K", "Q6_K", "Q8_0", "DeviceBuffer", "Graph", "Q4_KWeights", "Q6_KWeights", "Q8_0Weights", "QMatrix", "Stream",
-           "Tensor", "deq_raw", "f16_to_f32", "matvec_q8_0", "matvec_q8_0_span", "matvec_q8_0_threaded", "type_size"]
+           "Tensor", "deq_raw", "f16_to_f32", "matvec_q8_0", "matvec_q8_0_span", "matvec_q8_0_threaded", "type_size",
+           "Gguf", "GgufFile", "TensorInfo"]

@@ -9,7 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SO_PATH = os.path.join(_HERE, "libferric_hip.so")
 
-OK, ERR_UNSUPPORTED_TYPE, ERR_SHAPE, ERR_HIP, ERR_ARG = 0, -1, -2, -3, -4
+OK, ERR_UNSUPPORTED_TYPE, ERR_SHAPE, ERR_HIP, ERR_ARG, ERR_FORMAT = 0, -1, -2, -3, -4, -5
 
 _vp = C.c_void_p
 _sz = C.c_size_t
@@ -59,6 +59,23 @@ SYMBOLS = {
     "fhip_matmul_q_swiglu_id": (C.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _vp, _vp]),
     "fhip_matmul_q_id": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _vp, _vp]),
     "fhip_matmul_q_id_wsum": (C.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _vp, _vp, _vp]),
+    "fhip_gguf_parse": (C.c_int, [_vp, _sz, _vp]),
+    "fhip_gguf_open": (C.c_int, [C.c_char_p, _vp]),
+    "fhip_gguf_close": (None, [_vp]),
+    "fhip_gguf_version": (C.c_uint32, [_vp]),
+    "fhip_gguf_data_start": (C.c_uint64, [_vp]),
+    "fhip_gguf_n_tensors": (_sz, [_vp]),
+    "fhip_gguf_tensor": (C.c_int, [_vp, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "fhip_gguf_find": (C.c_long, [_vp, C.c_char_p]),
+    "fhip_gguf_raw": (C.c_int, [_vp, C.c_char_p, _vp, _vp]),
+    "fhip_gguf_n_meta": (_sz, [_vp]),
+    "fhip_gguf_meta_key": (C.c_char_p, [_vp, _sz]),
+    "fhip_gguf_meta_kind": (C.c_int, [_vp, C.c_char_p, _vp]),
+    "fhip_gguf_meta_u64": (C.c_int, [_vp, C.c_char_p, _sz, _vp]),
+    "fhip_gguf_meta_i64": (C.c_int, [_vp, C.c_char_p, _sz, _vp]),
+    "fhip_gguf_meta_f64": (C.c_int, [_vp, C.c_char_p, _sz, _vp]),
+    "fhip_gguf_meta_str": (C.c_int, [_vp, C.c_char_p, _sz, _vp, _vp]),
+    "fhip_weight_from_gguf": (C.c_int, [_vp, C.c_char_p, _vp]),
     "fhip_cvt_f32_bf16": (C.c_int, [_vp, _sz, _vp, _vp]),
     "fhip_matmul_q_coop": (C.c_int, [_vp, _vp, _sz, _vp, _vp, _vp]),
     "fhip_ffn_coop_ws_bytes": (_sz, [_vp, _vp, _sz]),
@@ -101,7 +118,7 @@ def check(rc):
     if rc == OK:
         return
     msg = last_error()
-    if rc == ERR_UNSUPPORTED_TYPE:
+    if rc in (ERR_UNSUPPORTED_TYPE, ERR_FORMAT):
         raise ValueError(msg)
     if rc == ERR_SHAPE:
         raise AssertionError(msg)

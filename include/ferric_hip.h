@@ -40,6 +40,7 @@ extern "C" {
 #define FHIP_ERR_SHAPE (-2)            /* reference: assert!/assert_eq! panic on cols % block, byte length, inner dim */
 #define FHIP_ERR_HIP (-3)              /* a HIP runtime call failed */
 #define FHIP_ERR_ARG (-4)              /* NULL pointer or otherwise unusable argument */
+#define FHIP_ERR_FORMAT (-5)           /* reference: Err(String) from the GGUF reader (not GGUF, truncated, stride refusal, no such tensor) */
 
 typedef struct fhip_weight fhip_weight; /* opaque: one packed weight resident in HBM */
 
@@ -209,6 +210,47 @@ int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, fl
 size_t fhip_ffn_coop_ws_bytes(const fhip_weight* gate_up, const fhip_weight* down, size_t rows_x);
 int fhip_ffn_coop(const fhip_weight* gate_up, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y,
                   void* d_ws, void* stream);
+
+/* ---- GGUF ingest: file -> HBM without a host copy or repack (host code; no device needed to parse) ------- */
+
+typedef struct fhip_gguf fhip_gguf;
+
+/* crates/ferric-gguf/src/lib.rs:105 parse(bytes): header, metadata, tensor table, then check_declared_strides
+ * (:387) against the data section. `bytes` must outlive the handle. Errors (FHIP_ERR_FORMAT, text as the
+ * reference's): "not a GGUF file", "GGUF header truncated or malformed", the two stride refusals.
+ * fhip_gguf_open maps the file read-only and parses the mapping (the native GgufFile, :520-573, without its
+ * read-per-tensor: the mapping IS the raw view). */
+int fhip_gguf_parse(const uint8_t* bytes, size_t n, fhip_gguf** out);
+int fhip_gguf_open(const char* path, fhip_gguf** out);
+void fhip_gguf_close(fhip_gguf* g);
+uint32_t fhip_gguf_version(const fhip_gguf* g);
+uint64_t fhip_gguf_data_start(const fhip_gguf* g);
+
+/* TensorInfo (lib.rs:41-47), in file order; pointers stay valid until close. fhip_gguf_find: index or -1
+ * (Gguf::tensor, lib.rs:441). */
+size_t fhip_gguf_n_tensors(const fhip_gguf* g);
+int fhip_gguf_tensor(const fhip_gguf* g, size_t i, const char** name, uint32_t* n_dims, const uint64_t** dims, uint32_t* ggml_type,
+                     uint64_t* offset);
+long fhip_gguf_find(const fhip_gguf* g, const char* name);
+
+/* Gguf::raw / GgufFile::raw (lib.rs:443-449, :566-573): the tensor's packed bytes exactly as stored, as a view into
+ * the parsed buffer / mapping (no copy). Unknown name -> FHIP_ERR_FORMAT "no tensor 'name'". */
+int fhip_gguf_raw(const fhip_gguf* g, const char* name, const uint8_t** bytes, size_t* nbytes);
+
+/* Metadata (lib.rs:38 enum Meta): kind 0 U, 1 I, 2 F, 3 Bool, 4 Str, 5 Arr, or -1 when absent; arr_len is set for
+ * arrays. The typed getters read the value itself (j = (size_t)-1) or element j of an array. */
+size_t fhip_gguf_n_meta(const fhip_gguf* g);
+const char* fhip_gguf_meta_key(const fhip_gguf* g, size_t i);
+int fhip_gguf_meta_kind(const fhip_gguf* g, const char* key, size_t* arr_len);
+int fhip_gguf_meta_u64(const fhip_gguf* g, const char* key, size_t j, uint64_t* out);
+int fhip_gguf_meta_i64(const fhip_gguf* g, const char* key, size_t j, int64_t* out);
+int fhip_gguf_meta_f64(const fhip_gguf* g, const char* key, size_t j, double* out);
+int fhip_gguf_meta_str(const fhip_gguf* g, const char* key, size_t j, const char** s, size_t* len);
+
+/* QShard::build from a GGUF tensor (crates/ferric-tensor/src/dtype.rs:839-857 over GgufSource::raw): uploads the
+ * tensor's bytes straight from the mapping. dims are [in, out] or, for an expert slab, [in, rows per expert,
+ * n_expert] (rows = product of the trailing dims). Types 8 / 12 / 14 only. */
+int fhip_weight_from_gguf(const fhip_gguf* g, const char* name, fhip_weight** out);
 
 /* crates/ferric-tensor/src/cpu_simd.rs:79 matvec_q8_0(x, w, rows, cols) with HOST buffers on both
  * sides (upload, GEMV, download, synchronise) -- the drop-in for the CPU mat-vec call.
