@@ -3,10 +3,10 @@
 The product is libferric_hip.so (C ABI in include/ferric_hip.h); this package is the host-side
 mirror of the reference's quantized-linear interface on top of it.
 """
-from .qmatrix import (Q4_K, Q6_K, Q8_0, DeviceBuffer, Graph, Q4_KWeights, Q6_KWeights, Q8_0Weights, QMatrix, Stream, Tensor,
+from .qmatrix import (Q4_0, Q4_1, Q4_K, Q5_0, Q5_1, Q5_K, Q6_K, Q8_0, DeviceBuffer, Graph, Q4_KWeights, Q6_KWeights, Q8_0Weights, QMatrix, Stream, Tensor,
                       deq_raw, f16_to_f32, matvec_q8_0, matvec_q8_0_span, matvec_q8_0_threaded, type_size)
 from .gguf import Gguf, GgufFile, TensorInfo
 
-__all__ = ["Q4_K", "Q6_K", "Q8_0", "DeviceBuffer", "Graph", "Q4_KWeights", "Q6_KWeights", "Q8_0Weights", "QMatrix", "Stream",
+__all__ = ["Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q5_K", "Q4_K", "Q6_K", "Q8_0", "DeviceBuffer", "Graph", "Q4_KWeights", "Q6_KWeights", "Q8_0Weights", "QMatrix", "Stream",
            "Tensor", "deq_raw", "f16_to_f32", "matvec_q8_0", "matvec_q8_0_span", "matvec_q8_0_threaded", "type_size",
            "Gguf", "GgufFile", "TensorInfo"]

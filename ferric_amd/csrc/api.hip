@@ -18,11 +18,28 @@ bool block_info(uint32_t ty, size_t& vals, size_t& bytes) {
         case FHIP_Q8_0: vals = 32; bytes = 34; return true;
         case FHIP_Q4_K: vals = 256; bytes = 144; return true;
         case FHIP_Q6_K: vals = 256; bytes = 210; return true;
+        case FHIP_Q4_0: vals = 32; bytes = 18; return true;
+        case FHIP_Q4_1: vals = 32; bytes = 20; return true;
+        case FHIP_Q5_0: vals = 32; bytes = 22; return true;
+        case FHIP_Q5_1: vals = 32; bytes = 24; return true;
+        case FHIP_Q5_K: vals = 256; bytes = 176; return true;
         default: return false;
     }
 }
 
-const char* type_name(uint32_t ty) { return ty == FHIP_Q8_0 ? "Q8_0" : ty == FHIP_Q4_K ? "Q4_K" : ty == FHIP_Q6_K ? "Q6_K" : "?"; }
+const char* type_name(uint32_t ty) {
+    switch (ty) {
+        case FHIP_Q8_0: return "Q8_0";
+        case FHIP_Q4_K: return "Q4_K";
+        case FHIP_Q6_K: return "Q6_K";
+        case FHIP_Q4_0: return "Q4_0";
+        case FHIP_Q4_1: return "Q4_1";
+        case FHIP_Q5_0: return "Q5_0";
+        case FHIP_Q5_1: return "Q5_1";
+        case FHIP_Q5_K: return "Q5_K";
+        default: return "?";
+    }
+}
 
 int need_init() {
     if (g_device < 0) return fhip::set_error(FHIP_ERR_ARG, "fhip_init has not been called");
@@ -264,8 +281,8 @@ int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ty, flo
     size_t nb = n / vals;
     if (nbytes / bytes < nb) nb = nbytes / bytes;  // chunks_exact(..).take(n / blk)
     if (nb && !h_raw) return set_error(FHIP_ERR_ARG, "fhip_deq_raw: NULL bytes");
-    // The K-quant dequantizers pre-size the output to n zeros (lib.rs:794, :722); Q8_0 pushes whole
-    // blocks only and so returns a shorter vector (lib.rs:609-614).
+    // Every dequantizer but Q8_0's pre-sizes the output to n zeros (lib.rs:619, :634, :651, :670, :693, :722, :794); Q8_0
+    // pushes whole blocks only and so returns a shorter vector (lib.rs:609-614).
     size_t produced = ty == FHIP_Q8_0 ? nb * vals : n;
     if (n_written) *n_written = produced;
     if (nb) {

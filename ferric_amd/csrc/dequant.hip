@@ -1,4 +1,4 @@
-// Bit-exact block unpackers for Q8_0 / Q4_K / Q6_K on gfx950.
+// Bit-exact block unpackers for Q8_0 / Q4_K / Q6_K (and Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q5_K) on gfx950.
 //
 // The reference CPU dequantizers round every f32 operation separately (Rust never fuses a*b+c):
 //   Q8_0  y = f32(q) * d                       crates/ferric-gguf/src/lib.rs:608-615
@@ -106,6 +106,61 @@ __global__ void deq_q6_k_kernel(const uint8_t* __restrict__ raw, size_t nquads, 
     *(float4*)(out + t * 4) = o;
 }
 
+// ---- the 32-value formats: [f16 d][f16 m]?[u32 qh]?[u8 qs[16]], blocks 2-byte aligned ----------------------
+// value i < 16 is the low nibble of qs[i], value 16 + i the high one; the fifth bit of value v is bit v of qh.
+//   Q4_0 y = f32(n - 8) * d            lib.rs:618-629      Q4_1 y = f32(n) * d + m            lib.rs:633-645
+//   Q5_0 y = f32((n | b<<4) - 16) * d  lib.rs:650-665      Q5_1 y = f32(n | b<<4) * d + m     lib.rs:669-684
+template <int BYTES, bool HAS_M, bool HAS_QH, int OFF>
+__global__ void deq_legacy_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane = 4 values, 8 lanes = one block
+    if (t >= nquads) return;
+    size_t blk = t >> 3;
+    int v = (int)(t & 7) * 4;
+    const uint8_t* b = raw + blk * BYTES;
+    constexpr int QH = HAS_M ? 4 : 2, QS = QH + (HAS_QH ? 4 : 0);
+    float d = f16_bits(*(const uint16_t*)b);
+    float m = HAS_M ? f16_bits(*(const uint16_t*)(b + 2)) : 0.f;
+    uint32_t q = ld4_a2(b + QS + (v & 15));
+    if (v >= 16) q >>= 4;
+    q &= 0x0F0F0F0Fu;
+    if (HAS_QH) {
+        uint32_t hb = (ld4_a2(b + QH) >> v) & 0xFu;
+        q |= ((hb * 0x00204081u) & 0x01010101u) << 4;   // bit j of hb -> bit 4 of byte j
+    }
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float f = (float)((int)((q >> (8 * k)) & 0xFF) - OFF);
+        o[k] = HAS_M ? __fadd_rn(__fmul_rn(f, d), m) : __fmul_rn(f, d);
+    }
+    *(float4*)(out + t * 4) = make_float4(o[0], o[1], o[2], o[3]);
+}
+
+// ---- Q5_K: 176 B = [f16 d][f16 dmin][u8 s[12]][u8 qh[32]][u8 qs[128]]; y = (d*sc)*(n + 16*bit) - dmin*m, lib.rs:692-716
+__global__ void deq_q5_k_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= nquads) return;
+    size_t blk = t >> 6;
+    int v = (int)(t & 63) * 4;
+    int sb = v >> 5, l = v & 31;
+    const uint8_t* b = raw + blk * 176;  // 16-byte aligned
+    uint32_t hd = *(const uint32_t*)b;
+    float d = f16_bits(hd & 0xFFFFu), dmin = f16_bits(hd >> 16);
+    uint32_t sc, m;
+    q4k_sc_min(b + 4, sb, sc, m);
+    uint32_t q = *(const uint32_t*)(b + 48 + 32 * (sb >> 1) + l);
+    if (sb & 1) q >>= 4;
+    q &= 0x0F0F0F0Fu;
+    q |= ((*(const uint32_t*)(b + 16 + l) >> sb) & 0x01010101u) << 4;   // bit sb of qh[l + k]
+    float d1 = __fmul_rn(d, (float)sc), mm = __fmul_rn(dmin, (float)m);
+    float4 o;
+    o.x = __fsub_rn(__fmul_rn(d1, (float)(q & 0xFF)), mm);
+    o.y = __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xFF)), mm);
+    o.z = __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xFF)), mm);
+    o.w = __fsub_rn(__fmul_rn(d1, (float)(q >> 24)), mm);
+    *(float4*)(out + t * 4) = o;
+}
+
 }  // namespace
 
 namespace fhip {
@@ -119,7 +174,7 @@ int launch_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_
 
 int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d_out, hipStream_t s) {
     if (nblocks == 0) return FHIP_OK;
-    size_t vals = type == FHIP_Q8_0 ? 32 : 256;
+    size_t vals = (type == FHIP_Q4_K || type == FHIP_Q5_K || type == FHIP_Q6_K) ? 256 : 32;
     size_t nquads = nblocks * vals / 4;
     size_t grid = (nquads + 255) / 256;
     if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_ARG, "dequant: %zu blocks exceed one launch", nblocks);
@@ -127,6 +182,11 @@ int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d
         case FHIP_Q8_0: hipLaunchKernelGGL(deq_q8_0_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
         case FHIP_Q4_K: hipLaunchKernelGGL(deq_q4_k_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
         case FHIP_Q6_K: hipLaunchKernelGGL(deq_q6_k_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_Q5_K: hipLaunchKernelGGL(deq_q5_k_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_Q4_0: hipLaunchKernelGGL((deq_legacy_kernel<18, false, false, 8>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_Q4_1: hipLaunchKernelGGL((deq_legacy_kernel<20, true, false, 0>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_Q5_0: hipLaunchKernelGGL((deq_legacy_kernel<22, false, true, 16>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_Q5_1: hipLaunchKernelGGL((deq_legacy_kernel<24, true, true, 0>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", type);
     }
     return check_hip(hipGetLastError(), "dequant launch");

@@ -1,5 +1,6 @@
 // General-shape mat-vec (and small-batch mat-mat) on the raw GGUF block stream, gfx950: covers every
-// cols the formats allow (any multiple of 256, or of 32 for Q8_0), with plain f32 multiply-adds.
+// cols the formats allow (any multiple of 256, or of 32 for the 32-value formats), with plain f32 multiply-adds,
+// and every block format of the path (Q8_0, Q4_K, Q6_K, and Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q5_K).
 // The streaming kernel in gemv.hip takes over for row lengths it tiles exactly; this one is the
 // shape-complete path behind it.
 //
@@ -221,6 +222,119 @@ struct Q80 {
     }
 };
 
+// The four 32-value formats: [f16 d][f16 m]?[u32 qh]?[u8 qs[16]], one unit = one block; value i < 16 is the low nibble
+// of qs[i], value 16 + i the high one, the fifth bit of value v is bit v of qh (crates/ferric-gguf/src/lib.rs:618-684).
+//   Q4_0 (n - 8) d      Q4_1 n d + m      Q5_0 ((n | b<<4) - 16) d      Q5_1 (n | b<<4) d + m
+template <int BYTES, bool HAS_M, bool HAS_QH, int OFF>
+struct Legacy {
+    static constexpr int QH = HAS_M ? 4 : 2, QS = QH + (HAS_QH ? 4 : 0);
+    struct Lane { uint32_t off; };
+    struct Data { u32x4 q; uint32_t dm, qh; __device__ __forceinline__ void pin_all() { pin(q); pin(dm); pin(qh); } };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&xo)[4]) {
+        L.off = u * BYTES;
+        xo[0] = 32 * u; xo[1] = 32 * u + 8; xo[2] = 32 * u + 16; xo[3] = 32 * u + 24;
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+        Data d;
+        const uint16_t* h = (const uint16_t*)(row + L.off);
+        d.dm = HAS_M ? ((uint32_t)h[0] | ((uint32_t)h[1] << 16)) : (uint32_t)h[0];
+        d.qh = HAS_QH ? ((uint32_t)h[QH / 2] | ((uint32_t)h[QH / 2 + 1] << 16)) : 0u;
+        d.q = ((const U4A2*)(row + L.off + QS))->v;
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const float (&x)[M][32], const float (&sx)[M][4],
+                                               float (&out)[M]) {
+        float acc[M];
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[m] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t lo = D.q[i] & 0x0F0F0F0Fu, hi = (D.q[i] >> 4) & 0x0F0F0F0Fu;
+            if (HAS_QH) {   // bit j of a 4-bit field -> bit 4 of byte j
+                lo |= ((((D.qh >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+                hi |= ((((D.qh >> (16 + 4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+            }
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float fl = ub(lo, k), fh = ub(hi, k);
+#pragma unroll
+                for (int m = 0; m < M; m++) {
+                    acc[m] = fmaf(x[m][4 * i + k], fl, acc[m]);
+                    acc[m] = fmaf(x[m][16 + 4 * i + k], fh, acc[m]);
+                }
+            }
+        }
+        const float d = f16_bits(D.dm & 0xFFFFu), mn = HAS_M ? f16_bits(D.dm >> 16) : 0.f;
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float s = (sx[m][0] + sx[m][1]) + (sx[m][2] + sx[m][3]);
+            // sum x (q - OFF) d + m sum x
+            out[m] = fmaf(d, fmaf(-(float)OFF, s, acc[m]), mn * s);
+        }
+    }
+};
+typedef Legacy<18, false, false, 8> Q40;
+typedef Legacy<20, true, false, 0> Q41;
+typedef Legacy<22, false, true, 16> Q50;
+typedef Legacy<24, true, true, 0> Q51;
+
+struct Q5K {
+    // 176 B = [f16 d][f16 dmin][12 B packed 6-bit scales/mins][32 B high bits][128 B nibbles]: Q4_K plus bit s of qh[l] as
+    // the fifth bit of element l of sub-block s (crates/ferric-gguf/src/lib.rs:692-716); every piece 16-byte aligned.
+    struct Lane { uint32_t off_h, off_q, off_b, sh, g2; bool high; };
+    struct Data { u32x4 h, q, b; __device__ __forceinline__ void pin_all() { pin(h); pin(q); pin(b); } };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&xo)[4]) {
+        int b = u >> 3, p = u & 7, g = p >> 1, hf = p & 1;
+        L.off_h = b * 176;
+        L.off_b = b * 176 + 16 + 16 * hf;   // qh[16hf, 16hf+16)
+        L.off_q = b * 176 + 48 + 16 * p;    // qs[16p, 16p+16): group g, l in [16hf, 16hf+16)
+        L.sh = 16 * (g & 1);
+        L.g2 = 2 * g;
+        L.high = g >= 2;
+        int base = 256 * b + 64 * g + 16 * hf;
+        xo[0] = base; xo[1] = base + 8; xo[2] = base + 32; xo[3] = base + 40;  // sub-block 2g, then 2g+1
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+        Data d;
+        d.h = *(const u32x4*)(row + L.off_h);
+        d.q = *(const u32x4*)(row + L.off_q);
+        d.b = *(const u32x4*)(row + L.off_b);
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const float (&x)[M][32], const float (&sx)[M][4],
+                                               float (&out)[M]) {
+        uint32_t a = D.h[1] >> L.sh, b = D.h[2] >> L.sh, c = D.h[3] >> L.sh;
+        uint32_t scp = L.high ? ((c & 0x0F0Fu) | ((a >> 2) & 0x3030u)) : (a & 0x3F3Fu);
+        uint32_t mp = L.high ? (((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u)) : (b & 0x3F3Fu);
+        float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
+        float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1);
+        float m0 = dmin * ub(mp, 0), m1 = dmin * ub(mp, 1);
+        float lo[M], hi[M];
+#pragma unroll
+        for (int m = 0; m < M; m++) { lo[m] = 0.f; hi[m] = 0.f; }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t hb = D.b[i] >> L.g2;
+            uint32_t ql = (D.q[i] & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4);
+            uint32_t qh = ((D.q[i] >> 4) & 0x0F0F0F0Fu) | ((hb & 0x02020202u) << 3);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float fl = ub(ql, k), fh = ub(qh, k);
+#pragma unroll
+                for (int m = 0; m < M; m++) {
+                    lo[m] = fmaf(x[m][4 * i + k], fl, lo[m]);
+                    hi[m] = fmaf(x[m][16 + 4 * i + k], fh, hi[m]);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            out[m] = d0 * lo[m] - m0 * (sx[m][0] + sx[m][1]) + (d1 * hi[m] - m1 * (sx[m][2] + sx[m][3]));
+    }
+};
+
 struct GemvParams {
     const uint8_t* W;
     const float* x;      // [M, cols]
@@ -420,6 +534,14 @@ int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, f
         case FHIP_Q8_0:
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for Q8_0");
             return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, s);
+        case FHIP_Q5_K: return n_ff ? launch_fmt<Q5K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_fmt<Q5K, false>(w, d_x, rows_x, d_y, out_rows, s);
+        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1:
+            // the reference fuses gate/up + SwiGLU for the K-quants only (crates/ferric-tensor/src/dtype.rs:949-959)
+            if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for ggml type %u", w->type);
+            if (w->type == FHIP_Q4_0) return launch_fmt<Q40, false>(w, d_x, rows_x, d_y, out_rows, s);
+            if (w->type == FHIP_Q4_1) return launch_fmt<Q41, false>(w, d_x, rows_x, d_y, out_rows, s);
+            if (w->type == FHIP_Q5_0) return launch_fmt<Q50, false>(w, d_x, rows_x, d_y, out_rows, s);
+            return launch_fmt<Q51, false>(w, d_x, rows_x, d_y, out_rows, s);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }
@@ -431,6 +553,11 @@ int launch_gemv_generic_sel(const fhip_weight* w, const float* d_x, float* d_y, 
         case FHIP_Q4_K: return swiglu ? launch_one<Q4K, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q4K, 1, false>(w, d_x, d_y, out_rows, s, &sel);
         case FHIP_Q6_K: return swiglu ? launch_one<Q6K, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q6K, 1, false>(w, d_x, d_y, out_rows, s, &sel);
         case FHIP_Q8_0: return swiglu ? launch_one<Q80, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q80, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_Q5_K: return swiglu ? launch_one<Q5K, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q5K, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_Q4_0: return swiglu ? launch_one<Q40, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q40, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_Q4_1: return swiglu ? launch_one<Q41, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q41, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_Q5_0: return swiglu ? launch_one<Q50, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q50, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_Q5_1: return swiglu ? launch_one<Q51, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q51, 1, false>(w, d_x, d_y, out_rows, s, &sel);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

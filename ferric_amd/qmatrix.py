@@ -19,6 +19,7 @@ import numpy as np
 from . import _lib
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13   # further formats: unpackers, mat-vec / small batch, "_id" variants
 
 
 def _vp(a):
@@ -168,10 +169,25 @@ class Tensor:
     def matmul_q6_k(self, w, stream=None):  # dtype.rs:1172
         return self._matmul_typed(w, Q6_K, stream)
 
+    def matmul_q5_k(self, w, stream=None):  # dtype.rs:1049
+        return self._matmul_typed(w, Q5_K, stream)
+
+    def matmul_q4_0(self, w, stream=None):  # dtype.rs:1838
+        return self._matmul_typed(w, Q4_0, stream)
+
+    def matmul_q4_1(self, w, stream=None):  # dtype.rs:1860
+        return self._matmul_typed(w, Q4_1, stream)
+
+    def matmul_q5_0(self, w, stream=None):  # dtype.rs:1882
+        return self._matmul_typed(w, Q5_0, stream)
+
+    def matmul_q5_1(self, w, stream=None):  # dtype.rs:1904
+        return self._matmul_typed(w, Q5_1, stream)
+
     def try_matmul_swiglu(self, w, stream=None):
         """Fused gate/up + SwiGLU -- dtype.rs:949. None when the format has no fused kernel
-        (Q8_0); the caller then runs matmul_q(w).swiglu(n_ff)."""
-        if w.ggml_type not in (Q4_K, Q6_K):
+        (Q8_0 and the 32-value formats); the caller then runs matmul_q(w).swiglu(n_ff)."""
+        if w.ggml_type not in (Q4_K, Q6_K, Q5_K):
             return None
         rows, inn = self._rows_inner()
         assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
@@ -185,6 +201,10 @@ class Tensor:
 
     def matmul_q6_k_swiglu(self, w, stream=None):  # dtype.rs:1802
         assert w.ggml_type == Q6_K
+        return self.try_matmul_swiglu(w, stream)
+
+    def matmul_q5_k_swiglu(self, w, stream=None):  # dtype.rs:1784
+        assert w.ggml_type == Q5_K
         return self.try_matmul_swiglu(w, stream)
 
     def swiglu(self, d, stream=None):
@@ -221,7 +241,8 @@ class Tensor:
                                              float(scale), int(bool(norm)), out.buf.ptr, _stream_handle(stream)))
         return out
 
-    def _swiglu_id(self, w, selw, k, eff, stream):
+    def matmul_q_swiglu_id(self, w, selw, k, eff, stream=None):
+        """Any format's selected-expert gate|up + SwiGLU (the typed methods below assert the format and call this)."""
         t, inn = self._rows_inner()
         assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
         assert 1 <= k <= 8, "k must be 1..=8"
@@ -232,12 +253,12 @@ class Tensor:
     def matmul_q4_k_swiglu_id(self, w, selw, k, eff, stream=None):
         """Selected experts' gate|up + SwiGLU for every (token, slot): [T, in] -> [T, k, eff] -- dtype.rs:1620."""
         assert w.ggml_type == Q4_K
-        return self._swiglu_id(w, selw, k, eff, stream)
+        return self.matmul_q_swiglu_id(w, selw, k, eff, stream)
 
     def matmul_q8_0_swiglu_id(self, w, selw, k, eff, stream=None):
         """dtype.rs:1731."""
         assert w.ggml_type == Q8_0
-        return self._swiglu_id(w, selw, k, eff, stream)
+        return self.matmul_q_swiglu_id(w, selw, k, eff, stream)
 
     def matmul_q6_k_id(self, w, selw, out_pe, stream=None):
         """Selected experts' down projection, one row per slot: [k, in] -> [k, out_pe] -- dtype.rs:1640."""
@@ -248,7 +269,8 @@ class Tensor:
         _lib.check(_lib.load().fhip_matmul_q_id(w.handle, self.buf.ptr, selw.buf.ptr, k, out_pe, out.buf.ptr, _stream_handle(stream)))
         return out
 
-    def _id_wsum(self, w, selw, out_pe, stream):
+    def matmul_q_id_wsum(self, w, selw, out_pe, stream=None):
+        """Any format's selected-expert down projection with the weighted sum over slots fused."""
         t, k, inn = self.shape if len(self.shape) == 3 else (1, self.shape[0], self.shape[1])
         assert 1 <= k <= 8, "k must be 1..=8"
         assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
@@ -265,17 +287,22 @@ class Tensor:
     def matmul_q6_k_id_wsum(self, w, selw, out_pe, stream=None):
         """Down projection with the weighted sum over slots fused: [T, k, in] -> [T, out_pe] -- dtype.rs:1662."""
         assert w.ggml_type == Q6_K
-        return self._id_wsum(w, selw, out_pe, stream)
+        return self.matmul_q_id_wsum(w, selw, out_pe, stream)
 
     def matmul_q4_k_id_wsum(self, w, selw, out_pe, stream=None):
         """dtype.rs:1765."""
         assert w.ggml_type == Q4_K
-        return self._id_wsum(w, selw, out_pe, stream)
+        return self.matmul_q_id_wsum(w, selw, out_pe, stream)
 
     def matmul_q8_0_id_wsum(self, w, selw, out_pe, stream=None):
         """dtype.rs:1748."""
         assert w.ggml_type == Q8_0
-        return self._id_wsum(w, selw, out_pe, stream)
+        return self.matmul_q_id_wsum(w, selw, out_pe, stream)
+
+    def matmul_q5_0_id_wsum(self, w, selw, out_pe, stream=None):
+        """dtype.rs:1686 (the expert down slab of a mixed-precision checkpoint)."""
+        assert w.ggml_type == Q5_0
+        return self.matmul_q_id_wsum(w, selw, out_pe, stream)
 
     def cvt_bf16(self, stream=None):
         """f32 -> bf16 bit patterns (round to nearest even), same shape."""
@@ -413,6 +440,11 @@ def _typed(ty, name):
 Q8_0Weights = _typed(Q8_0, "Q8_0Weights")
 Q4_KWeights = _typed(Q4_K, "Q4_KWeights")
 Q6_KWeights = _typed(Q6_K, "Q6_KWeights")
+Q5_KWeights = _typed(Q5_K, "Q5_KWeights")
+Q4_0Weights = _typed(Q4_0, "Q4_0Weights")
+Q4_1Weights = _typed(Q4_1, "Q4_1Weights")
+Q5_0Weights = _typed(Q5_0, "Q5_0Weights")
+Q5_1Weights = _typed(Q5_1, "Q5_1Weights")
 
 
 def type_size(ty, n):
@@ -424,7 +456,7 @@ def type_size(ty, n):
 
 def deq_raw(raw, n, ty):
     """Dequantize n elements out of raw block bytes on the GPU -- lib.rs:497. Same edge behaviour:
-    K-quants return n values with a ragged tail left 0.0, Q8_0 returns whole blocks only."""
+    every format returns n values with a ragged tail left 0.0, except Q8_0, which returns whole blocks only."""
     lib = _lib.init()
     a = np.ascontiguousarray(raw, dtype=np.uint8)
     out = np.empty(n, dtype=np.float32)

@@ -5,7 +5,9 @@ Pure data generation (numpy); no arithmetic of the matmul path lives here.
 import numpy as np
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13
+BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24),
+         Q5_K: (256, 176)}
 
 
 def q4k_pack_scales(sc, m):
@@ -35,6 +37,18 @@ def synth_weights(ty, rows, cols, seed):
         b[:, 2:4] = (np.abs(rng.standard_normal(nb)) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)
         b[:, 4:16] = q4k_pack_scales(rng.integers(0, 64, (nb, 8), dtype=np.uint8), rng.integers(0, 64, (nb, 8), dtype=np.uint8))
         b[:, 16:] = rng.integers(0, 256, (nb, 128), dtype=np.uint8)
+    elif ty in (Q4_0, Q4_1, Q5_0, Q5_1):
+        # f16 scale (and a signed f16 offset for the affine formats), every other byte uniform
+        f16 = lambda v: v.astype(np.float16).view(np.uint8).reshape(nb, 2)
+        b[:, 2:] = rng.integers(0, 256, (nb, bytes_ - 2), dtype=np.uint8)
+        b[:, 0:2] = f16(np.abs(rng.standard_normal(nb)) * 0.02)
+        if ty in (Q4_1, Q5_1):
+            b[:, 2:4] = f16(rng.standard_normal(nb) * 0.1)
+    elif ty == Q5_K:
+        b[:, 0:2] = (np.abs(rng.standard_normal(nb)) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)
+        b[:, 2:4] = (np.abs(rng.standard_normal(nb)) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)
+        b[:, 4:16] = q4k_pack_scales(rng.integers(0, 64, (nb, 8), dtype=np.uint8), rng.integers(0, 64, (nb, 8), dtype=np.uint8))
+        b[:, 16:] = rng.integers(0, 256, (nb, 160), dtype=np.uint8)
     else:
         b[:, 0:192] = rng.integers(0, 256, (nb, 192), dtype=np.uint8)
         b[:, 192:208] = rng.integers(-32, 32, (nb, 16), dtype=np.int8).view(np.uint8)

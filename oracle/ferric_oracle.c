@@ -30,8 +30,13 @@
 #include <stdlib.h>
 #include <string.h>
 
+#define GGML_Q4_0 2u
+#define GGML_Q4_1 3u
+#define GGML_Q5_0 6u
+#define GGML_Q5_1 7u
 #define GGML_Q8_0 8u
 #define GGML_Q4_K 12u
+#define GGML_Q5_K 13u
 #define GGML_Q6_K 14u
 
 /* ---------------------------------------------------------------- f16 <-> f32 */
@@ -100,6 +105,11 @@ size_t fo_type_size(uint32_t ty, size_t n) {
         case GGML_Q8_0: return n / 32 * 34;
         case GGML_Q4_K: return n / 256 * 144;
         case GGML_Q6_K: return n / 256 * 210;
+        case GGML_Q4_0: return n / 32 * 18;
+        case GGML_Q4_1: return n / 32 * 20;
+        case GGML_Q5_0: return n / 32 * 22;
+        case GGML_Q5_1: return n / 32 * 24;
+        case GGML_Q5_K: return n / 256 * 176;
         default: return 0;
     }
 }
@@ -110,6 +120,11 @@ int fo_block_bytes(uint32_t ty, size_t* vals, size_t* bytes) {
         case GGML_Q8_0: *vals = 32; *bytes = 34; return 1;
         case GGML_Q4_K: *vals = 256; *bytes = 144; return 1;
         case GGML_Q6_K: *vals = 256; *bytes = 210; return 1;
+        case GGML_Q4_0: *vals = 32; *bytes = 18; return 1;
+        case GGML_Q4_1: *vals = 32; *bytes = 20; return 1;
+        case GGML_Q5_0: *vals = 32; *bytes = 22; return 1;
+        case GGML_Q5_1: *vals = 32; *bytes = 24; return 1;
+        case GGML_Q5_K: *vals = 256; *bytes = 176; return 1;
         default: return 0;
     }
 }
@@ -195,6 +210,112 @@ size_t fo_deq_q6_k(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
     return n;
 }
 
+/* ---- the other block formats of the same reader (the "next" formats of the path) ----
+ * Pinning: each sequential form is checked bit for bit against its element formula taken from the
+ * reference's GPU kernels (second formulation, below), against a numpy twin written from the layout, and
+ * against closed-form relations to the formats pinned above (Q5_K with qh = 0 is Q4_K on the same bytes;
+ * Q5_1 with qh = 0 is Q4_1; Q5_0 = Q4_0 - 8d when qh = 0; Q4_1 with m = -8d is Q4_0 where -8d is exact).
+ * The reference tree holds no known-answer vectors for these five. */
+
+static inline uint32_t rd_u32(const uint8_t* b) { return (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24); }
+
+/* crates/ferric-gguf/src/lib.rs:618-629: x = (nibble - 8) * d, low nibbles then high. */
+size_t fo_deq_q4_0(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 32, have = raw_len / 18;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 18;
+        float d = fo_f16_to_f32(rd_u16(blk));
+        for (int i = 0; i < 16; i++) {
+            uint8_t byte = blk[2 + i];
+            out[bi * 32 + i] = (float)((int)(byte & 0x0F) - 8) * d;
+            out[bi * 32 + i + 16] = (float)((int)(byte >> 4) - 8) * d;
+        }
+    }
+    return n;
+}
+
+/* crates/ferric-gguf/src/lib.rs:633-645: x = nibble * d + m. */
+size_t fo_deq_q4_1(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 32, have = raw_len / 20;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 20;
+        float d = fo_f16_to_f32(rd_u16(blk)), m = fo_f16_to_f32(rd_u16(blk + 2));
+        for (int i = 0; i < 16; i++) {
+            uint8_t byte = blk[4 + i];
+            out[bi * 32 + i] = (float)(byte & 0x0F) * d + m;
+            out[bi * 32 + i + 16] = (float)(byte >> 4) * d + m;
+        }
+    }
+    return n;
+}
+
+/* crates/ferric-gguf/src/lib.rs:650-665: x = ((nibble | bit << 4) - 16) * d, bit i of qh for value i, bit i+16 for i+16. */
+size_t fo_deq_q5_0(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 32, have = raw_len / 22;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 22;
+        float d = fo_f16_to_f32(rd_u16(blk));
+        uint32_t qh = rd_u32(blk + 2);
+        for (int i = 0; i < 16; i++) {
+            uint8_t byte = blk[6 + i];
+            uint32_t xh0 = ((qh >> i) & 1u) << 4, xh1 = ((qh >> (i + 16)) & 1u) << 4;
+            out[bi * 32 + i] = (float)((int)((uint32_t)(byte & 0x0F) | xh0) - 16) * d;
+            out[bi * 32 + i + 16] = (float)((int)((uint32_t)(byte >> 4) | xh1) - 16) * d;
+        }
+    }
+    return n;
+}
+
+/* crates/ferric-gguf/src/lib.rs:669-684: x = (nibble | bit << 4) * d + m. */
+size_t fo_deq_q5_1(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 32, have = raw_len / 24;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 24;
+        float d = fo_f16_to_f32(rd_u16(blk)), m = fo_f16_to_f32(rd_u16(blk + 2));
+        uint32_t qh = rd_u32(blk + 4);
+        for (int i = 0; i < 16; i++) {
+            uint8_t byte = blk[8 + i];
+            uint32_t xh0 = ((qh >> i) & 1u) << 4, xh1 = ((qh >> (i + 16)) & 1u) << 4;
+            out[bi * 32 + i] = (float)((uint32_t)(byte & 0x0F) | xh0) * d + m;
+            out[bi * 32 + i + 16] = (float)((uint32_t)(byte >> 4) | xh1) * d + m;
+        }
+    }
+    return n;
+}
+
+/* crates/ferric-gguf/src/lib.rs:692-716: Q4_K plus one high bit per value, y = (d*sc)*(nibble + 16*bit) - dmin*m. */
+size_t fo_deq_q5_k(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 256, have = raw_len / 176;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 176;
+        float d = fo_f16_to_f32(rd_u16(blk)), dmin = fo_f16_to_f32(rd_u16(blk + 2));
+        const uint8_t* scales = blk + 4; const uint8_t* qh = blk + 16; const uint8_t* qs = blk + 48;
+        size_t y = bi * 256, q = 0; int is = 0;
+        for (int jg = 0; jg < 4; jg++) {
+            uint8_t sc1, m1, sc2, m2;
+            get_sc_min(scales, is, &sc1, &m1);
+            get_sc_min(scales, is + 1, &sc2, &m2);
+            float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+            float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
+            uint8_t b1 = (uint8_t)(1u << (2 * jg)), b2 = (uint8_t)(1u << (2 * jg + 1));
+            for (int l = 0; l < 32; l++) out[y + l] = d1 * (float)((qs[q + l] & 0x0F) + ((qh[l] & b1) ? 16 : 0)) - mm1;
+            for (int l = 0; l < 32; l++) out[y + l + 32] = d2 * (float)((qs[q + l] >> 4) + ((qh[l] & b2) ? 16 : 0)) - mm2;
+            y += 64; q += 32; is += 2;
+        }
+    }
+    return n;
+}
+
 /* crates/ferric-gguf/src/lib.rs:497-520 (deq_raw), in-scope types. Returns the number of f32 the
  * reference's Vec would hold, or (size_t)-1 for "unsupported ggml type". */
 size_t fo_deq_raw(const uint8_t* raw, size_t raw_len, size_t n, uint32_t ty, float* out) {
@@ -202,6 +323,11 @@ size_t fo_deq_raw(const uint8_t* raw, size_t raw_len, size_t n, uint32_t ty, flo
         case GGML_Q8_0: return fo_deq_q8_0(raw, raw_len, n, out);
         case GGML_Q4_K: return fo_deq_q4_k(raw, raw_len, n, out);
         case GGML_Q6_K: return fo_deq_q6_k(raw, raw_len, n, out);
+        case GGML_Q4_0: return fo_deq_q4_0(raw, raw_len, n, out);
+        case GGML_Q4_1: return fo_deq_q4_1(raw, raw_len, n, out);
+        case GGML_Q5_0: return fo_deq_q5_0(raw, raw_len, n, out);
+        case GGML_Q5_1: return fo_deq_q5_1(raw, raw_len, n, out);
+        case GGML_Q5_K: return fo_deq_q5_k(raw, raw_len, n, out);
         default: return (size_t)-1;
     }
 }
@@ -242,12 +368,63 @@ float fo_q8_0_elem(const uint8_t* blk, int v) {
     return (float)(int8_t)blk[2 + v] * fo_f16_to_f32(rd_u16(blk));
 }
 
+/* crates/ferric-tensor/src/dtype.rs:3548-3555 (Q4_0: word w of a block holds values 4w..4w+3 in its low nibbles and
+ * 16+4w.. in its high nibbles) and :3613-3620 (Q4_1, the same words with + m). */
+float fo_q4_0_elem(const uint8_t* blk, int v) {
+    uint32_t word = rd_u32(blk + 2 + 4 * ((v & 15) >> 2));
+    int nib = (int)((word >> (8 * (v & 3) + (v >= 16 ? 4 : 0))) & 0xFu);
+    return (float)(nib - 8) * fo_f16_to_f32(rd_u16(blk));
+}
+float fo_q4_1_elem(const uint8_t* blk, int v) {
+    uint32_t word = rd_u32(blk + 4 + 4 * ((v & 15) >> 2));
+    uint32_t nib = (word >> (8 * (v & 3) + (v >= 16 ? 4 : 0))) & 0xFu;
+    return (float)nib * fo_f16_to_f32(rd_u16(blk)) + fo_f16_to_f32(rd_u16(blk + 2));
+}
+/* crates/ferric-tensor/src/dtype.rs:3778-3792 (Q5_0: fifth bit of value base+c is qh bit base+c, of 16+base+c bit
+ * base+16+c) and :3858-3874 (Q5_1). */
+float fo_q5_0_elem(const uint8_t* blk, int v) {
+    uint32_t qh = rd_u32(blk + 2), word = rd_u32(blk + 6 + 4 * ((v & 15) >> 2));
+    uint32_t nib = (word >> (8 * (v & 3) + (v >= 16 ? 4 : 0))) & 0xFu;
+    return (float)((int)(nib | (((qh >> v) & 1u) << 4)) - 16) * fo_f16_to_f32(rd_u16(blk));
+}
+float fo_q5_1_elem(const uint8_t* blk, int v) {
+    uint32_t qh = rd_u32(blk + 4), word = rd_u32(blk + 8 + 4 * ((v & 15) >> 2));
+    uint32_t nib = (word >> (8 * (v & 3) + (v >= 16 ? 4 : 0))) & 0xFu;
+    return (float)(nib | (((qh >> v) & 1u) << 4)) * fo_f16_to_f32(rd_u16(blk)) + fo_f16_to_f32(rd_u16(blk + 2));
+}
+/* crates/ferric-tensor/src/dtype.rs:1108-1121 (Q5_K element of the matrix-unit kernel: sub-block s = v/32, l = v%32,
+ * nibble from qs word 8*(s/2) + l/4, fifth bit = bit s of qh byte l), in raw-block offsets (qh at 16, qs at 48). */
+float fo_q5k_elem(const uint8_t* blk, int v) {
+    float d = fo_f16_to_f32(rd_u16(blk)), dmin = fo_f16_to_f32(rd_u16(blk + 2));
+    const uint8_t* s = blk + 4;
+    int sb = v / 32, l = v % 32;
+    uint32_t sc, m;
+    if (sb < 4) { sc = s[sb] & 63u; m = s[sb + 4] & 63u; }
+    else { sc = (s[sb + 4] & 15u) | ((uint32_t)(s[sb - 4] >> 6) << 4); m = (uint32_t)(s[sb + 4] >> 4) | ((uint32_t)(s[sb] >> 6) << 4); }
+    uint32_t qsw = rd_u32(blk + 48 + 4 * (8 * (sb >> 1) + (l >> 2)));
+    uint32_t nib = (qsw >> (8 * (l & 3) + ((sb & 1) ? 4 : 0))) & 0xFu;
+    uint32_t qhw = rd_u32(blk + 16 + 4 * (l >> 2));
+    uint32_t bit = (qhw >> (8 * (l & 3) + sb)) & 1u;
+    float ds = d * (float)sc, mm = dmin * (float)m;
+    return ds * (float)(nib + bit * 16u) - mm;
+}
+
 void fo_deq_elemwise(const uint8_t* raw, size_t n, uint32_t ty, float* out) {
     size_t vals, bytes;
     if (!fo_block_bytes(ty, &vals, &bytes)) return;
     for (size_t i = 0; i < n; i++) {
         const uint8_t* blk = raw + (i / vals) * bytes; int v = (int)(i % vals);
-        out[i] = ty == GGML_Q8_0 ? fo_q8_0_elem(blk, v) : ty == GGML_Q4_K ? fo_q4k_elem(blk, v) : fo_q6k_elem(blk, v);
+        switch (ty) {
+            case GGML_Q8_0: out[i] = fo_q8_0_elem(blk, v); break;
+            case GGML_Q4_K: out[i] = fo_q4k_elem(blk, v); break;
+            case GGML_Q6_K: out[i] = fo_q6k_elem(blk, v); break;
+            case GGML_Q4_0: out[i] = fo_q4_0_elem(blk, v); break;
+            case GGML_Q4_1: out[i] = fo_q4_1_elem(blk, v); break;
+            case GGML_Q5_0: out[i] = fo_q5_0_elem(blk, v); break;
+            case GGML_Q5_1: out[i] = fo_q5_1_elem(blk, v); break;
+            case GGML_Q5_K: out[i] = fo_q5k_elem(blk, v); break;
+            default: break;
+        }
     }
 }
 

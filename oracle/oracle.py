@@ -14,7 +14,9 @@ import subprocess
 import numpy as np
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13
+BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24),
+         Q5_K: (256, 176)}
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libferric_oracle.so")
@@ -398,5 +400,51 @@ def np_deq_q6_k(raw, n):
     return out
 
 
+def _np_legacy(raw, n, bytes_, has_m, has_qh, off):
+    """The four 32-value formats from their layout: [f16 d][f16 m]?[u32 qh]?[16 bytes of nibbles]; value i takes the
+    low nibble of byte i, value 16+i the high one; the fifth bit of value v is bit v of qh."""
+    out = np.zeros(n, np.float32)
+    nb = min(n // 32, len(raw) // bytes_)
+    b = np.asarray(raw[: nb * bytes_], dtype=np.uint8).reshape(nb, bytes_)
+    d = _np_f16(b[:, 0:2]).reshape(nb, 1)
+    p = 2
+    m = None
+    if has_m:
+        m = _np_f16(b[:, 2:4]).reshape(nb, 1)
+        p = 4
+    q = np.concatenate([b[:, p + 4 * has_qh:] & 0x0F, b[:, p + 4 * has_qh:] >> 4], axis=1).astype(np.int32)   # [nb, 32]
+    if has_qh:
+        qh = b[:, p:p + 4].copy().view("<u4").reshape(nb, 1)
+        q = q | (((qh >> np.arange(32, dtype=np.uint32)) & 1).astype(np.int32) << 4)
+    v = (q - off).astype(np.float32) * d
+    if has_m:
+        v = v + m
+    out[: nb * 32] = v.reshape(-1)
+    return out
+
+
+def np_deq_q4_0(raw, n): return _np_legacy(raw, n, 18, False, False, 8)
+def np_deq_q4_1(raw, n): return _np_legacy(raw, n, 20, True, False, 0)
+def np_deq_q5_0(raw, n): return _np_legacy(raw, n, 22, False, True, 16)
+def np_deq_q5_1(raw, n): return _np_legacy(raw, n, 24, True, True, 0)
+
+
+def np_deq_q5_k(raw, n):
+    out = np.zeros(n, np.float32)
+    nb = min(n // 256, len(raw) // 176)
+    b = np.asarray(raw[: nb * 176], dtype=np.uint8).reshape(nb, 176)
+    d = _np_f16(b[:, 0:2]).reshape(nb, 1); dmin = _np_f16(b[:, 2:4]).reshape(nb, 1)
+    sc, m = np_q4k_scales(b[:, 4:16])
+    qh = b[:, 16:48].reshape(nb, 1, 32)
+    qs = b[:, 48:].reshape(nb, 4, 32)
+    nib = np.stack([qs & 0x0F, qs >> 4], axis=2).reshape(nb, 8, 32).astype(np.int32)       # sub-block 2g, 2g+1
+    bit = ((qh >> np.arange(8, dtype=np.uint8).reshape(1, 8, 1)) & 1).astype(np.int32)        # bit s of qh[l]
+    d1 = (d * sc.astype(np.float32)).reshape(nb, 8, 1)
+    mm = (dmin * m.astype(np.float32)).reshape(nb, 8, 1)
+    out[: nb * 256] = (d1 * (nib + 16 * bit).astype(np.float32) - mm).reshape(-1)
+    return out
+
+
 def np_deq_raw(raw, n, ty):
-    return {Q8_0: np_deq_q8_0, Q4_K: np_deq_q4_k, Q6_K: np_deq_q6_k}[ty](np.asarray(raw, dtype=np.uint8), n)
+    return {Q8_0: np_deq_q8_0, Q4_K: np_deq_q4_k, Q6_K: np_deq_q6_k, Q4_0: np_deq_q4_0, Q4_1: np_deq_q4_1, Q5_0: np_deq_q5_0,
+            Q5_1: np_deq_q5_1, Q5_K: np_deq_q5_k}[ty](np.asarray(raw, dtype=np.uint8), n)

@@ -37,11 +37,13 @@ def test_size_tables_need_no_device():
     # crates/ferric-gguf/src/lib.rs:471-494 and crates/ferric-tensor/src/dtype.rs:873-889
     from ferric_amd import QMatrix, type_size
     assert QMatrix.block_bytes(8) == (32, 34) and QMatrix.block_bytes(12) == (256, 144) and QMatrix.block_bytes(14) == (256, 210)
-    assert QMatrix.block_bytes(13) is None and QMatrix.block_bytes(0) is None
+    assert [QMatrix.block_bytes(t) for t in (2, 3, 6, 7, 13)] == [(32, 18), (32, 20), (32, 22), (32, 24), (256, 176)]
+    assert QMatrix.block_bytes(10) is None and QMatrix.block_bytes(0) is None
     assert type_size(8, 4096 * 4096) == 17825792 and type_size(12, 5120 * 5120) == 14745600 and type_size(14, 5120 * 17408) == 73113600
     assert type_size(12, 300) == 144
-    with pytest.raises(ValueError, match="unsupported ggml type 7"):
-        type_size(7, 32)
+    assert type_size(13, 5120 * 5120) == 18022400 and type_size(2, 64) == 36 and type_size(7, 33) == 24
+    with pytest.raises(ValueError, match="unsupported ggml type 10"):
+        type_size(10, 256)
 
 
 def test_compute_refuses_to_run_uninitialised():

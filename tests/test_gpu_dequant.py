@@ -87,8 +87,8 @@ def test_deq_raw_edge_semantics(F, O):
         got = F.deq_raw(w, n, Q8_0)
         assert got.size == min(n // 32, 4) * 32
         assert_bits_equal(got, O.deq_raw(w, n, Q8_0), f"Q8_0 n={n}")
-    with pytest.raises(ValueError, match="unsupported ggml type 13"):     # lib.rs:518
-        F.deq_raw(np.zeros(176, np.uint8), 256, 13)
+    with pytest.raises(ValueError, match="unsupported ggml type 10"):     # lib.rs:518 (Q2_K)
+        F.deq_raw(np.zeros(84, np.uint8), 256, 10)
 
 
 @pytest.mark.parametrize("ty,rows,cols", [(Q4_K, 64, 5120), (Q6_K, 33, 5120), (Q8_0, 40, 4096)])

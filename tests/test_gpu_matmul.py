@@ -227,8 +227,8 @@ def test_swiglu_unsupported_for_q8_0(F, O):
 
 def test_constructor_errors_match_the_reference(F):
     z = np.zeros(144 * 4, np.uint8)
-    with pytest.raises(ValueError, match="no native matmul for ggml type 13"):         # dtype.rs:855
-        F.QMatrix.from_bytes(z, 13, 1, 256)
+    with pytest.raises(ValueError, match="no native matmul for ggml type 10"):         # dtype.rs:855 (Q2_K)
+        F.QMatrix.from_bytes(z, 10, 1, 256)
     with pytest.raises(AssertionError, match="Q4_K cols must be a multiple of 256"):    # dtype.rs:1389
         F.Q4_KWeights.from_bytes(z, 1, 300)
     with pytest.raises(AssertionError, match="unexpected Q4_K byte length"):            # dtype.rs:1390
