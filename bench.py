@@ -59,7 +59,7 @@ class Timer:
 
 def weight_bytes(ty, rows, cols):
     vals, b = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), 2: (32, 18), 3: (32, 20), 6: (32, 22), 7: (32, 24),
-               13: (256, 176)}[ty]
+               13: (256, 176), 20: (32, 18), 23: (256, 136), 39: (32, 17)}[ty]
     return rows * (cols // vals) * b
 
 
@@ -402,9 +402,9 @@ def main():
         log("[bench] routed-expert block of an MoE decode layer ...")
         line["moe_routed_experts_q4k_q6k"] = bench_moe(F, lib, check, stream, timer)
     if not args.no_moe:
-        log("[bench] Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 GEMV 5120x5120 (generic kernel) ...")
+        log("[bench] Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / IQ4_XS / MXFP4 GEMV 5120x5120 (generic kernel) ...")
         other = {}
-        for name, ty in (("q5_k", 13), ("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7)):
+        for name, ty in (("q5_k", 13), ("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("iq4_nl", 20), ("iq4_xs", 23), ("mxfp4", 39)):
             r, a, nb = bench_gemv(F, lib, check, stream, timer, ty, rows, cols, 1024, 64, seed=20 + ty, x_seed=2, ncopy=48)
             other[name] = {"cold_us": r["cold"]["ms_per_step"] * 1e3, "cold_GBps": r["cold"]["GBps"],
                            "warm_us": r["warm"]["ms_per_step"] * 1e3, "algorithmic_bytes": a}

@@ -23,6 +23,9 @@ bool block_info(uint32_t ty, size_t& vals, size_t& bytes) {
         case FHIP_Q5_0: vals = 32; bytes = 22; return true;
         case FHIP_Q5_1: vals = 32; bytes = 24; return true;
         case FHIP_Q5_K: vals = 256; bytes = 176; return true;
+        case FHIP_IQ4_NL: vals = 32; bytes = 18; return true;
+        case FHIP_IQ4_XS: vals = 256; bytes = 136; return true;
+        case FHIP_MXFP4: vals = 32; bytes = 17; return true;
         default: return false;
     }
 }
@@ -37,6 +40,9 @@ const char* type_name(uint32_t ty) {
         case FHIP_Q5_0: return "Q5_0";
         case FHIP_Q5_1: return "Q5_1";
         case FHIP_Q5_K: return "Q5_K";
+        case FHIP_IQ4_NL: return "IQ4_NL";
+        case FHIP_IQ4_XS: return "IQ4_XS";
+        case FHIP_MXFP4: return "MXFP4";
         default: return "?";
     }
 }

@@ -8,7 +8,7 @@
 #include "../../include/ferric_hip.h"
 
 struct fhip_weight {
-    uint32_t type;      // ggml id: 2 / 3 / 6 / 7 / 8 / 12 / 13 / 14
+    uint32_t type;      // ggml id: 2 / 3 / 6 / 7 / 8 / 12 / 13 / 14 / 20 / 23 / 39
     size_t rows, cols;  // [out, in]
     size_t row_bytes;   // cols / block_values * block_bytes
     size_t nbytes;      // rows * row_bytes

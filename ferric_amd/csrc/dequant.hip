@@ -161,6 +161,65 @@ __global__ void deq_q5_k_kernel(const uint8_t* __restrict__ raw, size_t nquads, 
     *(float4*)(out + t * 4) = o;
 }
 
+// ---- IQ4_NL / IQ4_XS: 4-bit indices into a 16-level non-linear codebook (lib.rs:751), value = scale * level.
+//   IQ4_NL 18 B = [f16 d][qs[16]]                                  y = d * kv[idx]                  lib.rs:755-767
+//   IQ4_XS 136 B = [f16 d][u16 scales_h][scales_l[4]][qs[128]]     y = (d * (ls - 32)) * kv[idx]    lib.rs:772-791
+// element j of a 32-value (sub-)block is the low nibble of its qs[j], element 16 + j the high nibble. Every product is exact
+// in f32 (11-bit d x 6-bit ls x 7-bit level), so the order of the two multiplies cannot change a bit.
+__device__ const float KV_IQ4NL[16] = {-127.f, -104.f, -83.f, -65.f, -49.f, -35.f, -22.f, -10.f, 1.f, 13.f, 25.f, 38.f, 53.f, 69.f, 89.f, 113.f};
+
+template <bool XS>
+__global__ void deq_iq4_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane = 4 values
+    if (t >= nquads) return;
+    uint32_t q;
+    float dl;
+    bool high;
+    if (XS) {
+        size_t blk = t >> 6;
+        int v = (int)(t & 63) * 4, ib = v >> 5, l = v & 31;
+        const uint8_t* b = raw + blk * 136;  // 8-byte aligned
+        uint32_t hd = *(const uint32_t*)b, sl = *(const uint32_t*)(b + 4);
+        int ls = (int)(((sl >> (4 * ib)) & 0xFu) | ((((hd >> 16) >> (2 * ib)) & 3u) << 4));
+        dl = __fmul_rn(f16_bits(hd & 0xFFFFu), (float)(ls - 32));
+        q = *(const uint32_t*)(b + 8 + 16 * ib + (l & 15));
+        high = l >= 16;
+    } else {
+        size_t blk = t >> 3;
+        int v = (int)(t & 7) * 4;
+        const uint8_t* b = raw + blk * 18;
+        dl = f16_bits(*(const uint16_t*)b);
+        q = ld4_a2(b + 2 + (v & 15));
+        high = v >= 16;
+    }
+    if (high) q >>= 4;
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = __fmul_rn(dl, KV_IQ4NL[(q >> (8 * k)) & 0xFu]);
+    *(float4*)(out + t * 4) = make_float4(o[0], o[1], o[2], o[3]);
+}
+
+// ---- MXFP4: 17 B = [u8 e][qs[16]]; y = (2 * E2M1[code]) * 2^(e - 128), lib.rs:857-908. The doubled table with the halved
+// scale keeps (e = 255, code = 1) at the finite 2^127; e = 0 and 1 give subnormal scales, built from their bit patterns.
+// One IEEE multiply per value: it rounds only where the result is subnormal or overflows, exactly as the reference's does.
+__device__ const float KV_MXFP4_2X[16] = {0.f, 1.f, 2.f, 3.f, 4.f, 6.f, 8.f, 12.f, 0.f, -1.f, -2.f, -3.f, -4.f, -6.f, -8.f, -12.f};
+
+__global__ void deq_mxfp4_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
+    size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= nquads) return;
+    size_t blk = t >> 3;
+    int v = (int)(t & 7) * 4;
+    const uint8_t* b = raw + blk * 17;  // no alignment at all: byte loads
+    uint32_t e = b[0];
+    float d = __uint_as_float(e == 0 ? (1u << 21) : e == 1 ? (1u << 22) : (e - 1u) << 23);
+    const uint8_t* qs = b + 1 + (v & 15);
+    int sh = v >= 16 ? 4 : 0;
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = __fmul_rn(KV_MXFP4_2X[(qs[k] >> sh) & 0xFu], d);
+    *(float4*)(out + t * 4) = make_float4(o[0], o[1], o[2], o[3]);
+}
+
 }  // namespace
 
 namespace fhip {
@@ -174,7 +233,7 @@ int launch_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_
 
 int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d_out, hipStream_t s) {
     if (nblocks == 0) return FHIP_OK;
-    size_t vals = (type == FHIP_Q4_K || type == FHIP_Q5_K || type == FHIP_Q6_K) ? 256 : 32;
+    size_t vals = (type == FHIP_Q4_K || type == FHIP_Q5_K || type == FHIP_Q6_K || type == FHIP_IQ4_XS) ? 256 : 32;
     size_t nquads = nblocks * vals / 4;
     size_t grid = (nquads + 255) / 256;
     if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_ARG, "dequant: %zu blocks exceed one launch", nblocks);
@@ -187,6 +246,9 @@ int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d
         case FHIP_Q4_1: hipLaunchKernelGGL((deq_legacy_kernel<20, true, false, 0>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
         case FHIP_Q5_0: hipLaunchKernelGGL((deq_legacy_kernel<22, false, true, 16>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
         case FHIP_Q5_1: hipLaunchKernelGGL((deq_legacy_kernel<24, true, true, 0>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_IQ4_NL: hipLaunchKernelGGL((deq_iq4_kernel<false>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_IQ4_XS: hipLaunchKernelGGL((deq_iq4_kernel<true>), dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
+        case FHIP_MXFP4: hipLaunchKernelGGL(deq_mxfp4_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_raw, nquads, d_out); break;
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", type);
     }
     return check_hip(hipGetLastError(), "dequant launch");

@@ -628,7 +628,7 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
         case FHIP_Q8_0:
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for Q8_0");
             return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
-        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_Q5_K:
+        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_Q5_K: case FHIP_IQ4_NL: case FHIP_IQ4_XS: case FHIP_MXFP4:
             return launch_gemv_generic(w, d_x, rows_x, d_y, n_ff, s);   // no streaming kernel for these formats
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
@@ -648,7 +648,7 @@ int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t o
         case FHIP_Q4_K: return launch_sel_fmt<Q4K>(w, d_x, d_y, out_rows, swiglu, sel, s);
         case FHIP_Q6_K: return launch_sel_fmt<Q6K>(w, d_x, d_y, out_rows, swiglu, sel, s);
         case FHIP_Q8_0: return launch_sel_fmt<Q80>(w, d_x, d_y, out_rows, swiglu, sel, s);
-        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_Q5_K:
+        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_Q5_K: case FHIP_IQ4_NL: case FHIP_IQ4_XS: case FHIP_MXFP4:
             return launch_gemv_generic_sel(w, d_x, d_y, out_rows, swiglu, sel, s);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }

@@ -1,6 +1,6 @@
 // General-shape mat-vec (and small-batch mat-mat) on the raw GGUF block stream, gfx950: covers every
 // cols the formats allow (any multiple of 256, or of 32 for the 32-value formats), with plain f32 multiply-adds,
-// and every block format of the path (Q8_0, Q4_K, Q6_K, and Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q5_K).
+// and every block format of the path (Q8_0, Q4_K, Q6_K, and Q4_0 / Q4_1 / Q5_0 / Q5_1 / Q5_K / IQ4_NL / IQ4_XS / MXFP4).
 // The streaming kernel in gemv.hip takes over for row lengths it tiles exactly; this one is the
 // shape-complete path behind it.
 //
@@ -335,6 +335,123 @@ struct Q5K {
     }
 };
 
+// Four 4-bit indices (one per byte of idx, the upper nibbles clear) looked up in a 16-entry byte table held in t0..t3.
+__device__ __forceinline__ uint32_t lut16x4(uint32_t idx, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
+    uint32_t sel = idx & 0x07070707u;
+    uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel);   // selector 0..3: bytes of t0, 4..7: bytes of t1
+    uint32_t hi = __builtin_amdgcn_perm(t3, t2, sel);
+    uint32_t m = ((idx >> 3) & 0x01010101u) * 0xFFu;
+    return (hi & m) | (lo & ~m);
+}
+struct __attribute__((packed, aligned(8))) U4A8 { u32x4 v; };
+struct __attribute__((packed, aligned(1))) U4A1 { u32x4 v; };
+
+// IQ4_NL (18 B = [f16 d][qs[16]]) and IQ4_XS (136 B = [f16 d][u16 scales_h][scales_l[4]][qs[128]]): 4-bit indices into the
+// codebook {-127 .. 113} (crates/ferric-gguf/src/lib.rs:751-791); one unit = one 32-value (sub-)block, element j the low
+// nibble of its qs[j], element 16 + j the high one. The table is held biased by +128 so that a lookup result converts as an
+// unsigned byte; the bias leaves as 128 * sum(x): out = dl * (sum x (kv + 128) - 128 sum x), dl = d or d * (ls - 32).
+template <bool XS>
+struct IQ4 {
+    struct Lane { uint32_t off_h, off_q, ib; };
+    struct Data { u32x4 q; uint32_t h0, h1; __device__ __forceinline__ void pin_all() { pin(q); pin(h0); pin(h1); } };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&xo)[4]) {
+        if (XS) { L.ib = u & 7; L.off_h = (u >> 3) * 136; L.off_q = L.off_h + 8 + 16 * L.ib; }
+        else { L.ib = 0; L.off_h = u * 18; L.off_q = L.off_h + 2; }
+        xo[0] = 32 * u; xo[1] = 32 * u + 8; xo[2] = 32 * u + 16; xo[3] = 32 * u + 24;
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+        Data d;
+        if (XS) {
+            d.h0 = *(const uint32_t*)(row + L.off_h);
+            d.h1 = *(const uint32_t*)(row + L.off_h + 4);
+            d.q = ((const U4A8*)(row + L.off_q))->v;
+        } else {
+            d.h0 = *(const uint16_t*)(row + L.off_h);
+            d.h1 = 0;
+            d.q = ((const U4A2*)(row + L.off_q))->v;
+        }
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const float (&x)[M][32], const float (&sx)[M][4],
+                                               float (&out)[M]) {
+        float acc[M];
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[m] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t lo = lut16x4(D.q[i] & 0x0F0F0F0Fu, 0x3F2D1801u, 0x766A5D4Fu, 0xA6998D81u, 0xF1D9C5B5u);
+            uint32_t hi = lut16x4((D.q[i] >> 4) & 0x0F0F0F0Fu, 0x3F2D1801u, 0x766A5D4Fu, 0xA6998D81u, 0xF1D9C5B5u);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float fl = ub(lo, k), fh = ub(hi, k);
+#pragma unroll
+                for (int m = 0; m < M; m++) {
+                    acc[m] = fmaf(x[m][4 * i + k], fl, acc[m]);
+                    acc[m] = fmaf(x[m][16 + 4 * i + k], fh, acc[m]);
+                }
+            }
+        }
+        float dl = f16_bits(D.h0 & 0xFFFFu);
+        if (XS) {
+            int ls = (int)(((D.h1 >> (4 * L.ib)) & 0xFu) | ((((D.h0 >> 16) >> (2 * L.ib)) & 3u) << 4));
+            dl *= (float)(ls - 32);
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            const float s = (sx[m][0] + sx[m][1]) + (sx[m][2] + sx[m][3]);
+            out[m] = dl * fmaf(-128.f, s, acc[m]);
+        }
+    }
+};
+typedef IQ4<false> IQ4NL;
+typedef IQ4<true> IQ4XS;
+
+// MXFP4 (17 B = [u8 e][qs[16]], crates/ferric-gguf/src/lib.rs:857-908): weight = (2 * E2M1[code]) * 2^(e - 128), formed BEFORE
+// it meets the activation as the reference's kernel does (crates/ferric-tensor/src/dtype.rs:3331-3344): a block whose scale
+// saturates contributes inf whatever x is. Magnitudes {0,1,2,3,4,6,8,12} by byte permute on the low three bits of a code, the
+// fourth bit is the sign. Blocks have no alignment; the hardware's unaligned global loads take them.
+struct MXF4 {
+    struct Lane { uint32_t off; };
+    struct Data { u32x4 q; uint32_t e; __device__ __forceinline__ void pin_all() { pin(q); pin(e); } };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&xo)[4]) {
+        L.off = u * 17;
+        xo[0] = 32 * u; xo[1] = 32 * u + 8; xo[2] = 32 * u + 16; xo[3] = 32 * u + 24;
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+        Data d;
+        d.e = row[L.off];
+        d.q = ((const U4A1*)(row + L.off + 1))->v;
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const float (&x)[M][32], const float (&)[M][4],
+                                               float (&out)[M]) {
+        const float d = __uint_as_float(D.e == 0 ? (1u << 21) : D.e == 1 ? (1u << 22) : (D.e - 1u) << 23);
+        float acc[M];
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[m] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t q = D.q[i];
+            uint32_t lo = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, q & 0x07070707u);
+            uint32_t hi = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, (q >> 4) & 0x07070707u);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float wl = __uint_as_float(__float_as_uint(ub(lo, k) * d) | ((q << (28 - 8 * k)) & 0x80000000u));
+                float wh = __uint_as_float(__float_as_uint(ub(hi, k) * d) | ((q << (24 - 8 * k)) & 0x80000000u));
+#pragma unroll
+                for (int m = 0; m < M; m++) {
+                    acc[m] = fmaf(x[m][4 * i + k], wl, acc[m]);
+                    acc[m] = fmaf(x[m][16 + 4 * i + k], wh, acc[m]);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++) out[m] = acc[m];
+    }
+};
+
 struct GemvParams {
     const uint8_t* W;
     const float* x;      // [M, cols]
@@ -535,13 +652,16 @@ int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, f
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for Q8_0");
             return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, s);
         case FHIP_Q5_K: return n_ff ? launch_fmt<Q5K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_fmt<Q5K, false>(w, d_x, rows_x, d_y, out_rows, s);
-        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1:
+        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_IQ4_NL: case FHIP_IQ4_XS: case FHIP_MXFP4:
             // the reference fuses gate/up + SwiGLU for the K-quants only (crates/ferric-tensor/src/dtype.rs:949-959)
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for ggml type %u", w->type);
             if (w->type == FHIP_Q4_0) return launch_fmt<Q40, false>(w, d_x, rows_x, d_y, out_rows, s);
             if (w->type == FHIP_Q4_1) return launch_fmt<Q41, false>(w, d_x, rows_x, d_y, out_rows, s);
             if (w->type == FHIP_Q5_0) return launch_fmt<Q50, false>(w, d_x, rows_x, d_y, out_rows, s);
-            return launch_fmt<Q51, false>(w, d_x, rows_x, d_y, out_rows, s);
+            if (w->type == FHIP_Q5_1) return launch_fmt<Q51, false>(w, d_x, rows_x, d_y, out_rows, s);
+            if (w->type == FHIP_IQ4_NL) return launch_fmt<IQ4NL, false>(w, d_x, rows_x, d_y, out_rows, s);
+            if (w->type == FHIP_IQ4_XS) return launch_fmt<IQ4XS, false>(w, d_x, rows_x, d_y, out_rows, s);
+            return launch_fmt<MXF4, false>(w, d_x, rows_x, d_y, out_rows, s);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }
@@ -558,6 +678,9 @@ int launch_gemv_generic_sel(const fhip_weight* w, const float* d_x, float* d_y, 
         case FHIP_Q4_1: return swiglu ? launch_one<Q41, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q41, 1, false>(w, d_x, d_y, out_rows, s, &sel);
         case FHIP_Q5_0: return swiglu ? launch_one<Q50, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q50, 1, false>(w, d_x, d_y, out_rows, s, &sel);
         case FHIP_Q5_1: return swiglu ? launch_one<Q51, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<Q51, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_IQ4_NL: return swiglu ? launch_one<IQ4NL, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<IQ4NL, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_IQ4_XS: return swiglu ? launch_one<IQ4XS, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<IQ4XS, 1, false>(w, d_x, d_y, out_rows, s, &sel);
+        case FHIP_MXFP4: return swiglu ? launch_one<MXF4, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<MXF4, 1, false>(w, d_x, d_y, out_rows, s, &sel);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

@@ -20,6 +20,7 @@ from . import _lib
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13   # further formats: unpackers, mat-vec / small batch, "_id" variants
+IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39             # codebook / microscaling formats, same coverage
 
 
 def _vp(a):
@@ -183,6 +184,15 @@ class Tensor:
 
     def matmul_q5_1(self, w, stream=None):  # dtype.rs:1904
         return self._matmul_typed(w, Q5_1, stream)
+
+    def matmul_iq4_nl(self, w, stream=None):  # dtype.rs:3259
+        return self._matmul_typed(w, IQ4_NL, stream)
+
+    def matmul_iq4_xs(self, w, stream=None):  # dtype.rs:3185
+        return self._matmul_typed(w, IQ4_XS, stream)
+
+    def matmul_mxfp4(self, w, stream=None):  # dtype.rs:3396
+        return self._matmul_typed(w, MXFP4, stream)
 
     def try_matmul_swiglu(self, w, stream=None):
         """Fused gate/up + SwiGLU -- dtype.rs:949. None when the format has no fused kernel
@@ -445,6 +455,9 @@ Q4_0Weights = _typed(Q4_0, "Q4_0Weights")
 Q4_1Weights = _typed(Q4_1, "Q4_1Weights")
 Q5_0Weights = _typed(Q5_0, "Q5_0Weights")
 Q5_1Weights = _typed(Q5_1, "Q5_1Weights")
+Iq4NlWeights = _typed(IQ4_NL, "Iq4NlWeights")
+Iq4XsWeights = _typed(IQ4_XS, "Iq4XsWeights")
+Mxfp4Weights = _typed(MXFP4, "Mxfp4Weights")
 
 
 def type_size(ty, n):

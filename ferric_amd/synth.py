@@ -6,8 +6,9 @@ import numpy as np
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13
+IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39
 BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24),
-         Q5_K: (256, 176)}
+         Q5_K: (256, 176), IQ4_NL: (32, 18), IQ4_XS: (256, 136), MXFP4: (32, 17)}
 
 
 def q4k_pack_scales(sc, m):
@@ -49,7 +50,16 @@ def synth_weights(ty, rows, cols, seed):
         b[:, 2:4] = (np.abs(rng.standard_normal(nb)) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)
         b[:, 4:16] = q4k_pack_scales(rng.integers(0, 64, (nb, 8), dtype=np.uint8), rng.integers(0, 64, (nb, 8), dtype=np.uint8))
         b[:, 16:] = rng.integers(0, 256, (nb, 160), dtype=np.uint8)
+    elif ty in (IQ4_NL, IQ4_XS):
+        # f16 super-scale; the 6-bit sub-scales of IQ4_XS (offset by 32 when used) and all codebook indices uniform
+        b[:, 2:] = rng.integers(0, 256, (nb, bytes_ - 2), dtype=np.uint8)
+        b[:, 0:2] = (np.abs(rng.standard_normal(nb)) * (0.0005 if ty == IQ4_XS else 0.002)).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    elif ty == MXFP4:
+        # shared exponents around 2^-9 .. 2^-6 (the range a released checkpoint's blocks use), codes uniform
+        b[:, 0] = rng.integers(0x75, 0x7A, nb, dtype=np.uint8)
+        b[:, 1:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
     else:
+        assert ty == Q6_K, f"no generator for ggml type {ty}"
         b[:, 0:192] = rng.integers(0, 256, (nb, 192), dtype=np.uint8)
         b[:, 192:208] = rng.integers(-32, 32, (nb, 16), dtype=np.int8).view(np.uint8)
         b[:, 208:210] = (np.abs(rng.standard_normal(nb)) * 0.01).astype(np.float16).view(np.uint8).reshape(nb, 2)

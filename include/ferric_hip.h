@@ -34,13 +34,16 @@ extern "C" {
 #define FHIP_Q8_0 8u
 #define FHIP_Q4_K 12u
 #define FHIP_Q6_K 14u
-/* further block formats of the same reader (crates/ferric-gguf/src/lib.rs:618-716): unpackers, mat-vec / small batch and
+/* further block formats of the same reader (crates/ferric-gguf/src/lib.rs:618-716, 748-791, 843-908): unpackers, mat-vec / small batch and
  * the "_id" variants; the matrix-core entry points take the three formats above only */
 #define FHIP_Q4_0 2u
 #define FHIP_Q4_1 3u
 #define FHIP_Q5_0 6u
 #define FHIP_Q5_1 7u
 #define FHIP_Q5_K 13u
+#define FHIP_IQ4_NL 20u
+#define FHIP_IQ4_XS 23u
+#define FHIP_MXFP4 39u
 
 #define FHIP_OK 0
 #define FHIP_ERR_UNSUPPORTED_TYPE (-1) /* reference: Err("unsupported ggml type N") / Err("QMatrix: no native matmul ...") */
@@ -256,7 +259,7 @@ int fhip_gguf_meta_str(const fhip_gguf* g, const char* key, size_t j, const char
 
 /* QShard::build from a GGUF tensor (crates/ferric-tensor/src/dtype.rs:839-857 over GgufSource::raw): uploads the
  * tensor's bytes straight from the mapping. dims are [in, out] or, for an expert slab, [in, rows per expert,
- * n_expert] (rows = product of the trailing dims). Types 2 / 3 / 6 / 7 / 8 / 12 / 13 / 14 only. */
+ * n_expert] (rows = product of the trailing dims). Types 2 / 3 / 6 / 7 / 8 / 12 / 13 / 14 / 20 / 23 / 39 only. */
 int fhip_weight_from_gguf(const fhip_gguf* g, const char* name, fhip_weight** out);
 
 /* crates/ferric-tensor/src/cpu_simd.rs:79 matvec_q8_0(x, w, rows, cols) with HOST buffers on both

@@ -1,5 +1,5 @@
 /*
- * CPU oracle for the quantized-GGUF matmul path (Q8_0 / Q4_K / Q6_K).
+ * CPU oracle for the quantized-GGUF matmul path (Q8_0 / Q4_K / Q6_K, and the further block formats of the same reader).
  *
  * THIS FILE IS TEST INFRASTRUCTURE. It is a plain-C restatement of the reference's own CPU
  * algorithms, used only as the checker in tests, the smoke check and the CPU-baseline leg of the
@@ -22,7 +22,14 @@
  *                         (the reference holds no known-answer vector for Q6_K)
  *   row_q8_0/matvec       reference tests cpu_simd.rs:162-200 restated (ground truth built beside the
  *                         bytes, partition invariance, span composition)
- *   parity with ggml itself for these three formats is not pinned anywhere in the reference tree.
+ *   deq_q4_0/q4_1/q5_0/q5_1/q5_k, deq_iq4_nl/iq4_xs
+ *                         second formulation from the reference's GPU kernel bodies, numpy twin, closed-form relations
+ *                         between formats and single-field perturbations (tests/test_oracle_formats.py); the IQ4
+ *                         codebook constant is restated from crates/ferric-gguf/src/lib.rs:751
+ *   deq_mxfp4             ggml-captured known answers held by the reference's tests (lib.rs:1099-1222: 10 scale bytes
+ *                         x 16 codes, 8 blocks of a released checkpoint), all 256 x 16 (scale, code) pairs vs ldexp
+ *   parity with ggml itself is pinned for MXFP4 only (through those captured answers); for the other formats it is
+ *   not pinned anywhere in the reference tree.
  */
 #include <math.h>
 #include <pthread.h>
@@ -38,6 +45,9 @@
 #define GGML_Q4_K 12u
 #define GGML_Q5_K 13u
 #define GGML_Q6_K 14u
+#define GGML_IQ4_NL 20u
+#define GGML_IQ4_XS 23u
+#define GGML_MXFP4 39u
 
 /* ---------------------------------------------------------------- f16 <-> f32 */
 
@@ -110,6 +120,9 @@ size_t fo_type_size(uint32_t ty, size_t n) {
         case GGML_Q5_0: return n / 32 * 22;
         case GGML_Q5_1: return n / 32 * 24;
         case GGML_Q5_K: return n / 256 * 176;
+        case GGML_IQ4_NL: return n / 32 * 18;
+        case GGML_IQ4_XS: return n / 256 * 136;
+        case GGML_MXFP4: return n / 32 * 17;
         default: return 0;
     }
 }
@@ -125,6 +138,9 @@ int fo_block_bytes(uint32_t ty, size_t* vals, size_t* bytes) {
         case GGML_Q5_0: *vals = 32; *bytes = 22; return 1;
         case GGML_Q5_1: *vals = 32; *bytes = 24; return 1;
         case GGML_Q5_K: *vals = 256; *bytes = 176; return 1;
+        case GGML_IQ4_NL: *vals = 32; *bytes = 18; return 1;
+        case GGML_IQ4_XS: *vals = 256; *bytes = 136; return 1;
+        case GGML_MXFP4: *vals = 32; *bytes = 17; return 1;
         default: return 0;
     }
 }
@@ -316,6 +332,74 @@ size_t fo_deq_q5_k(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
     return n;
 }
 
+/* crates/ferric-gguf/src/lib.rs:751: the 16 signed levels of the IQ4 non-linear codebook (llama.cpp kvalues_iq4nl). */
+static const int FO_KVALUES_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+/* crates/ferric-gguf/src/lib.rs:755-767: 18-byte block [f16 d][qs[16]], value = d * kvalues[index]. */
+size_t fo_deq_iq4_nl(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 32, have = raw_len / 18;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 18;
+        float d = fo_f16_to_f32(rd_u16(blk));
+        for (int j = 0; j < 16; j++) {
+            out[bi * 32 + j] = d * (float)FO_KVALUES_IQ4NL[blk[2 + j] & 0x0F];
+            out[bi * 32 + j + 16] = d * (float)FO_KVALUES_IQ4NL[blk[2 + j] >> 4];
+        }
+    }
+    return n;
+}
+
+/* crates/ferric-gguf/src/lib.rs:772-791: 136-byte super-block [f16 d][u16 scales_h][scales_l[4]][qs[128]]; sub-block ib
+ * has the 6-bit scale ls = nibble ib of scales_l | bits 2ib, 2ib+1 of scales_h << 4; dl = d * (ls - 32). */
+size_t fo_deq_iq4_xs(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 256, have = raw_len / 136;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 136;
+        float d = fo_f16_to_f32(rd_u16(blk));
+        uint32_t scales_h = rd_u16(blk + 2);
+        const uint8_t* scales_l = blk + 4; const uint8_t* qs = blk + 8;
+        for (int ib = 0; ib < 8; ib++) {
+            int ls = (int)(((uint32_t)(scales_l[ib / 2] >> (4 * (ib % 2))) & 0x0Fu) | (((scales_h >> (2 * ib)) & 3u) << 4));
+            float dl = d * (float)(ls - 32);
+            const uint8_t* q = qs + ib * 16;
+            for (int j = 0; j < 16; j++) {
+                out[bi * 256 + ib * 32 + j] = dl * (float)FO_KVALUES_IQ4NL[q[j] & 0x0F];
+                out[bi * 256 + ib * 32 + j + 16] = dl * (float)FO_KVALUES_IQ4NL[q[j] >> 4];
+            }
+        }
+    }
+    return n;
+}
+
+/* crates/ferric-gguf/src/lib.rs:857-860: the E2M1 value table, doubled ({0, .5, 1, 1.5, 2, 3, 4, 6} * 2); code 8 is +0.0. */
+static const float FO_KVALUES_MXFP4_2X[16] = {0.0f, 1.0f, 2.0f, 3.0f, 4.0f, 6.0f, 8.0f, 12.0f,
+                                              0.0f, -1.0f, -2.0f, -3.0f, -4.0f, -6.0f, -8.0f, -12.0f};
+/* crates/ferric-gguf/src/lib.rs:880-886: 2^(e - 128) from the E8M0 byte; e = 0 and e = 1 are subnormal bit patterns. */
+float fo_e8m0_half(uint8_t e) {
+    uint32_t bits = e == 0 ? (1u << 21) : e == 1 ? (1u << 22) : ((uint32_t)e - 1u) << 23;
+    float f; memcpy(&f, &bits, 4); return f;
+}
+/* crates/ferric-gguf/src/lib.rs:896-908: 17-byte block [u8 e][qs[16]], value = table[code] * 2^(e - 128); element i is the
+ * low nibble of qs[i], element i + 16 the high nibble. */
+size_t fo_deq_mxfp4(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    size_t nb = n / 32, have = raw_len / 17;
+    if (have < nb) nb = have;
+    for (size_t bi = 0; bi < nb; bi++) {
+        const uint8_t* blk = raw + bi * 17;
+        float d = fo_e8m0_half(blk[0]);
+        for (int i = 0; i < 16; i++) {
+            out[bi * 32 + i] = FO_KVALUES_MXFP4_2X[blk[1 + i] & 0x0F] * d;
+            out[bi * 32 + i + 16] = FO_KVALUES_MXFP4_2X[blk[1 + i] >> 4] * d;
+        }
+    }
+    return n;
+}
+
 /* crates/ferric-gguf/src/lib.rs:497-520 (deq_raw), in-scope types. Returns the number of f32 the
  * reference's Vec would hold, or (size_t)-1 for "unsupported ggml type". */
 size_t fo_deq_raw(const uint8_t* raw, size_t raw_len, size_t n, uint32_t ty, float* out) {
@@ -328,6 +412,9 @@ size_t fo_deq_raw(const uint8_t* raw, size_t raw_len, size_t n, uint32_t ty, flo
         case GGML_Q5_0: return fo_deq_q5_0(raw, raw_len, n, out);
         case GGML_Q5_1: return fo_deq_q5_1(raw, raw_len, n, out);
         case GGML_Q5_K: return fo_deq_q5_k(raw, raw_len, n, out);
+        case GGML_IQ4_NL: return fo_deq_iq4_nl(raw, raw_len, n, out);
+        case GGML_IQ4_XS: return fo_deq_iq4_xs(raw, raw_len, n, out);
+        case GGML_MXFP4: return fo_deq_mxfp4(raw, raw_len, n, out);
         default: return (size_t)-1;
     }
 }
@@ -409,6 +496,35 @@ float fo_q5k_elem(const uint8_t* blk, int v) {
     return ds * (float)(nib + bit * 16u) - mm;
 }
 
+/* crates/ferric-tensor/src/dtype.rs:3205-3214 (IQ4_NL body): byte j of the block's four code words, codebook value of
+ * its low nibble for element j and of its high nibble for element j + 16. */
+float fo_iq4_nl_elem(const uint8_t* blk, int v) {
+    int j = v & 15;
+    uint32_t b = (rd_u32(blk + 2 + 4 * (j >> 2)) >> (8 * (j & 3))) & 0xFFu;
+    return fo_f16_to_f32(rd_u16(blk)) * (float)FO_KVALUES_IQ4NL[v >= 16 ? (b >> 4) : (b & 0x0Fu)];
+}
+/* crates/ferric-tensor/src/dtype.rs:3119-3145 (IQ4_XS body): scales_l read as one u32, the sub-block's four code words. */
+float fo_iq4_xs_elem(const uint8_t* blk, int v) {
+    uint32_t scales_h = rd_u16(blk + 2), scales_l = rd_u32(blk + 4);
+    uint32_t ib = (uint32_t)v >> 5; int j = v & 15;
+    uint32_t sl = (scales_l >> (8 * (ib >> 1))) & 0xFFu;
+    uint32_t lo = (sl >> (4 * (ib & 1))) & 0x0Fu, hi = (scales_h >> (2 * ib)) & 3u;
+    float dl = fo_f16_to_f32(rd_u16(blk)) * (float)((int)(lo | (hi << 4)) - 32);
+    uint32_t b = (rd_u32(blk + 8 + 4 * (ib * 4 + (uint32_t)(j >> 2))) >> (8 * (j & 3))) & 0xFFu;
+    return dl * (float)FO_KVALUES_IQ4NL[(v & 16) ? (b >> 4) : (b & 0x0Fu)];
+}
+/* crates/ferric-tensor/src/dtype.rs:3318-3344 (MXFP4 helpers + body): the integral table and the scale split in two
+ * factors 2^(a - 64) * 2^(b - 64), a = e >> 1, b = e - a, applied one after the other. */
+float fo_mxfp4_elem(const uint8_t* blk, int v) {
+    static const int KM[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+    uint32_t e = blk[0], a = e >> 1, b2 = e - a;
+    uint32_t xa = (a + 63u) << 23, xb = (b2 + 63u) << 23;
+    float dx, dy; memcpy(&dx, &xa, 4); memcpy(&dy, &xb, 4);
+    int j = v & 15;
+    uint32_t b = (rd_u32(blk + 1 + 4 * (j >> 2)) >> (8 * (j & 3))) & 0xFFu;
+    return ((float)KM[v >= 16 ? (b >> 4) : (b & 0x0Fu)] * dx) * dy;
+}
+
 void fo_deq_elemwise(const uint8_t* raw, size_t n, uint32_t ty, float* out) {
     size_t vals, bytes;
     if (!fo_block_bytes(ty, &vals, &bytes)) return;
@@ -423,6 +539,9 @@ void fo_deq_elemwise(const uint8_t* raw, size_t n, uint32_t ty, float* out) {
             case GGML_Q5_0: out[i] = fo_q5_0_elem(blk, v); break;
             case GGML_Q5_1: out[i] = fo_q5_1_elem(blk, v); break;
             case GGML_Q5_K: out[i] = fo_q5k_elem(blk, v); break;
+            case GGML_IQ4_NL: out[i] = fo_iq4_nl_elem(blk, v); break;
+            case GGML_IQ4_XS: out[i] = fo_iq4_xs_elem(blk, v); break;
+            case GGML_MXFP4: out[i] = fo_mxfp4_elem(blk, v); break;
             default: break;
         }
     }

@@ -15,8 +15,9 @@ import numpy as np
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13
+IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39
 BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24),
-         Q5_K: (256, 176)}
+         Q5_K: (256, 176), IQ4_NL: (32, 18), IQ4_XS: (256, 136), MXFP4: (32, 17)}
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libferric_oracle.so")
@@ -445,6 +446,48 @@ def np_deq_q5_k(raw, n):
     return out
 
 
+_KV_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)  # lib.rs:751
+
+
+def np_deq_iq4_nl(raw, n):
+    out = np.zeros(n, np.float32)
+    nb = min(n // 32, len(raw) // 18)
+    b = np.asarray(raw[: nb * 18], dtype=np.uint8).reshape(nb, 18)
+    d = _np_f16(b[:, 0:2]).reshape(nb, 1)
+    idx = np.concatenate([b[:, 2:] & 0x0F, b[:, 2:] >> 4], axis=1)
+    out[: nb * 32] = (d * _KV_IQ4NL[idx]).reshape(-1)
+    return out
+
+
+def np_deq_iq4_xs(raw, n):
+    out = np.zeros(n, np.float32)
+    nb = min(n // 256, len(raw) // 136)
+    b = np.asarray(raw[: nb * 136], dtype=np.uint8).reshape(nb, 136)
+    d = _np_f16(b[:, 0:2]).reshape(nb, 1)
+    sh = b[:, 2].astype(np.int32) | (b[:, 3].astype(np.int32) << 8)
+    ib = np.arange(8)
+    lo = (b[:, 4:8][:, ib // 2].astype(np.int32) >> (4 * (ib % 2))) & 0x0F
+    hi = (sh.reshape(nb, 1) >> (2 * ib)) & 3
+    dl = (d * ((lo | (hi << 4)) - 32).astype(np.float32)).reshape(nb, 8, 1)
+    q = b[:, 8:].reshape(nb, 8, 16)
+    idx = np.concatenate([q & 0x0F, q >> 4], axis=2)
+    out[: nb * 256] = (dl * _KV_IQ4NL[idx]).reshape(-1)
+    return out
+
+
+def np_deq_mxfp4(raw, n):
+    """lib.rs:896-908 through numpy.ldexp: table[code] / 2 * 2^(e - 127) formed in f64 and rounded once to f32, which is
+    what a single correctly-rounded f32 multiply by 2^(e - 128) gives (subnormals and overflow included)."""
+    out = np.zeros(n, np.float32)
+    nb = min(n // 32, len(raw) // 17)
+    b = np.asarray(raw[: nb * 17], dtype=np.uint8).reshape(nb, 17)
+    mag = np.array([0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12], np.float64)
+    idx = np.concatenate([b[:, 1:] & 0x0F, b[:, 1:] >> 4], axis=1)
+    with np.errstate(over="ignore"):
+        out[: nb * 32] = np.ldexp(mag[idx], b[:, 0:1].astype(np.int64) - 128).astype(np.float32).reshape(-1)
+    return out
+
+
 def np_deq_raw(raw, n, ty):
     return {Q8_0: np_deq_q8_0, Q4_K: np_deq_q4_k, Q6_K: np_deq_q6_k, Q4_0: np_deq_q4_0, Q4_1: np_deq_q4_1, Q5_0: np_deq_q5_0,
-            Q5_1: np_deq_q5_1, Q5_K: np_deq_q5_k}[ty](np.asarray(raw, dtype=np.uint8), n)
+            Q5_1: np_deq_q5_1, Q5_K: np_deq_q5_k, IQ4_NL: np_deq_iq4_nl, IQ4_XS: np_deq_iq4_xs, MXFP4: np_deq_mxfp4}[ty](np.asarray(raw, dtype=np.uint8), n)

@@ -1,4 +1,4 @@
-"""The further block formats (Q4_0, Q4_1, Q5_0, Q5_1, Q5_K) through the C ABI: unpackers bit-exact against the
+"""The further block formats (Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, IQ4_NL, IQ4_XS, MXFP4) through the C ABI: unpackers bit-exact against the
 oracle, mat-vec / small batch against f64 on oracle-dequantized weights (north-star bound per dot and 1e-5 of the
 largest output, the reference's bar for its scalar kernels), fused SwiGLU for Q5_K, and the "_id" variants."""
 import numpy as np
@@ -8,8 +8,10 @@ from conftest import bits
 
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q6_K, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 8, 12, 14, 2, 3, 6, 7, 13
-NEW = [Q4_0, Q4_1, Q5_0, Q5_1, Q5_K]
-GEOM = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q5_K: (256, 176)}
+IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39
+NEW = [Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, IQ4_NL, IQ4_XS, MXFP4]
+GEOM = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q5_K: (256, 176), IQ4_NL: (32, 18), IQ4_XS: (256, 136),
+        MXFP4: (32, 17)}
 
 
 @pytest.mark.parametrize("ty", NEW)
@@ -55,7 +57,8 @@ def test_matmul_small_batch(F, O, ty):
         # a row of a batch is bit-identical to the same row alone
         y1 = F.Tensor.from_vec(x[b - 1], (1, cols)).matmul_q(w).to_vec()
         assert np.array_equal(bits(y1), bits(y[b - 1]))
-    name = {Q4_0: "matmul_q4_0", Q4_1: "matmul_q4_1", Q5_0: "matmul_q5_0", Q5_1: "matmul_q5_1", Q5_K: "matmul_q5_k"}[ty]
+    name = {Q4_0: "matmul_q4_0", Q4_1: "matmul_q4_1", Q5_0: "matmul_q5_0", Q5_1: "matmul_q5_1", Q5_K: "matmul_q5_k",
+            IQ4_NL: "matmul_iq4_nl", IQ4_XS: "matmul_iq4_xs", MXFP4: "matmul_mxfp4"}[ty]
     assert np.array_equal(bits(getattr(F.Tensor.from_vec(x[0], (1, cols)), name)(w).to_vec()), bits(y[0]))
     with pytest.raises(AssertionError, match="inner dim mismatch"):
         F.Tensor.from_vec(np.zeros(cols + vals, np.float32), (1, cols + vals)).matmul_q(w)
@@ -90,7 +93,7 @@ def test_id_variants_on_the_other_formats(F, O):
         sel[ti, k:] = rng.choice(n_expert, size=k, replace=False)
     st = F.Tensor.from_vec(sel.reshape(-1), (t, 2 * k))
     x = rng.standard_normal((t, k, cols)).astype(np.float32)
-    for ty in (Q5_0, Q5_K, Q4_1):
+    for ty in (Q5_0, Q5_K, Q4_1, IQ4_NL, IQ4_XS, MXFP4):
         raw = synth_weights(ty, n_expert * out_pe, cols, 13 + ty)
         w = F.QMatrix.from_bytes(raw, ty, n_expert * out_pe, cols)
         got = F.Tensor.from_vec(x.reshape(-1), (t, k, cols)).matmul_q_id_wsum(w, st, out_pe).to_vec().reshape(t, out_pe)
@@ -132,3 +135,84 @@ def test_these_formats_load_from_a_gguf_file(F, O, tmp_path):
         w = g.qmatrix(name)
         assert (w.rows(), w.cols(), w.ggml_type, w.nbytes()) == (r, c, ty, raw[name].size)
         assert np.array_equal(bits(w.dequant().to_vec()), bits(O.deq_raw(raw[name], r * c, ty)))
+
+
+def _mxfp4_golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "mxfp4_ggml.json")) as f:
+        return json.load(f)
+
+
+def test_mxfp4_unpacker_against_the_ggml_captured_answers(F):
+    # the reference's own known answers (crates/ferric-gguf/src/lib.rs:1099-1222), which include subnormal scales (e = 0, 1)
+    # and both saturating ends (e = 254, 255): the device must neither flush the former nor overflow early on the latter
+    g = _mxfp4_golden()
+    blocks, want = [], []
+    for ei, e in enumerate(g["e"]):
+        for code in range(16):
+            lo = np.zeros(17, np.uint8); lo[0] = e; lo[1] = code
+            hi = np.zeros(17, np.uint8); hi[0] = e; hi[1] = code << 4
+            blocks += [lo, hi]
+            w = g["grid_bits"][ei * 16 + code]
+            a = np.zeros(32, np.uint32); a[0] = w
+            b = np.zeros(32, np.uint32); b[16] = w
+            want += [a, b]
+    raw = np.concatenate(blocks)
+    assert np.array_equal(bits(F.deq_raw(raw, 32 * len(blocks), MXFP4)), np.concatenate(want))
+    real = np.array(g["real_raw"], np.uint8)
+    assert np.array_equal(bits(F.deq_raw(real, 256, MXFP4)), np.array(g["real_bits"], np.uint32))
+    w = F.Mxfp4Weights.from_bytes(real, 1, 256)
+    assert np.array_equal(bits(w.dequant().to_vec()), np.array(g["real_bits"], np.uint32))
+
+
+def test_mxfp4_matvec_forms_the_weight_before_it_meets_the_activation(F, O):
+    # crates/ferric-tensor/src/dtype.rs:3331-3335: a block whose weights saturate contributes inf (not a finite x*d*k), a
+    # subnormal scale is not flushed, and every (scale, code) pair gives x * w with the oracle's w
+    blk = np.zeros((256, 17), np.uint8)
+    blk[:, 0] = np.arange(256)
+    blk[:, 1:9] = np.arange(16, dtype=np.uint8).reshape(8, 2)[:, 0] | (np.arange(16, dtype=np.uint8).reshape(8, 2)[:, 1] << 4)
+    w = F.QMatrix.from_bytes(blk.reshape(-1), MXFP4, 256, 32)            # row e: one block under scale byte e
+    wd = O.deq_raw(blk.reshape(-1), 256 * 32, MXFP4).reshape(256, 32)
+    for j in (0, 1, 16, 7, 23):                                           # x = 0.5 * unit vector j picks out 0.5 * w[e, j]
+        x = np.zeros(32, np.float32); x[j] = 0.5
+        y = F.Tensor.from_vec(x, (1, 32)).matmul_q(w).to_vec()
+        with np.errstate(over="ignore", invalid="ignore"):
+            want = (x[None, :] * wd).sum(axis=1, dtype=np.float32)       # one non-zero product per row; 0 * inf = NaN stays NaN
+        assert np.array_equal(y, want, equal_nan=True), j
+        assert np.isnan(want[255]) and np.isfinite(want[:250]).all()
+    assert np.isinf(wd[255, 1]) and wd[0, 16] == np.float32(2.0 ** -128) and wd[255, 16] == np.float32(2.0 ** 127)
+    x = np.zeros(32, np.float32); x[16] = 0.5
+    one = F.QMatrix.from_bytes(np.concatenate([blk[255, :1], np.array([0x10], np.uint8), np.zeros(15, np.uint8)]), MXFP4, 1, 32)
+    assert F.Tensor.from_vec(x, (1, 32)).matmul_q(one).to_vec()[0] == np.float32(2.0 ** 126)    # finite at the top scale
+
+
+def test_iq4_xs_packed_kernel_matches_the_dense_reference(F, O):
+    # crates/ferric-tensor/examples/iq4_xs.rs restated: its block generator, its activation ramp, its shapes and its bar
+    # (max |got - want| / max |want| < 1e-5 against the dense product of the dequantized weight)
+    def half_bits(x):
+        b = int(np.array([x], np.float32).view(np.uint32)[0])
+        exp = ((b >> 23) & 0xFF) - 127 + 15
+        return ((b >> 16) & 0x8000) if exp <= 0 else (((b >> 16) & 0x8000) | (exp << 10) | ((b >> 13) & 0x3FF))
+
+    def blocks(nblk, seed):
+        s = (seed * 2654435761 + 1) & 0xFFFFFFFF
+        out = bytearray()
+
+        def rnd():
+            nonlocal s
+            s = (s * 1664525 + 1013904223) & 0xFFFFFFFF
+            return (s >> 16) & 0xFFFF
+        for _ in range(nblk):
+            out += int(half_bits(np.float32(0.005) + np.float32(rnd() % 40) * np.float32(0.0007))).to_bytes(2, "little")
+            out += rnd().to_bytes(2, "little")
+            out += bytes(rnd() & 0xFF for _ in range(4))
+            out += bytes(rnd() & 0xFF for _ in range(128))
+        return np.frombuffer(bytes(out), np.uint8)
+    for rows, cols in [(8, 256), (32, 512), (7, 1024), (64, 256)]:
+        raw = blocks(rows * (cols // 256), rows * 31 + cols)
+        deq = O.deq_raw(raw, rows * cols, IQ4_XS).reshape(rows, cols)
+        xv = ((np.arange(cols) * 37 % 101).astype(np.float32) - np.float32(50.0)) / np.float32(50.0)
+        want = deq.astype(np.float64) @ xv.astype(np.float64)
+        got = F.Tensor.from_vec(xv, (1, cols)).matmul_iq4_xs(F.Iq4XsWeights.from_bytes(raw, rows, cols)).to_vec()
+        assert np.abs(got - want).max() / max(1e-6, np.abs(want).max()) < 1e-5, (rows, cols)

@@ -1,5 +1,6 @@
-"""Pins the oracle's dequantizers for the five further block formats (Q4_0, Q4_1, Q5_0, Q5_1, Q5_K). The reference
-tree holds no known-answer vectors for them, so each sequential restatement (crates/ferric-gguf/src/lib.rs:618-716)
+"""Pins the oracle's dequantizers for the further block formats (Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, IQ4_NL, IQ4_XS, MXFP4).
+MXFP4 has known-answer data captured from ggml in the reference's own tests (tests/golden/mxfp4_ggml.json); for the
+others the reference tree holds no known-answer vectors, so each sequential restatement (crates/ferric-gguf/src/lib.rs:618-716)
 must agree bit for bit with (i) the element formula of the reference's own GPU kernels, restated separately
 (crates/ferric-tensor/src/dtype.rs:3548-3555, 3613-3620, 3778-3792, 3858-3874, 1108-1121), (ii) a numpy twin written
 from the block layout, and satisfy (iii) closed-form relations to the formats pinned in test_oracle.py and (iv)
@@ -10,8 +11,11 @@ import pytest
 from conftest import bits
 
 Q8_0, Q4_K, Q6_K, Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 8, 12, 14, 2, 3, 6, 7, 13
-NEW = [Q4_0, Q4_1, Q5_0, Q5_1, Q5_K]
-GEOM = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q5_K: (256, 176)}
+IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39
+NEW = [Q4_0, Q4_1, Q5_0, Q5_1, Q5_K, IQ4_NL, IQ4_XS, MXFP4]
+GEOM = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q5_K: (256, 176), IQ4_NL: (32, 18), IQ4_XS: (256, 136),
+        MXFP4: (32, 17)}
+KV = [-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113]
 
 
 def f16b(v):
@@ -108,3 +112,88 @@ def test_ragged_inputs_follow_the_reference(O, ty):
     # n not a multiple of the block: the trailing partial block is left zero
     part = O.deq_raw(raw, vals * 2 + 7, ty)
     assert part.size == vals * 2 + 7 and np.array_equal(part[: 2 * vals], full[: 2 * vals]) and not part[2 * vals:].any()
+
+
+# ---------------------------------------------------------------- MXFP4: ggml-captured known answers
+
+def _mxfp4_golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "mxfp4_ggml.json")) as f:
+        return json.load(f)
+
+
+def test_mxfp4_grid_is_bit_identical_to_ggml(O):
+    # crates/ferric-gguf/src/lib.rs:1173-1200: each code in the low nibble of qs[0] (element 0) and in the high nibble
+    # (element 16), under ten scale bytes that include both subnormal and both saturating ends
+    g = _mxfp4_golden()
+    for form in (O.deq_raw, O.deq_elemwise, O.np_deq_raw):
+        for ei, e in enumerate(g["e"]):
+            for code in range(16):
+                want = g["grid_bits"][ei * 16 + code]
+                blk = np.zeros(17, np.uint8); blk[0] = e; blk[1] = code
+                assert bits(form(blk, 32, MXFP4))[0] == want, (form.__name__, e, code)
+                blk[1] = code << 4
+                hi = bits(form(blk, 32, MXFP4))
+                assert hi[16] == want and hi[0] == 0, (form.__name__, e, code)
+
+
+def test_mxfp4_real_blocks_are_bit_identical_to_ggml(O):
+    # crates/ferric-gguf/src/lib.rs:1205-1222: 8 blocks of a released checkpoint, three distinct exponents, 17-byte stride
+    g = _mxfp4_golden()
+    raw = np.array(g["real_raw"], np.uint8)
+    want = np.array(g["real_bits"], np.uint32)
+    for form in (O.deq_raw, O.deq_elemwise, O.np_deq_raw):
+        assert np.array_equal(bits(form(raw, 256, MXFP4)), want), form.__name__
+    assert O.type_size(MXFP4, 802816) == 426496            # lib.rs:1224-1229, the measured on-disk length of an 896x896 tensor
+
+
+def test_mxfp4_every_scale_and_code_against_ldexp(O):
+    # all 256 x 16 (scale, code) pairs: table[code] / 2 * 2^(e - 127) through f64 ldexp, rounded once to f32
+    blk = np.zeros((256, 17), np.uint8)
+    blk[:, 0] = np.arange(256)
+    blk[:, 1:9] = np.arange(16, dtype=np.uint8).reshape(8, 2)[:, 0] | (np.arange(16, dtype=np.uint8).reshape(8, 2)[:, 1] << 4)
+    mag = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, 0, -.5, -1, -1.5, -2, -3, -4, -6])
+    got = O.deq_raw(blk.reshape(-1), 256 * 32, MXFP4).reshape(256, 32)
+    codes = np.concatenate([blk[:, 1:] & 15, blk[:, 1:] >> 4], axis=1)
+    with np.errstate(over="ignore"):
+        want = np.ldexp(mag[codes], np.arange(256).reshape(256, 1) - 127).astype(np.float32)
+    assert np.array_equal(bits(got), bits(want))
+    # e = 255: code 1 (element 16) is the finite 2^127, code 2 (element 1) saturates, code 0 stays +0.0
+    assert got[255, 16] == np.float32(2.0 ** 127) and np.isinf(got[255, 1]) and bits(got[255])[0] == 0
+
+
+# ---------------------------------------------------------------- IQ4_NL / IQ4_XS: closed forms
+
+def test_iq4_nl_codebook_and_nibble_order(O):
+    blk = np.zeros(18, np.uint8); blk[0:2] = f16b(1.0)
+    blk[2:] = np.arange(16) | ((15 - np.arange(16)) << 4)
+    want = np.array(KV + KV[::-1], np.float32)             # element j: index j; element 16 + j: index 15 - j
+    assert np.array_equal(O.deq_raw(blk, 32, IQ4_NL), want)
+    blk[0:2] = f16b(-0.375)
+    assert np.array_equal(O.deq_raw(blk, 32, IQ4_NL), want * np.float32(-0.375))
+    assert KV == sorted(KV) and KV[0] == -127 and KV[8] == 1 and sum(KV) == -94   # 16 increasing int8 levels, denser near 0
+
+
+def test_iq4_xs_sub_scales_sit_where_the_layout_says(O):
+    rng = np.random.default_rng(4)
+    qs = rng.integers(0, 256, 128, dtype=np.uint8)
+    nl = np.zeros((8, 18), np.uint8); nl[:, 0:2] = f16b(0.5); nl[:, 2:] = qs.reshape(8, 16)
+    as_nl = O.deq_raw(nl.reshape(-1), 256, IQ4_NL)         # the same indices under a plain scale of 0.5
+
+    def xs(ls):                                             # ls[ib] in 0..63 -> one super-block with d = 0.5
+        b = np.zeros(136, np.uint8); b[0:2] = f16b(0.5)
+        sh = 0
+        for ib, v in enumerate(ls):
+            b[4 + ib // 2] |= (v & 15) << (4 * (ib % 2))
+            sh |= (v >> 4) << (2 * ib)
+        b[2], b[3] = sh & 255, sh >> 8
+        b[8:] = qs
+        return b
+    assert np.array_equal(O.deq_raw(xs([33] * 8), 256, IQ4_XS), as_nl)             # ls - 32 = 1: exactly IQ4_NL
+    assert not O.deq_raw(xs([32] * 8), 256, IQ4_XS).any()                           # ls - 32 = 0
+    for ib in range(8):
+        for v in (0, 15, 16, 48, 63):                       # low nibble only, each high bit alone, everything
+            ls = [33] * 8; ls[ib] = v
+            want = as_nl.copy(); want[32 * ib: 32 * ib + 32] *= np.float32(v - 32)
+            assert np.array_equal(O.deq_raw(xs(ls), 256, IQ4_XS), want), (ib, v)
