@@ -236,6 +236,55 @@ def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
                       "ops still execute in stream order"}
 
 
+def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096), layers=64, steps=6):
+    """configs[4] as a real decode step: the same 64-layer stack (fused QKV 5120->7168 with 40 query / 8 KV heads of 128, O,
+    fused gate|up 5120->34816 + SwiGLU, all Q4_K; down 17408->5120 Q6_K; output norm + lm_head 151936 Q6_K), but with every op fed
+    by the one before it: RMSNorm, q/k norm + rope + KV append, attention over `context` cached tokens (f32 cache), residual
+    adds. One graph per step, replayed `steps` times at consecutive positions."""
+    from ferric_amd import decode as X
+    from ferric_amd.synth import synth_weights
+    d, nh, nkv, hd, n_ff, vocab = 5120, 40, 8, 128, 17408, 151936
+    shapes = [("qkv", Q4_K, (nh + 2 * nkv) * hd, d), ("o", Q4_K, d, nh * hd), ("gate_up", Q4_K, 2 * n_ff, d), ("down", Q6_K, d, n_ff)]
+    host = {n: synth_weights(ty, r, c, 40 + i) for i, (n, ty, r, c) in enumerate(shapes)}
+    stacks = {n: replicate(F, lib, check, host[n], layers) for n, _, _, _ in shapes}
+    head_host = synth_weights(Q6_K, vocab, d, 50)
+    head = F.QMatrix.from_bytes(head_host, Q6_K, vocab, d)
+    weight_bytes_total = sum(h.size for h in host.values()) * layers + head_host.size
+    del head_host
+    rng = np.random.default_rng(8)
+    T = lambda a: F.Tensor.from_vec(a, a.shape)
+    # block norms small enough that a normalised vector projects to O(1) through the synthetic weights (rows of norm ~ 2 sqrt(cols))
+    small, unit = T(((rng.random(d) + 0.5) * 0.01).astype(np.float32)), T((rng.random(hd) + 0.5).astype(np.float32))
+    W = {}
+    for n, ty, r, c in shapes:
+        nb = host[n].size
+        W[n] = [F.QMatrix.wrap_device(stacks[n], nb, ty, r, c, offset=l * nb) for l in range(layers)]
+    lay = [X.Qwen3Layer(small, W["qkv"][l], W["o"][l], small, W["gate_up"][l], W["down"][l], unit, unit) for l in range(layers)]
+    cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6)
+    out = {}
+    for ctx in contexts:
+        dec = X.Qwen3Decoder(cfg, lay, max_len=ctx + steps + 2, stream=stream, output_norm=small, lm_head=head)
+        kv_fill = (rng.standard_normal((ctx, nkv * hd)) * 0.5).astype(np.float32)
+        for c in dec.caches:                      # `ctx` earlier tokens' keys and values (synthetic)
+            check(lib.fhip_memcpy_h2d(c.k.buf.ptr, kv_fill.ctypes.data_as(C.c_void_p), kv_fill.nbytes, None))
+            check(lib.fhip_memcpy_h2d(c.v.buf.ptr, kv_fill.ctypes.data_as(C.c_void_p), kv_fill.nbytes, None))
+        check(lib.fhip_stream_sync(None))
+        dec.set_pos(ctx)
+        dec.set_input((rng.standard_normal(d) * 0.5).astype(np.float32))
+        dec.capture()
+        dec.step_graph()                          # warm-up step (also: instantiation costs)
+        ms = timer.time_ms(lambda: [dec.step_graph() for _ in range(steps)]) / steps
+        logits = dec.logits.to_vec(stream)
+        kv_bytes = 2 * (ctx + steps // 2) * nkv * hd * 4 * layers
+        out[str(ctx)] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * 9 + 3,
+                         "kv_bytes_read": kv_bytes, "GBps_weights_plus_kv": (weight_bytes_total + kv_bytes) / (ms * 1e-3) / 1e9,
+                         "logits_finite": bool(np.isfinite(logits).all())}
+        del dec
+    out["weight_bytes"] = weight_bytes_total
+    out["model"] = "64 layers, d 5120, 40 query / 8 KV heads x 128, n_ff 17408, vocab 151936; Q4_K projections, Q6_K down and lm_head; f32 KV cache"
+    return out
+
+
 def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
     """configs[3]: W 5120x5120 Q4_K, X [T, 5120] bf16 -> f32 [T, 5120] on the matrix cores; and the same on the
     layer's largest projection (fused gate|up, 34816x5120), where the launch has enough tiles to fill the chip."""
@@ -337,6 +386,7 @@ def main():
     ap.add_argument("--no-q8", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the cold-rotation Q4_K 5120x5120 GEMV loop (what `value` is computed from); for profiling")
     ap.add_argument("--probe", action="store_true",
@@ -367,7 +417,7 @@ def main():
     c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
                                  cold_only=args.headline_only)
     if args.headline_only:
-        args.no_q8 = args.no_ffn = args.no_prefill = args.no_moe = args.no_sweep = args.no_cpu = True
+        args.no_q8 = args.no_ffn = args.no_prefill = args.no_moe = args.no_sweep = args.no_cpu = args.no_decode = True
         c2["warm"] = None
     ms_step = c2["cold"]["ms_per_step"]
     value = c2["cold"]["GBps"]
@@ -415,6 +465,9 @@ def main():
     if not args.no_sweep:
         log("[bench] 64-layer decode weight sweep (14.0 GB) ...")
         line["decode_sweep"] = bench_sweep(F, lib, check, stream, timer)
+    if not args.no_decode:
+        log("[bench] 64-layer decode step with attention (context 128 / 4096) ...")
+        line["decode_step_chained"] = bench_decode(F, lib, check, stream, timer)
     if not args.no_cpu:
         log("[bench] CPU baseline (oracle port) ...")
         line["cpu_baseline"] = cpu_baseline(rows, cols, 2)

@@ -80,6 +80,16 @@ SYMBOLS = {
     "fhip_matmul_q_coop": (C.c_int, [_vp, _vp, _sz, _vp, _vp, _vp]),
     "fhip_ffn_coop_ws_bytes": (_sz, [_vp, _vp, _sz]),
     "fhip_ffn_coop": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _vp, _vp]),
+    "fhip_rmsnorm": (C.c_int, [_vp, _vp, _sz, _sz, C.c_float, _vp, _vp]),
+    "fhip_add_rmsnorm": (C.c_int, [_vp, _vp, _vp, _sz, _sz, C.c_float, _vp, _vp, _vp]),
+    "fhip_add": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
+    "fhip_rope": (C.c_int, [_vp, _sz, _sz, _sz, _sz, _sz, C.c_float, _vp, _u32, _vp, C.c_int, _vp, _vp]),
+    "fhip_kv_append2": (C.c_int, [_vp, _vp, _sz, _sz, _vp, _u32, _vp, _vp, _sz, _vp]),
+    "fhip_qkv_post": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_int, C.c_float, C.c_float, _vp, _vp, _vp,
+                                _sz, _vp]),
+    "fhip_decode_attention_ws_bytes": (_sz, [_sz, _sz, _sz, _sz]),
+    "fhip_decode_attention": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
+    "fhip_u32_add": (C.c_int, [_vp, _sz, _u32, _vp]),
     "fhip_matvec_q8_0_host": (C.c_int, [_vp, _vp, _sz, _sz, _sz, _vp]),
 }
 

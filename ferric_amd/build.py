@@ -25,6 +25,7 @@ UNITS = {
     "gemv_generic.hip": [],
     "gemm_mfma.hip": [],
     "moe.hip": [],
+    "decode_ops.hip": [],
     "gguf.hip": [],
 }
 

@@ -369,6 +369,99 @@ int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float*
 
 // ---- mixture-of-experts entry points (crates/ferric-tensor/src/dtype.rs:1582-1780) ----------------------
 
+// ---- decode-layer steps --------------------------------------------------------------------------
+
+int fhip_rmsnorm(const float* d_x, const float* d_weight, size_t rows, size_t d, float eps, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (rows == 0 || d == 0) return FHIP_OK;
+    if (!d_x || !d_weight || !d_out) return set_error(FHIP_ERR_ARG, "fhip_rmsnorm: NULL pointer");
+    return fhip::launch_rmsnorm(d_x, nullptr, d_weight, rows, d, eps, nullptr, d_out, (hipStream_t)stream);
+}
+
+int fhip_add_rmsnorm(const float* d_a, const float* d_b, const float* d_weight, size_t rows, size_t d, float eps, float* d_sum,
+                     float* d_norm, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (rows == 0 || d == 0) return FHIP_OK;
+    if (!d_a || !d_b || !d_weight || !d_sum || !d_norm) return set_error(FHIP_ERR_ARG, "fhip_add_rmsnorm: NULL pointer");
+    return fhip::launch_rmsnorm(d_a, d_b, d_weight, rows, d, eps, d_sum, d_norm, (hipStream_t)stream);
+}
+
+int fhip_add(const float* d_a, const float* d_b, size_t n, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (n == 0) return FHIP_OK;
+    if (!d_a || !d_b || !d_out) return set_error(FHIP_ERR_ARG, "fhip_add: NULL pointer");
+    return fhip::launch_add(d_a, d_b, n, d_out, (hipStream_t)stream);
+}
+
+static int rope_checks(const char* who, size_t n_heads, size_t head_dim, size_t n_rot) {
+    if (n_rot > head_dim || n_rot % 2 != 0) return set_error(FHIP_ERR_SHAPE, "n_rot must be even and <= head_dim");   // lib.rs:437
+    if (n_heads > 0xFFFFu || head_dim > 0xFFFFu) return set_error(FHIP_ERR_SHAPE, "%s: n_heads / head_dim exceed 65535", who);
+    return FHIP_OK;
+}
+
+int fhip_rope(const float* d_x, size_t src_row_stride, size_t t, size_t n_heads, size_t head_dim, size_t n_rot, float base,
+              const uint32_t* d_positions, uint32_t pos_off, const float* d_freq_scale, int interleaved, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = rope_checks("fhip_rope", n_heads, head_dim, n_rot))) return rc;
+    if (t == 0 || n_heads == 0 || head_dim == 0) return FHIP_OK;
+    if (!d_x || !d_out) return set_error(FHIP_ERR_ARG, "fhip_rope: NULL pointer");
+    if (src_row_stride == 0) src_row_stride = n_heads * head_dim;
+    return fhip::launch_rope(d_x, src_row_stride, t, (int)n_heads, (int)head_dim, (int)n_rot, base, d_positions, pos_off, d_freq_scale,
+                             interleaved != 0, d_out, (hipStream_t)stream);
+}
+
+int fhip_kv_append2(const float* d_k, const float* d_v, size_t t, size_t width, const uint32_t* d_positions, uint32_t pos_off,
+                    float* d_k_cache, float* d_v_cache, size_t cap, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (t == 0 || width == 0) return FHIP_OK;
+    if (!d_k || !d_v || !d_k_cache || !d_v_cache) return set_error(FHIP_ERR_ARG, "fhip_kv_append2: NULL pointer");
+    if (cap > 0xFFFFFFFFull) return set_error(FHIP_ERR_SHAPE, "fhip_kv_append2: capacity exceeds 2^32 rows");
+    return fhip::launch_kv_append(d_k, d_v, t, width, d_positions, pos_off, cap, d_k_cache, d_v_cache, (hipStream_t)stream);
+}
+
+int fhip_qkv_post(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_positions,
+                  const float* d_freq_scale, size_t t, size_t n_head, size_t n_kv, size_t head_dim, size_t n_rot, int interleaved,
+                  float eps, float base, float* d_q_out, float* d_k_cache, float* d_v_cache, size_t cap, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = rope_checks("fhip_qkv_post", n_head + 2 * n_kv, head_dim, n_rot))) return rc;
+    if (t == 0 || head_dim == 0 || n_head + n_kv == 0) return FHIP_OK;
+    if (!d_qkv || !d_positions || !d_q_out || !d_k_cache || !d_v_cache) return set_error(FHIP_ERR_ARG, "fhip_qkv_post: NULL pointer");
+    if (cap > 0xFFFFFFFFull) return set_error(FHIP_ERR_SHAPE, "fhip_qkv_post: capacity exceeds 2^32 rows");
+    return fhip::launch_qkv_post(d_qkv, d_bias, d_q_norm, d_k_norm, d_positions, d_freq_scale, t, (int)n_head, (int)n_kv, (int)head_dim,
+                                 (int)n_rot, interleaved != 0, eps, base, d_q_out, d_k_cache, d_v_cache, cap, (hipStream_t)stream);
+}
+
+size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_dim, size_t len) {
+    if (g_device < 0 || n_kv == 0 || len == 0) return 0;
+    int splits = fhip::attn_splits(len, (int)n_kv);
+    return splits > 1 ? n_head * (size_t)splits * (head_dim + 2) * sizeof(float) : 0;
+}
+
+int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
+                          size_t len, const uint32_t* d_last_pos, float* d_ws, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (n_head > 0xFFFFu || n_kv > 0xFFFFu || head_dim > 0xFFFFu) return set_error(FHIP_ERR_SHAPE, "fhip_decode_attention: head counts exceed 65535");
+    if (n_head == 0 || head_dim == 0) return FHIP_OK;
+    if (!d_q || !d_k_cache || !d_v_cache || !d_out) return set_error(FHIP_ERR_ARG, "fhip_decode_attention: NULL pointer");
+    return fhip::launch_decode_attention(d_q, d_k_cache, d_v_cache, (int)n_head, (int)n_kv, (int)head_dim, len, d_last_pos, d_ws, d_out,
+                                         (hipStream_t)stream);
+}
+
+int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (n == 0) return FHIP_OK;
+    if (!d_words) return set_error(FHIP_ERR_ARG, "fhip_u32_add: NULL pointer");
+    return fhip::launch_u32_add(d_words, n, delta, (hipStream_t)stream);
+}
+
 int fhip_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t n_expert, size_t k, int sigmoid, float scale, int norm,
                   float* d_out, void* stream) {
     int rc = need_init();

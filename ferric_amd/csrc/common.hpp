@@ -82,4 +82,20 @@ int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s, 
 int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s, float* zero = nullptr,
                        size_t zero_n = 0);
 
+// decode_ops.hip: the steps either side of the matmuls in a decode layer
+int launch_rmsnorm(const float* a, const float* b, const float* weight, size_t rows, size_t d, float eps, float* sum_out, float* norm_out,
+                   hipStream_t s);
+int launch_add(const float* a, const float* b, size_t n, float* out, hipStream_t s);
+int launch_u32_add(uint32_t* w, size_t n, uint32_t delta, hipStream_t s);
+int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int hd, int n_rot, float base, const uint32_t* d_pos, uint32_t pos_off,
+                const float* freq_scale, int interleaved, float* out, hipStream_t s);
+int launch_qkv_post(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos, const float* freq_scale,
+                    size_t t, int n_head, int n_kv, int hd, int n_rot, int interleaved, float eps, float base, float* q_out, float* k_cache,
+                    float* v_cache, size_t cap, hipStream_t s);
+int launch_kv_append(const float* k, const float* v, size_t t, size_t width, const uint32_t* d_pos, uint32_t pos_off, size_t cap, float* kc,
+                     float* vc, hipStream_t s);
+int attn_splits(size_t len, int n_kv);
+int launch_decode_attention(const float* q, const float* K, const float* V, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len,
+                            float* ws, float* out, hipStream_t s);
+
 }  // namespace fhip

@@ -1,0 +1,426 @@
+// The steps either side of the quantized matmuls in one decode layer, gfx950: RMSNorm (plain and fused with the residual
+// add), rotary embedding, the per-head q/k norm + rotary + KV-cache append of a token's fused qkv row in one launch, the
+// KV append on its own, and single-query attention over the cache (split over the keys, all query heads of a KV head
+// sharing one pass over its keys and values).
+//
+// Replaces the reference's WGSL kernels RMSNORM / ADD_RMSNORM / ROPE / FUSED_ATTN / FUSED_ATTN_SPLIT / FUSED_ATTN_COMBINE
+// (crates/ferric-tensor/src/lib.rs:2018-2074, 2118-2162, 2675-2726 ff.) and `append2` (lib.rs:1379-1398), as
+// `Qwen3::attn` / `apply_layer` compose them (crates/ferric-llama/src/qwen3.rs:861-942, 979-1052).
+//
+// All of this is f32 arithmetic on small vectors: the kernels are launch- and latency-bound (a decode step has one row),
+// except attention, which streams the layer's K and V rows once (HBM-bound: 2 * len * n_kv * head_dim * 4 bytes).
+#include "common.hpp"
+
+#include <math.h>
+
+namespace {
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, false);
+    return v + __int_as_float(t);
+}
+// Sum over the 64 lanes of a wave, returned in every lane (through lane 63 and a scalar register).
+__device__ __forceinline__ float wave_sum(float v) {
+    v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+    v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane of a 16-lane row holds the row sum
+    v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+    v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// ---------------------------------------------------------------- RMSNorm, optionally of a + b
+// out[r, j] = x[r, j] * (1 / sqrt(mean_j x^2 + eps)) * weight[j]   (lib.rs:2018-2033); with b: x = a + b, and the sum is
+// written too (lib.rs:2057-2074). TPR threads share a row (a fixed-shape tree sum, so results do not depend on scheduling).
+template <int TPR>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* a, const float* __restrict__ b,
+                                                      const float* __restrict__ weight, size_t rows, int d, float eps,
+                                                      float* sum_out, float* __restrict__ norm_out) {   // sum_out may be a
+    constexpr int RPW = 256 / TPR;   // rows per workgroup
+    __shared__ float red[4];
+    const int tid = threadIdx.x, sub = tid / TPR, t = tid % TPR;
+    const size_t row = (size_t)blockIdx.x * RPW + sub;
+    const bool live = row < rows;
+    const float* xa = a + (live ? row : 0) * (size_t)d;
+    const float* xb = b ? b + (live ? row : 0) * (size_t)d : nullptr;
+    float ms = 0.f;
+    for (int j = t; j < d; j += TPR) {
+        float v = xb ? xa[j] + xb[j] : xa[j];
+        if (sum_out && live) sum_out[row * (size_t)d + j] = v;
+        ms = fmaf(v, v, ms);
+    }
+    ms = wave_sum(ms);
+    if (TPR == 256) {
+        if ((tid & 63) == 0) red[tid >> 6] = ms;
+        __syncthreads();
+        ms = (red[0] + red[1]) + (red[2] + red[3]);
+    }
+    const float inv = 1.0f / sqrtf(ms / (float)d + eps);
+    if (!live) return;
+    for (int j = t; j < d; j += TPR) {   // the same thread wrote sum_out[.., j] above, so reading it back is ordered
+        float v = sum_out ? sum_out[row * (size_t)d + j] : (xb ? xa[j] + xb[j] : xa[j]);
+        norm_out[row * (size_t)d + j] = v * inv * weight[j];
+    }
+}
+
+__global__ void u32_add_kernel(uint32_t* w, size_t n, uint32_t delta) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) w[i] += delta;
+}
+
+__global__ void add_kernel(const float* a, const float* __restrict__ b, size_t n, float* out) {   // out may be a
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] + b[i];
+}
+
+// ---------------------------------------------------------------- rotary embedding
+// Pair c of a head rotates by angle pos * base^(-2c / n_rot) (times freq_scale[c]); partners are (c, c + n_rot/2) in the
+// split-half layout and (2c, 2c + 1) interleaved; dims >= n_rot pass through (lib.rs:2118-2162, 2094-2116). The inverse
+// frequency is evaluated in f64 and rounded to f32 once, the angle is the f32 product the reference forms.
+__device__ __forceinline__ float rope_inv_freq(int c, int n_rot, float base, const float* freq_scale) {
+    float inv = (float)exp(-2.0 * (double)c / (double)n_rot * log((double)base));
+    return freq_scale ? inv * freq_scale[c] : inv;
+}
+
+__global__ void rope_kernel(const float* __restrict__ x, size_t src_row_stride, int t, int heads, int hd, int n_rot, float base,
+                            const uint32_t* __restrict__ pos, uint32_t pos_off, const float* __restrict__ freq_scale, int interleaved,
+                            float* __restrict__ out) {
+    const int half = n_rot / 2, per_head = hd - half;   // work items per head: the pairs, then the pass-through tail
+    size_t id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= (size_t)t * heads * per_head) return;
+    const int w = (int)(id % per_head), head = (int)((id / per_head) % heads), i = (int)(id / ((size_t)per_head * heads));
+    const float* xi = x + (size_t)i * src_row_stride + (size_t)head * hd;
+    float* oi = out + ((size_t)i * heads + head) * hd;
+    if (w >= half) { const int c = n_rot + (w - half); oi[c] = xi[c]; return; }
+    const int c = w;
+    const float p = (float)(pos ? pos[i] : pos_off + (uint32_t)i);
+    const float ang = p * rope_inv_freq(c, n_rot, base, freq_scale);
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    const int p0 = interleaved ? 2 * c : c, p1 = interleaved ? 2 * c + 1 : c + half;
+    const float x1 = xi[p0], x2 = xi[p1];
+    oi[p0] = x1 * cs - x2 * sn;
+    oi[p1] = x2 * cs + x1 * sn;
+}
+
+// ---------------------------------------------------------------- qkv row -> q, K cache, V cache
+// One wave per head of one token's fused qkv row (n_head query heads, n_kv key heads, n_kv value heads):
+//   query / key head: + bias, RMSNorm over the head with q_norm / k_norm (when given), rotary embedding at the token's position;
+//   the query goes to q_out[t, n_head * hd], the key to row pos of the K cache; a value head is copied (+ bias) to row pos of
+//   the V cache. This is qwen3.rs:861-905 (qn, rope, append2) in one launch.
+struct QkvPostParams {
+    const float* qkv;        // [t, (n_head + 2 n_kv) * hd]
+    const float* bias;       // same width, or null
+    const float* q_norm;     // [hd] or null
+    const float* k_norm;     // [hd] or null
+    const uint32_t* pos;     // [t] absolute positions (device)
+    const float* freq_scale; // [n_rot / 2] or null
+    float* q_out;            // [t, n_head * hd]
+    float* k_cache;          // [cap, n_kv * hd]
+    float* v_cache;
+    int t, n_head, n_kv, hd, n_rot, interleaved;
+    uint32_t cap;
+    float eps, base;
+};
+
+__global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
+    const int lane = threadIdx.x & 63;
+    const int per_tok = p.n_head + 2 * p.n_kv;
+    const size_t wid = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wid >= (size_t)p.t * per_tok) return;
+    const int i = (int)(wid / per_tok), h = (int)(wid % per_tok);
+    const uint32_t pos = p.pos[i];
+    const size_t col = (size_t)h * p.hd;
+    const float* x = p.qkv + (size_t)i * per_tok * p.hd + col;
+    const float* bias = p.bias ? p.bias + col : nullptr;
+    const int kvw = p.n_kv * p.hd;
+    float* dst;
+    const float* nw;
+    bool rotate = true;
+    if (h < p.n_head) { dst = p.q_out + ((size_t)i * p.n_head + h) * p.hd; nw = p.q_norm; }
+    else if (h < p.n_head + p.n_kv) { dst = p.k_cache + (size_t)pos * kvw + (size_t)(h - p.n_head) * p.hd; nw = p.k_norm; }
+    else { dst = p.v_cache + (size_t)pos * kvw + (size_t)(h - p.n_head - p.n_kv) * p.hd; nw = nullptr; rotate = false; }
+    if (h >= p.n_head && pos >= p.cap) return;   // a position past the cache is dropped, never written out of bounds
+    if (!rotate) {
+        for (int j = lane; j < p.hd; j += 64) dst[j] = bias ? x[j] + bias[j] : x[j];
+        return;
+    }
+    float inv = 1.f;
+    if (nw) {
+        float ms = 0.f;
+        for (int j = lane; j < p.hd; j += 64) { float v = bias ? x[j] + bias[j] : x[j]; ms = fmaf(v, v, ms); }
+        ms = wave_sum(ms);
+        inv = 1.0f / sqrtf(ms / (float)p.hd + p.eps);
+    }
+    auto val = [&](int j) { float v = bias ? x[j] + bias[j] : x[j]; return nw ? v * inv * nw[j] : v; };
+    const int half = p.n_rot / 2;
+    for (int c = lane; c < half; c += 64) {
+        const float ang = (float)pos * rope_inv_freq(c, p.n_rot, p.base, p.freq_scale);
+        float sn, cs;
+        sincosf(ang, &sn, &cs);
+        const int p0 = p.interleaved ? 2 * c : c, p1 = p.interleaved ? 2 * c + 1 : c + half;
+        const float x1 = val(p0), x2 = val(p1);
+        dst[p0] = x1 * cs - x2 * sn;
+        dst[p1] = x2 * cs + x1 * sn;
+    }
+    for (int j = p.n_rot + lane; j < p.hd; j += 64) dst[j] = val(j);
+}
+
+// K and V rows of t tokens into their caches at the tokens' positions, one launch (lib.rs:1379-1398).
+__global__ void kv_append_kernel(const float* __restrict__ k, const float* __restrict__ v, int t, int width, const uint32_t* __restrict__ pos,
+                                 uint32_t pos_off, uint32_t cap, float* __restrict__ kc, float* __restrict__ vc) {
+    size_t id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= (size_t)t * width) return;
+    const int i = (int)(id / width), j = (int)(id % width);
+    const uint32_t r = pos ? pos[i] : pos_off + (uint32_t)i;
+    if (r >= cap) return;
+    kc[(size_t)r * width + j] = k[id];
+    vc[(size_t)r * width + j] = v[id];
+}
+
+// ---------------------------------------------------------------- single-query attention over the cache
+// out[h] = softmax_j(q[h] . K[j, kv(h)] * scale) @ V[:, kv(h)]   for one query row (nn.rs:140-166, lib.rs:2675-2726).
+// Workgroup (kv head, split): its 4 waves walk the split's keys in blocks of KB; a lane holds DPL = hd / 64 consecutive
+// dims of a row, so one key or value row is one coalesced wave load, read ONCE for all G = n_head / n_kv query heads of the
+// group. Running (max, sum, accumulator) per query head, merged across the waves through LDS and across splits by
+// attn_combine_kernel -- the reference's own rescale exp(m_old - m_new), applied across partitions.
+constexpr int ATT_KB = 8;
+
+template <int DPL>
+__device__ __forceinline__ void load_dims(const float* p, float (&r)[DPL]) {   // p is 4 * DPL-byte aligned
+    if constexpr (DPL == 2) { float2 v = *(const float2*)p; r[0] = v.x; r[1] = v.y; }
+    else { r[0] = *p; }
+}
+
+template <int G, int DPL>
+__global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict__ q, const float* __restrict__ K, const float* __restrict__ V,
+                                                         int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
+                                                         float* __restrict__ part, float* __restrict__ out) {
+    constexpr int HD = 64 * DPL;
+    __shared__ float sm_m[4][G], sm_l[4][G];
+    __shared__ float sm_acc[4][G][HD];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int kvh = blockIdx.x, split = blockIdx.y;
+    uint32_t len = len_dev ? *len_dev + 1u : len_host;   // the device word is the newest token's position
+    if (len > len_host) len = len_host;
+    const uint32_t per = (len + splits - 1) / splits;
+    const uint32_t k0 = (uint32_t)split * per, k1 = min(len, k0 + per);
+    const size_t stride = (size_t)n_kv * HD;
+    const float* Kb = K + (size_t)kvh * HD + lane * DPL;
+    const float* Vb = V + (size_t)kvh * HD + lane * DPL;
+
+    float qr[G][DPL], acc[G][DPL], m[G], l[G];
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        m[h] = -3.0e38f; l[h] = 0.f;
+#pragma unroll
+        for (int i = 0; i < DPL; i++) { qr[h][i] = q[((size_t)kvh * G + h) * HD + lane * DPL + i]; acc[h][i] = 0.f; }
+    }
+    for (uint32_t kb = k0 + wave * ATT_KB; kb < k1; kb += 4 * ATT_KB) {
+        float kr[ATT_KB][DPL], vr[ATT_KB][DPL];
+#pragma unroll
+        for (int j = 0; j < ATT_KB; j++) {
+            const uint32_t key = min(kb + j, k1 - 1);   // rows past the split re-read its last row and are masked below
+            load_dims<DPL>(Kb + key * stride, kr[j]);
+            load_dims<DPL>(Vb + key * stride, vr[j]);
+        }
+        float s[G][ATT_KB];
+#pragma unroll
+        for (int h = 0; h < G; h++)
+#pragma unroll
+            for (int j = 0; j < ATT_KB; j++) {
+                float d = 0.f;
+#pragma unroll
+                for (int i = 0; i < DPL; i++) d = fmaf(qr[h][i], kr[j][i], d);
+                const float r = wave_sum(d) * scale;
+                s[h][j] = (kb + j < k1) ? r : -3.0e38f;
+            }
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float bm = s[h][0];
+#pragma unroll
+            for (int j = 1; j < ATT_KB; j++) bm = fmaxf(bm, s[h][j]);
+            const float m_new = fmaxf(m[h], bm), corr = expf(m[h] - m_new);
+            float ps = 0.f, a[DPL];
+#pragma unroll
+            for (int i = 0; i < DPL; i++) a[i] = 0.f;
+#pragma unroll
+            for (int j = 0; j < ATT_KB; j++) {
+                const float e = (kb + j < k1) ? expf(s[h][j] - m_new) : 0.f;
+                ps += e;
+#pragma unroll
+                for (int i = 0; i < DPL; i++) a[i] = fmaf(e, vr[j][i], a[i]);
+            }
+            l[h] = l[h] * corr + ps;
+#pragma unroll
+            for (int i = 0; i < DPL; i++) acc[h][i] = acc[h][i] * corr + a[i];
+            m[h] = m_new;
+        }
+    }
+    // merge the four waves
+#pragma unroll
+    for (int h = 0; h < G; h++) {
+        if (lane == 0) { sm_m[wave][h] = m[h]; sm_l[wave][h] = l[h]; }
+#pragma unroll
+        for (int i = 0; i < DPL; i++) sm_acc[wave][h][lane * DPL + i] = acc[h][i];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
+        const int h = idx / HD, d = idx % HD;
+        const float M = fmaxf(fmaxf(sm_m[0][h], sm_m[1][h]), fmaxf(sm_m[2][h], sm_m[3][h]));
+        float L = 0.f, A = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float f = expf(sm_m[w][h] - M);
+            L = fmaf(sm_l[w][h], f, L);
+            A = fmaf(sm_acc[w][h][d], f, A);
+        }
+        const int head = kvh * G + h;
+        if (splits == 1) {
+            out[(size_t)head * HD + d] = A / L;
+        } else {
+            float* pp = part + ((size_t)head * splits + split) * (HD + 2);
+            pp[d] = A;
+            if (d == 0) { pp[HD] = M; pp[HD + 1] = L; }
+        }
+    }
+}
+
+__global__ void attn_combine_kernel(const float* __restrict__ part, int hd, int splits, float* __restrict__ out) {
+    const int head = blockIdx.x;
+    const float* pp = part + (size_t)head * splits * (hd + 2);
+    float M = -3.0e38f;
+    for (int s = 0; s < splits; s++) M = fmaxf(M, pp[(size_t)s * (hd + 2) + hd]);
+    float L = 0.f;
+    for (int s = 0; s < splits; s++) L = fmaf(pp[(size_t)s * (hd + 2) + hd + 1], expf(pp[(size_t)s * (hd + 2) + hd] - M), L);
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float A = 0.f;
+        for (int s = 0; s < splits; s++) A = fmaf(pp[(size_t)s * (hd + 2) + d], expf(pp[(size_t)s * (hd + 2) + hd] - M), A);
+        out[(size_t)head * hd + d] = A / L;
+    }
+}
+
+template <int G>
+int launch_attn_g(int dpl, dim3 grid, hipStream_t s, const float* q, const float* K, const float* V, int n_kv, uint32_t len, const uint32_t* d_len,
+                  float scale, int splits, float* part, float* out) {
+    switch (dpl) {
+        case 1: hipLaunchKernelGGL((attn_split_kernel<G, 1>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
+        case 2: hipLaunchKernelGGL((attn_split_kernel<G, 2>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
+        default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
+    }
+    return FHIP_OK;
+}
+
+}  // namespace
+
+namespace fhip {
+
+int launch_rmsnorm(const float* a, const float* b, const float* weight, size_t rows, size_t d, float eps, float* sum_out, float* norm_out,
+                   hipStream_t s) {
+    if (rows == 0 || d == 0) return FHIP_OK;
+    if (d > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "rmsnorm: row length exceeds 2^31");
+    if (d <= 512) {
+        size_t grid = (rows + 3) / 4;
+        if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "rmsnorm: too many rows for one launch");
+        hipLaunchKernelGGL((rmsnorm_kernel<64>), dim3((unsigned)grid), dim3(256), 0, s, a, b, weight, rows, (int)d, eps, sum_out, norm_out);
+    } else {
+        if (rows > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "rmsnorm: too many rows for one launch");
+        hipLaunchKernelGGL((rmsnorm_kernel<256>), dim3((unsigned)rows), dim3(256), 0, s, a, b, weight, rows, (int)d, eps, sum_out, norm_out);
+    }
+    return check_hip(hipGetLastError(), "rmsnorm launch");
+}
+
+int launch_u32_add(uint32_t* w, size_t n, uint32_t delta, hipStream_t s) {
+    size_t grid = (n + 255) / 256;
+    if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "u32_add: too many words for one launch");
+    hipLaunchKernelGGL(u32_add_kernel, dim3((unsigned)grid), dim3(256), 0, s, w, n, delta);
+    return check_hip(hipGetLastError(), "u32_add launch");
+}
+
+int launch_add(const float* a, const float* b, size_t n, float* out, hipStream_t s) {
+    if (n == 0) return FHIP_OK;
+    size_t grid = (n + 255) / 256;
+    if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "add: too many elements for one launch");
+    hipLaunchKernelGGL(add_kernel, dim3((unsigned)grid), dim3(256), 0, s, a, b, n, out);
+    return check_hip(hipGetLastError(), "add launch");
+}
+
+int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int hd, int n_rot, float base, const uint32_t* d_pos, uint32_t pos_off,
+                const float* freq_scale, int interleaved, float* out, hipStream_t s) {
+    if (t == 0 || heads == 0 || hd == 0) return FHIP_OK;
+    size_t n = t * (size_t)heads * (size_t)(hd - n_rot / 2);
+    size_t grid = (n + 255) / 256;
+    if (t > 0x7FFFFFFFull || grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "rope: too many rows for one launch");
+    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)grid), dim3(256), 0, s, x, src_row_stride, (int)t, heads, hd, n_rot, base, d_pos, pos_off,
+                       freq_scale, interleaved, out);
+    return check_hip(hipGetLastError(), "rope launch");
+}
+
+int launch_qkv_post(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos, const float* freq_scale,
+                    size_t t, int n_head, int n_kv, int hd, int n_rot, int interleaved, float eps, float base, float* q_out, float* k_cache,
+                    float* v_cache, size_t cap, hipStream_t s) {
+    if (t == 0) return FHIP_OK;
+    QkvPostParams p;
+    p.qkv = qkv; p.bias = bias; p.q_norm = q_norm; p.k_norm = k_norm; p.pos = d_pos; p.freq_scale = freq_scale;
+    p.q_out = q_out; p.k_cache = k_cache; p.v_cache = v_cache;
+    p.t = (int)t; p.n_head = n_head; p.n_kv = n_kv; p.hd = hd; p.n_rot = n_rot; p.interleaved = interleaved;
+    p.cap = (uint32_t)cap; p.eps = eps; p.base = base;
+    size_t waves = t * (size_t)(n_head + 2 * n_kv), grid = (waves + 3) / 4;
+    if (t > 0x7FFFFFFFull || grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "qkv_post: too many rows for one launch");
+    hipLaunchKernelGGL(qkv_post_kernel, dim3((unsigned)grid), dim3(256), 0, s, p);
+    return check_hip(hipGetLastError(), "qkv_post launch");
+}
+
+int launch_kv_append(const float* k, const float* v, size_t t, size_t width, const uint32_t* d_pos, uint32_t pos_off, size_t cap, float* kc,
+                     float* vc, hipStream_t s) {
+    if (t == 0 || width == 0) return FHIP_OK;
+    size_t n = t * width, grid = (n + 255) / 256;
+    if (t > 0x7FFFFFFFull || width > 0x7FFFFFFFull || grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "kv_append: too large for one launch");
+    hipLaunchKernelGGL(kv_append_kernel, dim3((unsigned)grid), dim3(256), 0, s, k, v, (int)t, (int)width, d_pos, pos_off, (uint32_t)cap, kc, vc);
+    return check_hip(hipGetLastError(), "kv_append launch");
+}
+
+// Splits of the key range: enough workgroups to cover the chip once, at least 64 keys each.
+int attn_splits(size_t len, int n_kv) {
+    if (n_kv <= 0 || len == 0) return 1;
+    int want = (device_cus() + n_kv - 1) / n_kv;
+    size_t by_keys = (len + 63) / 64;
+    int splits = (int)(by_keys < (size_t)want ? by_keys : (size_t)want);
+    return splits < 1 ? 1 : splits;
+}
+
+int launch_decode_attention(const float* q, const float* K, const float* V, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len,
+                            float* ws, float* out, hipStream_t s) {
+    if (n_head == 0 || hd == 0) return FHIP_OK;
+    if (len == 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: empty cache");
+    if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: n_heads must be a multiple of n_kv_heads");
+    if (hd != 64 && hd != 128) return set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
+    if (len > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "decode_attention: cache length exceeds 2^31");
+    const int g = n_head / n_kv, splits = attn_splits(len, n_kv);
+    if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
+    const float scale = 1.0f / sqrtf((float)hd);
+    dim3 grid((unsigned)n_kv, (unsigned)splits);
+    int rc;
+    switch (g) {
+        case 1: rc = launch_attn_g<1>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 2: rc = launch_attn_g<2>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 3: rc = launch_attn_g<3>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 4: rc = launch_attn_g<4>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 5: rc = launch_attn_g<5>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 6: rc = launch_attn_g<6>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 7: rc = launch_attn_g<7>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 8: rc = launch_attn_g<8>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        default: return set_error(FHIP_ERR_SHAPE, "decode_attention: %d query heads per KV head (1..=8 supported)", g);
+    }
+    if (rc) return rc;
+    if ((rc = check_hip(hipGetLastError(), "decode_attention launch"))) return rc;
+    if (splits > 1) {
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(hd), 0, s, ws, hd, splits, out);
+        rc = check_hip(hipGetLastError(), "decode_attention combine launch");
+    }
+    return rc;
+}
+
+}  // namespace fhip

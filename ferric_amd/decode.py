@@ -1,0 +1,225 @@
+"""Host mirror of the reference's decode-layer ops and of `Qwen3::apply_layer` for one new token.
+
+The ops are the reference's `Tensor::rmsnorm / add_rmsnorm / add / rope*` (crates/ferric-tensor/src/lib.rs:279-520),
+`append2` (lib.rs:1379) and `nn::decode_attention` (crates/ferric-tensor/src/nn.rs:140); `Qwen3Decoder` is the default
+(pre-norm, no post-norms, no window, no softcap) arm of `Qwen3::attn / ffn / apply_layer`
+(crates/ferric-llama/src/qwen3.rs:861-966, 979-1052). Everything runs through libferric_hip; there is no CPU path.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from .qmatrix import DeviceBuffer, Graph, Tensor, _stream_handle, _vp
+
+
+def _check(rc):
+    _lib.check(rc)
+
+
+def _u32_tensor(values):
+    a = np.ascontiguousarray(values, dtype=np.uint32)
+    t = Tensor(DeviceBuffer(max(a.nbytes, 4)), a.shape, np.uint32)
+    _check(_lib.load().fhip_memcpy_h2d(t.buf.ptr, _vp(a), a.nbytes, None))
+    _check(_lib.load().fhip_stream_sync(None))
+    return t
+
+
+def rmsnorm(x, weight, eps, stream=None):
+    """lib.rs:346: x [.., d] normalised over the last dim, times weight [d]."""
+    d = x.shape[-1]
+    assert weight.numel() == d, f"rmsnorm: weight has {weight.numel()} elements, rows have {d}"
+    out = Tensor.empty(x.shape)
+    _check(_lib.load().fhip_rmsnorm(x.buf.ptr, weight.buf.ptr, x.numel() // d, d, eps, out.buf.ptr, _stream_handle(stream)))
+    return out
+
+
+def add_rmsnorm(a, b, weight, eps, stream=None):
+    """lib.rs:372: (a + b, rmsnorm(a + b, weight))."""
+    assert a.shape == b.shape, f"add_rmsnorm: shape mismatch {list(a.shape)} vs {list(b.shape)}"
+    d = a.shape[-1]
+    assert weight.numel() == d
+    s, n = Tensor.empty(a.shape), Tensor.empty(a.shape)
+    _check(_lib.load().fhip_add_rmsnorm(a.buf.ptr, b.buf.ptr, weight.buf.ptr, a.numel() // d, d, eps, s.buf.ptr, n.buf.ptr,
+                                        _stream_handle(stream)))
+    return s, n
+
+
+def add(a, b, stream=None):
+    """lib.rs:279 for equal shapes."""
+    assert a.shape == b.shape, "add: shapes differ (no broadcasting on this path)"
+    out = Tensor.empty(a.shape)
+    _check(_lib.load().fhip_add(a.buf.ptr, b.buf.ptr, a.numel(), out.buf.ptr, _stream_handle(stream)))
+    return out
+
+
+def rope(x, n_heads, head_dim, base, offset=0, positions=None, freq_scale=None, interleaved=False, n_rot=None, stream=None):
+    """lib.rs:417 rope (split-half pairs), :409 rope_interleaved, :429 rope_partial (n_rot), :465 rope_at / :489 rope_at_ex
+    (positions: one absolute position per row, host values or a device u32 Tensor)."""
+    n_rot = head_dim if n_rot is None else n_rot
+    assert n_rot <= head_dim and n_rot % 2 == 0, "n_rot must be even and <= head_dim"
+    t = x.numel() // (n_heads * head_dim)
+    pos_t = None
+    if positions is not None:
+        pos_t = positions if isinstance(positions, Tensor) else _u32_tensor(positions)
+        assert pos_t.numel() == t, f"rope_at needs one position per row: {t} rows, {pos_t.numel()} given"
+    out = Tensor.empty(x.shape)
+    _check(_lib.load().fhip_rope(x.buf.ptr, 0, t, n_heads, head_dim, n_rot, base, pos_t.buf.ptr if pos_t is not None else None, offset,
+                                 freq_scale.buf.ptr if freq_scale is not None else None, int(interleaved), out.buf.ptr,
+                                 _stream_handle(stream)))
+    if pos_t is not None and not isinstance(positions, Tensor) and stream is None:
+        _check(_lib.load().fhip_stream_sync(None))     # the temporary position buffer is freed on return
+    return out
+
+
+class KvCache:
+    """One layer's K and V history, [cap, width] f32 each, filled to `len` rows (the reference's pair of KvBuf, lib.rs:1287,
+    with a fixed capacity: a captured step cannot reallocate)."""
+
+    def __init__(self, cap, width):
+        self.cap, self.width, self.len = int(cap), int(width), 0
+        self.k, self.v = Tensor.empty((cap, width)), Tensor.empty((cap, width))
+
+    def append2(self, k, v, stream=None):
+        """lib.rs:1379: rows of k and v [t, width] appended to both caches in one launch."""
+        assert len(k.shape) == 2 and len(v.shape) == 2, "append2 expects 2D [t, width] tensors"
+        assert k.shape[0] == v.shape[0], "K and V must append the same number of rows"
+        assert k.shape[1] == self.width and v.shape[1] == self.width, "KvBuf width changed"
+        t = k.shape[0]
+        assert self.len + t <= self.cap, f"KvCache: {self.len} + {t} rows exceed the capacity {self.cap}"
+        _check(_lib.load().fhip_kv_append2(k.buf.ptr, v.buf.ptr, t, self.width, None, self.len, self.k.buf.ptr, self.v.buf.ptr, self.cap,
+                                           _stream_handle(stream)))
+        self.len += t
+        return self
+
+
+def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, ws=None, stream=None):
+    """nn.rs:140: q [1, n_heads * dh] against the first `length` rows of the cache (default: all filled rows). last_pos: a
+    device u32 Tensor holding the newest row's index, read at run time instead (for a captured step)."""
+    assert len(q.shape) == 2 and q.shape[0] == 1, "decode_attention takes one query row"
+    dh = q.shape[1] // n_heads
+    length = cache.len if length is None else length
+    assert cache.width == n_kv_heads * dh
+    lib = _lib.load()
+    need = lib.fhip_decode_attention_ws_bytes(n_heads, n_kv_heads, dh, length)
+    own = None
+    if need and ws is None:
+        own = ws = DeviceBuffer(need)
+    out = Tensor.empty((1, n_heads * dh))
+    _check(lib.fhip_decode_attention(q.buf.ptr, cache.k.buf.ptr, cache.v.buf.ptr, n_heads, n_kv_heads, dh, length,
+                                     last_pos.buf.ptr if last_pos is not None else None, ws.ptr if ws is not None else None, out.buf.ptr,
+                                     _stream_handle(stream)))
+    if own is not None:
+        _check(lib.fhip_stream_sync(_stream_handle(stream)))   # the scratch is freed on return
+    return out
+
+
+class Qwen3Cfg:
+    """The fields of the reference's Cfg this path reads (qwen3.rs: n_head, n_head_kv, head_dim, eps, rope pairing)."""
+
+    def __init__(self, d_model, n_head, n_head_kv, head_dim, n_ff, eps=1e-6, rope_base=1e6, rope_interleaved=False):
+        self.d_model, self.n_head, self.n_head_kv, self.head_dim, self.n_ff = d_model, n_head, n_head_kv, head_dim, n_ff
+        self.eps, self.rope_base, self.rope_interleaved = float(eps), float(rope_base), bool(rope_interleaved)
+
+
+class Qwen3Layer:
+    """qwen3.rs:230-253, the fields of the default arm: norms as f32 Tensors, projections as QMatrix (wqkv = q|k|v stacked,
+    ffn_gate_up = gate|up stacked)."""
+
+    def __init__(self, attn_norm, wqkv, wo, ffn_norm, ffn_gate_up, ffn_down, q_norm=None, k_norm=None, qkv_bias=None):
+        self.attn_norm, self.wqkv, self.wo, self.ffn_norm = attn_norm, wqkv, wo, ffn_norm
+        self.ffn_gate_up, self.ffn_down, self.q_norm, self.k_norm, self.qkv_bias = ffn_gate_up, ffn_down, q_norm, k_norm, qkv_bias
+
+
+class Qwen3Decoder:
+    """One-token decode through a stack of layers with preallocated activations, so that a whole step is a fixed sequence
+    of launches (capturable as one graph). Per layer, 9 launches:
+        h = rmsnorm(x) [fused with the previous layer's residual add]; qkv = h Wqkv^T; q/k norm + rope + cache append;
+        attention (+ combine); o = a Wo^T; (x, h) = add_rmsnorm(x, o); f = swiglu(h Wgu^T); y = f Wdown^T; x += y [next fused add]
+    """
+
+    def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None):
+        self.cfg, self.layers, self.max_len, self.stream = cfg, layers, int(max_len), stream
+        self.output_norm, self.lm_head = output_norm, lm_head          # final norm + LM head: hidden -> logits in the same step
+        assert (output_norm is None) == (lm_head is None), "output_norm and lm_head come together"
+        self.logits = Tensor.empty((1, lm_head.rows())) if lm_head is not None else None
+        c = cfg
+        self.q_out, self.kv_out = c.n_head * c.head_dim, c.n_head_kv * c.head_dim
+        self.caches = [KvCache(max_len, self.kv_out) for _ in layers]
+        self.pos = _u32_tensor([0])                       # device word: the position of the token being decoded
+        self.x = Tensor.empty((1, c.d_model))             # residual stream
+        self.h = Tensor.empty((1, c.d_model))             # normed input of the current block
+        self.qkv = Tensor.empty((1, self.q_out + 2 * self.kv_out))
+        self.q = Tensor.empty((1, self.q_out))
+        self.att = Tensor.empty((1, self.q_out))
+        self.o = Tensor.empty((1, c.d_model))
+        self.f = Tensor.empty((1, c.n_ff))
+        self.y = Tensor.empty((1, c.d_model))
+        lib = _lib.load()
+        need = lib.fhip_decode_attention_ws_bytes(c.n_head, c.n_head_kv, c.head_dim, self.max_len)
+        self.ws = DeviceBuffer(need) if need else None
+        self._graph = None
+
+    # -- state ------------------------------------------------------------------------------------
+    def set_pos(self, pos):
+        a = np.array([pos], np.uint32)
+        _check(_lib.load().fhip_memcpy_h2d(self.pos.buf.ptr, _vp(a), 4, _stream_handle(self.stream)))
+        _check(_lib.load().fhip_stream_sync(_stream_handle(self.stream)))
+        for c in self.caches:
+            c.len = pos
+
+    def set_input(self, x_host):
+        a = np.ascontiguousarray(x_host, dtype=np.float32).reshape(-1)
+        assert a.size == self.cfg.d_model
+        _check(_lib.load().fhip_memcpy_h2d(self.x.buf.ptr, _vp(a), a.nbytes, _stream_handle(self.stream)))
+        _check(_lib.load().fhip_stream_sync(_stream_handle(self.stream)))
+
+    # -- one step ---------------------------------------------------------------------------------
+    def _enqueue_step(self):
+        """All layers on the current x at position *pos; leaves the final hidden state in x and advances *pos."""
+        lib, c, s = _lib.load(), self.cfg, _stream_handle(self.stream)
+        d = c.d_model
+        for il, (l, kv) in enumerate(zip(self.layers, self.caches)):
+            if il == 0:
+                _check(lib.fhip_rmsnorm(self.x.buf.ptr, l.attn_norm.buf.ptr, 1, d, c.eps, self.h.buf.ptr, s))
+            else:   # x = x + y of the previous layer's FFN, and this layer's input norm, in one launch
+                _check(lib.fhip_add_rmsnorm(self.x.buf.ptr, self.y.buf.ptr, l.attn_norm.buf.ptr, 1, d, c.eps, self.x.buf.ptr, self.h.buf.ptr, s))
+            _check(lib.fhip_matmul_q(l.wqkv.handle, self.h.buf.ptr, 1, self.qkv.buf.ptr, s))
+            _check(lib.fhip_qkv_post(self.qkv.buf.ptr, l.qkv_bias.buf.ptr if l.qkv_bias is not None else None,
+                                     l.q_norm.buf.ptr if l.q_norm is not None else None, l.k_norm.buf.ptr if l.k_norm is not None else None,
+                                     self.pos.buf.ptr, None, 1, c.n_head, c.n_head_kv, c.head_dim, c.head_dim, int(c.rope_interleaved),
+                                     c.eps, c.rope_base, self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap, s))
+            _check(lib.fhip_decode_attention(self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, c.n_head, c.n_head_kv, c.head_dim, self.max_len,
+                                             self.pos.buf.ptr, self.ws.ptr if self.ws is not None else None, self.att.buf.ptr, s))
+            _check(lib.fhip_matmul_q(l.wo.handle, self.att.buf.ptr, 1, self.o.buf.ptr, s))
+            _check(lib.fhip_add_rmsnorm(self.x.buf.ptr, self.o.buf.ptr, l.ffn_norm.buf.ptr, 1, d, c.eps, self.x.buf.ptr, self.h.buf.ptr, s))
+            _check(lib.fhip_matmul_q_swiglu(l.ffn_gate_up.handle, self.h.buf.ptr, 1, self.f.buf.ptr, s))
+            _check(lib.fhip_matmul_q(l.ffn_down.handle, self.f.buf.ptr, 1, self.y.buf.ptr, s))
+        if self.lm_head is not None:   # last residual add fused with the output norm, then the LM head
+            _check(lib.fhip_add_rmsnorm(self.x.buf.ptr, self.y.buf.ptr, self.output_norm.buf.ptr, 1, d, c.eps, self.x.buf.ptr, self.h.buf.ptr, s))
+            _check(lib.fhip_matmul_q(self.lm_head.handle, self.h.buf.ptr, 1, self.logits.buf.ptr, s))
+        else:
+            _check(lib.fhip_add(self.x.buf.ptr, self.y.buf.ptr, d, self.x.buf.ptr, s))
+        _check(lib.fhip_u32_add(self.pos.buf.ptr, 1, 1, s))
+
+    def step(self):
+        """Eager: enqueue one step and account for the appended row."""
+        self._enqueue_step()
+        for c in self.caches:
+            c.len += 1
+
+    def capture(self):
+        """The same step as one graph; replay with step_graph()."""
+        assert self.stream is not None, "capture needs a stream from Stream()"
+        g = Graph.begin(self.stream)
+        self._enqueue_step()
+        self._graph = g.end()
+        return self._graph
+
+    def step_graph(self):
+        self._graph.launch()
+        for c in self.caches:
+            c.len += 1
+
+    def hidden(self):
+        return self.x.to_vec(self.stream)

@@ -201,6 +201,59 @@ int fhip_matmul_q_id(const fhip_weight* w, const float* d_x, const float* d_selw
 int fhip_matmul_q_id_wsum(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t out_pe, float* d_y,
                           float* d_ws, void* stream);
 
+/* ---- the steps either side of the matmuls in one decode layer (crates/ferric-llama/src/qwen3.rs:861-942 `attn`,
+ * :979-1052 `apply_layer`). f32 throughout; every pointer is device memory; all enqueue on `stream` and return. ---- */
+
+/* crates/ferric-tensor/src/lib.rs:346 Tensor::rmsnorm (kernel :2018): out[r, j] = x[r, j] / sqrt(mean_j x[r, :]^2 + eps)
+ * * weight[j], rows x d. The sum of squares is a fixed-shape tree over the row instead of the reference's one-thread
+ * serial loop: same value to rounding, not the same bits. */
+int fhip_rmsnorm(const float* d_x, const float* d_weight, size_t rows, size_t d, float eps, float* d_out, void* stream);
+
+/* lib.rs:372 Tensor::add_rmsnorm (kernel :2057): sum = a + b (bit-exact), norm = rmsnorm(sum, weight). d_sum may be d_a
+ * (the residual updated in place). */
+int fhip_add_rmsnorm(const float* d_a, const float* d_b, const float* d_weight, size_t rows, size_t d, float eps, float* d_sum,
+                     float* d_norm, void* stream);
+
+/* lib.rs:279 Tensor::add, same shapes: out = a + b, n elements. */
+int fhip_add(const float* d_a, const float* d_b, size_t n, float* d_out, void* stream);
+
+/* lib.rs:417 Tensor::rope / :409 rope_interleaved / :429 rope_partial / :465 rope_at / :489 rope_at_ex (kernels :2118,
+ * :2094). x: t rows of n_heads * head_dim, row i at d_x + i * src_row_stride (a strided window such as a slice of the
+ * fused qkv row is read in place; 0 = packed rows); out packed [t, n_heads * head_dim]. Row i sits at position
+ * d_positions[i] (device u32) or, when that is NULL, pos_off + i. Pair c rotates by position * base^(-2c / n_rot)
+ * [* d_freq_scale[c]]; partners are (c, c + n_rot/2), or (2c, 2c + 1) when interleaved; dims >= n_rot are copied.
+ * n_rot odd or > head_dim -> FHIP_ERR_SHAPE (the reference's assert, lib.rs:437). */
+int fhip_rope(const float* d_x, size_t src_row_stride, size_t t, size_t n_heads, size_t head_dim, size_t n_rot, float base,
+              const uint32_t* d_positions, uint32_t pos_off, const float* d_freq_scale, int interleaved, float* d_out, void* stream);
+
+/* lib.rs:1379 append2: rows of k and v [t, width] into the two caches [cap, width] at rows d_positions[i] (or pos_off +
+ * i), one launch. The caches are caller-owned, fixed-capacity buffers (the reference's KvBuf grows by reallocating, which
+ * a captured step cannot do); a row at or past cap is dropped. */
+int fhip_kv_append2(const float* d_k, const float* d_v, size_t t, size_t width, const uint32_t* d_positions, uint32_t pos_off,
+                    float* d_k_cache, float* d_v_cache, size_t cap, void* stream);
+
+/* qwen3.rs:861-905 in one launch, for t tokens' fused qkv rows [t, (n_head + 2 n_kv) * head_dim]: + d_bias (optional,
+ * :848), per-head RMSNorm of the query and key heads with d_q_norm / d_k_norm [head_dim] (optional, :851-855), rotary
+ * embedding of both at d_positions[i] (as fhip_rope), query heads to d_q_out [t, n_head * head_dim], key and value heads
+ * to row d_positions[i] of the caches [cap, n_kv * head_dim]. No single counterpart in the reference: it issues these as
+ * 4-5 dispatches. */
+int fhip_qkv_post(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_positions,
+                  const float* d_freq_scale, size_t t, size_t n_head, size_t n_kv, size_t head_dim, size_t n_rot, int interleaved,
+                  float eps, float base, float* d_q_out, float* d_k_cache, float* d_v_cache, size_t cap, void* stream);
+
+/* crates/ferric-tensor/src/nn.rs:140 decode_attention -> lib.rs:762 fused_decode_attention (kernels :2675, :2740 ff.):
+ * one query row q [n_head * head_dim] against the cache rows [0, len) of K and V [., n_kv * head_dim];
+ * out[h] = softmax_j(q_h . K[j, h / g] / sqrt(head_dim)) @ V[:, h / g], g = n_head / n_kv (1..=8), head_dim 64 or 128.
+ * When d_last_pos is given the length is *d_last_pos + 1 read on the device (clamped to len), so one captured launch
+ * serves a growing cache; len still sizes the launch. d_ws: fhip_decode_attention_ws_bytes(...) bytes of scratch (the
+ * per-split partial sums; may be NULL when that is 0). */
+size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_dim, size_t len);
+int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
+                          size_t len, const uint32_t* d_last_pos, float* d_ws, float* d_out, void* stream);
+
+/* words[i] += delta for n device u32 words: advances the position word(s) at the end of a captured decode step. */
+int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream);
+
 /* f32 -> bf16 bit patterns, round to nearest even, n values (both pointers 16-byte aligned). The reference's
  * matrix-unit kernels read f32 activations (crates/ferric-tensor/src/dtype.rs:1824-1830, `xp.buf`); the
  * matrix cores here take bf16, so this is the conversion in front of fhip_gemm_q_bf16. */

@@ -1,0 +1,225 @@
+"""The decode-layer steps around the quantized matmuls, through the C ABI, against the f64 oracle (oracle/decode_oracle.py).
+Floating-point kernels: tolerances are written at each comparison, relative to the largest expected magnitude; the
+residual sum of add_rmsnorm, the pass-through dims of rope and cache appends are copies or single f32 adds and must be
+bit-exact."""
+import numpy as np
+import pytest
+
+from conftest import bits
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+
+
+@pytest.fixture(scope="module")
+def D():
+    from oracle import decode_oracle
+    return decode_oracle
+
+
+@pytest.fixture(scope="module")
+def X(F):
+    from ferric_amd import decode
+    return decode
+
+
+def close(got, want, rel):
+    want = np.asarray(want, np.float64)
+    return np.abs(np.asarray(got, np.float64).reshape(want.shape) - want).max() <= rel * max(1e-30, np.abs(want).max())
+
+
+def test_rmsnorm_and_add_rmsnorm(F, X, D):
+    rng = np.random.default_rng(0)
+    for rows, d in [(1, 5120), (3, 4096), (40, 128), (7, 64), (1, 1), (5, 33), (2, 513), (1, 17408)]:
+        x = (rng.standard_normal((rows, d)) * 3).astype(np.float32)
+        y = rng.standard_normal((rows, d)).astype(np.float32)
+        w = rng.standard_normal(d).astype(np.float32)
+        xt, yt, wt = F.Tensor.from_vec(x, (rows, d)), F.Tensor.from_vec(y, (rows, d)), F.Tensor.from_vec(w, (d,))
+        assert close(X.rmsnorm(xt, wt, 1e-6).to_vec(), D.rmsnorm(x, w, 1e-6), 2e-6), (rows, d)
+        s, n = X.add_rmsnorm(xt, yt, wt, 1e-5)
+        so, no = D.add_rmsnorm(x, y, w, 1e-5)
+        assert np.array_equal(bits(s.to_vec()), bits(so.reshape(-1))), (rows, d)       # the next residual: exact f32 a + b
+        assert close(n.to_vec(), no, 2e-6), (rows, d)
+        assert np.array_equal(bits(X.add(xt, yt).to_vec()), bits((x + y).reshape(-1)))
+    # the residual updated in place (sum written over a)
+    lib = __import__("ferric_amd")._lib.load()
+    a = F.Tensor.from_vec(x, x.shape); nrm = F.Tensor.empty(x.shape)
+    F._lib.check(lib.fhip_add_rmsnorm(a.buf.ptr, yt.buf.ptr, wt.buf.ptr, x.shape[0], x.shape[1], 1e-5, a.buf.ptr, nrm.buf.ptr, None))
+    assert np.array_equal(bits(a.to_vec()), bits(so.reshape(-1))) and close(nrm.to_vec(), no, 2e-6)
+    zero = X.rmsnorm(F.Tensor.from_vec(np.zeros((2, 64), np.float32), (2, 64)), F.Tensor.from_vec(np.ones(64, np.float32), (64,)), 1e-6)
+    assert not zero.to_vec().any()
+    with pytest.raises(AssertionError, match="shape mismatch"):
+        X.add_rmsnorm(xt, F.Tensor.from_vec(np.zeros(4, np.float32), (1, 4)), wt, 1e-5)
+
+
+def test_rope_variants(F, X, D):
+    rng = np.random.default_rng(1)
+    for t, heads, hd, base, off in [(1, 40, 128, 1e6, 0), (1, 48, 128, 1e6, 4095), (5, 8, 64, 1e4, 129), (3, 2, 8, 1e4, 7), (2, 3, 256, 5e5, 31999)]:
+        x = rng.standard_normal((t, heads * hd)).astype(np.float32)
+        xt = F.Tensor.from_vec(x, x.shape)
+        pos = [off + i for i in range(t)]
+        # |error| <= 2e-6 of the largest magnitude: sin / cos of the same f32 angle to a few ulp, three roundings per output
+        assert close(X.rope(xt, heads, hd, base, off).to_vec(), D.rope(x, heads, hd, base, pos), 2e-6), (t, heads, hd)
+        assert close(X.rope(xt, heads, hd, base, off, interleaved=True).to_vec(), D.rope(x, heads, hd, base, pos, interleaved=True), 2e-6)
+        scattered = [int(p) for p in rng.integers(0, 40000, t)]
+        assert close(X.rope(xt, heads, hd, base, positions=scattered).to_vec(), D.rope(x, heads, hd, base, scattered), 2e-6)
+        fs = (rng.random(hd // 2) + 0.5).astype(np.float32)
+        got = X.rope(xt, heads, hd, base, positions=scattered, freq_scale=F.Tensor.from_vec(fs, fs.shape), interleaved=True).to_vec()
+        assert close(got, D.rope(x, heads, hd, base, scattered, interleaved=True, freq_scale=fs), 2e-6)
+        n_rot = hd // 2 + (hd // 2) % 2
+        part = X.rope(xt, heads, hd, base, off, n_rot=n_rot).to_vec().reshape(t, heads, hd)
+        assert close(part, D.rope(x, heads, hd, base, pos, n_rot=n_rot).reshape(t, heads, hd), 2e-6)
+        assert np.array_equal(bits(part[:, :, n_rot:]), bits(x.reshape(t, heads, hd)[:, :, n_rot:]))   # the tail is a copy
+    assert np.array_equal(bits(X.rope(xt, heads, hd, base, 0, positions=[0] * t).to_vec()), bits(x.reshape(-1)))   # position 0: identity
+    with pytest.raises(AssertionError, match="n_rot must be even"):
+        X.rope(xt, heads, hd, base, 0, n_rot=3)
+    with pytest.raises(AssertionError, match="one position per row"):
+        X.rope(xt, heads, hd, base, positions=[1] * (t + 1))
+    # a strided window (the q|k span of a fused qkv row) read in place
+    lib = F._lib.load()
+    t, nh, nkv, hd = 3, 4, 2, 64
+    qkv = rng.standard_normal((t, (nh + 2 * nkv) * hd)).astype(np.float32)
+    qt = F.Tensor.from_vec(qkv, qkv.shape)
+    out = F.Tensor.empty((t, (nh + nkv) * hd))
+    F._lib.check(lib.fhip_rope(qt.buf.ptr, (nh + 2 * nkv) * hd, t, nh + nkv, hd, hd, 1e6, None, 11, None, 0, out.buf.ptr, None))
+    assert close(out.to_vec(), D.rope(qkv[:, :(nh + nkv) * hd], nh + nkv, hd, 1e6, [11, 12, 13]), 2e-6)
+
+
+def test_kv_append2_and_decode_attention(F, X, D):
+    rng = np.random.default_rng(2)
+    for nh, nkv, hd, lens in [(40, 8, 128, [1, 7, 64, 65, 1000]), (8, 8, 64, [3, 257]), (16, 2, 128, [130]), (6, 2, 64, [33]), (5, 1, 128, [2049]),
+                              (64, 8, 128, [4097])]:
+        cap = max(lens) + 3
+        width = nkv * hd
+        k = rng.standard_normal((cap, width)).astype(np.float32)
+        v = rng.standard_normal((cap, width)).astype(np.float32)
+        k[:, :hd] *= 4.0                                      # one KV head with peaky scores
+        cache = X.KvCache(cap, width)
+        cache.append2(F.Tensor.from_vec(k[:5], (5, width)), F.Tensor.from_vec(v[:5], (5, width)))
+        cache.append2(F.Tensor.from_vec(k[5:], (cap - 5, width)), F.Tensor.from_vec(v[5:], (cap - 5, width)))
+        assert cache.len == cap and np.array_equal(bits(cache.k.to_vec()), bits(k.reshape(-1))) and np.array_equal(bits(cache.v.to_vec()), bits(v.reshape(-1)))
+        q = rng.standard_normal((1, nh * hd)).astype(np.float32)
+        qt = F.Tensor.from_vec(q, q.shape)
+        for s in lens:
+            want = D.decode_attention(q[0], k[:s], v[:s], nh, nkv)
+            got = X.decode_attention(qt, cache, nh, nkv, length=s).to_vec()
+            # <= 1e-5 of the largest value: f32 dots of head_dim terms, expf to a few ulp, sums over s keys in f32
+            assert close(got, want, 1e-5), (nh, nkv, hd, s)
+            # the length read on the device (newest row = s - 1) under a launch sized for the whole cache
+            last = X._u32_tensor([s - 1])
+            got2 = X.decode_attention(qt, cache, nh, nkv, length=cap, last_pos=last).to_vec()
+            assert close(got2, want, 1e-5), (nh, nkv, hd, s, "device length")
+    with pytest.raises(AssertionError, match="exceed the capacity"):
+        cache.append2(F.Tensor.from_vec(k[:1], (1, width)), F.Tensor.from_vec(v[:1], (1, width)))
+    with pytest.raises(AssertionError, match="head_dim must be 64 or 128"):
+        X.decode_attention(F.Tensor.from_vec(np.zeros((1, 96), np.float32), (1, 96)), X.KvCache(4, 96), 1, 1, length=1)
+    with pytest.raises(AssertionError, match="1..=8 supported"):
+        X.decode_attention(F.Tensor.from_vec(np.zeros((1, 9 * 64), np.float32), (1, 9 * 64)), X.KvCache(4, 64), 9, 1, length=1)
+
+
+def test_qkv_post_fuses_bias_norm_rope_and_append(F, X, D):
+    rng = np.random.default_rng(3)
+    lib = F._lib.load()
+    for nh, nkv, hd, t, use_bias, use_norm, inter in [(40, 8, 128, 1, False, True, False), (4, 2, 64, 3, True, False, False),
+                                                      (6, 3, 128, 2, True, True, True), (2, 1, 32, 2, False, False, False)]:
+        width = (nh + 2 * nkv) * hd
+        qkv = rng.standard_normal((t, width)).astype(np.float32)
+        bias = rng.standard_normal(width).astype(np.float32) if use_bias else None
+        qn = (rng.random(hd) + 0.5).astype(np.float32) if use_norm else None
+        kn = (rng.random(hd) + 0.5).astype(np.float32) if use_norm else None
+        pos = [int(p) for p in rng.choice(60, t, replace=False)]
+        cap = 64
+        kc0, vc0 = rng.standard_normal((cap, nkv * hd)).astype(np.float32), rng.standard_normal((cap, nkv * hd)).astype(np.float32)
+        kc, vc = F.Tensor.from_vec(kc0, kc0.shape), F.Tensor.from_vec(vc0, vc0.shape)
+        T = lambda a: F.Tensor.from_vec(a, a.shape) if a is not None else None
+        qt, bt, qnt, knt, pt = T(qkv), T(bias), T(qn), T(kn), X._u32_tensor(pos)
+        qo = F.Tensor.empty((t, nh * hd))
+        P = lambda x: x.buf.ptr if x is not None else None
+        F._lib.check(lib.fhip_qkv_post(qt.buf.ptr, P(bt), P(qnt), P(knt), pt.buf.ptr, None, t, nh, nkv, hd, hd, int(inter), 1e-6, 1e6,
+                                       qo.buf.ptr, kc.buf.ptr, vc.buf.ptr, cap, None))
+        wq, wk, wv = D.qkv_post(qkv, bias, qn, kn, pos, nh, nkv, hd, 1e-6, 1e6, interleaved=inter)
+        assert close(qo.to_vec(), wq, 3e-6), (nh, nkv, hd)
+        kg, vg = kc.to_vec().reshape(cap, -1), vc.to_vec().reshape(cap, -1)
+        assert close(kg[pos], wk, 3e-6)
+        assert np.array_equal(bits(vg[pos]), bits(wv.astype(np.float32)))                   # values are copied (+ bias: one f32 add)
+        rest = [r for r in range(cap) if r not in pos]
+        assert np.array_equal(bits(kg[rest]), bits(kc0[rest])) and np.array_equal(bits(vg[rest]), bits(vc0[rest]))   # no other row touched
+    # a position past the capacity leaves the caches alone (and still produces the query)
+    pt = X._u32_tensor([cap + 5] * t)
+    kc, vc = F.Tensor.from_vec(kc0, kc0.shape), F.Tensor.from_vec(vc0, vc0.shape)
+    F._lib.check(lib.fhip_qkv_post(qt.buf.ptr, None, None, None, pt.buf.ptr, None, t, nh, nkv, hd, hd, 0, 1e-6, 1e6, qo.buf.ptr, kc.buf.ptr,
+                                   vc.buf.ptr, cap, None))
+    assert np.array_equal(bits(kc.to_vec()), bits(kc0.reshape(-1))) and np.array_equal(bits(vc.to_vec()), bits(vc0.reshape(-1)))
+
+
+def _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, qk_norm):
+    """Random Q4_K / Q6_K projections (synthetic blocks have rows of norm ~ 2 sqrt(cols)), block norms small enough that the
+    projections of a normalised vector are O(1); the f64 twin holds the oracle-dequantized weights."""
+    from ferric_amd.synth import synth_weights
+    from oracle import decode_oracle as D
+    layers, olayers = [], []
+    T = lambda a: F.Tensor.from_vec(a, a.shape)
+    for il in range(n_layer):
+        shapes = {"wqkv": (Q4_K, (nh + 2 * nkv) * hd, d), "wo": (Q4_K, d, nh * hd), "gate_up": (Q4_K, 2 * n_ff, d), "down": (Q6_K, d, n_ff)}
+        qm, deq = {}, {}
+        for name, (ty, r, c) in shapes.items():
+            b = synth_weights(ty, r, c, 100 * il + len(qm))
+            qm[name] = F.QMatrix.from_bytes(b, ty, r, c)
+            deq[name] = O.deq_raw(b, r * c, ty).reshape(r, c).astype(np.float64)
+        norms = {"attn_norm": ((rng.random(d) + 0.5) * 0.02).astype(np.float32), "ffn_norm": ((rng.random(d) + 0.5) * 0.02).astype(np.float32),
+                 "q_norm": (rng.random(hd) + 0.5).astype(np.float32), "k_norm": (rng.random(hd) + 0.5).astype(np.float32)}
+        layers.append(X.Qwen3Layer(T(norms["attn_norm"]), qm["wqkv"], qm["wo"], T(norms["ffn_norm"]), qm["gate_up"], qm["down"],
+                                   T(norms["q_norm"]) if qk_norm else None, T(norms["k_norm"]) if qk_norm else None))
+        olayers.append(D.Layer(attn_norm=norms["attn_norm"], ffn_norm=norms["ffn_norm"], q_norm=norms["q_norm"] if qk_norm else None,
+                               k_norm=norms["k_norm"] if qk_norm else None, wqkv=deq["wqkv"], wo=deq["wo"], gate_up=deq["gate_up"], down=deq["down"]))
+    return layers, olayers
+
+
+@pytest.mark.parametrize("qk_norm", [True, False])
+def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, X, O, D, qk_norm):
+    rng = np.random.default_rng(4)
+    n_layer, d, nh, nkv, hd, n_ff, steps = 3, 1024, 8, 2, 128, 1536, 6
+    cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6)
+    layers, olayers = _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, qk_norm)
+    xs = (rng.standard_normal((steps, d)) * 0.5).astype(np.float32)
+    # oracle: f64 on the dequantized weights, token by token
+    kcs, vcs = [[] for _ in olayers], [[] for _ in olayers]
+    want = []
+    for pos in range(steps):
+        x = xs[pos].astype(np.float64)
+        for l, kc, vc in zip(olayers, kcs, vcs):
+            x = D.apply_layer(x, l, kc, vc, pos, cfg)
+        want.append(x)
+    stream = F.Stream()
+    dec = X.Qwen3Decoder(cfg, layers, max_len=steps + 2, stream=stream)
+    eager = []
+    for pos in range(steps):
+        dec.set_input(xs[pos])
+        dec.step()
+        eager.append(dec.hidden())
+        # <= 2e-4 of the largest hidden value: three layers of quantized dots (each within 1e-5 of its largest output)
+        # feeding norms, attention and the next projections
+        assert close(eager[-1], want[pos], 2e-4), pos
+    assert dec.caches[0].len == steps
+    # the same steps as one captured graph, replayed with host work and synchronisation between replays
+    dec.set_pos(0)
+    dec.capture()
+    for pos in range(steps):
+        dec.set_input(xs[pos])
+        dec.step_graph()
+        got = dec.hidden()
+        assert np.array_equal(bits(got), bits(eager[pos])), pos        # same launches, same order: bit-identical to eager
+    pos_word = np.empty(1, np.uint32)
+    F._lib.check(F._lib.load().fhip_memcpy_d2h(pos_word.ctypes.data, dec.pos.buf.ptr, 4, stream.handle))
+    assert pos_word[0] == steps
+    # with the output norm and LM head in the step: logits = rmsnorm(hidden) W_out^T
+    from ferric_amd.synth import synth_weights
+    head_raw = synth_weights(Q6_K, 300, d, 77)
+    onorm = ((rng.random(d) + 0.5) * 0.02).astype(np.float32)
+    dec2 = X.Qwen3Decoder(cfg, layers, max_len=4, stream=stream, output_norm=F.Tensor.from_vec(onorm, onorm.shape),
+                          lm_head=F.QMatrix.from_bytes(head_raw, Q6_K, 300, d))
+    dec2.set_input(xs[0])
+    dec2.step()
+    assert np.array_equal(bits(dec2.hidden()), bits(eager[0]))
+    head = O.deq_raw(head_raw, 300 * d, Q6_K).reshape(300, d).astype(np.float64)
+    assert close(dec2.logits.to_vec(stream), D.rmsnorm(want[0], onorm, 1e-6) @ head.T, 2e-4)
