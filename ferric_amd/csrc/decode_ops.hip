@@ -12,6 +12,7 @@
 #include "common.hpp"
 
 #include <math.h>
+#include <stdlib.h>
 
 namespace {
 
@@ -39,16 +40,53 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* a, const floa
                                                       const float* __restrict__ weight, size_t rows, int d, float eps,
                                                       float* sum_out, float* __restrict__ norm_out) {   // sum_out may be a
     constexpr int RPW = 256 / TPR;   // rows per workgroup
+    constexpr int NV = 8;            // float4 per thread held in registers: rows up to 4 * NV * TPR values
     __shared__ float red[4];
     const int tid = threadIdx.x, sub = tid / TPR, t = tid % TPR;
     const size_t row = (size_t)blockIdx.x * RPW + sub;
     const bool live = row < rows;
-    const float* xa = a + (live ? row : 0) * (size_t)d;
-    const float* xb = b ? b + (live ? row : 0) * (size_t)d : nullptr;
+    const size_t base = (live ? row : 0) * (size_t)d;
+    const bool vec = (d & 3) == 0 && d <= 4 * NV * TPR && (((uintptr_t)a | (uintptr_t)b | (uintptr_t)weight | (uintptr_t)sum_out | (uintptr_t)norm_out) & 15) == 0;
     float ms = 0.f;
+    if (vec) {
+        // every load of the row is issued before the first use, so the row costs one memory round trip, not one per element
+        const int nv = d >> 2;
+        float4 r[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int j = t + i * TPR;
+            r[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (j < nv) {
+                r[i] = ((const float4*)(a + base))[j];
+                if (b) { const float4 y = ((const float4*)(b + base))[j]; r[i].x += y.x; r[i].y += y.y; r[i].z += y.z; r[i].w += y.w; }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NV; i++) ms = fmaf(r[i].x, r[i].x, fmaf(r[i].y, r[i].y, fmaf(r[i].z, r[i].z, fmaf(r[i].w, r[i].w, ms))));
+        ms = wave_sum(ms);
+        if (TPR == 256) {
+            if ((tid & 63) == 0) red[tid >> 6] = ms;
+            __syncthreads();
+            ms = (red[0] + red[1]) + (red[2] + red[3]);
+        }
+        const float inv = 1.0f / sqrtf(ms / (float)d + eps);
+        if (!live) return;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int j = t + i * TPR;
+            if (j < nv) {
+                const float4 w = ((const float4*)weight)[j];
+                if (sum_out) ((float4*)(sum_out + base))[j] = r[i];
+                ((float4*)(norm_out + base))[j] = make_float4(r[i].x * inv * w.x, r[i].y * inv * w.y, r[i].z * inv * w.z, r[i].w * inv * w.w);
+            }
+        }
+        return;
+    }
+    const float* xa = a + base;
+    const float* xb = b ? b + base : nullptr;
     for (int j = t; j < d; j += TPR) {
         float v = xb ? xa[j] + xb[j] : xa[j];
-        if (sum_out && live) sum_out[row * (size_t)d + j] = v;
+        if (sum_out && live) sum_out[base + j] = v;
         ms = fmaf(v, v, ms);
     }
     ms = wave_sum(ms);
@@ -60,8 +98,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* a, const floa
     const float inv = 1.0f / sqrtf(ms / (float)d + eps);
     if (!live) return;
     for (int j = t; j < d; j += TPR) {   // the same thread wrote sum_out[.., j] above, so reading it back is ordered
-        float v = sum_out ? sum_out[row * (size_t)d + j] : (xb ? xa[j] + xb[j] : xa[j]);
-        norm_out[row * (size_t)d + j] = v * inv * weight[j];
+        float v = sum_out ? sum_out[base + j] : (xb ? xa[j] + xb[j] : xa[j]);
+        norm_out[base + j] = v * inv * weight[j];
     }
 }
 
@@ -182,89 +220,112 @@ __global__ void kv_append_kernel(const float* __restrict__ k, const float* __res
 
 // ---------------------------------------------------------------- single-query attention over the cache
 // out[h] = softmax_j(q[h] . K[j, kv(h)] * scale) @ V[:, kv(h)]   for one query row (nn.rs:140-166, lib.rs:2675-2726).
-// Workgroup (kv head, split): its 4 waves walk the split's keys in blocks of KB; a lane holds DPL = hd / 64 consecutive
-// dims of a row, so one key or value row is one coalesced wave load, read ONCE for all G = n_head / n_kv query heads of the
-// group. Running (max, sum, accumulator) per query head, merged across the waves through LDS and across splits by
-// attn_combine_kernel -- the reference's own rescale exp(m_old - m_new), applied across partitions.
-constexpr int ATT_KB = 8;
+// Workgroup (kv head, split). A key or value row is read by 16 lanes (DPL = hd / 16 consecutive dims each, 16-byte loads), so a
+// wave works on 4 keys at a time and a workgroup is 16 independent key streams, each with its own running (max, sum,
+// accumulator) per query head -- the reference's online softmax, lib.rs:2697-2722 -- over keys taken round-robin in pairs.
+// Every row is read ONCE for all G = n_head / n_kv query heads of the group. A dot product is reduced inside its 16-lane
+// row with 4 DPP adds. The 4 streams of a wave are merged by lane exchange, the 4 waves through LDS, the splits by
+// attn_combine_kernel: always the same rescale, exp(m_part - m_all).
+constexpr int ATT_KB = 2;         // keys in flight per stream
+constexpr int ATT_STREAMS = 16;   // per workgroup of 256 threads
+
+__device__ __forceinline__ float row16_sum(float v) {   // all 16 lanes of a DPP row get the row's sum
+    v = dpp_add<0xB1, 0xF>(v);
+    v = dpp_add<0x4E, 0xF>(v);
+    v = dpp_add<0x141, 0xF>(v);
+    v = dpp_add<0x140, 0xF>(v);
+    return v;
+}
 
 template <int DPL>
-__device__ __forceinline__ void load_dims(const float* p, float (&r)[DPL]) {   // p is 4 * DPL-byte aligned
-    if constexpr (DPL == 2) { float2 v = *(const float2*)p; r[0] = v.x; r[1] = v.y; }
-    else { r[0] = *p; }
+__device__ __forceinline__ void load_dims(const float* p, float (&r)[DPL]) {   // p is 16-byte aligned
+#pragma unroll
+    for (int i = 0; i < DPL; i += 4) {
+        float4 v = *(const float4*)(p + i);
+        r[i] = v.x; r[i + 1] = v.y; r[i + 2] = v.z; r[i + 3] = v.w;
+    }
 }
 
 template <int G, int DPL>
 __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict__ q, const float* __restrict__ K, const float* __restrict__ V,
                                                          int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
                                                          float* __restrict__ part, float* __restrict__ out) {
-    constexpr int HD = 64 * DPL;
+    constexpr int HD = 16 * DPL;
     __shared__ float sm_m[4][G], sm_l[4][G];
     __shared__ float sm_acc[4][G][HD];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15;
+    const int sid = wave * 4 + (lane >> 4);
     const int kvh = blockIdx.x, split = blockIdx.y;
     uint32_t len = len_dev ? *len_dev + 1u : len_host;   // the device word is the newest token's position
     if (len > len_host) len = len_host;
     const uint32_t per = (len + splits - 1) / splits;
     const uint32_t k0 = (uint32_t)split * per, k1 = min(len, k0 + per);
     const size_t stride = (size_t)n_kv * HD;
-    const float* Kb = K + (size_t)kvh * HD + lane * DPL;
-    const float* Vb = V + (size_t)kvh * HD + lane * DPL;
+    const float* Kb = K + (size_t)kvh * HD + sub * DPL;
+    const float* Vb = V + (size_t)kvh * HD + sub * DPL;
 
     float qr[G][DPL], acc[G][DPL], m[G], l[G];
 #pragma unroll
     for (int h = 0; h < G; h++) {
         m[h] = -3.0e38f; l[h] = 0.f;
+        load_dims<DPL>(q + ((size_t)kvh * G + h) * HD + sub * DPL, qr[h]);
 #pragma unroll
-        for (int i = 0; i < DPL; i++) { qr[h][i] = q[((size_t)kvh * G + h) * HD + lane * DPL + i]; acc[h][i] = 0.f; }
+        for (int i = 0; i < DPL; i++) acc[h][i] = 0.f;
     }
-    for (uint32_t kb = k0 + wave * ATT_KB; kb < k1; kb += 4 * ATT_KB) {
+    for (uint32_t kb = k0 + sid * ATT_KB; kb < k1; kb += ATT_STREAMS * ATT_KB) {
         float kr[ATT_KB][DPL], vr[ATT_KB][DPL];
 #pragma unroll
         for (int j = 0; j < ATT_KB; j++) {
-            const uint32_t key = min(kb + j, k1 - 1);   // rows past the split re-read its last row and are masked below
+            const uint32_t key = min(kb + j, k1 - 1);   // a row past the split re-reads its last row and is masked below
             load_dims<DPL>(Kb + key * stride, kr[j]);
             load_dims<DPL>(Vb + key * stride, vr[j]);
         }
-        float s[G][ATT_KB];
 #pragma unroll
-        for (int h = 0; h < G; h++)
+        for (int h = 0; h < G; h++) {
+            float sc[ATT_KB];
 #pragma unroll
             for (int j = 0; j < ATT_KB; j++) {
                 float d = 0.f;
 #pragma unroll
                 for (int i = 0; i < DPL; i++) d = fmaf(qr[h][i], kr[j][i], d);
-                const float r = wave_sum(d) * scale;
-                s[h][j] = (kb + j < k1) ? r : -3.0e38f;
+                d = row16_sum(d) * scale;
+                sc[j] = (kb + j < k1) ? d : -3.0e38f;
             }
+            float m_new = m[h];
 #pragma unroll
-        for (int h = 0; h < G; h++) {
-            float bm = s[h][0];
+            for (int j = 0; j < ATT_KB; j++) m_new = fmaxf(m_new, sc[j]);
+            const float corr = __expf(m[h] - m_new);
+            float e[ATT_KB], ps = 0.f;
 #pragma unroll
-            for (int j = 1; j < ATT_KB; j++) bm = fmaxf(bm, s[h][j]);
-            const float m_new = fmaxf(m[h], bm), corr = expf(m[h] - m_new);
-            float ps = 0.f, a[DPL];
+            for (int j = 0; j < ATT_KB; j++) { e[j] = (kb + j < k1) ? __expf(sc[j] - m_new) : 0.f; ps += e[j]; }
+            l[h] = fmaf(l[h], corr, ps);
 #pragma unroll
-            for (int i = 0; i < DPL; i++) a[i] = 0.f;
+            for (int i = 0; i < DPL; i++) {
+                float a = acc[h][i] * corr;
 #pragma unroll
-            for (int j = 0; j < ATT_KB; j++) {
-                const float e = (kb + j < k1) ? expf(s[h][j] - m_new) : 0.f;
-                ps += e;
-#pragma unroll
-                for (int i = 0; i < DPL; i++) a[i] = fmaf(e, vr[j][i], a[i]);
+                for (int j = 0; j < ATT_KB; j++) a = fmaf(e[j], vr[j][i], a);
+                acc[h][i] = a;
             }
-            l[h] = l[h] * corr + ps;
-#pragma unroll
-            for (int i = 0; i < DPL; i++) acc[h][i] = acc[h][i] * corr + a[i];
             m[h] = m_new;
         }
     }
-    // merge the four waves
+    // merge the wave's four streams (rows of 16 lanes) by exchange with lanes ^16 and ^32
 #pragma unroll
     for (int h = 0; h < G; h++) {
-        if (lane == 0) { sm_m[wave][h] = m[h]; sm_l[wave][h] = l[h]; }
+        float M = fmaxf(m[h], __shfl_xor(m[h], 16));
+        M = fmaxf(M, __shfl_xor(M, 32));
+        const float f = __expf(m[h] - M);
+        float lv = l[h] * f;
+        lv += __shfl_xor(lv, 16);
+        lv += __shfl_xor(lv, 32);
 #pragma unroll
-        for (int i = 0; i < DPL; i++) sm_acc[wave][h][lane * DPL + i] = acc[h][i];
+        for (int i = 0; i < DPL; i++) {
+            float a = acc[h][i] * f;
+            a += __shfl_xor(a, 16);
+            a += __shfl_xor(a, 32);
+            if (lane < 16) sm_acc[wave][h][sub * DPL + i] = a;
+        }
+        if (lane == 0) { sm_m[wave][h] = M; sm_l[wave][h] = lv; }
     }
     __syncthreads();
     for (int idx = threadIdx.x; idx < G * HD; idx += 256) {
@@ -273,7 +334,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
         float L = 0.f, A = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            const float f = expf(sm_m[w][h] - M);
+            const float f = __expf(sm_m[w][h] - M);
             L = fmaf(sm_l[w][h], f, L);
             A = fmaf(sm_acc[w][h][d], f, A);
         }
@@ -288,26 +349,35 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
     }
 }
 
-__global__ void attn_combine_kernel(const float* __restrict__ part, int hd, int splits, float* __restrict__ out) {
-    const int head = blockIdx.x;
+// One workgroup per query head: weights exp(m_s - max m) of the splits once (through LDS), then every output dim is a
+// weighted sum of the splits' accumulators over the weighted sum of their sums. splits <= 256.
+__global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restrict__ part, int hd, int splits, float* __restrict__ out) {
+    __shared__ float w[256], lw[256];
+    const int head = blockIdx.x, tid = threadIdx.x;
     const float* pp = part + (size_t)head * splits * (hd + 2);
+    for (int s = tid; s < splits; s += 128) { w[s] = pp[(size_t)s * (hd + 2) + hd]; lw[s] = pp[(size_t)s * (hd + 2) + hd + 1]; }
+    __syncthreads();
     float M = -3.0e38f;
-    for (int s = 0; s < splits; s++) M = fmaxf(M, pp[(size_t)s * (hd + 2) + hd]);
+    for (int s = 0; s < splits; s++) M = fmaxf(M, w[s]);
+    __syncthreads();
+    for (int s = tid; s < splits; s += 128) { const float f = __expf(w[s] - M); w[s] = f; lw[s] *= f; }
+    __syncthreads();
     float L = 0.f;
-    for (int s = 0; s < splits; s++) L = fmaf(pp[(size_t)s * (hd + 2) + hd + 1], expf(pp[(size_t)s * (hd + 2) + hd] - M), L);
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    for (int s = 0; s < splits; s++) L += lw[s];
+    for (int d = tid; d < hd; d += 128) {
         float A = 0.f;
-        for (int s = 0; s < splits; s++) A = fmaf(pp[(size_t)s * (hd + 2) + d], expf(pp[(size_t)s * (hd + 2) + hd] - M), A);
+#pragma unroll 8
+        for (int s = 0; s < splits; s++) A = fmaf(pp[(size_t)s * (hd + 2) + d], w[s], A);
         out[(size_t)head * hd + d] = A / L;
     }
 }
 
 template <int G>
-int launch_attn_g(int dpl, dim3 grid, hipStream_t s, const float* q, const float* K, const float* V, int n_kv, uint32_t len, const uint32_t* d_len,
+int launch_attn_g(int hd, dim3 grid, hipStream_t s, const float* q, const float* K, const float* V, int n_kv, uint32_t len, const uint32_t* d_len,
                   float scale, int splits, float* part, float* out) {
-    switch (dpl) {
-        case 1: hipLaunchKernelGGL((attn_split_kernel<G, 1>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
-        case 2: hipLaunchKernelGGL((attn_split_kernel<G, 2>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
+    switch (hd) {
+        case 64: hipLaunchKernelGGL((attn_split_kernel<G, 4>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
+        case 128: hipLaunchKernelGGL((attn_split_kernel<G, 8>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
         default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     }
     return FHIP_OK;
@@ -382,13 +452,15 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
     return check_hip(hipGetLastError(), "kv_append launch");
 }
 
-// Splits of the key range: enough workgroups to cover the chip once, at least 64 keys each.
+// Splits of the key range: about two workgroups per CU over all KV heads, at least `keys` keys each (FHIP_ATTN_KEYS, default 64:
+// two rounds of the workgroup's 16 streams x 2 keys), at most 256 (the combine kernel's LDS tables).
 int attn_splits(size_t len, int n_kv) {
     if (n_kv <= 0 || len == 0) return 1;
-    int want = (device_cus() + n_kv - 1) / n_kv;
-    size_t by_keys = (len + 63) / 64;
+    static const int keys = [] { const char* e = getenv("FHIP_ATTN_KEYS"); int v = e ? atoi(e) : 64; return v < 1 ? 64 : v; }();
+    int want = (2 * device_cus() + n_kv - 1) / n_kv;
+    size_t by_keys = (len + keys - 1) / keys;
     int splits = (int)(by_keys < (size_t)want ? by_keys : (size_t)want);
-    return splits < 1 ? 1 : splits;
+    return splits < 1 ? 1 : (splits > 256 ? 256 : splits);
 }
 
 int launch_decode_attention(const float* q, const float* K, const float* V, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len,
@@ -404,14 +476,14 @@ int launch_decode_attention(const float* q, const float* K, const float* V, int 
     dim3 grid((unsigned)n_kv, (unsigned)splits);
     int rc;
     switch (g) {
-        case 1: rc = launch_attn_g<1>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 2: rc = launch_attn_g<2>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 3: rc = launch_attn_g<3>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 4: rc = launch_attn_g<4>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 5: rc = launch_attn_g<5>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 6: rc = launch_attn_g<6>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 7: rc = launch_attn_g<7>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 8: rc = launch_attn_g<8>(hd / 64, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 1: rc = launch_attn_g<1>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 2: rc = launch_attn_g<2>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 3: rc = launch_attn_g<3>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 4: rc = launch_attn_g<4>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 5: rc = launch_attn_g<5>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 6: rc = launch_attn_g<6>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 7: rc = launch_attn_g<7>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 8: rc = launch_attn_g<8>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
         default: return set_error(FHIP_ERR_SHAPE, "decode_attention: %d query heads per KV head (1..=8 supported)", g);
     }
     if (rc) return rc;
