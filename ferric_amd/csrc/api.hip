@@ -454,6 +454,24 @@ int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float*
                                          (hipStream_t)stream);
 }
 
+int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_resid, const float* d_norm_w, float eps, float* d_x_out,
+                       float* d_h_scratch, int swiglu, float* d_y, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!w || !d_x || !d_norm_w || !d_h_scratch || !d_y) return set_error(FHIP_ERR_ARG, "fhip_norm_matmul_q: NULL pointer");
+    if (d_x_out && d_x_out == d_x) return set_error(FHIP_ERR_ARG, "fhip_norm_matmul_q: x_out must not be x");
+    if (swiglu && (w->type == FHIP_Q8_0 || w->rows % 2 != 0))
+        return set_error(w->type == FHIP_Q8_0 ? FHIP_ERR_UNSUPPORTED_TYPE : FHIP_ERR_SHAPE, "fhip_norm_matmul_q: no fused SwiGLU for this weight");
+    if (((uintptr_t)d_x | (uintptr_t)d_resid | (uintptr_t)d_norm_w | (uintptr_t)d_x_out) & 15)
+        return set_error(FHIP_ERR_ARG, "fhip_norm_matmul_q: x, resid, norm_w and x_out must be 16-byte aligned");
+    const size_t n_ff = swiglu ? w->rows / 2 : 0;
+    fhip::NormParams np{d_norm_w, d_resid, d_resid ? d_x_out : nullptr, eps};   // without a residual there is no sum to store
+    rc = fhip::launch_gemv_norm(w, d_x, d_y, n_ff, np, (hipStream_t)stream);
+    if (rc != fhip::NORM_NOT_FUSED) return rc;
+    if ((rc = fhip::launch_rmsnorm(d_x, d_resid, d_norm_w, 1, w->cols, eps, d_resid ? d_x_out : nullptr, d_h_scratch, (hipStream_t)stream))) return rc;
+    return fhip::launch_gemv(w, d_h_scratch, 1, d_y, n_ff, (hipStream_t)stream);
+}
+
 int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream) {
     int rc = need_init();
     if (rc) return rc;

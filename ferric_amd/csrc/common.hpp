@@ -45,6 +45,16 @@ __device__ __forceinline__ void apply_selection(P& p) {
     }
 }
 
+// Input norm fused into a batch-1 mat-vec: the activation row is rmsnorm(x [+ resid]) * norm_w; x + resid goes to x_out
+// (optional, must not be x).
+struct NormParams {
+    const float* norm_w;
+    const float* resid;
+    float* x_out;
+    float eps;
+};
+constexpr int NORM_NOT_FUSED = -100;   // internal: launch_gemv_norm launched nothing, run the two steps apart
+
 int set_error(int code, const char* fmt, ...);
 int check_hip(hipError_t e, const char* what);
 int device_cus();
@@ -63,6 +73,7 @@ int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, f
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s);
 // One batch-1 GEMV per (token, slot) pair on the selected expert's `out_rows` rows (fused SwiGLU over its
 // gate|up halves when swiglu: then expert_rows = 2 * out_rows). Both files provide it, same contract as above.
+int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s);
 int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel,
                     hipStream_t s);
 int launch_gemv_generic_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu,

@@ -277,6 +277,13 @@ struct GemvParams {
     int G;               // row groups per workgroup
     int rpg;             // output rows per row group
     fhip::SelParams sel; // expert selection (selw == nullptr: none)
+    // Fused input norm (norm_w != nullptr; M = 1, cols <= 8 * threads): the activation row is rmsnorm(x [+ resid]) * norm_w,
+    // formed by every workgroup while it stages the row; workgroup 0 also stores x + resid to x_out (never x itself).
+    const float* norm_w;
+    const float* resid;
+    float* x_out;
+    float eps;
+    uint32_t red_off;    // byte offset in LDS of 16 floats for the workgroup's sum of squares
 };
 
 // Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 768 -> 168, 512 -> 256).
@@ -289,7 +296,7 @@ template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? (F::WPL
 // Activation rows one pass can hold in registers (48 plane dwords per row for the 64-weight units, 24 for Q8_0).
 template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
 
-template <class F, int M, int U, bool SWIGLU>
+template <class F, int M, int U, bool SWIGLU, bool NORM>
 __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     fhip::apply_selection(p);
@@ -347,10 +354,36 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     const int e0 = tid * 8;
     float4 xa0 = {0, 0, 0, 0}, xb0 = {0, 0, 0, 0};
     if (e0 < M * p.cols) { xa0 = *(const float4*)(p.x + e0); xb0 = *(const float4*)(p.x + e0 + 4); }
+    constexpr bool fused_norm = NORM && M == 1;   // a separate instantiation: the plain kernel carries none of this
+    float4 nwa = {1, 1, 1, 1}, nwb = {1, 1, 1, 1}, rsa = {0, 0, 0, 0}, rsb = {0, 0, 0, 0};
+    if (fused_norm && e0 < p.cols) {
+        nwa = *(const float4*)(p.norm_w + e0); nwb = *(const float4*)(p.norm_w + e0 + 4);
+        if (p.resid) { rsa = *(const float4*)(p.resid + e0); rsb = *(const float4*)(p.resid + e0 + 4); }
+    }
     typename F::Data buf[U];
 #pragma unroll
     for (int j = 0; j < U; j++)
         if (j < n_it) buf[j] = fetch(j);
+
+    if (fused_norm) {
+        // x <- rmsnorm(x + resid) * norm_w (crates/ferric-tensor/src/lib.rs:2057-2074): each thread holds at most one
+        // 8-value piece of the row (cols <= 8 * threads), so the row's sum of squares is one wave sum + one LDS round.
+        xa0.x += rsa.x; xa0.y += rsa.y; xa0.z += rsa.z; xa0.w += rsa.w;
+        xb0.x += rsb.x; xb0.y += rsb.y; xb0.z += rsb.z; xb0.w += rsb.w;
+        if (p.x_out && blockIdx.x == 0 && e0 < p.cols) { *(float4*)(p.x_out + e0) = xa0; *(float4*)(p.x_out + e0 + 4) = xb0; }
+        float ss = fmaf(xa0.x, xa0.x, fmaf(xa0.y, xa0.y, fmaf(xa0.z, xa0.z, xa0.w * xa0.w)))
+                 + fmaf(xb0.x, xb0.x, fmaf(xb0.y, xb0.y, fmaf(xb0.z, xb0.z, xb0.w * xb0.w)));
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        float* red = (float*)(smem + p.red_off);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+        for (int wv = 0; wv < (int)(blockDim.x >> 6); wv++) tot += red[wv];
+        const float ninv = 1.0f / sqrtf(tot / (float)p.cols + p.eps);
+        xa0.x = xa0.x * ninv * nwa.x; xa0.y = xa0.y * ninv * nwa.y; xa0.z = xa0.z * ninv * nwa.z; xa0.w = xa0.w * ninv * nwa.w;
+        xb0.x = xb0.x * ninv * nwb.x; xb0.y = xb0.y * ninv * nwb.y; xb0.z = xb0.z * ninv * nwb.z; xb0.w = xb0.w * ninv * nwb.w;
+    }
 
     // ---- activations -> 24-bit block fixed point, once per workgroup, through LDS
     constexpr float QMAX = F::SIGNED_W ? QMAX_S : QMAX_U;
@@ -530,15 +563,19 @@ size_t lds_bytes(size_t cols, int NG, int G, int rpg) {
 }
 
 template <class F, int M, bool SWIGLU>
-int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr) {
+int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr,
+               const fhip::NormParams* norm = nullptr) {
     static const int tune_g = env_int("FHIP_GEMV_G", 0), tune_rpg = env_int("FHIP_GEMV_RPG", 0);
     constexpr int U = rows_in_flight<F>(M);
-    auto kernel = gemv_stream_kernel<F, M, U, SWIGLU>;
-    static bool lds_raised = false;
-    if (!lds_raised) {  // workgroups may use more than the default 64 KiB of the CU's 160 KiB
+    void (*kernel)(GemvParams) = gemv_stream_kernel<F, M, U, SWIGLU, false>;
+    if constexpr (M == 1) {
+        if (norm) kernel = gemv_stream_kernel<F, M, U, SWIGLU, true>;
+    }
+    static bool lds_raised[2] = {false, false};
+    if (!lds_raised[norm ? 1 : 0]) {  // workgroups may use more than the default 64 KiB of the CU's 160 KiB
         (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fhip::device_lds_bytes());
         (void)hipGetLastError();
-        lds_raised = true;
+        lds_raised[norm ? 1 : 0] = true;
     }
     GemvParams p;
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
@@ -570,7 +607,15 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     p.G = G; p.rpg = rpg;
     const size_t per_wg = (size_t)G * rpg;
     const size_t grid = (out_rows + per_wg - 1) / per_wg;
-    const size_t lds = lds_bytes<F, M, SWIGLU>(w->cols, p.NG, G, rpg);
+    size_t lds = lds_bytes<F, M, SWIGLU>(w->cols, p.NG, G, rpg);
+    p.norm_w = nullptr; p.resid = nullptr; p.x_out = nullptr; p.eps = 0.f; p.red_off = 0;
+    if (norm) {
+        if (M != 1 || w->cols > (size_t)8 * 64 * WPR * G) return fhip::NORM_NOT_FUSED;   // nothing launched
+        p.norm_w = norm->norm_w; p.resid = norm->resid; p.x_out = norm->x_out; p.eps = norm->eps;
+        lds = (lds + 15) & ~(size_t)15;
+        p.red_off = (uint32_t)lds;
+        lds += 64;
+    }
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid, (unsigned)p.sel.npairs), dim3(64 * WPR * G), lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
 }
@@ -631,6 +676,26 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
         case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_Q5_K: case FHIP_IQ4_NL: case FHIP_IQ4_XS: case FHIP_MXFP4:
             return launch_gemv_generic(w, d_x, rows_x, d_y, n_ff, s);   // no streaming kernel for these formats
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
+    }
+}
+
+// One activation row with the input norm fused into its staging; NORM_NOT_FUSED (nothing launched) when this weight's
+// shape goes to the generic kernel or its row is longer than one pass of the workgroup.
+template <class F>
+int launch_norm_fmt(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const NormParams& norm, hipStream_t s) {
+    const bool covered = swiglu ? max_batch<F, true>(w, 1) != 0 : max_batch<F, false>(w, 1) != 0;
+    if (!covered) return NORM_NOT_FUSED;
+    return swiglu ? launch_one<F, 1, true>(w, d_x, d_y, out_rows, s, nullptr, &norm) : launch_one<F, 1, false>(w, d_x, d_y, out_rows, s, nullptr, &norm);
+}
+
+int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s) {
+    if (w->rows == 0 || w->cols == 0) return NORM_NOT_FUSED;
+    const size_t out_rows = n_ff ? n_ff : w->rows;
+    switch (w->type) {
+        case FHIP_Q4_K: return launch_norm_fmt<Q4K>(w, d_x, d_y, out_rows, n_ff != 0, norm, s);
+        case FHIP_Q6_K: return launch_norm_fmt<Q6K>(w, d_x, d_y, out_rows, n_ff != 0, norm, s);
+        case FHIP_Q8_0: return n_ff ? NORM_NOT_FUSED : launch_norm_fmt<Q80>(w, d_x, d_y, out_rows, false, norm, s);
+        default: return NORM_NOT_FUSED;
     }
 }
 

@@ -133,13 +133,15 @@ class Qwen3Layer:
 
 class Qwen3Decoder:
     """One-token decode through a stack of layers with preallocated activations, so that a whole step is a fixed sequence
-    of launches (capturable as one graph). Per layer, 9 launches:
-        h = rmsnorm(x) [fused with the previous layer's residual add]; qkv = h Wqkv^T; q/k norm + rope + cache append;
-        attention (+ combine); o = a Wo^T; (x, h) = add_rmsnorm(x, o); f = swiglu(h Wgu^T); y = f Wdown^T; x += y [next fused add]
+    of launches (capturable as one graph). Per layer, 7 launches:
+        qkv = rmsnorm(x [+ previous FFN output]) Wqkv^T   [norm and residual add formed inside the mat-vec]
+        q/k norm + rope + cache append;  attention;  combine of its splits;  o = a Wo^T
+        f = swiglu(rmsnorm(x + o) Wgu^T)                  [again inside the mat-vec];  y = f Wdown^T
+    With fuse_norm=False the norms run as their own launches (9 per layer), as the reference issues them.
     """
 
-    def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None):
-        self.cfg, self.layers, self.max_len, self.stream = cfg, layers, int(max_len), stream
+    def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None, fuse_norm=True):
+        self.cfg, self.layers, self.max_len, self.stream, self.fuse_norm = cfg, layers, int(max_len), stream, bool(fuse_norm)
         self.output_norm, self.lm_head = output_norm, lm_head          # final norm + LM head: hidden -> logits in the same step
         assert (output_norm is None) == (lm_head is None), "output_norm and lm_head come together"
         self.logits = Tensor.empty((1, lm_head.rows())) if lm_head is not None else None
@@ -147,8 +149,10 @@ class Qwen3Decoder:
         self.q_out, self.kv_out = c.n_head * c.head_dim, c.n_head_kv * c.head_dim
         self.caches = [KvCache(max_len, self.kv_out) for _ in layers]
         self.pos = _u32_tensor([0])                       # device word: the position of the token being decoded
-        self.x = Tensor.empty((1, c.d_model))             # residual stream
-        self.h = Tensor.empty((1, c.d_model))             # normed input of the current block
+        self.xa = Tensor.empty((1, c.d_model))            # residual stream: the step's input is written here ...
+        self.xb = Tensor.empty((1, c.d_model))            # ... and the residual alternates between the two buffers
+        self.x = self.xa                                  # where the last step left the hidden state
+        self.h = Tensor.empty((1, c.d_model))             # normed input of the current block (unfused path / scratch)
         self.qkv = Tensor.empty((1, self.q_out + 2 * self.kv_out))
         self.q = Tensor.empty((1, self.q_out))
         self.att = Tensor.empty((1, self.q_out))
@@ -171,20 +175,33 @@ class Qwen3Decoder:
     def set_input(self, x_host):
         a = np.ascontiguousarray(x_host, dtype=np.float32).reshape(-1)
         assert a.size == self.cfg.d_model
-        _check(_lib.load().fhip_memcpy_h2d(self.x.buf.ptr, _vp(a), a.nbytes, _stream_handle(self.stream)))
+        _check(_lib.load().fhip_memcpy_h2d(self.xa.buf.ptr, _vp(a), a.nbytes, _stream_handle(self.stream)))
         _check(_lib.load().fhip_stream_sync(_stream_handle(self.stream)))
 
     # -- one step ---------------------------------------------------------------------------------
-    def _enqueue_step(self):
-        """All layers on the current x at position *pos; leaves the final hidden state in x and advances *pos."""
+    def _norm_matmul(self, w, cur, alt, resid, norm_w, y, swiglu):
+        """y = [swiglu] rmsnorm(cur [+ resid]) W^T; returns the buffer that holds cur + resid afterwards."""
         lib, c, s = _lib.load(), self.cfg, _stream_handle(self.stream)
-        d = c.d_model
+        if self.fuse_norm:
+            _check(lib.fhip_norm_matmul_q(w.handle, cur.buf.ptr, resid.buf.ptr if resid is not None else None, norm_w.buf.ptr, c.eps,
+                                          alt.buf.ptr if resid is not None else None, self.h.buf.ptr, int(swiglu), y.buf.ptr, s))
+            return alt if resid is not None else cur
+        if resid is None:
+            _check(lib.fhip_rmsnorm(cur.buf.ptr, norm_w.buf.ptr, 1, c.d_model, c.eps, self.h.buf.ptr, s))
+        else:   # the residual updated in place, and its norm, in one launch
+            _check(lib.fhip_add_rmsnorm(cur.buf.ptr, resid.buf.ptr, norm_w.buf.ptr, 1, c.d_model, c.eps, cur.buf.ptr, self.h.buf.ptr, s))
+        fn = lib.fhip_matmul_q_swiglu if swiglu else lib.fhip_matmul_q
+        _check(fn(w.handle, self.h.buf.ptr, 1, y.buf.ptr, s))
+        return cur
+
+    def _enqueue_step(self):
+        """All layers on the input in xa at position *pos; leaves the final hidden state in self.x and advances *pos."""
+        lib, c, s = _lib.load(), self.cfg, _stream_handle(self.stream)
+        cur, alt = self.xa, self.xb
+        other = lambda t: self.xb if t is self.xa else self.xa
         for il, (l, kv) in enumerate(zip(self.layers, self.caches)):
-            if il == 0:
-                _check(lib.fhip_rmsnorm(self.x.buf.ptr, l.attn_norm.buf.ptr, 1, d, c.eps, self.h.buf.ptr, s))
-            else:   # x = x + y of the previous layer's FFN, and this layer's input norm, in one launch
-                _check(lib.fhip_add_rmsnorm(self.x.buf.ptr, self.y.buf.ptr, l.attn_norm.buf.ptr, 1, d, c.eps, self.x.buf.ptr, self.h.buf.ptr, s))
-            _check(lib.fhip_matmul_q(l.wqkv.handle, self.h.buf.ptr, 1, self.qkv.buf.ptr, s))
+            cur = self._norm_matmul(l.wqkv, cur, alt, self.y if il else None, l.attn_norm, self.qkv, False)
+            alt = other(cur)
             _check(lib.fhip_qkv_post(self.qkv.buf.ptr, l.qkv_bias.buf.ptr if l.qkv_bias is not None else None,
                                      l.q_norm.buf.ptr if l.q_norm is not None else None, l.k_norm.buf.ptr if l.k_norm is not None else None,
                                      self.pos.buf.ptr, None, 1, c.n_head, c.n_head_kv, c.head_dim, c.head_dim, int(c.rope_interleaved),
@@ -192,14 +209,14 @@ class Qwen3Decoder:
             _check(lib.fhip_decode_attention(self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, c.n_head, c.n_head_kv, c.head_dim, self.max_len,
                                              self.pos.buf.ptr, self.ws.ptr if self.ws is not None else None, self.att.buf.ptr, s))
             _check(lib.fhip_matmul_q(l.wo.handle, self.att.buf.ptr, 1, self.o.buf.ptr, s))
-            _check(lib.fhip_add_rmsnorm(self.x.buf.ptr, self.o.buf.ptr, l.ffn_norm.buf.ptr, 1, d, c.eps, self.x.buf.ptr, self.h.buf.ptr, s))
-            _check(lib.fhip_matmul_q_swiglu(l.ffn_gate_up.handle, self.h.buf.ptr, 1, self.f.buf.ptr, s))
+            cur = self._norm_matmul(l.ffn_gate_up, cur, alt, self.o, l.ffn_norm, self.f, True)
+            alt = other(cur)
             _check(lib.fhip_matmul_q(l.ffn_down.handle, self.f.buf.ptr, 1, self.y.buf.ptr, s))
         if self.lm_head is not None:   # last residual add fused with the output norm, then the LM head
-            _check(lib.fhip_add_rmsnorm(self.x.buf.ptr, self.y.buf.ptr, self.output_norm.buf.ptr, 1, d, c.eps, self.x.buf.ptr, self.h.buf.ptr, s))
-            _check(lib.fhip_matmul_q(self.lm_head.handle, self.h.buf.ptr, 1, self.logits.buf.ptr, s))
+            cur = self._norm_matmul(self.lm_head, cur, alt, self.y, self.output_norm, self.logits, False)
         else:
-            _check(lib.fhip_add(self.x.buf.ptr, self.y.buf.ptr, d, self.x.buf.ptr, s))
+            _check(lib.fhip_add(cur.buf.ptr, self.y.buf.ptr, c.d_model, cur.buf.ptr, s))
+        self.x = cur
         _check(lib.fhip_u32_add(self.pos.buf.ptr, 1, 1, s))
 
     def step(self):

@@ -251,6 +251,15 @@ size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_di
 int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
                           size_t len, const uint32_t* d_last_pos, float* d_ws, float* d_out, void* stream);
 
+/* rmsnorm / add_rmsnorm (lib.rs:346, :372) fused into the mat-vec that consumes it, for ONE activation row:
+ *   h = rmsnorm(x [+ resid], norm_w, eps);   y = h W^T   (swiglu != 0: y = silu(gate . h) * (up . h), as fhip_matmul_q_swiglu)
+ * and, when d_x_out is given, x_out = x + resid (the next residual; must not alias d_x). The norm is formed while the
+ * activation row is staged, so the layer saves a launch; weights whose shape the streaming kernel does not take run the two
+ * steps apart through d_h_scratch [cols] (required). d_resid may be NULL (plain rmsnorm). Same value as the unfused pair to
+ * rounding (the sum of squares is added in a different order), not the same bits. No single counterpart in the reference. */
+int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_resid, const float* d_norm_w, float eps, float* d_x_out,
+                       float* d_h_scratch, int swiglu, float* d_y, void* stream);
+
 /* words[i] += delta for n device u32 words: advances the position word(s) at the end of a captured decode step. */
 int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream);
 

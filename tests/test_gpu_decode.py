@@ -152,6 +152,46 @@ def test_qkv_post_fuses_bias_norm_rope_and_append(F, X, D):
     assert np.array_equal(bits(kc.to_vec()), bits(kc0.reshape(-1))) and np.array_equal(bits(vc.to_vec()), bits(vc0.reshape(-1)))
 
 
+def test_norm_fused_into_the_matvec(F, X, D, O):
+    """fhip_norm_matmul_q against rmsnorm / add_rmsnorm followed by the mat-vec: the residual sum bit-exact, the product
+    within the dot-product bound of the unfused pair (the sum of squares is added in another order: ~1e-7 on the scale),
+    on shapes the streaming kernel takes (fused) and on ones it does not (the two steps run apart)."""
+    from ferric_amd.synth import synth_weights
+    rng = np.random.default_rng(6)
+    lib = F._lib.load()
+    for ty, rows, cols, swiglu in [(Q4_K, 7168, 5120, False), (Q4_K, 2 * 1024, 5120, True), (Q6_K, 512, 5120, False), (Q8_0, 96, 4096, False),
+                                   (Q4_K, 64, 768, False), (Q6_K, 40, 17408, False), (Q4_K, 2 * 96, 1024, True)]:
+        raw = synth_weights(ty, rows, cols, 3)
+        w = F.QMatrix.from_bytes(raw, ty, rows, cols)
+        x = rng.standard_normal(cols).astype(np.float32)
+        r = rng.standard_normal(cols).astype(np.float32)
+        nw = ((rng.random(cols) + 0.5) * 0.05).astype(np.float32)
+        xt, rt, nt = F.Tensor.from_vec(x, (1, cols)), F.Tensor.from_vec(r, (1, cols)), F.Tensor.from_vec(nw, (cols,))
+        out_rows = rows // 2 if swiglu else rows
+        for resid in (rt, None):
+            xo, hs, y = F.Tensor.from_vec(np.full(cols, 7.0, np.float32), (1, cols)), F.Tensor.empty((1, cols)), F.Tensor.empty((1, out_rows))
+            F._lib.check(lib.fhip_norm_matmul_q(w.handle, xt.buf.ptr, resid.buf.ptr if resid is not None else None, nt.buf.ptr, 1e-6,
+                                                xo.buf.ptr, hs.buf.ptr, int(swiglu), y.buf.ptr, None))
+            if resid is not None:
+                s_ref, h_ref = X.add_rmsnorm(xt, rt, nt, 1e-6)
+                assert np.array_equal(bits(xo.to_vec()), bits(s_ref.to_vec())), (ty, rows, cols)
+            else:
+                h_ref = X.rmsnorm(xt, nt, 1e-6)
+                assert np.array_equal(xo.to_vec(), np.full(cols, 7.0, np.float32))        # nothing to store without a residual
+            y_ref = (h_ref.matmul_q(w).swiglu(out_rows) if swiglu else h_ref.matmul_q(w)).to_vec()
+            h64 = D.rmsnorm((x + r) if resid is not None else x, nw, 1e-6)
+            y64, wn = O.matmul_f64(h64.astype(np.float32), raw, ty, rows, cols)
+            if swiglu:
+                y64 = D.silu_mul(y64, out_rows)
+                assert close(y.to_vec(), y64, 2e-5), (ty, rows, cols)
+            else:
+                assert (np.abs(y.to_vec() - y64[0]) <= 1e-3 * wn * np.linalg.norm(h64)).all()
+                assert close(y.to_vec(), y64, 1e-5), (ty, rows, cols)
+            assert close(y.to_vec(), y_ref, 2e-5)
+    with pytest.raises(F._lib.FerricHipError, match="x_out must not be x"):
+        F._lib.check(lib.fhip_norm_matmul_q(w.handle, xt.buf.ptr, rt.buf.ptr, nt.buf.ptr, 1e-6, xt.buf.ptr, hs.buf.ptr, 0, y.buf.ptr, None))
+
+
 def _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, qk_norm):
     """Random Q4_K / Q6_K projections (synthetic blocks have rows of norm ~ 2 sqrt(cols)), block norms small enough that the
     projections of a normalised vector are O(1); the f64 twin holds the oracle-dequantized weights."""
@@ -175,8 +215,8 @@ def _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, qk_norm):
     return layers, olayers
 
 
-@pytest.mark.parametrize("qk_norm", [True, False])
-def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, X, O, D, qk_norm):
+@pytest.mark.parametrize("qk_norm,fuse_norm", [(True, True), (False, True), (True, False)])
+def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, X, O, D, qk_norm, fuse_norm):
     rng = np.random.default_rng(4)
     n_layer, d, nh, nkv, hd, n_ff, steps = 3, 1024, 8, 2, 128, 1536, 6
     cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6)
@@ -191,7 +231,7 @@ def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, 
             x = D.apply_layer(x, l, kc, vc, pos, cfg)
         want.append(x)
     stream = F.Stream()
-    dec = X.Qwen3Decoder(cfg, layers, max_len=steps + 2, stream=stream)
+    dec = X.Qwen3Decoder(cfg, layers, max_len=steps + 2, stream=stream, fuse_norm=fuse_norm)
     eager = []
     for pos in range(steps):
         dec.set_input(xs[pos])
@@ -217,7 +257,7 @@ def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, 
     head_raw = synth_weights(Q6_K, 300, d, 77)
     onorm = ((rng.random(d) + 0.5) * 0.02).astype(np.float32)
     dec2 = X.Qwen3Decoder(cfg, layers, max_len=4, stream=stream, output_norm=F.Tensor.from_vec(onorm, onorm.shape),
-                          lm_head=F.QMatrix.from_bytes(head_raw, Q6_K, 300, d))
+                          lm_head=F.QMatrix.from_bytes(head_raw, Q6_K, 300, d), fuse_norm=fuse_norm)
     dec2.set_input(xs[0])
     dec2.step()
     assert np.array_equal(bits(dec2.hidden()), bits(eager[0]))
