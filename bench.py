@@ -102,6 +102,20 @@ def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed
     return out, alg, nbytes
 
 
+def launch_floor_us(F, lib, check, stream, timer, n=2048):
+    """What one launch costs in a graph on this box when the kernel does nothing to speak of (one workgroup adds 0 to a
+    word): the part of every per-launch figure in this file that no kernel can win back."""
+    from ferric_amd import decode as X
+    w = X._u32_tensor([0])
+    g = F.Graph.begin(stream)
+    for _ in range(n):
+        check(lib.fhip_u32_add(w.buf.ptr, 1, 0, stream.handle))
+    g = g.end()
+    g.launch()
+    check(lib.fhip_stream_sync(stream.handle))
+    return min(timer.time_ms(g.launch) for _ in range(3)) * 1e3 / n
+
+
 def bench_ffn(F, lib, check, stream, timer, batches, reps=20):
     from ferric_amd.synth import synth_weights
     n_embd, n_ff = 5120, 17408
@@ -433,8 +447,8 @@ def main():
         "warm_single_copy": c2["warm"],
         "roofline": {"bound": "hbm", "achieved": alg / (ms_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": Q4K_5120_TRAFFIC_BYTES,
-                     "kernel": "gemv_stream_kernel<Q4K, M=1, U=3>", "algorithmic_bytes_per_launch": alg,
-                     "launch_us": ms_step * 1e3},
+                     "kernel": "gemv_stream_kernel<Q4K, M=1, U=3, plain>", "algorithmic_bytes_per_launch": alg,
+                     "launch_us": ms_step * 1e3, "empty_launch_us": launch_floor_us(F, lib, check, stream, timer)},
     }
     if not args.no_q8:
         log("[bench] Q8_0 GEMV 4096x4096 ...")
