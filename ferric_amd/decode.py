@@ -67,8 +67,8 @@ def rope(x, n_heads, head_dim, base, offset=0, positions=None, freq_scale=None, 
     _check(_lib.load().fhip_rope(x.buf.ptr, 0, t, n_heads, head_dim, n_rot, base, pos_t.buf.ptr if pos_t is not None else None, offset,
                                  freq_scale.buf.ptr if freq_scale is not None else None, int(interleaved), out.buf.ptr,
                                  _stream_handle(stream)))
-    if pos_t is not None and not isinstance(positions, Tensor) and stream is None:
-        _check(_lib.load().fhip_stream_sync(None))     # the temporary position buffer is freed on return
+    if pos_t is not None and not isinstance(positions, Tensor):
+        _check(_lib.load().fhip_stream_sync(_stream_handle(stream)))     # the temporary position buffer is freed on return
     return out
 
 
@@ -99,6 +99,7 @@ def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, 
     assert len(q.shape) == 2 and q.shape[0] == 1, "decode_attention takes one query row"
     dh = q.shape[1] // n_heads
     length = cache.len if length is None else length
+    assert 1 <= length <= cache.cap, f"decode_attention: length {length} outside the cache's 1..={cache.cap} rows"
     assert cache.width == n_kv_heads * dh
     lib = _lib.load()
     need = lib.fhip_decode_attention_ws_bytes(n_heads, n_kv_heads, dh, length)
