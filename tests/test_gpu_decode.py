@@ -117,6 +117,33 @@ def test_kv_append2_and_decode_attention(F, X, D):
         X.decode_attention(F.Tensor.from_vec(np.zeros((1, 9 * 64), np.float32), (1, 9 * 64)), X.KvCache(4, 64), 9, 1, length=1)
 
 
+def test_attention_properties_at_a_32k_context(F, X):
+    """Sizes the f64 loop oracle does not reach: properties that hold at any length. Attention is linear in V; adding
+    one constant to every score (q -> q, K -> K + c e with q.e = 0 is not available, so: duplicate the cache) leaves the
+    output unchanged -- keys [K; K], values [V; V] give the same output as K, V; equal keys give the mean of the values."""
+    rng = np.random.default_rng(11)
+    nh, nkv, hd, s = 40, 8, 128, 16384
+    width = nkv * hd
+    k = (rng.standard_normal((s, width)) * 0.3).astype(np.float32)
+    v1 = rng.standard_normal((s, width)).astype(np.float32)
+    v2 = rng.standard_normal((s, width)).astype(np.float32)
+    q = rng.standard_normal((1, nh * hd)).astype(np.float32)
+    qt = F.Tensor.from_vec(q, q.shape)
+
+    def run(keys, vals):
+        c = X.KvCache(keys.shape[0], width)
+        c.append2(F.Tensor.from_vec(keys, keys.shape), F.Tensor.from_vec(vals, vals.shape))
+        return X.decode_attention(qt, c, nh, nkv).to_vec().astype(np.float64)
+    a1, a2 = run(k, v1), run(k, v2)
+    mix = run(k, (np.float32(0.5) * v1 - np.float32(2.0) * v2).astype(np.float32))
+    assert np.abs(mix - (0.5 * a1 - 2.0 * a2)).max() <= 2e-5 * np.abs(a2).max()
+    twice = run(np.concatenate([k, k]), np.concatenate([v1, v1]))          # 32768 keys
+    assert np.abs(twice - a1).max() <= 1e-5 * np.abs(a1).max()
+    flat = run(np.tile(k[:1], (s, 1)), v1)
+    want = np.repeat(v1.astype(np.float64).mean(axis=0).reshape(nkv, 1, hd), nh // nkv, axis=1).reshape(-1)
+    assert np.abs(flat - want).max() <= 1e-5 * np.abs(want).max() + 1e-6
+
+
 def test_qkv_post_fuses_bias_norm_rope_and_append(F, X, D):
     rng = np.random.default_rng(3)
     lib = F._lib.load()
