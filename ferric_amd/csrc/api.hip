@@ -443,15 +443,21 @@ size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_di
     return splits > 1 ? n_head * (size_t)splits * (head_dim + 2) * sizeof(float) : 0;
 }
 
-int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
-                          size_t len, const uint32_t* d_last_pos, float* d_ws, float* d_out, void* stream) {
+int fhip_decode_attention_ex(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
+                             size_t len, const uint32_t* d_last_pos, size_t window, float softcap, float* d_ws, float* d_out, void* stream) {
     int rc = need_init();
     if (rc) return rc;
     if (n_head > 0xFFFFu || n_kv > 0xFFFFu || head_dim > 0xFFFFu) return set_error(FHIP_ERR_SHAPE, "fhip_decode_attention: head counts exceed 65535");
     if (n_head == 0 || head_dim == 0) return FHIP_OK;
     if (!d_q || !d_k_cache || !d_v_cache || !d_out) return set_error(FHIP_ERR_ARG, "fhip_decode_attention: NULL pointer");
-    return fhip::launch_decode_attention(d_q, d_k_cache, d_v_cache, (int)n_head, (int)n_kv, (int)head_dim, len, d_last_pos, d_ws, d_out,
-                                         (hipStream_t)stream);
+    if (!(softcap >= 0.f)) return set_error(FHIP_ERR_ARG, "fhip_decode_attention: softcap must be >= 0");
+    return fhip::launch_decode_attention(d_q, d_k_cache, d_v_cache, (int)n_head, (int)n_kv, (int)head_dim, len, d_last_pos, window, softcap, d_ws,
+                                         d_out, (hipStream_t)stream);
+}
+
+int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
+                          size_t len, const uint32_t* d_last_pos, float* d_ws, float* d_out, void* stream) {
+    return fhip_decode_attention_ex(d_q, d_k_cache, d_v_cache, n_head, n_kv, head_dim, len, d_last_pos, 0, 0.f, d_ws, d_out, stream);
 }
 
 int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_resid, const float* d_norm_w, float eps, float* d_x_out,

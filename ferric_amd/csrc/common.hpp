@@ -107,6 +107,6 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
                      float* vc, hipStream_t s);
 int attn_splits(size_t len, int n_kv);
 int launch_decode_attention(const float* q, const float* K, const float* V, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len,
-                            float* ws, float* out, hipStream_t s);
+                            size_t window, float softcap, float* ws, float* out, hipStream_t s);
 
 }  // namespace fhip

@@ -249,7 +249,7 @@ __device__ __forceinline__ void load_dims(const float* p, float (&r)[DPL]) {   /
 template <int G, int DPL>
 __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict__ q, const float* __restrict__ K, const float* __restrict__ V,
                                                          int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
-                                                         float* __restrict__ part, float* __restrict__ out) {
+                                                         uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out) {
     constexpr int HD = 16 * DPL;
     __shared__ float sm_m[4][G], sm_l[4][G];
     __shared__ float sm_acc[4][G][HD];
@@ -258,8 +258,10 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
     const int kvh = blockIdx.x, split = blockIdx.y;
     uint32_t len = len_dev ? *len_dev + 1u : len_host;   // the device word is the newest token's position
     if (len > len_host) len = len_host;
-    const uint32_t per = (len + splits - 1) / splits;
-    const uint32_t k0 = (uint32_t)split * per, k1 = min(len, k0 + per);
+    // sliding window (nn.rs:92-111): only the last `window` keys count; 0 or >= len: all of them
+    const uint32_t first = (window > 0 && window < len) ? len - window : 0u;
+    const uint32_t per = (len - first + splits - 1) / splits;
+    const uint32_t k0 = first + (uint32_t)split * per, k1 = min(len, k0 + per);
     const size_t stride = (size_t)n_kv * HD;
     const float* Kb = K + (size_t)kvh * HD + sub * DPL;
     const float* Vb = V + (size_t)kvh * HD + sub * DPL;
@@ -289,6 +291,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
 #pragma unroll
                 for (int i = 0; i < DPL; i++) d = fmaf(qr[h][i], kr[j][i], d);
                 d = row16_sum(d) * scale;
+                if (softcap > 0.f) d = softcap * tanhf(d / softcap);   // cap * tanh(x / cap), crates/ferric-tensor/src/lib.rs:308
                 sc[j] = (kb + j < k1) ? d : -3.0e38f;
             }
             float m_new = m[h];
@@ -374,10 +377,10 @@ __global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restri
 
 template <int G>
 int launch_attn_g(int hd, dim3 grid, hipStream_t s, const float* q, const float* K, const float* V, int n_kv, uint32_t len, const uint32_t* d_len,
-                  float scale, int splits, float* part, float* out) {
+                  float scale, int splits, uint32_t window, float softcap, float* part, float* out) {
     switch (hd) {
-        case 64: hipLaunchKernelGGL((attn_split_kernel<G, 4>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
-        case 128: hipLaunchKernelGGL((attn_split_kernel<G, 8>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, part, out); break;
+        case 64: hipLaunchKernelGGL((attn_split_kernel<G, 4>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        case 128: hipLaunchKernelGGL((attn_split_kernel<G, 8>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
         default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     }
     return FHIP_OK;
@@ -464,7 +467,7 @@ int attn_splits(size_t len, int n_kv) {
 }
 
 int launch_decode_attention(const float* q, const float* K, const float* V, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len,
-                            float* ws, float* out, hipStream_t s) {
+                            size_t window, float softcap, float* ws, float* out, hipStream_t s) {
     if (n_head == 0 || hd == 0) return FHIP_OK;
     if (len == 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: empty cache");
     if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: n_heads must be a multiple of n_kv_heads");
@@ -473,17 +476,18 @@ int launch_decode_attention(const float* q, const float* K, const float* V, int 
     const int g = n_head / n_kv, splits = attn_splits(len, n_kv);
     if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
     const float scale = 1.0f / sqrtf((float)hd);
+    const uint32_t win = window > 0x7FFFFFFFull ? 0u : (uint32_t)window;   // a window that large is no window
     dim3 grid((unsigned)n_kv, (unsigned)splits);
     int rc;
     switch (g) {
-        case 1: rc = launch_attn_g<1>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 2: rc = launch_attn_g<2>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 3: rc = launch_attn_g<3>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 4: rc = launch_attn_g<4>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 5: rc = launch_attn_g<5>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 6: rc = launch_attn_g<6>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 7: rc = launch_attn_g<7>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
-        case 8: rc = launch_attn_g<8>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, ws, out); break;
+        case 1: rc = launch_attn_g<1>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case 2: rc = launch_attn_g<2>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case 3: rc = launch_attn_g<3>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case 4: rc = launch_attn_g<4>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case 5: rc = launch_attn_g<5>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case 6: rc = launch_attn_g<6>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case 7: rc = launch_attn_g<7>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case 8: rc = launch_attn_g<8>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
         default: return set_error(FHIP_ERR_SHAPE, "decode_attention: %d query heads per KV head (1..=8 supported)", g);
     }
     if (rc) return rc;

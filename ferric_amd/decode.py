@@ -93,8 +93,8 @@ class KvCache:
         return self
 
 
-def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, ws=None, stream=None):
-    """nn.rs:140: q [1, n_heads * dh] against the first `length` rows of the cache (default: all filled rows). last_pos: a
+def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, ws=None, stream=None, window=0, softcap=0.0):
+    """nn.rs:140 (window / softcap: nn.rs:92 decode_attention_win and the softcapped scores of nn.rs:61): q [1, n_heads * dh] against the first `length` rows of the cache (default: all filled rows). last_pos: a
     device u32 Tensor holding the newest row's index, read at run time instead (for a captured step)."""
     assert len(q.shape) == 2 and q.shape[0] == 1, "decode_attention takes one query row"
     dh = q.shape[1] // n_heads
@@ -107,9 +107,9 @@ def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, 
     if need and ws is None:
         own = ws = DeviceBuffer(need)
     out = Tensor.empty((1, n_heads * dh))
-    _check(lib.fhip_decode_attention(q.buf.ptr, cache.k.buf.ptr, cache.v.buf.ptr, n_heads, n_kv_heads, dh, length,
-                                     last_pos.buf.ptr if last_pos is not None else None, ws.ptr if ws is not None else None, out.buf.ptr,
-                                     _stream_handle(stream)))
+    _check(lib.fhip_decode_attention_ex(q.buf.ptr, cache.k.buf.ptr, cache.v.buf.ptr, n_heads, n_kv_heads, dh, length,
+                                        last_pos.buf.ptr if last_pos is not None else None, window, softcap,
+                                        ws.ptr if ws is not None else None, out.buf.ptr, _stream_handle(stream)))
     if own is not None:
         _check(lib.fhip_stream_sync(_stream_handle(stream)))   # the scratch is freed on return
     return out

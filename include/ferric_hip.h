@@ -250,6 +250,12 @@ int fhip_qkv_post(const float* d_qkv, const float* d_bias, const float* d_q_norm
 size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_dim, size_t len);
 int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
                           size_t len, const uint32_t* d_last_pos, float* d_ws, float* d_out, void* stream);
+/* nn.rs:92 decode_attention_win and the softcapped scores of nn.rs:61 / lib.rs:308 (Gemma-2), which the reference's fused
+ * kernel does not take (it falls back to ~12 composed dispatches): window > 0 attends to the last `window` keys only
+ * (0, or >= the length: all keys); softcap > 0 replaces each scaled score x by softcap * tanh(x / softcap). With
+ * (0, 0.0f) this is fhip_decode_attention. */
+int fhip_decode_attention_ex(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
+                             size_t len, const uint32_t* d_last_pos, size_t window, float softcap, float* d_ws, float* d_out, void* stream);
 
 /* rmsnorm / add_rmsnorm (lib.rs:346, :372) fused into the mat-vec that consumes it, for ONE activation row:
  *   h = rmsnorm(x [+ resid], norm_w, eps);   y = h W^T   (swiglu != 0: y = silu(gate . h) * (up . h), as fhip_matmul_q_swiglu)

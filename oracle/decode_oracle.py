@@ -55,9 +55,11 @@ def rope(x, n_heads, head_dim, base, positions, interleaved=False, n_rot=None, f
     return out.reshape(t, n_heads * head_dim)
 
 
-def decode_attention(q, k, v, n_heads, n_kv_heads):
+def decode_attention(q, k, v, n_heads, n_kv_heads, window=0, softcap=0.0):
     """crates/ferric-tensor/src/nn.rs:153-166 (the composed form the fused kernel is defined by): q [n_heads * dh], k / v
-    [S, n_kv_heads * dh]; head h uses KV head h // (n_heads / n_kv_heads); softmax(q.k / sqrt(dh)) @ v."""
+    [S, n_kv_heads * dh]; head h uses KV head h // (n_heads / n_kv_heads); softmax(q.k / sqrt(dh)) @ v. softcap > 0: scaled
+    scores x become cap * tanh(x / cap) (nn.rs:61, lib.rs:308); 0 < window < S: keys older than the last `window` are masked
+    out (nn.rs:92-111; the reference adds -1e30 to them, which exp() turns into exactly 0)."""
     q = np.asarray(q, np.float64).reshape(n_heads, -1)
     dh = q.shape[1]
     s = np.asarray(k).shape[0]
@@ -68,6 +70,10 @@ def decode_attention(q, k, v, n_heads, n_kv_heads):
     out = np.zeros((n_heads, dh))
     for h in range(n_heads):
         sc = k[:, h // g, :] @ q[h] * scale
+        if softcap > 0:
+            sc = np.float64(np.float32(softcap)) * np.tanh(sc / np.float64(np.float32(softcap)))
+        if 0 < window < s:
+            sc[: s - window] = -np.inf
         p = np.exp(sc - sc.max())
         out[h] = (p / p.sum()) @ v[:, h // g, :]
     return out.reshape(1, n_heads * dh)

@@ -117,6 +117,28 @@ def test_kv_append2_and_decode_attention(F, X, D):
         X.decode_attention(F.Tensor.from_vec(np.zeros((1, 9 * 64), np.float32), (1, 9 * 64)), X.KvCache(4, 64), 9, 1, length=1)
 
 
+def test_attention_window_and_softcap(F, X, D):
+    rng = np.random.default_rng(12)
+    for nh, nkv, hd, s in [(40, 8, 128, 1500), (8, 2, 64, 70)]:
+        width = nkv * hd
+        k = rng.standard_normal((s, width)).astype(np.float32)
+        v = rng.standard_normal((s, width)).astype(np.float32)
+        q = (rng.standard_normal((1, nh * hd)) * 2).astype(np.float32)
+        cache = X.KvCache(s, width)
+        cache.append2(F.Tensor.from_vec(k, k.shape), F.Tensor.from_vec(v, v.shape))
+        qt = F.Tensor.from_vec(q, q.shape)
+        for window, cap in [(0, 0.0), (1, 0.0), (33, 0.0), (s - 1, 0.0), (s, 0.0), (s + 7, 0.0), (0, 50.0), (0, 2.5), (100, 30.0)]:
+            got = X.decode_attention(qt, cache, nh, nkv, window=window, softcap=cap).to_vec()
+            want = D.decode_attention(q[0], k, v, nh, nkv, window=window, softcap=cap)
+            assert close(got, want, 1e-5), (nh, s, window, cap)
+        # a window under a length read on the device
+        last = X._u32_tensor([s // 2 - 1])
+        got = X.decode_attention(qt, cache, nh, nkv, length=s, last_pos=last, window=20).to_vec()
+        assert close(got, D.decode_attention(q[0], k[: s // 2], v[: s // 2], nh, nkv, window=20), 1e-5)
+    with pytest.raises(F._lib.FerricHipError, match="softcap must be >= 0"):
+        X.decode_attention(qt, cache, nh, nkv, softcap=-1.0)
+
+
 def test_attention_properties_at_a_32k_context(F, X):
     """Sizes the f64 loop oracle does not reach: properties that hold at any length. Attention is linear in V; adding
     one constant to every score (q -> q, K -> K + c e with q.e = 0 is not available, so: duplicate the cache) leaves the

@@ -101,6 +101,29 @@ def test_decode_attention_against_loops_and_special_cases():
     assert np.allclose(D.decode_attention(q1, k2, v2, 1, 1), 1.0 / (1.0 + math.exp(-4.0 / math.sqrt(dh))), rtol=1e-7)
 
 
+def test_window_and_softcap_in_the_attention_oracle():
+    rng = np.random.default_rng(6)
+    nh, nkv, dh, s = 4, 2, 8, 11
+    q = rng.standard_normal(nh * dh).astype(np.float32)
+    k = rng.standard_normal((s, nkv * dh)).astype(np.float32)
+    v = rng.standard_normal((s, nkv * dh)).astype(np.float32)
+    full = D.decode_attention(q, k, v, nh, nkv)
+    assert np.array_equal(D.decode_attention(q, k, v, nh, nkv, window=0), full)
+    assert np.array_equal(D.decode_attention(q, k, v, nh, nkv, window=s), full) and np.array_equal(D.decode_attention(q, k, v, nh, nkv, window=s + 5), full)
+    # the last w keys only == attention over the truncated cache (nn.rs:92-111)
+    for w in (1, 3, 10):
+        assert np.allclose(D.decode_attention(q, k, v, nh, nkv, window=w), D.decode_attention(q, k[s - w:], v[s - w:], nh, nkv), rtol=1e-13)
+    # softcap: cap * tanh(x / cap); a huge cap is the identity, a tiny one flattens the scores to +-cap
+    assert np.allclose(D.decode_attention(q, k, v, nh, nkv, softcap=1e6), full, rtol=1e-9)
+    flat = D.decode_attention(q * np.float32(1e4), k, v, nh, nkv, softcap=1e-3)     # every score is +-1e-3: nearly the mean
+    assert np.allclose(flat.reshape(nh, dh)[0], v[:, :dh].astype(np.float64).mean(axis=0), atol=2e-3)
+    q1 = np.zeros(dh, np.float32); q1[0] = 6.0
+    k2 = np.zeros((2, dh), np.float32); k2[0, 0] = 1.0
+    v2 = np.array([[1.0] * dh, [0.0] * dh], np.float32)
+    x = 6.0 / math.sqrt(dh)
+    assert np.allclose(D.decode_attention(q1, k2, v2, 1, 1, softcap=1.5), 1.0 / (1.0 + math.exp(-1.5 * math.tanh(x / 1.5))), rtol=1e-7)
+
+
 def test_qkv_post_composes_bias_norm_and_rope():
     rng = np.random.default_rng(4)
     nh, nkv, hd = 4, 2, 8
