@@ -3,7 +3,9 @@
 //   y[m, o] = sum_k x[m, k] * dequant(W[o, k])
 //
 // Replaces the reference's split-K / flat WGSL kernels (crates/ferric-tensor/src/dtype.rs:2995-3051
-// Q4_K, :3423-3469 Q6_K, :3473-3529 Q8_0) and the fused gate/up SwiGLU kernels (:2372-2410, :2734-2775).
+// Q4_K, :3423-3469 Q6_K, :3473-3529 Q8_0) and the fused gate/up SwiGLU kernels (:2372-2410, :2734-2775);
+// the same skeleton takes Q5_K, Q4_0 / Q4_1 / Q5_0 / Q5_1, IQ4_NL / IQ4_XS and MXFP4 (:1049, :1838-1904, :3185-3420)
+// as further per-format structs.
 //
 // Why it looks the way it does. At 8 TB/s a CU gets ~13 weight bytes per clock, i.e. ~23 Q4_K weights,
 // while it can issue 64 lane-instructions per clock: under 3 instructions per weight all-in. A plain
@@ -88,7 +90,7 @@ __device__ __forceinline__ float planes_to_f32(int a, int b, int c) { return fma
 // ------------------------------------------------------------------------------------------------
 
 struct Q4K {
-    static constexpr int WPL = 64, RUN = 32, NRUN = 2, BLOCK_VALUES = 256;
+    static constexpr int WPL = 64, RUN = 32, NRUN = 2, BLOCK_VALUES = 256, U1 = 3;
     static constexpr bool SIGNED_W = false;
     struct Lane { uint32_t off_h, off_q, sh, m1, m2, m3; };
     struct Data {
@@ -154,7 +156,7 @@ struct Q4K {
 };
 
 struct Q6K {
-    static constexpr int WPL = 64, RUN = 16, NRUN = 4, BLOCK_VALUES = 256;
+    static constexpr int WPL = 64, RUN = 16, NRUN = 4, BLOCK_VALUES = 256, U1 = 2;
     static constexpr bool SIGNED_W = false;
     struct Lane { uint32_t off_a, off_h, off_s, off_d, ssh; };
     struct Data {
@@ -223,7 +225,7 @@ struct Q6K {
 };
 
 struct Q80 {
-    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32;
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32, U1 = 4;
     static constexpr bool SIGNED_W = true;
     struct Lane { uint32_t off; };
     struct Data {
@@ -264,6 +266,278 @@ struct Q80 {
     }
 };
 
+// Q5_K: 176 B = [f16 d][f16 dmin][12 B 6-bit scales/mins][qh 32 B][qs 128 B] -- Q4_K plus bit s of qh[l] as the fifth bit of
+// element l of sub-block s (crates/ferric-gguf/src/lib.rs:692-716). Unit = group g of block b (sub-blocks 2g, 2g+1): its 32
+// quant bytes and the whole 32 bytes of high bits; codes 0..31, unsigned planes as Q4_K.
+struct Q5K {
+    static constexpr int WPL = 64, RUN = 32, NRUN = 2, BLOCK_VALUES = 256, U1 = 2;
+    static constexpr bool SIGNED_W = false;
+    struct Lane { uint32_t off_h, off_q, sh, g2, m1, m2, m3; };
+    struct Data {
+        u32x4 h, b0, b1, q0, q1;
+        __device__ __forceinline__ void pin_all() { pin(h); pin(b0); pin(b1); pin(q0); pin(q1); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        int b = u >> 2, g = u & 3;
+        L.off_h = b * 176;
+        L.off_q = b * 176 + 48 + 32 * g;
+        L.sh = 16 * (g & 1);
+        L.g2 = 2 * g;
+        L.m1 = g >= 2 ? 0u : 0x3F3Fu;
+        L.m2 = g >= 2 ? 0x0F0Fu : 0u;
+        L.m3 = g >= 2 ? 0x3030u : 0u;
+        run[0] = 2 * u;
+        run[1] = 2 * u + 1;
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
+        Data d;
+        d.h = *(const u32x4*)(row + (L.off_h + eo));
+        d.b0 = *(const u32x4*)(row + (L.off_h + eo) + 16);
+        d.b1 = *(const u32x4*)(row + (L.off_h + eo) + 32);
+        d.q0 = *(const u32x4*)(row + (L.off_q + eo));
+        d.q1 = *(const u32x4*)(row + (L.off_q + eo) + 16);
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
+        uint32_t a = D.h[1] >> L.sh, b = D.h[2] >> L.sh, c = D.h[3] >> L.sh;
+        uint32_t scp = (a & L.m1) | (c & L.m2) | ((a >> 2) & L.m3);
+        uint32_t mp = (b & L.m1) | ((c >> 4) & L.m2) | ((b >> 2) & L.m3);
+        float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
+        float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1), m0 = dmin * ub(mp, 0), m1 = dmin * ub(mp, 1);
+        int acc[M][2][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int p = 0; p < 3; p++) acc[m][j][p] = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            uint32_t w = i < 4 ? D.q0[i] : D.q1[i - 4];
+            uint32_t hb = (i < 4 ? D.b0[i] : D.b1[i - 4]) >> L.g2;      // bit 0: sub-block 2g, bit 1: sub-block 2g+1
+            uint32_t lo = (w & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4);
+            uint32_t hi = ((w >> 4) & 0x0F0F0F0Fu) | ((hb & 0x02020202u) << 3);
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int p = 0; p < 3; p++) {
+                    acc[m][0][p] = pdot<false>(p, xp[m][0][p][i], lo, acc[m][0][p]);
+                    acc[m][1][p] = pdot<false>(p, xp[m][1][p][i], hi, acc[m][1][p]);
+                }
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+            float f0 = xs[m][0] * planes_to_f32(acc[m][0][0], acc[m][0][1], acc[m][0][2]);
+            float f1 = xs[m][1] * planes_to_f32(acc[m][1][0], acc[m][1][1], acc[m][1][2]);
+            out[m] = (d0 * f0 - m0 * xsum[m][0]) + (d1 * f1 - m1 * xsum[m][1]);
+        }
+    }
+};
+
+// The four 32-value formats, [f16 d][f16 m]?[u32 qh]?[qs 16 B] (crates/ferric-gguf/src/lib.rs:618-684): value i < 16 is the low
+// nibble of qs[i], value 16 + i the high one, the fifth bit of value v is bit v of qh; (n - OFF) d or n d + m. Unit = one block;
+// the offset leaves as OFF * sum(x), the affine term as m * sum(x).
+template <int BYTES, bool HAS_M, bool HAS_QH, int OFF>
+struct LegS {
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32, U1 = 4;
+    static constexpr bool SIGNED_W = false;
+    static constexpr int QH = HAS_M ? 4 : 2, QS = QH + (HAS_QH ? 4 : 0);
+    struct Lane { uint32_t off; };
+    struct Data {
+        u32x4 q; uint32_t dm, qh;
+        __device__ __forceinline__ void pin_all() { pin(q); pin(dm); pin(qh); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        L.off = u * BYTES;
+        run[0] = u;
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
+        Data d;
+        const uint16_t* h = (const uint16_t*)(row + (L.off + eo));
+        d.dm = HAS_M ? ((uint32_t)h[0] | ((uint32_t)h[1] << 16)) : (uint32_t)h[0];
+        d.qh = HAS_QH ? ((uint32_t)h[QH / 2] | ((uint32_t)h[QH / 2 + 1] << 16)) : 0u;
+        d.q = ((const U4A2*)(row + (L.off + eo) + QS))->v;
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
+        int acc[M][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int p = 0; p < 3; p++) acc[m][p] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t lo = D.q[j] & 0x0F0F0F0Fu, hi = (D.q[j] >> 4) & 0x0F0F0F0Fu;
+            if (HAS_QH) {   // bit k of a 4-bit field -> bit 4 of byte k
+                lo |= ((((D.qh >> (4 * j)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+                hi |= ((((D.qh >> (16 + 4 * j)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+            }
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int p = 0; p < 3; p++) {
+                    acc[m][p] = pdot<false>(p, xp[m][0][p][j], lo, acc[m][p]);
+                    acc[m][p] = pdot<false>(p, xp[m][0][p][4 + j], hi, acc[m][p]);
+                }
+        }
+        const float d = f16_bits(D.dm & 0xFFFFu), mn = HAS_M ? f16_bits(D.dm >> 16) : 0.f;
+#pragma unroll
+        for (int m = 0; m < M; m++)
+            out[m] = fmaf(d, fmaf(-(float)OFF, xsum[m][0], xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])), mn * xsum[m][0]);
+    }
+};
+typedef LegS<18, false, false, 8> Q40;
+typedef LegS<20, true, false, 0> Q41;
+typedef LegS<22, false, true, 16> Q50;
+typedef LegS<24, true, true, 0> Q51;
+
+// IQ4_NL (18 B = [f16 d][qs 16 B]) and IQ4_XS (136 B = [f16 d][u16 scales_h][scales_l 4 B][qs 128 B]): 4-bit indices into the
+// 16-level codebook {-127 .. 113} (crates/ferric-gguf/src/lib.rs:751-791), looked up four at a time by byte permute; the levels
+// are int8, so the activation planes are the balanced digits Q8_0 uses. Unit = one 32-value (sub-)block.
+__device__ __forceinline__ uint32_t lut16x4(uint32_t idx, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
+    uint32_t sel = idx & 0x07070707u;
+    uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel);   // selector 0..3: bytes of t0, 4..7: bytes of t1
+    uint32_t hi = __builtin_amdgcn_perm(t3, t2, sel);
+    uint32_t m = ((idx >> 3) & 0x01010101u) * 0xFFu;
+    return (hi & m) | (lo & ~m);
+}
+struct __attribute__((packed, aligned(8))) U4A8 { u32x4 v; };
+
+template <bool XS>
+struct IQ4S {
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = XS ? 256 : 32, U1 = 4;
+    static constexpr bool SIGNED_W = true;
+    struct Lane { uint32_t off_h, off_q, ib; };
+    struct Data {
+        u32x4 q; uint32_t h0, h1;
+        __device__ __forceinline__ void pin_all() { pin(q); pin(h0); pin(h1); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        if (XS) { L.ib = u & 7; L.off_h = (u >> 3) * 136; L.off_q = L.off_h + 8 + 16 * L.ib; }
+        else { L.ib = 0; L.off_h = u * 18; L.off_q = L.off_h + 2; }
+        run[0] = u;
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
+        Data d;
+        if (XS) {
+            d.h0 = *(const uint32_t*)(row + (L.off_h + eo));
+            d.h1 = *(const uint32_t*)(row + (L.off_h + eo) + 4);
+            d.q = ((const U4A8*)(row + (L.off_q + eo)))->v;
+        } else {
+            d.h0 = *(const uint16_t*)(row + (L.off_h + eo));
+            d.h1 = 0;
+            d.q = ((const U4A2*)(row + (L.off_q + eo)))->v;
+        }
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&)[M][NRUN], float (&out)[M]) {
+        // the codebook as int8 bytes, four levels per word
+        constexpr uint32_t T0 = 0xBFAD9881u, T1 = 0xF6EADDCFu, T2 = 0x26190D01u, T3 = 0x71594535u;
+        int acc[M][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int p = 0; p < 3; p++) acc[m][p] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t lo = lut16x4(D.q[j] & 0x0F0F0F0Fu, T0, T1, T2, T3), hi = lut16x4((D.q[j] >> 4) & 0x0F0F0F0Fu, T0, T1, T2, T3);
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int p = 0; p < 3; p++) {
+                    acc[m][p] = dot4(xp[m][0][p][j], lo, acc[m][p]);
+                    acc[m][p] = dot4(xp[m][0][p][4 + j], hi, acc[m][p]);
+                }
+        }
+        float dl = f16_bits(D.h0 & 0xFFFFu);
+        if (XS) {
+            int ls = (int)(((D.h1 >> (4 * L.ib)) & 0xFu) | ((((D.h0 >> 16) >> (2 * L.ib)) & 3u) << 4));
+            dl *= (float)(ls - 32);
+        }
+#pragma unroll
+        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])) * dl;
+    }
+};
+typedef IQ4S<false> IQ4NL;
+typedef IQ4S<true> IQ4XS;
+
+// MXFP4 (17 B = [u8 e][qs 16 B], crates/ferric-gguf/src/lib.rs:857-908): weight = k * 2^(e - 128) with k the doubled E2M1 value,
+// an integer in {0, +-1, +-2, +-3, +-4, +-6, +-8, +-12}: int8 codes and balanced activation planes as for IQ4, the power of two
+// applied to the block's integer dot product. The reference forms k * scale per element BEFORE it meets the activation
+// (crates/ferric-tensor/src/dtype.rs:3331-3344), which only differs where that product overflows (e >= 252): such a block takes
+// the element-by-element branch below, on the activations as the planes hold them (zeros stay zeros, so inf * 0 is still NaN).
+struct __attribute__((packed, aligned(1))) U4A1 { u32x4 v; };
+struct MXF4S {
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32, U1 = 4;
+    static constexpr bool SIGNED_W = true;
+    struct Lane { uint32_t off; };
+    struct Data {
+        u32x4 q; uint32_t e;
+        __device__ __forceinline__ void pin_all() { pin(q); pin(e); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        L.off = u * 17;
+        run[0] = u;
+    }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
+        Data d;
+        d.e = row[L.off + eo];
+        d.q = ((const U4A1*)(row + (L.off + eo) + 1))->v;
+        return d;
+    }
+    template <int M>
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&)[M][NRUN], float (&out)[M]) {
+        constexpr uint32_t T0 = 0x03020100u, T1 = 0x0C080604u, T2 = 0xFDFEFF00u, T3 = 0xF4F8FAFCu;
+        const float d = __uint_as_float(D.e == 0 ? (1u << 21) : D.e == 1 ? (1u << 22) : (D.e - 1u) << 23);
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            lo[j] = lut16x4(D.q[j] & 0x0F0F0F0Fu, T0, T1, T2, T3);
+            hi[j] = lut16x4((D.q[j] >> 4) & 0x0F0F0F0Fu, T0, T1, T2, T3);
+        }
+        if (D.e >= 252u) {   // a weight of this block may be +-inf: the reference's per-element products
+#pragma unroll 1
+            for (int m = 0; m < M; m++) {
+                float a = 0.f;
+#pragma unroll 1
+                for (int el = 0; el < 32; el++) {
+                    const int i = el >> 2, sh = 8 * (el & 3);
+                    const int v = ((int)(int8_t)(xp[m][0][0][i] >> sh)) * 65536 + ((int)(int8_t)(xp[m][0][1][i] >> sh)) * 256 +
+                                  (int)(int8_t)(xp[m][0][2][i] >> sh);
+                    const uint32_t kw = el < 16 ? lo[el >> 2] : hi[(el - 16) >> 2];
+                    const float w = (float)(int)(int8_t)(kw >> sh) * d;
+                    a = fmaf(xs[m][0] * (float)v, w, a);
+                }
+                out[m] = a;
+            }
+            return;
+        }
+        int acc[M][3];
+#pragma unroll
+        for (int m = 0; m < M; m++)
+#pragma unroll
+            for (int p = 0; p < 3; p++) acc[m][p] = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int m = 0; m < M; m++)
+#pragma unroll
+                for (int p = 0; p < 3; p++) {
+                    acc[m][p] = dot4(xp[m][0][p][j], lo[j], acc[m][p]);
+                    acc[m][p] = dot4(xp[m][0][p][4 + j], hi[j], acc[m][p]);
+                }
+#pragma unroll
+        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])) * d;
+    }
+};
+
 struct GemvParams {
     const uint8_t* W;
     const float* x;      // [M, cols]
@@ -292,7 +566,7 @@ constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
 // Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit 128 VGPRs
 // at batch 1 (16 waves per CU). Measured: 16 waves with 3 rows in flight beat 12 waves with 6-8 in flight
 // on every shape but the 638 MB head, and there by 6 % only.
-template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? (F::WPL == 64 ? (F::RUN == 16 ? 2 : 3) : 4) : 2; }
+template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? F::U1 : 2; }
 // Activation rows one pass can hold in registers (48 plane dwords per row for the 64-weight units, 24 for Q8_0).
 template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
 
@@ -673,8 +947,19 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
         case FHIP_Q8_0:
             if (n_ff) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "matmul_q_swiglu: no fused kernel for Q8_0");
             return launch_fmt<Q80, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
-        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_Q5_K: case FHIP_IQ4_NL: case FHIP_IQ4_XS: case FHIP_MXFP4:
-            return launch_gemv_generic(w, d_x, rows_x, d_y, n_ff, s);   // no streaming kernel for these formats
+        case FHIP_Q5_K: return n_ff ? launch_fmt<Q5K, true>(w, d_x, rows_x, d_y, out_rows, n_ff, s) : launch_fmt<Q5K, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1:
+            if (n_ff) return launch_gemv_generic(w, d_x, rows_x, d_y, n_ff, s);   // reports that these formats have no fused SwiGLU
+            if (w->type == FHIP_Q4_0) return launch_fmt<Q40, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+            if (w->type == FHIP_Q4_1) return launch_fmt<Q41, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+            if (w->type == FHIP_Q5_0) return launch_fmt<Q50, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+            return launch_fmt<Q51, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+        case FHIP_IQ4_NL: case FHIP_IQ4_XS:
+            if (n_ff) return launch_gemv_generic(w, d_x, rows_x, d_y, n_ff, s);
+            return w->type == FHIP_IQ4_NL ? launch_fmt<IQ4NL, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s)
+                                          : launch_fmt<IQ4XS, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
+        case FHIP_MXFP4:
+            return n_ff ? launch_gemv_generic(w, d_x, rows_x, d_y, n_ff, s) : launch_fmt<MXF4S, false>(w, d_x, rows_x, d_y, out_rows, n_ff, s);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }
@@ -695,8 +980,16 @@ int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t 
         case FHIP_Q4_K: return launch_norm_fmt<Q4K>(w, d_x, d_y, out_rows, n_ff != 0, norm, s);
         case FHIP_Q6_K: return launch_norm_fmt<Q6K>(w, d_x, d_y, out_rows, n_ff != 0, norm, s);
         case FHIP_Q8_0: return n_ff ? NORM_NOT_FUSED : launch_norm_fmt<Q80>(w, d_x, d_y, out_rows, false, norm, s);
+        case FHIP_Q5_K: return launch_norm_fmt<Q5K>(w, d_x, d_y, out_rows, n_ff != 0, norm, s);
         default: return NORM_NOT_FUSED;
     }
+}
+
+// the same without the fused-SwiGLU instantiation (formats the reference has no fused gate/up kernel for)
+template <class F>
+int launch_sel_plain(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, const SelParams& sel, hipStream_t s) {
+    if (max_batch<F, false>(w, 1) == 0) return launch_gemv_generic_sel(w, d_x, d_y, out_rows, false, sel, s);
+    return launch_one<F, 1, false>(w, d_x, d_y, out_rows, s, &sel);
 }
 
 template <class F>
@@ -713,8 +1006,18 @@ int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t o
         case FHIP_Q4_K: return launch_sel_fmt<Q4K>(w, d_x, d_y, out_rows, swiglu, sel, s);
         case FHIP_Q6_K: return launch_sel_fmt<Q6K>(w, d_x, d_y, out_rows, swiglu, sel, s);
         case FHIP_Q8_0: return launch_sel_fmt<Q80>(w, d_x, d_y, out_rows, swiglu, sel, s);
-        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1: case FHIP_Q5_K: case FHIP_IQ4_NL: case FHIP_IQ4_XS: case FHIP_MXFP4:
-            return launch_gemv_generic_sel(w, d_x, d_y, out_rows, swiglu, sel, s);
+        case FHIP_Q5_K: return launch_sel_fmt<Q5K>(w, d_x, d_y, out_rows, swiglu, sel, s);
+        case FHIP_Q4_0: case FHIP_Q4_1: case FHIP_Q5_0: case FHIP_Q5_1:
+            if (swiglu) return launch_gemv_generic_sel(w, d_x, d_y, out_rows, swiglu, sel, s);
+            if (w->type == FHIP_Q4_0) return launch_sel_plain<Q40>(w, d_x, d_y, out_rows, sel, s);
+            if (w->type == FHIP_Q4_1) return launch_sel_plain<Q41>(w, d_x, d_y, out_rows, sel, s);
+            if (w->type == FHIP_Q5_0) return launch_sel_plain<Q50>(w, d_x, d_y, out_rows, sel, s);
+            return launch_sel_plain<Q51>(w, d_x, d_y, out_rows, sel, s);
+        case FHIP_IQ4_NL: case FHIP_IQ4_XS:
+            if (swiglu) return launch_gemv_generic_sel(w, d_x, d_y, out_rows, swiglu, sel, s);
+            return w->type == FHIP_IQ4_NL ? launch_sel_plain<IQ4NL>(w, d_x, d_y, out_rows, sel, s) : launch_sel_plain<IQ4XS>(w, d_x, d_y, out_rows, sel, s);
+        case FHIP_MXFP4:
+            return swiglu ? launch_gemv_generic_sel(w, d_x, d_y, out_rows, swiglu, sel, s) : launch_sel_plain<MXF4S>(w, d_x, d_y, out_rows, sel, s);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

@@ -187,6 +187,31 @@ def test_mxfp4_matvec_forms_the_weight_before_it_meets_the_activation(F, O):
     assert F.Tensor.from_vec(x, (1, 32)).matmul_q(one).to_vec()[0] == np.float32(2.0 ** 126)    # finite at the top scale
 
 
+def test_mxfp4_saturating_blocks_through_the_streaming_kernel(F, O):
+    # a row long enough for the integer-plane kernel (512 columns): blocks whose scale byte can overflow the weight (e >= 252)
+    # must still give the reference's x * (k * scale) per element -- inf where a product overflows, NaN where inf meets a zero
+    # activation -- and ordinary blocks beside them must not be disturbed
+    rng = np.random.default_rng(21)
+    rows, cols = 24, 512
+    blk = rng.integers(0, 256, (rows, cols // 32, 17), dtype=np.uint8)
+    blk[:, :, 0] = rng.integers(0x70, 0x80, (rows, cols // 32), dtype=np.uint8)
+    blk[3, 5, 0], blk[7, 0, 0], blk[7, 9, 0], blk[11, 15, 0], blk[12, 2, 0] = 255, 254, 253, 252, 251
+    raw = blk.reshape(-1)
+    w = F.QMatrix.from_bytes(raw, MXFP4, rows, cols)
+    wd = O.deq_raw(raw, rows * cols, MXFP4).reshape(rows, cols)
+    x = rng.standard_normal(cols).astype(np.float32)
+    x[5 * 32: 5 * 32 + 8] = 0.0                                           # zeros under the e = 255 block of row 3
+    y = F.Tensor.from_vec(x, (1, cols)).matmul_q(w).to_vec()
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = (wd.astype(np.float64) * x.astype(np.float64)).sum(axis=1)
+    plain = [r for r in range(rows) if r not in (3, 7, 11, 12)]
+    assert np.abs(y[plain] - want[plain]).max() <= 1e-5 * np.abs(want[plain]).max()     # ordinary rows, beside the special blocks
+    assert np.isnan(y[3])                                                 # inf weights over zero activations
+    assert not np.isfinite(y[7])                                          # e = 254 / 253: weights of both signs overflow
+    for r in (11, 12):                                                    # e = 252 / 251: finite weights near the top of f32; the f32
+        assert np.isinf(y[r]) or abs(y[r] - want[r]) <= 1e-5 * abs(want[r])   # sum may overflow, but it may not be NaN or wrong
+
+
 def test_iq4_xs_packed_kernel_matches_the_dense_reference(F, O):
     # crates/ferric-tensor/examples/iq4_xs.rs restated: its block generator, its activation ramp, its shapes and its bar
     # (max |got - want| / max |want| < 1e-5 against the dense product of the dequantized weight)
