@@ -117,6 +117,40 @@ def test_kv_append2_and_decode_attention(F, X, D):
         X.decode_attention(F.Tensor.from_vec(np.zeros((1, 9 * 64), np.float32), (1, 9 * 64)), X.KvCache(4, 64), 9, 1, length=1)
 
 
+def test_empty_inputs_and_argument_errors(F, X):
+    """Zero-sized calls return without touching memory; bad shapes and NULL pointers are reported, never launched."""
+    lib, chk, E = F._lib.load(), F._lib.check, F._lib.FerricHipError
+    t = F.Tensor.from_vec(np.ones(256, np.float32), (2, 128))
+    o = F.Tensor.from_vec(np.full(256, 5.0, np.float32), (2, 128))
+    w = F.Tensor.from_vec(np.ones(128, np.float32), (128,))
+    pos = X._u32_tensor([0, 1])
+    chk(lib.fhip_rmsnorm(t.buf.ptr, w.buf.ptr, 0, 128, 1e-6, o.buf.ptr, None))
+    chk(lib.fhip_add_rmsnorm(t.buf.ptr, t.buf.ptr, w.buf.ptr, 2, 0, 1e-6, o.buf.ptr, o.buf.ptr, None))
+    chk(lib.fhip_add(t.buf.ptr, t.buf.ptr, 0, o.buf.ptr, None))
+    chk(lib.fhip_rope(t.buf.ptr, 0, 0, 1, 128, 128, 1e4, None, 0, None, 0, o.buf.ptr, None))
+    chk(lib.fhip_kv_append2(t.buf.ptr, t.buf.ptr, 0, 128, None, 0, o.buf.ptr, o.buf.ptr, 2, None))
+    chk(lib.fhip_qkv_post(t.buf.ptr, None, None, None, pos.buf.ptr, None, 0, 1, 1, 64, 64, 0, 1e-6, 1e4, o.buf.ptr, o.buf.ptr, o.buf.ptr, 2, None))
+    chk(lib.fhip_u32_add(pos.buf.ptr, 0, 1, None))
+    assert np.array_equal(o.to_vec(), np.full(256, 5.0, np.float32))                      # nothing was written
+    assert lib.fhip_decode_attention_ws_bytes(8, 2, 64, 0) == 0
+    for call, msg in [
+        (lambda: lib.fhip_rmsnorm(None, w.buf.ptr, 1, 128, 1e-6, o.buf.ptr, None), "NULL pointer"),
+        (lambda: lib.fhip_rope(t.buf.ptr, 0, 2, 1, 128, 130, 1e4, None, 0, None, 0, o.buf.ptr, None), "n_rot must be even and <= head_dim"),
+        (lambda: lib.fhip_rope(t.buf.ptr, 0, 2, 1, 128, 7, 1e4, None, 0, None, 0, o.buf.ptr, None), "n_rot must be even"),
+        (lambda: lib.fhip_decode_attention(t.buf.ptr, t.buf.ptr, t.buf.ptr, 2, 1, 64, 0, None, None, o.buf.ptr, None), "empty cache"),
+        (lambda: lib.fhip_decode_attention(t.buf.ptr, t.buf.ptr, t.buf.ptr, 3, 2, 64, 1, None, None, o.buf.ptr, None), "multiple of n_kv_heads"),
+        (lambda: lib.fhip_decode_attention(t.buf.ptr, t.buf.ptr, t.buf.ptr, 2, 1, 32, 1, None, None, o.buf.ptr, None), "head_dim must be 64 or 128"),
+        (lambda: lib.fhip_qkv_post(t.buf.ptr, None, None, None, None, None, 1, 1, 1, 64, 64, 0, 1e-6, 1e4, o.buf.ptr, o.buf.ptr, o.buf.ptr, 2, None), "NULL pointer"),
+        (lambda: lib.fhip_norm_matmul_q(None, t.buf.ptr, None, w.buf.ptr, 1e-6, None, o.buf.ptr, 0, o.buf.ptr, None), "NULL pointer"),
+    ]:
+        with pytest.raises((E, AssertionError), match=msg):
+            chk(call())
+    # a long cache without its workspace is refused, not run with a NULL scratch
+    with pytest.raises(E, match="needs the workspace"):
+        big = X.KvCache(4096, 64)
+        chk(lib.fhip_decode_attention(t.buf.ptr, big.k.buf.ptr, big.v.buf.ptr, 2, 1, 64, 4096, None, None, o.buf.ptr, None))
+
+
 def test_attention_window_and_softcap(F, X, D):
     rng = np.random.default_rng(12)
     for nh, nkv, hd, s in [(40, 8, 128, 1500), (8, 2, 64, 70)]:
