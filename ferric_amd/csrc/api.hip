@@ -478,6 +478,11 @@ int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_re
     return fhip::launch_gemv(w, d_h_scratch, 1, d_y, n_ff, (hipStream_t)stream);
 }
 
+int fhip_debug_generic_matvec(int on) {
+    fhip::gemv_force_generic(on != 0);
+    return FHIP_OK;
+}
+
 int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream) {
     int rc = need_init();
     if (rc) return rc;

@@ -71,6 +71,7 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
 // gemv_generic.hip: same contract, any cols the format allows (up to 32768)
 int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s);
+void gemv_force_generic(bool on);   // debugging / tests: every mat-vec through gemv_generic.hip
 // One batch-1 GEMV per (token, slot) pair on the selected expert's `out_rows` rows (fused SwiGLU over its
 // gate|up halves when swiglu: then expert_rows = 2 * out_rows). Both files provide it, same contract as above.
 int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s);

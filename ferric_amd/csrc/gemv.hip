@@ -546,7 +546,8 @@ struct GemvParams {
     int cols;
     size_t row_bytes;
     size_t pair_bytes;   // fused SwiGLU: byte distance from gate row r to up row r (= n_ff * row_bytes)
-    int NG;              // 16-lane slots per row = cols / (16 * WPL)
+    int NG;              // 16-lane slots per row = ceil(units / 16)
+    int units;           // units per row = cols / WPL; the last slot may be partly filled
     int RF;              // replicas of the full-wave set, each taking every RF-th row (balances them against the tail wave)
     int G;               // row groups per workgroup
     int rpg;             // output rows per row group
@@ -601,7 +602,9 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     else { group = 4 * NGF + (NT == 2 ? (slot & 1) : 0); row_off = NT == 2 ? (slot >> 1) : slot; }
     typename F::Lane L;
     int run[NRUN];
-    F::setup(group * 16 + l16, L, run);
+    // a lane past the row's last unit (rows whose length does not fill the last slot) works on unit 0 and contributes 0
+    const bool unit_ok = group * 16 + l16 < p.units;
+    F::setup(unit_ok ? group * 16 + l16 : 0, L, run);
 
     const int r0 = (blockIdx.x * p.G + rg) * p.rpg;
     int nrows = p.out_rows - r0;
@@ -743,7 +746,7 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
         const bool ok = lane_ok && v < nv;
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            float t = slot_sum(acc[m]);
+            float t = slot_sum(unit_ok ? acc[m] : 0.f);
             if (ok && l16 == 0) mypart[((size_t)v * p.NG + group) * M + m] = t;
         }
     };
@@ -814,6 +817,8 @@ __global__ void zero_kernel(float* __restrict__ out, size_t n) {
     if (i < n) out[i] = 0.f;
 }
 
+bool g_force_generic = false;   // tests: send every shape to the shape-complete f32 kernel
+
 int env_int(const char* name, int dflt) {
     const char* v = getenv(name);
     return v && *v ? atoi(v) : dflt;
@@ -856,7 +861,8 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
     p.pair_bytes = SWIGLU ? out_rows * w->row_bytes : 0;
     p.sel = sel ? *sel : fhip::SelParams{nullptr, 0, 0, 0, 0, 0, 1};
-    p.NG = (int)(w->cols / (16 * F::WPL));
+    p.units = (int)(w->cols / F::WPL);
+    p.NG = (p.units + 15) / 16;
     constexpr int MAXW = max_threads(M) / 64;
     p.RF = full_wave_replicas(p.NG, MAXW);
     const int WPR = waves_per_row_group(p.NG, MAXW);
@@ -897,8 +903,8 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
 // Largest batch width (4, 2, 1, or 0 = shape not covered) whose workgroup fits the wave and LDS limits.
 template <class F, bool SWIGLU>
 int max_batch(const fhip_weight* w, size_t left) {
-    if (w->cols % (16 * F::WPL) != 0) return 0;
-    const int NG = (int)(w->cols / (16 * F::WPL));
+    if (w->cols % F::WPL != 0 || g_force_generic) return 0;
+    const int NG = (int)((w->cols / F::WPL + 15) / 16);
     auto WPRm = [&](int m) { return waves_per_row_group(NG, max_threads(m) / 64); };
     const size_t cap = fhip::device_lds_bytes();
     if (left >= 4 && max_m<F>() >= 4 && WPRm(4) * 64 <= max_threads(4) && lds_bytes<F, 4, SWIGLU>(w->cols, NG, max_threads(4) / 64 / WPRm(4), 256) <= cap) return 4;
@@ -1021,6 +1027,8 @@ int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t o
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }
+
+void gemv_force_generic(bool on) { g_force_generic = on; }
 
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s) {
     size_t n = t * d;

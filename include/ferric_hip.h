@@ -266,6 +266,10 @@ int fhip_decode_attention_ex(const float* d_q, const float* d_k_cache, const flo
 int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_resid, const float* d_norm_w, float eps, float* d_x_out,
                        float* d_h_scratch, int swiglu, float* d_y, void* stream);
 
+/* Debugging and tests: on != 0 sends every mat-vec to the shape-complete f32 kernel instead of the streaming one (process-wide,
+ * not thread-safe against concurrent launches). No counterpart in the reference. */
+int fhip_debug_generic_matvec(int on);
+
 /* words[i] += delta for n device u32 words: advances the position word(s) at the end of a captured decode step. */
 int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream);
 

@@ -241,3 +241,34 @@ def test_iq4_xs_packed_kernel_matches_the_dense_reference(F, O):
         want = deq.astype(np.float64) @ xv.astype(np.float64)
         got = F.Tensor.from_vec(xv, (1, cols)).matmul_iq4_xs(F.Iq4XsWeights.from_bytes(raw, rows, cols)).to_vec()
         assert np.abs(got - want).max() / max(1e-6, np.abs(want).max()) < 1e-5, (rows, cols)
+
+
+def test_the_shape_complete_f32_kernel_still_agrees(F, O):
+    """Every legal row length now runs the streaming kernel; the f32 kernel behind it stays the fallback for rows too long
+    for one workgroup. Forced on here so that it keeps its own parity check, for every format."""
+    from ferric_amd.synth import synth_weights
+    lib = F._lib.load()
+    rng = np.random.default_rng(31)
+    geom = dict(GEOM); geom.update({Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)})
+    F._lib.check(lib.fhip_debug_generic_matvec(1))
+    try:
+        for ty, (vals, _) in geom.items():
+            for rows, cols, b in [(70, vals * 3, 1), (33, 5120, 2), (40, 1024, 3)]:
+                raw = synth_weights(ty, rows, cols, rows + ty)
+                w = F.QMatrix.from_bytes(raw, ty, rows, cols)
+                x = rng.standard_normal((b, cols)).astype(np.float32)
+                y = F.Tensor.from_vec(x.reshape(-1), (b, cols)).matmul_q(w).to_vec().reshape(b, rows)
+                y64, wn = O.matmul_f64(x, raw, ty, rows, cols)
+                assert (np.abs(y - y64) <= 1e-3 * wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None]).all(), (ty, rows, cols)
+                assert np.abs(y - y64).max() <= 1e-5 * max(1e-3, np.abs(y64).max()), (ty, rows, cols)
+        n_ff = 96
+        for ty in (Q4_K, Q6_K, Q5_K):
+            raw = synth_weights(ty, 2 * n_ff, 768, 5)
+            w = F.QMatrix.from_bytes(raw, ty, 2 * n_ff, 768)
+            x = rng.standard_normal((2, 768)).astype(np.float32)
+            got = F.Tensor.from_vec(x.reshape(-1), (2, 768)).try_matmul_swiglu(w).to_vec().reshape(2, n_ff)
+            g64, _ = O.matmul_f64(x, raw, ty, 2 * n_ff, 768)
+            want = g64[:, :n_ff] / (1 + np.exp(-g64[:, :n_ff])) * g64[:, n_ff:]
+            assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max(), ty
+    finally:
+        F._lib.check(lib.fhip_debug_generic_matvec(0))
