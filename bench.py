@@ -365,6 +365,37 @@ def probe_prefill(F, lib, check):
             check(lib.fhip_stream_sync(None))
 
 
+def probe_decode(F, lib, check):
+    """Work for a hardware-counter run on the decode attention kernel: a copy of known size (calibrates FETCH_SIZE /
+    WRITE_SIZE), then 8 launches of fhip_decode_attention on 8 different caches of 4096 rows (40 query / 8 KV heads x 128:
+    33.6 MB of K and V rows each, none touched before), then 8 at 128 rows."""
+    from ferric_amd import decode as X
+    n = 256 << 20
+    src, dst = F.DeviceBuffer(n), F.DeviceBuffer(n)
+    check(lib.fhip_memset(src.ptr, 1, n, None))
+    check(lib.fhip_stream_sync(None))
+    check(lib.fhip_memcpy_d2d(dst.ptr, src.ptr, n, None))
+    check(lib.fhip_stream_sync(None))
+    nh, nkv, hd = 40, 8, 128
+    rng = np.random.default_rng(3)
+    fill = (rng.standard_normal((4096, nkv * hd)) * 0.5).astype(np.float32)
+    caches = []
+    for _ in range(8):
+        c = X.KvCache(4096, nkv * hd)
+        check(lib.fhip_memcpy_h2d(c.k.buf.ptr, fill.ctypes.data_as(C.c_void_p), fill.nbytes, None))
+        check(lib.fhip_memcpy_h2d(c.v.buf.ptr, fill.ctypes.data_as(C.c_void_p), fill.nbytes, None))
+        c.len = 4096
+        caches.append(c)
+    check(lib.fhip_stream_sync(None))
+    check(lib.fhip_memcpy_d2d(dst.ptr, src.ptr, n, None))          # pushes the freshly written caches out of the cache levels
+    check(lib.fhip_stream_sync(None))
+    q = F.Tensor.from_vec(rng.standard_normal(nh * hd).astype(np.float32), (1, nh * hd))
+    for length in (4096, 128):
+        for c in caches:
+            X.decode_attention(q, c, nh, nkv, length=length)
+    check(lib.fhip_stream_sync(None))
+
+
 def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
     """The reference's CPU route for Q4_K (deq_raw then a sequential f32 dot per row, rows split in
     contiguous spans over threads), timed through the C oracle on this host's cores."""
@@ -406,6 +437,8 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for rocprofv3 --pmc: one 256 MiB device copy (calibration), then 16 cold Q4_K 5120x5120 "
                          "GEMVs, one fused gate|up 34816x5120 and one Q6_K 5120x17408 GEMV; prints nothing else")
+    ap.add_argument("--probe-decode", action="store_true",
+                    help="profiler probe for the decode attention kernel: 8 launches each at 4096 and 128 cached rows; prints nothing else")
     ap.add_argument("--probe-prefill", action="store_true",
                     help="profiler probe for the matrix-core GEMM: Q4_K 5120x5120 and 34816x5120 at T = 2048, 128 and 8, "
                          "5 launches each; prints nothing else")
@@ -426,6 +459,9 @@ def main():
         return
     if args.probe_prefill:
         probe_prefill(F, lib, check)
+        return
+    if args.probe_decode:
+        probe_decode(F, lib, check)
         return
     log("[bench] Q4_K GEMV 5120x5120 ...")
     c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
