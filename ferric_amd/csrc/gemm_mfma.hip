@@ -77,6 +77,7 @@ __device__ __forceinline__ constexpr int kcol(int t, int h) { return 32 * (t >> 
 
 struct Q4K {
     static constexpr int BLOCK = 144;
+    static constexpr float UNPACK_US = 1.4f;   // unpack of a 256 x 256 chunk by one workgroup (fitted, see plan_cost_us)
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 hd, hdn, q[4]; };
@@ -130,6 +131,7 @@ struct Q6K {
     // ql for G even, high nibbles for G odd); slice T is group g = g0 + (T >> 1), l = 16h + 8(T & 1) + [0, 8),
     // whose scale is sc[8hf + 2g + h]  (crates/ferric-gguf/src/lib.rs:833-851).
     static constexpr int BLOCK = 210;
+    static constexpr float UNPACK_US = 2.3f;
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 ql[2][2], qh[2], sc, scn; uint32_t d, dn; };
@@ -194,6 +196,7 @@ struct Q80 {
     // elements 16h + 8(T & 1) + [0, 8). A trailing partial chunk is allowed: blocks past the row's end are
     // read from the last valid block's address and given scale 0 (their activations are staged as 0 too).
     static constexpr int BLOCK = 34;
+    static constexpr float UNPACK_US = 5.1f;
     static constexpr bool PARTIAL = true;   // a row may end inside a chunk
     static __host__ __device__ int chunks(int K) { return (K + 255) / 256; }
     struct Raw { u32x4 q[4][2]; uint32_t d[4][2]; };
@@ -625,40 +628,84 @@ int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
+// How a launch of the tiled kernel with tile height 64 * mi is dealt to the chip: `whole_rounds` whole tiles per workgroup,
+// then the left-over tiles cut along K into runs of `per` chunks.
+struct TilePlan {
+    int whole_rounds, per;
+    long long left, units, split_wgs;   // left-over tiles, their chunks, workgroups that add a partial run atomically
+    unsigned grid;
+};
+
+static TilePlan plan_tiles(long long tiles_n, int nchunks, size_t t, int mi, long long cus) {
+    TilePlan q;
+    const long long tiles = tiles_n * (long long)((t + 64 * mi - 1) / (64 * mi));
+    q.whole_rounds = (int)(tiles / cus);
+    q.left = tiles - q.whole_rounds * cus;
+    q.units = q.left * nchunks;
+    long long per = (q.units + cus - 1) / cus;
+    // a run shorter than a tile's K that is close to it is rounded up to whole tiles: no atomics, no clearing
+    if (per * 4 >= (long long)nchunks * 3) per = nchunks;
+    if (per < 1) per = 1;
+    q.per = (int)per;
+    const long long runs = (q.units + per - 1) / per;
+    q.grid = q.whole_rounds > 0 ? (unsigned)cus : (unsigned)runs;
+    q.split_wgs = (q.left > 0 && per % nchunks != 0) ? runs : 0;
+    return q;
+}
+
+// Estimated duration of a plan in us: chunks per workgroup x (unpack of a 256 x 256 weight chunk + mi MFMA slabs of 64 rows),
+// plus the atomic epilogue of the split runs (a tile of 64 * mi x 256 f32 per workgroup; the chip retires about 380 G
+// f32 atomics a second, 11 us for 64 x 256 from each of 256 workgroups). Constants fitted to measured launches (Q4_K
+// 34816 x 5120, T = 2048: 8.3 us a chunk at mi = 4, 4.85 at mi = 2; Q6_K and Q8_0 likewise) and checked against 21 shapes:
+// the model ranks the tile heights like the measurement wherever they differ by more than 6 %.
+template <class F>
+static float plan_cost_us(const TilePlan& q, int nchunks, int mi, long long cus) {
+    const float chunk_us = F::UNPACK_US + 1.75f * (float)mi;
+    const float chunks = (float)q.whole_rounds * (float)nchunks + (q.left > 0 ? (float)q.per : 0.f);
+    return chunks * chunk_us + 11.f * (float)mi * (float)q.split_wgs / (float)cus;
+}
+
 template <class F, int MI>
-int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s) {
+int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, const TilePlan& q, long long cus) {
     GemmParams p;
     p.W = w->d_raw; p.X = d_x; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
     p.nblk = (int)(w->row_bytes / F::BLOCK);
     p.nchunks = F::chunks(p.K);
     p.tiles_n = (int)((w->rows + 255) / 256);
-    const int tiles_t = (int)((t + 64 * MI - 1) / (64 * MI));
-    const long long tiles = (long long)p.tiles_n * tiles_t;
     // one workgroup per CU (its LDS tiles take most of a CU's 160 KB)
-    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    p.whole_rounds = (int)(tiles / cus);
-    const long long left = tiles - p.whole_rounds * cus;
-    p.units = left * p.nchunks;
-    long long per = (p.units + cus - 1) / cus;
-    // a run shorter than a tile's K that is close to it is rounded up to whole tiles: no atomics, no clearing
-    if (per * 4 >= (long long)p.nchunks * 3) per = p.nchunks;
-    if (per < 1) per = 1;
-    p.per = (int)per;
-    const unsigned grid = p.whole_rounds > 0 ? (unsigned)cus : (unsigned)((p.units + per - 1) / per);
-    if (left > 0 && per % p.nchunks != 0)
-        hipLaunchKernelGGL(zero_split_tiles_kernel, dim3((unsigned)left), dim3(256), 0, s, d_y, p.T, p.N, 64 * MI,
+    p.whole_rounds = q.whole_rounds;
+    p.units = q.units;
+    p.per = q.per;
+    if (q.split_wgs > 0)
+        hipLaunchKernelGGL(zero_split_tiles_kernel, dim3((unsigned)q.left), dim3(256), 0, s, d_y, p.T, p.N, 64 * MI,
                            p.tiles_n, p.nchunks, p.per, (int)(p.whole_rounds * cus));
-    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(grid), dim3(512), 0, s, p);
+    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(q.grid), dim3(512), 0, s, p);
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
 template <class F>
 int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
     if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, y_cleared);
-    if (t > 128) return launch_cfg<F, 4>(w, d_x, t, d_y, s);  // 256 x 256 workgroup tile
-    if (t > 64) return launch_cfg<F, 2>(w, d_x, t, d_y, s);
-    return launch_cfg<F, 1>(w, d_x, t, d_y, s);
+    // Tile height 64 * MI. The 256 x 256 tile unpacks each weight once per 256 activation rows, but when there is no whole
+    // round of such tiles for the chip every tile is cut along K, each workgroup adds a whole tile atomically for a few
+    // chunks of work, and a lower tile (twice the tiles, half the atomics, longer runs) can win: the estimate decides
+    // (measured, Q4_K 5120 x 5120: T = 512 78 -> 63 us and T = 1024 109 -> 91 us with 128-row tiles, T = 128 36 -> 30 us with
+    // 64-row tiles; Q6_K 5120 x 17408 and Q8_0, dearer to unpack, keep the tall tile from T = 512 on).
+    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256, tiles_n = (long long)((w->rows + 255) / 256);
+    const int nchunks = F::chunks((int)w->cols);
+    TilePlan q[3];
+    float cost[3];
+    int best = 0;
+    for (int i = 0; i < 3; i++) {
+        const int mi = 4 >> i;
+        q[i] = plan_tiles(tiles_n, nchunks, t, mi, cus);
+        cost[i] = plan_cost_us<F>(q[i], nchunks, mi, cus);
+        if (cost[i] < cost[best]) best = i;
+    }
+    if (best == 0) return launch_cfg<F, 4>(w, d_x, t, d_y, s, q[0], cus);
+    if (best == 1) return launch_cfg<F, 2>(w, d_x, t, d_y, s, q[1], cus);
+    return launch_cfg<F, 1>(w, d_x, t, d_y, s, q[2], cus);
 }
 
 // f32 -> bf16 (round to nearest even), 8 values per thread; `n8` full groups of 8, the tail one by one
