@@ -80,6 +80,10 @@ SYMBOLS = {
     "fhip_matmul_q_coop": (C.c_int, [_vp, _vp, _sz, _vp, _vp, _vp]),
     "fhip_ffn_coop_ws_bytes": (_sz, [_vp, _vp, _sz]),
     "fhip_ffn_coop": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _vp, _vp]),
+    "fhip_matmul_q_f16x2_ws_bytes": (_sz, [_vp, _sz]),
+    "fhip_matmul_q_f16x2": (C.c_int, [_vp, _vp, _sz, _vp, _vp, _vp]),
+    "fhip_ffn_f16x2_ws_bytes": (_sz, [_vp, _vp, _sz]),
+    "fhip_ffn_f16x2": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _vp, _vp]),
     "fhip_rmsnorm": (C.c_int, [_vp, _vp, _sz, _sz, C.c_float, _vp, _vp]),
     "fhip_add_rmsnorm": (C.c_int, [_vp, _vp, _vp, _sz, _sz, C.c_float, _vp, _vp, _vp]),
     "fhip_add": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),

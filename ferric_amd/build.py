@@ -24,6 +24,7 @@ UNITS = {
     "gemv.hip": [],
     "gemv_generic.hip": [],
     "gemm_mfma.hip": [],
+    "gemm_f16x2.hip": [],
     "moe.hip": [],
     "decode_ops.hip": [],
     "gguf.hip": [],

@@ -602,6 +602,67 @@ int fhip_ffn_coop(const fhip_weight* gu, const fhip_weight* down, const float* d
     return fhip::launch_gemm_bf16(down, hb, rows_x, d_y, s, clr);
 }
 
+size_t fhip_matmul_q_f16x2_ws_bytes(const fhip_weight* w, size_t rows_x) {
+    if (!fhip::gemm_f16x2_supports(w, rows_x)) return 0;
+    return align256(fhip::gemm_f16x2_xp_bytes(w, rows_x)) + align256(fhip::gemm_f16x2_aux_bytes());
+}
+
+static int f16x2_checks(const char* who, const fhip_weight* w, size_t rows_x) {
+    if (rows_x > 32) return set_error(FHIP_ERR_SHAPE, "%s: at most 32 activation rows (got %zu)", who, rows_x);
+    if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K)
+        return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "%s: no kernel for ggml type %u (Q4_K and Q6_K only)", who, w->type);
+    return FHIP_OK;
+}
+
+int fhip_matmul_q_f16x2(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, void* d_ws, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!w) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_f16x2: NULL weight");
+    if ((rc = f16x2_checks("fhip_matmul_q_f16x2", w, rows_x))) return rc;
+    if (rows_x == 0 || w->rows == 0) return FHIP_OK;
+    if (!d_x || !d_y || !d_ws) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_f16x2: NULL pointer");
+    if (((uintptr_t)d_ws & 255) != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_f16x2: workspace must be 256-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    uint16_t* xp = (uint16_t*)d_ws;
+    float* rs = (float*)((uint8_t*)d_ws + align256(fhip::gemm_f16x2_xp_bytes(w, rows_x)));
+    const bool clr = fhip::gemm_f16x2_adds_into_y(w, rows_x);   // then the split clears y on the side
+    if ((rc = fhip::launch_xsplit_f16(w, d_x, rows_x, false, xp, rs, s, clr ? d_y : nullptr, clr ? rows_x * w->rows : 0))) return rc;
+    return fhip::launch_gemm_f16x2(w, xp, rs, rows_x, d_y, s, clr);
+}
+
+size_t fhip_ffn_f16x2_ws_bytes(const fhip_weight* gu, const fhip_weight* down, size_t rows_x) {
+    if (!fhip::gemm_f16x2_supports(gu, rows_x) || !fhip::gemm_f16x2_supports(down, rows_x)) return 0;
+    return align256(fhip::gemm_f16x2_xp_bytes(gu, rows_x)) + align256(rows_x * gu->rows * 4) +
+           align256(fhip::gemm_f16x2_xp_bytes(down, rows_x)) + 2 * align256(fhip::gemm_f16x2_aux_bytes());
+}
+
+int fhip_ffn_f16x2(const fhip_weight* gu, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y, void* d_ws,
+                   void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!gu || !down) return set_error(FHIP_ERR_ARG, "fhip_ffn_f16x2: NULL weight");
+    if (gu->rows % 2 != 0) return set_error(FHIP_ERR_SHAPE, "ffn: gate_up rows must be even");
+    const size_t n_ff = gu->rows / 2;
+    if (down->cols != n_ff) return set_error(FHIP_ERR_SHAPE, "down in dim must equal n_ff");
+    if ((rc = f16x2_checks("fhip_ffn_f16x2", gu, rows_x)) || (rc = f16x2_checks("fhip_ffn_f16x2", down, rows_x))) return rc;
+    if (rows_x == 0) return FHIP_OK;
+    if (!d_x || !d_y || !d_ws) return set_error(FHIP_ERR_ARG, "fhip_ffn_f16x2: NULL pointer");
+    if (((uintptr_t)d_ws & 255) != 0) return set_error(FHIP_ERR_ARG, "fhip_ffn_f16x2: workspace must be 256-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    uint8_t* ws = (uint8_t*)d_ws;
+    uint16_t* xp1 = (uint16_t*)ws;
+    float* rs1 = (float*)(ws + align256(fhip::gemm_f16x2_xp_bytes(gu, rows_x)));
+    float* g = (float*)((uint8_t*)rs1 + align256(fhip::gemm_f16x2_aux_bytes()));
+    uint16_t* xp2 = (uint16_t*)((uint8_t*)g + align256(rows_x * gu->rows * 4));
+    float* rs2 = (float*)((uint8_t*)xp2 + align256(fhip::gemm_f16x2_xp_bytes(down, rows_x)));
+    const bool clr1 = fhip::gemm_f16x2_adds_into_y(gu, rows_x), clr2 = fhip::gemm_f16x2_adds_into_y(down, rows_x);
+    if ((rc = fhip::launch_xsplit_f16(gu, d_x, rows_x, false, xp1, rs1, s, clr1 ? g : nullptr, clr1 ? rows_x * gu->rows : 0))) return rc;
+    if ((rc = fhip::launch_gemm_f16x2(gu, xp1, rs1, rows_x, g, s, clr1))) return rc;
+    // SwiGLU of [gate | up] is computed while the rows are split for the down projection
+    if ((rc = fhip::launch_xsplit_f16(down, g, rows_x, true, xp2, rs2, s, clr2 ? d_y : nullptr, clr2 ? rows_x * down->rows : 0))) return rc;
+    return fhip::launch_gemm_f16x2(down, xp2, rs2, rows_x, d_y, s, clr2);
+}
+
 int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, size_t rows, size_t cols, float* h_y) {
     int rc = need_init();
     if (rc) return rc;

@@ -1,0 +1,568 @@
+// Small-batch (2..32 activation rows) quantized matmul on the f16 matrix cores with f32-grade results, gfx950:
+//     Y[t, n] = sum_k X[t, k] * dequant(W[n, k]),   X f32 [T, K], W raw GGUF blocks [N, K], Y f32 [T, N]
+//
+// Stands for Tensor::matmul_q with a few activation rows (crates/ferric-tensor/src/dtype.rs:935-944; kernels
+// :2995-3051 Q4_K, :3423-3469 Q6_K), which the reference runs as one thread per output walking the weight row: the
+// weights are re-read per activation row there. Here one pass over the weights serves every row.
+//
+// How the matrix cores give f32-grade results from 16-bit operands:
+//   * Weights. A K-quant weight is (super-block scale d) x (small integer): d * (sc * q) - dmin * (m) for Q4_K with
+//     sc, m < 64 and q < 16, d * (sc * (q - 32)) for Q6_K. The integer factor sc*q <= 945 is exact in f16, so the B
+//     operand holds sc*q as f16 and the f32 factor d is applied to the f32 accumulator once per super-block. The Q4_K
+//     minima are one more MFMA per super-block: sum_sb m[n, sb] * (sum of the activations of sub-block sb). (Q6_K:
+//     |sc*(q-32)| can reach 4096; products above 2048 are rounded to even, a relative 2^-12 on those weights.)
+//   * Activations. A row is scaled by a power of two so that its largest magnitude lies in [2^14, 2^15), then split
+//     into hi = f16(x) and lo = f16(x - hi): two operand rows per activation row, 22 significant bits. The 16 rows of
+//     a v_mfma_f32_16x16x32_f16 hold hi and lo of 8 activation rows; the two partial results are added in f32 at the
+//     end and the scale is taken out again.
+//   * Unpack cost. A lane turns a dword of 8 nibbles into 8 f16 with 1 shift, 4 and-or (the nibble lands in the
+//     mantissa of the f16 constant 1024 or, for the high nibble, 16 positions up) and 4 packed f16 fma that remove the
+//     constant and apply the sub-block scale: 9 VALU for 8 weights, against ~30 for the bf16 path's f32 arithmetic.
+//     The k order inside an MFMA is free as long as both operands agree, so the activations are laid out in the
+//     order the nibbles come out (xsplit_f16_kernel does that once per call).
+//
+// Lane (g4 = lane / 16, c = lane % 16) of a wave works on weight row c of a 16-row set and on k-group g4 of each
+// 32-wide MFMA slice; a wave carries two row sets (32 weight rows), a workgroup four waves (128 rows). The
+// (128-row group, 256-column chunk) units are dealt to the workgroups in equal contiguous runs; a run that covers its
+// group's whole K stores, any other adds atomically into a Y cleared beforehand.
+#include "common.hpp"
+#include "loads.hpp"
+
+#include <hip/hip_fp16.h>
+
+#include <cmath>
+#include <type_traits>
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float f16_bits(uint32_t b) { return __half2float(__ushort_as_half((unsigned short)b)); }
+__device__ __forceinline__ uint32_t hfma2(uint32_t v, uint32_t s, uint32_t c) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(f16x2, v), __builtin_bit_cast(f16x2, s),
+                                                                  __builtin_bit_cast(f16x2, c)));
+}
+__device__ __forceinline__ uint32_t hmul2(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, a) * __builtin_bit_cast(f16x2, b));
+}
+__device__ __forceinline__ uint32_t hadd2(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, a) + __builtin_bit_cast(f16x2, b));
+}
+__device__ __forceinline__ uint32_t splat_h(_Float16 h) { return __builtin_bit_cast(uint32_t, (f16x2){h, h}); }
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t m, uint32_t o) { return (a & m) | o; }
+
+constexpr uint32_t H1024 = 0x64006400u;      // f16 pair (1024, 1024): mantissa step 1
+constexpr uint32_t H64 = 0x54005400u;        // f16 pair (64, 64): mantissa step 1/16
+constexpr uint32_t HNEG1024 = 0xE400E400u;   // (-1024, -1024)
+constexpr uint32_t HNEG64 = 0xD400D400u;     // (-64, -64)
+constexpr uint32_t HNEG96 = 0xD600D600u;     // (-96, -96)
+constexpr uint32_t H16TH = 0x2C002C00u;      // (1/16, 1/16)
+
+constexpr int CHUNK = 256;   // columns per chunk: one K-quant super-block
+// f16 per staged operand row of a chunk: 256 activations, 8 sub-block sums, 8 zeros, 8 of padding (row stride 35 x 16
+// bytes: the 16 rows a 16-byte read instruction touches fall into different bank groups)
+constexpr int XR = 280;
+
+__host__ __device__ constexpr int p4(int j) { return ((j & 1) << 1) | (j >> 1); }   // 0, 2, 1, 3: byte pairs (b0,b2), (b1,b3)
+
+template <int I, int N, class Fn>
+__device__ __forceinline__ void static_for(Fn&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-format weight streams. `Raw` is the register image of the bytes of one chunk of one weight row that lane
+// k-group g4 unpacks; pre<I>() derives the scales slice I is the first to need; frag<I>() is the B operand of slice I (8 per chunk): the
+// 8 weights this lane contributes, as integers times their sub-block scale; src_k(pos) is the column (inside the chunk)
+// whose activation belongs at operand position pos = (I * 4 + g4) * 8 + j.
+// ------------------------------------------------------------------------------------------------
+
+struct Q4K {
+    static constexpr int BLOCK = 144;
+    static constexpr bool HAS_MIN = true;
+    static __host__ __device__ constexpr int occupancy(int nt) { return nt == 1 ? 4 : (nt == 2 ? 3 : 2); }   // workgroups per CU the registers allow
+    // lane g4 owns bytes qs[32 g4, +32): the low nibbles are sub-block 2 g4, the high nibbles 2 g4 + 1
+    // (crates/ferric-gguf/src/lib.rs:805-823); slice I is dword I of those, j < 4 its low, j >= 4 its high nibbles.
+    static __host__ __device__ constexpr int src_k(int pos) {
+        const int j = pos & 7, g4 = (pos >> 3) & 3, i = pos >> 5;
+        return 64 * g4 + 32 * (j >> 2) + 4 * i + p4(j & 3);
+    }
+    static __host__ __device__ constexpr int pos_of(int k) {   // inverse of src_k
+        return (((k >> 2) & 7) * 4 + (k >> 6)) * 8 + 4 * ((k >> 5) & 1) + p4(k & 3);
+    }
+    struct Raw { u32x4 hd, q0, q1; };
+    struct Head { u32x4 hd; };
+    struct Ctx { uint32_t s0, c0, s1, c1; float d, dm; };
+    static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int g4) {
+        const uint8_t* blk = row + (size_t)c * BLOCK;
+        r.hd = *(const u32x4*)blk;
+        r.q0 = *(const u32x4*)(blk + 16 + 32 * g4);
+        r.q1 = *(const u32x4*)(blk + 32 + 32 * g4);
+    }
+    static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) { h.hd = *(const u32x4*)(row + (size_t)c * BLOCK); }
+    static __device__ __forceinline__ void take(Raw& r, const Head& h) { r.hd = h.hd; }
+    // after slice I the registers it was the last to read are reloaded with the same bytes of chunk nc
+    template <int I>
+    static __device__ __forceinline__ void refill(Raw& r, const uint8_t* row, int nc, int g4) {
+        const uint8_t* blk = row + (size_t)nc * BLOCK;
+        if (I == 3) r.q0 = *(const u32x4*)(blk + 16 + 32 * g4);
+        if (I == 7) r.q1 = *(const u32x4*)(blk + 32 + 32 * g4);
+    }
+    // get_sc_min (crates/ferric-gguf/src/lib.rs:795-804) as bytes: scales 0..3 / 4..7 and minima 0..3 / 4..7
+    static __device__ __forceinline__ uint32_t sc_bytes(const u32x4& hd, bool upper) {
+        return upper ? ((hd[3] & 0x0F0F0F0Fu) | ((hd[1] >> 2) & 0x30303030u)) : (hd[1] & 0x3F3F3F3Fu);
+    }
+    static __device__ __forceinline__ uint32_t min_bytes(const u32x4& hd, bool upper) {
+        return upper ? (((hd[3] >> 4) & 0x0F0F0F0Fu) | ((hd[2] >> 2) & 0x30303030u)) : (hd[2] & 0x3F3F3F3Fu);
+    }
+    template <int I>
+    static __device__ __forceinline__ void pre(const Raw& r, int g4, Ctx& x) {
+        if (I != 0) return;
+        const uint32_t scw = sc_bytes(r.hd, g4 >= 2) >> (16 * (g4 & 1));
+        const uint32_t s0 = splat_h((_Float16)(unsigned short)(scw & 0xFFu)), s1 = splat_h((_Float16)(unsigned short)((scw >> 8) & 0xFFu));
+        // low nibble: (1024 + q) * sc - 1024 sc; high nibble in place: (1024 + 16 q) * (sc / 16) - 64 sc. All exact in f16.
+        x.s0 = s0; x.c0 = hmul2(s0, HNEG1024);
+        x.s1 = hmul2(s1, H16TH); x.c1 = hmul2(s1, HNEG64);
+        x.d = f16_bits(r.hd[0] & 0xFFFFu);
+        x.dm = -64.0f * f16_bits(r.hd[0] >> 16);   // the sub-block sums are staged divided by 64
+    }
+    template <int I>
+    static __device__ __forceinline__ f16x8 frag(const Raw& r, const Ctx& x) {
+        const uint32_t w = I < 4 ? r.q0[I & 3] : r.q1[I & 3], w8 = w >> 8;
+        u32x4 o;
+        o[0] = hfma2(and_or(w, 0x000F000Fu, H1024), x.s0, x.c0);
+        o[1] = hfma2(and_or(w8, 0x000F000Fu, H1024), x.s0, x.c0);
+        o[2] = hfma2(and_or(w, 0x00F000F0u, H1024), x.s1, x.c1);
+        o[3] = hfma2(and_or(w8, 0x00F000F0u, H1024), x.s1, x.c1);
+        return __builtin_bit_cast(f16x8, o);
+    }
+    // B operand of the minima MFMA: m[0..7] of this row as f16 in k-group 0, zeros in the others
+    static __device__ __forceinline__ f16x8 mins(const Raw& r, int g4) {
+        const uint32_t lo = min_bytes(r.hd, false), hi = min_bytes(r.hd, true);
+        u32x4 o;
+        o[0] = hadd2(__builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u), HNEG1024);
+        o[1] = hadd2(__builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u), HNEG1024);
+        o[2] = hadd2(__builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u), HNEG1024);
+        o[3] = hadd2(__builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u), HNEG1024);
+        if (g4 != 0) o = (u32x4){0u, 0u, 0u, 0u};
+        return __builtin_bit_cast(f16x8, o);
+    }
+};
+
+struct Q6K {
+    static constexpr int BLOCK = 210;
+    static constexpr bool HAS_MIN = false;
+    static __host__ __device__ constexpr int occupancy(int nt) { return nt == 1 ? 3 : (nt == 2 ? 2 : 1); }
+    // lane g4 = (hf, lh) owns l in [16 lh, 16 lh + 16) of half hf (crates/ferric-gguf/src/lib.rs:833-851): slice I = (par, dd) is
+    // dword dd of ql[64 hf + 32 par + 16 lh ..] and of qh[32 hf + 16 lh ..]; j < 4 are the low nibbles (quarter par of the
+    // half, high bits in field par of the qh byte), j >= 4 the high nibbles (quarter par + 2, field par + 2). All of a
+    // lane's l share l / 16 = lh, so it needs four scales a chunk: sc[8 hf + 2 qt + lh].
+    static __host__ __device__ constexpr int src_k(int pos) {
+        const int j = pos & 7, g4 = (pos >> 3) & 3, i = pos >> 5;
+        const int hf = g4 >> 1, lh = g4 & 1, par = i >> 2, dd = i & 3;
+        return 128 * hf + 32 * (par + 2 * (j >> 2)) + 16 * lh + 4 * dd + p4(j & 3);
+    }
+    static __host__ __device__ constexpr int pos_of(int k) {   // inverse of src_k
+        const int hf = k >> 7, qt = (k >> 5) & 3, lh = (k >> 4) & 1, dd = (k >> 2) & 3;
+        return ((4 * (qt & 1) + dd) * 4 + 2 * hf + lh) * 8 + 4 * (qt >> 1) + p4(k & 3);
+    }
+    struct Raw { u32x4 ql[2], qh, sc; uint32_t d; };
+    struct Head { u32x4 sc; uint32_t d; };
+    struct Ctx { uint32_t s[4]; float d, dm; };
+    static __device__ __forceinline__ u32x4 ld16(const uint8_t* p) { return fhip::load16_a2(p); }   // blocks of 210 bytes
+    static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) {
+        const uint8_t* blk = row + (size_t)c * BLOCK;
+        h.sc = ld16(blk + 192);
+        h.d = *(const uint16_t*)(blk + 208);
+    }
+    static __device__ __forceinline__ void take(Raw& r, const Head& h) { r.sc = h.sc; r.d = h.d; }
+    static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int g4) {
+        const uint8_t* blk = row + (size_t)c * BLOCK;
+        const int hf = g4 >> 1, lh = g4 & 1;
+        r.ql[0] = ld16(blk + 64 * hf + 16 * lh);
+        r.ql[1] = ld16(blk + 64 * hf + 32 + 16 * lh);
+        r.qh = ld16(blk + 128 + 32 * hf + 16 * lh);
+        r.sc = ld16(blk + 192);
+        r.d = *(const uint16_t*)(blk + 208);
+    }
+    // after slice I the registers it was the last to read are reloaded with the same bytes of chunk nc
+    template <int I>
+    static __device__ __forceinline__ void refill(Raw& r, const uint8_t* row, int nc, int g4) {
+        const uint8_t* blk = row + (size_t)nc * BLOCK;
+        const int hf = g4 >> 1, lh = g4 & 1;
+        if (I == 3) r.ql[0] = ld16(blk + 64 * hf + 16 * lh);
+        if (I == 7) {
+            r.ql[1] = ld16(blk + 64 * hf + 32 + 16 * lh);
+            r.qh = ld16(blk + 128 + 32 * hf + 16 * lh);
+        }
+    }
+    template <int I>
+    static __device__ __forceinline__ void pre(const Raw& r, int g4, Ctx& x) {
+        if (I != 0) return;
+        const int hf = g4 >> 1, lh = g4 & 1;
+        const uint32_t w0 = (hf ? r.sc[2] : r.sc[0]) >> (8 * lh), w1 = (hf ? r.sc[3] : r.sc[1]) >> (8 * lh);
+#pragma unroll
+        for (int qt = 0; qt < 4; qt++) {
+            const uint32_t w = qt < 2 ? w0 : w1;
+            const int v = (int)(int8_t)((w >> (16 * (qt & 1))) & 0xFFu);
+            const uint32_t sp = splat_h((_Float16)(short)v);
+            x.s[qt] = sp;
+        }
+        x.d = f16_bits(r.d);
+        x.dm = 0.f;
+    }
+    template <int I>
+    static __device__ __forceinline__ f16x8 frag(const Raw& r, const Ctx& x) {
+        constexpr int par = I >> 2, dd = I & 3, flo = par, fhi = par + 2;
+        const uint32_t ql = r.ql[par][dd], qh = r.qh[dd];
+        constexpr uint32_t NM = 0x00F000F0u, HM = 0x03000300u;
+        // a 6-bit q lands in mantissa bits 4..9 of the f16 constant 64 (step 1/16): the value is 64 + q
+        const uint32_t p0 = and_or(qh << (8 - 2 * flo), HM, and_or(ql << 4, NM, H64));
+        const uint32_t p1 = and_or(qh >> (2 * flo), HM, and_or(ql >> 4, NM, H64));
+        const uint32_t p2 = and_or(qh << (8 - 2 * fhi), HM, and_or(ql, NM, H64));
+        const uint32_t p3 = and_or(qh >> (2 * fhi), HM, and_or(ql >> 8, NM, H64));
+        u32x4 o;
+        const uint32_t clo = hmul2(x.s[flo], HNEG96), chi = hmul2(x.s[fhi], HNEG96);   // (64 + q) * sc - 96 sc = (q - 32) * sc
+        o[0] = hfma2(p0, x.s[flo], clo);
+        o[1] = hfma2(p1, x.s[flo], clo);
+        o[2] = hfma2(p2, x.s[fhi], chi);
+        o[3] = hfma2(p3, x.s[fhi], chi);
+        return __builtin_bit_cast(f16x8, o);
+    }
+    static __device__ __forceinline__ f16x8 mins(const Raw&, int) { return (f16x8){0, 0, 0, 0, 0, 0, 0, 0}; }
+};
+
+// ------------------------------------------------------------------------------------------------
+// Activation preparation, two short kernels. Output per chunk: 16 NT operand rows of XR f16 (rows 16 q + i, i < 8: hi of
+// activation row 8 q + i; rows 16 q + 8 + i: its lo), columns in operand order (F::pos_of), followed by the 8 sub-block
+// sums / 64 (formats with minima) and zeros. rs[t] is the factor that takes the row's power-of-two scale out again.
+// SWIGLU: the row is silu(gate) * up of a [T, 2d] = [gate | up] matrix (crates/ferric-tensor/src/lib.rs:2603-2618).
+// ------------------------------------------------------------------------------------------------
+constexpr int MAXW = 64;   // partial maxima per row: one per 1024 columns, rows of up to 65 536 columns
+
+template <bool SWIGLU>
+__device__ __forceinline__ float act(const float* __restrict__ x, int K, int k) {
+    if (SWIGLU) {
+        const float g = x[k], u = x[(size_t)K + k];
+        return (g / (1.0f + expf(-g))) * u;
+    }
+    return x[k];
+}
+
+// mx[t * MAXW + b] = largest magnitude among columns [1024 b, 1024 b + 1024) of activation row t
+template <bool SWIGLU>
+__global__ void __launch_bounds__(256) rowmax_kernel(const float* __restrict__ X, int K, float* __restrict__ mx) {
+    __shared__ float red[4];
+    const int tid = threadIdx.x, t = blockIdx.y;
+    const float* x = X + (size_t)t * (SWIGLU ? 2 * (size_t)K : (size_t)K);
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int k = blockIdx.x * 1024 + 256 * j + tid;
+        if (k < K) m = fmaxf(m, fabsf(act<SWIGLU>(x, K, k)));
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if ((tid & 63) == 0) red[tid >> 6] = m;
+    __syncthreads();
+    if (tid == 0) mx[t * MAXW + blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+// one workgroup per (chunk, operand row group of 8): thread k of it converts column k of the chunk
+template <class F, bool SWIGLU>
+__global__ void __launch_bounds__(256) xsplit_f16_kernel(const float* __restrict__ X, int T, int K, int NT, const float* __restrict__ mx,
+                                                       int nmx, uint16_t* __restrict__ Xp, float* __restrict__ rs,
+                                                       float* __restrict__ zero, size_t zero_n) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const size_t nwg = (size_t)gridDim.x * gridDim.y;
+    for (size_t k = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + tid; k < zero_n; k += nwg * 256) zero[k] = 0.f;
+    const int ck = blockIdx.x, t = blockIdx.y;
+    const bool live = t < T;
+    float m = (live && lane < nmx) ? mx[t * MAXW + lane] : 0.f;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    float sc = 1.0f, inv = 1.0f;
+    if (m > 0.f && m < INFINITY) {
+        int ex;
+        (void)frexpf(m, &ex);            // m < 2^ex
+        ex = ex < -100 ? -100 : ex;
+        sc = ldexpf(1.0f, 15 - ex);      // scaled maximum in [2^14, 2^15)
+        inv = ldexpf(1.0f, ex - 15);
+    }
+    if (tid == 0 && ck == 0 && live) rs[t] = inv;
+    auto put = [&](int col, float v) {
+        const _Float16 h = (_Float16)v;
+        const _Float16 l = (_Float16)(v - (float)h);
+        const size_t at = ((size_t)(ck * NT + (t >> 3)) * 16 + (t & 7)) * XR + col;
+        Xp[at] = __builtin_bit_cast(uint16_t, h);
+        Xp[at + 8 * XR] = __builtin_bit_cast(uint16_t, l);
+    };
+    const int k = ck * CHUNK + tid;
+    const float* x = X + (size_t)(live ? t : 0) * (SWIGLU ? 2 * (size_t)K : (size_t)K);
+    const float v = (live && k < K) ? act<SWIGLU>(x, K, k) * sc : 0.f;
+    put(F::pos_of(tid), v);
+    // columns 256..263: sub-block sums / 64 (|sum| <= 32 * 2^15, so the quotient stays below 2^14); 264..279: zeros
+    float s = F::HAS_MIN ? v : 0.f;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    if ((tid & 31) == 0) put(CHUNK + (tid >> 5), s * 0.015625f);
+    if (tid < 16) put(CHUNK + 8 + tid, 0.f);
+}
+
+struct F16Params {
+    const uint8_t* W;
+    const uint16_t* Xp;   // prepared activations: [nchunks][16 NT][XR] f16
+    const float* rs;      // [T] row scales to take out
+    float* Y;             // [T, N]
+    int T, N, nchunks;
+    size_t row_bytes;
+    long long units;      // 128-row groups * nchunks, chunk fastest
+    int per;              // units per workgroup
+};
+
+template <class F, int NT>
+__global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16Params p) {
+    constexpr int ROWS = 16 * NT, PIECES = ROWS * XR / 8, NP = (PIECES + 255) / 256;
+    __shared__ __attribute__((aligned(16))) uint16_t Xs[2][ROWS * XR];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g4 = lane >> 4, c = lane & 15;
+    const int nchunks = p.nchunks;
+    long long u = (long long)blockIdx.x * p.per;
+    const long long u_end = u + p.per < p.units ? u + p.per : p.units;
+
+    u32x4 stage[NP];
+    auto load_x = [&](int ck) {
+        const u32x4* src = (const u32x4*)(p.Xp + (size_t)ck * ROWS * XR);
+#pragma unroll
+        for (int q = 0; q < NP; q++)
+            if (tid + 256 * q < PIECES) stage[q] = src[tid + 256 * q];
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < NP; q++)
+            if (tid + 256 * q < PIECES) ((u32x4*)Xs[buf])[tid + 256 * q] = stage[q];
+    };
+    const int a_rd = c * XR + 8 * g4;                     // + 16 q XR + 32 I
+    const int m_rd = c * XR + CHUNK + (g4 ? 8 : 0);       // sub-block sums for k-group 0, zeros for the others
+
+    for (int seg = 0; u < u_end; seg++) {
+        const int grp = (int)(u / nchunks);
+        const int c_begin = (int)(u - (long long)grp * nchunks);
+        const int c_end = (long long)(nchunks - c_begin) < u_end - u ? nchunks : c_begin + (int)(u_end - u);
+        u += c_end - c_begin;
+        const bool whole = c_begin == 0 && c_end == nchunks;
+        int n[2];
+        const uint8_t* wrow[2];
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            n[s] = grp * 128 + wave * 32 + 16 * s + c;
+            wrow[s] = p.W + (size_t)(n[s] < p.N ? n[s] : p.N - 1) * p.row_bytes;
+        }
+        f32x4 total[2][NT];
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int q = 0; q < NT; q++) total[s][q] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        // the scales of this lane's activation rows, asked for now and used after the chunk loop
+        float rsv[NT][4];
+#pragma unroll
+        for (int q = 0; q < NT; q++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int t = 8 * q + 4 * (g4 & 1) + r;
+                rsv[q][r] = p.rs[t < p.T ? t : 0];
+            }
+
+        // Weight bytes: the quant registers of a chunk are reloaded with the next chunk's bytes as soon as their last slice
+        // has read them (half a chunk to a chunk ahead of their use); the few header bytes go through `hd` a chunk ahead.
+        typename F::Raw raw[2];
+        typename F::Head hd[2];
+#pragma unroll
+        for (int s = 0; s < 2; s++) F::prime(raw[s], wrow[s], c_begin, g4);
+        load_x(c_begin);
+        if (seg > 0) __syncthreads();   // the previous segment's last reads of buffer 0 are done
+        store_x(0);
+        __syncthreads();
+
+        for (int ck = c_begin; ck < c_end; ck++) {
+            const int buf = (ck - c_begin) & 1;
+            const int cn = ck + 1 < c_end ? ck + 1 : ck;
+#pragma unroll
+            for (int s = 0; s < 2; s++) F::head(hd[s], wrow[s], cn);
+            load_x(cn);
+            typename F::Ctx x[2];
+            f32x4 acc[2][NT];
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int q = 0; q < NT; q++) acc[s][q] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            static_for<0, 8>([&](auto Ic) {
+                constexpr int I = decltype(Ic)::value;
+                f16x8 a[NT];
+#pragma unroll
+                for (int q = 0; q < NT; q++) a[q] = *(const f16x8*)(&Xs[buf][a_rd + 16 * q * XR + 32 * I]);
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    F::template pre<I>(raw[s], g4, x[s]);
+                    const f16x8 b = F::template frag<I>(raw[s], x[s]);
+#pragma unroll
+                    for (int q = 0; q < NT; q++) acc[s][q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[q], b, acc[s][q], 0, 0, 0);
+                    F::template refill<I>(raw[s], wrow[s], cn, g4);
+                }
+            });
+            if constexpr (F::HAS_MIN) {
+                f16x8 am[NT];
+#pragma unroll
+                for (int q = 0; q < NT; q++) am[q] = *(const f16x8*)(&Xs[buf][m_rd + 16 * q * XR]);
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    const f16x8 bm = F::mins(raw[s], g4);
+#pragma unroll
+                    for (int q = 0; q < NT; q++) {
+                        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                        const f32x4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(am[q], bm, z, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x[s].dm, accm[r], total[s][q][r]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int q = 0; q < NT; q++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x[s].d, acc[s][q][r], total[s][q][r]);
+            store_x(buf ^ 1);
+            __syncthreads();
+#pragma unroll
+            for (int s = 0; s < 2; s++) F::take(raw[s], hd[s]);
+        }
+
+        // D layout of the 16x16 MFMA: register r of lane (g4, c) is operand row 4 g4 + r, column c. Operand rows 0..7
+        // are the hi parts of activation rows 8 q + [0, 8), rows 8..15 their lo parts: lanes g4 and g4 ^ 2 hold the
+        // two parts of the same output.
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int q = 0; q < NT; q++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int t = 8 * q + 4 * (g4 & 1) + r;
+                    float v = total[s][q][r];
+                    v += __shfl_xor(v, 32);
+                    if (g4 < 2 && t < p.T && n[s] < p.N) {
+                        v *= rsv[q][r];
+                        float* y = p.Y + (size_t)t * p.N + n[s];
+                        if (whole) *y = v;
+                        else unsafeAtomicAdd(y, v);
+                    }
+                }
+    }
+}
+
+__global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = 0.f;
+}
+
+struct Plan {
+    int nt, nchunks, per;
+    long long units;
+    unsigned grid;
+    bool split;
+};
+
+Plan make_plan(const fhip_weight* w, size_t t) {
+    Plan q;
+    q.nt = t <= 8 ? 1 : (t <= 16 ? 2 : 4);
+    q.nchunks = (int)(w->cols / CHUNK);
+    const long long groups = ((long long)w->rows + 127) / 128;
+    q.units = groups * q.nchunks;
+    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    const long long wgs = cus * (w->type == FHIP_Q6_K ? Q6K::occupancy(q.nt) : Q4K::occupancy(q.nt));
+    long long per = (q.units + wgs - 1) / wgs;
+    if (per * 4 >= (long long)q.nchunks * 3 && per < q.nchunks) per = q.nchunks;   // nearly whole groups: make them whole
+    if (per < 1) per = 1;
+    q.per = (int)per;
+    q.grid = (unsigned)((q.units + per - 1) / per);
+    q.split = per % q.nchunks != 0;
+    return q;
+}
+
+template <class F>
+int launch_xsplit_fmt(const float* d_x, size_t t, size_t k, bool swiglu, const Plan& q, uint16_t* d_xp, float* d_rs, float* d_mx,
+                      hipStream_t s, float* zero, size_t zero_n) {
+    const int nmx = (int)((k + 1023) / 1024);
+    const dim3 gm((unsigned)nmx, (unsigned)t), grid((unsigned)q.nchunks, (unsigned)(8 * q.nt)), wg(256);
+    if (swiglu) {
+        hipLaunchKernelGGL((rowmax_kernel<true>), gm, wg, 0, s, d_x, (int)k, d_mx);
+        hipLaunchKernelGGL((xsplit_f16_kernel<F, true>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_mx, nmx, d_xp, d_rs, zero, zero_n);
+    } else {
+        hipLaunchKernelGGL((rowmax_kernel<false>), gm, wg, 0, s, d_x, (int)k, d_mx);
+        hipLaunchKernelGGL((xsplit_f16_kernel<F, false>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_mx, nmx, d_xp, d_rs, zero, zero_n);
+    }
+    return fhip::check_hip(hipGetLastError(), "xsplit_f16 launch");
+}
+
+template <class F>
+int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+    const Plan q = make_plan(w, t);
+    F16Params p;
+    p.W = w->d_raw; p.Xp = d_xp; p.rs = d_rs; p.Y = d_y;
+    p.T = (int)t; p.N = (int)w->rows; p.nchunks = q.nchunks; p.row_bytes = w->row_bytes;
+    p.units = q.units; p.per = q.per;
+    if (q.split && !y_cleared) {
+        const size_t n = t * w->rows;
+        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
+    }
+    if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 1>), dim3(q.grid), dim3(256), 0, s, p);
+    else if (q.nt == 2) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 4>), dim3(q.grid), dim3(256), 0, s, p);
+    return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
+}
+
+}  // namespace
+
+namespace fhip {
+
+bool gemm_f16x2_supports(const fhip_weight* w, size_t t) {
+    return w && (w->type == FHIP_Q4_K || w->type == FHIP_Q6_K) && t >= 1 && t <= 32 && w->cols % CHUNK == 0 && w->cols > 0 &&
+           w->cols <= (size_t)MAXW * 1024;
+}
+
+size_t gemm_f16x2_aux_bytes() { return 256 + 32 * MAXW * sizeof(float); }   // row scales, then the partial row maxima
+
+size_t gemm_f16x2_xp_bytes(const fhip_weight* w, size_t t) {
+    const Plan q = make_plan(w, t);
+    return (size_t)q.nchunks * 16 * q.nt * XR * sizeof(uint16_t);
+}
+
+bool gemm_f16x2_adds_into_y(const fhip_weight* w, size_t t) { return make_plan(w, t).split; }
+
+int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, float* d_aux, hipStream_t s,
+                      float* zero, size_t zero_n) {
+    const Plan q = make_plan(w, t);
+    float* d_mx = d_aux + 64;
+    switch (w->type) {
+        case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
+        case FHIP_Q6_K: return launch_xsplit_fmt<Q6K>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
+        default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
+    }
+}
+
+int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+    switch (w->type) {
+        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, d_rs, t, d_y, s, y_cleared);
+        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, d_rs, t, d_y, s, y_cleared);
+        default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
+    }
+}
+
+}  // namespace fhip

@@ -349,6 +349,35 @@ class Tensor:
         assert w.ggml_type == 8
         return self.matmul_q_coop(w, stream)
 
+    def matmul_q_f16x2(self, w, stream=None):
+        """x [rows <= 32, in] @ W^T in one pass over the weights, f32-grade results -- dtype.rs:935-944 for small batches."""
+        assert self.dtype == np.float32, "matmul_q_f16x2 expects f32 activations"
+        rows, inn = self._rows_inner()
+        assert inn == w.cols(), "inner dim mismatch"
+        lib = _lib.load()
+        ws = DeviceBuffer(max(256, lib.fhip_matmul_q_f16x2_ws_bytes(w.handle, rows)))
+        out = Tensor.empty((rows, w.rows()))
+        _lib.check(lib.fhip_matmul_q_f16x2(w.handle, self.buf.ptr, rows, out.buf.ptr, ws.ptr, _stream_handle(stream)))
+        if stream is not None:
+            stream.synchronize()      # ws is freed on return
+        else:
+            _lib.check(lib.fhip_stream_sync(None))
+        return out
+
+    def ffn_f16x2(self, gate_up, down, stream=None):
+        """down(swiglu(gate_up(x))) for a batch of rows <= 32 in one pass over each weight -- qwen3.rs:944-964."""
+        rows, inn = self._rows_inner()
+        assert inn == gate_up.cols(), "inner dim mismatch"
+        lib = _lib.load()
+        ws = DeviceBuffer(max(256, lib.fhip_ffn_f16x2_ws_bytes(gate_up.handle, down.handle, rows)))
+        out = Tensor.empty((rows, down.rows()))
+        _lib.check(lib.fhip_ffn_f16x2(gate_up.handle, down.handle, self.buf.ptr, rows, out.buf.ptr, ws.ptr, _stream_handle(stream)))
+        if stream is not None:
+            stream.synchronize()      # ws is freed on return
+        else:
+            _lib.check(lib.fhip_stream_sync(None))
+        return out
+
     def ffn_coop(self, gate_up, down, stream=None):
         """down(swiglu(gate_up(x))) on the matrix cores, for a batch of rows -- qwen3.rs:944-964 over dtype.rs:1818."""
         rows, inn = self._rows_inner()
