@@ -292,7 +292,7 @@ __global__ void __launch_bounds__(256) xsplit_f16_kernel(const float* __restrict
     if (m > 0.f && m < INFINITY) {
         int ex;
         (void)frexpf(m, &ex);            // m < 2^ex
-        ex = ex < -100 ? -100 : ex;
+        ex = ex < -111 ? -111 : ex;      // the scale stays a finite f32; rows below 2^-111 keep fewer bits
         sc = ldexpf(1.0f, 15 - ex);      // scaled maximum in [2^14, 2^15)
         inv = ldexpf(1.0f, ex - 15);
     }

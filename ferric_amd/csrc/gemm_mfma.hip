@@ -24,6 +24,7 @@
 // Dequantized values are exactly the f32 the CPU dequantizer produces, rounded to bf16 (RNE) by
 // v_cvt_pk_bf16_f32.
 #include "common.hpp"
+#include "loads.hpp"
 
 #include <hip/hip_fp16.h>
 
@@ -37,7 +38,6 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };
 
 __device__ __forceinline__ float f16_bits(uint32_t b) { return __half2float(__ushort_as_half((unsigned short)b)); }
 __device__ __forceinline__ float ub(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
@@ -136,7 +136,7 @@ struct Q6K {
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 ql[2][2], qh[2], sc, scn; uint32_t d, dn; };
     struct Ctx { float d; };
-    static __device__ __forceinline__ u32x4 ld16(const uint8_t* p) { return ((const U4A2*)p)->v; }
+    static __device__ __forceinline__ u32x4 ld16(const uint8_t* p) { return fhip::load16_a2(p); }   // 210-byte blocks: see loads.hpp
     static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int h, int) {
         const uint8_t* blk = row + (size_t)c * BLOCK;
 #pragma unroll
@@ -213,7 +213,7 @@ struct Q80 {
             for (int u = 0; u < 2; u++) {
                 const uint8_t* p = blk(row, c, 2 * g + u, nblk);
                 r.d[g][u] = *(const uint16_t*)p;
-                r.q[g][u] = ((const U4A2*)(p + 2 + 16 * h))->v;
+                r.q[g][u] = fhip::load16_a2(p + 2 + 16 * h);
             }
     }
     template <int G>
@@ -233,7 +233,7 @@ struct Q80 {
         for (int u = 0; u < 2; u++) {
             const uint8_t* p = blk(row, nc, 2 * G + u, nblk);
             r.d[G][u] = *(const uint16_t*)p;
-            r.q[G][u] = ((const U4A2*)(p + 2 + 16 * h))->v;
+            r.q[G][u] = fhip::load16_a2(p + 2 + 16 * h);
         }
     }
 };

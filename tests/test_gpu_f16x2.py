@@ -1,0 +1,156 @@
+"""Small-batch matmul on the f16 matrix cores (fhip_matmul_q_f16x2 / fhip_ffn_f16x2) vs the CPU oracle, through the C ABI.
+
+The path claims f32-grade results: weights enter the matrix cores as exact integers, activations as a scaled hi/lo pair
+of f16 (22 significant bits). Bars, against the oracle's dequantized weights in f64:
+  * |y - y64| <= 2.5e-7 * ||w_row|| * ||x_t||  (measured <= 6e-8; the exact-f32 mat-vec path measures <= 5e-8 on the same
+    inputs), 4000x inside the north-star bound 1e-3 * ||w_row|| * ||x_t||;
+  * max|d| / max|ref| < 1e-5, the bar the f32 mat-vec tests use;
+  * Q6_K only, blocks whose |scale * (q - 32)| exceeds 2048: such a product is rounded to an even integer on its way
+    into f16, a relative 2^-12 on that weight, so the bar there is 2.5e-4 * ||w_row|| * ||x_t|| (still 4x inside the
+    north-star bound) -- the test builds such blocks on purpose and also checks that ordinary ones stay at 2.5e-7.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+TIGHT = 2.5e-7
+
+
+def run_case(F, O, ty, t, n, k, seed, x=None, w=None, tol=TIGHT):
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(ty, n, k, seed) if w is None else w
+    x = np.random.default_rng(seed + 1).standard_normal((t, k)).astype(np.float32) if x is None else x
+    qm = F.QMatrix.from_bytes(w, ty, n, k)
+    y = F.Tensor.from_vec(x, x.shape).matmul_q_f16x2(qm).to_vec().reshape(t, n)
+    y64, wn = O.matmul_f64(x, w, ty, n, k)
+    err = np.abs(y - y64)
+    bound = tol * wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None]
+    assert (err <= bound + 1e-300).all(), (ty, t, n, k, float(np.max(err / (bound + 1e-300))))
+    assert err.max() / max(1e-30, np.abs(y64).max()) < 1e-5 * max(1.0, tol / TIGHT)
+    return y, y64
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+def test_small_and_ragged_shapes(F, O, ty):
+    # every activation-row count class (1..8 -> one group of operand rows, 9..16 -> two, 17..32 -> four), weight rows that
+    # do not fill a 16-row set, a 128-row group or a workgroup's share, one chunk and many
+    shapes = [(1, 32, 256), (2, 100, 512), (3, 128, 256), (5, 300, 1024), (8, 256, 2048), (9, 130, 768), (16, 257, 1024),
+              (17, 64, 512), (31, 15, 256), (32, 200, 1536), (4, 1, 256), (7, 1000, 5120)]
+    for i, (t, n, k) in enumerate(shapes):
+        run_case(F, O, ty, t, n, k, 100 + i)
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+def test_rows_of_very_different_magnitude(F, O, ty):
+    # each row is scaled by its own power of two: tiny, huge, zero and outlier rows side by side keep the per-row bound
+    t, n, k = 8, 96, 1024
+    x = np.random.default_rng(7).standard_normal((t, k)).astype(np.float32)
+    x[0] *= np.float32(1e-30)
+    x[1] *= np.float32(1e30)
+    x[2] = 0.0
+    x[3, 17] = np.float32(3e6)            # one outlier sets the scale; the rest of the row is 2^-21 of it
+    x[4] *= np.float32(65504.0 * 4)       # beyond the f16 range before scaling
+    x[5] *= np.float32(2.0 ** -118)       # near the bottom of the f32 normal range: the scale is capped at 2^126
+    y, y64 = run_case(F, O, ty, t, n, k, 8, x=x)
+    assert not y[2].any()
+
+
+def test_nonfinite_values_stay_in_their_row(F, O):
+    t, n, k = 6, 64, 512
+    x = np.random.default_rng(9).standard_normal((t, k)).astype(np.float32)
+    x[1, 5] = np.inf
+    x[4, 300] = np.nan
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(Q4_K, n, k, 10)
+    qm = F.QMatrix.from_bytes(w, Q4_K, n, k)
+    y = F.Tensor.from_vec(x, x.shape).matmul_q_f16x2(qm).to_vec().reshape(t, n)
+    assert not np.isfinite(y[1]).any() and np.isnan(y[4]).all()      # as a dot product with inf / nan in it comes out
+    good = [0, 2, 3, 5]
+    y64, wn = O.matmul_f64(x[good], w, Q4_K, n, k)
+    bound = TIGHT * wn[None, :] * np.linalg.norm(x[good].astype(np.float64), axis=1)[:, None]
+    assert (np.abs(y[good] - y64) <= bound).all()
+
+
+def test_q6_k_products_beyond_the_exact_f16_range(F, O):
+    # scales of +-127 / -128 with quants at the ends of their range: |sc * (q - 32)| up to 4096
+    from ferric_amd.synth import synth_weights
+    n, k, t = 64, 1024, 8
+    w = synth_weights(Q6_K, n, k, 11).reshape(n, k // 256, 210).copy()
+    rng = np.random.default_rng(12)
+    w[:, :, 192:208] = rng.choice(np.array([127, 125, -127, -128], np.int8).view(np.uint8), size=(n, k // 256, 16))
+    w[:, :, 0:128] = rng.choice(np.array([0x00, 0xFF, 0x0F, 0xF0, 0x1E], np.uint8), size=(n, k // 256, 128))
+    w[:, :, 128:192] = rng.choice(np.array([0x00, 0xFF, 0xCC, 0x33], np.uint8), size=(n, k // 256, 64))
+    y, y64 = run_case(F, O, Q6_K, t, n, k, 13, w=w.reshape(-1), tol=2.5e-4)
+    # the same blocks with small scales are exact again
+    w[:, :, 192:208] = rng.choice(np.array([31, -32, 17, -5], np.int8).view(np.uint8), size=(n, k // 256, 16))
+    run_case(F, O, Q6_K, t, n, k, 13, w=w.reshape(-1))
+
+
+@pytest.mark.parametrize("ty,n,k", [(Q4_K, 512, 2048), (Q6_K, 384, 1024)])
+def test_agrees_with_the_f32_matvec_path_and_rows_are_independent(F, O, ty, n, k):
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(ty, n, k, 20)
+    qm = F.QMatrix.from_bytes(w, ty, n, k)
+    x = np.random.default_rng(21).standard_normal((12, k)).astype(np.float32)
+    y = F.Tensor.from_vec(x, x.shape).matmul_q_f16x2(qm).to_vec().reshape(12, n)
+    f32 = F.Tensor.from_vec(x, x.shape).matmul_q(qm).to_vec().reshape(12, n)
+    assert np.abs(y - f32).max() <= 2e-6 * np.abs(f32).max()
+    # a row computed in a batch of 12 (two operand-row groups) and alone (one group): same value up to the order of the
+    # f32 additions of K slices
+    one = F.Tensor.from_vec(x[9:10], (1, k)).matmul_q_f16x2(qm).to_vec()
+    assert np.abs(one - y[9]).max() <= 2e-6 * np.abs(y[9]).max()
+
+
+@pytest.mark.parametrize("batch", [4, 8])
+def test_config3_ffn_block(F, O, batch):
+    # gate|up 2 x (5120 -> 17408) Q4_K stacked gate-first, down 17408 -> 5120 Q6_K, SwiGLU between, one call
+    from ferric_amd.synth import synth_weights
+    n_embd, n_ff = 5120, 17408
+    gu = synth_weights(Q4_K, 2 * n_ff, n_embd, 3)
+    dn = synth_weights(Q6_K, n_embd, n_ff, 4)
+    x = np.random.default_rng(5).standard_normal((batch, n_embd)).astype(np.float32)
+    wgu = F.QMatrix.from_bytes(gu, Q4_K, 2 * n_ff, n_embd)
+    wdn = F.QMatrix.from_bytes(dn, Q6_K, n_embd, n_ff)
+    xt = F.Tensor.from_vec(x, x.shape)
+    y = xt.ffn_f16x2(wgu, wdn).to_vec().reshape(batch, n_embd)
+    g64, _ = O.matmul_f64(x, gu, Q4_K, 2 * n_ff, n_embd)
+    g, u = g64[:, :n_ff], g64[:, n_ff:]
+    h64 = g / (1.0 + np.exp(-g)) * u
+    # the down projection of the f64 SwiGLU (matmul_f64 takes f32 activations: its rounding of h is 6e-8 relative)
+    y64, wn = O.matmul_f64(h64.astype(np.float32), dn, Q6_K, n_embd, n_ff)
+    err = np.abs(y - y64)
+    assert (err <= 1e-6 * wn[None, :] * np.linalg.norm(h64, axis=1)[:, None]).all()
+    assert err.max() / np.abs(y64).max() < 1e-5
+    # and the exact-f32 block gives the same answer to f32 rounding
+    y32 = xt.ffn(wgu, wdn).to_vec().reshape(batch, n_embd)
+    assert np.abs(y - y32).max() / np.abs(y32).max() < 2e-6
+
+
+def test_argument_checks(F):
+    from ferric_amd import _lib
+    import ctypes as C
+    lib = _lib.load()
+    from ferric_amd.synth import synth_weights
+    q4 = F.QMatrix.from_bytes(synth_weights(Q4_K, 32, 256, 1), Q4_K, 32, 256)
+    q8 = F.QMatrix.from_bytes(synth_weights(Q8_0, 32, 256, 1), Q8_0, 32, 256)
+    assert lib.fhip_matmul_q_f16x2_ws_bytes(q4.handle, 8) > 0
+    assert lib.fhip_matmul_q_f16x2_ws_bytes(q4.handle, 33) == 0 and lib.fhip_matmul_q_f16x2_ws_bytes(q8.handle, 8) == 0
+    with pytest.raises(AssertionError, match="at most 32 activation rows"):
+        F.Tensor.from_vec(np.zeros((33, 256), np.float32), (33, 256)).matmul_q_f16x2(q4)
+    with pytest.raises(ValueError, match="Q4_K and Q6_K only"):
+        F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256)).matmul_q_f16x2(q8)
+    with pytest.raises(AssertionError, match="inner dim mismatch"):
+        F.Tensor.from_vec(np.zeros((2, 512), np.float32), (2, 512)).matmul_q_f16x2(q4)
+    x = F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256))
+    y = F.Tensor.empty((2, 32))
+    ws = F.DeviceBuffer(lib.fhip_matmul_q_f16x2_ws_bytes(q4.handle, 2) + 256)
+    with pytest.raises(_lib.FerricHipError, match="256-byte aligned"):
+        _lib.check(lib.fhip_matmul_q_f16x2(q4.handle, x.buf.ptr, 2, y.buf.ptr, C.c_void_p(ws.ptr.value + 16), None))
+    with pytest.raises(_lib.FerricHipError, match="NULL pointer"):
+        _lib.check(lib.fhip_matmul_q_f16x2(q4.handle, x.buf.ptr, 2, y.buf.ptr, None, None))
+    # no rows: nothing to do, nothing touched
+    assert F.Tensor.from_vec(np.zeros(0, np.float32), (0, 256)).matmul_q_f16x2(q4).to_vec().size == 0
+    dn = F.QMatrix.from_bytes(synth_weights(Q6_K, 32, 256, 2), Q6_K, 32, 256)
+    with pytest.raises(AssertionError, match="down in dim must equal n_ff"):
+        F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256)).ffn_f16x2(q4, dn)
