@@ -143,6 +143,16 @@ def bench_ffn(F, lib, check, stream, timer, batches, reps=20):
         g.launch()
         ms = timer.time_ms(g.launch) / reps
         res[str(b)]["matrix_core_path"] = {"ms": ms, "weight_GBps": wbytes / (ms * 1e-3) / 1e9, "tokens_per_s": b / (ms * 1e-3)}
+        # and through the f16 matrix cores with exact integer weights and hi/lo split activations: one pass over
+        # the weights, f32-grade results
+        wsh = F.DeviceBuffer(max(256, lib.fhip_ffn_f16x2_ws_bytes(gu.handle, dn.handle, b)))
+        g = F.Graph.begin(stream)
+        for _ in range(reps):
+            check(lib.fhip_ffn_f16x2(gu.handle, dn.handle, x.buf.ptr, b, y.buf.ptr, wsh.ptr, stream.handle))
+        g.end()
+        g.launch()
+        ms = timer.time_ms(g.launch) / reps
+        res[str(b)]["f16x2_path"] = {"ms": ms, "weight_GBps": wbytes / (ms * 1e-3) / 1e9, "tokens_per_s": b / (ms * 1e-3)}
     return res, wbytes
 
 
@@ -369,6 +379,30 @@ def probe_prefill(F, lib, check):
             check(lib.fhip_stream_sync(None))
 
 
+def probe_f16x2(F, lib, check):
+    """Work for a profiler run of the small-batch f16 matrix-core path at 8 activation rows: fhip_matmul_q_f16x2 on the
+    gate|up (34816 x 5120 Q4_K) and down (5120 x 17408 Q6_K) weights, then the whole block through fhip_ffn_f16x2, 5
+    launches each, eagerly on the null stream."""
+    from ferric_amd.synth import synth_weights
+    n_embd, n_ff, t = 5120, 17408, 8
+    gu = F.QMatrix.from_bytes(synth_weights(Q4_K, 2 * n_ff, n_embd, 3), Q4_K, 2 * n_ff, n_embd)
+    dn = F.QMatrix.from_bytes(synth_weights(Q6_K, n_embd, n_ff, 4), Q6_K, n_embd, n_ff)
+    rng = np.random.default_rng(5)
+    x = F.Tensor.from_vec(rng.standard_normal((t, n_embd)).astype(np.float32), (t, n_embd))
+    h = F.Tensor.from_vec(rng.standard_normal((t, n_ff)).astype(np.float32), (t, n_ff))
+    for w, xin in ((gu, x), (dn, h)):
+        y = F.Tensor.empty((t, w.rows()))
+        ws = F.DeviceBuffer(lib.fhip_matmul_q_f16x2_ws_bytes(w.handle, t))
+        for _ in range(5):
+            check(lib.fhip_matmul_q_f16x2(w.handle, xin.buf.ptr, t, y.buf.ptr, ws.ptr, None))
+        check(lib.fhip_stream_sync(None))
+    y = F.Tensor.empty((t, n_embd))
+    ws = F.DeviceBuffer(lib.fhip_ffn_f16x2_ws_bytes(gu.handle, dn.handle, t))
+    for _ in range(5):
+        check(lib.fhip_ffn_f16x2(gu.handle, dn.handle, x.buf.ptr, t, y.buf.ptr, ws.ptr, None))
+    check(lib.fhip_stream_sync(None))
+
+
 def probe_decode(F, lib, check):
     """Work for a hardware-counter run on the decode attention kernel: a copy of known size (calibrates FETCH_SIZE /
     WRITE_SIZE), then 8 launches of fhip_decode_attention on 8 different caches of 4096 rows (40 query / 8 KV heads x 128:
@@ -446,6 +480,9 @@ def main():
     ap.add_argument("--probe-prefill", action="store_true",
                     help="profiler probe for the matrix-core GEMM: Q4_K 5120x5120 and 34816x5120 at T = 2048, 128 and 8, "
                          "5 launches each; prints nothing else")
+    ap.add_argument("--probe-f16x2", action="store_true",
+                    help="profiler probe for the small-batch f16 matrix-core path: gate|up, down and the whole FFN block at 8 "
+                         "rows, 5 launches each; prints nothing else")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU sharding is a design note, not code")
@@ -460,6 +497,9 @@ def main():
     rows = cols = 5120
     if args.probe:
         probe(F, lib, check)
+        return
+    if args.probe_f16x2:
+        probe_f16x2(F, lib, check)
         return
     if args.probe_prefill:
         probe_prefill(F, lib, check)
