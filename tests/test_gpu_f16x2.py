@@ -127,6 +127,34 @@ def test_config3_ffn_block(F, O, batch):
     assert np.abs(y - y32).max() / np.abs(y32).max() < 2e-6
 
 
+def test_replays_in_a_graph(F, O):
+    # the six launches of the block captured once and replayed with new inputs in the same buffers: every replay must
+    # match an eager call on the same input (up to the order of the K-split additions)
+    import ctypes as C
+    from ferric_amd import _lib
+    from ferric_amd.synth import synth_weights
+    lib = _lib.load()
+    n_embd, n_ff, t = 512, 1280, 5
+    gu = F.QMatrix.from_bytes(synth_weights(Q4_K, 2 * n_ff, n_embd, 30), Q4_K, 2 * n_ff, n_embd)
+    dn = F.QMatrix.from_bytes(synth_weights(Q6_K, n_embd, n_ff, 31), Q6_K, n_embd, n_ff)
+    st = F.Stream()
+    x = F.Tensor.from_vec(np.zeros((t, n_embd), np.float32), (t, n_embd))
+    y = F.Tensor.empty((t, n_embd))
+    ws = F.DeviceBuffer(lib.fhip_ffn_f16x2_ws_bytes(gu.handle, dn.handle, t))
+    g = F.Graph.begin(st)
+    _lib.check(lib.fhip_ffn_f16x2(gu.handle, dn.handle, x.buf.ptr, t, y.buf.ptr, ws.ptr, st.handle))
+    g.end()
+    rng = np.random.default_rng(32)
+    for rep in range(4):
+        xin = (rng.standard_normal((t, n_embd)) * (10.0 ** rep)).astype(np.float32)
+        _lib.check(lib.fhip_memcpy_h2d(x.buf.ptr, xin.ctypes.data_as(C.c_void_p), xin.nbytes, st.handle))
+        g.launch()
+        st.synchronize()
+        got = y.to_vec().reshape(t, n_embd)
+        want = F.Tensor.from_vec(xin, xin.shape).ffn_f16x2(gu, dn).to_vec().reshape(t, n_embd)
+        assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max(), rep
+
+
 def test_argument_checks(F):
     from ferric_amd import _lib
     import ctypes as C
