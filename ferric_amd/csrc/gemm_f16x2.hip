@@ -1,4 +1,4 @@
-// Small-batch (2..32 activation rows) quantized matmul on the f16 matrix cores with f32-grade results, gfx950:
+// Small-batch (1..32 activation rows) quantized matmul on the f16 matrix cores with f32-grade results, gfx950:
 //     Y[t, n] = sum_k X[t, k] * dequant(W[n, k]),   X f32 [T, K], W raw GGUF blocks [N, K], Y f32 [T, N]
 //
 // Stands for Tensor::matmul_q with a few activation rows (crates/ferric-tensor/src/dtype.rs:935-944; kernels
@@ -31,6 +31,7 @@
 #include <hip/hip_fp16.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -107,6 +108,14 @@ struct Q4K {
         r.q1 = *(const u32x4*)(blk + 32 + 32 * g4);
     }
     static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) { h.hd = *(const u32x4*)(row + (size_t)c * BLOCK); }
+    // row-streaming kernel: a block is PARTS 16-byte pieces in global memory and a row of LROW bytes in the wave's LDS image
+    static constexpr int PARTS = 9, LROW = 144, TAIL = 0, ROWS_OCCUPANCY = 3;   // 120 VGPRs, 36 KB of LDS (four per CU ran slower: 36.7 vs 34.0 us)
+    static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return *(const u32x4*)p; }
+    static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) {
+        r.hd = *(const u32x4*)row;
+        r.q0 = *(const u32x4*)(row + 16 + 32 * g4);
+        r.q1 = *(const u32x4*)(row + 32 + 32 * g4);
+    }
     static __device__ __forceinline__ void take(Raw& r, const Head& h) { r.hd = h.hd; }
     // after slice I the registers it was the last to read are reloaded with the same bytes of chunk nc
     template <int I>
@@ -183,6 +192,20 @@ struct Q6K {
         h.d = *(const uint16_t*)(blk + 208);
     }
     static __device__ __forceinline__ void take(Raw& r, const Head& h) { r.sc = h.sc; r.d = h.d; }
+    // row-streaming kernel: 13 16-byte pieces + the 2-byte d; LDS rows of 240 bytes (a multiple of 16 whose dword count,
+    // 60, puts the 16 rows of a read instruction into different banks). Contiguous lanes read contiguous bytes here, which
+    // the 2-byte alignment of the blocks does not slow down.
+    static constexpr int PARTS = 13, LROW = 240, TAIL = 208, ROWS_OCCUPANCY = 3;   // 134 VGPRs, 49 KB of LDS
+    struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };
+    static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return ((const U4A2*)p)->v; }
+    static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) {
+        const int hf = g4 >> 1, lh = g4 & 1;
+        r.ql[0] = *(const u32x4*)(row + 64 * hf + 16 * lh);
+        r.ql[1] = *(const u32x4*)(row + 64 * hf + 32 + 16 * lh);
+        r.qh = *(const u32x4*)(row + 128 + 32 * hf + 16 * lh);
+        r.sc = *(const u32x4*)(row + 192);
+        r.d = *(const uint16_t*)(row + 208);
+    }
     static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int g4) {
         const uint8_t* blk = row + (size_t)c * BLOCK;
         const int hf = g4 >> 1, lh = g4 & 1;
@@ -324,7 +347,6 @@ struct F16Params {
     int T, N, nchunks;
     size_t row_bytes;
     long long units;      // 128-row groups * nchunks, chunk fastest
-    int per;              // units per workgroup
 };
 
 template <class F, int NT>
@@ -334,8 +356,9 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g4 = lane >> 4, c = lane & 15;
     const int nchunks = p.nchunks;
-    long long u = (long long)blockIdx.x * p.per;
-    const long long u_end = u + p.per < p.units ? u + p.per : p.units;
+    // the units are dealt evenly: workgroup b takes [b U / G, (b + 1) U / G), so every CU carries the same number of them
+    long long u = (long long)blockIdx.x * p.units / gridDim.x;
+    const long long u_end = (long long)(blockIdx.x + 1) * p.units / gridDim.x;
 
     u32x4 stage[NP];
     auto load_x = [&](int ck) {
@@ -467,13 +490,159 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Up to 8 activation rows, the same arithmetic with the weight bytes streamed the way the mat-vec kernel streams them: a
+// wave fetches the chunk blocks of its 32 rows with contiguous lanes on contiguous bytes (9 lanes per 144-byte Q4_K block,
+// 13 + a 2-byte tail per 210-byte Q6_K block), parks them in its own LDS image and reads them back one row per lane. Every
+// byte is requested once, in whole cache lines, and the registers that wait for memory (the next chunk in flight) are not
+// the registers in use, so loads are outstanding through all of a chunk's arithmetic. Cold weights (each launch on bytes
+// no cache holds): gate|up 39 -> see DESIGN; the one-row-per-lane loads of the kernel above ask for every line two or
+// three times, 16 bytes at a time.
+// ------------------------------------------------------------------------------------------------
+template <class F>
+__global__ void __launch_bounds__(256, F::ROWS_OCCUPANCY) gemm_q_f16x2_rows_kernel(F16Params p) {
+    constexpr int PIECES = 16 * XR / 8, NP = (PIECES + 255) / 256;
+    constexpr int WP = 32 * F::PARTS, NW = (WP + 63) / 64;
+    __shared__ __attribute__((aligned(16))) uint16_t Xs[2][16 * XR];
+    __shared__ __attribute__((aligned(16))) uint8_t Wl[4][32 * F::LROW];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g4 = lane >> 4, c = lane & 15;
+    const int nchunks = p.nchunks;
+    // the units are dealt evenly: workgroup b takes [b U / G, (b + 1) U / G), so every CU carries the same number of them
+    long long u = (long long)blockIdx.x * p.units / gridDim.x;
+    const long long u_end = (long long)(blockIdx.x + 1) * p.units / gridDim.x;
+
+    u32x4 stage[NP];
+    auto load_x = [&](int ck) {
+        const u32x4* src = (const u32x4*)(p.Xp + (size_t)ck * 16 * XR);
+#pragma unroll
+        for (int q = 0; q < NP; q++)
+            if (tid + 256 * q < PIECES) stage[q] = src[tid + 256 * q];
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < NP; q++)
+            if (tid + 256 * q < PIECES) ((u32x4*)Xs[buf])[tid + 256 * q] = stage[q];
+    };
+    const int a_rd = c * XR + 8 * g4;
+    const int m_rd = c * XR + CHUNK + (g4 ? 8 : 0);
+
+    // piece i * 64 + lane of the wave's chunk image is 16-byte part (piece % PARTS) of row (piece / PARTS)
+    uint8_t* const wl = Wl[wave];
+    u32x4 G[NW];
+    uint32_t gt = 0;
+    // requests the bytes of unit `v` = (128-row group, chunk); rows past the end of the weight repeat its last row
+    auto load_w = [&](long long v) {
+        const int grp = (int)(v / nchunks), ck = (int)(v - (long long)grp * nchunks);
+        const int row0 = grp * 128 + wave * 32 < p.N ? grp * 128 + wave * 32 : p.N - 1;
+        const int rmax = p.N - 1 - row0;
+        const uint8_t* b = p.W + (size_t)row0 * p.row_bytes + (size_t)ck * F::BLOCK;
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            const int pc = i * 64 + lane, row = pc / F::PARTS;
+            const uint32_t off = (uint32_t)(row < rmax ? row : rmax) * (uint32_t)p.row_bytes + 16u * (uint32_t)(pc - row * F::PARTS);
+            if (pc < WP) G[i] = F::ldg(b + off);
+        }
+        if (F::TAIL && lane < 32) gt = *(const uint16_t*)(b + (uint32_t)(lane < rmax ? lane : rmax) * (uint32_t)p.row_bytes + F::TAIL);
+    };
+    auto park_w = [&]() {
+#pragma unroll
+        for (int i = 0; i < NW; i++) {
+            const int pc = i * 64 + lane, row = pc / F::PARTS;
+            if (pc < WP) *(u32x4*)(wl + row * F::LROW + 16 * (pc - row * F::PARTS)) = G[i];
+        }
+        if (F::TAIL && lane < 32) *(uint16_t*)(wl + lane * F::LROW + F::TAIL) = (uint16_t)gt;
+    };
+    float rsv[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int t = 4 * (g4 & 1) + r;
+        rsv[r] = p.rs[t < p.T ? t : 0];
+    }
+    if (u >= u_end) return;
+
+    // The workgroup's run of units is one stream: the chunk after a group's last is the next group's first, fetched and
+    // parked like any other, so a run that crosses a group boundary pays no second start-up.
+    const long long u_begin = u;
+    load_w(u);
+    load_x((int)(u % nchunks));
+    store_x(0);
+    park_w();
+    if (u + 1 < u_end) load_w(u + 1);
+    __syncthreads();
+
+    f32x4 total[2];
+    for (int it = 0; u < u_end; u++, it++) {
+        const int buf = it & 1;
+        const int grp = (int)(u / nchunks), ck = (int)(u - (long long)grp * nchunks);
+        const bool more = u + 1 < u_end;
+        if (more) load_x(ck + 1 < nchunks ? ck + 1 : 0);
+        if (u == u_begin || ck == 0) {
+#pragma unroll
+            for (int s = 0; s < 2; s++) total[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            typename F::Raw raw;
+            F::from_lds(raw, wl + (16 * s + c) * F::LROW, g4);
+            typename F::Ctx x;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            static_for<0, 8>([&](auto Ic) {
+                constexpr int I = decltype(Ic)::value;
+                const f16x8 a = *(const f16x8*)(&Xs[buf][a_rd + 32 * I]);
+                F::template pre<I>(raw, g4, x);
+                const f16x8 b = F::template frag<I>(raw, x);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
+                // keeps the MFMA here: left alone, the optimiser sinks the whole chain below the last fragment and holds all eight
+                // fragments and operand rows in registers meanwhile
+                asm volatile("" : "+v"(acc));
+            });
+            if constexpr (F::HAS_MIN) {
+                const f16x8 am = *(const f16x8*)(&Xs[buf][m_rd]);
+                const f16x8 bm = F::mins(raw, g4);
+                const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                const f32x4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm, z, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; r++) total[s][r] = fmaf(x.dm, accm[r], total[s][r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) total[s][r] = fmaf(x.d, acc[r], total[s][r]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (more) {
+            park_w();                             // unit u + 1 over unit u, which this wave has finished reading
+            if (u + 2 < u_end) load_w(u + 2);     // in flight through all of the next unit's arithmetic
+            store_x(buf ^ 1);
+        }
+        if (!more || ck == nchunks - 1) {
+            // this group's share is complete: whole iff the run held all of its chunks
+            const bool whole = (long long)grp * nchunks >= u_begin && (long long)(grp + 1) * nchunks <= u_end;
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int t = 4 * (g4 & 1) + r, n = grp * 128 + wave * 32 + 16 * s + c;
+                    float v = total[s][r];
+                    v += __shfl_xor(v, 32);
+                    if (g4 < 2 && t < p.T && n < p.N) {
+                        v *= rsv[r];
+                        float* y = p.Y + (size_t)t * p.N + n;
+                        if (whole) *y = v;
+                        else unsafeAtomicAdd(y, v);
+                    }
+                }
+        }
+        __syncthreads();
+    }
+}
+
 __global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) out[i] = 0.f;
 }
 
 struct Plan {
-    int nt, nchunks, per;
+    int nt, nchunks;
     long long units;
     unsigned grid;
     bool split;
@@ -486,13 +655,14 @@ Plan make_plan(const fhip_weight* w, size_t t) {
     const long long groups = ((long long)w->rows + 127) / 128;
     q.units = groups * q.nchunks;
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    const long long wgs = cus * (w->type == FHIP_Q6_K ? Q6K::occupancy(q.nt) : Q4K::occupancy(q.nt));
-    long long per = (q.units + wgs - 1) / wgs;
-    if (per * 4 >= (long long)q.nchunks * 3 && per < q.nchunks) per = q.nchunks;   // nearly whole groups: make them whole
-    if (per < 1) per = 1;
-    q.per = (int)per;
-    q.grid = (unsigned)((q.units + per - 1) / per);
-    q.split = per % q.nchunks != 0;
+    const long long wgs = cus * (w->type == FHIP_Q6_K ? (q.nt == 1 ? Q6K::ROWS_OCCUPANCY : Q6K::occupancy(q.nt)) : (q.nt == 1 ? Q4K::ROWS_OCCUPANCY : Q4K::occupancy(q.nt)));
+    // one workgroup per resident slot, each with the same share of the units (a grid of 2.66 workgroups per CU leaves
+    // two thirds of the CUs with half as much again to do as the rest); shares of three quarters of a group's chunks or
+    // more are rounded to whole groups, which store instead of adding
+    const long long per = (q.units + wgs - 1) / wgs;
+    if (per >= q.nchunks || per * 4 >= (long long)q.nchunks * 3) q.grid = (unsigned)groups;
+    else q.grid = (unsigned)(q.units < wgs ? q.units : wgs);
+    q.split = q.grid != (unsigned)groups;
     return q;
 }
 
@@ -517,12 +687,14 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, si
     F16Params p;
     p.W = w->d_raw; p.Xp = d_xp; p.rs = d_rs; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.nchunks = q.nchunks; p.row_bytes = w->row_bytes;
-    p.units = q.units; p.per = q.per;
+    p.units = q.units;
     if (q.split && !y_cleared) {
         const size_t n = t * w->rows;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
     }
-    if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 1>), dim3(q.grid), dim3(256), 0, s, p);
+    static const bool lanes_per_row = getenv("FHIP_F16X2_ROW_PER_LANE") != nullptr;   // the other kernel, for comparison
+    if (q.nt == 1 && !lanes_per_row) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F>), dim3(q.grid), dim3(256), 0, s, p);
+    else if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 1>), dim3(q.grid), dim3(256), 0, s, p);
     else if (q.nt == 2) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
     else hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 4>), dim3(q.grid), dim3(256), 0, s, p);
     return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
