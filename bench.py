@@ -383,27 +383,31 @@ def probe_prefill(F, lib, check):
             check(lib.fhip_stream_sync(None))
 
 
-def probe_f16x2(F, lib, check):
+def probe_f16x2(F, lib, check, ncopy=4):
     """Work for a profiler run of the small-batch f16 matrix-core path at 8 activation rows: fhip_matmul_q_f16x2 on the
-    gate|up (34816 x 5120 Q4_K) and down (5120 x 17408 Q6_K) weights, then the whole block through fhip_ffn_f16x2, 5
-    launches each, eagerly on the null stream."""
+    gate|up (34816 x 5120 Q4_K) and down (5120 x 17408 Q6_K) weights, then the whole block through fhip_ffn_f16x2, 12
+    launches each, eagerly on the null stream, rotating over 4 copies of each weight (694 MB in all, more than the
+    Infinity Cache holds) so that every launch reads HBM."""
     from ferric_amd.synth import synth_weights
     n_embd, n_ff, t = 5120, 17408, 8
-    gu = F.QMatrix.from_bytes(synth_weights(Q4_K, 2 * n_ff, n_embd, 3), Q4_K, 2 * n_ff, n_embd)
-    dn = F.QMatrix.from_bytes(synth_weights(Q6_K, n_embd, n_ff, 4), Q6_K, n_embd, n_ff)
+    gbuf = replicate(F, lib, check, synth_weights(Q4_K, 2 * n_ff, n_embd, 3), ncopy)
+    dbuf = replicate(F, lib, check, synth_weights(Q6_K, n_embd, n_ff, 4), ncopy)
+    gb, db = weight_bytes(Q4_K, 2 * n_ff, n_embd), weight_bytes(Q6_K, n_embd, n_ff)
+    gus = [F.QMatrix.wrap_device(gbuf, gb, Q4_K, 2 * n_ff, n_embd, offset=i * gb) for i in range(ncopy)]
+    dns = [F.QMatrix.wrap_device(dbuf, db, Q6_K, n_embd, n_ff, offset=i * db) for i in range(ncopy)]
     rng = np.random.default_rng(5)
     x = F.Tensor.from_vec(rng.standard_normal((t, n_embd)).astype(np.float32), (t, n_embd))
     h = F.Tensor.from_vec(rng.standard_normal((t, n_ff)).astype(np.float32), (t, n_ff))
-    for w, xin in ((gu, x), (dn, h)):
-        y = F.Tensor.empty((t, w.rows()))
-        ws = F.DeviceBuffer(lib.fhip_matmul_q_f16x2_ws_bytes(w.handle, t))
-        for _ in range(5):
-            check(lib.fhip_matmul_q_f16x2(w.handle, xin.buf.ptr, t, y.buf.ptr, ws.ptr, None))
+    for ws_, xin in ((gus, x), (dns, h)):
+        y = F.Tensor.empty((t, ws_[0].rows()))
+        ws = F.DeviceBuffer(lib.fhip_matmul_q_f16x2_ws_bytes(ws_[0].handle, t))
+        for i in range(12):
+            check(lib.fhip_matmul_q_f16x2(ws_[i % ncopy].handle, xin.buf.ptr, t, y.buf.ptr, ws.ptr, None))
         check(lib.fhip_stream_sync(None))
     y = F.Tensor.empty((t, n_embd))
-    ws = F.DeviceBuffer(lib.fhip_ffn_f16x2_ws_bytes(gu.handle, dn.handle, t))
-    for _ in range(5):
-        check(lib.fhip_ffn_f16x2(gu.handle, dn.handle, x.buf.ptr, t, y.buf.ptr, ws.ptr, None))
+    ws = F.DeviceBuffer(lib.fhip_ffn_f16x2_ws_bytes(gus[0].handle, dns[0].handle, t))
+    for i in range(12):
+        check(lib.fhip_ffn_f16x2(gus[i % ncopy].handle, dns[i % ncopy].handle, x.buf.ptr, t, y.buf.ptr, ws.ptr, None))
     check(lib.fhip_stream_sync(None))
 
 
