@@ -31,7 +31,6 @@
 #include <hip/hip_fp16.h>
 
 #include <cmath>
-#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -493,8 +492,8 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
 // ------------------------------------------------------------------------------------------------
 // Up to 8 activation rows, the same arithmetic with the weight bytes streamed the way the mat-vec kernel streams them: a
 // wave fetches the chunk blocks of its 32 rows with contiguous lanes on contiguous bytes (9 lanes per 144-byte Q4_K block,
-// 13 + a 2-byte tail per 210-byte Q6_K block), parks them in its own LDS image and reads them back one row per lane. Every
-// byte is requested once, in whole cache lines, and the registers that wait for memory (the next chunk in flight) are not
+// 13 + a 2-byte tail per 210-byte Q6_K block), parks them in its own LDS image and reads them back one row per lane. A
+// block is requested once, as one run of bytes, and the registers that wait for memory (the next chunk in flight) are not
 // the registers in use, so loads are outstanding through all of a chunk's arithmetic. On weights no cache holds (each launch
 // on bytes it has not seen) this takes 34 us for a 34816 x 5120 Q4_K weight and 27 us for 5120 x 17408 Q6_K, the kernel
 // above 39 and 35.5 us: its one-row-per-lane loads ask for every cache line two or three times, 16 bytes at a time.
@@ -692,9 +691,7 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, si
         const size_t n = t * w->rows;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
     }
-    static const bool lanes_per_row = getenv("FHIP_F16X2_ROW_PER_LANE") != nullptr;   // the other kernel, for comparison
-    if (q.nt == 1 && !lanes_per_row) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F>), dim3(q.grid), dim3(256), 0, s, p);
-    else if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 1>), dim3(q.grid), dim3(256), 0, s, p);
+    if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F>), dim3(q.grid), dim3(256), 0, s, p);
     else if (q.nt == 2) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
     else hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 4>), dim3(q.grid), dim3(256), 0, s, p);
     return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
