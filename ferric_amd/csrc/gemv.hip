@@ -551,6 +551,10 @@ struct GemvParams {
     int RF;              // replicas of the full-wave set, each taking every RF-th row (balances them against the tail wave)
     int G;               // row groups per workgroup
     int rpg;             // output rows per row group
+    // ceil(2^32 / d) for the three divisors of the kernel's index arithmetic (waves per row group, full waves per row, RF), 0
+    // for d = 1: floor(n / d) = mulhi(n, magic) for n < 65 536, 2 <= d <= 1024; a hardware-less integer division costs ~35
+    // dependent instructions, and four of them stood in front of the first load
+    uint32_t m_wpr, m_ngf, m_rf;
     fhip::SelParams sel; // expert selection (selw == nullptr: none)
     // Fused input norm (norm_w != nullptr; M = 1, cols <= 8 * threads): the activation row is rmsnorm(x [+ resid]) * norm_w,
     // formed by every workgroup while it stages the row; workgroup 0 also stores x + resid to x_out (never x itself).
@@ -571,6 +575,8 @@ template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? F::U1 :
 // Activation rows one pass can hold in registers (48 plane dwords per row for the 64-weight units, 24 for Q8_0).
 template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
 
+__device__ __forceinline__ uint32_t div_magic(uint32_t n, uint32_t magic) { return magic ? __umulhi(n, magic) : n; }
+
 template <class F, int M, int U, bool SWIGLU, bool NORM>
 __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -578,13 +584,21 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     constexpr int VPR = SWIGLU ? 2 : 1;       // weight rows walked per output row
     constexpr int RUN = F::RUN, NRUN = F::NRUN, RD = RUN / 4;
     const int tid = threadIdx.x, lane = tid & 63;
+    // The activation loads go out before anything else: they need the thread index only, and the index arithmetic below
+    // (a few hundred scalar instructions, which the four waves of a SIMD get through one after the other, oldest first)
+    // then runs under their latency instead of in front of it.
+    const int e0 = tid * 8;
+    float4 xa0 = {0, 0, 0, 0}, xb0 = {0, 0, 0, 0};
+    if (e0 < M * p.cols) { xa0 = *(const float4*)(p.x + e0); xb0 = *(const float4*)(p.x + e0 + 4); }
+    asm volatile("" ::: "memory");   // keeps the loads here
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NGF = p.NG >> 2, NT = p.NG & 3, NFW = NGF * p.RF, WPR = NFW + (NT ? 1 : 0);
-    const int wr = wave % WPR, rg = wave / WPR;          // wave within row group, row group within workgroup
+    const int rg = (int)div_magic((uint32_t)wave, p.m_wpr), wr = wave - rg * WPR;   // row group within workgroup, wave within row group
+    const int wq = (int)div_magic((uint32_t)wr, p.m_ngf), wm = wr - wq * NGF;       // wr / NGF, wr % NGF (NGF = 0: never used)
     const bool tail = wr == NFW;                         // wave-uniform
     const int RT = tail ? (NT == 1 ? 4 : NT == 2 ? 2 : 1) : 1;   // rows this wave works on at once
     // iteration i of this wave works on virtual row v_start + i * v_step (+ row_off per lane in a tail wave)
-    const int v_start = tail ? 0 : wr / NGF, v_step = tail ? RT : p.RF;
+    const int v_start = tail ? 0 : wq, v_step = tail ? RT : p.RF;
 
     // LDS: activation planes [M][cols/RUN][3][RUN] bytes | scales [M][cols/RUN] | sums [M][cols/RUN] | partials
     const int nrun = p.cols / RUN;
@@ -597,7 +611,7 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     const int slot = lane >> 4, l16 = lane & 15;
     int group, row_off;
     bool lane_ok = true;
-    if (!tail) { group = 4 * (wr % NGF) + slot; row_off = 0; }
+    if (!tail) { group = 4 * wm + slot; row_off = 0; }
     else if (NT == 3) { lane_ok = slot < 3; group = 4 * NGF + (lane_ok ? slot : 0); row_off = 0; }
     else { group = 4 * NGF + (NT == 2 ? (slot & 1) : 0); row_off = NT == 2 ? (slot >> 1) : slot; }
     typename F::Lane L;
@@ -611,7 +625,9 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     nrows = nrows < 0 ? 0 : (nrows > p.rpg ? p.rpg : nrows);
     const int nv = nrows * VPR;                          // virtual rows: v -> weight row r0 + v/VPR (+ pair for odd v)
     const uint8_t* base = p.W + (size_t)(nrows > 0 ? r0 : 0) * p.row_bytes;   // a row group past the end points at row 0
-    const int n_it = nv > v_start ? (nv - v_start + v_step - 1) / v_step : 0;
+    // (nv - v_start + v_step - 1) / v_step with v_step = 4, 2, 1 (tail wave) or RF
+    const uint32_t n_num = (uint32_t)(nv - v_start + v_step - 1);
+    const int n_it = nv > v_start ? (int)(tail ? n_num >> (RT == 4 ? 2 : RT == 2 ? 1 : 0) : div_magic(n_num, p.m_rf)) : 0;
     // Address of iteration `it`: a wave-uniform row base (scalar registers) plus a 32-bit lane offset. A tail
     // wave's lanes sit row_off rows further (v_start + it*v_step is a multiple of RT there, so with fused
     // SwiGLU the gate/up split of row_off is fixed); lanes past the last row read the uniform row instead
@@ -628,9 +644,6 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     // (Loads return in issue order. Issuing exactly U row loads unconditionally would let the wait for the
     // activations be a counted one instead of a drain, but the dummy loads of waves with fewer than U rows
     // cost more than that saves: measured +40 % on the 4096x4096 Q8_0 GEMV.)
-    const int e0 = tid * 8;
-    float4 xa0 = {0, 0, 0, 0}, xb0 = {0, 0, 0, 0};
-    if (e0 < M * p.cols) { xa0 = *(const float4*)(p.x + e0); xb0 = *(const float4*)(p.x + e0 + 4); }
     constexpr bool fused_norm = NORM && M == 1;   // a separate instantiation: the plain kernel carries none of this
     float4 nwa = {1, 1, 1, 1}, nwb = {1, 1, 1, 1}, rsa = {0, 0, 0, 0}, rsb = {0, 0, 0, 0};
     if (fused_norm && e0 < p.cols) {
@@ -885,6 +898,8 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     if (tune_g > 0) G = tune_g;
     if (tune_rpg > 0) rpg = tune_rpg;
     p.G = G; p.rpg = rpg;
+    auto magic = [](int d) { return d > 1 ? (uint32_t)(((1ull << 32) + (unsigned)d - 1) / (unsigned)d) : 0u; };
+    p.m_wpr = magic(WPR); p.m_ngf = magic(p.NG >> 2); p.m_rf = magic(p.RF);
     const size_t per_wg = (size_t)G * rpg;
     const size_t grid = (out_rows + per_wg - 1) / per_wg;
     size_t lds = lds_bytes<F, M, SWIGLU>(w->cols, p.NG, G, rpg);
