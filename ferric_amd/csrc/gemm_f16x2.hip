@@ -109,6 +109,7 @@ struct Q4K {
     static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) { h.hd = *(const u32x4*)(row + (size_t)c * BLOCK); }
     // row-streaming kernel: a block is PARTS 16-byte pieces in global memory and a row of LROW bytes in the wave's LDS image
     static constexpr int PARTS = 9, LROW = 144, TAIL = 0, ROWS_OCCUPANCY = 3;   // 120 VGPRs, 36 KB of LDS (four per CU ran slower: 36.7 vs 34.0 us)
+    static constexpr bool ROWS_AT_16 = false;   // 9..16 rows, cold weights: 44.9 us against 42.0 us for the one-row-per-lane kernel
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return *(const u32x4*)p; }
     static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) {
         r.hd = *(const u32x4*)row;
@@ -195,6 +196,7 @@ struct Q6K {
     // 60, puts the 16 rows of a read instruction into different banks). Contiguous lanes read contiguous bytes here, which
     // the 2-byte alignment of the blocks does not slow down.
     static constexpr int PARTS = 13, LROW = 240, TAIL = 208, ROWS_OCCUPANCY = 3;   // 134 VGPRs, 49 KB of LDS
+    static constexpr bool ROWS_AT_16 = true;    // 9..16 rows, cold weights: 33.2 us against 41.2 us
     struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return ((const U4A2*)p)->v; }
     static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) {
@@ -498,11 +500,11 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
 // on bytes it has not seen) this takes 34 us for a 34816 x 5120 Q4_K weight and 27 us for 5120 x 17408 Q6_K, the kernel
 // above 39 and 35.5 us: its one-row-per-lane loads ask for every cache line two or three times, 16 bytes at a time.
 // ------------------------------------------------------------------------------------------------
-template <class F>
-__global__ void __launch_bounds__(256, F::ROWS_OCCUPANCY) gemm_q_f16x2_rows_kernel(F16Params p) {
-    constexpr int PIECES = 16 * XR / 8, NP = (PIECES + 255) / 256;
+template <class F, int NT>
+__global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f16x2_rows_kernel(F16Params p) {
+    constexpr int PIECES = 16 * NT * XR / 8, NP = (PIECES + 255) / 256;
     constexpr int WP = 32 * F::PARTS, NW = (WP + 63) / 64;
-    __shared__ __attribute__((aligned(16))) uint16_t Xs[2][16 * XR];
+    __shared__ __attribute__((aligned(16))) uint16_t Xs[2][16 * NT * XR];
     __shared__ __attribute__((aligned(16))) uint8_t Wl[4][32 * F::LROW];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g4 = lane >> 4, c = lane & 15;
@@ -513,7 +515,7 @@ __global__ void __launch_bounds__(256, F::ROWS_OCCUPANCY) gemm_q_f16x2_rows_kern
 
     u32x4 stage[NP];
     auto load_x = [&](int ck) {
-        const u32x4* src = (const u32x4*)(p.Xp + (size_t)ck * 16 * XR);
+        const u32x4* src = (const u32x4*)(p.Xp + (size_t)ck * 16 * NT * XR);
 #pragma unroll
         for (int q = 0; q < NP; q++)
             if (tid + 256 * q < PIECES) stage[q] = src[tid + 256 * q];
@@ -552,12 +554,14 @@ __global__ void __launch_bounds__(256, F::ROWS_OCCUPANCY) gemm_q_f16x2_rows_kern
         }
         if (F::TAIL && lane < 32) *(uint16_t*)(wl + lane * F::LROW + F::TAIL) = (uint16_t)gt;
     };
-    float rsv[4];
+    float rsv[NT][4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int t = 4 * (g4 & 1) + r;
-        rsv[r] = p.rs[t < p.T ? t : 0];
-    }
+    for (int q = 0; q < NT; q++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int t = 8 * q + 4 * (g4 & 1) + r;
+            rsv[q][r] = p.rs[t < p.T ? t : 0];
+        }
     if (u >= u_end) return;
 
     // The workgroup's run of units is one stream: the chunk after a group's last is the next group's first, fetched and
@@ -570,7 +574,7 @@ __global__ void __launch_bounds__(256, F::ROWS_OCCUPANCY) gemm_q_f16x2_rows_kern
     if (u + 1 < u_end) load_w(u + 1);
     __syncthreads();
 
-    f32x4 total[2];
+    f32x4 total[2][NT];
     for (int it = 0; u < u_end; u++, it++) {
         const int buf = it & 1;
         const int grp = (int)(u / nchunks), ck = (int)(u - (long long)grp * nchunks);
@@ -578,34 +582,46 @@ __global__ void __launch_bounds__(256, F::ROWS_OCCUPANCY) gemm_q_f16x2_rows_kern
         if (more) load_x(ck + 1 < nchunks ? ck + 1 : 0);
         if (u == u_begin || ck == 0) {
 #pragma unroll
-            for (int s = 0; s < 2; s++) total[s] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int q = 0; q < NT; q++) total[s][q] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
         for (int s = 0; s < 2; s++) {
             typename F::Raw raw;
             F::from_lds(raw, wl + (16 * s + c) * F::LROW, g4);
             typename F::Ctx x;
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            f32x4 acc[NT];
+#pragma unroll
+            for (int q = 0; q < NT; q++) acc[q] = (f32x4){0.f, 0.f, 0.f, 0.f};
             static_for<0, 8>([&](auto Ic) {
                 constexpr int I = decltype(Ic)::value;
-                const f16x8 a = *(const f16x8*)(&Xs[buf][a_rd + 32 * I]);
                 F::template pre<I>(raw, g4, x);
                 const f16x8 b = F::template frag<I>(raw, x);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
-                // keeps the MFMA here: left alone, the optimiser sinks the whole chain below the last fragment and holds all eight
-                // fragments and operand rows in registers meanwhile
-                asm volatile("" : "+v"(acc));
+#pragma unroll
+                for (int q = 0; q < NT; q++) {
+                    const f16x8 a = *(const f16x8*)(&Xs[buf][a_rd + 16 * q * XR + 32 * I]);
+                    acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[q], 0, 0, 0);
+                    // keeps the MFMA here: left alone, the optimiser sinks the whole chain below the last fragment and holds all
+                    // eight fragments and operand rows in registers meanwhile
+                    asm volatile("" : "+v"(acc[q]));
+                }
             });
             if constexpr (F::HAS_MIN) {
-                const f16x8 am = *(const f16x8*)(&Xs[buf][m_rd]);
                 const f16x8 bm = F::mins(raw, g4);
-                const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-                const f32x4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm, z, 0, 0, 0);
 #pragma unroll
-                for (int r = 0; r < 4; r++) total[s][r] = fmaf(x.dm, accm[r], total[s][r]);
+                for (int q = 0; q < NT; q++) {
+                    const f16x8 am = *(const f16x8*)(&Xs[buf][m_rd + 16 * q * XR]);
+                    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm, z, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x.dm, accm[r], total[s][q][r]);
+                }
             }
 #pragma unroll
-            for (int r = 0; r < 4; r++) total[s][r] = fmaf(x.d, acc[r], total[s][r]);
+            for (int q = 0; q < NT; q++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x.d, acc[q][r], total[s][q][r]);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (more) {
@@ -619,12 +635,14 @@ __global__ void __launch_bounds__(256, F::ROWS_OCCUPANCY) gemm_q_f16x2_rows_kern
 #pragma unroll
             for (int s = 0; s < 2; s++)
 #pragma unroll
+              for (int q = 0; q < NT; q++)
+#pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const int t = 4 * (g4 & 1) + r, n = grp * 128 + wave * 32 + 16 * s + c;
-                    float v = total[s][r];
+                    const int t = 8 * q + 4 * (g4 & 1) + r, n = grp * 128 + wave * 32 + 16 * s + c;
+                    float v = total[s][q][r];
                     v += __shfl_xor(v, 32);
                     if (g4 < 2 && t < p.T && n < p.N) {
-                        v *= rsv[r];
+                        v *= rsv[q][r];
                         float* y = p.Y + (size_t)t * p.N + n;
                         if (whole) *y = v;
                         else unsafeAtomicAdd(y, v);
@@ -654,7 +672,8 @@ Plan make_plan(const fhip_weight* w, size_t t) {
     const long long groups = ((long long)w->rows + 127) / 128;
     q.units = groups * q.nchunks;
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    const long long wgs = cus * (w->type == FHIP_Q6_K ? (q.nt == 1 ? Q6K::ROWS_OCCUPANCY : Q6K::occupancy(q.nt)) : (q.nt == 1 ? Q4K::ROWS_OCCUPANCY : Q4K::occupancy(q.nt)));
+    const long long wgs = cus * (w->type == FHIP_Q6_K ? (q.nt == 1 ? Q6K::ROWS_OCCUPANCY : q.nt == 2 && Q6K::ROWS_AT_16 ? 2 : Q6K::occupancy(q.nt))
+                                                   : (q.nt == 1 ? Q4K::ROWS_OCCUPANCY : q.nt == 2 && Q4K::ROWS_AT_16 ? 2 : Q4K::occupancy(q.nt)));
     // one workgroup per resident slot, each with the same share of the units (a grid of 2.66 workgroups per CU leaves
     // two thirds of the CUs with half as much again to do as the rest); shares of three quarters of a group's chunks or
     // more are rounded to whole groups, which store instead of adding
@@ -691,7 +710,8 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, si
         const size_t n = t * w->rows;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
     }
-    if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F>), dim3(q.grid), dim3(256), 0, s, p);
+    if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 1>), dim3(q.grid), dim3(256), 0, s, p);
+    else if (q.nt == 2 && F::ROWS_AT_16) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
     else if (q.nt == 2) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
     else hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 4>), dim3(q.grid), dim3(256), 0, s, p);
     return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
