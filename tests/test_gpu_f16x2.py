@@ -127,6 +127,26 @@ def test_config3_ffn_block(F, O, batch):
     assert np.abs(y - y32).max() / np.abs(y32).max() < 2e-6
 
 
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+def test_random_shapes_against_the_f32_path(F, O, ty):
+    # 24 seeded random (rows of x, rows of W, columns) triples: every branch of the launch plan (whole groups, dealt runs,
+    # runs that cross group boundaries, weights shorter than a workgroup's share) against the exact f32 mat-vec path
+    from ferric_amd.synth import synth_weights
+    rng = np.random.default_rng(1234 + ty)
+    for _ in range(24):
+        t = int(rng.integers(1, 33))
+        n = int(rng.choice([1, 7, 16, 31, 33, 127, 128, 129, 255, 300, 511, 777, 1500, 4100]))
+        k = 256 * int(rng.choice([1, 2, 3, 5, 8, 13, 20, 31]))
+        w = synth_weights(ty, n, k, int(rng.integers(1 << 30)))
+        x = (rng.standard_normal((t, k)) * 10.0 ** rng.uniform(-3, 3, size=(t, 1))).astype(np.float32)
+        qm = F.QMatrix.from_bytes(w, ty, n, k)
+        y = F.Tensor.from_vec(x, x.shape).matmul_q_f16x2(qm).to_vec().reshape(t, n)
+        f32 = F.Tensor.from_vec(x, x.shape).matmul_q(qm).to_vec().reshape(t, n)
+        wn = np.linalg.norm(O.deq_raw(w, n * k, ty).reshape(n, k).astype(np.float64), axis=1)
+        bound = 2 * TIGHT * wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None]   # two paths, each within TIGHT
+        assert (np.abs(y - f32) <= bound + 1e-300).all(), (ty, t, n, k)
+
+
 def test_replays_in_a_graph(F, O):
     # the six launches of the block captured once and replayed with new inputs in the same buffers: every replay must
     # match an eager call on the same input (up to the order of the K-split additions)
