@@ -102,6 +102,30 @@ def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed
     return out, alg, nbytes
 
 
+def bench_q80_batch(F, lib, check, stream, timer, rows=4096, cols=4096, batch=8, ncopy=32):
+    """configs[0]'s weight at a batch of 8 activation rows, cold (32 rotating copies, 571 MB): the one-pass f16 hi/lo
+    matmul against the exact-f32 mat-vec kernel, which needs a pass over the weights per two rows."""
+    from ferric_amd.synth import synth_weights
+    nbytes = weight_bytes(Q8_0, rows, cols)
+    buf = replicate(F, lib, check, synth_weights(Q8_0, rows, cols, 0), ncopy)
+    ws = [F.QMatrix.wrap_device(buf, nbytes, Q8_0, rows, cols, offset=i * nbytes) for i in range(ncopy)]
+    x = F.Tensor.from_vec(np.random.default_rng(2).standard_normal((batch, cols)).astype(np.float32), (batch, cols))
+    y = F.Tensor.empty((batch, rows))
+    scratch = F.DeviceBuffer(max(256, lib.fhip_matmul_q_f16x2_ws_bytes(ws[0].handle, batch)))
+
+    def timed(launch):
+        g = F.Graph.begin(stream)
+        for w in ws:
+            launch(w)
+        g.end()
+        g.launch()
+        return min(timer.time_ms(g.launch) for _ in range(3)) / ncopy * 1e3
+
+    one_pass = timed(lambda w: check(lib.fhip_matmul_q_f16x2(w.handle, x.buf.ptr, batch, y.buf.ptr, scratch.ptr, stream.handle)))
+    per_row = timed(lambda w: check(lib.fhip_matmul_q(w.handle, x.buf.ptr, batch, y.buf.ptr, stream.handle)))
+    return {"batch": batch, "f16x2_us": one_pass, "f16x2_weight_GBps": nbytes / one_pass / 1e3, "f32_matvec_us": per_row}
+
+
 def launch_floor_us(F, lib, check, stream, timer, n=2048):
     """What one launch costs in a graph on this box when the kernel does nothing to speak of (one workgroup adds 0 to a
     word): the part of every per-launch figure in this file that no kernel can win back."""
@@ -542,7 +566,8 @@ def main():
         log("[bench] Q8_0 GEMV 4096x4096 ...")
         c1, alg1, _ = bench_gemv(F, lib, check, stream, timer, Q8_0, 4096, 4096, args.steps, args.warmup, seed=0, x_seed=0, ncopy=56)
         line["q8_0_gemv_4096"] = {"cold_GBps": c1["cold"]["GBps"], "cold_us": c1["cold"]["ms_per_step"] * 1e3,
-                                  "warm_GBps": c1["warm"]["GBps"], "algorithmic_bytes": alg1}
+                                  "warm_GBps": c1["warm"]["GBps"], "algorithmic_bytes": alg1,
+                                  "batch8": bench_q80_batch(F, lib, check, stream, timer)}
     if not args.no_ffn:
         log("[bench] Q4_K_M FFN block, batch 1/4/8 ...")
         ffn, wb = bench_ffn(F, lib, check, stream, timer, (1, 4, 8))

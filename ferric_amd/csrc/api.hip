@@ -609,8 +609,11 @@ size_t fhip_matmul_q_f16x2_ws_bytes(const fhip_weight* w, size_t rows_x) {
 
 static int f16x2_checks(const char* who, const fhip_weight* w, size_t rows_x) {
     if (rows_x > 32) return set_error(FHIP_ERR_SHAPE, "%s: at most 32 activation rows (got %zu)", who, rows_x);
-    if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K)
-        return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "%s: no kernel for ggml type %u (Q4_K and Q6_K only)", who, w->type);
+    if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0)
+        return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "%s: no kernel for ggml type %u (Q4_K, Q6_K and Q8_0 only)", who, w->type);
+    if (w->type == FHIP_Q8_0 && rows_x > 16) return set_error(FHIP_ERR_SHAPE, "%s: at most 16 activation rows for Q8_0 (got %zu)", who, rows_x);
+    if (rows_x && w->rows && !fhip::gemm_f16x2_supports(w, rows_x))
+        return set_error(FHIP_ERR_SHAPE, "%s: weight rows of %zu columns are outside what the kernels take", who, w->cols);
     return FHIP_OK;
 }
 

@@ -11,6 +11,8 @@
 //     operand holds sc*q as f16 and the f32 factor d is applied to the f32 accumulator once per super-block. The Q4_K
 //     minima are one more MFMA per super-block: sum_sb m[n, sb] * (sum of the activations of sub-block sb). (Q6_K:
 //     |sc*(q-32)| can reach 4096; products above 2048 are rounded to even, a relative 2^-12 on those weights.)
+//     Q8_0 (:2948-2990) is d * (int8): the B operand holds the quant, the f32 result of every 32-wide slice takes its
+//     block's d.
 //   * Activations. A row is scaled by a power of two so that its largest magnitude lies in [2^14, 2^15), then split
 //     into hi = f16(x) and lo = f16(x - hi): two operand rows per activation row, 22 significant bits. The 16 rows of
 //     a v_mfma_f32_16x16x32_f16 hold hi and lo of 8 activation rows; the two partial results are added in f32 at the
@@ -62,6 +64,8 @@ constexpr uint32_t HNEG64 = 0xD400D400u;     // (-64, -64)
 constexpr uint32_t HNEG96 = 0xD600D600u;     // (-96, -96)
 constexpr uint32_t H16TH = 0x2C002C00u;      // (1/16, 1/16)
 
+struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };   // 16 bytes at an address that is only 2-byte aligned
+
 constexpr int CHUNK = 256;   // columns per chunk: one K-quant super-block
 // f16 per staged operand row of a chunk: 256 activations, 8 sub-block sums, 8 zeros, 8 of padding (row stride 35 x 16
 // bytes: the 16 rows a 16-byte read instruction touches fall into different bank groups)
@@ -108,9 +112,15 @@ struct Q4K {
     }
     static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) { h.hd = *(const u32x4*)(row + (size_t)c * BLOCK); }
     // row-streaming kernel: a block is PARTS 16-byte pieces in global memory and a row of LROW bytes in the wave's LDS image
-    static constexpr int PARTS = 9, LROW = 144, TAIL = 0, ROWS_OCCUPANCY = 3;   // 120 VGPRs, 36 KB of LDS (four per CU ran slower: 36.7 vs 34.0 us)
+    static constexpr int PARTS = 9, LROW = 144, TAILS = 0, ROWS_OCCUPANCY = 3;   // 120 VGPRs, 36 KB of LDS (four per CU ran slower: 36.7 vs 34.0 us)
     static constexpr bool ROWS_AT_16 = false;   // 9..16 rows, cold weights: 44.9 us against 42.0 us for the one-row-per-lane kernel
+    static constexpr bool ROW_PER_LANE = true, SLICE_SCALE = false;
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return *(const u32x4*)p; }
+    // where 16-byte piece `part` of chunk ck starts in the weight row / in the LDS row (tails: 2-byte pieces)
+    static __device__ __forceinline__ uint32_t piece_off(int ck, int part, int) { return (uint32_t)(ck * BLOCK + 16 * part); }
+    static __device__ __forceinline__ int piece_lds(int part) { return 16 * part; }
+    static __device__ __forceinline__ uint32_t tail_off(int, int, int, bool& live) { live = false; return 0; }
+    static __device__ __forceinline__ int tail_lds(int) { return 0; }
     static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) {
         r.hd = *(const u32x4*)row;
         r.q0 = *(const u32x4*)(row + 16 + 32 * g4);
@@ -195,10 +205,14 @@ struct Q6K {
     // row-streaming kernel: 13 16-byte pieces + the 2-byte d; LDS rows of 240 bytes (a multiple of 16 whose dword count,
     // 60, puts the 16 rows of a read instruction into different banks). Contiguous lanes read contiguous bytes here, which
     // the 2-byte alignment of the blocks does not slow down.
-    static constexpr int PARTS = 13, LROW = 240, TAIL = 208, ROWS_OCCUPANCY = 3;   // 134 VGPRs, 49 KB of LDS
+    static constexpr int PARTS = 13, LROW = 240, TAILS = 1, ROWS_OCCUPANCY = 3;   // 134 VGPRs, 49 KB of LDS
     static constexpr bool ROWS_AT_16 = true;    // 9..16 rows, cold weights: 33.2 us against 41.2 us
-    struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };
+    static constexpr bool ROW_PER_LANE = true, SLICE_SCALE = false;
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return ((const U4A2*)p)->v; }
+    static __device__ __forceinline__ uint32_t piece_off(int ck, int part, int) { return (uint32_t)(ck * BLOCK + 16 * part); }
+    static __device__ __forceinline__ int piece_lds(int part) { return 16 * part; }
+    static __device__ __forceinline__ uint32_t tail_off(int ck, int, int, bool& live) { live = true; return (uint32_t)(ck * BLOCK + 208); }
+    static __device__ __forceinline__ int tail_lds(int) { return 208; }
     static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) {
         const int hf = g4 >> 1, lh = g4 & 1;
         r.ql[0] = *(const u32x4*)(row + 64 * hf + 16 * lh);
@@ -258,6 +272,57 @@ struct Q6K {
         o[1] = hfma2(p1, x.s[flo], clo);
         o[2] = hfma2(p2, x.s[fhi], chi);
         o[3] = hfma2(p3, x.s[fhi], chi);
+        return __builtin_bit_cast(f16x8, o);
+    }
+    static __device__ __forceinline__ f16x8 mins(const Raw&, int) { return (f16x8){0, 0, 0, 0, 0, 0, 0, 0}; }
+};
+
+
+// Q8_0: 34-byte blocks of 32 int8 under one f16 scale (crates/ferric-gguf/src/lib.rs:855-872), eight blocks to a chunk.
+// Only the row-streaming kernel reads it. A weight enters the B operand as the exact integer q; the block's scale is
+// applied to the f32 result of each 32-wide slice, which is one block. The LDS row is the chunk's 256 quants followed
+// by its 8 scales: 272 bytes, 68 dwords, so the 8-byte reads of a half wave (16 rows x 2 k-groups) cover all 64 banks.
+struct Q80 {
+    static constexpr int BLOCK = 34;
+    static constexpr bool HAS_MIN = false;
+    static __host__ __device__ constexpr int occupancy(int) { return 2; }
+    static __host__ __device__ constexpr int src_k(int pos) { return pos; }   // slice I is block I, in order
+    static __host__ __device__ constexpr int pos_of(int k) { return k; }
+    static constexpr int PARTS = 16, LROW = 272, TAILS = 8, ROWS_OCCUPANCY = 3;
+    static constexpr bool ROWS_AT_16 = true;
+    static constexpr bool ROW_PER_LANE = false, SLICE_SCALE = true;
+    static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return ((const U4A2*)p)->v; }
+    // a row that ends inside its last chunk: the blocks past the end re-read the last real block and get scale 0
+    static __device__ __forceinline__ uint32_t piece_off(int ck, int part, int nblk) {
+        const int b = 8 * ck + (part >> 1);
+        return (uint32_t)(BLOCK * (b < nblk ? b : nblk - 1) + 2 + 16 * (part & 1));
+    }
+    static __device__ __forceinline__ int piece_lds(int part) { return 16 * part; }
+    static __device__ __forceinline__ uint32_t tail_off(int ck, int t, int nblk, bool& live) {
+        const int b = 8 * ck + t;
+        live = b < nblk;
+        return (uint32_t)(BLOCK * (live ? b : nblk - 1));
+    }
+    static __device__ __forceinline__ int tail_lds(int t) { return 256 + 2 * t; }
+    struct Raw { const uint8_t* row; };
+    struct Ctx { float d, dm; };
+    static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) { r.row = row + 8 * g4; }
+    template <int I>
+    static __device__ __forceinline__ void pre(const Raw& r, int g4, Ctx& x) {
+        x.d = f16_bits(*(const uint16_t*)(r.row - 8 * g4 + 256 + 2 * I));
+        x.dm = 0.f;
+    }
+    template <int I>
+    static __device__ __forceinline__ f16x8 frag(const Raw& r, const Ctx&) {
+        const u32x2 q = *(const u32x2*)(r.row + 32 * I);
+        // int8 q -> the byte q + 128 in the mantissa of the f16 constant 1024 -> minus 1152
+        const uint32_t a = q[0] ^ 0x80808080u, b = q[1] ^ 0x80808080u;
+        constexpr uint32_t HNEG1152 = 0xE480E480u;
+        u32x4 o;
+        o[0] = hadd2(__builtin_amdgcn_perm(0x64646464u, a, 0x04010400u), HNEG1152);
+        o[1] = hadd2(__builtin_amdgcn_perm(0x64646464u, a, 0x04030402u), HNEG1152);
+        o[2] = hadd2(__builtin_amdgcn_perm(0x64646464u, b, 0x04010400u), HNEG1152);
+        o[3] = hadd2(__builtin_amdgcn_perm(0x64646464u, b, 0x04030402u), HNEG1152);
         return __builtin_bit_cast(f16x8, o);
     }
     static __device__ __forceinline__ f16x8 mins(const Raw&, int) { return (f16x8){0, 0, 0, 0, 0, 0, 0, 0}; }
@@ -346,6 +411,7 @@ struct F16Params {
     const float* rs;      // [T] row scales to take out
     float* Y;             // [T, N]
     int T, N, nchunks;
+    int nblk;             // Q8_0: blocks in a weight row (the last chunk may hold fewer than 8)
     size_t row_bytes;
     long long units;      // 128-row groups * nchunks, chunk fastest
 };
@@ -531,28 +597,42 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
     // piece i * 64 + lane of the wave's chunk image is 16-byte part (piece % PARTS) of row (piece / PARTS)
     uint8_t* const wl = Wl[wave];
     u32x4 G[NW];
-    uint32_t gt = 0;
+    constexpr int NTL = (32 * F::TAILS + 63) / 64;   // 2-byte tail pieces per lane
+    uint32_t gt[NTL ? NTL : 1];
     // requests the bytes of unit `v` = (128-row group, chunk); rows past the end of the weight repeat its last row
     auto load_w = [&](long long v) {
         const int grp = (int)(v / nchunks), ck = (int)(v - (long long)grp * nchunks);
         const int row0 = grp * 128 + wave * 32 < p.N ? grp * 128 + wave * 32 : p.N - 1;
         const int rmax = p.N - 1 - row0;
-        const uint8_t* b = p.W + (size_t)row0 * p.row_bytes + (size_t)ck * F::BLOCK;
+        const uint8_t* b = p.W + (size_t)row0 * p.row_bytes;
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int pc = i * 64 + lane, row = pc / F::PARTS;
-            const uint32_t off = (uint32_t)(row < rmax ? row : rmax) * (uint32_t)p.row_bytes + 16u * (uint32_t)(pc - row * F::PARTS);
+            const uint32_t off = (uint32_t)(row < rmax ? row : rmax) * (uint32_t)p.row_bytes + F::piece_off(ck, pc - row * F::PARTS, p.nblk);
             if (pc < WP) G[i] = F::ldg(b + off);
         }
-        if (F::TAIL && lane < 32) gt = *(const uint16_t*)(b + (uint32_t)(lane < rmax ? lane : rmax) * (uint32_t)p.row_bytes + F::TAIL);
+#pragma unroll
+        for (int i = 0; i < NTL; i++) {
+            const int tc = i * 64 + lane, row = tc / (F::TAILS ? F::TAILS : 1);
+            bool live;
+            const uint32_t off = (uint32_t)(row < rmax ? row : rmax) * (uint32_t)p.row_bytes + F::tail_off(ck, tc - row * F::TAILS, p.nblk, live);
+            if (tc < 32 * F::TAILS) {
+                gt[i] = *(const uint16_t*)(b + off);
+                if (!live) gt[i] = 0;
+            }
+        }
     };
     auto park_w = [&]() {
 #pragma unroll
         for (int i = 0; i < NW; i++) {
             const int pc = i * 64 + lane, row = pc / F::PARTS;
-            if (pc < WP) *(u32x4*)(wl + row * F::LROW + 16 * (pc - row * F::PARTS)) = G[i];
+            if (pc < WP) *(u32x4*)(wl + row * F::LROW + F::piece_lds(pc - row * F::PARTS)) = G[i];
         }
-        if (F::TAIL && lane < 32) *(uint16_t*)(wl + lane * F::LROW + F::TAIL) = (uint16_t)gt;
+#pragma unroll
+        for (int i = 0; i < NTL; i++) {
+            const int tc = i * 64 + lane, row = tc / (F::TAILS ? F::TAILS : 1);
+            if (tc < 32 * F::TAILS) *(uint16_t*)(wl + row * F::LROW + F::tail_lds(tc - row * F::TAILS)) = (uint16_t)gt[i];
+        }
     };
     float rsv[NT][4];
 #pragma unroll
@@ -592,19 +672,44 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
             F::from_lds(raw, wl + (16 * s + c) * F::LROW, g4);
             typename F::Ctx x;
             f32x4 acc[NT];
+            float dprev = 0.f;
 #pragma unroll
             for (int q = 0; q < NT; q++) acc[q] = (f32x4){0.f, 0.f, 0.f, 0.f};
             static_for<0, 8>([&](auto Ic) {
                 constexpr int I = decltype(Ic)::value;
                 F::template pre<I>(raw, g4, x);
                 const f16x8 b = F::template frag<I>(raw, x);
+                if constexpr (F::SLICE_SCALE) {
+                    // every slice has a scale of its own: its product starts from zero, and joins the total while the next
+                    // slice's MFMA runs
+                    f32x4 cur[NT];
 #pragma unroll
-                for (int q = 0; q < NT; q++) {
-                    const f16x8 a = *(const f16x8*)(&Xs[buf][a_rd + 16 * q * XR + 32 * I]);
-                    acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[q], 0, 0, 0);
-                    // keeps the MFMA here: left alone, the optimiser sinks the whole chain below the last fragment and holds all
-                    // eight fragments and operand rows in registers meanwhile
-                    asm volatile("" : "+v"(acc[q]));
+                    for (int q = 0; q < NT; q++) {
+                        const f16x8 a = *(const f16x8*)(&Xs[buf][a_rd + 16 * q * XR + 32 * I]);
+                        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                        cur[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, z, 0, 0, 0);
+                        asm volatile("" : "+v"(cur[q]));
+                    }
+                    if constexpr (I > 0) {
+#pragma unroll
+                        for (int q = 0; q < NT; q++) {
+#pragma unroll
+                            for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(dprev, acc[q][r], total[s][q][r]);
+                            asm volatile("" : "+v"(total[s][q]));
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < NT; q++) acc[q] = cur[q];
+                    dprev = x.d;
+                } else {
+#pragma unroll
+                    for (int q = 0; q < NT; q++) {
+                        const f16x8 a = *(const f16x8*)(&Xs[buf][a_rd + 16 * q * XR + 32 * I]);
+                        acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[q], 0, 0, 0);
+                        // keeps the MFMA here: left alone, the optimiser sinks the whole chain below the last fragment and holds
+                        // all eight fragments and operand rows in registers meanwhile
+                        asm volatile("" : "+v"(acc[q]));
+                    }
                 }
             });
             if constexpr (F::HAS_MIN) {
@@ -618,6 +723,7 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
                     for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x.dm, accm[r], total[s][q][r]);
                 }
             }
+            // the chunk's product (the last slice's, where every slice has its own scale)
 #pragma unroll
             for (int q = 0; q < NT; q++)
 #pragma unroll
@@ -665,15 +771,18 @@ struct Plan {
     bool split;
 };
 
+// workgroups of the kernel that serves `nt` operand row sets that fit on a CU together
+template <class F>
+constexpr int slots(int nt) { return nt == 1 ? F::ROWS_OCCUPANCY : (nt == 2 && F::ROWS_AT_16 ? 2 : F::occupancy(nt)); }
+
 Plan make_plan(const fhip_weight* w, size_t t) {
     Plan q;
     q.nt = t <= 8 ? 1 : (t <= 16 ? 2 : 4);
-    q.nchunks = (int)(w->cols / CHUNK);
+    q.nchunks = (int)((w->cols + CHUNK - 1) / CHUNK);
     const long long groups = ((long long)w->rows + 127) / 128;
     q.units = groups * q.nchunks;
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    const long long wgs = cus * (w->type == FHIP_Q6_K ? (q.nt == 1 ? Q6K::ROWS_OCCUPANCY : q.nt == 2 && Q6K::ROWS_AT_16 ? 2 : Q6K::occupancy(q.nt))
-                                                   : (q.nt == 1 ? Q4K::ROWS_OCCUPANCY : q.nt == 2 && Q4K::ROWS_AT_16 ? 2 : Q4K::occupancy(q.nt)));
+    const long long wgs = cus * (w->type == FHIP_Q6_K ? slots<Q6K>(q.nt) : w->type == FHIP_Q8_0 ? slots<Q80>(q.nt) : slots<Q4K>(q.nt));
     // one workgroup per resident slot, each with the same share of the units (a grid of 2.66 workgroups per CU leaves
     // two thirds of the CUs with half as much again to do as the rest); shares of three quarters of a group's chunks or
     // more are rounded to whole groups, which store instead of adding
@@ -705,6 +814,7 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, si
     F16Params p;
     p.W = w->d_raw; p.Xp = d_xp; p.rs = d_rs; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.nchunks = q.nchunks; p.row_bytes = w->row_bytes;
+    p.nblk = (int)(w->cols / 32);
     p.units = q.units;
     if (q.split && !y_cleared) {
         const size_t n = t * w->rows;
@@ -712,8 +822,12 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, si
     }
     if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 1>), dim3(q.grid), dim3(256), 0, s, p);
     else if (q.nt == 2 && F::ROWS_AT_16) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
-    else if (q.nt == 2) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 4>), dim3(q.grid), dim3(256), 0, s, p);
+    else if constexpr (F::ROW_PER_LANE) {
+        if (q.nt == 2) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 4>), dim3(q.grid), dim3(256), 0, s, p);
+    } else {
+        return fhip::set_error(FHIP_ERR_SHAPE, "f16x2 matmul: this format takes at most 16 activation rows, got %zu", t);
+    }
     return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
 }
 
@@ -722,8 +836,9 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, si
 namespace fhip {
 
 bool gemm_f16x2_supports(const fhip_weight* w, size_t t) {
-    return w && (w->type == FHIP_Q4_K || w->type == FHIP_Q6_K) && t >= 1 && t <= 32 && w->cols % CHUNK == 0 && w->cols > 0 &&
-           w->cols <= (size_t)MAXW * 1024;
+    if (!w || t < 1 || w->cols == 0 || w->cols > (size_t)MAXW * 1024) return false;
+    if (w->type == FHIP_Q8_0) return t <= 16 && w->cols % 32 == 0;   // rows of any whole number of blocks
+    return (w->type == FHIP_Q4_K || w->type == FHIP_Q6_K) && t <= 32 && w->cols % CHUNK == 0;
 }
 
 size_t gemm_f16x2_aux_bytes() { return 256 + 32 * MAXW * sizeof(float); }   // row scales, then the partial row maxima
@@ -742,6 +857,7 @@ int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swi
     switch (w->type) {
         case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
         case FHIP_Q6_K: return launch_xsplit_fmt<Q6K>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
+        case FHIP_Q8_0: return launch_xsplit_fmt<Q80>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
     }
 }
@@ -750,6 +866,7 @@ int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, const float* d
     switch (w->type) {
         case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, d_rs, t, d_y, s, y_cleared);
         case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, d_rs, t, d_y, s, y_cleared);
+        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, d_rs, t, d_y, s, y_cleared);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
     }
 }

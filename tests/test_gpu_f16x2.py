@@ -5,6 +5,7 @@ of f16 (22 significant bits). Bars, against the oracle's dequantized weights in 
   * |y - y64| <= 2.5e-7 * ||w_row|| * ||x_t||  (measured <= 6e-8; the exact-f32 mat-vec path measures <= 5e-8 on the same
     inputs), 4000x inside the north-star bound 1e-3 * ||w_row|| * ||x_t||;
   * max|d| / max|ref| < 1e-5, the bar the f32 mat-vec tests use;
+  * Q8_0 (quants are exact in f16, one f32 scale per 32-wide slice) keeps the same 2.5e-7 bar; at most 16 activation rows;
   * Q6_K only, blocks whose |scale * (q - 32)| exceeds 2048: such a product is rounded to an even integer on its way
     into f16, a relative 2^-12 on that weight, so the bar there is 2.5e-4 * ||w_row|| * ||x_t|| (still 4x inside the
     north-star bound) -- the test builds such blocks on purpose and also checks that ordinary ones stay at 2.5e-7.
@@ -31,17 +32,21 @@ def run_case(F, O, ty, t, n, k, seed, x=None, w=None, tol=TIGHT):
     return y, y64
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
 def test_small_and_ragged_shapes(F, O, ty):
     # every activation-row count class (1..8 -> one group of operand rows, 9..16 -> two, 17..32 -> four), weight rows that
     # do not fill a 16-row set, a 128-row group or a workgroup's share, one chunk and many
     shapes = [(1, 32, 256), (2, 100, 512), (3, 128, 256), (5, 300, 1024), (8, 256, 2048), (9, 130, 768), (16, 257, 1024),
               (17, 64, 512), (31, 15, 256), (32, 200, 1536), (4, 1, 256), (7, 1000, 5120)]
+    if ty == Q8_0:
+        # at most 16 rows; rows of any whole number of 32-column blocks: shorter than a chunk, ending inside the last one
+        shapes = [s for s in shapes if s[0] <= 16] + [(3, 40, 32), (8, 64, 96), (9, 130, 288), (16, 70, 480), (5, 257, 1184),
+                                                      (1, 4096, 4096)]
     for i, (t, n, k) in enumerate(shapes):
         run_case(F, O, ty, t, n, k, 100 + i)
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
 def test_rows_of_very_different_magnitude(F, O, ty):
     # each row is scaled by its own power of two: tiny, huge, zero and outlier rows side by side keep the per-row bound
     t, n, k = 8, 96, 1024
@@ -87,7 +92,20 @@ def test_q6_k_products_beyond_the_exact_f16_range(F, O):
     run_case(F, O, Q6_K, t, n, k, 13, w=w.reshape(-1))
 
 
-@pytest.mark.parametrize("ty,n,k", [(Q4_K, 512, 2048), (Q6_K, 384, 1024)])
+def test_q8_0_every_int8_value_and_scale_signs(F, O):
+    # quants over all 256 byte values (-128 included), scales of both signs, zero and the largest finite f16 magnitude class
+    n, k, t = 48, 512, 4
+    rng = np.random.default_rng(14)
+    w = np.zeros((n, k // 32, 34), np.uint8)
+    w[:, :, 2:] = rng.integers(0, 256, (n, k // 32, 32), dtype=np.uint8)
+    w[0, 0, 2:] = np.arange(32, dtype=np.uint8) * 8          # 0, 8, .., 248: both halves of the int8 range in one block
+    w[1, 1, 2:] = 0x80
+    d = rng.choice(np.array([0.0, -0.03, 0.5, 1e-4, -2048.0, 6e-8], np.float16), size=(n, k // 32))
+    w[:, :, 0:2] = d.view(np.uint8).reshape(n, k // 32, 2)
+    run_case(F, O, Q8_0, t, n, k, 15, w=w.reshape(-1))
+
+
+@pytest.mark.parametrize("ty,n,k", [(Q4_K, 512, 2048), (Q6_K, 384, 1024), (Q8_0, 640, 1120)])
 def test_agrees_with_the_f32_matvec_path_and_rows_are_independent(F, O, ty, n, k):
     from ferric_amd.synth import synth_weights
     w = synth_weights(ty, n, k, 20)
@@ -127,16 +145,38 @@ def test_config3_ffn_block(F, O, batch):
     assert np.abs(y - y32).max() / np.abs(y32).max() < 2e-6
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("tg,td", [(Q8_0, Q8_0), (Q4_K, Q8_0), (Q8_0, Q6_K)])
+def test_ffn_block_with_q8_0_weights(F, O, tg, td):
+    # the block with Q8_0 on either side, a hidden width that ends inside a chunk for the Q8_0 down projection
+    from ferric_amd.synth import synth_weights
+    n_embd, n_ff, batch = 768, (1120 if td == Q8_0 else 1280), 7
+    gu = synth_weights(tg, 2 * n_ff, n_embd, 40)
+    dn = synth_weights(td, n_embd, n_ff, 41)
+    x = np.random.default_rng(42).standard_normal((batch, n_embd)).astype(np.float32)
+    wgu, wdn = F.QMatrix.from_bytes(gu, tg, 2 * n_ff, n_embd), F.QMatrix.from_bytes(dn, td, n_embd, n_ff)
+    xt = F.Tensor.from_vec(x, x.shape)
+    y = xt.ffn_f16x2(wgu, wdn).to_vec().reshape(batch, n_embd)
+    g64, _ = O.matmul_f64(x, gu, tg, 2 * n_ff, n_embd)
+    h64 = g64[:, :n_ff] / (1.0 + np.exp(-g64[:, :n_ff])) * g64[:, n_ff:]
+    y64, wn = O.matmul_f64(h64.astype(np.float32), dn, td, n_embd, n_ff)
+    assert (np.abs(y - y64) <= 1e-6 * wn[None, :] * np.linalg.norm(h64, axis=1)[:, None]).all()
+    if tg != Q8_0:      # the exact-f32 block takes K-quant gate|up weights only
+        y32 = xt.ffn(wgu, wdn).to_vec().reshape(batch, n_embd)
+        assert np.abs(y - y32).max() / np.abs(y32).max() < 2e-6
+
+
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
 def test_random_shapes_against_the_f32_path(F, O, ty):
     # 24 seeded random (rows of x, rows of W, columns) triples: every branch of the launch plan (whole groups, dealt runs,
     # runs that cross group boundaries, weights shorter than a workgroup's share) against the exact f32 mat-vec path
     from ferric_amd.synth import synth_weights
     rng = np.random.default_rng(1234 + ty)
     for _ in range(24):
-        t = int(rng.integers(1, 33))
+        t = int(rng.integers(1, 17 if ty == Q8_0 else 33))
         n = int(rng.choice([1, 7, 16, 31, 33, 127, 128, 129, 255, 300, 511, 777, 1500, 4100]))
         k = 256 * int(rng.choice([1, 2, 3, 5, 8, 13, 20, 31]))
+        if ty == Q8_0:
+            k = max(32, k - 32 * int(rng.integers(0, 8)))     # rows that end anywhere inside their last chunk
         w = synth_weights(ty, n, k, int(rng.integers(1 << 30)))
         x = (rng.standard_normal((t, k)) * 10.0 ** rng.uniform(-3, 3, size=(t, 1))).astype(np.float32)
         qm = F.QMatrix.from_bytes(w, ty, n, k)
@@ -182,12 +222,16 @@ def test_argument_checks(F):
     from ferric_amd.synth import synth_weights
     q4 = F.QMatrix.from_bytes(synth_weights(Q4_K, 32, 256, 1), Q4_K, 32, 256)
     q8 = F.QMatrix.from_bytes(synth_weights(Q8_0, 32, 256, 1), Q8_0, 32, 256)
-    assert lib.fhip_matmul_q_f16x2_ws_bytes(q4.handle, 8) > 0
-    assert lib.fhip_matmul_q_f16x2_ws_bytes(q4.handle, 33) == 0 and lib.fhip_matmul_q_f16x2_ws_bytes(q8.handle, 8) == 0
+    q40 = F.QMatrix.from_bytes(synth_weights(2, 32, 256, 1), 2, 32, 256)     # Q4_0: served by the mat-vec path only
+    assert lib.fhip_matmul_q_f16x2_ws_bytes(q4.handle, 8) > 0 and lib.fhip_matmul_q_f16x2_ws_bytes(q8.handle, 16) > 0
+    assert lib.fhip_matmul_q_f16x2_ws_bytes(q4.handle, 33) == 0 and lib.fhip_matmul_q_f16x2_ws_bytes(q40.handle, 8) == 0
+    assert lib.fhip_matmul_q_f16x2_ws_bytes(q8.handle, 17) == 0
     with pytest.raises(AssertionError, match="at most 32 activation rows"):
         F.Tensor.from_vec(np.zeros((33, 256), np.float32), (33, 256)).matmul_q_f16x2(q4)
-    with pytest.raises(ValueError, match="Q4_K and Q6_K only"):
-        F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256)).matmul_q_f16x2(q8)
+    with pytest.raises(AssertionError, match="at most 16 activation rows for Q8_0"):
+        F.Tensor.from_vec(np.zeros((17, 256), np.float32), (17, 256)).matmul_q_f16x2(q8)
+    with pytest.raises(ValueError, match="Q4_K, Q6_K and Q8_0 only"):
+        F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256)).matmul_q_f16x2(q40)
     with pytest.raises(AssertionError, match="inner dim mismatch"):
         F.Tensor.from_vec(np.zeros((2, 512), np.float32), (2, 512)).matmul_q_f16x2(q4)
     x = F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256))
