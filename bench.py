@@ -411,7 +411,8 @@ def probe_f16x2(F, lib, check, ncopy=4):
     """Work for a profiler run of the small-batch f16 matrix-core path at 8 activation rows: fhip_matmul_q_f16x2 on the
     gate|up (34816 x 5120 Q4_K) and down (5120 x 17408 Q6_K) weights, then the whole block through fhip_ffn_f16x2, 12
     launches each, eagerly on the null stream, rotating over 4 copies of each weight (694 MB in all, more than the
-    Infinity Cache holds) so that every launch reads HBM."""
+    Infinity Cache holds) so that every launch reads HBM. Last, 32 launches of fhip_matmul_q_f16x2 over 32 copies of a
+    4096 x 4096 Q8_0 weight (571 MB) and 16 over 16 copies of a 12288 x 4096 one (857 MB), 8 rows each."""
     from ferric_amd.synth import synth_weights
     n_embd, n_ff, t = 5120, 17408, 8
     gbuf = replicate(F, lib, check, synth_weights(Q4_K, 2 * n_ff, n_embd, 3), ncopy)
@@ -433,6 +434,18 @@ def probe_f16x2(F, lib, check, ncopy=4):
     for i in range(12):
         check(lib.fhip_ffn_f16x2(gus[i % ncopy].handle, dns[i % ncopy].handle, x.buf.ptr, t, y.buf.ptr, ws.ptr, None))
     check(lib.fhip_stream_sync(None))
+    del gus, dns, gbuf, dbuf
+    for rows, nc in ((4096, 32), (12288, 16)):
+        nb = weight_bytes(Q8_0, rows, 4096)
+        qbuf = replicate(F, lib, check, synth_weights(Q8_0, rows, 4096, 0), nc)
+        x8 = F.Tensor.from_vec(rng.standard_normal((t, 4096)).astype(np.float32), (t, 4096))
+        y8 = F.Tensor.empty((t, rows))
+        ws8 = None
+        for i in range(nc):
+            w = F.QMatrix.wrap_device(qbuf, nb, Q8_0, rows, 4096, offset=i * nb)
+            ws8 = ws8 or F.DeviceBuffer(lib.fhip_matmul_q_f16x2_ws_bytes(w.handle, t))
+            check(lib.fhip_matmul_q_f16x2(w.handle, x8.buf.ptr, t, y8.buf.ptr, ws8.ptr, None))
+        check(lib.fhip_stream_sync(None))
 
 
 def probe_decode(F, lib, check):
