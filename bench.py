@@ -3,15 +3,15 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-sweep] [--no-ffn] [--no-cpu]
 
-Headline workload (BASELINE.json configs[1]): Q4_K GEMV, W 5120x5120 (102400 super-blocks, 14745600 B),
+Headline workload (the second of the benchmark configurations): Q4_K GEMV, W 5120x5120 (102400 super-blocks, 14745600 B),
 x f32[5120], batch 1. One "step" is one GEMV. Steps rotate over 64 distinct copies of the weight
 (944 MB, larger than the 256 MB Infinity Cache) so every step streams its weight bytes from HBM;
 the same loop over ONE copy is reported as the cache-resident ("warm") figure beside it.
 All K steps are recorded into one HIP graph on one stream and timed with HIP events on that stream.
 
 Prints ONE JSON line. `value` = algorithmic bytes per step (weights + x + y) * K / elapsed, in GB/s.
-Also measured in the same run and carried in the line: the 64-layer decode weight sweep (configs[4]),
-the Q4_K_M FFN block at batch 1/4/8 (configs[2]), the Q8_0 GEMV (configs[0]) and the CPU baseline.
+Also measured in the same run and carried in the line: the 64-layer decode weight sweep, the Q4_K_M FFN block at
+batch 1/4/8, the Q8_0 GEMV (the reference's CPU-runnable case), the prefill dequant-GEMM and the CPU baseline.
 """
 import argparse
 import ctypes as C
@@ -103,7 +103,7 @@ def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed
 
 
 def bench_q80_batch(F, lib, check, stream, timer, rows=4096, cols=4096, batch=8, ncopy=32):
-    """configs[0]'s weight at a batch of 8 activation rows, cold (32 rotating copies, 571 MB): the one-pass f16 hi/lo
+    """The 4096 x 4096 Q8_0 weight at a batch of 8 activation rows, cold (32 rotating copies, 571 MB): the one-pass f16 hi/lo
     matmul against the exact-f32 mat-vec kernel, which needs a pass over the weights per two rows."""
     from ferric_amd.synth import synth_weights
     nbytes = weight_bytes(Q8_0, rows, cols)
@@ -141,7 +141,7 @@ def launch_floor_us(F, lib, check, stream, timer, n=2048):
 
 
 def bench_ffn(F, lib, check, stream, timer, batches, reps=20, ncopy=4):
-    """The FFN block of configs[2] on its three paths. Cold figures: the launches of the timed graph rotate over `ncopy`
+    """The Q4_K_M FFN block (gate|up 2 x (5120 -> 17408) Q4_K, down 17408 -> 5120 Q6_K) on its three paths. Cold figures: the launches of the timed graph rotate over `ncopy`
     distinct copies of both weights (4 x 173 MB = 694 MB > the 256 MB Infinity Cache), so every launch reads HBM; the
     warm figure (one copy, which the cache can hold) is reported beside it for the f32 path."""
     from ferric_amd.synth import synth_weights
@@ -252,7 +252,7 @@ def bench_gguf(F, lib, check, n_tensors=8, rows=11008, cols=5120):
 
 
 def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
-    """configs[4]: per layer fused QKV 5120->7168, O 5120->5120, fused gate+up 5120->34816 (+SwiGLU), all Q4_K,
+    """The decode weight sweep: per layer fused QKV 5120->7168, O 5120->5120, fused gate+up 5120->34816 (+SwiGLU), all Q4_K,
     down 17408->5120 Q6_K; lm_head 5120->151936 Q6_K. One stream, one graph of layers*4+1 launches."""
     from ferric_amd.synth import synth_weights
     shapes = [("qkv", Q4_K, 7168, 5120), ("o", Q4_K, 5120, 5120), ("gate_up", Q4_K, 34816, 5120), ("down", Q6_K, 5120, 17408)]
@@ -289,7 +289,7 @@ def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
 
 
 def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), layers=64, steps=6):
-    """configs[4] as a real decode step: the same 64-layer stack (fused QKV 5120->7168 with 40 query / 8 KV heads of 128, O,
+    """The decode weight sweep as a real decode step: the same 64-layer stack (fused QKV 5120->7168 with 40 query / 8 KV heads of 128, O,
     fused gate|up 5120->34816 + SwiGLU, all Q4_K; down 17408->5120 Q6_K; output norm + lm_head 151936 Q6_K), but with every op fed
     by the one before it: RMSNorm, q/k norm + rope + KV append, attention over `context` cached tokens (f32 cache), residual
     adds. One graph per step, replayed `steps` times at consecutive positions."""
@@ -342,7 +342,7 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
 
 
 def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
-    """configs[3]: W 5120x5120 Q4_K, X [T, 5120] bf16 -> f32 [T, 5120] on the matrix cores; and the same on the
+    """Prefill: W 5120x5120 Q4_K, X [T, 5120] bf16 -> f32 [T, 5120] on the matrix cores; and the same on the
     layer's largest projection (fused gate|up, 34816x5120), where the launch has enough tiles to fill the chip."""
     from ferric_amd.synth import synth_weights
     res = {}
