@@ -112,7 +112,11 @@ int fhip_init(int device) {
 const char* fhip_last_error(void) { return g_err; }
 int fhip_device_cus(void) { return g_cus; }
 
+// bytes per element of the unquantized tensor types (crates/ferric-gguf/src/lib.rs:473-475), 0 for anything else
+static size_t dense_elem_bytes(uint32_t ty) { return ty == FHIP_F32 ? 4 : (ty == FHIP_F16 || ty == FHIP_BF16 ? 2 : 0); }
+
 size_t fhip_type_size(uint32_t ty, size_t n) {
+    if (const size_t eb = dense_elem_bytes(ty)) return n * eb;
     size_t vals, bytes;
     if (!block_info(ty, vals, bytes)) { set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", ty); return 0; }
     return n / vals * bytes;
@@ -281,6 +285,24 @@ int fhip_dequant_rows(const fhip_weight* w, size_t row0, size_t nrows, float* d_
 int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ty, float* h_out, size_t* n_written) {
     int rc = need_init();
     if (rc) return rc;
+    if (const size_t eb = dense_elem_bytes(ty)) {
+        // lib.rs:499-501: raw[..n * size] first (a panic when the bytes are short), then exactly n values
+        if (nbytes / eb < n) return set_error(FHIP_ERR_SHAPE, "range end index %zu out of range for slice of length %zu", n * eb, nbytes);
+        if (n_written) *n_written = n;
+        if (n == 0) return FHIP_OK;
+        if (!h_raw || !h_out) return set_error(FHIP_ERR_ARG, "fhip_deq_raw: NULL pointer");
+        if (ty == FHIP_F32) { memcpy(h_out, h_raw, n * 4); return FHIP_OK; }   // the bytes as they are
+        void *d_in = nullptr, *d_out = nullptr;
+        if ((rc = check_hip(hipMalloc(&d_in, n * 2), "hipMalloc"))) return rc;
+        if ((rc = check_hip(hipMalloc(&d_out, n * sizeof(float)), "hipMalloc"))) { (void)hipFree(d_in); return rc; }
+        rc = check_hip(hipMemcpy(d_in, h_raw, n * 2, hipMemcpyHostToDevice), "hipMemcpy H2D");
+        if (!rc) rc = ty == FHIP_F16 ? fhip::launch_f16_to_f32((const uint16_t*)d_in, n, (float*)d_out, nullptr)
+                                     : fhip::launch_bf16_to_f32((const uint16_t*)d_in, n, (float*)d_out, nullptr);
+        if (!rc) rc = check_hip(hipMemcpy(h_out, d_out, n * sizeof(float), hipMemcpyDeviceToHost), "hipMemcpy D2H");
+        (void)hipFree(d_in);
+        (void)hipFree(d_out);
+        return rc;
+    }
     size_t vals, bytes;
     if (!block_info(ty, vals, bytes)) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "unsupported ggml type %u", ty);
     if (n && !h_out) return set_error(FHIP_ERR_ARG, "fhip_deq_raw: NULL output");

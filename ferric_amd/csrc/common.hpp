@@ -62,6 +62,7 @@ size_t device_lds_bytes();  // LDS one workgroup may use
 
 // dequant.hip
 int launch_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_t s);
+int launch_bf16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_t s);
 int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d_out, hipStream_t s);
 
 // gemv.hip

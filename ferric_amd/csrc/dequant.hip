@@ -31,6 +31,12 @@ __global__ void f16_to_f32_kernel(const uint16_t* __restrict__ in, size_t n, flo
     if (i < n) out[i] = f16_bits(in[i]);
 }
 
+// crates/ferric-gguf/src/lib.rs:501: a bf16 pattern is the top half of the f32 pattern
+__global__ void bf16_to_f32_kernel(const uint16_t* __restrict__ in, size_t n, float* __restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = __uint_as_float((uint32_t)in[i] << 16);
+}
+
 // ---- Q8_0: 34 B = [f16 d][i8 q[32]] ------------------------------------------------------------
 __global__ void deq_q8_0_kernel(const uint8_t* __restrict__ raw, size_t nquads, float* __restrict__ out) {
     size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;  // one lane = 4 values
@@ -229,6 +235,13 @@ int launch_f16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_
     unsigned grid = (unsigned)((n + 255) / 256);
     hipLaunchKernelGGL(f16_to_f32_kernel, dim3(grid), dim3(256), 0, s, d_bits, n, d_out);
     return check_hip(hipGetLastError(), "f16_to_f32 launch");
+}
+
+int launch_bf16_to_f32(const uint16_t* d_bits, size_t n, float* d_out, hipStream_t s) {
+    if (n == 0) return FHIP_OK;
+    unsigned grid = (unsigned)((n + 255) / 256);
+    hipLaunchKernelGGL(bf16_to_f32_kernel, dim3(grid), dim3(256), 0, s, d_bits, n, d_out);
+    return check_hip(hipGetLastError(), "bf16_to_f32 launch");
 }
 
 int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d_out, hipStream_t s) {

@@ -106,6 +106,17 @@ class Gguf:
         a.flags.writeable = False
         return a
 
+    def dequant(self, name):
+        """The tensor as f32, row-major, whatever its type -- lib.rs:456 / :575 (deq_raw over the tensor's bytes, on the GPU)."""
+        from .qmatrix import deq_raw
+        t = self.tensor(name)
+        if t is None:
+            raise ValueError(f"no tensor '{name}'")
+        n = 1
+        for d in t.dims:
+            n *= int(d)
+        return deq_raw(self.raw(name), n, t.ggml_type)
+
     def qmatrix(self, name):
         """Upload the tensor straight from the mapping: dims [in, out] (or [in, rows per expert, n_expert])."""
         t = self.tensor(name)

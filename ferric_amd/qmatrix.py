@@ -21,6 +21,7 @@ from . import _lib
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13   # further formats: unpackers, mat-vec / small batch, "_id" variants
 IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39             # codebook / microscaling formats, same coverage
+F32, F16, BF16 = 0, 1, 30                      # unquantized tensor types: type_size and deq_raw only (lib.rs:473-475, 499-501)
 
 
 def _vp(a):
@@ -491,14 +492,15 @@ Mxfp4Weights = _typed(MXFP4, "Mxfp4Weights")
 
 def type_size(ty, n):
     """Bytes of n elements of ggml type ty -- lib.rs:471; unknown type -> ValueError."""
-    if QMatrix.block_bytes(ty) is None:
+    if QMatrix.block_bytes(ty) is None and ty not in (F32, F16, BF16):
         raise ValueError(f"unsupported ggml type {ty}")
     return int(_lib.load().fhip_type_size(ty, n))
 
 
 def deq_raw(raw, n, ty):
     """Dequantize n elements out of raw block bytes on the GPU -- lib.rs:497. Same edge behaviour:
-    every format returns n values with a ragged tail left 0.0, except Q8_0, which returns whole blocks only."""
+    every format returns n values with a ragged tail left 0.0, except Q8_0, which returns whole blocks only; the
+    unquantized types F32 / F16 / BF16 need all n elements' bytes (fewer: AssertionError, the reference's slice panic)."""
     lib = _lib.init()
     a = np.ascontiguousarray(raw, dtype=np.uint8)
     out = np.empty(n, dtype=np.float32)

@@ -44,6 +44,11 @@ extern "C" {
 #define FHIP_IQ4_NL 20u
 #define FHIP_IQ4_XS 23u
 #define FHIP_MXFP4 39u
+/* unquantized tensor types (crates/ferric-gguf/src/lib.rs:473-475, 499-501): sizes and deq_raw only; a weight handle
+ * takes block formats only (crates/ferric-tensor/src/dtype.rs:853-855 sends these to the dense matmul) */
+#define FHIP_F32 0u
+#define FHIP_F16 1u
+#define FHIP_BF16 30u
 
 #define FHIP_OK 0
 #define FHIP_ERR_UNSUPPORTED_TYPE (-1) /* reference: Err("unsupported ggml type N") / Err("QMatrix: no native matmul ...") */
@@ -143,7 +148,9 @@ int fhip_dequant_rows(const fhip_weight* w, size_t row0, size_t nrows, float* d_
 /* crates/ferric-gguf/src/lib.rs:497 deq_raw(raw, n, ty) with host buffers on both sides: uploads,
  * dequantizes on the GPU, downloads, synchronises. h_out must hold n f32. *n_written receives what
  * the reference's Vec would hold: n for the K-quants (a ragged tail stays 0.0), whole blocks only
- * for Q8_0. Only min(n / block_values, nbytes / block_bytes) whole blocks are read. */
+ * for Q8_0. Only min(n / block_values, nbytes / block_bytes) whole blocks are read. The unquantized types
+ * (FHIP_F32 / FHIP_F16 / FHIP_BF16, lib.rs:499-501) give exactly n values and need n elements' bytes: fewer is
+ * FHIP_ERR_SHAPE (the reference's slice panics). F32 is a byte copy on the host; the other two convert on the GPU. */
 int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ggml_type, float* h_out, size_t* n_written);
 
 /* ---- matmuls ------------------------------------------------------------------------------- */

@@ -37,6 +37,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#define GGML_F32 0u
+#define GGML_F16 1u
+#define GGML_BF16 30u
 #define GGML_Q4_0 2u
 #define GGML_Q4_1 3u
 #define GGML_Q5_0 6u
@@ -112,6 +115,9 @@ static inline uint16_t rd_u16(const uint8_t* b) { return (uint16_t)(b[0] | (b[1]
  * Integer division truncates exactly as the reference's `n / 32 * 34`. */
 size_t fo_type_size(uint32_t ty, size_t n) {
     switch (ty) {
+        case GGML_F32: return n * 4;
+        case GGML_F16: return n * 2;
+        case GGML_BF16: return n * 2;
         case GGML_Q8_0: return n / 32 * 34;
         case GGML_Q4_K: return n / 256 * 144;
         case GGML_Q6_K: return n / 256 * 210;
@@ -402,8 +408,29 @@ size_t fo_deq_mxfp4(const uint8_t* raw, size_t raw_len, size_t n, float* out) {
 
 /* crates/ferric-gguf/src/lib.rs:497-520 (deq_raw), in-scope types. Returns the number of f32 the
  * reference's Vec would hold, or (size_t)-1 for "unsupported ggml type". */
+/* The unquantized arms (lib.rs:499-501) slice raw[..n * size] first, which panics when the bytes are short:
+ * (size_t)-2 stands for that panic. F32: little-endian bytes as they are; F16: the exact decode; BF16: the 16
+ * bits become the top half of the f32 pattern. */
 size_t fo_deq_raw(const uint8_t* raw, size_t raw_len, size_t n, uint32_t ty, float* out) {
     switch (ty) {
+        case GGML_F32:
+            if (raw_len < n * 4) return (size_t)-2;
+            for (size_t i = 0; i < n; i++) {
+                uint32_t b = (uint32_t)raw[4 * i] | ((uint32_t)raw[4 * i + 1] << 8) | ((uint32_t)raw[4 * i + 2] << 16) | ((uint32_t)raw[4 * i + 3] << 24);
+                memcpy(out + i, &b, 4);
+            }
+            return n;
+        case GGML_F16:
+            if (raw_len < n * 2) return (size_t)-2;
+            for (size_t i = 0; i < n; i++) out[i] = fo_f16_to_f32(rd_u16(raw + 2 * i));
+            return n;
+        case GGML_BF16:
+            if (raw_len < n * 2) return (size_t)-2;
+            for (size_t i = 0; i < n; i++) {
+                uint32_t b = (uint32_t)rd_u16(raw + 2 * i) << 16;
+                memcpy(out + i, &b, 4);
+            }
+            return n;
         case GGML_Q8_0: return fo_deq_q8_0(raw, raw_len, n, out);
         case GGML_Q4_K: return fo_deq_q4_k(raw, raw_len, n, out);
         case GGML_Q6_K: return fo_deq_q6_k(raw, raw_len, n, out);

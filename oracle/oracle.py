@@ -19,6 +19,9 @@ IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39
 BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24),
          Q5_K: (256, 176), IQ4_NL: (32, 18), IQ4_XS: (256, 136), MXFP4: (32, 17)}
 
+F32, F16, BF16 = 0, 1, 30
+DENSE = {F32: 4, F16: 2, BF16: 2}          # unquantized tensor types: bytes per element
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libferric_oracle.so")
 
@@ -112,18 +115,21 @@ def f32_to_f16_bits(x):
 def type_size(ty, n):
     """Bytes of n elements of ggml type ty; raises ValueError('unsupported ggml type N') like the
     reference's Err(String)."""
-    if ty not in BLOCK:
+    if ty not in BLOCK and ty not in DENSE:
         raise ValueError(f"unsupported ggml type {ty}")
     return int(lib().fo_type_size(ty, n))
 
 
 def deq_raw(raw, n, ty):
-    """Reference-order dequantization of n elements (Q8_0 returns a shorter array on a ragged tail)."""
-    if ty not in BLOCK:
+    """Reference-order dequantization of n elements (Q8_0 returns a shorter array on a ragged tail; the unquantized
+    types slice the bytes first and so panic -- AssertionError here -- when there are fewer than n elements)."""
+    if ty not in BLOCK and ty not in DENSE:
         raise ValueError(f"unsupported ggml type {ty}")
     raw, rp = _u8(raw)
     out = np.zeros(n, dtype=np.float32)
     got = lib().fo_deq_raw(rp, raw.size, n, ty, out.ctypes.data_as(_f32p))
+    if got == C.c_size_t(-2).value:
+        raise AssertionError(f"range end index {n * DENSE[ty]} out of range for slice of length {raw.size}")
     return out[:got]
 
 

@@ -41,6 +41,7 @@ def test_size_tables_need_no_device():
     assert QMatrix.block_bytes(10) is None and QMatrix.block_bytes(0) is None
     assert type_size(8, 4096 * 4096) == 17825792 and type_size(12, 5120 * 5120) == 14745600 and type_size(14, 5120 * 17408) == 73113600
     assert type_size(12, 300) == 144
+    assert type_size(0, 5120) == 20480 and type_size(1, 5120) == 10240 and type_size(30, 5120) == 10240   # F32, F16, BF16
     assert type_size(13, 5120 * 5120) == 18022400 and type_size(2, 64) == 36 and type_size(7, 33) == 24
     with pytest.raises(ValueError, match="unsupported ggml type 10"):
         type_size(10, 256)

@@ -91,6 +91,27 @@ def test_deq_raw_edge_semantics(F, O):
         F.deq_raw(np.zeros(84, np.uint8), 256, 10)
 
 
+def test_deq_raw_unquantized_types(F, O):
+    # lib.rs:499-501: F32 / F16 / BF16 tensors through the same entry point, every 16-bit pattern, bit for bit
+    pats = np.arange(65536, dtype=np.uint16).view(np.uint8)
+    for ty in (F.F16, F.BF16):
+        got, want = F.deq_raw(pats, 65536, ty), O.deq_raw(pats, 65536, ty)
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan)
+        assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+        assert_bits_equal(F.deq_raw(pats[:2000], 1000, ty), O.deq_raw(pats[:2000], 1000, ty))
+        assert F.deq_raw(pats, 0, ty).size == 0
+        with pytest.raises(AssertionError, match="out of range"):
+            F.deq_raw(pats[:7], 4, ty)
+    raw32 = np.random.default_rng(0).integers(0, 1 << 32, 5000, dtype=np.uint64).astype(np.uint32)
+    raw32[:4] = [0x7FC00001, 0xFF800000, 0x00000001, 0x80000000]
+    assert np.array_equal(F.deq_raw(raw32.view(np.uint8), 5000, F.F32).view(np.uint32), raw32)
+    assert F.deq_raw(raw32.view(np.uint8), 17, F.F32).size == 17
+    with pytest.raises(AssertionError, match="out of range"):
+        F.deq_raw(raw32.view(np.uint8)[:15], 4, F.F32)
+    assert F.type_size(F.F32, 5120) == 20480 and F.type_size(F.F16, 5120) == 10240 and F.type_size(F.BF16, 3) == 6
+
+
 @pytest.mark.parametrize("ty,rows,cols", [(Q4_K, 64, 5120), (Q6_K, 33, 5120), (Q8_0, 40, 4096)])
 def test_resident_weight_row_dequant(F, O, ty, rows, cols):
     # embedding-row dequant out of a weight already in HBM (crates/ferric-llama/src/qwen3.rs:749)

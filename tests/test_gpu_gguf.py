@@ -20,8 +20,10 @@ def test_weights_from_a_gguf_file(F, O, tmp_path):
     raw["blk.0.ffn_down_exps.weight"] = synth_weights(Q4_K, n_expert * rows_pe, cols, 9)
     tensors = [(n, [c, r], ty, raw[n]) for n, (ty, r, c) in shapes.items()]
     tensors.append(("blk.0.ffn_down_exps.weight", [cols, rows_pe, n_expert], Q4_K, raw["blk.0.ffn_down_exps.weight"]))
-    tensors.append(("blk.0.attn_norm.weight", [1024], 0, np.zeros(4096, np.uint8)))
-    tensors.append(("token_embd.weight", [64, 8], 1, np.zeros(1024, np.uint8)))
+    norm = np.random.default_rng(3).standard_normal(1024).astype(np.float32)
+    embd = np.random.default_rng(4).standard_normal(512).astype(np.float16)
+    tensors.append(("blk.0.attn_norm.weight", [1024], 0, norm.view(np.uint8)))
+    tensors.append(("token_embd.weight", [64, 8], 1, embd.view(np.uint8)))
     data = write_gguf([("general.architecture", "str", "qwen3")], tensors)[0]
     path = tmp_path / "tiny.gguf"
     path.write_bytes(data)
@@ -49,5 +51,11 @@ def test_weights_from_a_gguf_file(F, O, tmp_path):
     with pytest.raises(ValueError, match="no native matmul for ggml type 1"):
         g.qmatrix("token_embd.weight")               # F16 [64, 8]: not one of the quantized formats of this path
     assert g.raw("token_embd.weight").size == 1024
+    # lib.rs:575 dequant(name): any tensor of the file as f32, the unquantized ones included
+    assert np.array_equal(g.dequant("blk.0.attn_norm.weight").view(np.uint32), norm.view(np.uint32))
+    assert np.array_equal(g.dequant("token_embd.weight").view(np.uint32), embd.astype(np.float32).view(np.uint32))
+    assert np.array_equal(g.dequant("blk.0.ffn_down.weight").view(np.uint32), O.deq_raw(raw["blk.0.ffn_down.weight"], 40 * 512, Q6_K).view(np.uint32))
+    with pytest.raises(ValueError, match="no tensor"):
+        g.dequant("missing")
     with pytest.raises(ValueError, match="no tensor"):
         g.qmatrix("missing")

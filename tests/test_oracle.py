@@ -29,6 +29,32 @@ def test_f16_exhaustive_against_numpy(O):
     assert np.array_equal(bits(got)[~nan], bits(want)[~nan])
 
 
+def test_deq_raw_unquantized_types(O):
+    # crates/ferric-gguf/src/lib.rs:499-501. F16 against numpy over every pattern; BF16 against torch's own bfloat16 -> float32
+    # conversion over every pattern; F32 is the bytes as they are, NaN payloads included.
+    import torch
+    F32, F16, BF16 = 0, 1, 30
+    pats = np.arange(65536, dtype=np.uint16)
+    got = O.deq_raw(pats.view(np.uint8), 65536, F16)
+    want = pats.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(bits(got)[~nan], bits(want)[~nan])
+    got = O.deq_raw(pats.view(np.uint8), 65536, BF16)
+    want = torch.from_numpy(pats.view(np.int16).copy()).view(torch.bfloat16).to(torch.float32).numpy()
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(bits(got)[~nan], bits(want)[~nan])
+    assert bits(O.deq_raw(np.array([0x80, 0x3F], np.uint8), 1, BF16))[0] == 0x3F800000        # 1.0
+    assert float(O.deq_raw(np.array([0x49, 0x40], np.uint8), 1, BF16)[0]) == 3.140625        # bf16(pi)
+    raw32 = np.random.default_rng(0).integers(0, 1 << 32, 4096, dtype=np.uint64).astype(np.uint32)
+    raw32[:4] = [0x7FC00001, 0xFF800000, 0x00000001, 0x80000000]
+    assert np.array_equal(bits(O.deq_raw(raw32.view(np.uint8), 4096, F32)), raw32)
+    assert O.deq_raw(raw32.view(np.uint8), 100, F32).size == 100 and O.deq_raw(np.zeros(0, np.uint8), 0, BF16).size == 0
+    assert O.type_size(F32, 7) == 28 and O.type_size(F16, 7) == 14 and O.type_size(BF16, 7) == 14
+    for ty, short in ((F32, 15), (F16, 7), (BF16, 7)):      # four elements asked for, bytes for three and a half
+        with pytest.raises(AssertionError, match="out of range"):
+            O.deq_raw(np.zeros(short, np.uint8), 4, ty)
+
+
 def test_f16_reference_landmarks(O, golden):
     # crates/ferric-tensor/src/cpu_simd.rs:203-213
     t = O.f16_table()
