@@ -98,6 +98,12 @@ SYMBOLS = {
     "fhip_debug_generic_matvec": (C.c_int, [C.c_int]),
     "fhip_u32_add": (C.c_int, [_vp, _sz, _u32, _vp]),
     "fhip_matvec_q8_0_host": (C.c_int, [_vp, _vp, _sz, _sz, _sz, _vp]),
+    "fhip_pool_create": (C.c_int, [_sz, _vp]),
+    "fhip_pool_threads": (_sz, [_vp]),
+    "fhip_pool_uploads": (_sz, [_vp]),
+    "fhip_pool_forget": (None, [_vp]),
+    "fhip_pool_destroy": (None, [_vp]),
+    "fhip_matvec_q8_0_pooled": (C.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _sz, _sz, _vp]),
 }
 
 _lib = None

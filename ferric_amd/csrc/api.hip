@@ -713,4 +713,94 @@ int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, si
     return rc;
 }
 
+// ---- crates/ferric-tensor/src/cpu_simd.rs:238-331: Pool / matvec_q8_0_pooled --------------------------------
+// The reference's pool exists so that a call does not pay its set-up again (thread creation there). What a call of the
+// host-buffer mat-vec pays here is the upload of the weight bytes, so the pool keeps those resident: the weight the
+// last call used stays in HBM, keyed by the caller's (pointer, length, cols) -- `w` is an immutable Arc<Vec<u8>> in the
+// reference -- together with the staging buffers and a stream of its own.
+struct fhip_pool {
+    size_t threads;
+    hipStream_t stream;
+    const uint8_t* key;
+    size_t key_len, key_cols;
+    uint8_t* d_w;
+    size_t w_cap;
+    float *d_x, *d_y;
+    size_t x_cap, y_cap;
+    size_t uploads;
+};
+
+int fhip_pool_create(size_t threads, fhip_pool** out) {
+    if (!out) return set_error(FHIP_ERR_ARG, "fhip_pool_create: NULL output");
+    *out = nullptr;
+    int rc = need_init();
+    if (rc) return rc;
+    fhip_pool* p = new (std::nothrow) fhip_pool();
+    if (!p) return set_error(FHIP_ERR_HIP, "fhip_pool_create: out of host memory");
+    p->threads = threads ? threads : 1;   // Pool::new: n.max(1)
+    if ((rc = check_hip(hipStreamCreate(&p->stream), "hipStreamCreate"))) { delete p; return rc; }
+    *out = p;
+    return FHIP_OK;
+}
+
+size_t fhip_pool_threads(const fhip_pool* p) { return p ? p->threads : 0; }
+size_t fhip_pool_uploads(const fhip_pool* p) { return p ? p->uploads : 0; }
+
+void fhip_pool_forget(fhip_pool* p) {
+    if (p) { p->key = nullptr; p->key_len = 0; p->key_cols = 0; }
+}
+
+void fhip_pool_destroy(fhip_pool* p) {
+    if (!p) return;
+    (void)hipStreamSynchronize(p->stream);
+    if (p->d_w) (void)hipFree(p->d_w);
+    if (p->d_x) (void)hipFree(p->d_x);
+    if (p->d_y) (void)hipFree(p->d_y);
+    (void)hipStreamDestroy(p->stream);
+    delete p;
+}
+
+static int pool_reserve(void** d, size_t* cap, size_t need, const char* what) {
+    if (need <= *cap) return FHIP_OK;
+    if (*d) (void)hipFree(*d);
+    *d = nullptr; *cap = 0;
+    int rc = check_hip(hipMalloc(d, need), what);
+    if (!rc) *cap = need;
+    return rc;
+}
+
+int fhip_matvec_q8_0_pooled(fhip_pool* p, const float* h_x, size_t x_len, const uint8_t* h_w, size_t w_len, size_t cols, size_t lo,
+                            size_t hi, float* h_y) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!p) return set_error(FHIP_ERR_ARG, "fhip_matvec_q8_0_pooled: NULL pool");
+    if (lo > hi) return set_error(FHIP_ERR_SHAPE, "empty or inverted span");             // cpu_simd.rs:311
+    const size_t rows = hi - lo;
+    if (rows == 0) return FHIP_OK;                                                        // :313
+    if (!h_y) return set_error(FHIP_ERR_ARG, "fhip_matvec_q8_0_pooled: NULL output");
+    const size_t nblk = cols / 32, row_bytes = nblk * 34;                                 // :314; row_q8_0 walks cols / 32 blocks
+    if (nblk == 0) { memset(h_y, 0, rows * sizeof(float)); return FHIP_OK; }              // no block: every sum is 0.0
+    // the slices of :321 and of row_q8_0 (:62, :64) panic when the row span or the activations run past their arrays
+    if (hi > w_len / row_bytes) return set_error(FHIP_ERR_SHAPE, "range end index %zu out of range for slice of length %zu", hi * row_bytes, w_len);
+    if (x_len < nblk * 32) return set_error(FHIP_ERR_SHAPE, "range end index %zu out of range for slice of length %zu", nblk * 32, x_len);
+    if (!h_x || !h_w) return set_error(FHIP_ERR_ARG, "fhip_matvec_q8_0_pooled: NULL pointer");
+    const size_t kcols = nblk * 32, all_rows = w_len / row_bytes;
+    if (p->key != h_w || p->key_len != w_len || p->key_cols != kcols) {
+        fhip_pool_forget(p);
+        if ((rc = pool_reserve((void**)&p->d_w, &p->w_cap, all_rows * row_bytes, "hipMalloc"))) return rc;
+        if ((rc = check_hip(hipMemcpyAsync(p->d_w, h_w, all_rows * row_bytes, hipMemcpyHostToDevice, p->stream), "hipMemcpy H2D"))) return rc;
+        p->key = h_w; p->key_len = w_len; p->key_cols = kcols;
+        p->uploads++;
+    }
+    if ((rc = pool_reserve((void**)&p->d_x, &p->x_cap, kcols * sizeof(float), "hipMalloc"))) return rc;
+    if ((rc = pool_reserve((void**)&p->d_y, &p->y_cap, rows * sizeof(float), "hipMalloc"))) return rc;
+    if ((rc = check_hip(hipMemcpyAsync(p->d_x, h_x, kcols * sizeof(float), hipMemcpyHostToDevice, p->stream), "hipMemcpy H2D"))) return rc;
+    fhip_weight view;
+    if ((rc = make_weight(FHIP_Q8_0, rows * row_bytes, rows, kcols, view))) return rc;
+    view.d_raw = p->d_w + lo * row_bytes;
+    if ((rc = fhip::launch_gemv(&view, p->d_x, 1, p->d_y, 0, p->stream))) return rc;
+    if ((rc = check_hip(hipMemcpyAsync(h_y, p->d_y, rows * sizeof(float), hipMemcpyDeviceToHost, p->stream), "hipMemcpy D2H"))) return rc;
+    return check_hip(hipStreamSynchronize(p->stream), "hipStreamSynchronize");
+}
+
 }  // extern "C"

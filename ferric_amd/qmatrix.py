@@ -546,3 +546,48 @@ def matvec_q8_0_span(x, w, cols, lo, hi, threads=1):
     row_bytes = cols // 32 * 34
     w = np.ascontiguousarray(w, dtype=np.uint8)
     return matvec_q8_0_threaded(x, w[lo * row_bytes: hi * row_bytes], hi - lo, cols, threads)
+
+
+class Pool:
+    """cpu_simd.rs:238 Pool: set up once, reused by every matvec_q8_0_pooled call. On the GPU what it keeps is the weight
+    of the last call resident in HBM (and staging buffers, and a stream), so a repeated call uploads the activations only."""
+
+    def __init__(self, n):
+        lib = _lib.init()
+        self.handle = C.c_void_p()
+        _lib.check(lib.fhip_pool_create(int(n), C.byref(self.handle)))
+        self._w = None      # keeps the keyed array alive: its address is the pool's key
+
+    def threads(self):
+        return int(_lib.load().fhip_pool_threads(self.handle))
+
+    def uploads(self):
+        return int(_lib.load().fhip_pool_uploads(self.handle))
+
+    def forget(self):
+        _lib.load().fhip_pool_forget(self.handle)
+        self._w = None
+
+    def close(self):
+        if self.handle:
+            _lib.load().fhip_pool_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def matvec_q8_0_pooled(pool, x, w, cols, lo, hi):
+    """Rows [lo, hi) of y = x . W^T on a pool -- cpu_simd.rs:303. `w` must be a contiguous uint8 array (its address keys the
+    pool's resident copy, as the Arc does in the reference); anything else is copied and uploaded on every call."""
+    lib = _lib.load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if not (isinstance(w, np.ndarray) and w.dtype == np.uint8 and w.flags.c_contiguous):
+        w = np.ascontiguousarray(w, dtype=np.uint8)
+    pool._w = w
+    y = np.empty(max(0, hi - lo), dtype=np.float32)
+    _lib.check(lib.fhip_matvec_q8_0_pooled(pool.handle, _vp(x), x.size, _vp(w), w.size, cols, lo, hi, _vp(y)))
+    return y

@@ -365,6 +365,24 @@ int fhip_weight_from_gguf(const fhip_gguf* g, const char* name, fhip_weight** ou
  * Errors as the reference's asserts: cols % 32, w_len != rows * cols/32*34 -> FHIP_ERR_SHAPE. */
 int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, size_t rows, size_t cols, float* h_y);
 
+/* crates/ferric-tensor/src/cpu_simd.rs:238-300 Pool and :303-331 matvec_q8_0_pooled(pool, x, w, cols, lo, hi): rows
+ * [lo, hi) of y = x . W^T with host buffers on both sides, on a pool that is set up once. The reference's pool saves
+ * the thread creation of every call; what a host-buffer call pays here is the upload of the weight, so the pool keeps
+ * the bytes of the last `h_w` it was given resident in HBM (with its staging buffers and a stream of its own) and a
+ * call with the same (h_w, w_len, cols) uploads the activations only. `w` is an immutable Arc<Vec<u8>> in the
+ * reference; a caller that rewrites the bytes in place calls fhip_pool_forget first. h_y receives hi - lo values.
+ * `threads` is kept for Pool::threads() (at least 1) and partitions nothing here. lo > hi, a span past the rows in
+ * h_w or fewer than cols activations: FHIP_ERR_SHAPE (the reference's assert and slice panics). One call at a time
+ * per pool (the reference serialises Pool::run behind a mutex). */
+typedef struct fhip_pool fhip_pool;
+int fhip_pool_create(size_t threads, fhip_pool** out);
+size_t fhip_pool_threads(const fhip_pool* p);
+size_t fhip_pool_uploads(const fhip_pool* p);   /* weight uploads so far: 1 after any number of calls on one weight */
+void fhip_pool_forget(fhip_pool* p);
+void fhip_pool_destroy(fhip_pool* p);
+int fhip_matvec_q8_0_pooled(fhip_pool* p, const float* h_x, size_t x_len, const uint8_t* h_w, size_t w_len, size_t cols,
+                            size_t lo, size_t hi, float* h_y);
+
 #ifdef __cplusplus
 }
 #endif

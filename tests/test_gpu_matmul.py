@@ -89,6 +89,67 @@ def test_partitioning_changes_nothing_about_the_answer(F, O):  # cpu_simd.rs:175
         assert np.array_equal(bits(whole), bits(joined)), cut
 
 
+# ---------------------------------------------------------------- cpu_simd.rs pool_tests (:333-410) against the pooled entry
+
+def test_pooled_matches_the_plain_answer_for_any_pool_size(F, O):     # cpu_simd.rs:349-360, :362-373
+    rows, cols = 256, 128
+    raw, _ = O.gen_q8_0_synth(rows, cols, 5)
+    x = ((np.arange(cols) * 31 % 97).astype(np.float32) - 48.0) / np.float32(48.0)
+    want = F.matvec_q8_0(x, raw, rows, cols)
+    cpu = O.matvec_q8_0(x, raw, rows, cols)
+    assert np.abs(want - cpu).max() / max(1e-6, np.abs(cpu).max()) < 1e-4
+    for n in (1, 2, 5, 16):
+        pool = F.Pool(n)
+        assert pool.threads() == n
+        assert np.array_equal(bits(F.matvec_q8_0_pooled(pool, x, raw, cols, 0, rows)), bits(want)), n
+    assert F.Pool(0).threads() == 1                                     # Pool::new: n.max(1)
+
+
+def test_spans_compose_through_the_pool_and_the_weight_is_uploaded_once(F, O):   # cpu_simd.rs:375-387, :389-401
+    rows, cols = 128, 64
+    raw, _ = O.gen_q8_0_synth(rows, cols, 2)
+    x = np.full(cols, -1.25, np.float32)
+    pool = F.Pool(4)
+    whole = F.matvec_q8_0(x, raw, rows, cols)
+    for cut in (0, 1, 63, 127, 128):
+        j = np.concatenate([F.matvec_q8_0_pooled(pool, x, raw, cols, 0, cut), F.matvec_q8_0_pooled(pool, x, raw, cols, cut, rows)])
+        assert np.array_equal(bits(j), bits(whole)), cut
+    first = F.matvec_q8_0_pooled(pool, x, raw, cols, 0, rows)
+    for _ in range(20):                                                 # a reused pool does not drift ...
+        assert np.array_equal(bits(F.matvec_q8_0_pooled(pool, x, raw, cols, 0, rows)), bits(first))
+    assert pool.uploads() == 1                                          # ... and sets up once: the point of a pool
+    other, _ = O.gen_q8_0_synth(40, 96, 9)                              # another weight replaces the resident one
+    x2 = np.linspace(-1, 1, 96, dtype=np.float32)
+    assert np.array_equal(bits(F.matvec_q8_0_pooled(pool, x2, other, 96, 3, 29)), bits(F.matvec_q8_0_span(x2, other, 96, 3, 29)))
+    assert pool.uploads() == 2
+    changed = raw.copy()
+    changed[2:34] ^= 0x55                                               # same shape, new array: keyed by address, so uploaded
+    got = F.matvec_q8_0_pooled(pool, x, changed, cols, 0, rows)
+    assert pool.uploads() == 3 and np.array_equal(bits(got), bits(F.matvec_q8_0(x, changed, rows, cols)))
+    changed[36:68] ^= 0x33                                              # rewritten in place: the caller says so
+    pool.forget()
+    got = F.matvec_q8_0_pooled(pool, x, changed, cols, 0, rows)
+    assert pool.uploads() == 4 and np.array_equal(bits(got), bits(F.matvec_q8_0(x, changed, rows, cols)))
+    pool.close()                                                        # cpu_simd.rs:403-409: dropping the pool must not hang
+
+
+def test_pooled_edge_cases(F, O):
+    raw, _ = O.gen_q8_0_synth(8, 64, 1)
+    x = np.ones(64, np.float32)
+    pool = F.Pool(2)
+    assert F.matvec_q8_0_pooled(pool, x, raw, 64, 5, 5).size == 0       # cpu_simd.rs:313
+    with pytest.raises(AssertionError, match="empty or inverted span"):  # :311
+        F.matvec_q8_0_pooled(pool, x, raw, 64, 6, 5)
+    with pytest.raises(AssertionError, match="out of range"):            # the row slice of :321 past the weight
+        F.matvec_q8_0_pooled(pool, x, raw, 64, 0, 9)
+    with pytest.raises(AssertionError, match="out of range"):            # row_q8_0's activation slice
+        F.matvec_q8_0_pooled(pool, x[:40], raw, 64, 0, 8)
+    # a longer activation array is fine (only the first cols values are read), and cols / 32 truncates as in row_q8_0
+    long_x = np.concatenate([x, np.full(7, 9.0, np.float32)])
+    assert np.array_equal(bits(F.matvec_q8_0_pooled(pool, long_x, raw, 64, 0, 8)), bits(F.matvec_q8_0(x, raw, 8, 64)))
+    assert not F.matvec_q8_0_pooled(pool, x, raw, 0, 0, 3).any()        # no block: every sum is 0.0
+
+
 # ---------------------------------------------------------------- benchmark configurations at full size
 
 def test_config1_q8_0_4096(F, O):
