@@ -27,6 +27,7 @@ SYMBOLS = {
     "fhip_memcpy_h2d": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fhip_memcpy_d2h": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fhip_memcpy_d2d": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "fhip_memcpy_2d_d2d": (C.c_int, [_vp, _sz, _vp, _sz, _sz, _sz, _vp]),
     "fhip_memset": (C.c_int, [_vp, C.c_int, _sz, _vp]),
     "fhip_stream_create": (C.c_int, [C.POINTER(_vp)]),
     "fhip_stream_destroy": (C.c_int, [_vp]),
@@ -41,6 +42,7 @@ SYMBOLS = {
     "fhip_graph_launch": (C.c_int, [_vp, _vp]),
     "fhip_graph_destroy": (C.c_int, [_vp]),
     "fhip_weight_create": (C.c_int, [_u32, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "fhip_weight_create_parts": (C.c_int, [C.c_uint32, _vp, _vp, _sz, _sz, _sz, _vp]),
     "fhip_weight_wrap_device": (C.c_int, [_u32, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "fhip_weight_destroy": (None, [_vp]),
     "fhip_weight_rows": (_sz, [_vp]),
@@ -75,6 +77,7 @@ SYMBOLS = {
     "fhip_gguf_meta_i64": (C.c_int, [_vp, C.c_char_p, _sz, _vp]),
     "fhip_gguf_meta_f64": (C.c_int, [_vp, C.c_char_p, _sz, _vp]),
     "fhip_gguf_meta_str": (C.c_int, [_vp, C.c_char_p, _sz, _vp, _vp]),
+    "fhip_weight_from_gguf_cat": (C.c_int, [_vp, _vp, _sz, _vp]),
     "fhip_weight_from_gguf": (C.c_int, [_vp, C.c_char_p, _vp]),
     "fhip_cvt_f32_bf16": (C.c_int, [_vp, _sz, _vp, _vp]),
     "fhip_matmul_q_coop": (C.c_int, [_vp, _vp, _sz, _vp, _vp, _vp]),

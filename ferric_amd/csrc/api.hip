@@ -157,6 +157,12 @@ int fhip_memcpy_d2d(void* dst, const void* src, size_t n, void* s) {
     if (!dst || !src) return set_error(FHIP_ERR_ARG, "fhip_memcpy_d2d: NULL pointer");
     return check_hip(hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToDevice, (hipStream_t)s), "hipMemcpyAsync D2D");
 }
+int fhip_memcpy_2d_d2d(void* d, size_t dpitch, const void* src, size_t spitch, size_t width, size_t height, void* s) {
+    if (width == 0 || height == 0) return FHIP_OK;
+    if (!d || !src) return set_error(FHIP_ERR_ARG, "fhip_memcpy_2d_d2d: NULL pointer");
+    if (dpitch < width || spitch < width) return set_error(FHIP_ERR_ARG, "fhip_memcpy_2d_d2d: pitch smaller than the row width");
+    return check_hip(hipMemcpy2DAsync(d, dpitch, src, spitch, width, height, hipMemcpyDeviceToDevice, (hipStream_t)s), "hipMemcpy2D D2D");
+}
 int fhip_memset(void* d, int byte, size_t n, void* s) {
     if (n == 0) return FHIP_OK;
     if (!d) return set_error(FHIP_ERR_ARG, "fhip_memset: NULL pointer");
@@ -229,6 +235,35 @@ int fhip_weight_create(uint32_t ty, const uint8_t* h_raw, size_t nbytes, size_t 
     if ((rc = check_hip(hipMalloc(&d, nbytes + 256), "hipMalloc(weight)"))) return rc;
     if (nbytes && (rc = check_hip(hipMemcpy(d, h_raw, nbytes, hipMemcpyHostToDevice), "hipMemcpy(weight)"))) { (void)hipFree(d); return rc; }
     if ((rc = check_hip(hipMemset((uint8_t*)d + nbytes, 0, 256), "hipMemset(weight tail)"))) { (void)hipFree(d); return rc; }
+    w.d_raw = (const uint8_t*)d;
+    w.owns = true;
+    *out = new fhip_weight(w);
+    return FHIP_OK;
+}
+
+int fhip_weight_create_parts(uint32_t ty, const uint8_t* const* h_parts, const size_t* part_bytes, size_t n_parts, size_t rows, size_t cols,
+                             fhip_weight** out) {
+    if (!out) return set_error(FHIP_ERR_ARG, "fhip_weight_create_parts: NULL output");
+    *out = nullptr;
+    int rc = need_init();
+    if (rc) return rc;
+    if (n_parts && (!h_parts || !part_bytes)) return set_error(FHIP_ERR_ARG, "fhip_weight_create_parts: NULL part list");
+    size_t nbytes = 0;
+    for (size_t i = 0; i < n_parts; i++) {
+        if (part_bytes[i] && !h_parts[i]) return set_error(FHIP_ERR_ARG, "fhip_weight_create_parts: NULL bytes");
+        nbytes += part_bytes[i];
+    }
+    fhip_weight w;
+    if ((rc = make_weight(ty, nbytes, rows, cols, w))) return rc;
+    void* d = nullptr;
+    if ((rc = check_hip(hipMalloc(&d, nbytes + 256), "hipMalloc(weight)"))) return rc;
+    size_t at = 0;
+    for (size_t i = 0; i < n_parts && !rc; i++) {
+        if (part_bytes[i]) rc = check_hip(hipMemcpy((uint8_t*)d + at, h_parts[i], part_bytes[i], hipMemcpyHostToDevice), "hipMemcpy(weight)");
+        at += part_bytes[i];
+    }
+    if (!rc) rc = check_hip(hipMemset((uint8_t*)d + nbytes, 0, 256), "hipMemset(weight tail)");
+    if (rc) { (void)hipFree(d); return rc; }
     w.d_raw = (const uint8_t*)d;
     w.owns = true;
     *out = new fhip_weight(w);

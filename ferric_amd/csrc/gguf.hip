@@ -372,4 +372,30 @@ int fhip_weight_from_gguf(const fhip_gguf* g, const char* name, fhip_weight** ou
     return fhip_weight_create(t.ggml_type, bytes, nbytes, (size_t)rows, (size_t)t.dims[0], out);
 }
 
+int fhip_weight_from_gguf_cat(const fhip_gguf* g, const char* const* names, size_t n_names, fhip_weight** out) {
+    if (!out) return fhip::set_error(FHIP_ERR_ARG, "fhip_weight_from_gguf_cat: NULL output");
+    *out = nullptr;
+    if (!g || !names || n_names == 0) return fhip::set_error(FHIP_ERR_ARG, "fhip_weight_from_gguf_cat: nothing to concatenate");
+    // crates/ferric-llama/src/qwen35.rs:381-390: one format, one input width, the output widths add up
+    std::vector<const uint8_t*> parts(n_names);
+    std::vector<size_t> sizes(n_names);
+    uint32_t ty = 0;
+    uint64_t inn = 0, rows = 0;
+    for (size_t i = 0; i < n_names; i++) {
+        const char* name = names[i];
+        if (!name) return fhip::set_error(FHIP_ERR_ARG, "fhip_weight_from_gguf_cat: NULL name");
+        const int64_t at = fhip_gguf_find(g, name);
+        if (at < 0) return fhip::set_error(FHIP_ERR_FORMAT, "no tensor '%s'", name);
+        const TensorInfo& t = g->tensors[(size_t)at];
+        if (t.dims.size() < 2) return fhip::set_error(FHIP_ERR_SHAPE, "tensor '%s' has %zu dims; a weight needs [in, out]", name, t.dims.size());
+        if (i == 0) { ty = t.ggml_type; inn = t.dims[0]; }
+        if (t.ggml_type != ty) return fhip::set_error(FHIP_ERR_FORMAT, "%s: mixed quant formats in one fused matmul", name);
+        if (t.dims[0] != inn) return fhip::set_error(FHIP_ERR_FORMAT, "%s: input dim differs", name);
+        rows += t.dims[1];
+        int rc = fhip_gguf_raw(g, name, &parts[i], &sizes[i]);
+        if (rc) return rc;
+    }
+    return fhip_weight_create_parts(ty, parts.data(), sizes.data(), n_names, (size_t)rows, (size_t)inn, out);
+}
+
 }  // extern "C"

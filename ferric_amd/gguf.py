@@ -125,6 +125,23 @@ class Gguf:
         _lib.check(_lib.load().fhip_weight_from_gguf(self._h, name.encode(), C.byref(h)))
         return QMatrix(h, t.ggml_type)
 
+    def qm(self, name):
+        """crates/ferric-llama/src/qwen35.rs:366 qm(ctx, g, name): the tensor as a packed weight [out = dims[1], in = dims[0]]. (The
+        reference's dense fallback for formats without a packed kernel is not part of this path: ValueError.)"""
+        if self.tensor(name) is None:
+            raise ValueError(f"no tensor '{name}'")
+        return self.qmatrix(name)
+
+    def qm_cat(self, names):
+        """qwen35.rs:379 qm_cat(ctx, g, names): same-format tensors of one input width stacked along the output dim into one
+        weight (fused QKV, fused gate|up), each uploaded straight from the mapping to its place in HBM."""
+        names = list(names)
+        arr = (C.c_char_p * len(names))(*[n.encode() for n in names])
+        h = C.c_void_p()
+        _lib.init()
+        _lib.check(_lib.load().fhip_weight_from_gguf_cat(self._h, arr, len(names), C.byref(h)))
+        return QMatrix(h, self.tensor(names[0]).ggml_type)
+
     def close(self):
         if self._h:
             _lib.load().fhip_gguf_close(self._h)
@@ -138,3 +155,37 @@ class Gguf:
 
 
 GgufFile = Gguf
+
+
+class Proj:
+    """crates/ferric-llama/src/qwen3.rs:192-228: a projection made of one or several GGUF tensors. Tensors of one format are fused into
+    one weight (`Fused`); mixed formats (V is often Q6_K beside Q4_K Q and K) stay apart and their outputs are concatenated (`Split`)."""
+
+    def __init__(self, fused=None, split=None):
+        self.fused, self.split = fused, split
+
+    @staticmethod
+    def load(g, names):
+        names = list(names)
+        types = [(g.tensor(n).ggml_type if g.tensor(n) is not None else 0) for n in names]
+        if len(names) > 1 and all(a == b for a, b in zip(types, types[1:])):
+            return Proj(fused=g.qm_cat(names))
+        if len(names) == 1:
+            return Proj(fused=g.qm(names[0]))
+        return Proj(split=[g.qm(n) for n in names])
+
+    def matmul(self, x, stream=None):
+        if self.fused is not None:
+            return x.matmul_q(self.fused, stream)
+        out = x.matmul_q(self.split[0], stream)
+        for w in self.split[1:]:
+            out = out.cat(x.matmul_q(w, stream), 1, stream)
+        return out
+
+    def gate_up_swiglu(self, x, n_ff, stream=None):
+        """One fused kernel when gate|up is one K-quant weight, else the plain matmul and SwiGLU: the same result either way."""
+        if self.fused is not None:
+            o = x.try_matmul_swiglu(self.fused, stream)
+            if o is not None:
+                return o
+        return self.matmul(x, stream).swiglu(n_ff, stream)

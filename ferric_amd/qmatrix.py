@@ -145,6 +145,29 @@ class Tensor:
         _lib.check(_lib.load().fhip_memcpy_d2h(_vp(out), self.buf.ptr, out.nbytes, _stream_handle(stream)))
         return out
 
+    def cat(self, other, dim, stream=None):
+        """Concatenation of two tensors of the same dtype along `dim` -- lib.rs:201 (the reference's asserts; here for the vectors and
+        matrices this path handles: each side is copied into its rows or columns of the result)."""
+        assert len(self.shape) == len(other.shape), "cat: rank mismatch"
+        assert len(self.shape) in (1, 2) and 0 <= dim < len(self.shape), "cat: vectors and matrices only"
+        for d in range(len(self.shape)):
+            if d != dim:
+                assert self.shape[d] == other.shape[d], f"cat: dim {d} mismatch {list(self.shape)} vs {list(other.shape)}"
+        assert self.dtype == other.dtype, "cat: dtype mismatch"
+        shape = list(self.shape)
+        shape[dim] += other.shape[dim]
+        out = Tensor.empty(shape, self.dtype)
+        lib, sh, it = _lib.load(), _stream_handle(stream), self.dtype.itemsize
+        if dim == 0:
+            na = self.numel() * it
+            _lib.check(lib.fhip_memcpy_d2d(out.buf.ptr, self.buf.ptr, na, sh))
+            _lib.check(lib.fhip_memcpy_d2d(C.c_void_p(out.buf.ptr.value + na), other.buf.ptr, other.numel() * it, sh))
+        else:
+            rows, wa, wb = self.shape[0], self.shape[1] * it, other.shape[1] * it
+            _lib.check(lib.fhip_memcpy_2d_d2d(out.buf.ptr, wa + wb, self.buf.ptr, wa, wa, rows, sh))
+            _lib.check(lib.fhip_memcpy_2d_d2d(C.c_void_p(out.buf.ptr.value + wa), wa + wb, other.buf.ptr, wb, wb, rows, sh))
+        return out
+
     # -- quantized matmuls --------------------------------------------------------------------
     def _rows_inner(self):
         assert len(self.shape) == 2, "matmul_q expects a [rows, in] tensor"
@@ -425,6 +448,19 @@ class QMatrix:
                                  dtype=np.uint8)
         h = C.c_void_p()
         _lib.check(lib.fhip_weight_create(ggml_type, _vp(a), a.size, rows, cols, C.byref(h)))
+        return QMatrix(h, ggml_type)
+
+    @staticmethod
+    def from_parts(parts, ggml_type, rows, cols):
+        """One weight from several byte arrays stacked along the output dim (the fused QKV / gate|up of qwen35.rs:379-402):
+        every part is uploaded to its place, nothing is concatenated on the host. Errors as from_bytes."""
+        lib = _lib.init()
+        arrs = [np.ascontiguousarray(np.frombuffer(p, dtype=np.uint8) if isinstance(p, (bytes, bytearray, memoryview)) else p, dtype=np.uint8)
+                for p in parts]
+        ptrs = (C.c_void_p * len(arrs))(*[a.ctypes.data for a in arrs])
+        sizes = (C.c_size_t * len(arrs))(*[a.size for a in arrs])
+        h = C.c_void_p()
+        _lib.check(lib.fhip_weight_create_parts(ggml_type, ptrs, sizes, len(arrs), rows, cols, C.byref(h)))
         return QMatrix(h, ggml_type)
 
     @staticmethod

@@ -89,6 +89,9 @@ int fhip_free(void* d_ptr);
 int fhip_memcpy_h2d(void* d_dst, const void* h_src, size_t nbytes, void* stream); /* async on stream */
 int fhip_memcpy_d2h(void* h_dst, const void* d_src, size_t nbytes, void* stream); /* synchronises stream before returning */
 int fhip_memcpy_d2d(void* d_dst, const void* d_src, size_t nbytes, void* stream);
+/* `height` rows of `width` bytes between two pitched device arrays, async on stream (what Tensor::cat along the last
+ * dim of a matrix comes to, crates/ferric-tensor/src/lib.rs:201-221: each side is copied into its columns of the result) */
+int fhip_memcpy_2d_d2d(void* d_dst, size_t dpitch, const void* d_src, size_t spitch, size_t width, size_t height, void* stream);
 int fhip_memset(void* d_dst, int byte, size_t nbytes, void* stream);
 int fhip_stream_create(void** stream);
 int fhip_stream_destroy(void* stream);
@@ -120,6 +123,12 @@ int fhip_graph_destroy(void* graph_exec);
  * nbytes != rows*(cols/block_values)*block_bytes -> FHIP_ERR_SHAPE. */
 int fhip_weight_create(uint32_t ggml_type, const uint8_t* h_raw, size_t nbytes, size_t rows, size_t cols,
                        fhip_weight** out);
+
+/* The same from several host buffers laid end to end (the byte stacking of crates/ferric-llama/src/qwen35.rs:393-395
+ * and of Proj::load, crates/ferric-llama/src/qwen3.rs:197-213, without the host-side Vec): part i is uploaded behind
+ * part i - 1; the parts' sizes must add up to rows * row_bytes. */
+int fhip_weight_create_parts(uint32_t ggml_type, const uint8_t* const* h_parts, const size_t* part_bytes, size_t n_parts,
+                             size_t rows, size_t cols, fhip_weight** out);
 
 /* Same, but adopts block bytes that are already in device memory (no copy; the caller keeps the
  * buffer alive until fhip_weight_destroy). Used when a loader streams a file straight into HBM. */
@@ -359,6 +368,13 @@ int fhip_gguf_meta_str(const fhip_gguf* g, const char* key, size_t j, const char
  * tensor's bytes straight from the mapping. dims are [in, out] or, for an expert slab, [in, rows per expert,
  * n_expert] (rows = product of the trailing dims). Types 2 / 3 / 6 / 7 / 8 / 12 / 13 / 14 / 20 / 23 / 39 only. */
 int fhip_weight_from_gguf(const fhip_gguf* g, const char* name, fhip_weight** out);
+
+/* crates/ferric-llama/src/qwen35.rs:379-402 qm_cat(ctx, g, names) (fused QKV, fused gate|up): several tensors of one
+ * format and one input width stacked along the output dim into ONE weight. Each tensor's bytes go from the mapping to
+ * their place in the device allocation; nothing is concatenated on the host. Errors with the reference's messages:
+ * "no tensor 'X'", "X: mixed quant formats in one fused matmul", "X: input dim differs" (FHIP_ERR_FORMAT, the
+ * reference's Err(String)). */
+int fhip_weight_from_gguf_cat(const fhip_gguf* g, const char* const* names, size_t n_names, fhip_weight** out);
 
 /* crates/ferric-tensor/src/cpu_simd.rs:79 matvec_q8_0(x, w, rows, cols) with HOST buffers on both
  * sides (upload, GEMV, download, synchronise) -- the drop-in for the CPU mat-vec call.
