@@ -557,12 +557,13 @@ struct GemvParams {
     uint32_t m_wpr, m_ngf, m_rf;
     fhip::SelParams sel; // expert selection (selw == nullptr: none)
     // Fused input norm (norm_w != nullptr; M = 1, cols <= 8 * threads): the activation row is rmsnorm(x [+ resid]) * norm_w,
-    // formed by every workgroup while it stages the row; workgroup 0 also stores x + resid to x_out (never x itself).
+    // formed by every workgroup while it stages the row; one workgroup also stores x + resid to x_out (never x itself).
     const float* norm_w;
     const float* resid;
     float* x_out;
     float eps;
-    uint32_t red_off;    // byte offset in LDS of 16 floats for the workgroup's sum of squares
+    uint32_t red_off;    // byte offset in LDS of 64 floats: four partial sums of squares per wave
+    int row_wgs;         // workgroups that own rows; the launch may hold one more, which only stores x + resid
 };
 
 // Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 768 -> 168, 512 -> 256).
@@ -590,7 +591,24 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     const int e0 = tid * 8;
     float4 xa0 = {0, 0, 0, 0}, xb0 = {0, 0, 0, 0};
     if (e0 < M * p.cols) { xa0 = *(const float4*)(p.x + e0); xb0 = *(const float4*)(p.x + e0 + 4); }
+    constexpr bool fused_norm = NORM && M == 1;   // a separate instantiation: the plain kernel carries none of this
+    float4 nwa = {1, 1, 1, 1}, nwb = {1, 1, 1, 1}, rsa = {0, 0, 0, 0}, rsb = {0, 0, 0, 0};
+    if (fused_norm && e0 < p.cols) {              // the norm's weights and the residual ride with the activations
+        nwa = *(const float4*)(p.norm_w + e0); nwb = *(const float4*)(p.norm_w + e0 + 4);
+        if (p.resid) { rsa = *(const float4*)(p.resid + e0); rsb = *(const float4*)(p.resid + e0 + 4); }
+    }
     asm volatile("" ::: "memory");   // keeps the loads here
+    if (fused_norm && (int)blockIdx.x >= p.row_wgs) {
+        // A workgroup past the ones that own rows, launched when a CU is free for it: it stores x + resid and is done. Stored
+        // by a workgroup that streams rows, the sum costs that workgroup the store's acknowledgement (1.4 us measured on the
+        // gate|up shape): its later waits for weight rows count the store too.
+        if (p.x_out && e0 < p.cols) {
+            xa0.x += rsa.x; xa0.y += rsa.y; xa0.z += rsa.z; xa0.w += rsa.w;
+            xb0.x += rsb.x; xb0.y += rsb.y; xb0.z += rsb.z; xb0.w += rsb.w;
+            *(float4*)(p.x_out + e0) = xa0; *(float4*)(p.x_out + e0 + 4) = xb0;
+        }
+        return;
+    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NGF = p.NG >> 2, NT = p.NG & 3, NFW = NGF * p.RF, WPR = NFW + (NT ? 1 : 0);
     const int rg = (int)div_magic((uint32_t)wave, p.m_wpr), wr = wave - rg * WPR;   // row group within workgroup, wave within row group
@@ -644,12 +662,6 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     // (Loads return in issue order. Issuing exactly U row loads unconditionally would let the wait for the
     // activations be a counted one instead of a drain, but the dummy loads of waves with fewer than U rows
     // cost more than that saves: measured +40 % on the 4096x4096 Q8_0 GEMV.)
-    constexpr bool fused_norm = NORM && M == 1;   // a separate instantiation: the plain kernel carries none of this
-    float4 nwa = {1, 1, 1, 1}, nwb = {1, 1, 1, 1}, rsa = {0, 0, 0, 0}, rsb = {0, 0, 0, 0};
-    if (fused_norm && e0 < p.cols) {
-        nwa = *(const float4*)(p.norm_w + e0); nwb = *(const float4*)(p.norm_w + e0 + 4);
-        if (p.resid) { rsa = *(const float4*)(p.resid + e0); rsb = *(const float4*)(p.resid + e0 + 4); }
-    }
     typename F::Data buf[U];
 #pragma unroll
     for (int j = 0; j < U; j++)
@@ -657,22 +669,23 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
 
     if (fused_norm) {
         // x <- rmsnorm(x + resid) * norm_w (crates/ferric-tensor/src/lib.rs:2057-2074): each thread holds at most one
-        // 8-value piece of the row (cols <= 8 * threads), so the row's sum of squares is one wave sum + one LDS round.
+        // 8-value piece of the row (cols <= 8 * threads). The row's scale 1 / rms is one number and the mat-vec is linear in
+        // x, so the row is staged as (x + resid) * norm_w, the waves leave their sums of squares in LDS on the way (the
+        // barrier behind the staging publishes them), and the scale meets the finished dot products at the end: no
+        // barrier of its own in front of the staging.
         xa0.x += rsa.x; xa0.y += rsa.y; xa0.z += rsa.z; xa0.w += rsa.w;
         xb0.x += rsb.x; xb0.y += rsb.y; xb0.z += rsb.z; xb0.w += rsb.w;
-        if (p.x_out && blockIdx.x == 0 && e0 < p.cols) { *(float4*)(p.x_out + e0) = xa0; *(float4*)(p.x_out + e0 + 4) = xb0; }
+        // with no CU to spare, the last workgroup that owns rows stores the sum
+        if (p.x_out && (int)gridDim.x == p.row_wgs && (int)blockIdx.x == p.row_wgs - 1 && e0 < p.cols) {
+            *(float4*)(p.x_out + e0) = xa0; *(float4*)(p.x_out + e0 + 4) = xb0;
+        }
         float ss = fmaf(xa0.x, xa0.x, fmaf(xa0.y, xa0.y, fmaf(xa0.z, xa0.z, xa0.w * xa0.w)))
                  + fmaf(xb0.x, xb0.x, fmaf(xb0.y, xb0.y, fmaf(xb0.z, xb0.z, xb0.w * xb0.w)));
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+        ss = slot_sum(ss);                                    // four 16-lane sums per wave, no trip through LDS to combine them
         float* red = (float*)(smem + p.red_off);
-        if (lane == 0) red[wave] = ss;
-        __syncthreads();
-        float tot = 0.f;
-        for (int wv = 0; wv < (int)(blockDim.x >> 6); wv++) tot += red[wv];
-        const float ninv = 1.0f / sqrtf(tot / (float)p.cols + p.eps);
-        xa0.x = xa0.x * ninv * nwa.x; xa0.y = xa0.y * ninv * nwa.y; xa0.z = xa0.z * ninv * nwa.z; xa0.w = xa0.w * ninv * nwa.w;
-        xb0.x = xb0.x * ninv * nwb.x; xb0.y = xb0.y * ninv * nwb.y; xb0.z = xb0.z * ninv * nwb.z; xb0.w = xb0.w * ninv * nwb.w;
+        if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)] = ss;
+        xa0.x *= nwa.x; xa0.y *= nwa.y; xa0.z *= nwa.z; xa0.w *= nwa.w;
+        xb0.x *= nwb.x; xb0.y *= nwb.y; xb0.z *= nwb.z; xb0.w *= nwb.w;
     }
 
     // ---- activations -> 24-bit block fixed point, once per workgroup, through LDS
@@ -728,6 +741,22 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
         if (within == 0) { scales[r] = amax / QMAX; sums[r] = sum; }
     }
     __syncthreads();
+
+    // The row scale the staged activations went without, for the threads that will write outputs: worked out here, under
+    // the wait for the first weight rows, and not behind the last barrier where every cycle is on the critical path.
+    const int per_wg = p.G * p.rpg;
+    float ninv = 1.0f;
+    if (fused_norm && tid < per_wg) {
+        const float4* red = (const float4*)(smem + p.red_off);
+        const int nwaves = (int)(blockDim.x >> 6);
+        float tot = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < 16; wv++) {
+            const float4 r4 = red[wv < nwaves ? wv : 0];
+            tot += wv < nwaves ? (r4.x + r4.y) + (r4.z + r4.w) : 0.f;
+        }
+        ninv = 1.0f / sqrtf(tot / (float)p.cols + p.eps);
+    }
 
     uint32_t xp[M][NRUN][3][RD];
     float xs[M][NRUN], xsum[M][NRUN];
@@ -797,7 +826,6 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
 
     // ---- add the NG slot partials of each output in a fixed order, apply SwiGLU, store.
     // Local row rr = g*rpg + rl is output row blockIdx.x*G*rpg + rr, and its partials start at rr*VPR*NG.
-    const int per_wg = p.G * p.rpg;
     const int row0 = blockIdx.x * per_wg;
 #pragma unroll
     for (int m = 0; m < M; m++)
@@ -807,9 +835,11 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
             const float* q = part + ((size_t)rr * VPR * p.NG) * M + m;
             float a = 0.f;
             for (int s = 0; s < p.NG; s++) a += q[s * M];
+            if (fused_norm) a *= ninv;
             if (SWIGLU) {
                 float b = 0.f;
                 for (int s = 0; s < p.NG; s++) b += q[(p.NG + s) * M];
+                if (fused_norm) b *= ninv;
                 a = (a / (1.0f + expf(-a))) * b;             // silu(gate) * up, crates/ferric-tensor/src/dtype.rs:2408
             }
             p.y[(size_t)m * p.out_rows + r] = a;
@@ -909,9 +939,12 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
         p.norm_w = norm->norm_w; p.resid = norm->resid; p.x_out = norm->x_out; p.eps = norm->eps;
         lds = (lds + 15) & ~(size_t)15;
         p.red_off = (uint32_t)lds;
-        lds += 64;
+        lds += 256;
+        if (lds > fhip::device_lds_bytes()) return fhip::NORM_NOT_FUSED;   // no room left beside the staged row
     }
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid, (unsigned)p.sel.npairs), dim3(64 * WPR * G), lds, s, p);
+    p.row_wgs = (int)grid;
+    const size_t launch_wgs = grid + ((norm && norm->x_out && grid < (size_t)cus) ? 1 : 0);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)launch_wgs, (unsigned)p.sel.npairs), dim3(64 * WPR * G), lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
 }
 
