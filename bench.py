@@ -490,7 +490,7 @@ def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
     x = np.random.default_rng(x_seed).standard_normal(cols).astype(np.float32)
     O.matmul_cpu(x, w, Q4_K, rows, cols, threads=threads)  # warm-up, excluded
     times, t_end = [], time.perf_counter() + budget_s
-    while len(times) < 9 or (time.perf_counter() < t_end and len(times) < 200):
+    while len(times) < 9 or (time.perf_counter() < t_end and len(times) < 1000):
         t0 = time.perf_counter()
         O.matmul_cpu(x, w, Q4_K, rows, cols, threads=threads)
         times.append(time.perf_counter() - t0)
