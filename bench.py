@@ -332,7 +332,7 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
         ms = timer.time_ms(lambda: [dec.step_graph() for _ in range(steps)]) / steps
         logits = dec.logits.to_vec(stream)
         kv_bytes = 2 * (ctx + steps // 2) * nkv * hd * 4 * layers
-        out[str(ctx)] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * 7 + 2,
+        out[str(ctx)] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * dec.launches_per_layer + 2,
                          "kv_bytes_read": kv_bytes, "GBps_weights_plus_kv": (weight_bytes_total + kv_bytes) / (ms * 1e-3) / 1e9,
                          "logits_finite": bool(np.isfinite(logits).all())}
         del dec

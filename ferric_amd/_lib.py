@@ -96,6 +96,8 @@ SYMBOLS = {
                                 _sz, _vp]),
     "fhip_decode_attention_ws_bytes": (_sz, [_sz, _sz, _sz, _sz]),
     "fhip_decode_attention": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
+    "fhip_qkv_post_attention": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_int, C.c_float, C.c_float, _vp, _vp, _sz, _sz, _sz,
+                                          C.c_float, _vp, _vp, _vp]),
     "fhip_decode_attention_ex": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, C.c_float, _vp, _vp, _vp]),
     "fhip_norm_matmul_q": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, C.c_int, _vp, _vp]),
     "fhip_debug_generic_matvec": (C.c_int, [C.c_int]),

@@ -517,6 +517,22 @@ int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float*
     return fhip_decode_attention_ex(d_q, d_k_cache, d_v_cache, n_head, n_kv, head_dim, len, d_last_pos, 0, 0.f, d_ws, d_out, stream);
 }
 
+int fhip_qkv_post_attention(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_pos,
+                            const float* d_freq_scale, size_t n_head, size_t n_kv, size_t head_dim, size_t n_rot, int interleaved, float eps,
+                            float base, float* d_k_cache, float* d_v_cache, size_t cap, size_t len, size_t window, float softcap, float* d_ws,
+                            float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = rope_checks("fhip_qkv_post_attention", n_head + 2 * n_kv, head_dim, n_rot))) return rc;
+    if (n_head == 0 || head_dim == 0) return FHIP_OK;
+    if (!d_qkv || !d_pos || !d_k_cache || !d_v_cache || !d_out) return set_error(FHIP_ERR_ARG, "fhip_qkv_post_attention: NULL pointer");
+    if (cap > 0xFFFFFFFFull) return set_error(FHIP_ERR_SHAPE, "fhip_qkv_post_attention: capacity exceeds 2^32 rows");
+    if (!(softcap >= 0.f)) return set_error(FHIP_ERR_ARG, "fhip_qkv_post_attention: softcap must be >= 0");
+    return fhip::launch_qkv_post_attention(d_qkv, d_bias, d_q_norm, d_k_norm, d_pos, d_freq_scale, (int)n_head, (int)n_kv, (int)head_dim, (int)n_rot,
+                                           interleaved != 0, eps, base, d_k_cache, d_v_cache, cap, len, window, softcap, d_ws, d_out,
+                                           (hipStream_t)stream);
+}
+
 int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_resid, const float* d_norm_w, float eps, float* d_x_out,
                        float* d_h_scratch, int swiglu, float* d_y, void* stream) {
     int rc = need_init();

@@ -246,13 +246,23 @@ __device__ __forceinline__ void load_dims(const float* p, float (&r)[DPL]) {   /
     }
 }
 
-template <int G, int DPL>
-__global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict__ q, const float* __restrict__ K, const float* __restrict__ V,
-                                                         int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
-                                                         uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out) {
+// FUSED: the query heads do not come from memory but are formed here from the raw QKV row of the newest token -- bias, per-head
+// RMSNorm, rotation, exactly qkv_post_kernel's arithmetic -- by every workgroup for its own G heads, into LDS; and the
+// workgroup whose key range holds the token's position also forms that token's K and V rows for its KV head and appends them
+// to the cache before it starts on the keys (a store, a workgroup barrier, then the ordinary loop reads the row back like any
+// other: no other workgroup's range holds that row). One launch less per layer than post-processing + attention.
+template <bool FUSED> struct CachePtr { typedef const float* __restrict__ type; };
+template <> struct CachePtr<true> { typedef const float* type; };   // the fused kernel also writes the cache: no promise of no alias
+
+template <int G, int DPL, bool FUSED>
+__device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typename CachePtr<FUSED>::type K, typename CachePtr<FUSED>::type V,
+                                                int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
+                                                uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out,
+                                                const QkvPostParams& fp) {
     constexpr int HD = 16 * DPL;
     __shared__ float sm_m[4][G], sm_l[4][G];
     __shared__ float sm_acc[4][G][HD];
+    __shared__ float sm_q[FUSED ? G : 1][FUSED ? HD : 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15;
     const int sid = wave * 4 + (lane >> 4);
     const int kvh = blockIdx.x, split = blockIdx.y;
@@ -266,11 +276,52 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
     const float* Kb = K + (size_t)kvh * HD + sub * DPL;
     const float* Vb = V + (size_t)kvh * HD + sub * DPL;
 
+    if constexpr (FUSED) {
+        const uint32_t pos = *len_dev;
+        const bool owner = pos < len && pos >= k0 && pos < k1 && pos < fp.cap;
+        const int njobs = G + (owner ? 2 : 0);
+        const int kvw = n_kv * HD, half = fp.n_rot / 2;
+        for (int j = wave; j < njobs; j += 4) {            // job j < G: query head j of the group; G: the K row; G + 1: the V row
+            const int src = j < G ? kvh * G + j : (j == G ? fp.n_head + kvh : fp.n_head + n_kv + kvh);
+            const float* x = fp.qkv + (size_t)src * HD;
+            const float* bias = fp.bias ? fp.bias + (size_t)src * HD : nullptr;
+            const float* nw = j < G ? fp.q_norm : (j == G ? fp.k_norm : nullptr);
+            float* dst = j < G ? &sm_q[FUSED ? j : 0][0] : (j == G ? fp.k_cache : fp.v_cache) + (size_t)pos * kvw + (size_t)kvh * HD;
+            if (j == G + 1) {
+                for (int e = lane; e < HD; e += 64) dst[e] = bias ? x[e] + bias[e] : x[e];
+                continue;
+            }
+            float inv = 1.f;
+            if (nw) {
+                float ms = 0.f;
+                for (int e = lane; e < HD; e += 64) { float v = bias ? x[e] + bias[e] : x[e]; ms = fmaf(v, v, ms); }
+                ms = wave_sum(ms);
+                inv = 1.0f / sqrtf(ms / (float)HD + fp.eps);
+            }
+            auto val = [&](int e) { float v = bias ? x[e] + bias[e] : x[e]; return nw ? v * inv * nw[e] : v; };
+            for (int c = lane; c < half; c += 64) {
+                const float ang = (float)pos * rope_inv_freq(c, fp.n_rot, fp.base, fp.freq_scale);
+                float sn, cs;
+                sincosf(ang, &sn, &cs);
+                const int p0 = fp.interleaved ? 2 * c : c, p1 = fp.interleaved ? 2 * c + 1 : c + half;
+                const float x1 = val(p0), x2 = val(p1);
+                dst[p0] = x1 * cs - x2 * sn;
+                dst[p1] = x2 * cs + x1 * sn;
+            }
+            for (int e = fp.n_rot + lane; e < HD; e += 64) dst[e] = val(e);
+        }
+        __syncthreads();
+    }
     float qr[G][DPL], acc[G][DPL], m[G], l[G];
 #pragma unroll
     for (int h = 0; h < G; h++) {
         m[h] = -3.0e38f; l[h] = 0.f;
-        load_dims<DPL>(q + ((size_t)kvh * G + h) * HD + sub * DPL, qr[h]);
+        if constexpr (FUSED) {
+#pragma unroll
+            for (int i = 0; i < DPL; i++) qr[h][i] = sm_q[FUSED ? h : 0][sub * DPL + i];
+        } else {
+            load_dims<DPL>(q + ((size_t)kvh * G + h) * HD + sub * DPL, qr[h]);
+        }
 #pragma unroll
         for (int i = 0; i < DPL; i++) acc[h][i] = 0.f;
     }
@@ -352,6 +403,20 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
     }
 }
 
+template <int G, int DPL>
+__global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict__ q, const float* __restrict__ K, const float* __restrict__ V,
+                                                         int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
+                                                         uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out) {
+    attn_split_body<G, DPL, false>(q, K, V, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, QkvPostParams{});
+}
+
+template <int G, int DPL>
+__global__ __launch_bounds__(256) void attn_split_fused_kernel(QkvPostParams fp, int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev,
+                                                               float scale, int splits, uint32_t window, float softcap, float* __restrict__ part,
+                                                               float* __restrict__ out) {
+    attn_split_body<G, DPL, true>(nullptr, fp.k_cache, fp.v_cache, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, fp);
+}
+
 // One workgroup per query head: weights exp(m_s - max m) of the splits once (through LDS), then every output dim is a
 // weighted sum of the splits' accumulators over the weighted sum of their sums. splits <= 256.
 __global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restrict__ part, int hd, int splits, float* __restrict__ out) {
@@ -381,6 +446,17 @@ int launch_attn_g(int hd, dim3 grid, hipStream_t s, const float* q, const float*
     switch (hd) {
         case 64: hipLaunchKernelGGL((attn_split_kernel<G, 4>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
         case 128: hipLaunchKernelGGL((attn_split_kernel<G, 8>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
+    }
+    return FHIP_OK;
+}
+
+template <int G>
+int launch_attn_fused_g(int hd, dim3 grid, hipStream_t s, const QkvPostParams& fp, int n_kv, uint32_t len, const uint32_t* d_len, float scale,
+                        int splits, uint32_t window, float softcap, float* part, float* out) {
+    switch (hd) {
+        case 64: hipLaunchKernelGGL((attn_split_fused_kernel<G, 4>), grid, dim3(256), 0, s, fp, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        case 128: hipLaunchKernelGGL((attn_split_fused_kernel<G, 8>), grid, dim3(256), 0, s, fp, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
         default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     }
     return FHIP_OK;
@@ -495,6 +571,46 @@ int launch_decode_attention(const float* q, const float* K, const float* V, int 
     if (splits > 1) {
         hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(hd), 0, s, ws, hd, splits, out);
         rc = check_hip(hipGetLastError(), "decode_attention combine launch");
+    }
+    return rc;
+}
+
+int launch_qkv_post_attention(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos,
+                              const float* freq_scale, int n_head, int n_kv, int hd, int n_rot, bool interleaved, float eps, float base,
+                              float* k_cache, float* v_cache, size_t cap, size_t len, size_t window, float softcap, float* ws, float* out,
+                              hipStream_t s) {
+    if (n_head == 0 || hd == 0) return FHIP_OK;
+    if (len == 0) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: empty cache");
+    if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: n_heads must be a multiple of n_kv_heads");
+    if (hd != 64 && hd != 128) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: head_dim must be 64 or 128");
+    if (len > 0x7FFFFFFFull || len > cap) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: length outside the cache");
+    const int g = n_head / n_kv, splits = attn_splits(len, n_kv);
+    if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "qkv_post_attention: this cache length needs the workspace");
+    QkvPostParams fp;
+    fp.qkv = qkv; fp.bias = bias; fp.q_norm = q_norm; fp.k_norm = k_norm; fp.pos = d_pos; fp.freq_scale = freq_scale;
+    fp.q_out = nullptr; fp.k_cache = k_cache; fp.v_cache = v_cache;
+    fp.t = 1; fp.n_head = n_head; fp.n_kv = n_kv; fp.hd = hd; fp.n_rot = n_rot; fp.interleaved = interleaved ? 1 : 0;
+    fp.cap = (uint32_t)cap; fp.eps = eps; fp.base = base;
+    const float scale = 1.0f / sqrtf((float)hd);
+    const uint32_t win = window > 0x7FFFFFFFull ? 0u : (uint32_t)window;
+    dim3 grid((unsigned)n_kv, (unsigned)splits);
+    int rc;
+    switch (g) {
+        case 1: rc = launch_attn_fused_g<1>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        case 2: rc = launch_attn_fused_g<2>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        case 3: rc = launch_attn_fused_g<3>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        case 4: rc = launch_attn_fused_g<4>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        case 5: rc = launch_attn_fused_g<5>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        case 6: rc = launch_attn_fused_g<6>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        case 7: rc = launch_attn_fused_g<7>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        case 8: rc = launch_attn_fused_g<8>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
+        default: return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: %d query heads per KV head (1..=8 supported)", g);
+    }
+    if (rc) return rc;
+    if ((rc = check_hip(hipGetLastError(), "qkv_post_attention launch"))) return rc;
+    if (splits > 1) {
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(hd), 0, s, ws, hd, splits, out);
+        rc = check_hip(hipGetLastError(), "qkv_post_attention combine launch");
     }
     return rc;
 }

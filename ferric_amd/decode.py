@@ -138,11 +138,14 @@ class Qwen3Decoder:
         qkv = rmsnorm(x [+ previous FFN output]) Wqkv^T   [norm and residual add formed inside the mat-vec]
         q/k norm + rope + cache append;  attention;  combine of its splits;  o = a Wo^T
         f = swiglu(rmsnorm(x + o) Wgu^T)                  [again inside the mat-vec];  y = f Wdown^T
-    With fuse_norm=False the norms run as their own launches (9 per layer), as the reference issues them.
+    With fuse_norm=False the norms run as their own launches (9 per layer), as the reference issues them. With fuse_attn=True
+    the q/k norm + rope + cache append happen inside the attention launch, 6 launches per layer; the default (None) takes that
+    for caches short enough that the key range is cut into at most 16 splits.
     """
 
-    def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None, fuse_norm=True):
+    def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None, fuse_norm=True, fuse_attn=None):
         self.cfg, self.layers, self.max_len, self.stream, self.fuse_norm = cfg, layers, int(max_len), stream, bool(fuse_norm)
+        self.fuse_attn = fuse_attn
         self.output_norm, self.lm_head = output_norm, lm_head          # final norm + LM head: hidden -> logits in the same step
         assert (output_norm is None) == (lm_head is None), "output_norm and lm_head come together"
         self.logits = Tensor.empty((1, lm_head.rows())) if lm_head is not None else None
@@ -163,6 +166,14 @@ class Qwen3Decoder:
         lib = _lib.load()
         need = lib.fhip_decode_attention_ws_bytes(c.n_head, c.n_head_kv, c.head_dim, self.max_len)
         self.ws = DeviceBuffer(need) if need else None
+        if self.fuse_attn is None:
+            # Every attention workgroup repeats the query post-processing in front of its keys. With few splits of the key range
+            # that is cheaper than a launch (4.92 -> 4.84 ms/token at 128 keys, 3 splits); with 64 splits it costs what the launch
+            # saved (5.33 -> 5.35 at 4096 keys), so long caches keep the two launches.
+            splits = need // (c.n_head * (c.head_dim + 2) * 4) if need else 1
+            self.fuse_attn = splits <= 16
+        self.fuse_attn = bool(self.fuse_attn)
+        self.launches_per_layer = (7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0)
         self._graph = None
 
     # -- state ------------------------------------------------------------------------------------
@@ -203,12 +214,19 @@ class Qwen3Decoder:
         for il, (l, kv) in enumerate(zip(self.layers, self.caches)):
             cur = self._norm_matmul(l.wqkv, cur, alt, self.y if il else None, l.attn_norm, self.qkv, False)
             alt = other(cur)
-            _check(lib.fhip_qkv_post(self.qkv.buf.ptr, l.qkv_bias.buf.ptr if l.qkv_bias is not None else None,
-                                     l.q_norm.buf.ptr if l.q_norm is not None else None, l.k_norm.buf.ptr if l.k_norm is not None else None,
-                                     self.pos.buf.ptr, None, 1, c.n_head, c.n_head_kv, c.head_dim, c.head_dim, int(c.rope_interleaved),
-                                     c.eps, c.rope_base, self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap, s))
-            _check(lib.fhip_decode_attention(self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, c.n_head, c.n_head_kv, c.head_dim, self.max_len,
-                                             self.pos.buf.ptr, self.ws.ptr if self.ws is not None else None, self.att.buf.ptr, s))
+            bias = l.qkv_bias.buf.ptr if l.qkv_bias is not None else None
+            qn = l.q_norm.buf.ptr if l.q_norm is not None else None
+            kn = l.k_norm.buf.ptr if l.k_norm is not None else None
+            ws = self.ws.ptr if self.ws is not None else None
+            if self.fuse_attn:
+                _check(lib.fhip_qkv_post_attention(self.qkv.buf.ptr, bias, qn, kn, self.pos.buf.ptr, None, c.n_head, c.n_head_kv, c.head_dim,
+                                                   c.head_dim, int(c.rope_interleaved), c.eps, c.rope_base, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap,
+                                                   self.max_len, 0, 0.0, ws, self.att.buf.ptr, s))
+            else:
+                _check(lib.fhip_qkv_post(self.qkv.buf.ptr, bias, qn, kn, self.pos.buf.ptr, None, 1, c.n_head, c.n_head_kv, c.head_dim, c.head_dim,
+                                         int(c.rope_interleaved), c.eps, c.rope_base, self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap, s))
+                _check(lib.fhip_decode_attention(self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, c.n_head, c.n_head_kv, c.head_dim, self.max_len,
+                                                 self.pos.buf.ptr, ws, self.att.buf.ptr, s))
             _check(lib.fhip_matmul_q(l.wo.handle, self.att.buf.ptr, 1, self.o.buf.ptr, s))
             cur = self._norm_matmul(l.ffn_gate_up, cur, alt, self.o, l.ffn_norm, self.f, True)
             alt = other(cur)

@@ -273,6 +273,17 @@ int fhip_decode_attention(const float* d_q, const float* d_k_cache, const float*
 int fhip_decode_attention_ex(const float* d_q, const float* d_k_cache, const float* d_v_cache, size_t n_head, size_t n_kv, size_t head_dim,
                              size_t len, const uint32_t* d_last_pos, size_t window, float softcap, float* d_ws, float* d_out, void* stream);
 
+/* fhip_qkv_post and fhip_decode_attention_ex for ONE new token in one launch (crates/ferric-llama/src/qwen3.rs:861-905 followed
+ * by crates/ferric-tensor/src/nn.rs:140-166): every attention workgroup forms its own query heads from the raw QKV row
+ * [(n_head + 2 n_kv) * head_dim] (bias, per-head RMSNorm, rotation at *d_pos), and the workgroup whose keys include position
+ * *d_pos forms and appends that token's K and V rows before it reads them back. Attention is over rows [0, min(*d_pos + 1,
+ * len)) of the caches; `len` (at most cap) is the host-side upper bound that sizes the launch, as in fhip_decode_attention.
+ * d_ws: fhip_decode_attention_ws_bytes(n_head, n_kv, head_dim, len) bytes. Same results as the two calls. */
+int fhip_qkv_post_attention(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_pos,
+                            const float* d_freq_scale, size_t n_head, size_t n_kv, size_t head_dim, size_t n_rot, int interleaved, float eps,
+                            float base, float* d_k_cache, float* d_v_cache, size_t cap, size_t len, size_t window, float softcap, float* d_ws,
+                            float* d_out, void* stream);
+
 /* rmsnorm / add_rmsnorm (lib.rs:346, :372) fused into the mat-vec that consumes it, for ONE activation row:
  *   h = rmsnorm(x [+ resid], norm_w, eps);   y = h W^T   (swiglu != 0: y = silu(gate . h) * (up . h), as fhip_matmul_q_swiglu)
  * and, when d_x_out is given, x_out = x + resid (the next residual; must not alias d_x). The norm is formed while the

@@ -235,6 +235,51 @@ def test_qkv_post_fuses_bias_norm_rope_and_append(F, X, D):
     assert np.array_equal(bits(kc.to_vec()), bits(kc0.reshape(-1))) and np.array_equal(bits(vc.to_vec()), bits(vc0.reshape(-1)))
 
 
+def test_post_processing_inside_the_attention_launch(F, X, D):
+    # fhip_qkv_post_attention against fhip_qkv_post followed by fhip_decode_attention_ex on copies of the same caches: the same
+    # attention output, the same appended K and V rows, nothing else touched; one split and many, windows, softcap, a position
+    # in the middle of a longer cache (keys past it do not count), group sizes 1..5, both head widths
+    rng = np.random.default_rng(31)
+    lib = F._lib.load()
+    cases = [(40, 8, 128, 700, 699, True, False, False, 0, 0.0), (40, 8, 128, 64, 63, True, False, False, 0, 0.0),
+             (4, 2, 64, 300, 120, False, True, False, 0, 0.0), (6, 3, 128, 2100, 2099, True, True, True, 0, 0.0),
+             (8, 8, 64, 90, 89, False, False, False, 0, 0.0), (12, 4, 128, 1500, 1499, True, False, False, 256, 0.0),
+             (10, 2, 128, 513, 512, True, True, False, 0, 30.0), (2, 1, 128, 1, 0, True, False, False, 0, 0.0)]
+    for nh, nkv, hd, cap, pos, use_norm, use_bias, inter, window, softcap in cases:
+        width = (nh + 2 * nkv) * hd
+        qkv = rng.standard_normal(width).astype(np.float32)
+        bias = rng.standard_normal(width).astype(np.float32) if use_bias else None
+        qn = (rng.random(hd) + 0.5).astype(np.float32) if use_norm else None
+        kn = (rng.random(hd) + 0.5).astype(np.float32) if use_norm else None
+        kc0 = (rng.standard_normal((cap, nkv * hd)) * 0.5).astype(np.float32)
+        vc0 = rng.standard_normal((cap, nkv * hd)).astype(np.float32)
+        T = lambda a: F.Tensor.from_vec(a, a.shape) if a is not None else None
+        P = lambda x: x.buf.ptr if x is not None else None
+        qt, bt, qnt, knt, pt = T(qkv.reshape(1, -1)), T(bias), T(qn), T(kn), X._u32_tensor([pos])
+        ws = F.DeviceBuffer(max(256, lib.fhip_decode_attention_ws_bytes(nh, nkv, hd, cap)))
+        # the two calls
+        kc, vc = T(kc0), T(vc0)
+        qo, want = F.Tensor.empty((1, nh * hd)), F.Tensor.empty((1, nh * hd))
+        F._lib.check(lib.fhip_qkv_post(qt.buf.ptr, P(bt), P(qnt), P(knt), pt.buf.ptr, None, 1, nh, nkv, hd, hd, int(inter), 1e-6, 1e6,
+                                       qo.buf.ptr, kc.buf.ptr, vc.buf.ptr, cap, None))
+        F._lib.check(lib.fhip_decode_attention_ex(qo.buf.ptr, kc.buf.ptr, vc.buf.ptr, nh, nkv, hd, cap, pt.buf.ptr, window, softcap, ws.ptr,
+                                                  want.buf.ptr, None))
+        # one call
+        kc2, vc2 = T(kc0), T(vc0)
+        got = F.Tensor.empty((1, nh * hd))
+        F._lib.check(lib.fhip_qkv_post_attention(qt.buf.ptr, P(bt), P(qnt), P(knt), pt.buf.ptr, None, nh, nkv, hd, hd, int(inter), 1e-6, 1e6,
+                                                 kc2.buf.ptr, vc2.buf.ptr, cap, cap, window, softcap, ws.ptr, got.buf.ptr, None))
+        case = (nh, nkv, hd, cap, pos)
+        assert np.array_equal(bits(kc2.to_vec()), bits(kc.to_vec())) and np.array_equal(bits(vc2.to_vec()), bits(vc.to_vec())), case
+        assert close(got.to_vec(), want.to_vec(), 2e-6), case
+    with pytest.raises(AssertionError, match="length outside the cache"):
+        F._lib.check(lib.fhip_qkv_post_attention(qt.buf.ptr, None, None, None, pt.buf.ptr, None, nh, nkv, hd, hd, 0, 1e-6, 1e6, kc2.buf.ptr,
+                                                 vc2.buf.ptr, cap, cap + 1, 0, 0.0, ws.ptr, got.buf.ptr, None))
+    with pytest.raises(F._lib.FerricHipError, match="NULL pointer"):
+        F._lib.check(lib.fhip_qkv_post_attention(None, None, None, None, pt.buf.ptr, None, nh, nkv, hd, hd, 0, 1e-6, 1e6, kc2.buf.ptr,
+                                                 vc2.buf.ptr, cap, cap, 0, 0.0, ws.ptr, got.buf.ptr, None))
+
+
 def test_norm_fused_into_the_matvec(F, X, D, O):
     """fhip_norm_matmul_q against rmsnorm / add_rmsnorm followed by the mat-vec: the residual sum bit-exact, the product
     within the dot-product bound of the unfused pair (the sum of squares is added in another order: ~1e-7 on the scale),
@@ -298,8 +343,8 @@ def _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, qk_norm):
     return layers, olayers
 
 
-@pytest.mark.parametrize("qk_norm,fuse_norm", [(True, True), (False, True), (True, False)])
-def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, X, O, D, qk_norm, fuse_norm):
+@pytest.mark.parametrize("qk_norm,fuse_norm,fuse_attn", [(True, True, True), (False, True, True), (True, False, False), (True, True, False)])
+def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, X, O, D, qk_norm, fuse_norm, fuse_attn):
     rng = np.random.default_rng(4)
     n_layer, d, nh, nkv, hd, n_ff, steps = 3, 1024, 8, 2, 128, 1536, 6
     cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6)
@@ -314,7 +359,7 @@ def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, 
             x = D.apply_layer(x, l, kc, vc, pos, cfg)
         want.append(x)
     stream = F.Stream()
-    dec = X.Qwen3Decoder(cfg, layers, max_len=steps + 2, stream=stream, fuse_norm=fuse_norm)
+    dec = X.Qwen3Decoder(cfg, layers, max_len=steps + 2, stream=stream, fuse_norm=fuse_norm, fuse_attn=fuse_attn)
     eager = []
     for pos in range(steps):
         dec.set_input(xs[pos])
