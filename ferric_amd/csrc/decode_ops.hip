@@ -532,12 +532,15 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
 }
 
 // Splits of the key range: about two workgroups per CU over all KV heads, at least `keys` keys each (FHIP_ATTN_KEYS, default 64:
-// two rounds of the workgroup's 16 streams x 2 keys), at most 256 (the combine kernel's LDS tables).
+// two rounds of the workgroup's 16 streams x 2 keys; 16 for caches of up to 256 rows), at most 256 (the combine kernel's LDS tables).
 int attn_splits(size_t len, int n_kv) {
     if (n_kv <= 0 || len == 0) return 1;
     static const int keys = [] { const char* e = getenv("FHIP_ATTN_KEYS"); int v = e ? atoi(e) : 64; return v < 1 ? 64 : v; }();
     int want = (2 * device_cus() + n_kv - 1) / n_kv;
-    size_t by_keys = (len + keys - 1) / keys;
+    // up to 256 keys a split of 16 (half of the streams, one round) beat one of 64 by 0.1 ms per token of the chained step;
+    // from 512 keys on the larger split count costs more in the combine than it saves
+    const size_t per_split = len <= 256 && keys > 16 ? 16 : (size_t)keys;
+    size_t by_keys = (len + per_split - 1) / per_split;
     int splits = (int)(by_keys < (size_t)want ? by_keys : (size_t)want);
     return splits < 1 ? 1 : (splits > 256 ? 256 : splits);
 }
