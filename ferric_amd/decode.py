@@ -139,8 +139,7 @@ class Qwen3Decoder:
         q/k norm + rope + cache append;  attention;  combine of its splits;  o = a Wo^T
         f = swiglu(rmsnorm(x + o) Wgu^T)                  [again inside the mat-vec];  y = f Wdown^T
     With fuse_norm=False the norms run as their own launches (9 per layer), as the reference issues them. With fuse_attn=True
-    the q/k norm + rope + cache append happen inside the attention launch, 6 launches per layer; the default (None) takes that
-    for caches short enough that the key range is cut into at most 16 splits.
+    (also what None, the default, means) the q/k norm + rope + cache append happen inside the attention launch, 6 launches per layer.
     """
 
     def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None, fuse_norm=True, fuse_attn=None):
@@ -167,11 +166,9 @@ class Qwen3Decoder:
         need = lib.fhip_decode_attention_ws_bytes(c.n_head, c.n_head_kv, c.head_dim, self.max_len)
         self.ws = DeviceBuffer(need) if need else None
         if self.fuse_attn is None:
-            # Every attention workgroup repeats the query post-processing in front of its keys. With few splits of the key range
-            # that is cheaper than a launch (4.92 -> 4.84 ms/token at 128 keys, 3 splits); with 64 splits it costs what the launch
-            # saved (5.33 -> 5.35 at 4096 keys), so long caches keep the two launches.
-            splits = need // (c.n_head * (c.head_dim + 2) * 4) if need else 1
-            self.fuse_attn = splits <= 16
+            # Every attention workgroup repeats the query post-processing in front of its keys; that stays cheaper than a launch
+            # of its own up to 2048 keys (5.12 -> 5.06 ms/token there, 4.92 -> 4.84 at 128) and is level with it from 4096 on.
+            self.fuse_attn = True
         self.fuse_attn = bool(self.fuse_attn)
         self.launches_per_layer = (7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0)
         self._graph = None
