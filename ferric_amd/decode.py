@@ -134,7 +134,7 @@ class Qwen3Layer:
 
 class Qwen3Decoder:
     """One-token decode through a stack of layers with preallocated activations, so that a whole step is a fixed sequence
-    of launches (capturable as one graph). Per layer, 7 launches:
+    of launches (capturable as one graph). Per layer, 7 launches (6 with the second and third in one):
         qkv = rmsnorm(x [+ previous FFN output]) Wqkv^T   [norm and residual add formed inside the mat-vec]
         q/k norm + rope + cache append;  attention;  combine of its splits;  o = a Wo^T
         f = swiglu(rmsnorm(x + o) Wgu^T)                  [again inside the mat-vec];  y = f Wdown^T
