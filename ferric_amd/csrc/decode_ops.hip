@@ -278,7 +278,9 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
 
     if constexpr (FUSED) {
         const uint32_t pos = *len_dev;
-        const bool owner = pos < len && pos >= k0 && pos < k1 && pos < fp.cap;
+        // the rows are appended by the workgroup whose keys include them; a position past the rows attention looks at (but
+        // inside the cache) is still appended, by the last split, as the separate post-processing launch would
+        const bool owner = pos < fp.cap && (pos < len ? (pos >= k0 && pos < k1) : split == splits - 1);
         const int njobs = G + (owner ? 2 : 0);
         const int kvw = n_kv * HD, half = fp.n_rot / 2;
         for (int j = wave; j < njobs; j += 4) {            // job j < G: query head j of the group; G: the K row; G + 1: the V row

@@ -272,6 +272,24 @@ def test_post_processing_inside_the_attention_launch(F, X, D):
         case = (nh, nkv, hd, cap, pos)
         assert np.array_equal(bits(kc2.to_vec()), bits(kc.to_vec())) and np.array_equal(bits(vc2.to_vec()), bits(vc.to_vec())), case
         assert close(got.to_vec(), want.to_vec(), 2e-6), case
+    # a position past the rows attention may look at (len 200 of a cache of 300 rows, position 250): the rows are still appended
+    nh, nkv, hd, cap, alen, pos = 8, 2, 128, 300, 200, 250
+    width = (nh + 2 * nkv) * hd
+    qkv = rng.standard_normal(width).astype(np.float32)
+    kc0 = (rng.standard_normal((cap, nkv * hd)) * 0.5).astype(np.float32)
+    vc0 = rng.standard_normal((cap, nkv * hd)).astype(np.float32)
+    qt, pt = T(qkv.reshape(1, -1)), X._u32_tensor([pos])
+    ws = F.DeviceBuffer(max(256, lib.fhip_decode_attention_ws_bytes(nh, nkv, hd, alen)))
+    kc, vc, kc2, vc2 = T(kc0), T(vc0), T(kc0), T(vc0)
+    qo, want, got = F.Tensor.empty((1, nh * hd)), F.Tensor.empty((1, nh * hd)), F.Tensor.empty((1, nh * hd))
+    F._lib.check(lib.fhip_qkv_post(qt.buf.ptr, None, None, None, pt.buf.ptr, None, 1, nh, nkv, hd, hd, 0, 1e-6, 1e6, qo.buf.ptr, kc.buf.ptr,
+                                   vc.buf.ptr, cap, None))
+    F._lib.check(lib.fhip_decode_attention_ex(qo.buf.ptr, kc.buf.ptr, vc.buf.ptr, nh, nkv, hd, alen, pt.buf.ptr, 0, 0.0, ws.ptr, want.buf.ptr, None))
+    F._lib.check(lib.fhip_qkv_post_attention(qt.buf.ptr, None, None, None, pt.buf.ptr, None, nh, nkv, hd, hd, 0, 1e-6, 1e6, kc2.buf.ptr,
+                                             vc2.buf.ptr, cap, alen, 0, 0.0, ws.ptr, got.buf.ptr, None))
+    assert np.array_equal(bits(kc2.to_vec()), bits(kc.to_vec())) and np.array_equal(bits(vc2.to_vec()), bits(vc.to_vec()))
+    assert not np.array_equal(bits(kc2.to_vec().reshape(cap, -1)[pos]), bits(kc0[pos]))
+    assert close(got.to_vec(), want.to_vec(), 2e-6)
     with pytest.raises(AssertionError, match="length outside the cache"):
         F._lib.check(lib.fhip_qkv_post_attention(qt.buf.ptr, None, None, None, pt.buf.ptr, None, nh, nkv, hd, hd, 0, 1e-6, 1e6, kc2.buf.ptr,
                                                  vc2.buf.ptr, cap, cap + 1, 0, 0.0, ws.ptr, got.buf.ptr, None))
