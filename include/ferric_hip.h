@@ -397,7 +397,9 @@ int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, si
  * the thread creation of every call; what a host-buffer call pays here is the upload of the weight, so the pool keeps
  * the bytes of the last `h_w` it was given resident in HBM (with its staging buffers and a stream of its own) and a
  * call with the same (h_w, w_len, cols) uploads the activations only. `w` is an immutable Arc<Vec<u8>> in the
- * reference; a caller that rewrites the bytes in place calls fhip_pool_forget first. h_y receives hi - lo values.
+ * reference; a caller that rewrites the bytes in place, or frees them (another buffer may then appear at the same address),
+ * calls fhip_pool_forget first -- a binding keeps a clone of the Arc beside the pool for as long as it is the key.
+ * h_y receives hi - lo values.
  * `threads` is kept for Pool::threads() (at least 1) and partitions nothing here. lo > hi, a span past the rows in
  * h_w or fewer than cols activations: FHIP_ERR_SHAPE (the reference's assert and slice panics). One call at a time
  * per pool (the reference serialises Pool::run behind a mutex). */
