@@ -101,6 +101,7 @@ SYMBOLS = {
     "fhip_decode_attention_ex": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, C.c_float, _vp, _vp, _vp]),
     "fhip_norm_matmul_q": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, C.c_int, _vp, _vp]),
     "fhip_debug_generic_matvec": (C.c_int, [C.c_int]),
+    "fhip_matvec_precision": (C.c_int, [C.c_int]),
     "fhip_u32_add": (C.c_int, [_vp, _sz, _u32, _vp]),
     "fhip_matvec_q8_0_host": (C.c_int, [_vp, _vp, _sz, _sz, _sz, _vp]),
     "fhip_pool_create": (C.c_int, [_sz, _vp]),

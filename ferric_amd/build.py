@@ -21,7 +21,8 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-
 UNITS = {
     "api.hip": [],
     "dequant.hip": ["-ffp-contract=off"],
-    "gemv.hip": [],
+    "gemv.hip": ["-DFHIP_GEMV_PLANES=2"],
+    "gemv.hip@p3": ["-DFHIP_GEMV_PLANES=3"],   # the same source again: the 24-bit-activation copy of the streaming mat-vec
     "gemv_generic.hip": [],
     "gemm_mfma.hip": [],
     "gemm_f16x2.hip": [],
@@ -32,8 +33,8 @@ UNITS = {
 
 
 def _compile(name, flags, objdir, verbose):
-    src = os.path.join(CSRC, name)
-    obj = os.path.join(objdir, name + ".o")
+    src = os.path.join(CSRC, name.split("@")[0])
+    obj = os.path.join(objdir, name.replace("@", "_") + ".o")
     cmd = [HIPCC] + COMMON + flags + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # hipcc's host pass does not know the device-only feature flag; that warning is noise.
@@ -48,7 +49,7 @@ def _compile(name, flags, objdir, verbose):
 def build(verbose=False):
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=6) as ex:
         objs = list(ex.map(lambda kv: _compile(kv[0], kv[1], objdir, verbose), UNITS.items()))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -85,6 +85,23 @@ int check_hip(hipError_t e, const char* what) {
 int device_cus() { return g_cus; }
 size_t device_lds_bytes() { return g_lds; }
 
+// The streaming mat-vec exists in two copies, one per activation precision; these forward to the selected one.
+static int g_planes = 2;
+int matvec_planes() { return g_planes; }
+int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s) {
+    return g_planes == 3 ? launch_gemv_p3(w, d_x, rows_x, d_y, n_ff, s) : launch_gemv_p2(w, d_x, rows_x, d_y, n_ff, s);
+}
+int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s) {
+    return g_planes == 3 ? launch_gemv_norm_p3(w, d_x, d_y, n_ff, norm, s) : launch_gemv_norm_p2(w, d_x, d_y, n_ff, norm, s);
+}
+int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel, hipStream_t s) {
+    return g_planes == 3 ? launch_gemv_sel_p3(w, d_x, d_y, out_rows, swiglu, sel, s) : launch_gemv_sel_p2(w, d_x, d_y, out_rows, swiglu, sel, s);
+}
+void gemv_force_generic(bool on) {
+    gemv_force_generic_p2(on);
+    gemv_force_generic_p3(on);
+}
+
 }  // namespace fhip
 
 using fhip::check_hip;
@@ -554,6 +571,14 @@ int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_re
 int fhip_debug_generic_matvec(int on) {
     fhip::gemv_force_generic(on != 0);
     return FHIP_OK;
+}
+
+int fhip_matvec_precision(int bits) {
+    const int before = fhip::g_planes == 3 ? 24 : 16;
+    if (bits == 0) return before;
+    if (bits != 16 && bits != 24) return set_error(FHIP_ERR_ARG, "fhip_matvec_precision: 16 or 24 bits (0 to query), not %d", bits);
+    fhip::g_planes = bits == 24 ? 3 : 2;
+    return before;
 }
 
 int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream) {

@@ -69,6 +69,20 @@ int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d
 // y[rows_x, out_rows] = x * W^T; when n_ff > 0 the weight stacks gate|up (2*n_ff rows) and
 // y[rows_x, n_ff] = silu(gate.x) * (up.x).
 int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
+// gemv.hip is built once per activation precision (two or three byte planes per run: a 16- or 24-bit significand at the run
+// maximum); launch_gemv, launch_gemv_norm, launch_gemv_sel and gemv_force_generic (api.hip) forward to the copy
+// matvec_planes() names.
+int matvec_planes();
+#define FHIP_GEMV_COPY(sfx)                                                                                                         \
+    int launch_gemv##sfx(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);            \
+    int launch_gemv_norm##sfx(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const struct NormParams& norm,        \
+                              hipStream_t s);                                                                                       \
+    int launch_gemv_sel##sfx(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu,                      \
+                             const struct SelParams& sel, hipStream_t s);                                                           \
+    void gemv_force_generic##sfx(bool on);
+FHIP_GEMV_COPY(_p2)
+FHIP_GEMV_COPY(_p3)
+#undef FHIP_GEMV_COPY
 // gemv_generic.hip: same contract, any cols the format allows (up to 32768)
 int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s);

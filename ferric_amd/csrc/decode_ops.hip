@@ -420,21 +420,23 @@ __global__ __launch_bounds__(256) void attn_split_fused_kernel(QkvPostParams fp,
 }
 
 // One workgroup per query head: weights exp(m_s - max m) of the splits once (through LDS), then every output dim is a
-// weighted sum of the splits' accumulators over the weighted sum of their sums. splits <= 256.
-__global__ __launch_bounds__(128) void attn_combine_kernel(const float* __restrict__ part, int hd, int splits, float* __restrict__ out) {
+// weighted sum of the splits' accumulators over the weighted sum of their sums. splits <= 256. Always launched with
+// COMBINE_THREADS threads, whatever the head size: the loops below stride by that constant.
+constexpr int COMBINE_THREADS = 128;
+__global__ __launch_bounds__(COMBINE_THREADS) void attn_combine_kernel(const float* __restrict__ part, int hd, int splits, float* __restrict__ out) {
     __shared__ float w[256], lw[256];
     const int head = blockIdx.x, tid = threadIdx.x;
     const float* pp = part + (size_t)head * splits * (hd + 2);
-    for (int s = tid; s < splits; s += 128) { w[s] = pp[(size_t)s * (hd + 2) + hd]; lw[s] = pp[(size_t)s * (hd + 2) + hd + 1]; }
+    for (int s = tid; s < splits; s += COMBINE_THREADS) { w[s] = pp[(size_t)s * (hd + 2) + hd]; lw[s] = pp[(size_t)s * (hd + 2) + hd + 1]; }
     __syncthreads();
     float M = -3.0e38f;
     for (int s = 0; s < splits; s++) M = fmaxf(M, w[s]);
     __syncthreads();
-    for (int s = tid; s < splits; s += 128) { const float f = __expf(w[s] - M); w[s] = f; lw[s] *= f; }
+    for (int s = tid; s < splits; s += COMBINE_THREADS) { const float f = __expf(w[s] - M); w[s] = f; lw[s] *= f; }
     __syncthreads();
     float L = 0.f;
     for (int s = 0; s < splits; s++) L += lw[s];
-    for (int d = tid; d < hd; d += 128) {
+    for (int d = tid; d < hd; d += COMBINE_THREADS) {
         float A = 0.f;
 #pragma unroll 8
         for (int s = 0; s < splits; s++) A = fmaf(pp[(size_t)s * (hd + 2) + d], w[s], A);
@@ -533,15 +535,15 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
     return check_hip(hipGetLastError(), "kv_append launch");
 }
 
-// Splits of the key range: about two workgroups per CU over all KV heads, at least `keys` keys each (FHIP_ATTN_KEYS, default 64:
-// two rounds of the workgroup's 16 streams x 2 keys; 16 for caches of up to 256 rows), at most 256 (the combine kernel's LDS tables).
+// Splits of the key range: about two workgroups per CU over all KV heads, at least 64 keys each (two rounds of the
+// workgroup's 16 streams x 2 keys; 16 for caches of up to 256 rows), at most 256 (the combine kernel's LDS tables).
 int attn_splits(size_t len, int n_kv) {
     if (n_kv <= 0 || len == 0) return 1;
-    static const int keys = [] { const char* e = getenv("FHIP_ATTN_KEYS"); int v = e ? atoi(e) : 64; return v < 1 ? 64 : v; }();
+    constexpr int keys = 64;
     int want = (2 * device_cus() + n_kv - 1) / n_kv;
     // up to 256 keys a split of 16 (half of the streams, one round) beat one of 64 by 0.1 ms per token of the chained step;
     // from 512 keys on the larger split count costs more in the combine than it saves
-    const size_t per_split = len <= 256 && keys > 16 ? 16 : (size_t)keys;
+    const size_t per_split = len <= 256 ? 16 : (size_t)keys;
     size_t by_keys = (len + per_split - 1) / per_split;
     int splits = (int)(by_keys < (size_t)want ? by_keys : (size_t)want);
     return splits < 1 ? 1 : (splits > 256 ? 256 : splits);
@@ -574,7 +576,7 @@ int launch_decode_attention(const float* q, const float* K, const float* V, int 
     if (rc) return rc;
     if ((rc = check_hip(hipGetLastError(), "decode_attention launch"))) return rc;
     if (splits > 1) {
-        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(hd), 0, s, ws, hd, splits, out);
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(COMBINE_THREADS), 0, s, ws, hd, splits, out);
         rc = check_hip(hipGetLastError(), "decode_attention combine launch");
     }
     return rc;
@@ -614,7 +616,7 @@ int launch_qkv_post_attention(const float* qkv, const float* bias, const float* 
     if (rc) return rc;
     if ((rc = check_hip(hipGetLastError(), "qkv_post_attention launch"))) return rc;
     if (splits > 1) {
-        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(hd), 0, s, ws, hd, splits, out);
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(COMBINE_THREADS), 0, s, ws, hd, splits, out);
         rc = check_hip(hipGetLastError(), "qkv_post_attention combine launch");
     }
     return rc;

@@ -616,7 +616,6 @@ int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_
     long long per = (p.units + wgs - 1) / wgs;
     if (per * 4 >= (long long)p.nchunks * 3 && per < p.nchunks) per = p.nchunks;   // nearly whole groups: make them whole
     if (per < 1) per = 1;
-    if (const char* e = getenv("FHIP_SKINNY_PER")) per = atoi(e) > 0 ? atoi(e) : per;
     p.per = (int)per;
     const unsigned grid = (unsigned)((p.units + per - 1) / per);
     if (per % p.nchunks != 0 && !y_cleared) {

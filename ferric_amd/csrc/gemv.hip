@@ -8,32 +8,65 @@
 // as further per-format structs.
 //
 // Why it looks the way it does. At 8 TB/s a CU gets ~13 weight bytes per clock, i.e. ~23 Q4_K weights,
-// while it can issue 64 lane-instructions per clock: under 3 instructions per weight all-in. A plain
-// "unpack nibble, convert, f32 multiply-add" loop costs ~4.7, so it is instruction-bound at about a
-// third of the memory roofline. This kernel gets below 2 by
-//   * holding the activations as 24-bit block fixed point (three signed byte planes per run of 32 or
-//     16 columns, one f32 scale per run: the same significand width as f32 at the run maximum) and
-//     doing the inner products with v_dot4_i32_i8 -- four weights per instruction and plane, exact
-//     integer sums, converted once per sub-block and from there on accumulated in f32;
+// while it can issue 64 lane-instructions per clock: under 3 instructions per weight all-in, and in
+// practice far fewer, because a wave that spends its cycles issuing cannot keep loads in flight. A plain
+// "unpack nibble, convert, f32 multiply-add" loop costs ~4.7. This kernel gets to ~1.4 by
+//   * holding the activations as block fixed point: per run of 32 or 16 columns (the format's own
+//     sub-block) NP signed byte planes ("balanced digits", each in [-128, 127]) and one f32 scale, so
+//     the inner products are v_dot4_i32_i8 -- four weights per instruction and plane, exact integer
+//     sums, converted to f32 once per sub-block and from there on accumulated in f32. NP = 2 is a
+//     16-bit significand at the run maximum (dot products to ~2e-5 of ||w|| ||x|| / sqrt(K)), NP = 3
+//     a 24-bit one (the f32 significand);
+//   * taking a Q4_K byte's high nibble where it stands: (w ^ 0x80808080) & 0xF0F0F0F0 is one
+//     v_bitop3 and reads, as a signed byte, 16 * (nibble - 8); the 16 goes into the sub-block scale and
+//     the 8 into the term that already multiplies the run's sum of activations;
 //   * giving a lane 64 weights that share one scale header (two nibble chunks of one Q4_K group, one
 //     ql/ql/qh triple of a Q6_K half), so the 6-bit scale decode is paid once per 64 weights;
 //   * keeping the lane -> column mapping fixed for the life of a wave, so the activation planes sit in
-//     registers (quantised once per workgroup through LDS) and are never re-read.
+//     registers (quantised once per workgroup through LDS) and are never re-read;
+//   * reducing the rows of a pipeline step together: U rows' lane partials go through one transposing
+//     butterfly (11 DPP/select operations for 4 rows instead of 16) and leave in one LDS store.
 //
-// Tiling. 16 lanes ("slot") cover 16 units = 1024 weights (512 for Q8_0) of one row; a row is NG slots.
-// Waves 0..NG/4-1 of a row group take 4 consecutive slots of the same row; the NG%4 left-over slots
-// go to one tail wave that works on 4 (or 2) rows at once, so no lane idles for K = 5120 or 17408.
-// Each slot reduces its 16 lanes with DPP and parks one float per row in LDS; after one barrier the
-// NG partials of a row are added in a fixed order (results do not depend on scheduling or on how rows
-// are partitioned over workgroups). Row groups walk contiguous row spans with U rows of 16-byte
-// loads in flight per wave; weight loads for the first rows are issued before the activations are
-// touched, so the two latencies overlap.
+// Tiling. 16 lanes ("slot") cover 16 units = 1024 weights (512 for the 32-value formats) of one row; a row
+// is NG slots. Waves 0..NG/4-1 of a row group take 4 consecutive slots of the same row; the NG%4 left-over
+// slots go to one tail wave that works on 4 (or 2) rows at once, so no lane idles for K = 5120 or 17408.
+// After one barrier the NG partials of a row are added in a fixed order (results do not depend on
+// scheduling or on how rows are partitioned over workgroups). Row groups walk contiguous row spans with U
+// rows of 16-byte loads in flight per wave; weight loads for the first rows are issued before the
+// activations are touched, so the two latencies overlap.
+//
+// Activations that block fixed point cannot hold (a run with a NaN or an infinity, a run whose sum overflows,
+// a run whose largest magnitude is below 2^-100) are marked by a NaN run scale; a lane that owns such a run
+// computes its share of every row element by element in f32 from the raw activations and the exactly
+// dequantised weights, which is what the reference's CPU path does (crates/ferric-tensor/src/cpu_simd.rs:57-72,
+// crates/ferric-gguf/src/lib.rs:497 then a dense dot): NaN stays NaN, inf * w is +-inf, inf * 0 is NaN.
 #include "common.hpp"
+#include "deq_at.hpp"
 
 #include <hip/hip_fp16.h>
-#include <stdlib.h>
+
+#include <type_traits>
+
+// This file is compiled twice, once per activation precision (FHIP_GEMV_PLANES = 2 and 3); the two copies export their
+// launchers under different names and fhip_matvec_precision() picks between them at run time.
+#ifndef FHIP_GEMV_PLANES
+#define FHIP_GEMV_PLANES 2
+#endif
+#if FHIP_GEMV_PLANES == 2
+#define GEMV_EXPORT(name) name##_p2
+#else
+#define GEMV_EXPORT(name) name##_p3
+#endif
 
 namespace {
+
+constexpr int NP = FHIP_GEMV_PLANES;   // byte planes per activation run
+static_assert(NP == 2 || NP == 3, "two or three activation planes");
+// Largest quantised magnitude: every digit at 127; the run's largest activation maps onto it. With two planes the rounding
+// of the reciprocal and of the product moves that by at most 0.02, never to the next integer; with three (8.4e6 * 2^-22 = 2)
+// the quantiser clamps.
+constexpr float QMAX = NP == 2 ? 32639.0f : 8355711.0f;
+constexpr float TINY_RUN = 7.888609052210118e-31f;   // 2^-100: below this QMAX / amax leaves the f32 range's comfortable part
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -44,13 +77,6 @@ __device__ __forceinline__ float f16_bits(uint32_t b) { return __half2float(__us
 __device__ __forceinline__ float ub(uint32_t v, int k) { return (float)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ float sb(uint32_t v, int k) { return (float)(int8_t)((v >> (8 * k)) & 0xFFu); }
 __device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
-__device__ __forceinline__ int udot4(uint32_t a, uint32_t b, int c) { return (int)__builtin_amdgcn_udot4(a, b, (uint32_t)c, false); }
-// Plane p of a run times 4 weight bytes. Plane 0 holds signed digits. Planes 1 and 2 hold unsigned bytes
-// when the weights are non-negative codes (K-quants) and signed balanced digits when they are int8 (Q8_0).
-template <bool SIGNED_W>
-__device__ __forceinline__ int pdot(int p, uint32_t x, uint32_t w, int acc) {
-    return (SIGNED_W || p == 0) ? dot4(x, w, acc) : udot4(x, w, acc);
-}
 
 // Keeps a prefetched row as the packed dwords that were loaded (otherwise the optimizer unpacks
 // bytes as soon as a load returns and carries the unpacked values across the pipeline, which spills).
@@ -62,36 +88,72 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140;   // quad_perm [1,0,3,2], [2,3,0,1]; row_*
+constexpr int DPP_ROR4 = 0x124, DPP_ROR8 = 0x128;   // rotate within the 16-lane row: lane l reads lane l - 4 / l - 8, so l & 3 is kept
 // All-reduce over the 16 lanes of a DPP row.
 __device__ __forceinline__ float slot_sum(float v) {
-    v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
-    v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
-    v += dpp_f<0x141>(v);  // row_half_mirror
-    v += dpp_f<0x140>(v);  // row_mirror
+    v += dpp_f<DPP_XOR1>(v);
+    v += dpp_f<DPP_XOR2>(v);
+    v += dpp_f<DPP_HALF_MIRROR>(v);
+    v += dpp_f<DPP_MIRROR>(v);
     return v;
 }
 
-// A 24-bit fixed-point value v = a*65536 + b*256 + c as three byte planes, in one of two digit systems:
-//   unsigned low digits: a = v >> 16 (signed), b, c = the low bytes of v, |v| <= 2^23 - 1   (weights >= 0)
-//   balanced digits:     a, b, c in [-127, 127], |v| <= 127*65536 + 127*256 + 127             (int8 weights)
-constexpr float QMAX_U = 8388607.0f, QMAX_S = 8355711.0f;
+// Sums U (<= 4) values over the 16 lanes of a DPP row at once. Afterwards lane l of the row holds the row sum of value
+// slot_of(l & 3), with slot_of = {0, 2, 1, 3}: each of the first two butterfly steps halves the number of values a lane
+// carries instead of repeating the whole sum for every value.
+template <int U>
+__device__ __forceinline__ float slot_sum_many(const float (&v)[U], bool bit0, bool bit1) {
+    static_assert(U >= 1 && U <= 4, "one to four values");
+    if constexpr (U == 1) return slot_sum(v[0]);
+    float a, b;
+    if constexpr (U == 2) {
+        a = v[0] + dpp_f<DPP_XOR1>(v[0]);
+        b = v[1] + dpp_f<DPP_XOR1>(v[1]);
+    } else {
+        const float v3 = U == 4 ? v[U - 1] : 0.f;
+        const float keep_a = bit0 ? v[2] : v[0], send_a = bit0 ? v[0] : v[2];
+        const float keep_b = bit0 ? v3 : v[1], send_b = bit0 ? v[1] : v3;
+        a = keep_a + dpp_f<DPP_XOR1>(send_a);
+        b = keep_b + dpp_f<DPP_XOR1>(send_b);
+    }
+    const float keep = bit1 ? b : a, send = bit1 ? a : b;
+    float r = keep + dpp_f<DPP_XOR2>(send);   // the quad's sum of this lane's value
+    r += dpp_f<DPP_ROR4>(r);                  // the four quads of the row (the mirrors would pair lanes that hold different values)
+    r += dpp_f<DPP_ROR8>(r);
+    return r;
+}
+// value index held by lane l (l & 3) after slot_sum_many<U>
+template <int U>
+__device__ __forceinline__ int slot_of(int l) {
+    if constexpr (U == 1) return 0;
+    if constexpr (U == 2) return (l >> 1) & 1;
+    return ((l & 1) << 1) | ((l >> 1) & 1);
+}
 
-// exact integer plane sums -> f32 (the only rounding is the final add, 2^-24 relative)
-__device__ __forceinline__ float planes_to_f32(int a, int b, int c) { return fmaf((float)a, 65536.0f, (float)((b << 8) + c)); }
+// exact integer plane sums -> f32 (one rounding, at most 2^-24 relative)
+__device__ __forceinline__ float planes_f32(const int (&a)[NP]) {
+    if constexpr (NP == 2) return (float)((a[0] << 8) + a[1]);
+    else return fmaf((float)a[0], 65536.0f, (float)((a[1] << 8) + a[NP - 1]));
+}
 
 // ------------------------------------------------------------------------------------------------
 // Per-format lane work. A unit is WPL weights of one row; RUN is the activation run that shares one
-// fixed-point scale (the format's own sub-block length); a lane needs NRUN runs.
+// fixed-point scale (the format's own sub-block length); a lane needs NRUN runs, and run j of the lane is
+// columns [run[j] * RUN, run[j] * RUN + RUN) of the row.
 //   setup(u)  -> byte offsets of unit u inside a row and the indices of its activation runs
 //   load      -> the raw bytes of the unit for one row (16-/8-byte loads, 2-byte aligned where the
 //                GGUF layout is)
 //   dot<M>    -> the lane's share of the M dot products
-// xp[m][j][p][i]: plane p, dword i of run j;  xs[m][j]: scale of run j;  xsum[m][j]: sum of x over run j.
+// xp[m][j][p][i]: plane p (most significant first), dword i of run j;  xs[m][j]: scale of run j;
+// xq[m][j]: scale * (sum of the run's quantised activations), i.e. the sum of x over the run as the planes hold it.
 // ------------------------------------------------------------------------------------------------
 
 struct Q4K {
-    static constexpr int WPL = 64, RUN = 32, NRUN = 2, BLOCK_VALUES = 256, U1 = 3;
-    static constexpr bool SIGNED_W = false;
+    static constexpr uint32_t TYPE = FHIP_Q4_K;
+    static constexpr int WPL = 64, RUN = 32, NRUN = 2, U1 = NP == 2 ? 4 : 3;
     struct Lane { uint32_t off_h, off_q, sh, m1, m2, m3; };
     struct Data {
         u32x4 h, q0, q1;
@@ -110,6 +172,8 @@ struct Q4K {
         run[0] = 2 * u;                        // low nibbles  -> sub-block 2g   = columns [64u, 64u+32)
         run[1] = 2 * u + 1;                    // high nibbles -> sub-block 2g+1 = columns [64u+32, 64u+64)
     }
+    // the unit that uses run r of a row, and which of that unit's runs it is (the inverse of `run` above)
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r >> 1; j = r & 1; }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
         d.h = *(const u32x4*)(row + (L.off_h + eo));
@@ -118,46 +182,48 @@ struct Q4K {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
-                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][NP][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xq)[M][NRUN], float (&out)[M]) {
         // 6-bit (scale, min) of sub-blocks 2g and 2g+1, two packed bytes each
         uint32_t a = D.h[1] >> L.sh, b = D.h[2] >> L.sh, c = D.h[3] >> L.sh;
         uint32_t scp = (a & L.m1) | (c & L.m2) | ((a >> 2) & L.m3);
         uint32_t mp = (b & L.m1) | ((c >> 4) & L.m2) | ((b >> 2) & L.m3);
-        float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
-        float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1), m0 = dmin * ub(mp, 0), m1 = dmin * ub(mp, 1);
-        int acc[M][2][3];
+        const float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
+        const float s0 = ub(scp, 0), s1 = ub(scp, 1), n0 = ub(mp, 0), n1 = ub(mp, 1);
+        int acc[M][2][NP];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) acc[m][j][p] = 0;
+                for (int p = 0; p < NP; p++) acc[m][j][p] = 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            uint32_t w = i < 4 ? D.q0[i] : D.q1[i - 4];
-            uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+            const uint32_t w = i < 4 ? D.q0[i] : D.q1[i - 4];
+            const uint32_t lo = w & 0x0F0F0F0Fu;
+            const uint32_t hi = (w ^ 0x80808080u) & 0xF0F0F0F0u;   // as signed bytes: 16 * (high nibble - 8)
 #pragma unroll
             for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) {
-                    acc[m][0][p] = pdot<false>(p, xp[m][0][p][i], lo, acc[m][0][p]);
-                    acc[m][1][p] = pdot<false>(p, xp[m][1][p][i], hi, acc[m][1][p]);
+                for (int p = 0; p < NP; p++) {
+                    acc[m][0][p] = dot4(xp[m][0][p][i], lo, acc[m][0][p]);
+                    acc[m][1][p] = dot4(xp[m][1][p][i], hi, acc[m][1][p]);
                 }
         }
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            float f0 = xs[m][0] * planes_to_f32(acc[m][0][0], acc[m][0][1], acc[m][0][2]);
-            float f1 = xs[m][1] * planes_to_f32(acc[m][1][0], acc[m][1][1], acc[m][1][2]);
-            // sum_l x_l (d*sc*q_l - dmin*m) = d*sc * sum x_l q_l - dmin*m * sum x_l
-            out[m] = (d0 * f0 - m0 * xsum[m][0]) + (d1 * f1 - m1 * xsum[m][1]);
+            const float f0 = xs[m][0] * planes_f32(acc[m][0]);
+            // sum x * nibble = (sum x * 16 (nibble - 8)) / 16 + 8 sum x
+            const float f1 = fmaf(xs[m][1] * 0.0625f, planes_f32(acc[m][1]), 8.0f * xq[m][1]);
+            // sum_l x_l (d*sc*q_l - dmin*m) = d * (sc0 f0 + sc1 f1) - dmin * (m0 sum0 + m1 sum1)
+            out[m] = d * fmaf(s1, f1, s0 * f0) - dmin * fmaf(n1, xq[m][1], n0 * xq[m][0]);
         }
     }
 };
 
 struct Q6K {
-    static constexpr int WPL = 64, RUN = 16, NRUN = 4, BLOCK_VALUES = 256, U1 = 2;
-    static constexpr bool SIGNED_W = false;
+    static constexpr uint32_t TYPE = FHIP_Q6_K;
+    static constexpr int WPL = 64, RUN = 16, NRUN = 4, U1 = NP == 2 ? 3 : 2;
     struct Lane { uint32_t off_a, off_h, off_s, off_d, ssh; };
     struct Data {
         u32x4 a, b, h; u32x2 s; uint32_t d;
@@ -173,6 +239,10 @@ struct Q6K {
 #pragma unroll
         for (int g = 0; g < 4; g++) run[g] = 16 * b + 8 * hf + t + 2 * g;   // columns 256b + 128hf + 32g + 16t + [0,16)
     }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) {
+        u = ((r >> 4) << 2) | (((r >> 3) & 1) << 1) | (r & 1);
+        j = (r >> 1) & 3;
+    }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
         d.a = ((const U4A2*)(row + (L.off_a + eo)))->v;
@@ -183,15 +253,15 @@ struct Q6K {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
-                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
-        int acc[M][4][3];
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][NP][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xq)[M][NRUN], float (&out)[M]) {
+        int acc[M][4][NP];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
             for (int g = 0; g < 4; g++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) acc[m][g][p] = 0;
+                for (int p = 0; p < NP; p++) acc[m][g][p] = 0;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             uint32_t A = D.a[i], B = D.b[i], H = D.h[i];
@@ -206,7 +276,7 @@ struct Q6K {
 #pragma unroll
                 for (int g = 0; g < 4; g++)
 #pragma unroll
-                    for (int p = 0; p < 3; p++) acc[m][g][p] = pdot<false>(p, xp[m][g][p][i], q[g], acc[m][g][p]);
+                    for (int p = 0; p < NP; p++) acc[m][g][p] = dot4(xp[m][g][p][i], q[g], acc[m][g][p]);
         }
         uint32_t s0 = D.s[0] >> L.ssh, s1 = D.s[1] >> L.ssh;  // sc[is], sc[is+2] | sc[is+4], sc[is+6]
         float c[4] = {sb(s0, 0), sb(s0, 2), sb(s1, 0), sb(s1, 2)};
@@ -216,8 +286,8 @@ struct Q6K {
             float t = 0.f;
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                float f = xs[m][g] * planes_to_f32(acc[m][g][0], acc[m][g][1], acc[m][g][2]);
-                t = fmaf(c[g], fmaf(-32.f, xsum[m][g], f), t);   // sum x*(q-32) = sum x*q - 32*sum x
+                const float f = fmaf(xs[m][g], planes_f32(acc[m][g]), -32.f * xq[m][g]);   // sum x*(q-32) = sum x*q - 32*sum x
+                t = fmaf(c[g], f, t);
             }
             out[m] = d * t;
         }
@@ -225,8 +295,8 @@ struct Q6K {
 };
 
 struct Q80 {
-    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32, U1 = 4;
-    static constexpr bool SIGNED_W = true;
+    static constexpr uint32_t TYPE = FHIP_Q8_0;
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
     struct Lane { uint32_t off; };
     struct Data {
         u32x4 q0, q1; uint32_t d;
@@ -236,6 +306,7 @@ struct Q80 {
         L.off = u * 34;
         run[0] = u;
     }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r; j = 0; }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
         d.d = *(const uint16_t*)(row + (L.off + eo));
@@ -244,34 +315,34 @@ struct Q80 {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][NP][RUN / 4],
                                                const float (&xs)[M][NRUN], const float (&)[M][NRUN], float (&out)[M]) {
-        int acc[M][3];
+        int acc[M][NP];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
-            for (int p = 0; p < 3; p++) acc[m][p] = 0;
+            for (int p = 0; p < NP; p++) acc[m][p] = 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             uint32_t w = i < 4 ? D.q0[i] : D.q1[i - 4];
 #pragma unroll
             for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) acc[m][p] = dot4(xp[m][0][p][i], w, acc[m][p]);
+                for (int p = 0; p < NP; p++) acc[m][p] = dot4(xp[m][0][p][i], w, acc[m][p]);
         }
         float d = f16_bits(D.d);
         // per block: part = sum x*q, then part*d -- crates/ferric-tensor/src/cpu_simd.rs:66-70
 #pragma unroll
-        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])) * d;
+        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_f32(acc[m])) * d;
     }
 };
 
 // Q5_K: 176 B = [f16 d][f16 dmin][12 B 6-bit scales/mins][qh 32 B][qs 128 B] -- Q4_K plus bit s of qh[l] as the fifth bit of
 // element l of sub-block s (crates/ferric-gguf/src/lib.rs:692-716). Unit = group g of block b (sub-blocks 2g, 2g+1): its 32
-// quant bytes and the whole 32 bytes of high bits; codes 0..31, unsigned planes as Q4_K.
+// quant bytes and the whole 32 bytes of high bits; codes 0..31.
 struct Q5K {
-    static constexpr int WPL = 64, RUN = 32, NRUN = 2, BLOCK_VALUES = 256, U1 = 2;
-    static constexpr bool SIGNED_W = false;
+    static constexpr uint32_t TYPE = FHIP_Q5_K;
+    static constexpr int WPL = 64, RUN = 32, NRUN = 2, U1 = 2;
     struct Lane { uint32_t off_h, off_q, sh, g2, m1, m2, m3; };
     struct Data {
         u32x4 h, b0, b1, q0, q1;
@@ -289,6 +360,7 @@ struct Q5K {
         run[0] = 2 * u;
         run[1] = 2 * u + 1;
     }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r >> 1; j = r & 1; }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
         d.h = *(const u32x4*)(row + (L.off_h + eo));
@@ -299,20 +371,20 @@ struct Q5K {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
-                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][NP][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xq)[M][NRUN], float (&out)[M]) {
         uint32_t a = D.h[1] >> L.sh, b = D.h[2] >> L.sh, c = D.h[3] >> L.sh;
         uint32_t scp = (a & L.m1) | (c & L.m2) | ((a >> 2) & L.m3);
         uint32_t mp = (b & L.m1) | ((c >> 4) & L.m2) | ((b >> 2) & L.m3);
-        float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
-        float d0 = d * ub(scp, 0), d1 = d * ub(scp, 1), m0 = dmin * ub(mp, 0), m1 = dmin * ub(mp, 1);
-        int acc[M][2][3];
+        const float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
+        const float s0 = ub(scp, 0), s1 = ub(scp, 1), n0 = ub(mp, 0), n1 = ub(mp, 1);
+        int acc[M][2][NP];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) acc[m][j][p] = 0;
+                for (int p = 0; p < NP; p++) acc[m][j][p] = 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             uint32_t w = i < 4 ? D.q0[i] : D.q1[i - 4];
@@ -322,16 +394,16 @@ struct Q5K {
 #pragma unroll
             for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) {
-                    acc[m][0][p] = pdot<false>(p, xp[m][0][p][i], lo, acc[m][0][p]);
-                    acc[m][1][p] = pdot<false>(p, xp[m][1][p][i], hi, acc[m][1][p]);
+                for (int p = 0; p < NP; p++) {
+                    acc[m][0][p] = dot4(xp[m][0][p][i], lo, acc[m][0][p]);
+                    acc[m][1][p] = dot4(xp[m][1][p][i], hi, acc[m][1][p]);
                 }
         }
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            float f0 = xs[m][0] * planes_to_f32(acc[m][0][0], acc[m][0][1], acc[m][0][2]);
-            float f1 = xs[m][1] * planes_to_f32(acc[m][1][0], acc[m][1][1], acc[m][1][2]);
-            out[m] = (d0 * f0 - m0 * xsum[m][0]) + (d1 * f1 - m1 * xsum[m][1]);
+            const float f0 = xs[m][0] * planes_f32(acc[m][0]);
+            const float f1 = xs[m][1] * planes_f32(acc[m][1]);
+            out[m] = d * fmaf(s1, f1, s0 * f0) - dmin * fmaf(n1, xq[m][1], n0 * xq[m][0]);
         }
     }
 };
@@ -339,10 +411,10 @@ struct Q5K {
 // The four 32-value formats, [f16 d][f16 m]?[u32 qh]?[qs 16 B] (crates/ferric-gguf/src/lib.rs:618-684): value i < 16 is the low
 // nibble of qs[i], value 16 + i the high one, the fifth bit of value v is bit v of qh; (n - OFF) d or n d + m. Unit = one block;
 // the offset leaves as OFF * sum(x), the affine term as m * sum(x).
-template <int BYTES, bool HAS_M, bool HAS_QH, int OFF>
+template <uint32_t TY, int BYTES, bool HAS_M, bool HAS_QH, int OFF>
 struct LegS {
-    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32, U1 = 4;
-    static constexpr bool SIGNED_W = false;
+    static constexpr uint32_t TYPE = TY;
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
     static constexpr int QH = HAS_M ? 4 : 2, QS = QH + (HAS_QH ? 4 : 0);
     struct Lane { uint32_t off; };
     struct Data {
@@ -353,6 +425,7 @@ struct LegS {
         L.off = u * BYTES;
         run[0] = u;
     }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r; j = 0; }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
         const uint16_t* h = (const uint16_t*)(row + (L.off + eo));
@@ -362,13 +435,13 @@ struct LegS {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
-                                               const float (&xs)[M][NRUN], const float (&xsum)[M][NRUN], float (&out)[M]) {
-        int acc[M][3];
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][NP][RUN / 4],
+                                               const float (&xs)[M][NRUN], const float (&xq)[M][NRUN], float (&out)[M]) {
+        int acc[M][NP];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
-            for (int p = 0; p < 3; p++) acc[m][p] = 0;
+            for (int p = 0; p < NP; p++) acc[m][p] = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             uint32_t lo = D.q[j] & 0x0F0F0F0Fu, hi = (D.q[j] >> 4) & 0x0F0F0F0Fu;
@@ -379,25 +452,25 @@ struct LegS {
 #pragma unroll
             for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) {
-                    acc[m][p] = pdot<false>(p, xp[m][0][p][j], lo, acc[m][p]);
-                    acc[m][p] = pdot<false>(p, xp[m][0][p][4 + j], hi, acc[m][p]);
+                for (int p = 0; p < NP; p++) {
+                    acc[m][p] = dot4(xp[m][0][p][j], lo, acc[m][p]);
+                    acc[m][p] = dot4(xp[m][0][p][4 + j], hi, acc[m][p]);
                 }
         }
         const float d = f16_bits(D.dm & 0xFFFFu), mn = HAS_M ? f16_bits(D.dm >> 16) : 0.f;
 #pragma unroll
         for (int m = 0; m < M; m++)
-            out[m] = fmaf(d, fmaf(-(float)OFF, xsum[m][0], xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])), mn * xsum[m][0]);
+            out[m] = fmaf(d, fmaf(-(float)OFF, xq[m][0], xs[m][0] * planes_f32(acc[m])), mn * xq[m][0]);
     }
 };
-typedef LegS<18, false, false, 8> Q40;
-typedef LegS<20, true, false, 0> Q41;
-typedef LegS<22, false, true, 16> Q50;
-typedef LegS<24, true, true, 0> Q51;
+typedef LegS<FHIP_Q4_0, 18, false, false, 8> Q40;
+typedef LegS<FHIP_Q4_1, 20, true, false, 0> Q41;
+typedef LegS<FHIP_Q5_0, 22, false, true, 16> Q50;
+typedef LegS<FHIP_Q5_1, 24, true, true, 0> Q51;
 
 // IQ4_NL (18 B = [f16 d][qs 16 B]) and IQ4_XS (136 B = [f16 d][u16 scales_h][scales_l 4 B][qs 128 B]): 4-bit indices into the
-// 16-level codebook {-127 .. 113} (crates/ferric-gguf/src/lib.rs:751-791), looked up four at a time by byte permute; the levels
-// are int8, so the activation planes are the balanced digits Q8_0 uses. Unit = one 32-value (sub-)block.
+// 16-level codebook {-127 .. 113} (crates/ferric-gguf/src/lib.rs:751-791), looked up four at a time by byte permute into int8
+// levels. Unit = one 32-value (sub-)block.
 __device__ __forceinline__ uint32_t lut16x4(uint32_t idx, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
     uint32_t sel = idx & 0x07070707u;
     uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel);   // selector 0..3: bytes of t0, 4..7: bytes of t1
@@ -409,8 +482,8 @@ struct __attribute__((packed, aligned(8))) U4A8 { u32x4 v; };
 
 template <bool XS>
 struct IQ4S {
-    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = XS ? 256 : 32, U1 = 4;
-    static constexpr bool SIGNED_W = true;
+    static constexpr uint32_t TYPE = XS ? FHIP_IQ4_XS : FHIP_IQ4_NL;
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
     struct Lane { uint32_t off_h, off_q, ib; };
     struct Data {
         u32x4 q; uint32_t h0, h1;
@@ -421,6 +494,7 @@ struct IQ4S {
         else { L.ib = 0; L.off_h = u * 18; L.off_q = L.off_h + 2; }
         run[0] = u;
     }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r; j = 0; }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
         if (XS) {
@@ -435,22 +509,22 @@ struct IQ4S {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+    static __device__ __forceinline__ void dot(const Data& D, const Lane& L, const uint32_t (&xp)[M][NRUN][NP][RUN / 4],
                                                const float (&xs)[M][NRUN], const float (&)[M][NRUN], float (&out)[M]) {
         // the codebook as int8 bytes, four levels per word
         constexpr uint32_t T0 = 0xBFAD9881u, T1 = 0xF6EADDCFu, T2 = 0x26190D01u, T3 = 0x71594535u;
-        int acc[M][3];
+        int acc[M][NP];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
-            for (int p = 0; p < 3; p++) acc[m][p] = 0;
+            for (int p = 0; p < NP; p++) acc[m][p] = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             uint32_t lo = lut16x4(D.q[j] & 0x0F0F0F0Fu, T0, T1, T2, T3), hi = lut16x4((D.q[j] >> 4) & 0x0F0F0F0Fu, T0, T1, T2, T3);
 #pragma unroll
             for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) {
+                for (int p = 0; p < NP; p++) {
                     acc[m][p] = dot4(xp[m][0][p][j], lo, acc[m][p]);
                     acc[m][p] = dot4(xp[m][0][p][4 + j], hi, acc[m][p]);
                 }
@@ -461,21 +535,21 @@ struct IQ4S {
             dl *= (float)(ls - 32);
         }
 #pragma unroll
-        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])) * dl;
+        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_f32(acc[m])) * dl;
     }
 };
 typedef IQ4S<false> IQ4NL;
 typedef IQ4S<true> IQ4XS;
 
 // MXFP4 (17 B = [u8 e][qs 16 B], crates/ferric-gguf/src/lib.rs:857-908): weight = k * 2^(e - 128) with k the doubled E2M1 value,
-// an integer in {0, +-1, +-2, +-3, +-4, +-6, +-8, +-12}: int8 codes and balanced activation planes as for IQ4, the power of two
-// applied to the block's integer dot product. The reference forms k * scale per element BEFORE it meets the activation
+// an integer in {0, +-1, +-2, +-3, +-4, +-6, +-8, +-12}: int8 codes, the power of two applied to the block's integer dot
+// product. The reference forms k * scale per element BEFORE it meets the activation
 // (crates/ferric-tensor/src/dtype.rs:3331-3344), which only differs where that product overflows (e >= 252): such a block takes
 // the element-by-element branch below, on the activations as the planes hold them (zeros stay zeros, so inf * 0 is still NaN).
 struct __attribute__((packed, aligned(1))) U4A1 { u32x4 v; };
 struct MXF4S {
-    static constexpr int WPL = 32, RUN = 32, NRUN = 1, BLOCK_VALUES = 32, U1 = 4;
-    static constexpr bool SIGNED_W = true;
+    static constexpr uint32_t TYPE = FHIP_MXFP4;
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
     struct Lane { uint32_t off; };
     struct Data {
         u32x4 q; uint32_t e;
@@ -485,6 +559,7 @@ struct MXF4S {
         L.off = u * 17;
         run[0] = u;
     }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r; j = 0; }
     static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L, uint32_t eo) {
         Data d;
         d.e = row[L.off + eo];
@@ -492,7 +567,7 @@ struct MXF4S {
         return d;
     }
     template <int M>
-    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][3][RUN / 4],
+    static __device__ __forceinline__ void dot(const Data& D, const Lane&, const uint32_t (&xp)[M][NRUN][NP][RUN / 4],
                                                const float (&xs)[M][NRUN], const float (&)[M][NRUN], float (&out)[M]) {
         constexpr uint32_t T0 = 0x03020100u, T1 = 0x0C080604u, T2 = 0xFDFEFF00u, T3 = 0xF4F8FAFCu;
         const float d = __uint_as_float(D.e == 0 ? (1u << 21) : D.e == 1 ? (1u << 22) : (D.e - 1u) << 23);
@@ -509,8 +584,9 @@ struct MXF4S {
 #pragma unroll 1
                 for (int el = 0; el < 32; el++) {
                     const int i = el >> 2, sh = 8 * (el & 3);
-                    const int v = ((int)(int8_t)(xp[m][0][0][i] >> sh)) * 65536 + ((int)(int8_t)(xp[m][0][1][i] >> sh)) * 256 +
-                                  (int)(int8_t)(xp[m][0][2][i] >> sh);
+                    int v = 0;
+#pragma unroll
+                    for (int p = 0; p < NP; p++) v = v * 256 + (int)(int8_t)(xp[m][0][p][i] >> sh);
                     const uint32_t kw = el < 16 ? lo[el >> 2] : hi[(el - 16) >> 2];
                     const float w = (float)(int)(int8_t)(kw >> sh) * d;
                     a = fmaf(xs[m][0] * (float)v, w, a);
@@ -519,22 +595,22 @@ struct MXF4S {
             }
             return;
         }
-        int acc[M][3];
+        int acc[M][NP];
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
-            for (int p = 0; p < 3; p++) acc[m][p] = 0;
+            for (int p = 0; p < NP; p++) acc[m][p] = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++)
 #pragma unroll
             for (int m = 0; m < M; m++)
 #pragma unroll
-                for (int p = 0; p < 3; p++) {
+                for (int p = 0; p < NP; p++) {
                     acc[m][p] = dot4(xp[m][0][p][j], lo[j], acc[m][p]);
                     acc[m][p] = dot4(xp[m][0][p][4 + j], hi[j], acc[m][p]);
                 }
 #pragma unroll
-        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_to_f32(acc[m][0], acc[m][1], acc[m][2])) * d;
+        for (int m = 0; m < M; m++) out[m] = (xs[m][0] * planes_f32(acc[m])) * d;
     }
 };
 
@@ -550,6 +626,7 @@ struct GemvParams {
     int units;           // units per row = cols / WPL; the last slot may be partly filled
     int RF;              // replicas of the full-wave set, each taking every RF-th row (balances them against the tail wave)
     int G;               // row groups per workgroup
+    int S;               // waves that stage the activations (all of them when the input norm is fused)
     int rpg;             // output rows per row group
     // ceil(2^32 / d) for the three divisors of the kernel's index arithmetic (waves per row group, full waves per row, RF), 0
     // for d = 1: floor(n / d) = mulhi(n, magic) for n < 65 536, 2 <= d <= 1024; a hardware-less integer division costs ~35
@@ -566,17 +643,71 @@ struct GemvParams {
     int row_wgs;         // workgroups that own rows; the launch may hold one more, which only stores x + resid
 };
 
-// Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 768 -> 168, 512 -> 256).
+// Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 512 -> 256).
 constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
-// Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit that budget.
 // Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit 128 VGPRs
-// at batch 1 (16 waves per CU). Measured: 16 waves with 3 rows in flight beat 12 waves with 6-8 in flight
-// on every shape but the 638 MB head, and there by 6 % only.
+// at batch 1 (16 waves per CU).
 template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? F::U1 : 2; }
-// Activation rows one pass can hold in registers (48 plane dwords per row for the 64-weight units, 24 for Q8_0).
+// Activation rows one pass can hold in registers.
 template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
 
 __device__ __forceinline__ uint32_t div_magic(uint32_t n, uint32_t magic) { return magic ? __umulhi(n, magic) : n; }
+
+// Eight consecutive activations of one run -> NP plane dword pairs, the run's scale and the run's quantised sum.
+// The 2 (RUN 16) or 4 (RUN 32) lanes of a run sit in one quad and agree on amax, the scale and the sum afterwards.
+template <int RUN>
+__device__ __forceinline__ void quantize8(const float (&v)[8], uint32_t (&pl)[NP][2], float& scale_out, float& sum_out) {
+    float amax = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
+                       fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
+    float sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));   // NaN / inf detector (fmaxf drops NaNs)
+    amax = fmaxf(amax, dpp_f<DPP_XOR1>(amax));
+    sum += dpp_f<DPP_XOR1>(sum);
+    if (RUN == 32) {
+        amax = fmaxf(amax, dpp_f<DPP_XOR2>(amax));
+        sum += dpp_f<DPP_XOR2>(sum);
+    }
+    // not representable in block fixed point: non-finite members, a sum beyond the f32 range, or a run so small that
+    // QMAX / amax would overflow
+    const bool special = !(fabsf(sum) <= 3.4028234663852886e38f) || (amax < TINY_RUN && amax > 0.f);
+    const float inv = amax > 0.f ? QMAX * __builtin_amdgcn_rcpf(amax) : 0.f;
+    uint32_t t[8];
+    if constexpr (NP == 2) {
+        // round to nearest by adding 1.5 * 2^23; the 128 makes the low byte an offset-binary digit
+#pragma unroll
+        for (int i = 0; i < 8; i++) t[i] = __float_as_uint(fmaf(v[i], inv, 12582912.0f + 128.0f));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            int q = __float2int_rn(v[i] * inv);
+            q = q > (int)QMAX ? (int)QMAX : (q < -(int)QMAX ? -(int)QMAX : q);
+            t[i] = (uint32_t)(q + 0x8080);
+        }
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+        const uint32_t t0 = t[4 * hh], t1 = t[4 * hh + 1], t2 = t[4 * hh + 2], t3 = t[4 * hh + 3];
+        const uint32_t p01 = __builtin_amdgcn_perm(t1, t0, 0x05010400u), p23 = __builtin_amdgcn_perm(t3, t2, 0x05010400u);
+        pl[NP - 1][hh] = __builtin_amdgcn_perm(p23, p01, 0x05040100u) ^ 0x80808080u;   // bytes 0, back to signed digits
+        if constexpr (NP == 2) {
+            pl[0][hh] = __builtin_amdgcn_perm(p23, p01, 0x07060302u);                  // bytes 1: the signed top digit
+        } else {
+            pl[1][hh] = __builtin_amdgcn_perm(p23, p01, 0x07060302u) ^ 0x80808080u;
+            const uint32_t u01 = __builtin_amdgcn_perm(t1, t0, 0x00000602u), u23 = __builtin_amdgcn_perm(t3, t2, 0x00000602u);
+            pl[0][hh] = __builtin_amdgcn_perm(u23, u01, 0x05040100u);                  // bytes 2
+        }
+    }
+    int qs[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) qs[p] = dot4(pl[p][1], 0x01010101u, dot4(pl[p][0], 0x01010101u, 0));
+    int qsum = qs[0];
+#pragma unroll
+    for (int p = 1; p < NP; p++) qsum = (qsum << 8) + qs[p];
+    qsum += dpp_i<DPP_XOR1>(qsum);
+    if (RUN == 32) qsum += dpp_i<DPP_XOR2>(qsum);
+    const float scale = amax * (1.0f / QMAX);
+    scale_out = special ? __uint_as_float(0x7FC00000u) : scale;
+    sum_out = scale * (float)qsum;
+}
 
 template <class F, int M, int U, bool SWIGLU, bool NORM>
 __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams p) {
@@ -588,9 +719,22 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     // The activation loads go out before anything else: they need the thread index only, and the index arithmetic below
     // (a few hundred scalar instructions, which the four waves of a SIMD get through one after the other, oldest first)
     // then runs under their latency instead of in front of it.
-    const int e0 = tid * 8;
+    // The activations are staged by the first p.S waves of the workgroup only (the oldest, so the first to be scheduled in
+    // every phase): up to four 8-value pieces per thread, all requested here so that they arrive under one memory round
+    // trip. The other waves go straight to their weight rows and meet the stagers at the barrier.
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool stager = wave < p.S;
+    const int e0 = stager ? tid * 8 : M * p.cols, e_step = p.S * 512;
     float4 xa0 = {0, 0, 0, 0}, xb0 = {0, 0, 0, 0};
     if (e0 < M * p.cols) { xa0 = *(const float4*)(p.x + e0); xb0 = *(const float4*)(p.x + e0 + 4); }
+    constexpr int XR = 3;
+    float4 xar[XR], xbr[XR];
+#pragma unroll
+    for (int k = 0; k < XR; k++) {
+        const int e = e0 + (k + 1) * e_step;
+        xar[k] = xbr[k] = float4{0, 0, 0, 0};
+        if (e < M * p.cols) { xar[k] = *(const float4*)(p.x + e); xbr[k] = *(const float4*)(p.x + e + 4); }
+    }
     constexpr bool fused_norm = NORM && M == 1;   // a separate instantiation: the plain kernel carries none of this
     float4 nwa = {1, 1, 1, 1}, nwb = {1, 1, 1, 1}, rsa = {0, 0, 0, 0}, rsb = {0, 0, 0, 0};
     if (fused_norm && e0 < p.cols) {              // the norm's weights and the residual ride with the activations
@@ -609,19 +753,23 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
         }
         return;
     }
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NGF = p.NG >> 2, NT = p.NG & 3, NFW = NGF * p.RF, WPR = NFW + (NT ? 1 : 0);
     const int rg = (int)div_magic((uint32_t)wave, p.m_wpr), wr = wave - rg * WPR;   // row group within workgroup, wave within row group
     const int wq = (int)div_magic((uint32_t)wr, p.m_ngf), wm = wr - wq * NGF;       // wr / NGF, wr % NGF (NGF = 0: never used)
     const bool tail = wr == NFW;                         // wave-uniform
-    const int RT = tail ? (NT == 1 ? 4 : NT == 2 ? 2 : 1) : 1;   // rows this wave works on at once
+    const int RTL = tail ? (NT == 1 ? 2 : NT == 2 ? 1 : 0) : 0;   // log2 of the rows this wave works on at once
+    const int RT = 1 << RTL;
     // iteration i of this wave works on virtual row v_start + i * v_step (+ row_off per lane in a tail wave)
     const int v_start = tail ? 0 : wq, v_step = tail ? RT : p.RF;
 
-    // LDS: activation planes [M][cols/RUN][3][RUN] bytes | scales [M][cols/RUN] | sums [M][cols/RUN] | partials
+    // LDS: activation planes | scales [M][NRUN][units] | sums [M][NRUN][units] | partials. The planes are laid out for the
+    // readers: the 16-byte piece c of plane pp of run j of unit u (of activation row m) sits at
+    // ((((m NRUN + j) NP + pp) RD/4 + c) units + u) * 16, so the lanes of a wave (consecutive units) read consecutive pieces
+    // and a 16-byte read of 64 lanes touches every bank once (run-major storage put the lanes 128 bytes apart: 8 banks).
     const int nrun = p.cols / RUN;
+    constexpr int RC = RD / 4;                           // 16-byte pieces per plane of a run
     uint8_t* planes = smem;
-    float* scales = (float*)(smem + (size_t)M * p.cols * 3);
+    float* scales = (float*)(smem + (size_t)M * p.cols * NP);
     float* sums = scales + (size_t)M * nrun;
     float* part = sums + (size_t)M * nrun;               // [G][rpg*VPR][NG][M]
 
@@ -636,7 +784,8 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     int run[NRUN];
     // a lane past the row's last unit (rows whose length does not fill the last slot) works on unit 0 and contributes 0
     const bool unit_ok = group * 16 + l16 < p.units;
-    F::setup(unit_ok ? group * 16 + l16 : 0, L, run);
+    const int my_unit = unit_ok ? group * 16 + l16 : 0;
+    F::setup(my_unit, L, run);
 
     const int r0 = (blockIdx.x * p.G + rg) * p.rpg;
     int nrows = p.out_rows - r0;
@@ -645,7 +794,9 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     const uint8_t* base = p.W + (size_t)(nrows > 0 ? r0 : 0) * p.row_bytes;   // a row group past the end points at row 0
     // (nv - v_start + v_step - 1) / v_step with v_step = 4, 2, 1 (tail wave) or RF
     const uint32_t n_num = (uint32_t)(nv - v_start + v_step - 1);
-    const int n_it = nv > v_start ? (int)(tail ? n_num >> (RT == 4 ? 2 : RT == 2 ? 1 : 0) : div_magic(n_num, p.m_rf)) : 0;
+    const int n_it = nv > v_start ? (int)(tail ? n_num >> RTL : div_magic(n_num, p.m_rf)) : 0;
+    // iterations all of whose rows exist (a tail wave's last iteration may hold fewer than RT)
+    const int n_full = tail ? nv >> RTL : n_it;
     // Address of iteration `it`: a wave-uniform row base (scalar registers) plus a 32-bit lane offset. A tail
     // wave's lanes sit row_off rows further (v_start + it*v_step is a multiple of RT there, so with fused
     // SwiGLU the gate/up split of row_off is fixed); lanes past the last row read the uniform row instead
@@ -656,16 +807,18 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
         const int v = v_start + it * v_step;             // wave-uniform
         return SWIGLU ? base + (size_t)(v >> 1) * p.row_bytes + (size_t)(v & 1) * p.pair_bytes : base + (size_t)v * p.row_bytes;
     };
-    auto fetch = [&](int it) { return F::load(row_base(it), L, (v_start + it * v_step + row_off < nv) ? lane_extra : 0u); };
+    auto lane_eo = [&](int it) { return (v_start + it * v_step + row_off < nv) ? lane_extra : 0u; };
+    auto fetch = [&](int it) { return F::load(row_base(it), L, lane_eo(it)); };
+    auto fetch_full = [&](int it) { return F::load(row_base(it), L, lane_extra); };   // it < n_full: every lane's row exists
 
-    // ---- the (cache-resident) activation loads go out first, then the weight bytes of the first U iterations.
-    // (Loads return in issue order. Issuing exactly U row loads unconditionally would let the wait for the
-    // activations be a counted one instead of a drain, but the dummy loads of waves with fewer than U rows
-    // cost more than that saves: measured +40 % on the 4096x4096 Q8_0 GEMV.)
+    // ---- the activation loads went out first; now the weight bytes of the wave's first row, UNCONDITIONALLY (a wave
+    // without rows reads the weight's row 0 and drops it). Loads return in issue order, so the wait for the activations
+    // is a counted one only if the compiler knows how many loads follow them; behind a conditional load it has to drain
+    // the queue, and the quantisation below then waits for every prefetched row of the wave (seconds of microseconds on
+    // the large shapes, during which the memory pipe runs dry). The rest of the prefetch goes out behind the quantisation.
     typename F::Data buf[U];
-#pragma unroll
-    for (int j = 0; j < U; j++)
-        if (j < n_it) buf[j] = fetch(j);
+    buf[0] = F::load(n_it > 0 ? row_base(0) : p.W, L, n_it > 0 ? lane_eo(0) : 0u);
+    asm volatile("" ::: "memory");
 
     if (fused_norm) {
         // x <- rmsnorm(x + resid) * norm_w (crates/ferric-tensor/src/lib.rs:2057-2074): each thread holds at most one
@@ -688,58 +841,36 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
         xb0.x *= nwb.x; xb0.y *= nwb.y; xb0.z *= nwb.z; xb0.w *= nwb.w;
     }
 
-    // ---- activations -> 24-bit block fixed point, once per workgroup, through LDS
-    constexpr float QMAX = F::SIGNED_W ? QMAX_S : QMAX_U;
-    for (int e = e0; e < M * p.cols; e += blockDim.x * 8) {
-        float4 a = xa0, b = xb0;
-        if (e != e0) { a = *(const float4*)(p.x + e); b = *(const float4*)(p.x + e + 4); }
-        float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-        float amax = fmaxf(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))),
-                           fmaxf(fmaxf(fabsf(v[4]), fabsf(v[5])), fmaxf(fabsf(v[6]), fabsf(v[7]))));
-        float sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
-        amax = fmaxf(amax, dpp_f<0xB1>(amax));           // the 2 (RUN 16) or 4 (RUN 32) lanes of a run sit in one quad
-        sum += dpp_f<0xB1>(sum);
-        if (RUN == 32) {
-            amax = fmaxf(amax, dpp_f<0x4E>(amax));
-            sum += dpp_f<0x4E>(sum);
-        }
-        float inv = amax > 0.f ? QMAX / amax : 0.f;
-        int q[8];
+    // ---- activations -> block fixed point, once per workgroup, through LDS
+    if (!fused_norm && stager) __builtin_amdgcn_s_setprio(3);   // the whole workgroup waits for this
+    auto stage = [&](int e, const float4& a, const float4& b) {
+        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        uint32_t pl[NP][2];
+        float scale, qsum;
+        quantize8<RUN>(v, pl, scale, qsum);
+        const int m = M == 1 ? 0 : e / p.cols, col = M == 1 ? e : e - m * p.cols;
+        const int within = col % RUN;
+        int u, j;
+        F::owner(col / RUN, u, j);
+        const int mj = m * NRUN + j;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            q[i] = __float2int_rn(v[i] * inv);
-            q[i] = q[i] > (int)QMAX ? (int)QMAX : (q[i] < -(int)QMAX ? -(int)QMAX : q[i]);   // rounding of v*inv may overshoot by one
-        }
-        uint32_t pl[3][2];
-        if (F::SIGNED_W) {
+        for (int pp = 0; pp < NP; pp++)
+            *(u32x2*)(planes + ((size_t)((mj * NP + pp) * RC + (within >> 4)) * p.units + u) * 16 + (within & 15)) = u32x2{pl[pp][0], pl[pp][1]};
+        if (within == 0) { scales[mj * p.units + u] = scale; sums[mj * p.units + u] = qsum; }
+    };
+    if (e0 < M * p.cols) stage(e0, xa0, xb0);
 #pragma unroll
-            for (int pp = 0; pp < 3; pp++) pl[pp][0] = pl[pp][1] = 0;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {                // balanced digits
-                int c = (q[i] << 24) >> 24;
-                int q1 = (q[i] - c) >> 8;
-                int b8 = (q1 << 24) >> 24;
-                int a8 = (q1 - b8) >> 8;
-                pl[0][i >> 2] |= (uint32_t)(a8 & 0xFF) << (8 * (i & 3));
-                pl[1][i >> 2] |= (uint32_t)(b8 & 0xFF) << (8 * (i & 3));
-                pl[2][i >> 2] |= (uint32_t)(c & 0xFF) << (8 * (i & 3));
-            }
-        } else {
-#pragma unroll
-            for (int hh = 0; hh < 2; hh++) {             // planes = byte lanes 2, 1, 0 of the two's complement integers
-                uint32_t q0 = q[4 * hh], q1 = q[4 * hh + 1], q2 = q[4 * hh + 2], q3 = q[4 * hh + 3];
-                uint32_t t01 = __builtin_amdgcn_perm(q1, q0, 0x05010400u), t23 = __builtin_amdgcn_perm(q3, q2, 0x05010400u);
-                uint32_t u01 = __builtin_amdgcn_perm(q1, q0, 0x00000602u), u23 = __builtin_amdgcn_perm(q3, q2, 0x00000602u);
-                pl[2][hh] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);   // bytes 0
-                pl[1][hh] = __builtin_amdgcn_perm(t23, t01, 0x07060302u);   // bytes 1
-                pl[0][hh] = __builtin_amdgcn_perm(u23, u01, 0x05040100u);   // bytes 2 (sign carried by the arithmetic shift)
-            }
-        }
-        int r = e / RUN, within = e % RUN;               // run index counts across the M activation rows
-#pragma unroll
-        for (int pp = 0; pp < 3; pp++) *(u32x2*)(planes + ((size_t)r * 3 + pp) * RUN + within) = u32x2{pl[pp][0], pl[pp][1]};
-        if (within == 0) { scales[r] = amax / QMAX; sums[r] = sum; }
+    for (int k = 0; k < XR; k++) {
+        const int e = e0 + (k + 1) * e_step;
+        if (e < M * p.cols) stage(e, xar[k], xbr[k]);
     }
+    for (int e = e0 + (XR + 1) * e_step; e < M * p.cols; e += e_step)      // rows beyond four passes
+        stage(e, *(const float4*)(p.x + e), *(const float4*)(p.x + e + 4));
+    if (!fused_norm && stager) __builtin_amdgcn_s_setprio(0);
+    // the rest of the prefetch: in flight while the workgroup meets at the barrier and copies its planes out of LDS
+#pragma unroll
+    for (int j = 1; j < U; j++)
+        if (j < n_it) buf[j] = fetch(j);
     __syncthreads();
 
     // The row scale the staged activations went without, for the threads that will write outputs: worked out here, under
@@ -758,69 +889,121 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
         ninv = 1.0f / sqrtf(tot / (float)p.cols + p.eps);
     }
 
-    uint32_t xp[M][NRUN][3][RD];
-    float xs[M][NRUN], xsum[M][NRUN];
+    uint32_t xp[M][NRUN][NP][RD];
+    float xs[M][NRUN], xq[M][NRUN];
+    bool special = false;                                // one of this lane's runs needs the element-by-element branch
 #pragma unroll
     for (int m = 0; m < M; m++)
 #pragma unroll
         for (int j = 0; j < NRUN; j++) {
-            int r = m * nrun + run[j];
-            xs[m][j] = scales[r];
-            xsum[m][j] = sums[r];
+            const int mj = m * NRUN + j;
+            xs[m][j] = scales[mj * p.units + my_unit];
+            xq[m][j] = sums[mj * p.units + my_unit];
+            special = special || xs[m][j] != xs[m][j];
 #pragma unroll
-            for (int pp = 0; pp < 3; pp++)
+            for (int pp = 0; pp < NP; pp++)
 #pragma unroll
                 for (int i = 0; i < RD; i += 4) {
-                    u32x4 t = *(const u32x4*)(planes + ((size_t)r * 3 + pp) * RUN + 4 * i);
+                    u32x4 t = *(const u32x4*)(planes + ((size_t)((mj * NP + pp) * RC + (i >> 2)) * p.units + my_unit) * 16);
                     xp[m][j][pp][i] = t[0]; xp[m][j][pp][i + 1] = t[1]; xp[m][j][pp][i + 2] = t[2]; xp[m][j][pp][i + 3] = t[3];
                 }
         }
+    special = special && unit_ok;
 
     // ---- stream the rows. Software pipeline over the U row buffers, written so that the steady-state
     // loop has no conditional reload: a reload under a condition makes the loop-carried buffers phi
     // nodes whose copies wait for every outstanding load at the back edge, which serialises the stream.
     float* mypart = part + (size_t)rg * p.rpg * VPR * p.NG * M;
-    auto consume = [&](typename F::Data& cur, int it) {
-        cur.pin_all();
-        float acc[M];
-        F::template dot<M>(cur, L, xp, xs, xsum, acc);
-        const int v = v_start + it * v_step + row_off;
-        const bool ok = lane_ok && v < nv;
+    // The U rows of a pipeline step are summed over the slot together; lane l < 4 of a slot then holds the sum for the
+    // step's row slot_of(l) and stores it.
+    const bool bit0 = (lane & 1) != 0, bit1 = (lane & 2) != 0;
+    const int my_j = slot_of<U>(l16);
+    const bool store_lane = lane_ok && l16 < (U == 1 ? 1 : U == 2 ? 4 : 4) && my_j < U && (U != 2 || (l16 & 1) == 0);
+    auto store_step = [&](const float (&outs)[M][U], int it0) {
+        const int v = v_start + (it0 + my_j) * v_step + row_off;
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            float t = slot_sum(unit_ok ? acc[m] : 0.f);
-            if (ok && l16 == 0) mypart[((size_t)v * p.NG + group) * M + m] = t;
+            const float t = slot_sum_many<U>(outs[m], bit0, bit1);
+            if (store_lane && v < nv) mypart[((size_t)v * p.NG + group) * M + m] = t;
         }
     };
+    const bool contributes = unit_ok && !special;        // a special lane's share is added by the pass behind the loop
+    auto consume = [&](typename F::Data& cur, int it, float (&outs)[M][U], int j) {
+        cur.pin_all();
+        float acc[M];
+        F::template dot<M>(cur, L, xp, xs, xq, acc);
+#pragma unroll
+        for (int m = 0; m < M; m++) outs[m][j] = contributes ? acc[m] : 0.f;
+    };
     int i0 = 0;
+    float outs[M][U];
     // All prologue loads have landed by now (they overlapped the activation quantisation). Saying so
     // explicitly gives the compiler's wait-count tracking a clean state at the loop head; without it the
     // merge of the prologue's load order with the loop's makes every iteration wait for vmcnt(0).
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt/lgkmcnt untouched
 #pragma unroll 1
-    for (; i0 + 2 * U <= n_it; i0 += U) {        // every row of this step and of the next one exists
+    for (; i0 + 2 * U <= n_full; i0 += U) {      // every row of this step and of the next one exists
 #pragma unroll
         for (int j = 0; j < U; j++) {
             // consume, then refill the same registers: the old bytes are dead when the new load is issued,
             // so the loop-carried buffer needs no copy (and no wait) at the back edge
-            consume(buf[j], i0 + j);
-            buf[j] = fetch(i0 + j + U);
+            consume(buf[j], i0 + j, outs, j);
+            buf[j] = fetch_full(i0 + j + U);
         }
+        store_step(outs, i0);
     }
     // drain, step A: iterations [i0, i0+U) that exist, reloading what is left of the step after it
 #pragma unroll
     for (int j = 0; j < U; j++) {
         const int it = i0 + j;
         if (it < n_it) {
-            consume(buf[j], it);
+            consume(buf[j], it, outs, j);
             if (it + U < n_it) buf[j] = fetch(it + U);
+        } else {
+#pragma unroll
+            for (int m = 0; m < M; m++) outs[m][j] = 0.f;
         }
     }
+    if (i0 < n_it) store_step(outs, i0);
     // drain, step B: iterations [i0+U, n_it)
 #pragma unroll
     for (int j = 0; j < U; j++) {
         const int it = i0 + U + j;
-        if (it < n_it) consume(buf[j], it);
+        if (it < n_it) consume(buf[j], it, outs, j);
+        else {
+#pragma unroll
+            for (int m = 0; m < M; m++) outs[m][j] = 0.f;
+        }
+    }
+    if (i0 + U < n_it) store_step(outs, i0 + U);
+
+    // ---- the element-by-element pass of the lanes whose activations block fixed point cannot hold (rare: only waves
+    // that own such a run enter): the unit's columns from the raw activations (for the fused norm: as staged,
+    // (x + resid) * norm_w) times the exactly dequantised weights, summed over the slot and added to what the slot's
+    // other lanes left in LDS for the row.
+    if (__builtin_amdgcn_ballot_w64(special) != 0) {
+#pragma unroll 1
+        for (int it = 0; it < n_it; it++) {
+            const uint8_t* rowp = row_base(it) + lane_eo(it);
+            const int v = v_start + it * v_step + row_off;
+#pragma unroll 1
+            for (int m = 0; m < M; m++) {
+                float a = 0.f;
+                if (special) {
+#pragma unroll 1
+                    for (int j = 0; j < NRUN; j++)
+#pragma unroll 1
+                        for (int i = 0; i < RUN; i++) {
+                            const int col = run[j] * RUN + i;
+                            float xv = p.x[(size_t)m * p.cols + col];
+                            if (fused_norm) xv = (xv + (p.resid ? p.resid[col] : 0.f)) * p.norm_w[col];
+                            a += xv * fhip::deq_at<F::TYPE>(rowp, col);
+                        }
+                }
+                a = slot_sum(a);
+                if (lane_ok && l16 == 0 && v < nv) mypart[((size_t)v * p.NG + group) * M + m] += a;
+            }
+        }
     }
     __syncthreads();
 
@@ -862,11 +1045,6 @@ __global__ void zero_kernel(float* __restrict__ out, size_t n) {
 
 bool g_force_generic = false;   // tests: send every shape to the shape-complete f32 kernel
 
-int env_int(const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v && *v ? atoi(v) : dflt;
-}
-
 // The tail wave of a row group works on 4 (NG%4 == 1) or 2 (NG%4 == 2) rows per iteration while a full
 // wave works on one; replicating the full-wave set RF times, each replica taking every RF-th row, evens
 // the iteration counts out (K = 5120: 4 full waves + 1 tail wave, one iteration each per 4 rows).
@@ -881,13 +1059,12 @@ int waves_per_row_group(int NG, int maxw) { return (NG / 4) * full_wave_replicas
 
 template <class F, int M, bool SWIGLU>
 size_t lds_bytes(size_t cols, int NG, int G, int rpg) {
-    return M * cols * 3 + 2 * M * (cols / F::RUN) * sizeof(float) + (size_t)G * rpg * (SWIGLU ? 2 : 1) * NG * M * sizeof(float);
+    return M * cols * NP + 2 * M * (cols / F::RUN) * sizeof(float) + (size_t)G * rpg * (SWIGLU ? 2 : 1) * NG * M * sizeof(float);
 }
 
 template <class F, int M, bool SWIGLU>
 int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr,
                const fhip::NormParams* norm = nullptr) {
-    static const int tune_g = env_int("FHIP_GEMV_G", 0), tune_rpg = env_int("FHIP_GEMV_RPG", 0);
     constexpr int U = rows_in_flight<F>(M);
     void (*kernel)(GemvParams) = gemv_stream_kernel<F, M, U, SWIGLU, false>;
     if constexpr (M == 1) {
@@ -925,8 +1102,6 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     if (rpg < 1) rpg = 1;
     const size_t nrg = (out_rows + rpg - 1) / rpg;
     int G = nrg >= slots ? Gcap : (int)((nrg + cus - 1) / cus);
-    if (tune_g > 0) G = tune_g;
-    if (tune_rpg > 0) rpg = tune_rpg;
     p.G = G; p.rpg = rpg;
     auto magic = [](int d) { return d > 1 ? (uint32_t)(((1ull << 32) + (unsigned)d - 1) / (unsigned)d) : 0u; };
     p.m_wpr = magic(WPR); p.m_ngf = magic(p.NG >> 2); p.m_rf = magic(p.RF);
@@ -943,6 +1118,12 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
         if (lds > fhip::device_lds_bytes()) return fhip::NORM_NOT_FUSED;   // no room left beside the staged row
     }
     p.row_wgs = (int)grid;
+    {   // staging waves: enough for at most four 8-value pieces per thread, at least four (one per SIMD)
+        const int nwaves = WPR * G;
+        int S = (int)((M * w->cols + 2047) / 2048);
+        S = S < 4 ? 4 : S;
+        p.S = norm || S > nwaves ? nwaves : S;
+    }
     const size_t launch_wgs = grid + ((norm && norm->x_out && grid < (size_t)cus) ? 1 : 0);
     hipLaunchKernelGGL(kernel, dim3((unsigned)launch_wgs, (unsigned)p.sel.npairs), dim3(64 * WPR * G), lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
@@ -986,7 +1167,7 @@ int launch_fmt(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y
 
 namespace fhip {
 
-int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s) {
+int GEMV_EXPORT(launch_gemv)(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s) {
     if (w->rows == 0 || rows_x == 0) return FHIP_OK;
     const size_t out_rows = n_ff ? n_ff : w->rows;
     if (w->cols == 0) {  // empty inner dimension: every dot product is 0 (and silu(0)*0 = 0)
@@ -1027,7 +1208,7 @@ int launch_norm_fmt(const fhip_weight* w, const float* d_x, float* d_y, size_t o
     return swiglu ? launch_one<F, 1, true>(w, d_x, d_y, out_rows, s, nullptr, &norm) : launch_one<F, 1, false>(w, d_x, d_y, out_rows, s, nullptr, &norm);
 }
 
-int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s) {
+int GEMV_EXPORT(launch_gemv_norm)(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s) {
     if (w->rows == 0 || w->cols == 0) return NORM_NOT_FUSED;
     const size_t out_rows = n_ff ? n_ff : w->rows;
     switch (w->type) {
@@ -1053,7 +1234,7 @@ int launch_sel_fmt(const fhip_weight* w, const float* d_x, float* d_y, size_t ou
     return swiglu ? launch_one<F, 1, true>(w, d_x, d_y, out_rows, s, &sel) : launch_one<F, 1, false>(w, d_x, d_y, out_rows, s, &sel);
 }
 
-int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel,
+int GEMV_EXPORT(launch_gemv_sel)(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel,
                     hipStream_t s) {
     if (sel.npairs == 0 || out_rows == 0) return FHIP_OK;
     switch (w->type) {
@@ -1076,13 +1257,15 @@ int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t o
     }
 }
 
-void gemv_force_generic(bool on) { g_force_generic = on; }
+void GEMV_EXPORT(gemv_force_generic)(bool on) { g_force_generic = on; }
 
+#if FHIP_GEMV_PLANES == 2
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s) {
     size_t n = t * d;
     if (n == 0) return FHIP_OK;
     hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gu, n, d, d_out);
     return check_hip(hipGetLastError(), "swiglu launch");
 }
+#endif
 
 }  // namespace fhip

@@ -576,14 +576,8 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_kernel(GemvParams p) {
     }
 }
 
-int env_int(const char* name, int dflt) {
-    const char* v = getenv(name);
-    return v && *v ? atoi(v) : dflt;
-}
-
 template <class F, int M, bool SWIGLU>
 int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr) {
-    static const int tune_g = env_int("FHIP_GEMV_G", 0), tune_rpg = env_int("FHIP_GEMV_RPG", 0), tune_u = env_int("FHIP_GEMV_U", 0);
     GemvParams p;
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
@@ -594,7 +588,7 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     constexpr int MAXW = max_threads(M) / 64;
     if (p.S > MAXW) return fhip::set_error(FHIP_ERR_SHAPE, "matmul_q: cols %zu exceeds the %d this kernel covers", w->cols, MAXW * 2048);
     // Row groups per workgroup: fill the workgroup with waves.
-    int G = tune_g > 0 ? tune_g : MAXW / p.S;
+    int G = MAXW / p.S;
     if (G < 1) G = 1;
     while (G > 1 && p.S * G > MAXW) G--;
     p.stage = (size_t)M * w->cols * 4 <= 48 * 1024 ? 1 : 0;
@@ -603,11 +597,9 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     // few rows per wave so the one-time activation load is amortised.
     int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     if (p.sel.npairs > 1) cus = cus / p.sel.npairs > 0 ? cus / p.sel.npairs : 1;   // the pairs of an "_id" launch share the chip
-    int rpg = tune_rpg > 0 ? tune_rpg : (int)((out_rows + (size_t)cus * G - 1) / ((size_t)cus * G));
-    if (tune_rpg <= 0) {
-        if (rpg > 32) rpg = 32;
-        if (rpg < 1) rpg = 1;
-    }
+    int rpg = (int)((out_rows + (size_t)cus * G - 1) / ((size_t)cus * G));
+    if (rpg > 32) rpg = 32;
+    if (rpg < 1) rpg = 1;
     p.rpg = rpg;
     const size_t per_wg = (size_t)G * rpg;
     const size_t grid = (out_rows + per_wg - 1) / per_wg;
@@ -616,8 +608,7 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     dim3 block(64 * p.S * G);
     constexpr int U = rows_in_flight(M);
     const dim3 g3((unsigned)grid, (unsigned)p.sel.npairs);
-    if (tune_u == 2 && U != 2) hipLaunchKernelGGL((gemv_kernel<F, M, 2, SWIGLU>), g3, block, lds, s, p);
-    else hipLaunchKernelGGL((gemv_kernel<F, M, U, SWIGLU>), g3, block, lds, s, p);
+    hipLaunchKernelGGL((gemv_kernel<F, M, U, SWIGLU>), g3, block, lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
 }
 

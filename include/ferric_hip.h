@@ -297,6 +297,16 @@ int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_re
  * not thread-safe against concurrent launches). No counterpart in the reference. */
 int fhip_debug_generic_matvec(int on);
 
+/* Precision of the activations inside the streaming mat-vec kernels (fhip_matmul_q, _swiglu, fhip_ffn, the "_id" entry points,
+ * fhip_norm_matmul_q): per run of 32 (16 for Q6_K) columns the activations are held as block fixed point with a `bits`-bit
+ * significand at the run's largest magnitude, the weights exactly, the sums exactly, and everything above the sub-block in
+ * f32. bits = 16 (the default): dot products within about 1e-4 of the largest output, three orders of magnitude inside
+ * 1e-3 * ||w_row|| * ||x||. bits = 24: the significand of f32 itself, results within 1e-5 of the largest output (the bar of
+ * the reference's scalar kernels, crates/ferric-tensor/examples/q4_k.rs:54), 1-6 % slower. bits = 0 only queries. Returns the
+ * setting before the call (16 or 24), or FHIP_ERR_ARG. Process-wide; takes effect for launches enqueued afterwards, so do
+ * not change it while another thread enqueues. The reference has no such switch: its kernels multiply f32 by f32. */
+int fhip_matvec_precision(int bits);
+
 /* words[i] += delta for n device u32 words: advances the position word(s) at the end of a captured decode step. */
 int fhip_u32_add(uint32_t* d_words, size_t n, uint32_t delta, void* stream);
 

@@ -37,3 +37,37 @@ def golden():
 
 def bits(a):
     return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+# ---- precision of the streaming mat-vec's activations (fhip_matvec_precision): the tests of the mat-vec entry points run
+# once per setting. At 24 bits the dot products are held to the bar the reference's examples use for its scalar kernels
+# (1e-5 of the largest output, crates/ferric-tensor/examples/q4_k.rs:54); at 16 bits (the default) to 2e-4: a 16-bit
+# significand at the run maximum is 1.5e-5 of that maximum per activation, and the sum over a row measures 2e-5 .. 7e-5
+# of the largest output on these inputs. The north-star bound 1e-3 * ||w_row|| * ||x|| is asserted at both.
+_PRECISION = {"bits": 16}
+
+
+def dot_bar(scale=1.0):
+    return scale * (1e-5 if _PRECISION["bits"] == 24 else 2e-4)
+
+
+@pytest.fixture(params=[16, 24], ids=["x16", "x24"])
+def precision(request, F):
+    lib = F._lib.load()
+    before = lib.fhip_matvec_precision(request.param)
+    assert before in (16, 24)
+    _PRECISION["bits"] = request.param
+    yield request.param
+    lib.fhip_matvec_precision(before)
+    _PRECISION["bits"] = before
+
+
+@pytest.fixture
+def precision24(F):
+    """For tests that use the streaming mat-vec as the f32-grade side of a comparison."""
+    lib = F._lib.load()
+    before = lib.fhip_matvec_precision(24)
+    _PRECISION["bits"] = 24
+    yield
+    lib.fhip_matvec_precision(before)
+    _PRECISION["bits"] = before

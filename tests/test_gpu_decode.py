@@ -5,7 +5,7 @@ bit-exact."""
 import numpy as np
 import pytest
 
-from conftest import bits
+from conftest import bits, dot_bar
 
 pytestmark = pytest.mark.gpu
 Q8_0, Q4_K, Q6_K = 8, 12, 14
@@ -87,8 +87,10 @@ def test_rope_variants(F, X, D):
 
 def test_kv_append2_and_decode_attention(F, X, D):
     rng = np.random.default_rng(2)
+    # (14, 2, 64, [8192]): head_dim 64 with more than 64 splits of the key range (2 KV heads on 256 CUs), the case in which
+    # the combine kernel's thread count and its loop stride have to agree
     for nh, nkv, hd, lens in [(40, 8, 128, [1, 7, 64, 65, 1000]), (8, 8, 64, [3, 257]), (16, 2, 128, [130]), (6, 2, 64, [33]), (5, 1, 128, [2049]),
-                              (64, 8, 128, [4097])]:
+                              (64, 8, 128, [4097]), (14, 2, 64, [8192])]:
         cap = max(lens) + 3
         width = nkv * hd
         k = rng.standard_normal((cap, width)).astype(np.float32)
@@ -298,7 +300,7 @@ def test_post_processing_inside_the_attention_launch(F, X, D):
                                                  vc2.buf.ptr, cap, cap, 0, 0.0, ws.ptr, got.buf.ptr, None))
 
 
-def test_norm_fused_into_the_matvec(F, X, D, O):
+def test_norm_fused_into_the_matvec(F, X, D, O, precision):
     """fhip_norm_matmul_q against rmsnorm / add_rmsnorm followed by the mat-vec: the residual sum bit-exact, the product
     within the dot-product bound of the unfused pair (the sum of squares is added in another order: ~1e-7 on the scale),
     on shapes the streaming kernel takes (fused) and on ones it does not (the two steps run apart)."""
@@ -329,10 +331,10 @@ def test_norm_fused_into_the_matvec(F, X, D, O):
             y64, wn = O.matmul_f64(h64.astype(np.float32), raw, ty, rows, cols)
             if swiglu:
                 y64 = D.silu_mul(y64, out_rows)
-                assert close(y.to_vec(), y64, 2e-5), (ty, rows, cols)
+                assert close(y.to_vec(), y64, dot_bar(2)), (ty, rows, cols)
             else:
                 assert (np.abs(y.to_vec() - y64[0]) <= 1e-3 * wn * np.linalg.norm(h64)).all()
-                assert close(y.to_vec(), y64, 1e-5), (ty, rows, cols)
+                assert close(y.to_vec(), y64, dot_bar()), (ty, rows, cols)
             assert close(y.to_vec(), y_ref, 2e-5)
     with pytest.raises(F._lib.FerricHipError, match="x_out must not be x"):
         F._lib.check(lib.fhip_norm_matmul_q(w.handle, xt.buf.ptr, rt.buf.ptr, nt.buf.ptr, 1e-6, xt.buf.ptr, hs.buf.ptr, 0, y.buf.ptr, None))
@@ -362,7 +364,7 @@ def _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, qk_norm):
 
 
 @pytest.mark.parametrize("qk_norm,fuse_norm,fuse_attn", [(True, True, True), (False, True, True), (True, False, False), (True, True, False)])
-def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, X, O, D, qk_norm, fuse_norm, fuse_attn):
+def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, X, O, D, qk_norm, fuse_norm, fuse_attn, precision):
     rng = np.random.default_rng(4)
     n_layer, d, nh, nkv, hd, n_ff, steps = 3, 1024, 8, 2, 128, 1536, 6
     cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6)
@@ -383,9 +385,9 @@ def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, 
         dec.set_input(xs[pos])
         dec.step()
         eager.append(dec.hidden())
-        # <= 2e-4 of the largest hidden value: three layers of quantized dots (each within 1e-5 of its largest output)
-        # feeding norms, attention and the next projections
-        assert close(eager[-1], want[pos], 2e-4), pos
+        # <= 20 times the bar of one dot product, of the largest hidden value: three layers of quantized dots feeding
+        # norms, attention and the next projections
+        assert close(eager[-1], want[pos], dot_bar(20)), pos
     assert dec.caches[0].len == steps
     # the same steps as one captured graph, replayed with host work and synchronisation between replays
     dec.set_pos(0)
@@ -408,4 +410,4 @@ def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, 
     dec2.step()
     assert np.array_equal(bits(dec2.hidden()), bits(eager[0]))
     head = O.deq_raw(head_raw, 300 * d, Q6_K).reshape(300, d).astype(np.float64)
-    assert close(dec2.logits.to_vec(stream), D.rmsnorm(want[0], onorm, 1e-6) @ head.T, 2e-4)
+    assert close(dec2.logits.to_vec(stream), D.rmsnorm(want[0], onorm, 1e-6) @ head.T, dot_bar(20))

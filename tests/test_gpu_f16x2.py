@@ -13,7 +13,8 @@ of f16 (22 significant bits). Bars, against the oracle's dequantized weights in 
 import numpy as np
 import pytest
 
-pytestmark = pytest.mark.gpu
+# the f32 mat-vec path is the other side of most comparisons here: it runs with 24-bit activations
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("precision24")]
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 TIGHT = 2.5e-7
 
