@@ -7,7 +7,9 @@ Headline workload (the second of the benchmark configurations): Q4_K GEMV, W 512
 x f32[5120], batch 1. One "step" is one GEMV. Steps rotate over 64 distinct copies of the weight
 (944 MB, larger than the 256 MB Infinity Cache) so every step streams its weight bytes from HBM;
 the same loop over ONE copy is reported as the cache-resident ("warm") figure beside it.
-All K steps are recorded into one HIP graph on one stream and timed with HIP events on that stream.
+The K steps are recorded into HIP graphs on one stream (as many graphs of K launches as it takes to walk over all copies)
+and timed with HIP events on that stream: a batch replays the graphs back to back until at least 1024 launches ran, the
+figure is the median per step over 9 batches (so --steps 20 and --steps 4096 give the same number).
 
 Prints ONE JSON line. `value` = algorithmic bytes per step (weights + x + y) * K / elapsed, in GB/s.
 Also measured in the same run and carried in the line: the 64-layer decode weight sweep, the Q4_K_M FFN block at
@@ -26,10 +28,18 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
-# HBM bytes per launch of the headline kernel from hardware counters (FETCH_SIZE * 1.99976 + WRITE_SIZE * 1.0, both
-# calibrated on a 256 MiB copy); source and commands: profiles/gemv_hbm_traffic_pmc.txt
-Q4K_5120_TRAFFIC_BYTES = 15098461
 Q8_0, Q4_K, Q6_K = 8, 12, 14
+# HBM bytes per launch of the headline kernel from hardware counters: the figure, the commit it was measured on and the
+# commands are in this file, written beside the counter summary it was worked out from
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "gemv_q4k_5120x5120_hbm_traffic.json")
+
+
+def headline_traffic():
+    try:
+        with open(TRAFFIC_JSON) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return None
 
 
 def log(*a):
@@ -75,15 +85,37 @@ def replicate(F, lib, check, host_bytes, ncopy):
     return buf
 
 
-def gemv_graph(F, lib, check, stream, weights, x, y, steps, swiglu=False):
+def gemv_graph(F, lib, check, stream, weights, x, y, steps, swiglu=False, first=0):
     g = F.Graph.begin(stream)
     fn = lib.fhip_matmul_q_swiglu if swiglu else lib.fhip_matmul_q
     for i in range(steps):
-        check(fn(weights[i % len(weights)].handle, x.buf.ptr, x.shape[0], y.buf.ptr, stream.handle))
+        check(fn(weights[(first + i) % len(weights)].handle, x.buf.ptr, x.shape[0], y.buf.ptr, stream.handle))
     return g.end()
 
 
-def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed, x_seed, ncopy, cold_only=False):
+def time_per_launch(timer, graphs, launches_per_graph, min_launches=1024, batches=9):
+    """Median over `batches` batches of the time per launch. A batch replays the graphs round-robin, back to back inside one
+    event pair, often enough for at least `min_launches` launches: a single short graph (20 launches are 0.1 ms) would be
+    timed with the graph's start-up and the clock ramp in it."""
+    reps = max(1, -(-min_launches // (launches_per_graph * len(graphs))))
+
+    def batch():
+        for _ in range(reps):
+            for g in graphs:
+                g.launch()
+    batch()
+    ts = sorted(timer.time_ms(batch) for _ in range(batches))
+    return ts[len(ts) // 2] / (reps * len(graphs) * launches_per_graph)
+
+
+def rotating_graphs(make, steps, ncopy):
+    """Graphs of `steps` launches each that together walk over all `ncopy` weight copies in order, so that replaying them
+    round-robin never returns to a copy before every other copy has been read."""
+    n = 1 if steps >= ncopy else -(-ncopy // steps)
+    return [make(j * steps) for j in range(n)]
+
+
+def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed, x_seed, ncopy, cold_only=False, with_reader=False):
     from ferric_amd.synth import synth_weights
     nbytes = weight_bytes(ty, rows, cols)
     host = synth_weights(ty, rows, cols, seed)
@@ -93,12 +125,21 @@ def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed
     y = F.Tensor.empty((1, rows))
     alg = nbytes + 4 * cols + 4 * rows
     out = {}
+    gemv_graph(F, lib, check, stream, ws, x, y, max(warmup, 1)).launch()          # the untimed warm-up steps
     for name, wl in ((("cold", ws),) if cold_only else (("cold", ws), ("warm", ws[:1]))):
-        gw = gemv_graph(F, lib, check, stream, wl, x, y, max(warmup, 1))
-        g = gemv_graph(F, lib, check, stream, wl, x, y, steps)
-        gw.launch()
-        ms = min(timer.time_ms(g.launch) for _ in range(3)) if name == "warm" else timer.time_ms(g.launch)
-        out[name] = {"ms_per_step": ms / steps, "GBps": alg * steps / (ms * 1e-3) / 1e9}
+        graphs = rotating_graphs(lambda first: gemv_graph(F, lib, check, stream, wl, x, y, steps, first=first), steps, len(wl))
+        ms = time_per_launch(timer, graphs, steps)
+        out[name] = {"ms_per_step": ms, "GBps": alg / (ms * 1e-3) / 1e9}
+    if with_reader:
+        # the same bytes through a kernel that only reads them, same rotation, same timing: what a perfect reader gets
+        sink = F.DeviceBuffer(256)
+
+        def reader_graph(first):
+            g = F.Graph.begin(stream)
+            for i in range(steps):
+                check(lib.fhip_debug_read_probe(C.c_void_p(buf.ptr.value + ((first + i) % ncopy) * nbytes), nbytes, sink.ptr, stream.handle))
+            return g.end()
+        out["reader_ms"] = time_per_launch(timer, rotating_graphs(reader_graph, steps, ncopy), steps)
     return out, alg, nbytes
 
 
@@ -251,7 +292,7 @@ def bench_gguf(F, lib, check, n_tensors=8, rows=11008, cols=5120):
             "note": "page-cache-resident file, pageable mapping -> hipMemcpy; host I/O and PCIe bound"}
 
 
-def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
+def bench_sweep(F, lib, check, stream, timer, tokens=4, layers=64):
     """The decode weight sweep: per layer fused QKV 5120->7168, O 5120->5120, fused gate+up 5120->34816 (+SwiGLU), all Q4_K,
     down 17408->5120 Q6_K; lm_head 5120->151936 Q6_K. One stream, one graph of layers*4+1 launches."""
     from ferric_amd.synth import synth_weights
@@ -281,8 +322,9 @@ def bench_sweep(F, lib, check, stream, timer, tokens=8, layers=64):
     check(lib.fhip_matmul_q(head.handle, x.buf.ptr, 1, logits.buf.ptr, s))
     g.end()
     g.launch()
-    ms = timer.time_ms(lambda: [g.launch() for _ in range(tokens)]) / tokens
-    return {"ms_per_token": ms, "GBps": total / (ms * 1e-3) / 1e9, "frac_of_peak": total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+    ts = sorted(timer.time_ms(lambda: [g.launch() for _ in range(tokens)]) / tokens for _ in range(5))
+    ms = ts[len(ts) // 2]
+    return {"ms_per_token": ms, "ms_per_token_min_max": [ts[0], ts[-1]], "GBps": total / (ms * 1e-3) / 1e9, "frac_of_peak": total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
             "weight_bytes": total, "layers": layers, "launches_per_token": layers * 4 + 1,
             "inputs": "fixed N(0,1) activations per op (outputs are not fed forward, so values stay finite); "
                       "ops still execute in stream order"}
@@ -485,7 +527,11 @@ def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
     from ferric_amd.synth import synth_weights
     from oracle import oracle as O
     O.build()
-    threads = max(1, min(16, os.cpu_count() or 1))
+    try:
+        avail = len(os.sched_getaffinity(0))
+    except AttributeError:
+        avail = os.cpu_count() or 1
+    threads = max(1, min(16, avail))          # the GPU box's CPU share is 16 threads, whatever the host shows
     w = synth_weights(Q4_K, rows, cols, 1)
     x = np.random.default_rng(x_seed).standard_normal(cols).astype(np.float32)
     O.matmul_cpu(x, w, Q4_K, rows, cols, threads=threads)  # warm-up, excluded
@@ -498,7 +544,7 @@ def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
             break
     med = float(np.median(times))
     alg = w.size + 4 * cols + 4 * rows
-    return {"value": alg / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+    return {"value": alg / med / 1e9, "unit": "GB/s", "cores": threads, "host_logical_cpus": os.cpu_count(), "kind": "port",
             "sample": f"{len(times)} full Q4_K 5120x5120 batch-1 mat-vecs (dequantize row, then sequential f32 dot; "
                       f"contiguous row spans over {threads} threads), median {med * 1e3:.2f} ms each"}
 
@@ -506,8 +552,8 @@ def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4096)
-    ap.add_argument("--warmup", type=int, default=256)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-ffn", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
@@ -554,12 +600,14 @@ def main():
         return
     log("[bench] Q4_K GEMV 5120x5120 ...")
     c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
-                                 cold_only=args.headline_only)
+                                 cold_only=args.headline_only, with_reader=True)
     if args.headline_only:
         args.no_q8 = args.no_ffn = args.no_prefill = args.no_moe = args.no_sweep = args.no_cpu = args.no_decode = True
         c2["warm"] = None
     ms_step = c2["cold"]["ms_per_step"]
     value = c2["cold"]["GBps"]
+    traffic = headline_traffic()
+    bits = lib.fhip_matvec_precision(0)
     line = {
         "metric": "Q4_K GEMV HBM GB/s (% of 8 TB/s) at batch 1; decode-step weight-sweep ms",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -571,9 +619,16 @@ def main():
         "pct_of_peak": 100.0 * value / HBM_PEAK_GBPS,
         "warm_single_copy": c2["warm"],
         "roofline": {"bound": "hbm", "achieved": alg / (ms_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": Q4K_5120_TRAFFIC_BYTES,
-                     "kernel": "gemv_stream_kernel<Q4K, M=1, U=3, plain>", "algorithmic_bytes_per_launch": alg,
-                     "launch_us": ms_step * 1e3, "empty_launch_us": launch_floor_us(F, lib, check, stream, timer)},
+                     "frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": traffic["traffic_bytes"] if traffic else None, "traffic_source": traffic,
+                     "kernel": "gemv_stream_kernel<Q4K, M=1, plain>", "algorithmic_bytes_per_launch": alg,
+                     "launch_us": ms_step * 1e3,
+                     # the same 14.7 MB through a kernel that only reads them (same rotation, same timing), and a launch
+                     # that does nothing: what this box leaves a single cold launch of this size
+                     "reader_floor_us": c2["reader_ms"] * 1e3, "frac_of_reader": c2["reader_ms"] / ms_step,
+                     "empty_launch_us": launch_floor_us(F, lib, check, stream, timer)},
+        "activation_bits": bits,
+        "timing": "median of 9 batches; a batch = the K-step graph(s) replayed back to back until >= 1024 launches, one HIP event pair",
     }
     if not args.no_q8:
         log("[bench] Q8_0 GEMV 4096x4096 ...")
@@ -592,10 +647,10 @@ def main():
         log("[bench] routed-expert block of an MoE decode layer ...")
         line["moe_routed_experts_q4k_q6k"] = bench_moe(F, lib, check, stream, timer)
     if not args.no_moe:
-        log("[bench] Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / IQ4_XS / MXFP4 GEMV 5120x5120 (generic kernel) ...")
+        log("[bench] Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / IQ4_XS / MXFP4 GEMV 5120x5120 ...")
         other = {}
         for name, ty in (("q5_k", 13), ("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("iq4_nl", 20), ("iq4_xs", 23), ("mxfp4", 39)):
-            r, a, nb = bench_gemv(F, lib, check, stream, timer, ty, rows, cols, 1024, 64, seed=20 + ty, x_seed=2, ncopy=48)
+            r, a, nb = bench_gemv(F, lib, check, stream, timer, ty, rows, cols, 64, 64, seed=20 + ty, x_seed=2, ncopy=48)
             other[name] = {"cold_us": r["cold"]["ms_per_step"] * 1e3, "cold_GBps": r["cold"]["GBps"],
                            "warm_us": r["warm"]["ms_per_step"] * 1e3, "algorithmic_bytes": a}
         line["other_formats_gemv_5120"] = other

@@ -27,6 +27,7 @@ UNITS = {
     "gemm_mfma.hip": [],
     "gemm_f16x2.hip": [],
     "moe.hip": [],
+    "probe.hip": [],
     "decode_ops.hip": [],
     "gguf.hip": [],
 }

@@ -573,6 +573,14 @@ int fhip_debug_generic_matvec(int on) {
     return FHIP_OK;
 }
 
+int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!d_src || !d_sink) return set_error(FHIP_ERR_ARG, "fhip_debug_read_probe: NULL pointer");
+    if (((uintptr_t)d_src & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_debug_read_probe: src must be 16-byte aligned");
+    return fhip::launch_read_probe(d_src, nbytes, d_sink, (hipStream_t)stream);
+}
+
 int fhip_matvec_precision(int bits) {
     const int before = fhip::g_planes == 3 ? 24 : 16;
     if (bits == 0) return before;

@@ -95,6 +95,9 @@ int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t o
 int launch_gemv_generic_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu,
                             const SelParams& sel, hipStream_t s);
 
+// probe.hip: reads nbytes (a multiple of 16 is read) and stores nothing to speak of
+int launch_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, hipStream_t s);
+
 // moe.hip
 int launch_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t ne, int k, int sigmoid, float scale, int norm,
                     float* d_out, hipStream_t s);

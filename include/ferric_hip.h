@@ -297,6 +297,12 @@ int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_re
  * not thread-safe against concurrent launches). No counterpart in the reference. */
 int fhip_debug_generic_matvec(int on);
 
+/* Measurement aid: one launch that reads nbytes at d_src (16-byte loads over the whole chip) and does nothing else; d_sink is
+ * one device word that is practically never written. Timed beside a mat-vec of the same size it gives the time a perfect reader
+ * needs for those bytes on this device. No counterpart in the reference (its matvec_roofline example prints bytes / time of the
+ * kernel itself, crates/ferric-tensor/examples/matvec_roofline.rs:85-100). */
+int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, void* stream);
+
 /* Precision of the activations inside the streaming mat-vec kernels (fhip_matmul_q, _swiglu, fhip_ffn, the "_id" entry points,
  * fhip_norm_matmul_q): per run of 32 (16 for Q6_K) columns the activations are held as block fixed point with a `bits`-bit
  * significand at the run's largest magnitude, the weights exactly, the sums exactly, and everything above the sub-block in
