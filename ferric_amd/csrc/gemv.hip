@@ -35,8 +35,8 @@
 // rows of 16-byte loads in flight per wave; weight loads for the first rows are issued before the
 // activations are touched, so the two latencies overlap.
 //
-// Activations that block fixed point cannot hold (a run with a NaN or an infinity, a run whose sum overflows,
-// a run whose largest magnitude is below 2^-100) are marked by a NaN run scale; a lane that owns such a run
+// Activations that block fixed point cannot hold (a run with a NaN or an infinity, a run whose largest magnitude is
+// above 2^96 or below 2^-100) are marked by a NaN run scale; a lane that owns such a run
 // computes its share of every row element by element in f32 from the raw activations and the exactly
 // dequantised weights, which is what the reference's CPU path does (crates/ferric-tensor/src/cpu_simd.rs:57-72,
 // crates/ferric-gguf/src/lib.rs:497 then a dense dot): NaN stays NaN, inf * w is +-inf, inf * 0 is NaN.
@@ -67,6 +67,7 @@ static_assert(NP == 2 || NP == 3, "two or three activation planes");
 // the quantiser clamps.
 constexpr float QMAX = NP == 2 ? 32639.0f : 8355711.0f;
 constexpr float TINY_RUN = 7.888609052210118e-31f;   // 2^-100: below this QMAX / amax leaves the f32 range's comfortable part
+constexpr float HUGE_RUN = 7.922816251426434e28f;    // 2^96
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -666,9 +667,10 @@ __device__ __forceinline__ void quantize8(const float (&v)[8], uint32_t (&pl)[NP
         amax = fmaxf(amax, dpp_f<DPP_XOR2>(amax));
         sum += dpp_f<DPP_XOR2>(sum);
     }
-    // not representable in block fixed point: non-finite members, a sum beyond the f32 range, or a run so small that
-    // QMAX / amax would overflow
-    const bool special = !(fabsf(sum) <= 3.4028234663852886e38f) || (amax < TINY_RUN && amax > 0.f);
+    // not representable in block fixed point: non-finite members (their sum is not finite either), a run so large that a
+    // format's offset term (up to 128 times the run's sum) could leave the f32 range where the element-wise products do not,
+    // or a run so small that QMAX / amax would overflow
+    const bool special = !(fabsf(sum) <= 3.4028234663852886e38f) || amax > HUGE_RUN || (amax < TINY_RUN && amax > 0.f);
     const float inv = amax > 0.f ? QMAX * __builtin_amdgcn_rcpf(amax) : 0.f;
     uint32_t t[8];
     if constexpr (NP == 2) {

@@ -315,3 +315,44 @@ def test_empty_shapes(F):
     assert F.matvec_q8_0(np.zeros(0, np.float32), np.zeros(0, np.uint8), 0, 0).size == 0
     y = F.matvec_q8_0(np.zeros(0, np.float32), np.zeros(0, np.uint8), 5, 0)
     assert y.shape == (5,) and not y.any()
+
+
+# ---------------------------------------------------------------- activations block fixed point cannot hold
+
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q6_K, 13, 2, 3, 6, 7, 20, 23, 39],
+                         ids=["q8_0", "q4_k", "q6_k", "q5_k", "q4_0", "q4_1", "q5_0", "q5_1", "iq4_nl", "iq4_xs", "mxfp4"])
+def test_non_finite_and_tiny_activations_give_what_the_f32_dot_gives(F, O, ty):
+    """crates/ferric-tensor/src/cpu_simd.rs:57-72 and the dequantize-then-dot path sum x[k] * w[k] in f32: a NaN activation
+    makes the row NaN, an infinite one +-inf by the weight's sign (NaN against a zero weight, NaN when both signs meet), and
+    neither leaks into the other rows of a batch. Runs of activations far below the f32 normal range's middle still count."""
+    from ferric_amd.synth import synth_weights
+    rows, cols = 96, 2048
+    raw = synth_weights(ty, rows, cols, 21).copy()
+    if ty == Q4_K:                                    # dmin = 0: no min term to carry the NaN by accident
+        raw.reshape(-1, 144)[:, 2:4] = 0
+        raw.reshape(-1, 144)[::3, 16:24] = 0          # and some exactly-zero weights under the infinite activation
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((6, cols)).astype(np.float32)
+    x[0, 1000] = np.nan
+    x[1, 37] = np.inf
+    x[2, 37] = -np.inf
+    x[2, 1999] = np.inf
+    x[3, 512:640] *= np.float32(1e-36)                # four runs near the bottom of the normal range
+    x[4, 0:32] = np.float32(1e30)                     # a run above 2^96: 128 times its sum is near the end of the f32 range
+    # row 5 stays ordinary
+    qm = F.QMatrix.from_bytes(raw, ty, rows, cols)
+    with np.errstate(all="ignore"):
+        want = O.matmul_cpu(x, raw, ty, rows, cols)
+        y64, wn = O.matmul_f64(x, raw, ty, rows, cols)
+    for sl in (slice(0, 6), slice(0, 1), slice(1, 3), slice(2, 6)):      # batches of 6, 1, 2, 4 rows: every pass width
+        xs = x[sl]
+        y = F.Tensor.from_vec(xs, xs.shape).matmul_q(qm).to_vec().reshape(xs.shape[0], rows)
+        w_, y_ = want[sl], y64[sl]
+        with np.errstate(all="ignore"):
+            bound = 1e-3 * wn[None, :] * np.linalg.norm(xs.astype(np.float64), axis=1)[:, None]
+        for i, r in enumerate(range(sl.start, sl.stop)):
+            assert np.array_equal(np.isnan(y[i]), np.isnan(w_[i])), (ty, r)
+            assert np.array_equal(np.isposinf(y[i]), np.isposinf(w_[i])) and np.array_equal(np.isneginf(y[i]), np.isneginf(w_[i])), (ty, r)
+            fin = np.isfinite(w_[i])
+            assert (np.abs(y[i] - y_[i])[fin] <= bound[i][fin] + 1e-30).all(), (ty, r)
+    assert np.isnan(want[0]).all() and not np.isfinite(want[1]).any() and np.isfinite(want[3:6]).all()
