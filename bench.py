@@ -163,8 +163,14 @@ def bench_q80_batch(F, lib, check, stream, timer, rows=4096, cols=4096, batch=8,
         return min(timer.time_ms(g.launch) for _ in range(3)) / ncopy * 1e3
 
     one_pass = timed(lambda w: check(lib.fhip_matmul_q_f16x2(w.handle, x.buf.ptr, batch, y.buf.ptr, scratch.ptr, stream.handle)))
+    # the drop-in entry point takes the same kernels for this batch, out of the library's workspace
+    check(lib.fhip_workspace_reserve(stream.handle, lib.fhip_workspace_bytes(ws[0].handle, None, batch)))
+    drop_in = timed(lambda w: check(lib.fhip_matmul_q(w.handle, x.buf.ptr, batch, y.buf.ptr, stream.handle)))
+    before = lib.fhip_batch_policy(1)                  # FHIP_BATCH_F32_MATVEC
     per_row = timed(lambda w: check(lib.fhip_matmul_q(w.handle, x.buf.ptr, batch, y.buf.ptr, stream.handle)))
-    return {"batch": batch, "f16x2_us": one_pass, "f16x2_weight_GBps": nbytes / one_pass / 1e3, "f32_matvec_us": per_row}
+    lib.fhip_batch_policy(before)
+    return {"batch": batch, "matmul_q_us": drop_in, "matmul_q_weight_GBps": nbytes / drop_in / 1e3, "f16x2_us": one_pass,
+            "f32_matvec_policy_us": per_row}
 
 
 def launch_floor_us(F, lib, check, stream, timer, n=2048):
@@ -209,9 +215,17 @@ def bench_ffn(F, lib, check, stream, timer, batches, reps=20, ncopy=4):
     for b in batches:
         x = F.Tensor.from_vec(np.random.default_rng(5).standard_normal((b, n_embd)).astype(np.float32), (b, n_embd))
         ws, y = F.Tensor.empty((b, n_ff)), F.Tensor.empty((b, n_embd))
+        # fhip_ffn, the drop-in entry point: the mat-vec kernels for one and two rows, the one-pass f16 hi/lo kernels from three
+        # rows on (out of the library's workspace, reserved here because a capturing stream cannot allocate)
+        check(lib.fhip_workspace_reserve(stream.handle, lib.fhip_workspace_bytes(gus[0].handle, dns[0].handle, b)))
         f32 = lambda gu, dn: check(lib.fhip_ffn(gu.handle, dn.handle, x.buf.ptr, b, y.buf.ptr, ws.buf.ptr, stream.handle))
         res[str(b)] = entry(timed(f32, ncopy), b)
         res[str(b)]["warm_one_copy_ms"] = timed(f32, 1)
+        res[str(b)]["path"] = "streaming mat-vec" if b <= 2 else "one-pass f16 hi/lo matrix-core kernels"
+        if b > 2:
+            before = lib.fhip_batch_policy(1)          # FHIP_BATCH_F32_MATVEC: two rows per pass over the weights
+            res[str(b)]["f32_matvec_policy"] = entry(timed(f32, ncopy), b)
+            lib.fhip_batch_policy(before)
         # the same block through the matrix-core entry point (bf16 operands, f32 accumulate): one pass over
         # the weights for the whole batch
         wsb = F.DeviceBuffer(max(256, lib.fhip_ffn_coop_ws_bytes(gus[0].handle, dns[0].handle, b)))

@@ -102,6 +102,10 @@ SYMBOLS = {
     "fhip_norm_matmul_q": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, C.c_int, _vp, _vp]),
     "fhip_debug_generic_matvec": (C.c_int, [C.c_int]),
     "fhip_matvec_precision": (C.c_int, [C.c_int]),
+    "fhip_batch_policy": (C.c_int, [C.c_int]),
+    "fhip_workspace_bytes": (C.c_size_t, [_vp, _vp, C.c_size_t]),
+    "fhip_workspace_reserve": (C.c_int, [_vp, C.c_size_t]),
+    "fhip_workspace_release": (None, [_vp]),
     "fhip_debug_read_probe": (C.c_int, [_vp, _sz, _vp, _vp]),
     "fhip_u32_add": (C.c_int, [_vp, _sz, _u32, _vp]),
     "fhip_matvec_q8_0_host": (C.c_int, [_vp, _vp, _sz, _sz, _sz, _vp]),

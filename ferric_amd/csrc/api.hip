@@ -6,6 +6,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+#include <vector>
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -107,6 +110,82 @@ void gemv_force_generic(bool on) {
 using fhip::check_hip;
 using fhip::set_error;
 
+namespace {
+
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+// ---- the library's own workspace, one per stream -------------------------------------------------------------------------
+// The one-pass small-batch kernels need a few megabytes of device memory beside their operands (prepared activation rows,
+// the gate|up intermediate). The drop-in entry points (fhip_matmul_q, fhip_matmul_q_swiglu, fhip_ffn) have no argument for
+// it, so the library keeps a buffer per stream: work on one stream is ordered, so calls there can share it. It only ever
+// grows, to the next power of two, and a buffer that was outgrown stays allocated until fhip_workspace_release: a graph
+// captured earlier may still name it. Growing means hipMalloc, which a capturing stream does not allow.
+struct StreamWs { hipStream_t s; void* cur; size_t n; std::vector<void*> retired; };
+std::mutex g_ws_mu;
+std::vector<StreamWs> g_ws;
+
+int lib_workspace(hipStream_t s, size_t need, void** out, const char* who) {
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    StreamWs* e = nullptr;
+    for (auto& w : g_ws) if (w.s == s) e = &w;
+    if (e && e->n >= need) { *out = e->cur; return FHIP_OK; }
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) != hipSuccess) (void)hipGetLastError();
+    if (st != hipStreamCaptureStatusNone)
+        return set_error(FHIP_ERR_ARG, "%s: the library workspace of this stream has to grow to %zu bytes, which a capturing stream does not "
+                         "allow: call fhip_workspace_reserve(stream, %zu) before the capture begins", who, need, need);
+    size_t n = 1 << 20;
+    while (n < need) n <<= 1;
+    void* p = nullptr;
+    int rc = check_hip(hipMalloc(&p, n), "hipMalloc (library workspace)");
+    if (rc) return rc;
+    if (!e) { g_ws.push_back(StreamWs{s, nullptr, 0, {}}); e = &g_ws.back(); }
+    if (e->cur) e->retired.push_back(e->cur);
+    e->cur = p; e->n = n;
+    *out = p;
+    return FHIP_OK;
+}
+
+void release_workspace(hipStream_t s) {
+    std::lock_guard<std::mutex> lock(g_ws_mu);
+    for (size_t i = 0; i < g_ws.size(); i++) {
+        if (g_ws[i].s != s) continue;
+        (void)hipStreamSynchronize(s);
+        if (g_ws[i].cur) (void)hipFree(g_ws[i].cur);
+        for (void* p : g_ws[i].retired) (void)hipFree(p);
+        g_ws.erase(g_ws.begin() + i);
+        return;
+    }
+}
+
+// ---- which kernel a batch takes ---------------------------------------------------------------------------------------------
+// One or two activation rows go through the streaming mat-vec (one pass over the weights serves two rows). From three rows on
+// (five for Q8_0) the f16 hi/lo matrix-core kernels read the weights once for up to 32 (Q8_0: 16) rows; longer batches are cut
+// into such groups. FHIP_BATCH_F32_MATVEC keeps every batch on the mat-vec kernel: a row then has the same bits whatever batch
+// it is part of.
+int g_batch_policy = FHIP_BATCH_AUTO;
+
+size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32; }
+bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
+    if (g_batch_policy != FHIP_BATCH_AUTO) return false;
+    if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0) return false;
+    if (rows_x < (w->type == FHIP_Q8_0 ? 5u : 3u)) return false;
+    return fhip::gemm_f16x2_supports(w, rows_x < f16x2_group(w) ? rows_x : f16x2_group(w));
+}
+
+// y [t, w->rows] = x [t, cols] W^T for t rows of one group; ws: f16x2_matmul_ws(w, t) bytes
+size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) { return align256(fhip::gemm_f16x2_xp_bytes(w, t)) + align256(fhip::gemm_f16x2_aux_bytes()); }
+int f16x2_matmul(const fhip_weight* w, const float* d_x, size_t t, bool swiglu_in, float* d_y, void* d_ws, hipStream_t s) {
+    uint16_t* xp = (uint16_t*)d_ws;
+    float* rs = (float*)((uint8_t*)d_ws + align256(fhip::gemm_f16x2_xp_bytes(w, t)));
+    const bool clr = fhip::gemm_f16x2_adds_into_y(w, t);   // then the split clears y on the side
+    int rc = fhip::launch_xsplit_f16(w, d_x, t, swiglu_in, xp, rs, s, clr ? d_y : nullptr, clr ? t * w->rows : 0);
+    if (rc) return rc;
+    return fhip::launch_gemm_f16x2(w, xp, rs, t, d_y, s, clr);
+}
+
+}  // namespace
+
 extern "C" {
 
 int fhip_init(int device) {
@@ -194,7 +273,11 @@ int fhip_stream_create(void** s) {
     *s = rc ? nullptr : (void*)st;
     return rc;
 }
-int fhip_stream_destroy(void* s) { return s ? check_hip(hipStreamDestroy((hipStream_t)s), "hipStreamDestroy") : FHIP_OK; }
+int fhip_stream_destroy(void* s) {
+    if (!s) return FHIP_OK;
+    release_workspace((hipStream_t)s);   // the library's buffer for this stream goes with it
+    return check_hip(hipStreamDestroy((hipStream_t)s), "hipStreamDestroy");
+}
 int fhip_stream_sync(void* s) { return check_hip(hipStreamSynchronize((hipStream_t)s), "hipStreamSynchronize"); }
 int fhip_event_create(void** e) {
     if (!e) return set_error(FHIP_ERR_ARG, "fhip_event_create: NULL output");
@@ -389,7 +472,18 @@ int fhip_matmul_q(const fhip_weight* w, const float* d_x, size_t rows_x, float* 
     if (rows_x == 0 || w->rows == 0) return FHIP_OK;
     if (!d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_matmul_q: NULL pointer");
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q: x must be 16-byte aligned");
-    return fhip::launch_gemv(w, d_x, rows_x, d_y, 0, (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    if (!takes_f16x2(w, rows_x)) return fhip::launch_gemv(w, d_x, rows_x, d_y, 0, s);
+    const size_t grp = f16x2_group(w);
+    void* ws = nullptr;
+    if ((rc = lib_workspace(s, f16x2_matmul_ws(w, rows_x < grp ? rows_x : grp), &ws, "fhip_matmul_q"))) return rc;
+    for (size_t m0 = 0; m0 < rows_x; m0 += grp) {
+        const size_t t = rows_x - m0 < grp ? rows_x - m0 : grp;
+        if (takes_f16x2(w, t)) rc = f16x2_matmul(w, d_x + m0 * w->cols, t, false, d_y + m0 * w->rows, ws, s);
+        else rc = fhip::launch_gemv(w, d_x + m0 * w->cols, t, d_y + m0 * w->rows, 0, s);   // a last group of one or two rows
+        if (rc) return rc;
+    }
+    return FHIP_OK;
 }
 
 int fhip_matmul_q_swiglu(const fhip_weight* gu, const float* d_x, size_t rows_x, float* d_y, void* stream) {
@@ -401,7 +495,22 @@ int fhip_matmul_q_swiglu(const fhip_weight* gu, const float* d_x, size_t rows_x,
     if (rows_x == 0 || gu->rows == 0) return FHIP_OK;
     if (!d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu: NULL pointer");
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu: x must be 16-byte aligned");
-    return fhip::launch_gemv(gu, d_x, rows_x, d_y, gu->rows / 2, (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    const size_t n_ff = gu->rows / 2;
+    if (!takes_f16x2(gu, rows_x)) return fhip::launch_gemv(gu, d_x, rows_x, d_y, n_ff, s);
+    // gate|up for the group in one pass into the workspace, then the reference's un-fused SwiGLU over it
+    const size_t grp = f16x2_group(gu), t0 = rows_x < grp ? rows_x : grp;
+    const size_t mm = f16x2_matmul_ws(gu, t0);
+    void* ws = nullptr;
+    if ((rc = lib_workspace(s, mm + align256(t0 * gu->rows * sizeof(float)), &ws, "fhip_matmul_q_swiglu"))) return rc;
+    float* g = (float*)((uint8_t*)ws + mm);
+    for (size_t m0 = 0; m0 < rows_x; m0 += grp) {
+        const size_t t = rows_x - m0 < grp ? rows_x - m0 : grp;
+        if (!takes_f16x2(gu, t)) { rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, d_y + m0 * n_ff, n_ff, s); }
+        else if (!(rc = f16x2_matmul(gu, d_x + m0 * gu->cols, t, false, g, ws, s))) rc = fhip::launch_swiglu(g, t, n_ff, d_y + m0 * n_ff, s);
+        if (rc) return rc;
+    }
+    return FHIP_OK;
 }
 
 int fhip_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, void* stream) {
@@ -428,9 +537,59 @@ int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, s
         // [rows_x, 2 n_ff] intermediate then also lives in d_ws, which this path needs 3x larger.
         return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "fhip_ffn: gate_up must be Q4_K or Q6_K");
     }
-    if ((rc = fhip::launch_gemv(gu, d_x, rows_x, d_ws, n_ff, (hipStream_t)stream))) return rc;
-    return fhip::launch_gemv(down, d_ws, rows_x, d_y, 0, (hipStream_t)stream);
+    hipStream_t s = (hipStream_t)stream;
+    if (!takes_f16x2(gu, rows_x) || !takes_f16x2(down, rows_x)) {
+        if ((rc = fhip::launch_gemv(gu, d_x, rows_x, d_ws, n_ff, s))) return rc;
+        return fhip::launch_gemv(down, d_ws, rows_x, d_y, 0, s);
+    }
+    // groups of up to 32 rows, each one pass over gate|up and one over down; SwiGLU happens while the rows are prepared
+    // for the down projection. The intermediates live in the library's workspace; d_ws is left alone.
+    size_t grp = f16x2_group(gu) < f16x2_group(down) ? f16x2_group(gu) : f16x2_group(down);
+    const size_t t0 = rows_x < grp ? rows_x : grp;
+    const size_t mm1 = f16x2_matmul_ws(gu, t0), gb = align256(t0 * gu->rows * sizeof(float));
+    void* ws = nullptr;
+    if ((rc = lib_workspace(s, mm1 + gb + f16x2_matmul_ws(down, t0), &ws, "fhip_ffn"))) return rc;
+    float* g = (float*)((uint8_t*)ws + mm1);
+    void* ws2 = (uint8_t*)ws + mm1 + gb;
+    for (size_t m0 = 0; m0 < rows_x; m0 += grp) {
+        const size_t t = rows_x - m0 < grp ? rows_x - m0 : grp;
+        if (!takes_f16x2(gu, t) || !takes_f16x2(down, t)) {
+            if ((rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, d_ws + m0 * n_ff, n_ff, s))) return rc;
+            rc = fhip::launch_gemv(down, d_ws + m0 * n_ff, t, d_y + m0 * down->rows, 0, s);
+        } else if (!(rc = f16x2_matmul(gu, d_x + m0 * gu->cols, t, false, g, ws, s))) {
+            rc = f16x2_matmul(down, g, t, true, d_y + m0 * down->rows, ws2, s);
+        }
+        if (rc) return rc;
+    }
+    return FHIP_OK;
 }
+
+int fhip_batch_policy(int policy) {
+    const int before = g_batch_policy;
+    if (policy == FHIP_BATCH_AUTO || policy == FHIP_BATCH_F32_MATVEC) g_batch_policy = policy;
+    return before;
+}
+
+int fhip_workspace_reserve(void* stream, size_t nbytes) {
+    int rc = need_init();
+    if (rc) return rc;
+    void* p = nullptr;
+    return nbytes ? lib_workspace((hipStream_t)stream, nbytes, &p, "fhip_workspace_reserve") : FHIP_OK;
+}
+
+size_t fhip_workspace_bytes(const fhip_weight* gu, const fhip_weight* down, size_t rows_x) {
+    // what fhip_matmul_q (down == NULL), fhip_matmul_q_swiglu (down == NULL) or fhip_ffn asks of the workspace: the largest
+    size_t need = 0;
+    if (!gu || rows_x == 0) return 0;
+    if (takes_f16x2(gu, rows_x)) {
+        const size_t t0 = rows_x < f16x2_group(gu) ? rows_x : f16x2_group(gu);
+        need = f16x2_matmul_ws(gu, t0) + align256(t0 * gu->rows * sizeof(float));
+        if (down && takes_f16x2(down, rows_x)) need += f16x2_matmul_ws(down, t0 < f16x2_group(down) ? t0 : f16x2_group(down));
+    }
+    return need;
+}
+
+void fhip_workspace_release(void* stream) { release_workspace((hipStream_t)stream); }
 
 int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, void* stream) {
     int rc = need_init();
@@ -678,7 +837,6 @@ int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, fl
     return fhip::launch_gemm_bf16(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream, clr);
 }
 
-static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 size_t fhip_ffn_coop_ws_bytes(const fhip_weight* gu, const fhip_weight* down, size_t rows_x) {
     if (!gu || !down) return 0;

@@ -166,14 +166,22 @@ int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ggml_ty
 
 /* crates/ferric-tensor/src/dtype.rs:935 Tensor::matmul_q (and :1292 matmul_q8_0, :1426 matmul_q4_k,
  * :1172 matmul_q6_k): y[rows_x, rows] = x[rows_x, cols] * W^T, f32 in, f32 accumulate, f32 out.
- * rows_x = 1 is the decode GEMV; any rows_x >= 1 is accepted. */
+ * rows_x = 1 is the decode GEMV; any rows_x >= 1 is accepted.
+ * Which kernel a batch takes (fhip_batch_policy): one or two rows go through the streaming mat-vec; from three rows on (five
+ * for Q8_0) Q4_K / Q6_K / Q8_0 weights are read once per group of up to 32 (Q8_0: 16) rows by the f16 hi/lo matrix-core
+ * kernels (see fhip_matmul_q_f16x2: f32-grade, 22-bit activations), longer batches group by group. That path keeps its
+ * prepared activations in a workspace the library owns per stream (fhip_workspace_reserve); inside a graph capture the
+ * workspace cannot grow, and the call then fails with FHIP_ERR_ARG and says how many bytes to reserve beforehand.
+ * Non-finite activations: on the mat-vec kernel a NaN or infinite x gives what the f32 dot gives (NaN, +-inf by the weight's
+ * sign); on the matrix-core kernels the whole output row of such an activation row is non-finite and no other row is touched. */
 int fhip_matmul_q(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, void* stream);
 
 /* crates/ferric-tensor/src/dtype.rs:949 try_matmul_swiglu / :1551 matmul_q4_k_swiglu / :1802
  * matmul_q6_k_swiglu: `gate_up` stacks gate rows [0, n_ff) then up rows [n_ff, 2 n_ff);
  * y[rows_x, n_ff] = silu(x*gate^T) * (x*up^T), silu(g) = g / (1 + exp(-g)).
  * Errors: odd row count -> FHIP_ERR_SHAPE; Q8_0 -> FHIP_ERR_UNSUPPORTED_TYPE (reference: None,
- * the caller then runs matmul_q + swiglu). */
+ * the caller then runs matmul_q + swiglu). Batches of three rows and more: as fhip_matmul_q, then the un-fused
+ * SwiGLU of crates/ferric-tensor/src/lib.rs:2603-2618 over the [rows, 2 n_ff] intermediate in the library's workspace. */
 int fhip_matmul_q_swiglu(const fhip_weight* gate_up, const float* d_x, size_t rows_x, float* d_y, void* stream);
 
 /* crates/ferric-tensor/src/lib.rs:728 Tensor::swiglu(d): gu is [t, 2d] = [gate | up] per row,
@@ -181,7 +189,8 @@ int fhip_matmul_q_swiglu(const fhip_weight* gate_up, const float* d_x, size_t ro
 int fhip_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, void* stream);
 
 /* The FFN block of crates/ferric-llama/src/qwen3.rs:944-964: y = down( swiglu( gate_up(x) ) ).
- * d_ws is caller-provided scratch of at least rows_x * n_ff f32 (n_ff = gate_up rows / 2). */
+ * d_ws is caller-provided scratch of at least rows_x * n_ff f32 (n_ff = gate_up rows / 2). Batches of three rows and more
+ * run as fhip_ffn_f16x2 does (one pass over each weight per group of up to 32 rows) out of the library's workspace. */
 int fhip_ffn(const fhip_weight* gate_up, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y,
              float* d_ws, void* stream);
 
@@ -292,6 +301,26 @@ int fhip_qkv_post_attention(const float* d_qkv, const float* d_bias, const float
  * rounding (the sum of squares is added in a different order), not the same bits. No single counterpart in the reference. */
 int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_resid, const float* d_norm_w, float eps, float* d_x_out,
                        float* d_h_scratch, int swiglu, float* d_y, void* stream);
+
+/* Which kernel fhip_matmul_q, fhip_matmul_q_swiglu and fhip_ffn give a batch of three rows or more. FHIP_BATCH_AUTO (the
+ * default): the one-pass matrix-core kernels as described at fhip_matmul_q. FHIP_BATCH_F32_MATVEC: the streaming mat-vec, two
+ * rows per pass over the weights; an output row then has the same bits whatever batch it was part of (the guarantee the
+ * reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200), at the price of rows_x / 2 passes. Returns the
+ * policy before the call; any other value only queries. Process-wide, as fhip_matvec_precision. */
+#define FHIP_BATCH_AUTO 0
+#define FHIP_BATCH_F32_MATVEC 1
+int fhip_batch_policy(int policy);
+
+/* The library's workspace of a stream (NULL: the default stream): device memory the batched paths of fhip_matmul_q,
+ * fhip_matmul_q_swiglu and fhip_ffn use for prepared activations and intermediates. It is allocated on first need, only
+ * grows (to a power of two), is shared by the calls enqueued on that stream, and is freed by fhip_workspace_release or
+ * fhip_stream_destroy (both wait for the stream first). fhip_workspace_bytes: what a call with these weights (down may be
+ * NULL) and rows_x rows needs at most, 0 when it takes the mat-vec kernel. fhip_workspace_reserve: grow it to nbytes now,
+ * e.g. before a graph capture, during which it cannot grow. A buffer that was outgrown stays allocated until the release,
+ * because a graph captured earlier may still name it. No counterpart in the reference (wgpu allocates per dispatch). */
+size_t fhip_workspace_bytes(const fhip_weight* w, const fhip_weight* down, size_t rows_x);
+int fhip_workspace_reserve(void* stream, size_t nbytes);
+void fhip_workspace_release(void* stream);
 
 /* Debugging and tests: on != 0 sends every mat-vec to the shape-complete f32 kernel instead of the streaming one (process-wide,
  * not thread-safe against concurrent launches). No counterpart in the reference. */

@@ -64,10 +64,13 @@ def precision(request, F):
 
 @pytest.fixture
 def precision24(F):
-    """For tests that use the streaming mat-vec as the f32-grade side of a comparison."""
+    """For tests that use the streaming mat-vec as the f32-grade side of a comparison: 24-bit activations, and every batch
+    on that kernel (by default a batch of three rows or more goes to the one-pass matrix-core kernels)."""
     lib = F._lib.load()
     before = lib.fhip_matvec_precision(24)
+    policy = lib.fhip_batch_policy(1)
     _PRECISION["bits"] = 24
     yield
     lib.fhip_matvec_precision(before)
+    lib.fhip_batch_policy(policy)
     _PRECISION["bits"] = before
