@@ -11,6 +11,15 @@
 
 namespace {
 
+// The intermediate of fhip_ffn_noalloc: [rows_x, n_ff] f32 between the gate|up and the down mat-vec. It lives in the code
+// object, so each device the library runs on holds its own copy (512 KiB) from load to process exit and no call has to
+// allocate. Host code never uses the array's name as an address: fhip_init asks the runtime for the device address of the
+// current device's copy and keeps it per device.
+constexpr size_t NOALLOC_FLOATS = 131072;
+__device__ __align__(256) float scratch[NOALLOC_FLOATS];
+constexpr int MAX_DEVICES = 64;
+float* g_scratch_ptr[MAX_DEVICES] = {};
+
 thread_local char g_err[512] = "";
 int g_device = -1;
 int g_cus = 0;
@@ -201,6 +210,11 @@ int fhip_init(int device) {
     g_cus = prop.multiProcessorCount;
     g_lds = prop.sharedMemPerBlockOptin > prop.sharedMemPerBlock ? prop.sharedMemPerBlockOptin : prop.sharedMemPerBlock;
     if (g_lds < 64 * 1024) g_lds = 64 * 1024;
+    if (device < MAX_DEVICES && !g_scratch_ptr[device]) {   // this device's copy of the built-in scratch array
+        float* ptr = nullptr;
+        if ((rc = check_hip(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)"))) return rc;
+        g_scratch_ptr[device] = ptr;
+    }
     g_device = device;
     return FHIP_OK;
 }
@@ -562,6 +576,28 @@ int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, s
         if (rc) return rc;
     }
     return FHIP_OK;
+}
+
+int fhip_ffn_noalloc(const fhip_weight* gu, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!gu || !down) return set_error(FHIP_ERR_ARG, "fhip_ffn_noalloc: NULL weight");
+    if (gu->rows % 2 != 0) return set_error(FHIP_ERR_SHAPE, "ffn: gate_up rows must be even");
+    const size_t n_ff = gu->rows / 2;
+    if (down->cols != n_ff) return set_error(FHIP_ERR_SHAPE, "down in dim must equal n_ff");
+    if (rows_x == 0) return FHIP_OK;
+    if (!d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_ffn_noalloc: NULL pointer");
+    if (gu->type == FHIP_Q8_0) return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "fhip_ffn_noalloc: gate_up must be Q4_K or Q6_K");
+    if (rows_x > NOALLOC_FLOATS / (n_ff ? n_ff : 1))
+        return set_error(FHIP_ERR_SHAPE, "fhip_ffn_noalloc: rows_x * n_ff = %zu * %zu floats do not fit the built-in scratch of %zu floats; use fhip_ffn",
+                         rows_x, n_ff, NOALLOC_FLOATS);
+    float* h = g_device < MAX_DEVICES ? g_scratch_ptr[g_device] : nullptr;
+    if (!h) return set_error(FHIP_ERR_HIP, "fhip_ffn_noalloc: no scratch address for device %d", g_device);
+    // the mat-vec kernels for every batch width (they need nothing beside operands and this intermediate; the one-pass
+    // kernels of fhip_ffn would need the library's workspace); every element of h is written before it is read
+    hipStream_t s = (hipStream_t)stream;
+    if ((rc = fhip::launch_gemv(gu, d_x, rows_x, h, n_ff, s))) return rc;
+    return fhip::launch_gemv(down, h, rows_x, d_y, 0, s);
 }
 
 int fhip_batch_policy(int policy) {

@@ -302,6 +302,14 @@ int fhip_qkv_post_attention(const float* d_qkv, const float* d_bias, const float
 int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_resid, const float* d_norm_w, float eps, float* d_x_out,
                        float* d_h_scratch, int swiglu, float* d_y, void* stream);
 
+/* fhip_ffn for callers that cannot allocate or bring a workspace (code under graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc): the [rows_x, n_ff] intermediate lives in a 512 KiB array built into the library's code object (one
+ * copy per device, held until the process ends), so the call takes inputs and outputs only and calls no allocating routine.
+ * Always the mat-vec kernels (two rows per pass over the weights), so its result has the bits of fhip_ffn under
+ * FHIP_BATCH_F32_MATVEC. rows_x * n_ff > 131072 floats: FHIP_ERR_SHAPE. Every call on a device shares that device's array:
+ * calls that overlap in time on one GPU (two streams, two threads) race on it. It has no counterpart in the reference. */
+int fhip_ffn_noalloc(const fhip_weight* gate_up, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y, void* stream);
+
 /* Which kernel fhip_matmul_q, fhip_matmul_q_swiglu and fhip_ffn give a batch of three rows or more. FHIP_BATCH_AUTO (the
  * default): the one-pass matrix-core kernels as described at fhip_matmul_q. FHIP_BATCH_F32_MATVEC: the streaming mat-vec, two
  * rows per pass over the weights; an output row then has the same bits whatever batch it was part of (the guarantee the
