@@ -424,8 +424,13 @@ def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
 
 
 def probe(F, lib, check):
-    """Work for a hardware-counter run: a copy of known size to calibrate FETCH_SIZE / WRITE_SIZE, then the
-    kernels of interest on weights no earlier launch has touched."""
+    """Work for a profiler run (kernel trace or hardware counters) of the mat-vec kernels, launched eagerly on the null stream:
+    a copy of known size first (it calibrates FETCH_SIZE / WRITE_SIZE), then every weight shape of the decode sweep and the
+    Q8_0 4096 x 4096 weight, each on rotating copies that add up to more than the 256 MB Infinity Cache so that every launch
+    reads HBM: 512 launches of the headline Q4_K 5120 x 5120 (the O projection's shape too) over 64 copies, 256 of the fused
+    QKV 7168 x 5120 over 40, 64 of gate|up 34816 x 5120 with SwiGLU over 8, 64 of down 5120 x 17408 Q6_K over 10, 512 of Q8_0
+    4096 x 4096 over 56 and 8 of the vocabulary head 151936 x 5120 Q6_K over 2. The launches of a shape are enqueued back to
+    back from native code (fhip_debug_matmul_q_loop), so the device sees the steady stream a captured graph would give it."""
     from ferric_amd.synth import synth_weights
     n = 256 << 20
     src, dst = F.DeviceBuffer(n), F.DeviceBuffer(n)
@@ -433,19 +438,20 @@ def probe(F, lib, check):
     check(lib.fhip_stream_sync(None))
     check(lib.fhip_memcpy_d2d(dst.ptr, src.ptr, n, None))          # calibration dispatch: reads n, writes n
     check(lib.fhip_stream_sync(None))
-    host = synth_weights(Q4_K, 5120, 5120, 1)
-    buf = replicate(F, lib, check, host, 48)
-    ws = [F.QMatrix.wrap_device(buf, host.size, Q4_K, 5120, 5120, offset=i * host.size) for i in range(48)]
     x = F.Tensor.from_vec(np.random.default_rng(2).standard_normal(5120).astype(np.float32), (1, 5120))
-    y = F.Tensor.empty((1, 34816))
-    for i in range(32, 48):                                         # the last copies written are the least likely to sit in a cache
-        check(lib.fhip_matmul_q(ws[i].handle, x.buf.ptr, 1, y.buf.ptr, None))
-    gu = F.QMatrix.from_bytes(synth_weights(Q4_K, 34816, 5120, 3), Q4_K, 34816, 5120)
-    dn = F.QMatrix.from_bytes(synth_weights(Q6_K, 5120, 17408, 4), Q6_K, 5120, 17408)
+    x4 = F.Tensor.from_vec(np.random.default_rng(2).standard_normal(4096).astype(np.float32), (1, 4096))
     h = F.Tensor.from_vec(np.random.default_rng(3).standard_normal(17408).astype(np.float32), (1, 17408))
-    check(lib.fhip_matmul_q_swiglu(gu.handle, x.buf.ptr, 1, y.buf.ptr, None))
-    check(lib.fhip_matmul_q(dn.handle, h.buf.ptr, 1, y.buf.ptr, None))
-    check(lib.fhip_stream_sync(None))
+    y = F.Tensor.empty((1, 151936))
+    plan = [(Q4_K, 5120, 5120, 64, 512, x, False), (Q4_K, 7168, 5120, 40, 256, x, False), (Q4_K, 34816, 5120, 8, 64, x, True),
+            (Q6_K, 5120, 17408, 10, 64, h, False), (Q8_0, 4096, 4096, 56, 512, x4, False), (Q6_K, 151936, 5120, 2, 8, x, False)]
+    for ty, rows, cols, ncopy, launches, xin, swiglu in plan:
+        host = synth_weights(ty, rows, cols, 1)
+        buf = replicate(F, lib, check, host, ncopy)
+        ws = [F.QMatrix.wrap_device(buf, host.size, ty, rows, cols, offset=i * host.size) for i in range(ncopy)]
+        handles = (C.c_void_p * ncopy)(*[w.handle for w in ws])
+        check(lib.fhip_debug_matmul_q_loop(handles, ncopy, launches, xin.buf.ptr, 1 if swiglu else 0, y.buf.ptr, None))
+        check(lib.fhip_stream_sync(None))
+        del ws, buf
 
 
 def probe_prefill(F, lib, check):

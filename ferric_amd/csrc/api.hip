@@ -776,6 +776,19 @@ int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, vo
     return fhip::launch_read_probe(d_src, nbytes, d_sink, (hipStream_t)stream);
 }
 
+int fhip_debug_matmul_q_loop(const fhip_weight* const* ws, size_t n_weights, size_t launches, const float* d_x, int swiglu, float* d_y,
+                             void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (!ws || n_weights == 0 || !d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_debug_matmul_q_loop: NULL pointer");
+    for (size_t i = 0; i < launches; i++) {
+        const fhip_weight* w = ws[i % n_weights];
+        rc = swiglu ? fhip_matmul_q_swiglu(w, d_x, 1, d_y, stream) : fhip_matmul_q(w, d_x, 1, d_y, stream);
+        if (rc) return rc;
+    }
+    return FHIP_OK;
+}
+
 int fhip_matvec_precision(int bits) {
     const int before = fhip::g_planes == 3 ? 24 : 16;
     if (bits == 0) return before;

@@ -340,6 +340,12 @@ int fhip_debug_generic_matvec(int on);
  * kernel itself, crates/ferric-tensor/examples/matvec_roofline.rs:85-100). */
 int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, void* stream);
 
+/* Measurement aid: `launches` one-row calls of fhip_matmul_q (swiglu != 0: fhip_matmul_q_swiglu) enqueued back to back from
+ * native code, launch i on weight ws[i % n_weights], all with the same x and y. A profiler run that cannot replay graphs gets
+ * the same steady stream of launches from it that a captured graph gives. No counterpart in the reference. */
+int fhip_debug_matmul_q_loop(const fhip_weight* const* ws, size_t n_weights, size_t launches, const float* d_x, int swiglu, float* d_y,
+                             void* stream);
+
 /* Precision of the activations inside the streaming mat-vec kernels (fhip_matmul_q, _swiglu, fhip_ffn, the "_id" entry points,
  * fhip_norm_matmul_q): per run of 32 (16 for Q6_K) columns the activations are held as block fixed point with a `bits`-bit
  * significand at the run's largest magnitude, the weights exactly, the sums exactly, and everything above the sub-block in
