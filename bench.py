@@ -344,11 +344,10 @@ def bench_sweep(F, lib, check, stream, timer, tokens=4, layers=64):
                       "ops still execute in stream order"}
 
 
-def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), layers=64, steps=6):
-    """The decode weight sweep as a real decode step: the same 64-layer stack (fused QKV 5120->7168 with 40 query / 8 KV heads of 128, O,
-    fused gate|up 5120->34816 + SwiGLU, all Q4_K; down 17408->5120 Q6_K; output norm + lm_head 151936 Q6_K), but with every op fed
-    by the one before it: RMSNorm, q/k norm + rope + KV append, attention over `context` cached tokens (f32 cache), residual
-    adds. One graph per step, replayed `steps` times at consecutive positions."""
+def decode_stack(F, lib, check, layers=64):
+    """The 64-layer stack of the decode sweep as a decoder: fused QKV 5120->7168 (40 query / 8 KV heads of 128), O, fused gate|up
+    5120->34816, all Q4_K; down 17408->5120 Q6_K; output norm + lm_head 151936 Q6_K. Synthetic weights, one distinct copy per
+    layer. Returns (cfg, layers, output norm, lm_head, weight bytes)."""
     from ferric_amd import decode as X
     from ferric_amd.synth import synth_weights
     d, nh, nkv, hd, n_ff, vocab = 5120, 40, 8, 128, 17408, 151936
@@ -369,20 +368,38 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
         W[n] = [F.QMatrix.wrap_device(stacks[n], nb, ty, r, c, offset=l * nb) for l in range(layers)]
     lay = [X.Qwen3Layer(small, W["qkv"][l], W["o"][l], small, W["gate_up"][l], W["down"][l], unit, unit) for l in range(layers)]
     cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6)
+    return cfg, lay, small, head, weight_bytes_total, stacks
+
+
+def decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, room, stream, rng):
+    """A decoder over the stack with `ctx` earlier tokens' keys and values (synthetic) in every layer's cache and an input set."""
+    from ferric_amd import decode as X
+    nkv, hd, d = cfg.n_head_kv, cfg.head_dim, cfg.d_model
+    dec = X.Qwen3Decoder(cfg, lay, max_len=ctx + room + 2, stream=stream, output_norm=small, lm_head=head)
+    kv_fill = (rng.standard_normal((ctx, nkv * hd)) * 0.5).astype(np.float32)
+    first = dec.caches[0]                         # uploaded once, copied on the device
+    check(lib.fhip_memcpy_h2d(first.k.buf.ptr, kv_fill.ctypes.data_as(C.c_void_p), kv_fill.nbytes, None))
+    check(lib.fhip_stream_sync(None))
+    for c in dec.caches:
+        if c is not first:
+            check(lib.fhip_memcpy_d2d(c.k.buf.ptr, first.k.buf.ptr, kv_fill.nbytes, None))
+        check(lib.fhip_memcpy_d2d(c.v.buf.ptr, first.k.buf.ptr, kv_fill.nbytes, None))
+    check(lib.fhip_stream_sync(None))
+    dec.set_pos(ctx)
+    dec.set_input((rng.standard_normal(d) * 0.5).astype(np.float32))
+    return dec
+
+
+def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), layers=64, steps=6):
+    """The decode weight sweep as a real decode step: the 64-layer stack of decode_stack(), with every op fed by the one before
+    it: RMSNorm, q/k norm + rope + KV append, attention over `context` cached tokens (f32 cache), residual adds. One graph per
+    step, replayed `steps` times at consecutive positions."""
+    cfg, lay, small, head, weight_bytes_total, stacks = decode_stack(F, lib, check, layers)
+    nkv, hd = cfg.n_head_kv, cfg.head_dim
+    rng = np.random.default_rng(9)
     out = {}
     for ctx in contexts:
-        dec = X.Qwen3Decoder(cfg, lay, max_len=ctx + steps + 2, stream=stream, output_norm=small, lm_head=head)
-        kv_fill = (rng.standard_normal((ctx, nkv * hd)) * 0.5).astype(np.float32)
-        first = dec.caches[0]                     # `ctx` earlier tokens' keys and values (synthetic): uploaded once, copied on the device
-        check(lib.fhip_memcpy_h2d(first.k.buf.ptr, kv_fill.ctypes.data_as(C.c_void_p), kv_fill.nbytes, None))
-        check(lib.fhip_stream_sync(None))
-        for c in dec.caches:
-            if c is not first:
-                check(lib.fhip_memcpy_d2d(c.k.buf.ptr, first.k.buf.ptr, kv_fill.nbytes, None))
-            check(lib.fhip_memcpy_d2d(c.v.buf.ptr, first.k.buf.ptr, kv_fill.nbytes, None))
-        check(lib.fhip_stream_sync(None))
-        dec.set_pos(ctx)
-        dec.set_input((rng.standard_normal(d) * 0.5).astype(np.float32))
+        dec = decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, steps, stream, rng)
         dec.capture()
         dec.step_graph()                          # warm-up step (also: instantiation costs)
         ms = timer.time_ms(lambda: [dec.step_graph() for _ in range(steps)]) / steps
@@ -395,6 +412,22 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
     out["weight_bytes"] = weight_bytes_total
     out["model"] = "64 layers, d 5120, 40 query / 8 KV heads x 128, n_ff 17408, vocab 151936; Q4_K projections, Q6_K down and lm_head; f32 KV cache"
     return out
+
+
+def probe_step(F, lib, check):
+    """Work for a kernel trace of the chained decode step without graph replay: the 64-layer decoder of bench_decode, three
+    steps enqueued eagerly at context 128 and three at context 4096 (every launch of a step on the decoder's stream, in the
+    order the captured graph holds them)."""
+    stream = F.Stream()
+    cfg, lay, small, head, _, stacks = decode_stack(F, lib, check, 64)
+    rng = np.random.default_rng(9)
+    for ctx in (128, 4096):
+        dec = decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, 4, stream, rng)
+        for _ in range(3):
+            dec.step()
+        check(lib.fhip_stream_sync(stream.handle))
+        assert np.isfinite(dec.logits.to_vec(stream)).all()
+        del dec
 
 
 def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
@@ -586,6 +619,7 @@ def main():
     ap.add_argument("--probe", action="store_true",
                     help="counter probe for rocprofv3 --pmc: one 256 MiB device copy (calibration), then 16 cold Q4_K 5120x5120 "
                          "GEMVs, one fused gate|up 34816x5120 and one Q6_K 5120x17408 GEMV; prints nothing else")
+    ap.add_argument("--probe-step", action="store_true", help="three eager decode steps at context 128 and 4096 (for a kernel trace)")
     ap.add_argument("--probe-decode", action="store_true",
                     help="profiler probe for the decode attention kernel: 8 launches each at 4096 and 128 cached rows; prints nothing else")
     ap.add_argument("--probe-prefill", action="store_true",
@@ -617,6 +651,9 @@ def main():
         return
     if args.probe_decode:
         probe_decode(F, lib, check)
+        return
+    if args.probe_step:
+        probe_step(F, lib, check)
         return
     log("[bench] Q4_K GEMV 5120x5120 ...")
     c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
