@@ -39,59 +39,67 @@ struct TensorInfo {
     uint64_t offset = 0;
 };
 
-// lib.rs:56-104
-struct Cur {
-    const uint8_t* b;
-    size_t n, p = 0;
-    bool ok = true;
-    const uint8_t* take(size_t k) {
-        if (!ok || k > n - p) { ok = false; return nullptr; }
-        const uint8_t* s = b + p;
-        p += k;
+// A window [at, end) over the mapped file that only moves forward. Every read is checked against what is left; the first
+// read that does not fit sets `bad` and from then on every read yields zeros, so a parser can run to its end and ask once.
+// (Bounds behaviour of crates/ferric-gguf/src/lib.rs:56-104: a short or hostile header is refused, never read past.)
+struct Window {
+    const uint8_t* at;
+    const uint8_t* end;
+    bool bad = false;
+    size_t left() const { return (size_t)(end - at); }
+    const uint8_t* bytes(uint64_t k) {
+        if (bad || k > left()) { bad = true; return nullptr; }
+        const uint8_t* s = at;
+        at += (size_t)k;
         return s;
     }
-    template <class T> T rd() {
-        const uint8_t* s = take(sizeof(T));
+    template <class T> T scalar() {
         T v{};
-        if (s) memcpy(&v, s, sizeof(T));
+        if (const uint8_t* s = bytes(sizeof(T))) memcpy(&v, s, sizeof(T));
         return v;
     }
-    std::string str() {
-        const uint64_t len = rd<uint64_t>();
-        if (len > n - p) { ok = false; return {}; }   // a garbage length must not become a huge reservation
-        const uint8_t* s = take((size_t)len);
+    // u64 length + bytes. The length is compared with what is left BEFORE anything is sized by it: a length field of
+    // 2^60 in a 1 KiB file is an error, not an allocation.
+    std::string text() {
+        const uint64_t len = scalar<uint64_t>();
+        const uint8_t* s = bytes(len);
         return s ? std::string((const char*)s, (size_t)len) : std::string();
     }
-    Meta val(uint32_t ty, int depth = 0) {
-        Meta m;
-        switch (ty) {
-            case 0: m.kind = K_U; m.u = rd<uint8_t>(); break;
-            case 1: m.kind = K_I; m.i = (int8_t)rd<uint8_t>(); break;
-            case 2: m.kind = K_U; m.u = rd<uint16_t>(); break;
-            case 3: m.kind = K_I; m.i = (int16_t)rd<uint16_t>(); break;
-            case 4: m.kind = K_U; m.u = rd<uint32_t>(); break;
-            case 5: m.kind = K_I; m.i = (int32_t)rd<uint32_t>(); break;
-            case 6: m.kind = K_F; m.f = (double)rd<float>(); break;
-            case 7: m.kind = K_BOOL; m.u = rd<uint8_t>() != 0; break;
-            case 8: m.kind = K_STR; m.s = str(); break;
-            case 9: {
-                m.kind = K_ARR;
-                const uint32_t et = rd<uint32_t>();
-                const uint64_t cnt = rd<uint64_t>();
-                // each element costs at least one byte on disk, so a count beyond the remaining bytes is garbage
-                if (cnt > n - p || depth > 8) { ok = false; break; }
-                m.a.reserve((size_t)cnt);
-                for (uint64_t k = 0; k < cnt && ok; k++) m.a.push_back(val(et, depth + 1));
-                break;
-            }
-            case 10: m.kind = K_U; m.u = rd<uint64_t>(); break;
-            case 11: m.kind = K_I; m.i = rd<int64_t>(); break;
-            case 12: m.kind = K_F; m.f = rd<double>(); break;
-            default: ok = false; break;
-        }
-        return m;
-    }
 };
+
+// One metadata value of GGUF value type `ty` (0..12; 9 = array of one element type, nested at most 8 deep).
+Meta read_value(Window& w, uint32_t ty, int depth = 0) {
+    Meta m;
+    auto as_u = [&](uint64_t v) { m.kind = K_U; m.u = v; };
+    auto as_i = [&](int64_t v) { m.kind = K_I; m.i = v; };
+    auto as_f = [&](double v) { m.kind = K_F; m.f = v; };
+    switch (ty) {
+        case 0: as_u(w.scalar<uint8_t>()); break;
+        case 1: as_i(w.scalar<int8_t>()); break;
+        case 2: as_u(w.scalar<uint16_t>()); break;
+        case 3: as_i(w.scalar<int16_t>()); break;
+        case 4: as_u(w.scalar<uint32_t>()); break;
+        case 5: as_i(w.scalar<int32_t>()); break;
+        case 6: as_f(w.scalar<float>()); break;
+        case 7: m.kind = K_BOOL; m.u = w.scalar<uint8_t>() != 0; break;
+        case 8: m.kind = K_STR; m.s = w.text(); break;
+        case 9: {
+            m.kind = K_ARR;
+            const uint32_t elem = w.scalar<uint32_t>();
+            const uint64_t count = w.scalar<uint64_t>();
+            // no element type is shorter than a byte, so more elements than bytes left cannot be a real array
+            if (count > w.left() || depth > 8) { w.bad = true; break; }
+            m.a.reserve((size_t)count);
+            for (uint64_t k = 0; k < count && !w.bad; k++) m.a.push_back(read_value(w, elem, depth + 1));
+            break;
+        }
+        case 10: as_u(w.scalar<uint64_t>()); break;
+        case 11: as_i(w.scalar<int64_t>()); break;
+        case 12: as_f(w.scalar<double>()); break;
+        default: w.bad = true; break;
+    }
+    return m;
+}
 
 // On-disk size of n elements of ggml type ty, the reference's whole table (lib.rs:460-484): the stride check
 // needs the size of every tensor in the file, not only of the formats this library computes with.
@@ -184,36 +192,36 @@ struct fhip_gguf {
 namespace {
 
 int parse_into(fhip_gguf& g) {
-    Cur c{g.bytes, g.len};
-    const uint32_t magic = c.rd<uint32_t>();
-    if (!c.ok || magic != 0x46554747u) return fhip::set_error(FHIP_ERR_FORMAT, "not a GGUF file");   // "GGUF" little endian
-    g.version = c.rd<uint32_t>();
-    const uint64_t n_tensors = c.rd<uint64_t>(), n_meta = c.rd<uint64_t>();
-    for (uint64_t k = 0; k < n_meta && c.ok; k++) {
-        std::string key = c.str();
-        const uint32_t ty = c.rd<uint32_t>();
-        Meta m = c.val(ty);
+    Window c{g.bytes, g.bytes + g.len};
+    const uint32_t magic = c.scalar<uint32_t>();
+    if (c.bad || magic != 0x46554747u) return fhip::set_error(FHIP_ERR_FORMAT, "not a GGUF file");   // "GGUF" little endian
+    g.version = c.scalar<uint32_t>();
+    const uint64_t n_tensors = c.scalar<uint64_t>(), n_meta = c.scalar<uint64_t>();
+    for (uint64_t k = 0; k < n_meta && !c.bad; k++) {
+        std::string key = c.text();
+        const uint32_t ty = c.scalar<uint32_t>();
+        Meta m = read_value(c, ty);
         auto it = g.meta_ix.find(key);
         if (it != g.meta_ix.end()) g.meta[it->second].second = std::move(m);   // a repeated key keeps the last value (HashMap::insert)
         else { g.meta_ix[key] = g.meta.size(); g.meta.emplace_back(std::move(key), std::move(m)); }
     }
-    for (uint64_t k = 0; k < n_tensors && c.ok; k++) {
+    for (uint64_t k = 0; k < n_tensors && !c.bad; k++) {
         TensorInfo t;
-        t.name = c.str();
-        const uint32_t nd = c.rd<uint32_t>();
-        if ((uint64_t)nd * 8 > c.n - c.p) { c.ok = false; break; }
-        for (uint32_t d = 0; d < nd; d++) t.dims.push_back(c.rd<uint64_t>());
-        t.ggml_type = c.rd<uint32_t>();
-        t.offset = c.rd<uint64_t>();
+        t.name = c.text();
+        const uint32_t nd = c.scalar<uint32_t>();
+        if ((uint64_t)nd * 8 > c.left()) { c.bad = true; break; }
+        for (uint32_t d = 0; d < nd; d++) t.dims.push_back(c.scalar<uint64_t>());
+        t.ggml_type = c.scalar<uint32_t>();
+        t.offset = c.scalar<uint64_t>();
         g.tensors.push_back(std::move(t));
     }
-    if (!c.ok) return fhip::set_error(FHIP_ERR_FORMAT, "GGUF header truncated or malformed");
+    if (c.bad) return fhip::set_error(FHIP_ERR_FORMAT, "GGUF header truncated or malformed");
     for (size_t i = 0; i < g.tensors.size(); i++) g.tensor_ix.emplace(g.tensors[i].name, i);   // first of a repeated name, as `find`
     uint64_t align = 32;
     auto al = g.meta_ix.find("general.alignment");
     if (al != g.meta_ix.end() && g.meta[al->second].second.kind == K_U) align = g.meta[al->second].second.u;
     if (align == 0) return fhip::set_error(FHIP_ERR_FORMAT, "GGUF general.alignment is 0");
-    g.data_start = (c.p + align - 1) / align * align;
+    g.data_start = ((size_t)(c.at - g.bytes) + align - 1) / align * align;
     const uint64_t data_len = g.len > g.data_start ? g.len - g.data_start : 0;
     const std::string why = check_declared_strides(g.tensors, data_len, align);
     if (!why.empty()) return fhip::set_error(FHIP_ERR_FORMAT, "%s", why.c_str());
