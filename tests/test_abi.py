@@ -33,6 +33,23 @@ def test_no_undeclared_fhip_exports():
     assert exported == _declared()
 
 
+def test_the_rust_binding_declares_the_same_entry_points():
+    # crates/ferric-hip/src/ffi.rs is the binding a maintainer links: one `pub fn` per entry point of the header, with as many
+    # arguments as the C prototype has
+    text = open(os.path.join(ROOT, "include", "ferric_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    c_args = {}
+    for name, args in re.findall(r"\b(fhip_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        args = " ".join(args.split())
+        c_args[name] = 0 if args in ("", "void") else args.count(",") + 1
+    rust = open(os.path.join(ROOT, "crates", "ferric-hip", "src", "ffi.rs")).read()
+    r_args = {}
+    for name, args in re.findall(r"pub fn (fhip_[a-z0-9_]+)\(([^)]*)\)", rust):
+        r_args[name] = 0 if not args.strip() else args.count(",") + 1
+    assert sorted(r_args) == _declared()
+    assert r_args == c_args
+
+
 def test_size_tables_need_no_device():
     # crates/ferric-gguf/src/lib.rs:471-494 and crates/ferric-tensor/src/dtype.rs:873-889
     from ferric_amd import QMatrix, type_size
