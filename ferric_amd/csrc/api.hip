@@ -15,6 +15,7 @@ namespace {
 // object, so each device the library runs on holds its own copy (512 KiB) from load to process exit and no call has to
 // allocate. Host code never uses the array's name as an address: fhip_init asks the runtime for the device address of the
 // current device's copy and keeps it per device.
+constexpr size_t WEIGHT_SLACK = 256;   // readable bytes every weight has behind its last block
 constexpr size_t NOALLOC_FLOATS = 131072;
 __device__ __align__(256) float scratch[NOALLOC_FLOATS];
 constexpr int MAX_DEVICES = 64;
@@ -182,6 +183,13 @@ bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
     return fhip::gemm_f16x2_supports(w, rows_x < f16x2_group(w) ? rows_x : f16x2_group(w));
 }
 
+// y [t, rows] = 0 on the stream, by the mat-vec launcher's fill kernel (what a weight without columns gives)
+int zero_outputs(size_t t, size_t rows, float* d_y, hipStream_t s) {
+    fhip_weight z{};
+    z.type = FHIP_Q8_0; z.rows = rows; z.cols = 0;
+    return fhip::launch_gemv(&z, d_y, t, d_y, 0, s);
+}
+
 // y [t, w->rows] = x [t, cols] W^T for t rows of one group; ws: f16x2_matmul_ws(w, t) bytes
 size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) { return align256(fhip::gemm_f16x2_xp_bytes(w, t)) + align256(fhip::gemm_f16x2_aux_bytes()); }
 int f16x2_matmul(const fhip_weight* w, const float* d_x, size_t t, bool swiglu_in, float* d_y, void* d_ws, hipStream_t s) {
@@ -247,7 +255,9 @@ int fhip_malloc(void** d_ptr, size_t nbytes) {
     int rc = need_init();
     if (rc) return rc;
     *d_ptr = nullptr;
-    return check_hip(hipMalloc(d_ptr, nbytes ? nbytes : 1), "hipMalloc");
+    // 256 bytes more than asked for: a weight wrapped at the end of such a buffer (fhip_weight_wrap_device) keeps the slack
+    // behind its last block that fhip_weight_create gives its own allocations
+    return check_hip(hipMalloc(d_ptr, nbytes + WEIGHT_SLACK), "hipMalloc");
 }
 int fhip_free(void* d_ptr) { return d_ptr ? check_hip(hipFree(d_ptr), "hipFree") : FHIP_OK; }
 int fhip_memcpy_h2d(void* d, const void* h, size_t n, void* s) {
@@ -345,10 +355,10 @@ int fhip_weight_create(uint32_t ty, const uint8_t* h_raw, size_t nbytes, size_t 
     if ((rc = make_weight(ty, nbytes, rows, cols, w))) return rc;
     if (nbytes && !h_raw) return set_error(FHIP_ERR_ARG, "fhip_weight_create: NULL bytes");
     void* d = nullptr;
-    // 256 bytes of slack past the stream: wide loads of lanes that are masked out stay inside the allocation.
-    if ((rc = check_hip(hipMalloc(&d, nbytes + 256), "hipMalloc(weight)"))) return rc;
+    // slack past the stream: a wide load that starts inside the last block may end behind it
+    if ((rc = check_hip(hipMalloc(&d, nbytes + WEIGHT_SLACK), "hipMalloc(weight)"))) return rc;
     if (nbytes && (rc = check_hip(hipMemcpy(d, h_raw, nbytes, hipMemcpyHostToDevice), "hipMemcpy(weight)"))) { (void)hipFree(d); return rc; }
-    if ((rc = check_hip(hipMemset((uint8_t*)d + nbytes, 0, 256), "hipMemset(weight tail)"))) { (void)hipFree(d); return rc; }
+    if ((rc = check_hip(hipMemset((uint8_t*)d + nbytes, 0, WEIGHT_SLACK), "hipMemset(weight tail)"))) { (void)hipFree(d); return rc; }
     w.d_raw = (const uint8_t*)d;
     w.owns = true;
     *out = new fhip_weight(w);
@@ -393,6 +403,18 @@ int fhip_weight_wrap_device(uint32_t ty, const uint8_t* d_raw, size_t nbytes, si
     if ((rc = make_weight(ty, nbytes, rows, cols, w))) return rc;
     if (nbytes && !d_raw) return set_error(FHIP_ERR_ARG, "fhip_weight_wrap_device: NULL bytes");
     if (((uintptr_t)d_raw & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_weight_wrap_device: bytes must be 16-byte aligned");
+    if (nbytes) {   // the allocation has to reach WEIGHT_SLACK bytes past the last block, as the library's own weights do
+        hipDeviceptr_t base = nullptr;
+        size_t size = 0;
+        if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)d_raw) != hipSuccess) {
+            (void)hipGetLastError();
+            return set_error(FHIP_ERR_ARG, "fhip_weight_wrap_device: not a device allocation");
+        }
+        const uintptr_t end = (uintptr_t)base + size, need = (uintptr_t)d_raw + nbytes + WEIGHT_SLACK;
+        if (need > end)
+            return set_error(FHIP_ERR_ARG, "fhip_weight_wrap_device: the allocation must extend %zu bytes past the weight's last block "
+                             "(it ends %zu bytes behind it); buffers from fhip_malloc always do", WEIGHT_SLACK, (size_t)(end - ((uintptr_t)d_raw + nbytes)));
+    }
     w.d_raw = d_raw;
     w.owns = false;
     *out = new fhip_weight(w);
@@ -632,7 +654,8 @@ int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float*
     if (rc) return rc;
     if (!w) return set_error(FHIP_ERR_ARG, "fhip_gemm_q_bf16: NULL weight");
     if (t == 0 || w->rows == 0) return FHIP_OK;
-    if (!d_x || !d_y) return set_error(FHIP_ERR_ARG, "fhip_gemm_q_bf16: NULL pointer");
+    if (!d_y || (!d_x && w->cols)) return set_error(FHIP_ERR_ARG, "fhip_gemm_q_bf16: NULL pointer");
+    if (w->cols == 0) return zero_outputs(t, w->rows, d_y, (hipStream_t)stream);   // empty inner dimension: every dot product is 0
     return fhip::launch_gemm_bf16(w, d_x, t, d_y, (hipStream_t)stream);
 }
 
@@ -750,7 +773,17 @@ int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_re
     int rc = need_init();
     if (rc) return rc;
     if (!w || !d_x || !d_norm_w || !d_h_scratch || !d_y) return set_error(FHIP_ERR_ARG, "fhip_norm_matmul_q: NULL pointer");
-    if (d_x_out && d_x_out == d_x) return set_error(FHIP_ERR_ARG, "fhip_norm_matmul_q: x_out must not be x");
+    // every workgroup reads all of x and resid while one of them stores x_out, and all of them store y: none of the outputs
+    // may share memory with an input or with each other
+    {
+        const size_t out_rows = swiglu ? w->rows / 2 : w->rows;
+        auto overlap = [](const float* a, size_t na, const float* b, size_t nb) { return a && b && a < b + nb && b < a + na; };
+        if (overlap(d_x_out, w->cols, d_x, w->cols) || overlap(d_x_out, w->cols, d_resid, w->cols) || overlap(d_x_out, w->cols, d_norm_w, w->cols))
+            return set_error(FHIP_ERR_ARG, "fhip_norm_matmul_q: x_out must not overlap x, resid or norm_w");
+        if (overlap(d_y, out_rows, d_x, w->cols) || overlap(d_y, out_rows, d_resid, w->cols) || overlap(d_y, out_rows, d_norm_w, w->cols) ||
+            overlap(d_y, out_rows, d_x_out, w->cols))
+            return set_error(FHIP_ERR_ARG, "fhip_norm_matmul_q: y must not overlap x, resid, norm_w or x_out");
+    }
     if (swiglu && (w->type == FHIP_Q8_0 || w->rows % 2 != 0))
         return set_error(w->type == FHIP_Q8_0 ? FHIP_ERR_UNSUPPORTED_TYPE : FHIP_ERR_SHAPE, "fhip_norm_matmul_q: no fused SwiGLU for this weight");
     if (((uintptr_t)d_x | (uintptr_t)d_resid | (uintptr_t)d_norm_w | (uintptr_t)d_x_out) & 15)
@@ -879,6 +912,7 @@ int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, fl
     if (rc) return rc;
     if (!w) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL weight");
     if (rows_x == 0 || w->rows == 0) return FHIP_OK;
+    if (w->cols == 0) return d_y ? zero_outputs(rows_x, w->rows, d_y, (hipStream_t)stream) : set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL pointer");
     if (!d_x || !d_y || !d_ws_bf16) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL pointer");
     const bool clr = fhip::gemm_bf16_adds_into_y(rows_x);
     if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * w->cols, d_ws_bf16, (hipStream_t)stream, clr ? d_y : nullptr, clr ? rows_x * w->rows : 0)))
@@ -903,6 +937,8 @@ int fhip_ffn_coop(const fhip_weight* gu, const fhip_weight* down, const float* d
     if (rows_x == 0) return FHIP_OK;
     if (!d_x || !d_y || !d_ws) return set_error(FHIP_ERR_ARG, "fhip_ffn_coop: NULL pointer");
     if (((uintptr_t)d_ws & 255) != 0) return set_error(FHIP_ERR_ARG, "fhip_ffn_coop: workspace must be 256-byte aligned");
+    // an empty inner dimension on either side: gate and up are 0, silu(0) * 0 = 0, and so is every output
+    if (gu->cols == 0 || n_ff == 0) return zero_outputs(rows_x, down->rows, d_y, (hipStream_t)stream);
     uint8_t* ws = (uint8_t*)d_ws;
     uint16_t* xb = (uint16_t*)ws;
     float* g = (float*)(ws + align256(rows_x * gu->cols * 2));

@@ -131,7 +131,9 @@ int fhip_weight_create_parts(uint32_t ggml_type, const uint8_t* const* h_parts, 
                              size_t rows, size_t cols, fhip_weight** out);
 
 /* Same, but adopts block bytes that are already in device memory (no copy; the caller keeps the
- * buffer alive until fhip_weight_destroy). Used when a loader streams a file straight into HBM. */
+ * buffer alive until fhip_weight_destroy). Used when a loader streams a file straight into HBM. d_raw: 16-byte aligned, and
+ * the allocation it lies in must extend 256 bytes past the weight's last block (readable, content irrelevant), as the library's
+ * own weights do: buffers from fhip_malloc always qualify; anything else is checked and refused with FHIP_ERR_ARG. */
 int fhip_weight_wrap_device(uint32_t ggml_type, const uint8_t* d_raw, size_t nbytes, size_t rows, size_t cols,
                             fhip_weight** out);
 
@@ -295,7 +297,8 @@ int fhip_qkv_post_attention(const float* d_qkv, const float* d_bias, const float
 
 /* rmsnorm / add_rmsnorm (lib.rs:346, :372) fused into the mat-vec that consumes it, for ONE activation row:
  *   h = rmsnorm(x [+ resid], norm_w, eps);   y = h W^T   (swiglu != 0: y = silu(gate . h) * (up . h), as fhip_matmul_q_swiglu)
- * and, when d_x_out is given, x_out = x + resid (the next residual; must not alias d_x). The norm is formed while the
+ * and, when d_x_out is given, x_out = x + resid (the next residual). Neither x_out nor y may overlap x, resid, norm_w or each
+ * other (FHIP_ERR_ARG): every workgroup reads the whole inputs while the outputs are being stored. The norm is formed while the
  * activation row is staged, so the layer saves a launch; weights whose shape the streaming kernel does not take run the two
  * steps apart through d_h_scratch [cols] (required). d_resid may be NULL (plain rmsnorm). Same value as the unfused pair to
  * rounding (the sum of squares is added in a different order), not the same bits. No single counterpart in the reference. */

@@ -336,8 +336,13 @@ def test_norm_fused_into_the_matvec(F, X, D, O, precision):
                 assert (np.abs(y.to_vec() - y64[0]) <= 1e-3 * wn * np.linalg.norm(h64)).all()
                 assert close(y.to_vec(), y64, dot_bar()), (ty, rows, cols)
             assert close(y.to_vec(), y_ref, 2e-5)
-    with pytest.raises(F._lib.FerricHipError, match="x_out must not be x"):
+    # outputs that share memory with an input (the in-place residual update included) or with each other are refused
+    with pytest.raises(F._lib.FerricHipError, match="x_out must not overlap"):
         F._lib.check(lib.fhip_norm_matmul_q(w.handle, xt.buf.ptr, rt.buf.ptr, nt.buf.ptr, 1e-6, xt.buf.ptr, hs.buf.ptr, 0, y.buf.ptr, None))
+    with pytest.raises(F._lib.FerricHipError, match="x_out must not overlap"):
+        F._lib.check(lib.fhip_norm_matmul_q(w.handle, xt.buf.ptr, rt.buf.ptr, nt.buf.ptr, 1e-6, rt.buf.ptr, hs.buf.ptr, 0, y.buf.ptr, None))
+    with pytest.raises(F._lib.FerricHipError, match="y must not overlap"):
+        F._lib.check(lib.fhip_norm_matmul_q(w.handle, xt.buf.ptr, rt.buf.ptr, nt.buf.ptr, 1e-6, xo.buf.ptr, hs.buf.ptr, 0, xo.buf.ptr, None))
 
 
 def _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, qk_norm):

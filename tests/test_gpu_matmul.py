@@ -344,6 +344,17 @@ def test_empty_shapes(F):
     assert F.matvec_q8_0(np.zeros(0, np.float32), np.zeros(0, np.uint8), 0, 0).size == 0
     y = F.matvec_q8_0(np.zeros(0, np.float32), np.zeros(0, np.uint8), 5, 0)
     assert y.shape == (5,) and not y.any()
+    # a weight without columns: every dot product is the empty sum, on every entry point that takes the weight
+    lib, check = F._lib.load(), F._lib.check
+    qm = F.QMatrix.from_bytes(np.zeros(0, np.uint8), Q4_K, 7, 0)
+    yt = F.Tensor.from_vec(np.full((3, 7), 5.0, np.float32), (3, 7))
+    dummy = F.Tensor.empty((1, 64))
+    for call in (lambda: lib.fhip_matmul_q(qm.handle, dummy.buf.ptr, 3, yt.buf.ptr, None),
+                 lambda: lib.fhip_gemm_q_bf16(qm.handle, dummy.buf.ptr, 3, yt.buf.ptr, None),
+                 lambda: lib.fhip_matmul_q_coop(qm.handle, dummy.buf.ptr, 3, yt.buf.ptr, dummy.buf.ptr, None)):
+        check(lib.fhip_memset(yt.buf.ptr, 0x41, 3 * 7 * 4, None))
+        check(call())
+        assert not yt.to_vec().any()
 
 
 # ---------------------------------------------------------------- activations block fixed point cannot hold
