@@ -1050,12 +1050,32 @@ struct fhip_pool {
     hipStream_t stream;
     const uint8_t* key;
     size_t key_len, key_cols;
+    uint64_t key_print;   // fingerprint of the bytes the key pointed at when they were uploaded
     uint8_t* d_w;
     size_t w_cap;
     float *d_x, *d_y;
     size_t x_cap, y_cap;
     size_t uploads;
 };
+
+// FNV-1a over the first and the last 4 KiB and 64 evenly spaced 64-byte samples of the weight: about 12 KiB per call. It catches
+// a buffer that was freed and reused, or rewritten, at the same address and length (what pointer + length alone would take for
+// the resident weight); it is not a proof of equality -- a caller that edits a few bytes in place still calls fhip_pool_forget.
+static uint64_t pool_fingerprint(const uint8_t* w, size_t n) {
+    uint64_t h = 1469598103934665603ull;
+    auto eat = [&](size_t from, size_t len) {
+        for (size_t i = from; i < from + len && i < n; i++) h = (h ^ w[i]) * 1099511628211ull;
+    };
+    eat(0, 4096);
+    if (n > 8192) {
+        eat(n - 4096, 4096);
+        const size_t step = (n - 8192) / 64;
+        for (size_t k = 0; k < 64 && step >= 64; k++) eat(4096 + k * step, 64);
+    } else if (n > 4096) {
+        eat(4096, n - 4096);
+    }
+    return h ^ n;
+}
 
 int fhip_pool_create(size_t threads, fhip_pool** out) {
     if (!out) return set_error(FHIP_ERR_ARG, "fhip_pool_create: NULL output");
@@ -1112,11 +1132,12 @@ int fhip_matvec_q8_0_pooled(fhip_pool* p, const float* h_x, size_t x_len, const 
     if (x_len < nblk * 32) return set_error(FHIP_ERR_SHAPE, "range end index %zu out of range for slice of length %zu", nblk * 32, x_len);
     if (!h_x || !h_w) return set_error(FHIP_ERR_ARG, "fhip_matvec_q8_0_pooled: NULL pointer");
     const size_t kcols = nblk * 32, all_rows = w_len / row_bytes;
-    if (p->key != h_w || p->key_len != w_len || p->key_cols != kcols) {
+    const uint64_t print = pool_fingerprint(h_w, all_rows * row_bytes);
+    if (p->key != h_w || p->key_len != w_len || p->key_cols != kcols || p->key_print != print) {
         fhip_pool_forget(p);
         if ((rc = pool_reserve((void**)&p->d_w, &p->w_cap, all_rows * row_bytes, "hipMalloc"))) return rc;
         if ((rc = check_hip(hipMemcpyAsync(p->d_w, h_w, all_rows * row_bytes, hipMemcpyHostToDevice, p->stream), "hipMemcpy H2D"))) return rc;
-        p->key = h_w; p->key_len = w_len; p->key_cols = kcols;
+        p->key = h_w; p->key_len = w_len; p->key_cols = kcols; p->key_print = print;
         p->uploads++;
     }
     if ((rc = pool_reserve((void**)&p->d_x, &p->x_cap, kcols * sizeof(float), "hipMalloc"))) return rc;

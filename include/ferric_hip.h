@@ -460,7 +460,10 @@ int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, si
  * the bytes of the last `h_w` it was given resident in HBM (with its staging buffers and a stream of its own) and a
  * call with the same (h_w, w_len, cols) uploads the activations only. `w` is an immutable Arc<Vec<u8>> in the
  * reference; a caller that rewrites the bytes in place, or frees them (another buffer may then appear at the same address),
- * calls fhip_pool_forget first -- a binding keeps a clone of the Arc beside the pool for as long as it is the key.
+ * calls fhip_pool_forget first -- a binding keeps a clone of the Arc beside the pool for as long as it is the key. As a
+ * second line of defence the key also holds a fingerprint of the bytes (first and last 4 KiB and 64 spread samples, hashed on
+ * every call): a buffer rewritten or reused at the same address and length is uploaded again unless the change misses all of
+ * those, so the fingerprint replaces no fhip_pool_forget.
  * h_y receives hi - lo values.
  * `threads` is kept for Pool::threads() (at least 1) and partitions nothing here. lo > hi, a span past the rows in
  * h_w or fewer than cols activations: FHIP_ERR_SHAPE (the reference's assert and slice panics). One call at a time

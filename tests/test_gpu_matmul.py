@@ -133,6 +133,23 @@ def test_spans_compose_through_the_pool_and_the_weight_is_uploaded_once(F, O):  
     pool.close()                                                        # cpu_simd.rs:403-409: dropping the pool must not hang
 
 
+def test_pool_notices_a_weight_rewritten_in_place(F, O):
+    # the pool's key is the host pointer, the length and a fingerprint of the bytes: the same buffer with other contents is
+    # uploaded again (crates/ferric-tensor/src/cpu_simd.rs:238-331 holds an immutable Arc, so the reference cannot meet this)
+    rows, cols = 64, 1024
+    w = O.gen_q8_0_synth(rows, cols, 5)[0].copy()
+    x = np.cos(np.arange(cols, dtype=np.float32) * np.float32(0.01)).astype(np.float32)
+    pool = F.Pool(4)
+    y1 = F.matvec_q8_0_pooled(pool, x, w, cols, 0, rows)
+    assert pool.uploads() == 1 and np.array_equal(bits(y1), bits(F.matvec_q8_0(x, w, rows, cols)))
+    w[:] = O.gen_q8_0_synth(rows, cols, 6)[0]                    # same address, same length, new bytes
+    y2 = F.matvec_q8_0_pooled(pool, x, w, cols, 0, rows)
+    assert pool.uploads() == 2 and np.array_equal(bits(y2), bits(F.matvec_q8_0(x, w, rows, cols)))
+    assert not np.array_equal(bits(y1), bits(y2))
+    y3 = F.matvec_q8_0_pooled(pool, x, w, cols, 0, rows)         # unchanged: resident
+    assert pool.uploads() == 2 and np.array_equal(bits(y3), bits(y2))
+
+
 def test_pooled_edge_cases(F, O):
     raw, _ = O.gen_q8_0_synth(8, 64, 1)
     x = np.ones(64, np.float32)
