@@ -136,3 +136,34 @@ def test_layers_of_the_sweep_chained_in_one_graph(F, O):
                 assert (err <= 1e-3 * wn * np.linalg.norm(xin.astype(np.float64))).all(), (l, name)
                 assert err.max() <= dot_bar() * np.abs(y64).max(), (l, name)
     check_rows(O, logits.to_vec(stream), x, head_raw, Q6_K, 5120, [(0, 3001)], "head")
+
+
+@pytest.mark.parametrize("ty,rows,cols,swiglu", [(Q4_K, 12301, 5120, False), (Q4_K, 2 * 12303, 5120, True), (Q6_K, 4099, 17408, False),
+                                                 (Q8_0, 33001, 1024, False)])
+def test_large_weights_whose_rows_are_dealt_in_chunks_of_four(F, O, ty, rows, cols, swiglu):
+    """From 16 rows per row group on, the launch deals the rows to the row groups round-robin in chunks of 4 instead of giving
+    each a contiguous span. Row counts that leave the last round of chunks, and the last chunk, partly filled; every output
+    against the oracle, and a span of the rows computed alone (which takes the other dealing) gives the same bits."""
+    from ferric_amd.synth import synth_weights
+    raw = synth_weights(ty, rows, cols, 80)
+    w = F.QMatrix.from_bytes(raw, ty, rows, cols)
+    x = (np.random.default_rng(81).standard_normal(cols) * (0.1 if swiglu else 1.0)).astype(np.float32)
+    xt = F.Tensor.from_vec(x, (1, cols))
+    y64, wn = O.matmul_f64(x, raw, ty, rows, cols)
+    if swiglu:
+        n_ff = rows // 2
+        got = xt.try_matmul_swiglu(w).to_vec()
+        gate, up = y64[0, :n_ff], y64[0, n_ff:]
+        want = gate / (1.0 + np.exp(-gate)) * up
+        assert got.shape == (n_ff,) and np.abs(got - want).max() <= dot_bar() * np.abs(want).max()
+        return
+    got = xt.matmul_q(w).to_vec()
+    err = np.abs(got - y64[0])
+    assert (err <= 1e-3 * wn * np.linalg.norm(x.astype(np.float64))).all()
+    assert err.max() <= dot_bar() * np.abs(y64).max()
+    rb = row_bytes(ty, cols)
+    for r0, n in ((0, 37), (rows - 50, 50), (rows // 2 & ~7, 1001)):
+        if (r0 * rb) % 16:
+            continue
+        part = F.QMatrix.from_bytes(raw[r0 * rb:(r0 + n) * rb], ty, n, cols)
+        assert np.array_equal(bits(xt.matmul_q(part).to_vec()), bits(got[r0:r0 + n])), r0
