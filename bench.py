@@ -315,8 +315,9 @@ def bench_sweep(F, lib, check, stream, timer, tokens=4, layers=64):
     layer_bytes = sum(h.size for h in host.values())
     stacks = {n: replicate(F, lib, check, host[n], layers) for n, _, _, _ in shapes}
     head_host = synth_weights(Q6_K, 151936, 5120, 50)
-    head = F.QMatrix.from_bytes(head_host, Q6_K, 151936, 5120)
-    total = layer_bytes * layers + head_host.size
+    head_buf, head_bytes = replicate(F, lib, check, head_host, 1), head_host.size
+    head = F.QMatrix.wrap_device(head_buf, head_bytes, Q6_K, 151936, 5120)
+    total = layer_bytes * layers + head_bytes
     del head_host
     rng = np.random.default_rng(6)
     x = F.Tensor.from_vec(rng.standard_normal(5120).astype(np.float32), (1, 5120))
@@ -338,7 +339,20 @@ def bench_sweep(F, lib, check, stream, timer, tokens=4, layers=64):
     g.launch()
     ts = sorted(timer.time_ms(lambda: [g.launch() for _ in range(tokens)]) / tokens for _ in range(5))
     ms = ts[len(ts) // 2]
+    # The same 257 launches with a kernel that only reads each weight's bytes (fhip_debug_read_probe): what this device gives
+    # a sweep cut into these launches when no arithmetic, staging or reduction stands in the way.
+    sink = F.DeviceBuffer(256)
+    gr = F.Graph.begin(stream)
+    for l in range(layers):
+        for n, _, _, _ in shapes:
+            check(lib.fhip_debug_read_probe(C.c_void_p(stacks[n].ptr.value + l * host[n].size), host[n].size, sink.ptr, s))
+    check(lib.fhip_debug_read_probe(head_buf.ptr, head_bytes, sink.ptr, s))
+    gr.end()
+    gr.launch()
+    tr = sorted(timer.time_ms(lambda: [gr.launch() for _ in range(tokens)]) / tokens for _ in range(5))
+    floor_ms = tr[len(tr) // 2]
     return {"ms_per_token": ms, "ms_per_token_min_max": [ts[0], ts[-1]], "GBps": total / (ms * 1e-3) / 1e9, "frac_of_peak": total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "reader_floor_ms": floor_ms, "reader_floor_GBps": total / (floor_ms * 1e-3) / 1e9, "frac_of_reader": floor_ms / ms,
             "weight_bytes": total, "layers": layers, "launches_per_token": layers * 4 + 1,
             "inputs": "fixed N(0,1) activations per op (outputs are not fed forward, so values stay finite); "
                       "ops still execute in stream order"}
@@ -677,7 +691,7 @@ def main():
         "warm_single_copy": c2["warm"],
         "roofline": {"bound": "hbm", "achieved": alg / (ms_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                     "traffic": traffic["traffic_bytes"] if traffic else None, "traffic_source": traffic,
+                     "traffic": traffic.get("hbm_bytes_per_launch") if traffic else None, "traffic_source": traffic,
                      "kernel": "gemv_stream_kernel<Q4K, M=1, plain>", "algorithmic_bytes_per_launch": alg,
                      "launch_us": ms_step * 1e3,
                      # the same 14.7 MB through a kernel that only reads them (same rotation, same timing), and a launch
