@@ -271,6 +271,28 @@ def bench_moe(F, lib, check, stream, timer, reps=64):
     return res
 
 
+def bench_host_entry(F, rows=4096, cols=4096, reps=12):
+    """The host-buffer entry points of the CPU path (cpu_simd::matvec_q8_0 and its pooled form): weights, activations and
+    results cross PCIe inside the call. Never `value`: it measures the bus, not the kernel."""
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(Q8_0, rows, cols, 0)
+    x = np.random.default_rng(2).standard_normal(cols).astype(np.float32)
+    F.matvec_q8_0(x, w, rows, cols)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        F.matvec_q8_0(x, w, rows, cols)
+    each = (time.perf_counter() - t0) / reps
+    pool = F.Pool(1)
+    F.matvec_q8_0_pooled(pool, x, w, cols, 0, rows)
+    t0 = time.perf_counter()
+    for _ in range(reps * 4):
+        F.matvec_q8_0_pooled(pool, x, w, cols, 0, rows)
+    pooled = (time.perf_counter() - t0) / (reps * 4)
+    pool.close()
+    return {"workload": "Q8_0 4096x4096, host buffers in and out", "matvec_q8_0_host_ms": each * 1e3, "weight_GBps_with_upload": w.size / each / 1e9,
+            "matvec_q8_0_pooled_ms": pooled * 1e3, "note": "the pooled call keeps the weight resident and uploads the activations only"}
+
+
 def bench_gguf(F, lib, check, n_tensors=8, rows=11008, cols=5120):
     """GGUF ingest: a synthetic file of n_tensors Q4_K [rows, cols] tensors (31.7 MB each) written to a temporary
     file, then opened (mmap + header parse + stride check) and every tensor uploaded straight from the mapping.
@@ -728,6 +750,7 @@ def main():
     if not args.no_moe:
         log("[bench] GGUF ingest ...")
         line["gguf_ingest"] = bench_gguf(F, lib, check)
+        line["host_buffer_entry_points"] = bench_host_entry(F)
     if not args.no_sweep:
         log("[bench] 64-layer decode weight sweep (14.0 GB) ...")
         line["decode_sweep"] = bench_sweep(F, lib, check, stream, timer)
