@@ -480,6 +480,7 @@ def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
             xb = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
             x = F.Tensor.from_bf16_bits(xb, (t, k))
             y = F.Tensor.empty((t, n))
+            check(lib.fhip_workspace_reserve(stream.handle, lib.fhip_workspace_bytes_coop(qm.handle, None, t)))
             g = F.Graph.begin(stream)
             for _ in range(reps):
                 check(lib.fhip_gemm_q_bf16(qm.handle, x.buf.ptr, t, y.buf.ptr, stream.handle))

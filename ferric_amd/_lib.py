@@ -105,6 +105,7 @@ SYMBOLS = {
     "fhip_ffn_noalloc": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _vp]),
     "fhip_batch_policy": (C.c_int, [C.c_int]),
     "fhip_workspace_bytes": (C.c_size_t, [_vp, _vp, C.c_size_t]),
+    "fhip_workspace_bytes_coop": (C.c_size_t, [_vp, _vp, C.c_size_t]),
     "fhip_workspace_reserve": (C.c_int, [_vp, C.c_size_t]),
     "fhip_workspace_release": (None, [_vp]),
     "fhip_debug_read_probe": (C.c_int, [_vp, _sz, _vp, _vp]),

@@ -168,6 +168,18 @@ void release_workspace(hipStream_t s) {
     }
 }
 
+// The matrix-core GEMM with its K-split scratch (partial tiles of the tiles that several workgroups share) taken from the
+// stream's library workspace.
+static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared, const char* who) {
+    const size_t need = fhip::gemm_bf16_ws_bytes(w, t);
+    void* ws = nullptr;
+    if (need) {
+        int rc = lib_workspace(s, need, &ws, who);
+        if (rc) return rc;
+    }
+    return fhip::launch_gemm_bf16(w, d_x, t, d_y, s, y_cleared, (float*)ws, need);
+}
+
 // ---- which kernel a batch takes ---------------------------------------------------------------------------------------------
 // One or two activation rows go through the streaming mat-vec (one pass over the weights serves two rows). From three rows on
 // (five for Q8_0) the f16 hi/lo matrix-core kernels read the weights once for up to 32 (Q8_0: 16) rows; longer batches are cut
@@ -647,6 +659,11 @@ size_t fhip_workspace_bytes(const fhip_weight* gu, const fhip_weight* down, size
     return need;
 }
 
+size_t fhip_workspace_bytes_coop(const fhip_weight* w, const fhip_weight* down, size_t rows_x) {
+    const size_t a = fhip::gemm_bf16_ws_bytes(w, rows_x), b = fhip::gemm_bf16_ws_bytes(down, rows_x);
+    return a > b ? a : b;
+}
+
 void fhip_workspace_release(void* stream) { release_workspace((hipStream_t)stream); }
 
 int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, void* stream) {
@@ -656,7 +673,7 @@ int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float*
     if (t == 0 || w->rows == 0) return FHIP_OK;
     if (!d_y || (!d_x && w->cols)) return set_error(FHIP_ERR_ARG, "fhip_gemm_q_bf16: NULL pointer");
     if (w->cols == 0) return zero_outputs(t, w->rows, d_y, (hipStream_t)stream);   // empty inner dimension: every dot product is 0
-    return fhip::launch_gemm_bf16(w, d_x, t, d_y, (hipStream_t)stream);
+    return gemm_bf16_lib_ws(w, d_x, t, d_y, (hipStream_t)stream, false, "fhip_gemm_q_bf16");
 }
 
 // ---- mixture-of-experts entry points (crates/ferric-tensor/src/dtype.rs:1582-1780) ----------------------
@@ -917,7 +934,7 @@ int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, fl
     const bool clr = fhip::gemm_bf16_adds_into_y(rows_x);
     if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * w->cols, d_ws_bf16, (hipStream_t)stream, clr ? d_y : nullptr, clr ? rows_x * w->rows : 0)))
         return rc;
-    return fhip::launch_gemm_bf16(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream, clr);
+    return gemm_bf16_lib_ws(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream, clr, "fhip_matmul_q_coop");
 }
 
 
@@ -946,9 +963,9 @@ int fhip_ffn_coop(const fhip_weight* gu, const fhip_weight* down, const float* d
     hipStream_t s = (hipStream_t)stream;
     const bool clr = fhip::gemm_bf16_adds_into_y(rows_x);   // then each conversion clears the next GEMM's output on the side
     if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * gu->cols, xb, s, clr ? g : nullptr, clr ? rows_x * gu->rows : 0))) return rc;
-    if ((rc = fhip::launch_gemm_bf16(gu, xb, rows_x, g, s, clr))) return rc;
+    if ((rc = gemm_bf16_lib_ws(gu, xb, rows_x, g, s, clr, "fhip_ffn_coop"))) return rc;
     if ((rc = fhip::launch_swiglu_bf16(g, rows_x, n_ff, hb, s, clr ? d_y : nullptr, clr ? rows_x * down->rows : 0))) return rc;
-    return fhip::launch_gemm_bf16(down, hb, rows_x, d_y, s, clr);
+    return gemm_bf16_lib_ws(down, hb, rows_x, d_y, s, clr, "fhip_ffn_coop");
 }
 
 size_t fhip_matmul_q_f16x2_ws_bytes(const fhip_weight* w, size_t rows_x) {

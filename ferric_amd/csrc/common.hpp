@@ -105,7 +105,10 @@ int launch_moe_wsum(const float* d_parts, const float* d_selw, size_t t, int k, 
 
 // gemm_mfma.hip
 // y_cleared: the caller has zeroed y on this stream already (see gemm_bf16_adds_into_y)
-int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared = false);
+// d_ws / ws_bytes: gemm_bf16_ws_bytes(w, t) bytes of scratch for launches that cut tiles along K (0: none needed)
+int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared = false,
+                     float* d_ws = nullptr, size_t ws_bytes = 0);
+size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t);
 bool gemm_bf16_adds_into_y(size_t t);   // true: a launch for t rows may add into y, so a cleared y saves it a launch
 // conversions in front of the GEMM; each can also clear `zero_n` floats at `zero`
 int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s, float* zero = nullptr, size_t zero_n = 0);

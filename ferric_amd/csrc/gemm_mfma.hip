@@ -250,6 +250,8 @@ struct GemmParams {
     int whole_rounds;    // rounds of whole tiles every workgroup computes first: tile = round * gridDim.x + blockIdx.x
     long long units;     // the remaining tiles' (tile, chunk) work units, chunk fastest
     int per;             // of those, units per workgroup
+    float* ws;           // partial tiles of the left-over tiles that several runs share: [left-over tile][contributor][BM x 256]
+    int kmax;            // contributor slots per left-over tile
 };
 
 template <int I, int N, class Fn>
@@ -272,7 +274,10 @@ __device__ __forceinline__ void static_for(Fn&& f) {
 // tiles left over, fewer than one per workgroup, are cut along K: their (tile, chunk) units are dealt out in
 // equal contiguous runs of `per`, so every CU does the same amount of MFMA work whatever the tile count (no
 // partial last round). A run may start and end inside a tile: a segment that covers its tile's whole K stores
-// the tile, any other adds it atomically into a Y that zero_split_tiles_kernel cleared beforehand.
+// the tile, any other stores its partial sums into the workspace slot (tile, contributor), contributor = the run's rank among
+// the runs that touch the tile, and sum_split_tiles_kernel adds a tile's slots in that order afterwards: the result does not
+// depend on which workgroup finishes first (f32 atomics into Y, which this replaced, gave run-to-run differences in the
+// last bits wherever a tile had three contributors or more).
 template <class F, int MI>
 __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
     constexpr int NI = 2;
@@ -428,6 +433,14 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
         step(std::integral_constant<int, 3>{}, ck);
     }
 
+    // a partial tile goes to the slot of this run in the tile's contributor list: runs are numbered by blockIdx.x, and the
+    // first run that touches left-over tile rt is the one that holds unit rt * nchunks
+    float* part = nullptr;
+    if (!whole) {
+        const int rt = tile - p.whole_rounds * (int)gridDim.x;
+        const int k = (int)blockIdx.x - (int)(((long long)rt * nchunks) / p.per);
+        part = p.ws + ((size_t)rt * p.kmax + k) * (size_t)(BM * 256);
+    }
     // D layout of the 32x32 MFMA: register r of lane (h, c) is row 8*(r/4) + 4*h + (r%4), column c
 #pragma unroll
     for (int i = 0; i < MI; i++)
@@ -439,27 +452,45 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
             for (int r = 0; r < 16; r++) {
                 const int t = t0 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
                 if (t < p.T) {
-                    float* y = p.Y + (size_t)t * p.N + n;
-                    if (whole) *y = acc[i][j][r];
-                    else unsafeAtomicAdd(y, acc[i][j][r]);
+                    if (whole) p.Y[(size_t)t * p.N + n] = acc[i][j][r];
+                    else part[(size_t)(t - tile_y * BM) * 256 + (n - tile_x * 256)] = acc[i][j][r];
                 }
             }
         }
   }
 }
 
-// Clears the output tiles that more than one workgroup contributes to (left-over tile `blockIdx.x` is split iff its first
-// and last chunk fall into different runs).
-__global__ void __launch_bounds__(256) zero_split_tiles_kernel(float* __restrict__ Y, int T, int N, int BM, int tiles_n,
-                                                             int nchunks, int per, int first_tile) {
-    const int tile = first_tile + blockIdx.x;
-    const long long u0 = (long long)blockIdx.x * nchunks;
-    if (u0 / per == (u0 + nchunks - 1) / per) return;
+// Rows 16 * blockIdx.y .. + 15 of left-over tile `blockIdx.x`, if more than one run contributed to it:
+// Y = slot 0 + slot 1 + ... in that order. A thread owns four adjacent columns of one row per pass.
+__global__ void __launch_bounds__(256) sum_split_tiles_kernel(float* __restrict__ Y, const float* __restrict__ ws, int T, int N, int BM,
+                                                            int tiles_n, int nchunks, int per, int kmax, int first_tile) {
+    const int rt = blockIdx.x, tile = first_tile + rt;
+    const long long u0 = (long long)rt * nchunks;
+    const int nk = (int)((u0 + nchunks - 1) / per) - (int)(u0 / per) + 1;
+    if (nk == 1) return;                          // one run covered the whole K of this tile and stored it
     const int tile_y = tile / tiles_n, tile_x = tile - tile_y * tiles_n;
-    const int col = tile_x * 256 + threadIdx.x;
-    if (col >= N) return;
-    const int t_end = (tile_y + 1) * BM < T ? (tile_y + 1) * BM : T;
-    for (int t = tile_y * BM; t < t_end; t++) Y[(size_t)t * N + col] = 0.f;
+    const int c4 = (threadIdx.x & 63) * 4, col = tile_x * 256 + c4;
+    const size_t slot = (size_t)BM * 256;
+    const float* base = ws + (size_t)rt * kmax * slot + c4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int lt = blockIdx.y * 16 + i * 4 + (threadIdx.x >> 6), t = tile_y * BM + lt;
+        if (t >= T || col >= N) continue;
+        const float* q = base + (size_t)lt * 256;
+        float4 a = *(const float4*)q;
+        for (int k = 1; k < nk; k++) {
+            const float4 v = *(const float4*)(q + (size_t)k * slot);
+            a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+        }
+        float* y = Y + (size_t)t * N + col;
+        if ((N & 3) == 0) *(float4*)y = a;
+        else {
+            y[0] = a.x;
+            if (col + 1 < N) y[1] = a.y;
+            if (col + 2 < N) y[2] = a.z;
+            if (col + 3 < N) y[3] = a.w;
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -631,7 +662,9 @@ int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_
 // then the left-over tiles cut along K into runs of `per` chunks.
 struct TilePlan {
     int whole_rounds, per;
-    long long left, units, split_wgs;   // left-over tiles, their chunks, workgroups that add a partial run atomically
+    long long left, units, split_wgs;   // left-over tiles, their chunks, workgroups whose run ends in partial tiles
+    int kmax;                           // most runs that touch one left-over tile
+    long long slots;                    // partial tiles the launch writes: over the left-over tiles cut along K, the runs that touch each
     unsigned grid;
 };
 
@@ -649,23 +682,38 @@ static TilePlan plan_tiles(long long tiles_n, int nchunks, size_t t, int mi, lon
     const long long runs = (q.units + per - 1) / per;
     q.grid = q.whole_rounds > 0 ? (unsigned)cus : (unsigned)runs;
     q.split_wgs = (q.left > 0 && per % nchunks != 0) ? runs : 0;
+    q.kmax = 1;
+    q.slots = 0;
+    for (long long rt = 0; rt < q.left && q.split_wgs > 0; rt++) {
+        const long long u0 = rt * nchunks;
+        const int k = (int)((u0 + nchunks - 1) / per - u0 / per) + 1;
+        if (k > q.kmax) q.kmax = k;
+        if (k > 1) q.slots += k;
+    }
     return q;
 }
 
 // Estimated duration of a plan in us: chunks per workgroup x (unpack of a 256 x 256 weight chunk + mi MFMA slabs of 64 rows),
-// plus the atomic epilogue of the split runs (a tile of 64 * mi x 256 f32 per workgroup; the chip retires about 380 G
-// f32 atomics a second, 11 us for 64 x 256 from each of 256 workgroups). Constants fitted to measured launches (Q4_K
+// plus the fix-up of the tiles cut along K (every partial tile of 64 * mi x 256 f32 is written to the workspace and read back by
+// the summing kernel: two passes over 16 MB per 64 rows of tile height for 256 partial tiles, ~6 us, and that kernel's launch;
+// a run that starts inside one tile and ends inside the next writes two).
+// Constants fitted to measured launches (Q4_K
 // 34816 x 5120, T = 2048: 8.3 us a chunk at mi = 4, 4.85 at mi = 2; Q6_K and Q8_0 likewise) and checked against 21 shapes:
 // the model ranks the tile heights like the measurement wherever they differ by more than 6 %.
 template <class F>
 static float plan_cost_us(const TilePlan& q, int nchunks, int mi, long long cus) {
     const float chunk_us = F::UNPACK_US + 1.75f * (float)mi;
     const float chunks = (float)q.whole_rounds * (float)nchunks + (q.left > 0 ? (float)q.per : 0.f);
-    return chunks * chunk_us + 11.f * (float)mi * (float)q.split_wgs / (float)cus;
+    return chunks * chunk_us + (q.split_wgs > 0 ? 3.f + 6.f * (float)mi * (float)q.slots / (float)cus : 0.f);
+}
+
+static size_t plan_ws_bytes(const TilePlan& q, int mi) {
+    return q.split_wgs > 0 ? (size_t)q.left * q.kmax * (size_t)(64 * mi * 256) * sizeof(float) : 0;
 }
 
 template <class F, int MI>
-int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, const TilePlan& q, long long cus) {
+int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, const TilePlan& q, long long cus, float* d_ws,
+               size_t ws_bytes) {
     GemmParams p;
     p.W = w->d_raw; p.X = d_x; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
@@ -676,35 +724,55 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     p.whole_rounds = q.whole_rounds;
     p.units = q.units;
     p.per = q.per;
-    if (q.split_wgs > 0)
-        hipLaunchKernelGGL(zero_split_tiles_kernel, dim3((unsigned)q.left), dim3(256), 0, s, d_y, p.T, p.N, 64 * MI,
-                           p.tiles_n, p.nchunks, p.per, (int)(p.whole_rounds * cus));
+    p.ws = d_ws; p.kmax = q.kmax;
+    if (q.split_wgs > 0 && (!d_ws || ws_bytes < plan_ws_bytes(q, MI)))
+        return fhip::set_error(FHIP_ERR_ARG, "gemm_q_bf16: the launch cuts tiles along K and needs %zu bytes of workspace", plan_ws_bytes(q, MI));
     hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(q.grid), dim3(512), 0, s, p);
+    if (q.split_wgs > 0)
+        hipLaunchKernelGGL(sum_split_tiles_kernel, dim3((unsigned)q.left, (unsigned)(64 * MI / 16)), dim3(256), 0, s, d_y, (const float*)d_ws, p.T, p.N, 64 * MI,
+                           p.tiles_n, p.nchunks, p.per, p.kmax, (int)(p.whole_rounds * cus));
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
+// the tile height the estimate picks for this launch, its plan, and the workspace it needs
 template <class F>
-int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
-    if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, y_cleared);
-    // Tile height 64 * MI. The 256 x 256 tile unpacks each weight once per 256 activation rows, but when there is no whole
-    // round of such tiles for the chip every tile is cut along K, each workgroup adds a whole tile atomically for a few
-    // chunks of work, and a lower tile (twice the tiles, half the atomics, longer runs) can win: the estimate decides
-    // (measured, Q4_K 5120 x 5120: T = 512 78 -> 63 us and T = 1024 109 -> 91 us with 128-row tiles, T = 128 36 -> 30 us with
-    // 64-row tiles; Q6_K 5120 x 17408 and Q8_0, dearer to unpack, keep the tall tile from T = 512 on).
+static int choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256, tiles_n = (long long)((w->rows + 255) / 256);
     const int nchunks = F::chunks((int)w->cols);
-    TilePlan q[3];
-    float cost[3];
     int best = 0;
+    float best_cost = 0.f;
     for (int i = 0; i < 3; i++) {
         const int mi = 4 >> i;
-        q[i] = plan_tiles(tiles_n, nchunks, t, mi, cus);
-        cost[i] = plan_cost_us<F>(q[i], nchunks, mi, cus);
-        if (cost[i] < cost[best]) best = i;
+        const TilePlan q = plan_tiles(tiles_n, nchunks, t, mi, cus);
+        const float c = plan_cost_us<F>(q, nchunks, mi, cus);
+        if (i == 0 || c < best_cost) { best = i; best_cost = c; out = q; }
     }
-    if (best == 0) return launch_cfg<F, 4>(w, d_x, t, d_y, s, q[0], cus);
-    if (best == 1) return launch_cfg<F, 2>(w, d_x, t, d_y, s, q[1], cus);
-    return launch_cfg<F, 1>(w, d_x, t, d_y, s, q[2], cus);
+    return 4 >> best;
+}
+
+template <class F>
+static size_t ws_bytes_fmt(const fhip_weight* w, size_t t) {
+    if (t <= 32) return 0;
+    TilePlan q;
+    const int mi = choose_plan<F>(w, t, q);
+    return plan_ws_bytes(q, mi);
+}
+
+template <class F>
+int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_ws, size_t ws_bytes) {
+    if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, y_cleared);
+    // Tile height 64 * MI. The 256 x 256 tile unpacks each weight once per 256 activation rows, but when there is no whole
+    // round of such tiles for the chip every tile is cut along K, each workgroup writes a whole partial tile for a few
+    // chunks of work, and a lower tile (twice the tiles, half the fix-up, longer runs) can win: the estimate decides
+    // (measured, Q4_K 5120 x 5120: T = 2048 175 -> 163 us with 128-row tiles, which give one whole round and a remainder cut
+    // in four; T = 128 42 -> 29 us with 64-row tiles; Q6_K 5120 x 17408 and Q8_0, dearer to unpack, keep the tall tile from
+    // T = 512 on).
+    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
+    TilePlan q;
+    const int mi = choose_plan<F>(w, t, q);
+    if (mi == 4) return launch_cfg<F, 4>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    if (mi == 2) return launch_cfg<F, 2>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    return launch_cfg<F, 1>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
 }
 
 // f32 -> bf16 (round to nearest even), 8 values per thread; `n8` full groups of 8, the tail one by one
@@ -760,15 +828,25 @@ int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s, 
 
 bool gemm_bf16_adds_into_y(size_t t) { return t <= 32; }
 
-int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t) {
+    if (!w || t == 0 || w->rows == 0) return 0;
+    switch (w->type) {
+        case FHIP_Q4_K: return ws_bytes_fmt<Q4K>(w, t);
+        case FHIP_Q6_K: return ws_bytes_fmt<Q6K>(w, t);
+        case FHIP_Q8_0: return ws_bytes_fmt<Q80>(w, t);
+        default: return 0;
+    }
+}
+
+int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_ws, size_t ws_bytes) {
     if (t == 0 || w->rows == 0) return FHIP_OK;
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "gemm_q_bf16: x must be 16-byte aligned");
     if ((unsigned long long)t * w->cols >= (1ull << 31))
         return set_error(FHIP_ERR_SHAPE, "gemm_q_bf16: t * cols must be below 2^31 (got %zu x %zu)", t, w->cols);
     switch (w->type) {
-        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s, y_cleared);
-        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s, y_cleared);
-        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_x, t, d_y, s, y_cleared);
+        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s, y_cleared, d_ws, ws_bytes);
+        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s, y_cleared, d_ws, ws_bytes);
+        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_x, t, d_y, s, y_cleared, d_ws, ws_bytes);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

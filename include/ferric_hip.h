@@ -198,7 +198,10 @@ int fhip_ffn(const fhip_weight* gate_up, const fhip_weight* down, const float* d
 
 /* Prefill dequant-GEMM, stands for crates/ferric-tensor/src/dtype.rs:1818 matmul_q4_k_coop (:1199
  * Q6_K, :1316 Q8_0): x is bf16 [t, cols] (raw 16-bit patterns), y f32 [t, rows]; weights are
- * dequantized tile by tile into LDS as bf16 and contracted on the matrix cores, f32 accumulate. */
+ * dequantized tile by tile into LDS as bf16 and contracted on the matrix cores, f32 accumulate. For more than 32
+ * rows a launch that cuts output tiles along K keeps their partial tiles in the library's workspace of the stream
+ * (fhip_workspace_bytes_coop) and adds them in a fixed order: the same inputs give the same bits on every run. Up to
+ * 32 rows the K slices are added with f32 atomics (last bits may differ run to run). */
 int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x_bf16, size_t t, float* d_y, void* stream);
 
 /* ---- mixture-of-experts decode: the "_id" variants that sit behind the same matmul entry points ---------- */
@@ -328,8 +331,11 @@ int fhip_batch_policy(int policy);
  * fhip_stream_destroy (both wait for the stream first). fhip_workspace_bytes: what a call with these weights (down may be
  * NULL) and rows_x rows needs at most, 0 when it takes the mat-vec kernel. fhip_workspace_reserve: grow it to nbytes now,
  * e.g. before a graph capture, during which it cannot grow. A buffer that was outgrown stays allocated until the release,
- * because a graph captured earlier may still name it. No counterpart in the reference (wgpu allocates per dispatch). */
+ * because a graph captured earlier may still name it. No counterpart in the reference (wgpu allocates per dispatch).
+ * fhip_workspace_bytes_coop: the same for the matrix-core entry points fhip_gemm_q_bf16, fhip_matmul_q_coop (down NULL) and
+ * fhip_ffn_coop, which keep there the partial tiles of a launch that cuts output tiles along K (0 when no tile is cut). */
 size_t fhip_workspace_bytes(const fhip_weight* w, const fhip_weight* down, size_t rows_x);
+size_t fhip_workspace_bytes_coop(const fhip_weight* w, const fhip_weight* down, size_t rows_x);
 int fhip_workspace_reserve(void* stream, size_t nbytes);
 void fhip_workspace_release(void* stream);
 

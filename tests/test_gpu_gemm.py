@@ -68,8 +68,8 @@ def test_prefill_other_formats_at_size(F, O):
 
 def test_rows_are_independent_of_the_batch(F, O):
     # A row of a T-row prefill is bit-identical to the same row computed in a smaller batch, as long as
-    # both launches have enough output tiles to run without splitting K (with a K split the slices are
-    # added atomically, so only the tolerance holds there, not bit equality).
+    # both launches have enough output tiles to run without splitting K (a K split changes where the sum over K is cut,
+    # so across batch sizes only the tolerance holds there, not bit equality).
     from ferric_amd.synth import synth_weights
     w = synth_weights(Q4_K, 5120, 512, 5)
     qm = F.QMatrix.from_bytes(w, Q4_K, 5120, 512)
@@ -81,6 +81,27 @@ def test_rows_are_independent_of_the_batch(F, O):
     assert np.array_equal(big[256:].view(np.uint32), part.view(np.uint32))
     again = F.Tensor.from_bf16_bits(xb, (1536, 512)).gemm_q_bf16(qm).to_vec().reshape(1536, 5120)
     assert np.array_equal(big.view(np.uint32), again.view(np.uint32))
+
+
+@pytest.mark.parametrize("ty,t,n,k", [(Q4_K, 128, 5120, 5120), (Q4_K, 512, 5120, 5120), (Q4_K, 2048, 5120, 5120),
+                                      (Q6_K, 300, 1000, 4096), (Q8_0, 200, 1300, 2080), (Q4_K, 70, 3000, 8192)])
+def test_two_runs_give_identical_bits(F, O, ty, t, n, k):
+    # Launches with fewer whole tiles than the chip has workgroups cut tiles along K (every shape here does; 2048 x 5120
+    # has one whole round and a cut remainder). The partial tiles are summed in a fixed order, so the bits may not depend
+    # on which workgroup finishes first: five runs, with other work on the device in between, one result.
+    from ferric_amd.synth import synth_weights
+    lib = F._lib.load()
+    w = synth_weights(ty, n, k, 31)
+    qm = F.QMatrix.from_bytes(w, ty, n, k)
+    assert lib.fhip_workspace_bytes_coop(qm.handle, None, t) > 0, "the case is meant to cut tiles along K"
+    xb, _ = bf16_round(np.random.default_rng(32).standard_normal((t, k)).astype(np.float32))
+    x = F.Tensor.from_bf16_bits(xb, (t, k))
+    first = x.gemm_q_bf16(qm).to_vec().view(np.uint32)
+    other = F.QMatrix.from_bytes(synth_weights(Q4_K, 512, 1024, 33), Q4_K, 512, 1024)
+    xo = F.Tensor.from_bf16_bits(bf16_round(np.ones((40, 1024), np.float32))[0], (40, 1024))
+    for _ in range(4):
+        xo.gemm_q_bf16(other)              # another launch that uses the same workspace
+        assert np.array_equal(first, x.gemm_q_bf16(qm).to_vec().view(np.uint32))
 
 
 def test_q8_0_rows_ending_inside_a_chunk(F, O):
