@@ -170,14 +170,14 @@ void release_workspace(hipStream_t s) {
 
 // The matrix-core GEMM with its K-split scratch (partial tiles of the tiles that several workgroups share) taken from the
 // stream's library workspace.
-static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared, const char* who) {
+static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, const char* who) {
     const size_t need = fhip::gemm_bf16_ws_bytes(w, t);
     void* ws = nullptr;
     if (need) {
         int rc = lib_workspace(s, need, &ws, who);
         if (rc) return rc;
     }
-    return fhip::launch_gemm_bf16(w, d_x, t, d_y, s, y_cleared, (float*)ws, need);
+    return fhip::launch_gemm_bf16(w, d_x, t, d_y, s, (float*)ws, need);
 }
 
 // ---- which kernel a batch takes ---------------------------------------------------------------------------------------------
@@ -673,7 +673,7 @@ int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float*
     if (t == 0 || w->rows == 0) return FHIP_OK;
     if (!d_y || (!d_x && w->cols)) return set_error(FHIP_ERR_ARG, "fhip_gemm_q_bf16: NULL pointer");
     if (w->cols == 0) return zero_outputs(t, w->rows, d_y, (hipStream_t)stream);   // empty inner dimension: every dot product is 0
-    return gemm_bf16_lib_ws(w, d_x, t, d_y, (hipStream_t)stream, false, "fhip_gemm_q_bf16");
+    return gemm_bf16_lib_ws(w, d_x, t, d_y, (hipStream_t)stream, "fhip_gemm_q_bf16");
 }
 
 // ---- mixture-of-experts entry points (crates/ferric-tensor/src/dtype.rs:1582-1780) ----------------------
@@ -931,10 +931,8 @@ int fhip_matmul_q_coop(const fhip_weight* w, const float* d_x, size_t rows_x, fl
     if (rows_x == 0 || w->rows == 0) return FHIP_OK;
     if (w->cols == 0) return d_y ? zero_outputs(rows_x, w->rows, d_y, (hipStream_t)stream) : set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL pointer");
     if (!d_x || !d_y || !d_ws_bf16) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_coop: NULL pointer");
-    const bool clr = fhip::gemm_bf16_adds_into_y(rows_x);
-    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * w->cols, d_ws_bf16, (hipStream_t)stream, clr ? d_y : nullptr, clr ? rows_x * w->rows : 0)))
-        return rc;
-    return gemm_bf16_lib_ws(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream, clr, "fhip_matmul_q_coop");
+    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * w->cols, d_ws_bf16, (hipStream_t)stream))) return rc;
+    return gemm_bf16_lib_ws(w, d_ws_bf16, rows_x, d_y, (hipStream_t)stream, "fhip_matmul_q_coop");
 }
 
 
@@ -961,11 +959,10 @@ int fhip_ffn_coop(const fhip_weight* gu, const fhip_weight* down, const float* d
     float* g = (float*)(ws + align256(rows_x * gu->cols * 2));
     uint16_t* hb = (uint16_t*)((uint8_t*)g + align256(rows_x * gu->rows * 4));
     hipStream_t s = (hipStream_t)stream;
-    const bool clr = fhip::gemm_bf16_adds_into_y(rows_x);   // then each conversion clears the next GEMM's output on the side
-    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * gu->cols, xb, s, clr ? g : nullptr, clr ? rows_x * gu->rows : 0))) return rc;
-    if ((rc = gemm_bf16_lib_ws(gu, xb, rows_x, g, s, clr, "fhip_ffn_coop"))) return rc;
-    if ((rc = fhip::launch_swiglu_bf16(g, rows_x, n_ff, hb, s, clr ? d_y : nullptr, clr ? rows_x * down->rows : 0))) return rc;
-    return gemm_bf16_lib_ws(down, hb, rows_x, d_y, s, clr, "fhip_ffn_coop");
+    if ((rc = fhip::launch_cvt_bf16(d_x, rows_x * gu->cols, xb, s))) return rc;
+    if ((rc = gemm_bf16_lib_ws(gu, xb, rows_x, g, s, "fhip_ffn_coop"))) return rc;
+    if ((rc = fhip::launch_swiglu_bf16(g, rows_x, n_ff, hb, s))) return rc;
+    return gemm_bf16_lib_ws(down, hb, rows_x, d_y, s, "fhip_ffn_coop");
 }
 
 size_t fhip_matmul_q_f16x2_ws_bytes(const fhip_weight* w, size_t rows_x) {

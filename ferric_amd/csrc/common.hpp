@@ -104,16 +104,12 @@ int launch_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t
 int launch_moe_wsum(const float* d_parts, const float* d_selw, size_t t, int k, size_t out_pe, float* d_y, hipStream_t s);
 
 // gemm_mfma.hip
-// y_cleared: the caller has zeroed y on this stream already (see gemm_bf16_adds_into_y)
-// d_ws / ws_bytes: gemm_bf16_ws_bytes(w, t) bytes of scratch for launches that cut tiles along K (0: none needed)
-int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared = false,
-                     float* d_ws = nullptr, size_t ws_bytes = 0);
+// d_ws / ws_bytes: gemm_bf16_ws_bytes(w, t) bytes of scratch for launches that cut output tiles along K (0: none needed)
+int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, float* d_ws = nullptr, size_t ws_bytes = 0);
 size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t);
-bool gemm_bf16_adds_into_y(size_t t);   // true: a launch for t rows may add into y, so a cleared y saves it a launch
-// conversions in front of the GEMM; each can also clear `zero_n` floats at `zero`
-int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s, float* zero = nullptr, size_t zero_n = 0);
-int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s, float* zero = nullptr,
-                       size_t zero_n = 0);
+// conversions in front of the GEMM
+int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s);
+int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s);
 
 // gemm_f16x2.hip: 2..32 activation rows in one pass over the weights, f16 matrix cores, f32-grade results
 bool gemm_f16x2_supports(const fhip_weight* w, size_t t);

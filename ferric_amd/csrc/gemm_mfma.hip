@@ -501,7 +501,8 @@ __global__ void __launch_bounds__(256) sum_split_tiles_kernel(float* __restrict_
 // activations of a chunk (TP rows x 256 columns, TP = 8 or 32) are staged once per workgroup in LDS, double
 // buffered, one barrier per chunk. The (128-row group, chunk) units, chunk fastest, are dealt to the
 // workgroups in equal contiguous runs, two to four workgroups per CU; a segment that covers its group's whole K
-// stores its tile, any other adds it atomically into a Y cleared beforehand.
+// stores its tile, any other stores partial sums into the workspace slot (group, contributor) and sum_split_groups_kernel
+// adds a group's slots in contributor order afterwards, as for the tiled kernel.
 // ------------------------------------------------------------------------------------------------
 struct SkinnyParams {
     const uint8_t* W;
@@ -513,6 +514,8 @@ struct SkinnyParams {
     int nchunks;
     long long units;   // 128-row groups * nchunks
     int per;           // units per workgroup
+    float* ws;         // partial sums of groups that several runs share: [group][contributor][TP x 128]
+    int kmax;          // contributor slots per group
 };
 
 constexpr int XROW = CHUNK + 8;   // bf16 per staged activation row of a chunk (+16 B pad)
@@ -613,48 +616,87 @@ __global__ void __launch_bounds__(256, TP == 8 ? 4 : 2) gemm_q_bf16_skinny_kerne
             });
             raw = nxt;
         }
+        // runs are numbered by blockIdx.x; the first run that touches group grp is the one that holds unit grp * nchunks
+        float* part = whole ? nullptr
+                            : p.ws + ((size_t)grp * p.kmax + ((int)blockIdx.x - (int)(((long long)grp * nchunks) / p.per))) * (size_t)(TP * 128) + wave * 32 + c;
         if (n < p.N) {
 #pragma unroll
             for (int r = 0; r < (TP == 8 ? 4 : 16); r++) {
                 const int t = 8 * (r >> 2) + 4 * h + (r & 3);
                 if (t < p.T) {
-                    float* y = p.Y + (size_t)t * p.N + n;
-                    if (whole) *y = acc[r];
-                    else unsafeAtomicAdd(y, acc[r]);
+                    if (whole) p.Y[(size_t)t * p.N + n] = acc[r];
+                    else part[t * 128] = acc[r];
                 }
             }
         }
     }
 }
 
-__global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = 0.f;
+// Group `blockIdx.x` of 128 outputs, if more than one run contributed to it: Y = slot 0 + slot 1 + ... in that order.
+// Thread = output column (threadIdx.x & 127) of row 2 * blockIdx.y + (threadIdx.x >> 7); eight slots are requested at a time.
+__global__ void __launch_bounds__(256) sum_split_groups_kernel(float* __restrict__ Y, const float* __restrict__ ws, int T, int N, int TP,
+                                                             int nchunks, int per, int kmax) {
+    const int grp = blockIdx.x;
+    const long long u0 = (long long)grp * nchunks;
+    const int nk = (int)((u0 + nchunks - 1) / per) - (int)(u0 / per) + 1;
+    if (nk == 1) return;
+    const int col = threadIdx.x & 127, n = grp * 128 + col, t = 2 * blockIdx.y + (threadIdx.x >> 7);
+    if (n >= N || t >= T) return;
+    const size_t slot = (size_t)TP * 128;
+    const float* q = ws + (size_t)grp * kmax * slot + t * 128 + col;
+    float a = q[0];
+    for (int k0 = 1; k0 < nk; k0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = q[(size_t)(k0 + j < nk ? k0 + j : 0) * slot];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (k0 + j < nk) a += v[j];
+    }
+    Y[(size_t)t * N + n] = a;
 }
 
+struct SkinnyPlan { long long groups, units, per; unsigned grid; int kmax; int tp; bool split; };
+
+static SkinnyPlan plan_skinny(size_t rows, int nchunks, size_t t, long long cus) {
+    SkinnyPlan q;
+    q.groups = ((long long)rows + 127) / 128;
+    q.units = q.groups * nchunks;
+    q.tp = t <= 8 ? 8 : 32;
+    // workgroups per CU as the register budget allows: four with 8 activation rows staged, two with 32
+    const long long wgs = cus * (t <= 8 ? 4 : 2);
+    long long per = (q.units + wgs - 1) / wgs;
+    if (per * 4 >= (long long)nchunks * 3 && per < nchunks) per = nchunks;   // nearly whole groups: make them whole
+    if (per < 1) per = 1;
+    q.per = per;
+    q.grid = (unsigned)((q.units + per - 1) / per);
+    q.split = per % nchunks != 0;
+    // a group's nchunks units lie in at most this many runs of `per`
+    q.kmax = q.split ? (int)((nchunks + per - 2) / per) + 1 : 1;
+    return q;
+}
+
+static size_t skinny_ws_bytes(const SkinnyPlan& q) { return q.split ? (size_t)q.groups * q.kmax * q.tp * 128 * sizeof(float) : 0; }
+
 template <class F>
-int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, float* d_ws, size_t ws_bytes) {
     SkinnyParams p;
     p.W = w->d_raw; p.X = d_x; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
     p.nblk = (int)(w->row_bytes / F::BLOCK);
     p.nchunks = F::chunks(p.K);
-    const long long groups = ((long long)w->rows + 127) / 128;
-    p.units = groups * p.nchunks;
-    // workgroups per CU as the register budget allows: four with 8 activation rows staged, two with 32
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    const long long wgs = cus * (t <= 8 ? 4 : 2);
-    long long per = (p.units + wgs - 1) / wgs;
-    if (per * 4 >= (long long)p.nchunks * 3 && per < p.nchunks) per = p.nchunks;   // nearly whole groups: make them whole
-    if (per < 1) per = 1;
-    p.per = (int)per;
-    const unsigned grid = (unsigned)((p.units + per - 1) / per);
-    if (per % p.nchunks != 0 && !y_cleared) {
-        const size_t n = t * w->rows;
-        hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
-    }
-    if (t <= 8) hipLaunchKernelGGL((gemm_q_bf16_skinny_kernel<F, 8>), dim3(grid), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((gemm_q_bf16_skinny_kernel<F, 32>), dim3(grid), dim3(256), 0, s, p);
+    const SkinnyPlan q = plan_skinny(w->rows, p.nchunks, t, cus);
+    p.units = q.units;
+    p.per = (int)q.per;
+    p.ws = d_ws; p.kmax = q.kmax;
+    if (q.split && (!d_ws || ws_bytes < skinny_ws_bytes(q)))
+        return fhip::set_error(FHIP_ERR_ARG, "gemm_q_bf16: the launch cuts row groups along K and needs %zu bytes of workspace", skinny_ws_bytes(q));
+    if (t <= 8) hipLaunchKernelGGL((gemm_q_bf16_skinny_kernel<F, 8>), dim3(q.grid), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((gemm_q_bf16_skinny_kernel<F, 32>), dim3(q.grid), dim3(256), 0, s, p);
+    if (q.split)
+        hipLaunchKernelGGL(sum_split_groups_kernel, dim3((unsigned)q.groups, (unsigned)((t + 1) / 2)), dim3(256), 0, s, d_y, (const float*)d_ws, p.T, p.N, q.tp, p.nchunks,
+                           p.per, p.kmax);
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
@@ -752,15 +794,15 @@ static int choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
 
 template <class F>
 static size_t ws_bytes_fmt(const fhip_weight* w, size_t t) {
-    if (t <= 32) return 0;
+    if (t <= 32) return skinny_ws_bytes(plan_skinny(w->rows, F::chunks((int)w->cols), t, fhip::device_cus() > 0 ? fhip::device_cus() : 256));
     TilePlan q;
     const int mi = choose_plan<F>(w, t, q);
     return plan_ws_bytes(q, mi);
 }
 
 template <class F>
-int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_ws, size_t ws_bytes) {
-    if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, y_cleared);
+int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, float* d_ws, size_t ws_bytes) {
+    if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, d_ws, ws_bytes);
     // Tile height 64 * MI. The 256 x 256 tile unpacks each weight once per 256 activation rows, but when there is no whole
     // round of such tiles for the chip every tile is cut along K, each workgroup writes a whole partial tile for a few
     // chunks of work, and a lower tile (twice the tiles, half the fix-up, longer runs) can win: the estimate decides
@@ -775,16 +817,8 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     return launch_cfg<F, 1>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
 }
 
-// f32 -> bf16 (round to nearest even), 8 values per thread; `n8` full groups of 8, the tail one by one
-// Both conversion kernels can clear a f32 region on the side (`zero`, `zero_n` values): the output of the
-// T <= 32 GEMM that follows, which adds K slices atomically, so that it needs no clearing launch of its own.
-__device__ __forceinline__ void zero_on_the_side(float* __restrict__ zero, size_t zero_n) {
-    for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < zero_n; k += (size_t)gridDim.x * blockDim.x) zero[k] = 0.f;
-}
-
-__global__ void __launch_bounds__(256) cvt_f32_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, size_t n,
-                                                         float* __restrict__ zero, size_t zero_n) {
-    zero_on_the_side(zero, zero_n);
+// f32 -> bf16 (round to nearest even), 8 values per thread, the tail one by one
+__global__ void __launch_bounds__(256) cvt_f32_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, size_t n) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
     if (i >= n) return;
     if (i + 8 <= n) {
@@ -798,9 +832,7 @@ __global__ void __launch_bounds__(256) cvt_f32_bf16_kernel(const float* __restri
 
 // SwiGLU of a [t, 2d] = [gate | up] f32 matrix, written as bf16 [t, d] for the down projection's A operand.
 // Same arithmetic as the un-fused f32 op (crates/ferric-tensor/src/lib.rs:2603-2618), then one RNE rounding.
-__global__ void __launch_bounds__(256) swiglu_bf16_kernel(const float* __restrict__ gu, size_t n, size_t d, uint16_t* __restrict__ out,
-                                                        float* __restrict__ zero, size_t zero_n) {
-    zero_on_the_side(zero, zero_n);
+__global__ void __launch_bounds__(256) swiglu_bf16_kernel(const float* __restrict__ gu, size_t n, size_t d, uint16_t* __restrict__ out) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const size_t row = i / d, col = i % d;
@@ -812,21 +844,19 @@ __global__ void __launch_bounds__(256) swiglu_bf16_kernel(const float* __restric
 
 namespace fhip {
 
-int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s, float* zero, size_t zero_n) {
+int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s) {
     const size_t n = t * d;
     if (n == 0) return FHIP_OK;
-    hipLaunchKernelGGL(swiglu_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gu, n, d, d_out, zero, zero_n);
+    hipLaunchKernelGGL(swiglu_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_gu, n, d, d_out);
     return check_hip(hipGetLastError(), "swiglu_bf16 launch");
 }
 
-int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s, float* zero, size_t zero_n) {
+int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s) {
     if (n == 0) return FHIP_OK;
     if ((((uintptr_t)d_x | (uintptr_t)d_out) & 15) != 0) return set_error(FHIP_ERR_ARG, "cvt_f32_bf16: pointers must be 16-byte aligned");
-    hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s, d_x, d_out, n, zero, zero_n);
+    hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s, d_x, d_out, n);
     return check_hip(hipGetLastError(), "cvt_f32_bf16 launch");
 }
-
-bool gemm_bf16_adds_into_y(size_t t) { return t <= 32; }
 
 size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t) {
     if (!w || t == 0 || w->rows == 0) return 0;
@@ -838,15 +868,15 @@ size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t) {
     }
 }
 
-int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_ws, size_t ws_bytes) {
+int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, float* d_ws, size_t ws_bytes) {
     if (t == 0 || w->rows == 0) return FHIP_OK;
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "gemm_q_bf16: x must be 16-byte aligned");
     if ((unsigned long long)t * w->cols >= (1ull << 31))
         return set_error(FHIP_ERR_SHAPE, "gemm_q_bf16: t * cols must be below 2^31 (got %zu x %zu)", t, w->cols);
     switch (w->type) {
-        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s, y_cleared, d_ws, ws_bytes);
-        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s, y_cleared, d_ws, ws_bytes);
-        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_x, t, d_y, s, y_cleared, d_ws, ws_bytes);
+        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s, d_ws, ws_bytes);
+        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s, d_ws, ws_bytes);
+        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_x, t, d_y, s, d_ws, ws_bytes);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

@@ -198,10 +198,9 @@ int fhip_ffn(const fhip_weight* gate_up, const fhip_weight* down, const float* d
 
 /* Prefill dequant-GEMM, stands for crates/ferric-tensor/src/dtype.rs:1818 matmul_q4_k_coop (:1199
  * Q6_K, :1316 Q8_0): x is bf16 [t, cols] (raw 16-bit patterns), y f32 [t, rows]; weights are
- * dequantized tile by tile into LDS as bf16 and contracted on the matrix cores, f32 accumulate. For more than 32
- * rows a launch that cuts output tiles along K keeps their partial tiles in the library's workspace of the stream
- * (fhip_workspace_bytes_coop) and adds them in a fixed order: the same inputs give the same bits on every run. Up to
- * 32 rows the K slices are added with f32 atomics (last bits may differ run to run). */
+ * dequantized tile by tile into LDS as bf16 and contracted on the matrix cores, f32 accumulate. A launch that cuts
+ * output tiles along K keeps their partial tiles in the library's workspace of the stream (fhip_workspace_bytes_coop)
+ * and adds them in a fixed order: the same inputs give the same bits on every run. */
 int fhip_gemm_q_bf16(const fhip_weight* w, const uint16_t* d_x_bf16, size_t t, float* d_y, void* stream);
 
 /* ---- mixture-of-experts decode: the "_id" variants that sit behind the same matmul entry points ---------- */
