@@ -489,6 +489,13 @@ def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
             ms = timer.time_ms(g.launch) / reps
             tf = 2.0 * t * n * k / (ms * 1e-3) / 1e12
             out[str(t)] = {"ms": ms, "TFLOPs": tf, "frac_of_bf16_mfma_peak": tf / 2500.0}
+            if t == max(ts):
+                # The same launches (same graph, same instruction stream) on activations that are all zero: the difference is
+                # what the switching activity of the operands costs in clock, i.e. how far the kernel is power-bound.
+                check(lib.fhip_memset(x.buf.ptr, 0, 2 * t * k, stream.handle))
+                g.launch()
+                ms0 = timer.time_ms(g.launch) / reps
+                out[str(t)]["ms_on_zero_activations"] = ms0
         res[name] = out
     return res
 
@@ -526,7 +533,8 @@ def probe(F, lib, check):
 
 def probe_prefill(F, lib, check):
     """Work for a profiler run of the matrix-core kernels: Q4_K 5120x5120 and 34816x5120 at T = 2048 (tiled kernel),
-    T = 128 (tiled, K split) and T = 8 (the T <= 32 kernel), 5 launches each."""
+    T = 128 (tiled, K split) and T = 8 (the T <= 32 kernel), 5 launches each; last, 5 more launches of 34816x5120 at
+    T = 2048 on activations that are all zero (the same instruction stream with idle multipliers: what the clock does)."""
     from ferric_amd.synth import synth_weights
     for n, k in ((5120, 5120), (34816, 5120)):
         qm = F.QMatrix.from_bytes(synth_weights(Q4_K, n, k, 1), Q4_K, n, k)
@@ -537,6 +545,12 @@ def probe_prefill(F, lib, check):
             for _ in range(5):
                 check(lib.fhip_gemm_q_bf16(qm.handle, x.buf.ptr, t, y.buf.ptr, None))
             check(lib.fhip_stream_sync(None))
+    t = 2048
+    x = F.Tensor.from_bf16_bits(np.zeros((t, k), np.uint16), (t, k))
+    y = F.Tensor.empty((t, n))
+    for _ in range(5):
+        check(lib.fhip_gemm_q_bf16(qm.handle, x.buf.ptr, t, y.buf.ptr, None))
+    check(lib.fhip_stream_sync(None))
 
 
 def probe_f16x2(F, lib, check, ncopy=4):
