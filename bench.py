@@ -217,7 +217,8 @@ def bench_ffn(F, lib, check, stream, timer, batches, reps=20, ncopy=4):
         ws, y = F.Tensor.empty((b, n_ff)), F.Tensor.empty((b, n_embd))
         # fhip_ffn, the drop-in entry point: the mat-vec kernels for one and two rows, the one-pass f16 hi/lo kernels from three
         # rows on (out of the library's workspace, reserved here because a capturing stream cannot allocate)
-        check(lib.fhip_workspace_reserve(stream.handle, lib.fhip_workspace_bytes(gus[0].handle, dns[0].handle, b)))
+        check(lib.fhip_workspace_reserve(stream.handle, max(lib.fhip_workspace_bytes(gus[0].handle, dns[0].handle, b),
+                                                            lib.fhip_workspace_bytes_coop(gus[0].handle, dns[0].handle, b))))
         f32 = lambda gu, dn: check(lib.fhip_ffn(gu.handle, dn.handle, x.buf.ptr, b, y.buf.ptr, ws.buf.ptr, stream.handle))
         res[str(b)] = entry(timed(f32, ncopy), b)
         res[str(b)]["warm_one_copy_ms"] = timed(f32, 1)
