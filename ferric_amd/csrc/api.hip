@@ -203,14 +203,13 @@ int zero_outputs(size_t t, size_t rows, float* d_y, hipStream_t s) {
 }
 
 // y [t, w->rows] = x [t, cols] W^T for t rows of one group; ws: f16x2_matmul_ws(w, t) bytes
-size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) { return align256(fhip::gemm_f16x2_xp_bytes(w, t)) + align256(fhip::gemm_f16x2_aux_bytes()); }
+size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) { return align256(fhip::gemm_f16x2_xp_bytes(w, t)); }
 int f16x2_matmul(const fhip_weight* w, const float* d_x, size_t t, bool swiglu_in, float* d_y, void* d_ws, hipStream_t s) {
     uint16_t* xp = (uint16_t*)d_ws;
-    float* rs = (float*)((uint8_t*)d_ws + align256(fhip::gemm_f16x2_xp_bytes(w, t)));
     const bool clr = fhip::gemm_f16x2_adds_into_y(w, t);   // then the split clears y on the side
-    int rc = fhip::launch_xsplit_f16(w, d_x, t, swiglu_in, xp, rs, s, clr ? d_y : nullptr, clr ? t * w->rows : 0);
+    int rc = fhip::launch_xsplit_f16(w, d_x, t, swiglu_in, xp, s, clr ? d_y : nullptr, clr ? t * w->rows : 0);
     if (rc) return rc;
-    return fhip::launch_gemm_f16x2(w, xp, rs, t, d_y, s, clr);
+    return fhip::launch_gemm_f16x2(w, xp, t, d_y, s, clr);
 }
 
 }  // namespace
@@ -967,7 +966,7 @@ int fhip_ffn_coop(const fhip_weight* gu, const fhip_weight* down, const float* d
 
 size_t fhip_matmul_q_f16x2_ws_bytes(const fhip_weight* w, size_t rows_x) {
     if (!fhip::gemm_f16x2_supports(w, rows_x)) return 0;
-    return align256(fhip::gemm_f16x2_xp_bytes(w, rows_x)) + align256(fhip::gemm_f16x2_aux_bytes());
+    return align256(fhip::gemm_f16x2_xp_bytes(w, rows_x));
 }
 
 static int f16x2_checks(const char* who, const fhip_weight* w, size_t rows_x) {
@@ -990,16 +989,15 @@ int fhip_matmul_q_f16x2(const fhip_weight* w, const float* d_x, size_t rows_x, f
     if (((uintptr_t)d_ws & 255) != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_f16x2: workspace must be 256-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     uint16_t* xp = (uint16_t*)d_ws;
-    float* rs = (float*)((uint8_t*)d_ws + align256(fhip::gemm_f16x2_xp_bytes(w, rows_x)));
     const bool clr = fhip::gemm_f16x2_adds_into_y(w, rows_x);   // then the split clears y on the side
-    if ((rc = fhip::launch_xsplit_f16(w, d_x, rows_x, false, xp, rs, s, clr ? d_y : nullptr, clr ? rows_x * w->rows : 0))) return rc;
-    return fhip::launch_gemm_f16x2(w, xp, rs, rows_x, d_y, s, clr);
+    if ((rc = fhip::launch_xsplit_f16(w, d_x, rows_x, false, xp, s, clr ? d_y : nullptr, clr ? rows_x * w->rows : 0))) return rc;
+    return fhip::launch_gemm_f16x2(w, xp, rows_x, d_y, s, clr);
 }
 
 size_t fhip_ffn_f16x2_ws_bytes(const fhip_weight* gu, const fhip_weight* down, size_t rows_x) {
     if (!fhip::gemm_f16x2_supports(gu, rows_x) || !fhip::gemm_f16x2_supports(down, rows_x)) return 0;
     return align256(fhip::gemm_f16x2_xp_bytes(gu, rows_x)) + align256(rows_x * gu->rows * 4) +
-           align256(fhip::gemm_f16x2_xp_bytes(down, rows_x)) + 2 * align256(fhip::gemm_f16x2_aux_bytes());
+           align256(fhip::gemm_f16x2_xp_bytes(down, rows_x));
 }
 
 int fhip_ffn_f16x2(const fhip_weight* gu, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y, void* d_ws,
@@ -1017,16 +1015,14 @@ int fhip_ffn_f16x2(const fhip_weight* gu, const fhip_weight* down, const float* 
     hipStream_t s = (hipStream_t)stream;
     uint8_t* ws = (uint8_t*)d_ws;
     uint16_t* xp1 = (uint16_t*)ws;
-    float* rs1 = (float*)(ws + align256(fhip::gemm_f16x2_xp_bytes(gu, rows_x)));
-    float* g = (float*)((uint8_t*)rs1 + align256(fhip::gemm_f16x2_aux_bytes()));
+    float* g = (float*)(ws + align256(fhip::gemm_f16x2_xp_bytes(gu, rows_x)));
     uint16_t* xp2 = (uint16_t*)((uint8_t*)g + align256(rows_x * gu->rows * 4));
-    float* rs2 = (float*)((uint8_t*)xp2 + align256(fhip::gemm_f16x2_xp_bytes(down, rows_x)));
     const bool clr1 = fhip::gemm_f16x2_adds_into_y(gu, rows_x), clr2 = fhip::gemm_f16x2_adds_into_y(down, rows_x);
-    if ((rc = fhip::launch_xsplit_f16(gu, d_x, rows_x, false, xp1, rs1, s, clr1 ? g : nullptr, clr1 ? rows_x * gu->rows : 0))) return rc;
-    if ((rc = fhip::launch_gemm_f16x2(gu, xp1, rs1, rows_x, g, s, clr1))) return rc;
+    if ((rc = fhip::launch_xsplit_f16(gu, d_x, rows_x, false, xp1, s, clr1 ? g : nullptr, clr1 ? rows_x * gu->rows : 0))) return rc;
+    if ((rc = fhip::launch_gemm_f16x2(gu, xp1, rows_x, g, s, clr1))) return rc;
     // SwiGLU of [gate | up] is computed while the rows are split for the down projection
-    if ((rc = fhip::launch_xsplit_f16(down, g, rows_x, true, xp2, rs2, s, clr2 ? d_y : nullptr, clr2 ? rows_x * down->rows : 0))) return rc;
-    return fhip::launch_gemm_f16x2(down, xp2, rs2, rows_x, d_y, s, clr2);
+    if ((rc = fhip::launch_xsplit_f16(down, g, rows_x, true, xp2, s, clr2 ? d_y : nullptr, clr2 ? rows_x * down->rows : 0))) return rc;
+    return fhip::launch_gemm_f16x2(down, xp2, rows_x, d_y, s, clr2);
 }
 
 int fhip_matvec_q8_0_host(const float* h_x, const uint8_t* h_w, size_t w_len, size_t rows, size_t cols, float* h_y) {

@@ -115,13 +115,11 @@ int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, h
 bool gemm_f16x2_supports(const fhip_weight* w, size_t t);
 size_t gemm_f16x2_xp_bytes(const fhip_weight* w, size_t t);       // prepared-activation buffer for t rows
 bool gemm_f16x2_adds_into_y(const fhip_weight* w, size_t t);      // true: the launch adds into y, a cleared y saves it a launch
-size_t gemm_f16x2_aux_bytes();                                    // row scales + partial row maxima, behind the buffer above
-// splits the rows of x [t, cols] (swiglu: of silu(gate) * up of x [t, 2 cols]) into scaled f16 hi / lo operand rows;
-// d_aux: gemm_f16x2_aux_bytes() bytes, its first t floats are the row scales launch_gemm_f16x2 takes as d_rs
-int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, float* d_aux, hipStream_t s,
-                      float* zero = nullptr, size_t zero_n = 0);
-int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, size_t t, float* d_y, hipStream_t s,
-                      bool y_cleared = false);
+// splits the rows of x [t, cols] (swiglu: of silu(gate) * up of x [t, 2 cols]) chunk by chunk into scaled f16 hi / lo
+// operand rows, each carrying the factor that takes its scale out again
+int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero = nullptr,
+                      size_t zero_n = 0);
+int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared = false);
 
 // decode_ops.hip: the steps either side of the matmuls in a decode layer
 int launch_rmsnorm(const float* a, const float* b, const float* weight, size_t rows, size_t d, float eps, float* sum_out, float* norm_out,

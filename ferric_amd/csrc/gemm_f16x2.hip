@@ -13,10 +13,12 @@
 //     |sc*(q-32)| can reach 4096; products above 2048 are rounded to even, a relative 2^-12 on those weights.)
 //     Q8_0 (:2948-2990) is d * (int8): the B operand holds the quant, the f32 result of every 32-wide slice takes its
 //     block's d.
-//   * Activations. A row is scaled by a power of two so that its largest magnitude lies in [2^14, 2^15), then split
-//     into hi = f16(x) and lo = f16(x - hi): two operand rows per activation row, 22 significant bits. The 16 rows of
-//     a v_mfma_f32_16x16x32_f16 hold hi and lo of 8 activation rows; the two partial results are added in f32 at the
-//     end and the scale is taken out again.
+//   * Activations. The 256 columns of a chunk of a row are scaled by a power of two so that their largest magnitude
+//     lies in [2^14, 2^15), then split into hi = f16(x) and lo = f16(x - hi): two operand rows per activation row, 22
+//     significant bits at the chunk's maximum. The 16 rows of a v_mfma_f32_16x16x32_f16 hold hi and lo of 8 activation
+//     rows; a chunk's f32 result takes the chunk's scale out again as it joins the total, and the two partial results
+//     are added in f32 at the end. (A scale per chunk, not per row: the preparation needs no pass over the whole row in
+//     front of it -- one launch less per matmul -- and a chunk of small values keeps its bits beside a large one.)
 //   * Unpack cost. A lane turns a dword of 8 nibbles into 8 f16 with 1 shift, 4 and-or (the nibble lands in the
 //     mantissa of the f16 constant 1024 or, for the high nibble, 16 positions up) and 4 packed f16 fma that remove the
 //     constant and apply the sub-block scale: 9 VALU for 8 weights, against ~30 for the bf16 path's f32 arithmetic.
@@ -67,9 +69,11 @@ constexpr uint32_t H16TH = 0x2C002C00u;      // (1/16, 1/16)
 struct __attribute__((packed, aligned(2))) U4A2 { u32x4 v; };   // 16 bytes at an address that is only 2-byte aligned
 
 constexpr int CHUNK = 256;   // columns per chunk: one K-quant super-block
-// f16 per staged operand row of a chunk: 256 activations, 8 sub-block sums, 8 zeros, 8 of padding (row stride 35 x 16
-// bytes: the 16 rows a 16-byte read instruction touches fall into different bank groups)
+// f16 per staged operand row of a chunk: 256 activations, 8 sub-block sums, 8 zeros, then the f32 factor that takes the
+// chunk's scale out again (two f16 places) and 6 of padding (row stride 35 x 16 bytes: the 16 rows a 16-byte read
+// instruction touches fall into different bank groups)
 constexpr int XR = 280;
+constexpr int XSCALE = 272;   // column of the f32 factor
 
 __host__ __device__ constexpr int p4(int j) { return ((j & 1) << 1) | (j >> 1); }   // 0, 2, 1, 3: byte pairs (b0,b2), (b1,b3)
 
@@ -329,12 +333,12 @@ struct Q80 {
 };
 
 // ------------------------------------------------------------------------------------------------
-// Activation preparation, two short kernels. Output per chunk: 16 NT operand rows of XR f16 (rows 16 q + i, i < 8: hi of
+// Activation preparation, one short kernel. Output per chunk: 16 NT operand rows of XR f16 (rows 16 q + i, i < 8: hi of
 // activation row 8 q + i; rows 16 q + 8 + i: its lo), columns in operand order (F::pos_of), followed by the 8 sub-block
-// sums / 64 (formats with minima) and zeros. rs[t] is the factor that takes the row's power-of-two scale out again.
+// sums / 64 (formats with minima), zeros, and the f32 factor that takes the chunk's power-of-two scale out again.
 // SWIGLU: the row is silu(gate) * up of a [T, 2d] = [gate | up] matrix (crates/ferric-tensor/src/lib.rs:2603-2618).
 // ------------------------------------------------------------------------------------------------
-constexpr int MAXW = 64;   // partial maxima per row: one per 1024 columns, rows of up to 65 536 columns
+constexpr int MAXW = 64;   // rows of up to 65 536 columns
 
 template <bool SWIGLU>
 __device__ __forceinline__ float act(const float* __restrict__ x, int K, int k) {
@@ -345,70 +349,61 @@ __device__ __forceinline__ float act(const float* __restrict__ x, int K, int k) 
     return x[k];
 }
 
-// mx[t * MAXW + b] = largest magnitude among columns [1024 b, 1024 b + 1024) of activation row t
-template <bool SWIGLU>
-__global__ void __launch_bounds__(256) rowmax_kernel(const float* __restrict__ X, int K, float* __restrict__ mx) {
-    __shared__ float red[4];
-    const int tid = threadIdx.x, t = blockIdx.y;
-    const float* x = X + (size_t)t * (SWIGLU ? 2 * (size_t)K : (size_t)K);
-    float m = 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int k = blockIdx.x * 1024 + 256 * j + tid;
-        if (k < K) m = fmaxf(m, fabsf(act<SWIGLU>(x, K, k)));
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-    if ((tid & 63) == 0) red[tid >> 6] = m;
-    __syncthreads();
-    if (tid == 0) mx[t * MAXW + blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-}
-
-// one workgroup per (chunk, operand row group of 8): thread k of it converts column k of the chunk
+// one workgroup per (chunk, operand row of a group of 8): thread k of it converts column k of the chunk
 template <class F, bool SWIGLU>
-__global__ void __launch_bounds__(256) xsplit_f16_kernel(const float* __restrict__ X, int T, int K, int NT, const float* __restrict__ mx,
-                                                       int nmx, uint16_t* __restrict__ Xp, float* __restrict__ rs,
+__global__ void __launch_bounds__(256) xsplit_f16_kernel(const float* __restrict__ X, int T, int K, int NT, uint16_t* __restrict__ Xp,
                                                        float* __restrict__ zero, size_t zero_n) {
+    __shared__ float red[4];
     const int tid = threadIdx.x, lane = tid & 63;
     const size_t nwg = (size_t)gridDim.x * gridDim.y;
     for (size_t k = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + tid; k < zero_n; k += nwg * 256) zero[k] = 0.f;
     const int ck = blockIdx.x, t = blockIdx.y;
     const bool live = t < T;
-    float m = (live && lane < nmx) ? mx[t * MAXW + lane] : 0.f;
+    const int k = ck * CHUNK + tid;
+    const float* x = X + (size_t)(live ? t : 0) * (SWIGLU ? 2 * (size_t)K : (size_t)K);
+    const float raw = (live && k < K) ? act<SWIGLU>(x, K, k) : 0.f;
+    // the chunk's largest magnitude (a NaN is not one: it reaches the operands as it is and makes the output row NaN)
+    float m = fabsf(raw);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if (lane == 0) red[tid >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     float sc = 1.0f, inv = 1.0f;
     if (m > 0.f && m < INFINITY) {
         int ex;
         (void)frexpf(m, &ex);            // m < 2^ex
-        ex = ex < -111 ? -111 : ex;      // the scale stays a finite f32; rows below 2^-111 keep fewer bits
+        ex = ex < -111 ? -111 : ex;      // the scale stays a finite f32; chunks below 2^-111 keep fewer bits
         sc = ldexpf(1.0f, 15 - ex);      // scaled maximum in [2^14, 2^15)
         inv = ldexpf(1.0f, ex - 15);
     }
-    if (tid == 0 && ck == 0 && live) rs[t] = inv;
+    const size_t row = ((size_t)(ck * NT + (t >> 3)) * 16 + (t & 7)) * XR;
     auto put = [&](int col, float v) {
         const _Float16 h = (_Float16)v;
         const _Float16 l = (_Float16)(v - (float)h);
-        const size_t at = ((size_t)(ck * NT + (t >> 3)) * 16 + (t & 7)) * XR + col;
-        Xp[at] = __builtin_bit_cast(uint16_t, h);
-        Xp[at + 8 * XR] = __builtin_bit_cast(uint16_t, l);
+        Xp[row + col] = __builtin_bit_cast(uint16_t, h);
+        Xp[row + 8 * XR + col] = __builtin_bit_cast(uint16_t, l);
     };
-    const int k = ck * CHUNK + tid;
-    const float* x = X + (size_t)(live ? t : 0) * (SWIGLU ? 2 * (size_t)K : (size_t)K);
-    const float v = (live && k < K) ? act<SWIGLU>(x, K, k) * sc : 0.f;
+    const float v = raw * sc;
     put(F::pos_of(tid), v);
-    // columns 256..263: sub-block sums / 64 (|sum| <= 32 * 2^15, so the quotient stays below 2^14); 264..279: zeros
+    // columns 256..263: sub-block sums / 64 (|sum| <= 32 * 2^15, so the quotient stays below 2^14); 264..271: zeros
     float s = F::HAS_MIN ? v : 0.f;
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o);
     if ((tid & 31) == 0) put(CHUNK + (tid >> 5), s * 0.015625f);
-    if (tid < 16) put(CHUNK + 8 + tid, 0.f);
+    if (tid < 8) put(CHUNK + 8 + tid, 0.f);
+    // columns 272, 273 of the hi and the lo row: the factor as f32; 274..279: zeros
+    if (tid >= 8 && tid < 16) {
+        const uint32_t bits = __float_as_uint(inv);
+        const uint16_t w = tid == 8 ? (uint16_t)(bits & 0xFFFFu) : tid == 9 ? (uint16_t)(bits >> 16) : (uint16_t)0;
+        Xp[row + XSCALE + (tid - 8)] = w;
+        Xp[row + 8 * XR + XSCALE + (tid - 8)] = w;
+    }
 }
 
 struct F16Params {
     const uint8_t* W;
     const uint16_t* Xp;   // prepared activations: [nchunks][16 NT][XR] f16
-    const float* rs;      // [T] row scales to take out
     float* Y;             // [T, N]
     int T, N, nchunks;
     int nblk;             // Q8_0: blocks in a weight row (the last chunk may hold fewer than 8)
@@ -460,16 +455,6 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
         for (int s = 0; s < 2; s++)
 #pragma unroll
             for (int q = 0; q < NT; q++) total[s][q] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        // the scales of this lane's activation rows, asked for now and used after the chunk loop
-        float rsv[NT][4];
-#pragma unroll
-        for (int q = 0; q < NT; q++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int t = 8 * q + 4 * (g4 & 1) + r;
-                rsv[q][r] = p.rs[t < p.T ? t : 0];
-            }
-
         // Weight bytes: the quant registers of a chunk are reloaded with the next chunk's bytes as soon as their last slice
         // has read them (half a chunk to a chunk ahead of their use); the few header bytes go through `hd` a chunk ahead.
         typename F::Raw raw[2];
@@ -507,6 +492,19 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
                     F::template refill<I>(raw[s], wrow[s], cn, g4);
                 }
             });
+            // the chunk's f32 result: super-block scale times the integer-weight products (and the minima's term), then the
+            // factor that takes the activation scale of the chunk's operand rows 4 g4 + r out again
+            float e[NT][4];
+#pragma unroll
+            for (int q = 0; q < NT; q++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) e[q][r] = *(const float*)(&Xs[buf][(16 * q + 4 * g4 + r) * XR + XSCALE]);
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int q = 0; q < NT; q++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) acc[s][q][r] *= x[s].d;
             if constexpr (F::HAS_MIN) {
                 f16x8 am[NT];
 #pragma unroll
@@ -519,7 +517,7 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
                         const f32x4 z = {0.f, 0.f, 0.f, 0.f};
                         const f32x4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(am[q], bm, z, 0, 0, 0);
 #pragma unroll
-                        for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x[s].dm, accm[r], total[s][q][r]);
+                        for (int r = 0; r < 4; r++) acc[s][q][r] = fmaf(x[s].dm, accm[r], acc[s][q][r]);
                     }
                 }
             }
@@ -528,7 +526,7 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
 #pragma unroll
                 for (int q = 0; q < NT; q++)
 #pragma unroll
-                    for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x[s].d, acc[s][q][r], total[s][q][r]);
+                    for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(e[q][r], acc[s][q][r], total[s][q][r]);
             store_x(buf ^ 1);
             __syncthreads();
 #pragma unroll
@@ -548,7 +546,6 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
                     float v = total[s][q][r];
                     v += __shfl_xor(v, 32);
                     if (g4 < 2 && t < p.T && n[s] < p.N) {
-                        v *= rsv[q][r];
                         float* y = p.Y + (size_t)t * p.N + n[s];
                         if (whole) *y = v;
                         else unsafeAtomicAdd(y, v);
@@ -634,14 +631,6 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
             if (tc < 32 * F::TAILS) *(uint16_t*)(wl + row * F::LROW + F::tail_lds(tc - row * F::TAILS)) = (uint16_t)gt[i];
         }
     };
-    float rsv[NT][4];
-#pragma unroll
-    for (int q = 0; q < NT; q++)
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int t = 8 * q + 4 * (g4 & 1) + r;
-            rsv[q][r] = p.rs[t < p.T ? t : 0];
-        }
     if (u >= u_end) return;
 
     // The workgroup's run of units is one stream: the chunk after a group's last is the next group's first, fetched and
@@ -666,15 +655,21 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
 #pragma unroll
                 for (int q = 0; q < NT; q++) total[s][q] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
+        // the factor that takes the activation scale of this chunk's operand rows 4 g4 + r out again
+        float e[NT][4];
+#pragma unroll
+        for (int q = 0; q < NT; q++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) e[q][r] = *(const float*)(&Xs[buf][(16 * q + 4 * g4 + r) * XR + XSCALE]);
 #pragma unroll
         for (int s = 0; s < 2; s++) {
             typename F::Raw raw;
             F::from_lds(raw, wl + (16 * s + c) * F::LROW, g4);
             typename F::Ctx x;
-            f32x4 acc[NT];
+            f32x4 acc[NT], ct[NT];     // the running MFMA result; the chunk's f32 result before the activation scale is taken out
             float dprev = 0.f;
 #pragma unroll
-            for (int q = 0; q < NT; q++) acc[q] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int q = 0; q < NT; q++) { acc[q] = (f32x4){0.f, 0.f, 0.f, 0.f}; ct[q] = (f32x4){0.f, 0.f, 0.f, 0.f}; }
             static_for<0, 8>([&](auto Ic) {
                 constexpr int I = decltype(Ic)::value;
                 F::template pre<I>(raw, g4, x);
@@ -694,8 +689,8 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
 #pragma unroll
                         for (int q = 0; q < NT; q++) {
 #pragma unroll
-                            for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(dprev, acc[q][r], total[s][q][r]);
-                            asm volatile("" : "+v"(total[s][q]));
+                            for (int r = 0; r < 4; r++) ct[q][r] = fmaf(dprev, acc[q][r], ct[q][r]);
+                            asm volatile("" : "+v"(ct[q]));
                         }
                     }
 #pragma unroll
@@ -720,14 +715,14 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
                     const f32x4 z = {0.f, 0.f, 0.f, 0.f};
                     const f32x4 accm = __builtin_amdgcn_mfma_f32_16x16x32_f16(am, bm, z, 0, 0, 0);
 #pragma unroll
-                    for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x.dm, accm[r], total[s][q][r]);
+                    for (int r = 0; r < 4; r++) ct[q][r] = fmaf(x.dm, accm[r], ct[q][r]);
                 }
             }
-            // the chunk's product (the last slice's, where every slice has its own scale)
+            // the chunk's product (the last slice's, where every slice has its own scale), then out with the activation scale
 #pragma unroll
             for (int q = 0; q < NT; q++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(x.d, acc[q][r], total[s][q][r]);
+                for (int r = 0; r < 4; r++) total[s][q][r] = fmaf(e[q][r], fmaf(x.d, acc[q][r], ct[q][r]), total[s][q][r]);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (more) {
@@ -748,7 +743,6 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
                     float v = total[s][q][r];
                     v += __shfl_xor(v, 32);
                     if (g4 < 2 && t < p.T && n < p.N) {
-                        v *= rsv[q][r];
                         float* y = p.Y + (size_t)t * p.N + n;
                         if (whole) *y = v;
                         else unsafeAtomicAdd(y, v);
@@ -794,25 +788,19 @@ Plan make_plan(const fhip_weight* w, size_t t) {
 }
 
 template <class F>
-int launch_xsplit_fmt(const float* d_x, size_t t, size_t k, bool swiglu, const Plan& q, uint16_t* d_xp, float* d_rs, float* d_mx,
-                      hipStream_t s, float* zero, size_t zero_n) {
-    const int nmx = (int)((k + 1023) / 1024);
-    const dim3 gm((unsigned)nmx, (unsigned)t), grid((unsigned)q.nchunks, (unsigned)(8 * q.nt)), wg(256);
-    if (swiglu) {
-        hipLaunchKernelGGL((rowmax_kernel<true>), gm, wg, 0, s, d_x, (int)k, d_mx);
-        hipLaunchKernelGGL((xsplit_f16_kernel<F, true>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_mx, nmx, d_xp, d_rs, zero, zero_n);
-    } else {
-        hipLaunchKernelGGL((rowmax_kernel<false>), gm, wg, 0, s, d_x, (int)k, d_mx);
-        hipLaunchKernelGGL((xsplit_f16_kernel<F, false>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_mx, nmx, d_xp, d_rs, zero, zero_n);
-    }
+int launch_xsplit_fmt(const float* d_x, size_t t, size_t k, bool swiglu, const Plan& q, uint16_t* d_xp, hipStream_t s, float* zero,
+                      size_t zero_n) {
+    const dim3 grid((unsigned)q.nchunks, (unsigned)(8 * q.nt)), wg(256);
+    if (swiglu) hipLaunchKernelGGL((xsplit_f16_kernel<F, true>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_xp, zero, zero_n);
+    else hipLaunchKernelGGL((xsplit_f16_kernel<F, false>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_xp, zero, zero_n);
     return fhip::check_hip(hipGetLastError(), "xsplit_f16 launch");
 }
 
 template <class F>
-int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
     const Plan q = make_plan(w, t);
     F16Params p;
-    p.W = w->d_raw; p.Xp = d_xp; p.rs = d_rs; p.Y = d_y;
+    p.W = w->d_raw; p.Xp = d_xp; p.Y = d_y;
     p.T = (int)t; p.N = (int)w->rows; p.nchunks = q.nchunks; p.row_bytes = w->row_bytes;
     p.nblk = (int)(w->cols / 32);
     p.units = q.units;
@@ -841,8 +829,6 @@ bool gemm_f16x2_supports(const fhip_weight* w, size_t t) {
     return (w->type == FHIP_Q4_K || w->type == FHIP_Q6_K) && t <= 32 && w->cols % CHUNK == 0;
 }
 
-size_t gemm_f16x2_aux_bytes() { return 256 + 32 * MAXW * sizeof(float); }   // row scales, then the partial row maxima
-
 size_t gemm_f16x2_xp_bytes(const fhip_weight* w, size_t t) {
     const Plan q = make_plan(w, t);
     return (size_t)q.nchunks * 16 * q.nt * XR * sizeof(uint16_t);
@@ -850,23 +836,21 @@ size_t gemm_f16x2_xp_bytes(const fhip_weight* w, size_t t) {
 
 bool gemm_f16x2_adds_into_y(const fhip_weight* w, size_t t) { return make_plan(w, t).split; }
 
-int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, float* d_aux, hipStream_t s,
-                      float* zero, size_t zero_n) {
+int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero, size_t zero_n) {
     const Plan q = make_plan(w, t);
-    float* d_mx = d_aux + 64;
     switch (w->type) {
-        case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
-        case FHIP_Q6_K: return launch_xsplit_fmt<Q6K>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
-        case FHIP_Q8_0: return launch_xsplit_fmt<Q80>(d_x, t, w->cols, swiglu, q, d_xp, d_aux, d_mx, s, zero, zero_n);
+        case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
+        case FHIP_Q6_K: return launch_xsplit_fmt<Q6K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
+        case FHIP_Q8_0: return launch_xsplit_fmt<Q80>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
     }
 }
 
-int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, const float* d_rs, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
     switch (w->type) {
-        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, d_rs, t, d_y, s, y_cleared);
-        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, d_rs, t, d_y, s, y_cleared);
-        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, d_rs, t, d_y, s, y_cleared);
+        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, t, d_y, s, y_cleared);
+        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, t, d_y, s, y_cleared);
+        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, t, d_y, s, y_cleared);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
     }
 }

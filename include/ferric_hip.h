@@ -391,7 +391,8 @@ int fhip_ffn_coop(const fhip_weight* gate_up, const fhip_weight* down, const flo
  * with f32-grade results (the reference's kernels, :2995-3051 and :3423-3469, walk the weight row once per activation
  * row): x f32 [rows_x, cols] -> y f32 [rows_x, rows]. Q4_K and Q6_K (cols a multiple of 256, as the formats require),
  * and Q8_0 (:2948-2990; cols a multiple of 32) for up to 16 rows.
- * Each activation row is scaled by a power of two and split into two f16 operand rows (22 significant bits), the
+ * Each 256-column chunk of an activation row is scaled by a power of two and split into two f16 operand rows (22
+ * significant bits at the chunk's largest magnitude), the
  * weights enter the f16 matrix cores as exact integers (sub-block scale x quant; the int8 quant for Q8_0) and the f32
  * block scale is applied to the f32 accumulator. d_ws: caller-provided scratch of fhip_matmul_q_f16x2_ws_bytes(...)
  * bytes, 256-byte aligned. rows_x > 32 (> 16 for Q8_0): FHIP_ERR_SHAPE; other formats: FHIP_ERR_UNSUPPORTED_TYPE

@@ -416,7 +416,8 @@ def test_non_finite_and_tiny_activations_give_what_the_f32_dot_gives(F, O, ty):
                 for i, r in enumerate(range(sl.start, sl.stop)):
                     fin = np.isfinite(w_[i])
                     if one_pass and not np.isfinite(xs[i]).all():
-                        # the matrix-core kernels scale a row by its largest magnitude: the whole output row is non-finite
+                        # the matrix-core kernels scale a row's chunks by their largest magnitudes, and a non-finite operand
+                        # meets every weight row: the whole output row is non-finite
                         assert not np.isfinite(y[i]).any(), (ty, r)
                         continue
                     assert np.array_equal(np.isnan(y[i]), np.isnan(w_[i])), (ty, r)
