@@ -48,6 +48,19 @@ def test_small_and_ragged_shapes(F, O, ty):
         run_case(F, O, ty, t, n, k, 10 + i)
 
 
+def test_seeded_random_shapes(F, O):
+    # 36 shapes drawn with a fixed seed: any row count on either side of the 32-row kernel switch, output widths that are
+    # no multiple of a tile (or of 4: the ordered sum of K-split tiles then stores element by element), 1 to 9 chunks of
+    # K -- whatever way the launch is cut, every output meets the oracle
+    rng = np.random.default_rng(20240607)
+    for i in range(36):
+        ty = (Q4_K, Q6_K, Q8_0)[i % 3]
+        t = int(rng.integers(1, 300)) if i % 4 else int(rng.integers(1, 33))
+        n = int(rng.integers(1, 700))
+        k = int(rng.integers(1, 10)) * 256 if ty != Q8_0 else int(rng.integers(1, 73)) * 32
+        run_case(F, O, ty, t, n, k, 1000 + i)
+
+
 def test_reference_coop_example_shapes(F, O):
     # crates/ferric-tensor/examples/coop_q4_k.rs: reference-generator weights, M a multiple of 8 and not
     run_case(F, O, Q4_K, 16, 64, 512, 3, gen=O.gen_kquant_matrix)
