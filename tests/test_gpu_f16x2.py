@@ -1,7 +1,7 @@
 """Small-batch matmul on the f16 matrix cores (fhip_matmul_q_f16x2 / fhip_ffn_f16x2) vs the CPU oracle, through the C ABI.
 
-The path claims f32-grade results: weights enter the matrix cores as exact integers, activations as a scaled hi/lo pair
-of f16 (22 significant bits). Bars, against the oracle's dequantized weights in f64:
+The path claims f32-grade results: weights enter the matrix cores as exact integers, activations as a hi/lo pair of f16
+scaled chunk by chunk (22 significant bits at a 256-column chunk's largest magnitude). Bars, against the oracle's dequantized weights in f64:
   * |y - y64| <= 2.5e-7 * ||w_row|| * ||x_t||  (measured <= 6e-8; the exact-f32 mat-vec path measures <= 5e-8 on the same
     inputs), 4000x inside the north-star bound 1e-3 * ||w_row|| * ||x_t||;
   * max|d| / max|ref| < 1e-5, the bar the f32 mat-vec tests use;
@@ -47,9 +47,34 @@ def test_small_and_ragged_shapes(F, O, ty):
         run_case(F, O, ty, t, n, k, 100 + i)
 
 
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+def test_a_chunk_of_small_values_keeps_its_bits_beside_a_large_one(F, O, ty):
+    # The scale is per 256-column chunk. Weights whose first super-block has scale 0 ignore the first chunk of x, so a
+    # first chunk 2^60 times larger than the rest must not cost the rest its precision: the outputs are held to the bound
+    # taken over the other chunks' activations only (with one scale per row their 22 bits would all lie above those values).
+    from ferric_amd.synth import synth_weights
+    t, n, k = 6, 160, 1280
+    blk = {Q4_K: 144, Q6_K: 210}[ty]
+    w = synth_weights(ty, n, k, 61).copy().reshape(n, k // 256, blk)
+    if ty == Q4_K:
+        w[:, 0, 0:4] = 0          # d and dmin of the first super-block of every row
+    else:
+        w[:, 0, 208:210] = 0      # d
+    w = w.reshape(-1)
+    x = np.random.default_rng(62).standard_normal((t, k)).astype(np.float32)
+    x[:, :256] *= np.float32(2.0 ** 60)
+    qm = F.QMatrix.from_bytes(w, ty, n, k)
+    y = F.Tensor.from_vec(x, x.shape).matmul_q_f16x2(qm).to_vec().reshape(t, n)
+    y64, _ = O.matmul_f64(x, w, ty, n, k)
+    wd = O.deq_raw(w, n * k, ty).reshape(n, k).astype(np.float64)
+    assert not wd[:, :256].any()
+    bound = TIGHT * np.linalg.norm(wd[:, 256:], axis=1)[None, :] * np.linalg.norm(x[:, 256:].astype(np.float64), axis=1)[:, None]
+    assert (np.abs(y - y64) <= bound).all(), float(np.max(np.abs(y - y64) / bound))
+
+
 @pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
 def test_rows_of_very_different_magnitude(F, O, ty):
-    # each row is scaled by its own power of two: tiny, huge, zero and outlier rows side by side keep the per-row bound
+    # each chunk of a row is scaled by its own power of two: tiny, huge, zero and outlier rows side by side keep the per-row bound
     t, n, k = 8, 96, 1024
     x = np.random.default_rng(7).standard_normal((t, k)).astype(np.float32)
     x[0] *= np.float32(1e-30)
