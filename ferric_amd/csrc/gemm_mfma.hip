@@ -460,23 +460,226 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
   }
 }
 
-// Rows 16 * blockIdx.y .. + 15 of left-over tile `blockIdx.x`, if more than one run contributed to it:
-// Y = slot 0 + slot 1 + ... in that order. A thread owns four adjacent columns of one row per pass.
-__global__ void __launch_bounds__(256) sum_split_tiles_kernel(float* __restrict__ Y, const float* __restrict__ ws, int T, int N, int BM,
+// ------------------------------------------------------------------------------------------------
+// The same kernel with a 256 x 160 workgroup tile. An output width of 5120 is 20 tiles of 256 columns but 32 of 160, and
+// 32 x (T / 256) tile rows deal 2048, 1024 or 512 activation rows to the chip's 256 workgroups exactly: one whole tile
+// each, or every tile cut along K in exactly two or four (no run that starts in one tile and ends in the next, so one
+// partial tile per workgroup). Wave layout: 8 waves along T, 32 rows each, every wave holding all five 32-column blocks
+// (MI = 1, NI = 5: 1.2 LDS operand reads per MFMA instead of 0.75). Waves 0..4 each unpack one 32-row weight block and
+// publish its fragments; waves 5..7 only multiply (and, for the formats dear to unpack, move the activations: below). (The fifth block shared by waves
+// 4..7, one slice each, so that every SIMD carries the same unpack arithmetic, was slower: 130 -> 141 us at T = 2048 --
+// four more waves fetch raw bytes and derive scales every step.) Work distribution and K-split slots are the tall
+// kernel's at MI = 4.
+// ------------------------------------------------------------------------------------------------
+template <class F>
+__global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
+    constexpr int MI = 4, NB = 5;
+    constexpr int BM = 64 * MI, BN = 32 * NB;
+    constexpr int FRAG = 512;
+    __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_ROW];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][NB * 4 * FRAG];   // [n-block 0..4][slice 0..3]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane >> 5, c = lane & 31;
+    const bool unpacker = wave < NB;                            // wave-uniform
+    const int nchunks = p.nchunks;
+    long long u = (long long)blockIdx.x * p.per;
+    const long long u_end = u + p.per < p.units ? u + p.per : p.units;
+  for (int round = 0;; round++) {
+    int tile, c_begin, c_end;
+    if (round < p.whole_rounds) {
+        tile = round * gridDim.x + blockIdx.x;
+        c_begin = 0;
+        c_end = nchunks;
+    } else {
+        if (u >= u_end) break;
+        const int rt = (int)(u / nchunks);
+        tile = p.whole_rounds * gridDim.x + rt;
+        c_begin = (int)(u - (long long)rt * nchunks);
+        c_end = (long long)(nchunks - c_begin) < u_end - u ? nchunks : c_begin + (int)(u_end - u);
+        u += c_end - c_begin;
+    }
+    const bool whole = c_begin == 0 && c_end == nchunks;
+    const int tile_y = tile / p.tiles_n, tile_x = tile - tile_y * p.tiles_n;
+    const int t0 = tile_y * BM + 32 * wave;
+    const int n0 = tile_x * BN;
+    const int c_last = c_end - 1;
+
+    // the weight row an unpacking lane works on: row c of n-block `wave` of the tile (clamped: rows past N are computed but
+    // not stored); the other waves point at a valid row and never read it
+    const uint8_t* wrow;
+    {
+        int n = n0 + 32 * (unpacker ? wave : 0) + c;
+        wrow = p.W + (size_t)(n < p.N ? n : p.N - 1) * p.row_bytes;
+    }
+    const int b_wr = (wave * 4) * FRAG + lane * 8;              // + t * FRAG (unpackers)
+    const int b_rd = lane * 8;                                  // + (4 * j + t) * FRAG
+
+    f32x16 acc[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+
+    // Activation staging, BM rows x 64 bf16 per step, global -> registers one step ahead -> padded LDS. Rows past T are read
+    // from row T-1 (their outputs are never stored); columns past K (a partial last chunk) are staged as zeros. Who moves
+    // them depends on what a weight costs to unpack. Q4_K: every thread, the 16-byte piece (tid & 7) of rows (tid >> 3) +
+    // 64 q, as in the tall kernel. Q6_K and Q8_0: the three waves that unpack nothing -- lane sl of those 192 moves piece
+    // (sl & 7) of rows (sl >> 3) + 24 q, q < 11 (the eleventh round holds 16 rows, for the first two of the three waves) --
+    // which takes 20 of some 190 instructions a step off the waves that set the pace (Q8_0 5120 x 4096 at T = 2048 150 ->
+    // 133 us, Q6_K 5120 x 17408 444 -> 432 us; Q4_K 5120 x 5120 131 -> 135 us, so it keeps the even split).
+    constexpr bool SPLIT = F::UNPACK_US > 2.f;
+    constexpr int NQ = SPLIT ? 11 : MI, RSTEP = SPLIT ? 24 : 64;
+    const bool stager = SPLIT ? !unpacker : true;               // wave-uniform
+    const bool qlast = SPLIT ? wave < NB + 2 : true;            // wave-uniform: the wave has a piece in the last round
+    const int sl = SPLIT ? (wave - NB) * 64 + lane : tid;
+    const int a_col = (sl & 7) * 8;
+    uint32_t a_src[NQ];
+    u32x4 stage[NQ];
+    if (stager) {
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            const int t = tile_y * BM + (sl >> 3) + RSTEP * q;
+            a_src[q] = (uint32_t)(t < p.T ? t : p.T - 1) * (uint32_t)p.K + a_col;
+        }
+    }
+    const int a_dst = (sl >> 3) * LDS_ROW + a_col;              // + RSTEP q LDS_ROW
+    auto load_a = [&](int s) {
+        if constexpr (F::PARTIAL) {
+            const bool ok = s * KSTEP + a_col < p.K;
+            const int off = ok ? s * KSTEP : 0;
+            const uint32_t keep = ok ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+            for (int q = 0; q < NQ; q++)
+                if (q < NQ - 1 || qlast) {
+                    u32x4 v = *(const u32x4*)(p.X + (a_src[q] + off));
+                    stage[q] = (u32x4){v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
+                }
+        } else {
+            const int off = s * KSTEP < p.K ? s * KSTEP : 0;   // past the end: any valid address, the tile is never read
+#pragma unroll
+            for (int q = 0; q < NQ; q++)
+                if (q < NQ - 1 || qlast) stage[q] = *(const u32x4*)(p.X + (a_src[q] + off));
+        }
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < NQ; q++)
+            if (q < NQ - 1 || qlast) *(u32x4*)(&As[buf][a_dst + RSTEP * q * LDS_ROW]) = stage[q];
+    };
+    const int a_rd = (32 * wave + c) * LDS_ROW + 16 * h;        // + kcol(t, 0)
+    typename F::Raw raw;
+    if (stager) load_a(4 * c_begin);
+    if (unpacker) {
+        F::prime(raw, wrow, c_begin, h, p.nblk);
+        const int nc = c_begin + 1 < c_last ? c_begin + 1 : c_last;
+        typename F::Ctx x;
+        F::template begin<0>(raw, c_begin, h, p.nblk, x);
+        static_for<0, 4>([&](auto T) {
+            *(bf16x8*)(&Bs[0][b_wr + T.value * FRAG]) = F::template frag<0, T.value>(raw, x);
+        });
+        F::template refill<0>(raw, wrow, nc, h, p.nblk);
+    }
+    if (stager) store_a(0);
+    __syncthreads();
+
+    // one k-step, as in the tall kernel; UNPACK: the wave produces its block's fragments, one behind each slice's MFMAs
+    auto step = [&](auto Gc, auto Uc, int ck) {
+        constexpr int G = decltype(Gc)::value;
+        constexpr bool UNPACK = decltype(Uc)::value;
+        constexpr int GN = (G + 1) & 3;
+        constexpr int buf = G & 1;
+        constexpr int VPM = (26 + NB - 1) / NB;
+        const int pc = G == 3 ? (ck + 1 < c_last ? ck + 1 : c_last) : ck;
+        const int nc = pc + 1 < c_last ? pc + 1 : c_last;
+        typename F::Ctx ctx;
+        bf16x8 a[2], b[2][NB];
+        auto read_ops = [&](int t, bf16x8& da, bf16x8 (&db)[NB]) {
+            da = *(const bf16x8*)(&As[buf][a_rd + kcol(t, 0)]);
+#pragma unroll
+            for (int j = 0; j < NB; j++) db[j] = *(const bf16x8*)(&Bs[buf][b_rd + (4 * j + t) * FRAG]);
+        };
+        read_ops(0, a[0], b[0]);
+        if constexpr (!(UNPACK && SPLIT)) load_a(4 * ck + G + 1);
+        if constexpr (UNPACK) F::template begin<GN>(raw, pc, h, p.nblk, ctx);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<0, 4>([&](auto S) {
+            constexpr int t = decltype(S)::value;
+            if constexpr (t < 3) read_ops(t + 1, a[(t + 1) & 1], b[(t + 1) & 1]);
+#pragma unroll
+            for (int j = 0; j < NB; j++) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t & 1], b[t & 1][j], acc[j], 0, 0, 0);
+            if constexpr (UNPACK) *(bf16x8*)(&Bs[buf ^ 1][b_wr + t * FRAG]) = F::template frag<GN, t>(raw, ctx);
+            if constexpr (t < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1 + NB, 0);
+#pragma unroll
+            for (int m = 0; m < NB; m++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if constexpr (UNPACK) __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);
+            }
+            if constexpr (UNPACK) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (UNPACK) F::template refill<GN>(raw, wrow, nc, h, p.nblk);
+        if constexpr (!(UNPACK && SPLIT)) store_a(buf ^ 1);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (unpacker) {
+        for (int ck = c_begin; ck < c_end; ck++) {
+            step(std::integral_constant<int, 0>{}, std::true_type{}, ck);
+            step(std::integral_constant<int, 1>{}, std::true_type{}, ck);
+            step(std::integral_constant<int, 2>{}, std::true_type{}, ck);
+            step(std::integral_constant<int, 3>{}, std::true_type{}, ck);
+        }
+    } else {
+        for (int ck = c_begin; ck < c_end; ck++) {
+            step(std::integral_constant<int, 0>{}, std::false_type{}, ck);
+            step(std::integral_constant<int, 1>{}, std::false_type{}, ck);
+            step(std::integral_constant<int, 2>{}, std::false_type{}, ck);
+            step(std::integral_constant<int, 3>{}, std::false_type{}, ck);
+        }
+    }
+
+    float* part = nullptr;
+    if (!whole) {
+        const int rt = tile - p.whole_rounds * (int)gridDim.x;
+        const int k = (int)blockIdx.x - (int)(((long long)rt * nchunks) / p.per);
+        part = p.ws + ((size_t)rt * p.kmax + k) * (size_t)(BM * BN);
+    }
+    // D layout of the 32x32 MFMA: register r of lane (h, c) is row 8*(r/4) + 4*h + (r%4), column c
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        const int n = n0 + 32 * j + c;
+        if (n >= p.N) continue;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int t = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (t < p.T) {
+                if (whole) p.Y[(size_t)t * p.N + n] = acc[j][r];
+                else part[(size_t)(t - tile_y * BM) * BN + (n - tile_x * BN)] = acc[j][r];
+            }
+        }
+    }
+  }
+}
+
+// Rows 16 * blockIdx.y .. + 15 of left-over tile `blockIdx.x` (BM x BN outputs, BN <= 256 a multiple of 4), if more than one
+// run contributed to it: Y = slot 0 + slot 1 + ... in that order. A thread owns four adjacent columns of one row per pass.
+__global__ void __launch_bounds__(256) sum_split_tiles_kernel(float* __restrict__ Y, const float* __restrict__ ws, int T, int N, int BM, int BN,
                                                             int tiles_n, int nchunks, int per, int kmax, int first_tile) {
     const int rt = blockIdx.x, tile = first_tile + rt;
     const long long u0 = (long long)rt * nchunks;
     const int nk = (int)((u0 + nchunks - 1) / per) - (int)(u0 / per) + 1;
     if (nk == 1) return;                          // one run covered the whole K of this tile and stored it
     const int tile_y = tile / tiles_n, tile_x = tile - tile_y * tiles_n;
-    const int c4 = (threadIdx.x & 63) * 4, col = tile_x * 256 + c4;
-    const size_t slot = (size_t)BM * 256;
+    const int c4 = (threadIdx.x & 63) * 4, col = tile_x * BN + c4;
+    if (c4 >= BN) return;
+    const size_t slot = (size_t)BM * BN;
     const float* base = ws + (size_t)rt * kmax * slot + c4;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int lt = blockIdx.y * 16 + i * 4 + (threadIdx.x >> 6), t = tile_y * BM + lt;
         if (t >= T || col >= N) continue;
-        const float* q = base + (size_t)lt * 256;
+        const float* q = base + (size_t)lt * BN;
         float4 a = *(const float4*)q;
         for (int k = 1; k < nk; k++) {
             const float4 v = *(const float4*)(q + (size_t)k * slot);
@@ -703,6 +906,7 @@ int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_
 // How a launch of the tiled kernel with tile height 64 * mi is dealt to the chip: `whole_rounds` whole tiles per workgroup,
 // then the left-over tiles cut along K into runs of `per` chunks.
 struct TilePlan {
+    int mi, bn;                         // tile of 64 * mi activation rows x bn outputs (256, or 160 with mi = 4)
     int whole_rounds, per;
     long long left, units, split_wgs;   // left-over tiles, their chunks, workgroups whose run ends in partial tiles
     int kmax;                           // most runs that touch one left-over tile
@@ -710,14 +914,15 @@ struct TilePlan {
     unsigned grid;
 };
 
-static TilePlan plan_tiles(long long tiles_n, int nchunks, size_t t, int mi, long long cus) {
+static TilePlan plan_tiles(long long tiles_n, int nchunks, size_t t, int mi, long long cus, int bn = 256) {
     TilePlan q;
+    q.mi = mi; q.bn = bn;
     const long long tiles = tiles_n * (long long)((t + 64 * mi - 1) / (64 * mi));
     q.whole_rounds = (int)(tiles / cus);
     q.left = tiles - q.whole_rounds * cus;
     q.units = q.left * nchunks;
     long long per = (q.units + cus - 1) / cus;
-    // a run shorter than a tile's K that is close to it is rounded up to whole tiles: no atomics, no clearing
+    // a run shorter than a tile's K that is close to it is rounded up to whole tiles: no partial tiles, no summing launch
     if (per * 4 >= (long long)nchunks * 3) per = nchunks;
     if (per < 1) per = 1;
     q.per = (int)per;
@@ -735,25 +940,27 @@ static TilePlan plan_tiles(long long tiles_n, int nchunks, size_t t, int mi, lon
     return q;
 }
 
-// Estimated duration of a plan in us: chunks per workgroup x (unpack of a 256 x 256 weight chunk + mi MFMA slabs of 64 rows),
-// plus the fix-up of the tiles cut along K (every partial tile of 64 * mi x 256 f32 is written to the workspace and read back by
-// the summing kernel: two passes over 16 MB per 64 rows of tile height for 256 partial tiles, ~6 us, and that kernel's launch;
-// a run that starts inside one tile and ends inside the next writes two).
-// Constants fitted to measured launches (Q4_K
-// 34816 x 5120, T = 2048: 8.3 us a chunk at mi = 4, 4.85 at mi = 2; Q6_K and Q8_0 likewise) and checked against 21 shapes:
-// the model ranks the tile heights like the measurement wherever they differ by more than 6 %.
+// Estimated duration of a plan in us: 1.5 per tile or run a workgroup starts, chunks per workgroup x the cost of a chunk, and,
+// when tiles are cut along K, the fix-up: 10.5 for the summing launch and 5 x mi per 256 partial tiles of 256 columns written
+// (and read back; a run that starts inside one tile and ends inside the next writes two). A chunk of a 256-column tile costs
+// the format's unpack time + 0.7 + 1.64 x mi (Q4_K: 3.7 / 5.4 / 8.6 us at 64 / 128 / 256 rows); a chunk of the 256 x 160 tile
+// 5.75 + 0.23 x the unpack time (its pace is set by the MFMAs and the operand reads; five of eight waves share the
+// unpacking). Constants fitted to forced-tile builds on 14 shapes of the three formats (53 launches, 7 % rms): the choice
+// is the fastest tile on all of them (candidates within 2 % of each other: the lower tile).
 template <class F>
-static float plan_cost_us(const TilePlan& q, int nchunks, int mi, long long cus) {
-    const float chunk_us = F::UNPACK_US + 1.75f * (float)mi;
+static float plan_cost_us(const TilePlan& q, int nchunks, long long cus) {
+    const float width = (float)q.bn / 256.f;
+    const float chunk_us = q.bn == 256 ? F::UNPACK_US + 0.68f + 1.64f * (float)q.mi : 5.75f + 0.23f * F::UNPACK_US;
     const float chunks = (float)q.whole_rounds * (float)nchunks + (q.left > 0 ? (float)q.per : 0.f);
-    return chunks * chunk_us + (q.split_wgs > 0 ? 3.f + 6.f * (float)mi * (float)q.slots / (float)cus : 0.f);
+    const float starts = (float)q.whole_rounds + (q.left > 0 ? 1.f : 0.f);
+    return 1.5f * starts + chunks * chunk_us + (q.split_wgs > 0 ? 10.5f + 4.96f * (float)q.mi * width * (float)q.slots / (float)cus : 0.f);
 }
 
-static size_t plan_ws_bytes(const TilePlan& q, int mi) {
-    return q.split_wgs > 0 ? (size_t)q.left * q.kmax * (size_t)(64 * mi * 256) * sizeof(float) : 0;
+static size_t plan_ws_bytes(const TilePlan& q) {
+    return q.split_wgs > 0 ? (size_t)q.left * q.kmax * (size_t)(64 * q.mi * q.bn) * sizeof(float) : 0;
 }
 
-template <class F, int MI>
+template <class F, int MI, int BN>
 int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, const TilePlan& q, long long cus, float* d_ws,
                size_t ws_bytes) {
     GemmParams p;
@@ -761,60 +968,64 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     p.T = (int)t; p.N = (int)w->rows; p.K = (int)w->cols; p.row_bytes = w->row_bytes;
     p.nblk = (int)(w->row_bytes / F::BLOCK);
     p.nchunks = F::chunks(p.K);
-    p.tiles_n = (int)((w->rows + 255) / 256);
+    p.tiles_n = (int)((w->rows + BN - 1) / BN);
     // one workgroup per CU (its LDS tiles take most of a CU's 160 KB)
     p.whole_rounds = q.whole_rounds;
     p.units = q.units;
     p.per = q.per;
     p.ws = d_ws; p.kmax = q.kmax;
-    if (q.split_wgs > 0 && (!d_ws || ws_bytes < plan_ws_bytes(q, MI)))
-        return fhip::set_error(FHIP_ERR_ARG, "gemm_q_bf16: the launch cuts tiles along K and needs %zu bytes of workspace", plan_ws_bytes(q, MI));
-    hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(q.grid), dim3(512), 0, s, p);
+    if (q.split_wgs > 0 && (!d_ws || ws_bytes < plan_ws_bytes(q)))
+        return fhip::set_error(FHIP_ERR_ARG, "gemm_q_bf16: the launch cuts tiles along K and needs %zu bytes of workspace", plan_ws_bytes(q));
+    if constexpr (BN == 256) hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(q.grid), dim3(512), 0, s, p);
+    else hipLaunchKernelGGL((gemm_q_bf16_n160_kernel<F>), dim3(q.grid), dim3(512), 0, s, p);
     if (q.split_wgs > 0)
         hipLaunchKernelGGL(sum_split_tiles_kernel, dim3((unsigned)q.left, (unsigned)(64 * MI / 16)), dim3(256), 0, s, d_y, (const float*)d_ws, p.T, p.N, 64 * MI,
-                           p.tiles_n, p.nchunks, p.per, p.kmax, (int)(p.whole_rounds * cus));
+                           BN, p.tiles_n, p.nchunks, p.per, p.kmax, (int)(p.whole_rounds * cus));
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
-// the tile height the estimate picks for this launch, its plan, and the workspace it needs
+// the tile the estimate picks for this launch (256 columns by 256, 128 or 64 rows, or 160 columns by 256 rows) with its plan
 template <class F>
-static int choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
-    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256, tiles_n = (long long)((w->rows + 255) / 256);
+static void choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
+    const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     const int nchunks = F::chunks((int)w->cols);
-    int best = 0;
     float best_cost = 0.f;
-    for (int i = 0; i < 3; i++) {
-        const int mi = 4 >> i;
-        const TilePlan q = plan_tiles(tiles_n, nchunks, t, mi, cus);
-        const float c = plan_cost_us<F>(q, nchunks, mi, cus);
-        if (i == 0 || c < best_cost) { best = i; best_cost = c; out = q; }
+    for (int i = 0; i < 4; i++) {                 // 64, 128, 256 rows x 256 columns, then 256 x 160
+        const int mi = i < 3 ? 1 << i : 4, bn = i < 3 ? 256 : 160;
+#ifdef FHIP_FORCE_TILE
+        if (i != FHIP_FORCE_TILE) continue;
+#endif
+        const TilePlan q = plan_tiles((long long)((w->rows + bn - 1) / bn), nchunks, t, mi, cus, bn);
+        const float c = plan_cost_us<F>(q, nchunks, cus);
+        if (best_cost == 0.f || c < 0.98f * best_cost) { best_cost = c; out = q; }
     }
-    return 4 >> best;
 }
 
 template <class F>
 static size_t ws_bytes_fmt(const fhip_weight* w, size_t t) {
     if (t <= 32) return skinny_ws_bytes(plan_skinny(w->rows, F::chunks((int)w->cols), t, fhip::device_cus() > 0 ? fhip::device_cus() : 256));
     TilePlan q;
-    const int mi = choose_plan<F>(w, t, q);
-    return plan_ws_bytes(q, mi);
+    choose_plan<F>(w, t, q);
+    return plan_ws_bytes(q);
 }
 
 template <class F>
 int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, float* d_ws, size_t ws_bytes) {
     if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, d_ws, ws_bytes);
-    // Tile height 64 * MI. The 256 x 256 tile unpacks each weight once per 256 activation rows, but when there is no whole
-    // round of such tiles for the chip every tile is cut along K, each workgroup writes a whole partial tile for a few
-    // chunks of work, and a lower tile (twice the tiles, half the fix-up, longer runs) can win: the estimate decides
-    // (measured, Q4_K 5120 x 5120: T = 2048 175 -> 163 us with 128-row tiles, which give one whole round and a remainder cut
-    // in four; T = 128 42 -> 29 us with 64-row tiles; Q6_K 5120 x 17408 and Q8_0, dearer to unpack, keep the tall tile from
-    // T = 512 on).
+    // Which tile. The 256 x 256 tile unpacks each weight once per 256 activation rows, but when there is no whole round of
+    // such tiles for the chip every tile is cut along K, each workgroup writes a whole partial tile for a few chunks of
+    // work, and a lower tile (twice the tiles, half the fix-up, longer runs) or the 256 x 160 tile (whose count divides the
+    // chip for output widths like 5120 and 4096) can win: the estimate decides (measured, us at 256 / 128 / 64 rows x 256 and
+    // 256 x 160; Q4_K 5120 x 5120: T = 2048 176 / 162 / 207 / 128, T = 512 57 / 60 / 66 / 50, T = 128 43 / 33 / 30 / 45;
+    // Q6_K 5120 x 17408 T = 2048 458 / 511 / 788 / 426; Q8_0 4096 x 4096 T = 2048 131 / 156 / 278 / 111; Q4_K 34816 x 5120
+    // T = 512 219 / 247 / 326 / 233).
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     TilePlan q;
-    const int mi = choose_plan<F>(w, t, q);
-    if (mi == 4) return launch_cfg<F, 4>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
-    if (mi == 2) return launch_cfg<F, 2>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
-    return launch_cfg<F, 1>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    choose_plan<F>(w, t, q);
+    if (q.bn == 160) return launch_cfg<F, 4, 160>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    if (q.mi == 4) return launch_cfg<F, 4, 256>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    if (q.mi == 2) return launch_cfg<F, 2, 256>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    return launch_cfg<F, 1, 256>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
 }
 
 // f32 -> bf16 (round to nearest even), 8 values per thread, the tail one by one

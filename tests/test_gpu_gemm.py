@@ -96,12 +96,12 @@ def test_rows_are_independent_of_the_batch(F, O):
     assert np.array_equal(big.view(np.uint32), again.view(np.uint32))
 
 
-@pytest.mark.parametrize("ty,t,n,k", [(Q4_K, 128, 5120, 5120), (Q4_K, 512, 5120, 5120), (Q4_K, 2048, 5120, 5120),
+@pytest.mark.parametrize("ty,t,n,k", [(Q4_K, 128, 5120, 5120), (Q4_K, 512, 5120, 5120), (Q4_K, 2048, 9216, 5120),
                                       (Q6_K, 300, 1000, 4096), (Q8_0, 200, 1300, 2080), (Q4_K, 70, 3000, 8192),
                                       (Q4_K, 8, 5120, 5120), (Q6_K, 20, 1000, 4096), (Q8_0, 3, 1300, 2080), (Q4_K, 32, 1024, 5120)])
 def test_two_runs_give_identical_bits(F, O, ty, t, n, k):
-    # Launches with fewer whole tiles than the chip has workgroups cut tiles along K (every shape here does; 2048 x 5120
-    # has one whole round and a cut remainder; up to 32 rows it is groups of 128 outputs that are cut). The partial tiles are
+    # Launches with fewer whole tiles than the chip has workgroups cut tiles along K (every shape here does; 2048 x 9216
+    # has a cut remainder behind whole tiles; up to 32 rows it is groups of 128 outputs that are cut). The partial tiles are
     # summed in a fixed order, so the bits may not depend on which workgroup finishes first: five runs, with other work on
     # the device in between, one result.
     from ferric_amd.synth import synth_weights
