@@ -817,6 +817,8 @@ int fhip_debug_generic_matvec(int on) {
     return FHIP_OK;
 }
 
+int fhip_debug_gemm_tile(int tile) { return fhip::gemm_bf16_force_tile(tile); }
+
 int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, void* stream) {
     int rc = need_init();
     if (rc) return rc;

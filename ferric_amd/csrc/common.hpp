@@ -107,6 +107,7 @@ int launch_moe_wsum(const float* d_parts, const float* d_selw, size_t t, int k, 
 // d_ws / ws_bytes: gemm_bf16_ws_bytes(w, t) bytes of scratch for launches that cut output tiles along K (0: none needed)
 int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, hipStream_t s, float* d_ws = nullptr, size_t ws_bytes = 0);
 size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t);
+int gemm_bf16_force_tile(int tile);   // debugging / tests: 0..3 pins the tile of launches of more than 32 rows, -1 frees it; returns the old value
 // conversions in front of the GEMM
 int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s);
 int launch_swiglu_bf16(const float* d_gu, size_t t, size_t d, uint16_t* d_out, hipStream_t s);

@@ -984,6 +984,8 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
+int g_force_tile = -1;   // tests: 0..3 = 64, 128, 256 rows x 256 columns, 256 x 160; anything else: the estimate decides
+
 // the tile the estimate picks for this launch (256 columns by 256, 128 or 64 rows, or 160 columns by 256 rows) with its plan
 template <class F>
 static void choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
@@ -992,9 +994,7 @@ static void choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
     float best_cost = 0.f;
     for (int i = 0; i < 4; i++) {                 // 64, 128, 256 rows x 256 columns, then 256 x 160
         const int mi = i < 3 ? 1 << i : 4, bn = i < 3 ? 256 : 160;
-#ifdef FHIP_FORCE_TILE
-        if (i != FHIP_FORCE_TILE) continue;
-#endif
+        if (g_force_tile >= 0 && g_force_tile <= 3 && i != g_force_tile) continue;
         const TilePlan q = plan_tiles((long long)((w->rows + bn - 1) / bn), nchunks, t, mi, cus, bn);
         const float c = plan_cost_us<F>(q, nchunks, cus);
         if (best_cost == 0.f || c < 0.98f * best_cost) { best_cost = c; out = q; }
@@ -1067,6 +1067,12 @@ int launch_cvt_bf16(const float* d_x, size_t n, uint16_t* d_out, hipStream_t s) 
     if ((((uintptr_t)d_x | (uintptr_t)d_out) & 15) != 0) return set_error(FHIP_ERR_ARG, "cvt_f32_bf16: pointers must be 16-byte aligned");
     hipLaunchKernelGGL(cvt_f32_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s, d_x, d_out, n);
     return check_hip(hipGetLastError(), "cvt_f32_bf16 launch");
+}
+
+int gemm_bf16_force_tile(int tile) {
+    const int before = g_force_tile;
+    g_force_tile = tile;
+    return before;
 }
 
 size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t) {

@@ -342,6 +342,12 @@ void fhip_workspace_release(void* stream);
  * not thread-safe against concurrent launches). No counterpart in the reference. */
 int fhip_debug_generic_matvec(int on);
 
+/* Debugging and tests: pins the workgroup tile of the matrix-core GEMM (fhip_gemm_q_bf16, fhip_matmul_q_coop, fhip_ffn_coop)
+ * for launches of more than 32 rows: 0, 1, 2 = 64, 128, 256 activation rows x 256 outputs, 3 = 256 x 160; -1 (the default)
+ * lets the cost estimate choose. Returns the value before the call. Process-wide, not thread-safe against concurrent
+ * launches; fhip_workspace_bytes_coop follows it. No counterpart in the reference. */
+int fhip_debug_gemm_tile(int tile);
+
 /* Measurement aid: one launch that reads nbytes at d_src (16-byte loads over the whole chip) and does nothing else; d_sink is
  * one device word that is practically never written. Timed beside a mat-vec of the same size it gives the time a perfect reader
  * needs for those bytes on this device. No counterpart in the reference (its matvec_roofline example prints bytes / time of the

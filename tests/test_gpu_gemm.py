@@ -61,6 +61,22 @@ def test_seeded_random_shapes(F, O):
         run_case(F, O, ty, t, n, k, 1000 + i)
 
 
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+def test_every_tile_on_ragged_shapes(F, O, tile):
+    # The launcher picks one of four workgroup tiles by estimate; here each is pinned in turn (64 / 128 / 256 rows x 256
+    # outputs, 256 x 160) and run on shapes that fill no tile: rows and outputs that end inside a tile, outputs that are no
+    # multiple of 4, launches with whole rounds of tiles and a cut remainder, launches where every tile is cut along K.
+    lib = F._lib.load()
+    before = lib.fhip_debug_gemm_tile(tile)
+    try:
+        shapes = [(Q4_K, 33, 100, 512), (Q4_K, 300, 4001, 1024), (Q6_K, 130, 257, 2048), (Q8_0, 70, 1283, 1184), (Q4_K, 520, 7000, 768),
+                  (Q6_K, 257, 161, 256), (Q8_0, 1025, 330, 96)]
+        for i, (ty, t, n, k) in enumerate(shapes):
+            run_case(F, O, ty, t, n, k, 300 + 10 * tile + i)
+    finally:
+        lib.fhip_debug_gemm_tile(before)
+
+
 def test_reference_coop_example_shapes(F, O):
     # crates/ferric-tensor/examples/coop_q4_k.rs: reference-generator weights, M a multiple of 8 and not
     run_case(F, O, Q4_K, 16, 64, 512, 3, gen=O.gen_kquant_matrix)
