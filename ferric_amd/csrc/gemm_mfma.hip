@@ -681,9 +681,13 @@ __global__ void __launch_bounds__(256) sum_split_tiles_kernel(float* __restrict_
         if (t >= T || col >= N) continue;
         const float* q = base + (size_t)lt * BN;
         float4 a = *(const float4*)q;
-        for (int k = 1; k < nk; k++) {
-            const float4 v = *(const float4*)(q + (size_t)k * slot);
-            a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+        for (int k0 = 1; k0 < nk; k0 += 4) {          // four slots requested at a time, added in slot order
+            float4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = *(const float4*)(q + (size_t)(k0 + j < nk ? k0 + j : 0) * slot);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (k0 + j < nk) { a.x += v[j].x; a.y += v[j].y; a.z += v[j].z; a.w += v[j].w; }
         }
         float* y = Y + (size_t)t * N + col;
         if ((N & 3) == 0) *(float4*)y = a;
