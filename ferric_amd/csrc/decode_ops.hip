@@ -266,7 +266,26 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15;
     const int sid = wave * 4 + (lane >> 4);
     const int kvh = blockIdx.x, split = blockIdx.y;
+    // FUSED: the raw values of every head this wave will post-process (job j = wave + 4 r: query head j of the group, then
+    // the key and the value row) are requested before anything else, the length word with them, so that one memory round
+    // trip covers what used to be three in a row (the length, the first round's rows, the second round's).
+    constexpr int ROUNDS = FUSED ? (G + 2 + 3) / 4 : 1, EPL = HD / 64;
+    float xr[ROUNDS][EPL];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int r = 0; r < ROUNDS; r++) {
+            const int j = wave + 4 * r;
+            if (j < G + 2) {
+                const int src = j < G ? kvh * G + j : (j == G ? fp.n_head + kvh : fp.n_head + n_kv + kvh);
+                const float* x = fp.qkv + (size_t)src * HD;
+                const float* bias = fp.bias ? fp.bias + (size_t)src * HD : nullptr;
+#pragma unroll
+                for (int i = 0; i < EPL; i++) xr[r][i] = bias ? x[lane + 64 * i] + bias[lane + 64 * i] : x[lane + 64 * i];
+            }
+        }
+    }
     uint32_t len = len_dev ? *len_dev + 1u : len_host;   // the device word is the newest token's position
+    asm volatile("" ::: "memory");                       // keeps the loads above in front of the arithmetic on the length
     if (len > len_host) len = len_host;
     // sliding window (nn.rs:92-111): only the last `window` keys count; 0 or >= len: all of them
     const uint32_t first = (window > 0 && window < len) ? len - window : 0u;
@@ -283,20 +302,25 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
         const bool owner = pos < fp.cap && (pos < len ? (pos >= k0 && pos < k1) : split == splits - 1);
         const int njobs = G + (owner ? 2 : 0);
         const int kvw = n_kv * HD, half = fp.n_rot / 2;
-        for (int j = wave; j < njobs; j += 4) {            // job j < G: query head j of the group; G: the K row; G + 1: the V row
+#pragma unroll
+        for (int r = 0; r < ROUNDS; r++) {                 // job j < G: query head j of the group; G: the K row; G + 1: the V row
+            const int j = wave + 4 * r;
+            if (j >= njobs) continue;
             const int src = j < G ? kvh * G + j : (j == G ? fp.n_head + kvh : fp.n_head + n_kv + kvh);
             const float* x = fp.qkv + (size_t)src * HD;
             const float* bias = fp.bias ? fp.bias + (size_t)src * HD : nullptr;
             const float* nw = j < G ? fp.q_norm : (j == G ? fp.k_norm : nullptr);
             float* dst = j < G ? &sm_q[FUSED ? j : 0][0] : (j == G ? fp.k_cache : fp.v_cache) + (size_t)pos * kvw + (size_t)kvh * HD;
             if (j == G + 1) {
-                for (int e = lane; e < HD; e += 64) dst[e] = bias ? x[e] + bias[e] : x[e];
+#pragma unroll
+                for (int i = 0; i < EPL; i++) dst[lane + 64 * i] = xr[r][i];
                 continue;
             }
             float inv = 1.f;
             if (nw) {
                 float ms = 0.f;
-                for (int e = lane; e < HD; e += 64) { float v = bias ? x[e] + bias[e] : x[e]; ms = fmaf(v, v, ms); }
+#pragma unroll
+                for (int i = 0; i < EPL; i++) ms = fmaf(xr[r][i], xr[r][i], ms);
                 ms = wave_sum(ms);
                 inv = 1.0f / sqrtf(ms / (float)HD + fp.eps);
             }
@@ -427,6 +451,12 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_combine_kernel(const flo
     __shared__ float w[256], lw[256];
     const int head = blockIdx.x, tid = threadIdx.x;
     const float* pp = part + (size_t)head * splits * (hd + 2);
+    // this thread's output dim of the first splits is requested together with the splits' maxima and sums: one memory round
+    // trip instead of two in a row for the short caches, where this kernel is nothing but latency
+    constexpr int EARLY = 16;
+    float pv[EARLY];
+#pragma unroll
+    for (int s = 0; s < EARLY; s++) pv[s] = (s < splits && tid < hd) ? pp[(size_t)s * (hd + 2) + tid] : 0.f;
     for (int s = tid; s < splits; s += COMBINE_THREADS) { w[s] = pp[(size_t)s * (hd + 2) + hd]; lw[s] = pp[(size_t)s * (hd + 2) + hd + 1]; }
     __syncthreads();
     float M = -3.0e38f;
@@ -438,8 +468,13 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_combine_kernel(const flo
     for (int s = 0; s < splits; s++) L += lw[s];
     for (int d = tid; d < hd; d += COMBINE_THREADS) {
         float A = 0.f;
+        if (d == tid) {
+#pragma unroll
+            for (int s = 0; s < EARLY; s++)
+                if (s < splits) A = fmaf(pv[s], w[s], A);
+        }
 #pragma unroll 8
-        for (int s = 0; s < splits; s++) A = fmaf(pp[(size_t)s * (hd + 2) + d], w[s], A);
+        for (int s = d == tid ? EARLY : 0; s < splits; s++) A = fmaf(pp[(size_t)s * (hd + 2) + d], w[s], A);
         out[(size_t)head * hd + d] = A / L;
     }
 }
