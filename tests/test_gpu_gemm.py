@@ -90,6 +90,29 @@ def test_config4_prefill_5120(F, O, t):
     run_case(F, O, Q4_K, t, 5120, 5120, 21)
 
 
+@pytest.mark.parametrize("ty,t,n,k", [(Q4_K, 2048, 34816, 5120), (Q6_K, 512, 5120, 17408), (Q8_0, 2048, 4096, 4096)])
+def test_the_layer_s_large_projections_on_sampled_outputs(F, O, ty, t, n, k):
+    # The fused gate|up weight at 2048 rows is four whole rounds of 256 x 256 tiles and a remainder cut in four, the down
+    # projection at 512 rows 256 x 160 tiles each cut in four, Q8_0 4096 x 4096 a grid of 208 whole 256 x 160 tiles. Too large for
+    # the f64 model in full: 384 weight rows spread over the first, the last and random tiles, every activation row.
+    from ferric_amd.synth import synth_weights
+    w = synth_weights(ty, n, k, 71)
+    x = np.random.default_rng(72).standard_normal((t, k)).astype(np.float32)
+    xb, xv = bf16_round(x)
+    qm = F.QMatrix.from_bytes(w, ty, n, k)
+    y = F.Tensor.from_bf16_bits(xb, (t, k)).gemm_q_bf16(qm).to_vec().reshape(t, n)
+    rows = np.unique(np.concatenate([np.arange(64), np.arange(n - 64, n), np.random.default_rng(73).integers(0, n, 256)]))
+    rb = len(w) // n
+    wd = O.deq_raw(np.ascontiguousarray(w.reshape(n, rb)[rows]).reshape(-1), len(rows) * k, ty).reshape(len(rows), k)
+    _, wb = bf16_round(wd)
+    model = xv.astype(np.float64) @ wb.astype(np.float64).T
+    got = y[:, rows]
+    assert np.abs(got - model).max() / np.abs(model).max() < 2e-5
+    exact = xv.astype(np.float64) @ wd.astype(np.float64).T
+    bound = 1e-3 * np.linalg.norm(wd.astype(np.float64), axis=1)[None, :] * np.linalg.norm(xv.astype(np.float64), axis=1)[:, None]
+    assert (np.abs(got - exact) <= bound).all()
+
+
 def test_prefill_other_formats_at_size(F, O):
     run_case(F, O, Q6_K, 256, 5120, 5120, 22)
     run_case(F, O, Q8_0, 256, 4096, 4096, 23)
