@@ -23,6 +23,10 @@
 // One k-step is 64 columns = 4 MFMA slices; a chunk is 4 steps = one K-quant super-block or 8 Q8_0 blocks.
 // Dequantized values are exactly the f32 the CPU dequantizer produces, rounded to bf16 (RNE) by
 // v_cvt_pk_bf16_f32.
+// Three kernels: the tiled one (64, 128 or 256 activation rows x 256 outputs per workgroup), its 256 x 160 variant for
+// output widths that 160 deals to the chip's workgroups exactly, and one for up to 32 rows; the launcher picks by a cost
+// estimate. A launch that cuts output tiles along K sums the partial tiles in a fixed order: the same inputs give the
+// same bits on every run.
 #include "common.hpp"
 #include "loads.hpp"
 
