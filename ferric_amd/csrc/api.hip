@@ -189,7 +189,7 @@ int g_batch_policy = FHIP_BATCH_AUTO;
 
 size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32; }
 bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
-    if (g_batch_policy != FHIP_BATCH_AUTO) return false;
+    if (g_batch_policy == FHIP_BATCH_F32_MATVEC) return false;
     if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0) return false;
     if (rows_x < (w->type == FHIP_Q8_0 ? 5u : 3u)) return false;
     return fhip::gemm_f16x2_supports(w, rows_x < f16x2_group(w) ? rows_x : f16x2_group(w));
@@ -203,13 +203,18 @@ int zero_outputs(size_t t, size_t rows, float* d_y, hipStream_t s) {
 }
 
 // y [t, w->rows] = x [t, cols] W^T for t rows of one group; ws: f16x2_matmul_ws(w, t) bytes
-size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) { return align256(fhip::gemm_f16x2_xp_bytes(w, t)); }
+// (FHIP_BATCH_ORDERED: behind the prepared activations, the partial sums of the groups the launch cuts along K)
+size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) {
+    return align256(fhip::gemm_f16x2_xp_bytes(w, t)) + (g_batch_policy == FHIP_BATCH_ORDERED ? align256(fhip::gemm_f16x2_part_bytes_upto(w, t)) : 0);
+}
 int f16x2_matmul(const fhip_weight* w, const float* d_x, size_t t, bool swiglu_in, float* d_y, void* d_ws, hipStream_t s) {
     uint16_t* xp = (uint16_t*)d_ws;
-    const bool clr = fhip::gemm_f16x2_adds_into_y(w, t);   // then the split clears y on the side
+    const bool ordered = g_batch_policy == FHIP_BATCH_ORDERED;
+    float* part = ordered && fhip::gemm_f16x2_part_bytes(w, t) ? (float*)((uint8_t*)d_ws + align256(fhip::gemm_f16x2_xp_bytes(w, t))) : nullptr;
+    const bool clr = !part && fhip::gemm_f16x2_adds_into_y(w, t);   // then the split clears y on the side
     int rc = fhip::launch_xsplit_f16(w, d_x, t, swiglu_in, xp, s, clr ? d_y : nullptr, clr ? t * w->rows : 0);
     if (rc) return rc;
-    return fhip::launch_gemm_f16x2(w, xp, t, d_y, s, clr);
+    return fhip::launch_gemm_f16x2(w, xp, t, d_y, s, clr, part);
 }
 
 }  // namespace
@@ -635,7 +640,7 @@ int fhip_ffn_noalloc(const fhip_weight* gu, const fhip_weight* down, const float
 
 int fhip_batch_policy(int policy) {
     const int before = g_batch_policy;
-    if (policy == FHIP_BATCH_AUTO || policy == FHIP_BATCH_F32_MATVEC) g_batch_policy = policy;
+    if (policy == FHIP_BATCH_AUTO || policy == FHIP_BATCH_F32_MATVEC || policy == FHIP_BATCH_ORDERED) g_batch_policy = policy;
     return before;
 }
 

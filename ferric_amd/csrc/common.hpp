@@ -120,7 +120,12 @@ bool gemm_f16x2_adds_into_y(const fhip_weight* w, size_t t);      // true: the l
 // operand rows, each carrying the factor that takes its scale out again
 int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero = nullptr,
                       size_t zero_n = 0);
-int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared = false);
+// d_part: null, or gemm_f16x2_part_bytes(w, t) bytes: partial sums of K-split groups go there and are added in a fixed
+// order by a launch behind the matmul (y then needs no clearing) instead of being added into y atomically
+int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared = false,
+                      float* d_part = nullptr);
+size_t gemm_f16x2_part_bytes(const fhip_weight* w, size_t t);
+size_t gemm_f16x2_part_bytes_upto(const fhip_weight* w, size_t t);   // the largest over batches of 1..t rows
 
 // decode_ops.hip: the steps either side of the matmuls in a decode layer
 int launch_rmsnorm(const float* a, const float* b, const float* weight, size_t rows, size_t d, float eps, float* sum_out, float* norm_out,

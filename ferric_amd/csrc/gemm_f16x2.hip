@@ -28,8 +28,10 @@
 // Lane (g4 = lane / 16, c = lane % 16) of a wave works on weight row c of a 16-row set and on k-group g4 of each
 // 32-wide MFMA slice; a wave carries two row sets (32 weight rows), a workgroup four waves (128 rows). The
 // (128-row group, 256-column chunk) units are dealt to the workgroups in equal contiguous runs; a run that covers its
-// group's whole K stores, any other adds atomically into a Y cleared beforehand.
+// group's whole K stores, any other adds atomically into a Y cleared beforehand (or, when the caller asks for ordered sums, stores
+// into a slot of its own that sum_split_kernel adds in contributor order).
 #include "common.hpp"
+#include <algorithm>
 #include "loads.hpp"
 
 #include <hip/hip_fp16.h>
@@ -409,7 +411,18 @@ struct F16Params {
     int nblk;             // Q8_0: blocks in a weight row (the last chunk may hold fewer than 8)
     size_t row_bytes;
     long long units;      // 128-row groups * nchunks, chunk fastest
+    float* part;          // null: a run that holds part of a group's K adds into Y atomically. Else it stores its partial sums
+                          // into slot (group, contributor) of [groups][kmax][32][128] floats, and sum_split_kernel adds them in order
+    int kmax;
 };
+
+// Workgroup b of G takes units [b U / G, (b + 1) U / G): the workgroup that holds unit u
+__device__ __host__ __forceinline__ int holder_of(long long u, long long G, long long U) { return (int)(((u + 1) * G - 1) / U); }
+// where a partial output (activation row t, output n of group grp) goes in ordered mode
+__device__ __forceinline__ float* part_slot(const F16Params& p, int grp, int t, int n) {
+    const int k = (int)blockIdx.x - holder_of((long long)grp * p.nchunks, gridDim.x, p.units);
+    return p.part + (((size_t)grp * p.kmax + k) * 32 + t) * 128 + (n - grp * 128);
+}
 
 template <class F, int NT>
 __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16Params p) {
@@ -548,6 +561,7 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
                     if (g4 < 2 && t < p.T && n[s] < p.N) {
                         float* y = p.Y + (size_t)t * p.N + n[s];
                         if (whole) *y = v;
+                        else if (p.part) *part_slot(p, grp, t, n[s]) = v;
                         else unsafeAtomicAdd(y, v);
                     }
                 }
@@ -745,12 +759,37 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
                     if (g4 < 2 && t < p.T && n < p.N) {
                         float* y = p.Y + (size_t)t * p.N + n;
                         if (whole) *y = v;
+                        else if (p.part) *part_slot(p, grp, t, n) = v;
                         else unsafeAtomicAdd(y, v);
                     }
                 }
         }
         __syncthreads();
     }
+}
+
+// Ordered mode: group `blockIdx.x` of 128 outputs, if more than one workgroup held part of its K: Y = slot 0 + slot 1 + ...
+// in that order. Thread = output column (threadIdx.x & 127) of activation row 2 * blockIdx.y + (threadIdx.x >> 7).
+__global__ void __launch_bounds__(256) sum_split_kernel(float* __restrict__ Y, const float* __restrict__ part, int T, int N, int nchunks,
+                                                      long long units, int grid, int kmax) {
+    const int grp = blockIdx.x;
+    const int first = holder_of((long long)grp * nchunks, grid, units), last = holder_of((long long)(grp + 1) * nchunks - 1, grid, units);
+    const int nk = last - first + 1;
+    if (nk == 1) return;
+    const int col = threadIdx.x & 127, n = grp * 128 + col, t = 2 * blockIdx.y + (threadIdx.x >> 7);
+    if (n >= N || t >= T) return;
+    const size_t slot = 32 * 128;
+    const float* q = part + (size_t)grp * kmax * slot + t * 128 + col;
+    float a = q[0];
+    for (int k0 = 1; k0 < nk; k0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = q[(size_t)(k0 + j < nk ? k0 + j : 0) * slot];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (k0 + j < nk) a += v[j];
+    }
+    Y[(size_t)t * N + n] = a;
 }
 
 __global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
@@ -760,9 +799,10 @@ __global__ void zero_f32_kernel(float* __restrict__ out, size_t n) {
 
 struct Plan {
     int nt, nchunks;
-    long long units;
+    long long units, groups;
     unsigned grid;
     bool split;
+    int kmax;             // most workgroups that hold part of one group's K
 };
 
 // workgroups of the kernel that serves `nt` operand row sets that fit on a CU together
@@ -784,6 +824,12 @@ Plan make_plan(const fhip_weight* w, size_t t) {
     if (per >= q.nchunks || per * 4 >= (long long)q.nchunks * 3) q.grid = (unsigned)groups;
     else q.grid = (unsigned)(q.units < wgs ? q.units : wgs);
     q.split = q.grid != (unsigned)groups;
+    q.groups = groups;
+    q.kmax = 1;
+    for (long long g = 0; g < groups && q.split; g++) {
+        const int nk = holder_of((g + 1) * q.nchunks - 1, q.grid, q.units) - holder_of(g * q.nchunks, q.grid, q.units) + 1;
+        if (nk > q.kmax) q.kmax = nk;
+    }
     return q;
 }
 
@@ -797,14 +843,15 @@ int launch_xsplit_fmt(const float* d_x, size_t t, size_t k, bool swiglu, const P
 }
 
 template <class F>
-int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_part) {
     const Plan q = make_plan(w, t);
     F16Params p;
     p.W = w->d_raw; p.Xp = d_xp; p.Y = d_y;
+    p.part = q.split ? d_part : nullptr; p.kmax = q.kmax;
     p.T = (int)t; p.N = (int)w->rows; p.nchunks = q.nchunks; p.row_bytes = w->row_bytes;
     p.nblk = (int)(w->cols / 32);
     p.units = q.units;
-    if (q.split && !y_cleared) {
+    if (q.split && !y_cleared && !d_part) {
         const size_t n = t * w->rows;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
     }
@@ -816,6 +863,9 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y,
     } else {
         return fhip::set_error(FHIP_ERR_SHAPE, "f16x2 matmul: this format takes at most 16 activation rows, got %zu", t);
     }
+    if (p.part)
+        hipLaunchKernelGGL(sum_split_kernel, dim3((unsigned)q.groups, (unsigned)((t + 1) / 2)), dim3(256), 0, s, d_y, (const float*)d_part, p.T, p.N,
+                           p.nchunks, p.units, (int)q.grid, p.kmax);
     return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
 }
 
@@ -836,6 +886,18 @@ size_t gemm_f16x2_xp_bytes(const fhip_weight* w, size_t t) {
 
 bool gemm_f16x2_adds_into_y(const fhip_weight* w, size_t t) { return make_plan(w, t).split; }
 
+size_t gemm_f16x2_part_bytes(const fhip_weight* w, size_t t) {
+    const Plan q = make_plan(w, t);
+    return q.split ? (size_t)q.groups * q.kmax * 32 * 128 * sizeof(float) : 0;
+}
+// the most any batch of up to t rows needs (fewer rows can mean more resident workgroups, and so more contributors)
+size_t gemm_f16x2_part_bytes_upto(const fhip_weight* w, size_t t) {
+    size_t m = gemm_f16x2_part_bytes(w, t);
+    for (size_t u : {(size_t)8, (size_t)16})
+        if (u < t) m = std::max(m, gemm_f16x2_part_bytes(w, u));
+    return m;
+}
+
 int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero, size_t zero_n) {
     const Plan q = make_plan(w, t);
     switch (w->type) {
@@ -846,11 +908,11 @@ int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swi
     }
 }
 
-int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared) {
+int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_part) {
     switch (w->type) {
-        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, t, d_y, s, y_cleared);
-        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, t, d_y, s, y_cleared);
-        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, t, d_y, s, y_cleared);
+        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, t, d_y, s, y_cleared, d_part);
+        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, t, d_y, s, y_cleared, d_part);
+        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, t, d_y, s, y_cleared, d_part);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
     }
 }

@@ -318,10 +318,15 @@ int fhip_ffn_noalloc(const fhip_weight* gate_up, const fhip_weight* down, const 
 /* Which kernel fhip_matmul_q, fhip_matmul_q_swiglu and fhip_ffn give a batch of three rows or more. FHIP_BATCH_AUTO (the
  * default): the one-pass matrix-core kernels as described at fhip_matmul_q. FHIP_BATCH_F32_MATVEC: the streaming mat-vec, two
  * rows per pass over the weights; an output row then has the same bits whatever batch it was part of (the guarantee the
- * reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200), at the price of rows_x / 2 passes. Returns the
- * policy before the call; any other value only queries. Process-wide, as fhip_matvec_precision. */
+ * reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200), at the price of rows_x / 2 passes.
+ * FHIP_BATCH_ORDERED: the one-pass kernels of FHIP_BATCH_AUTO, but where a launch cuts a weight row's columns between
+ * workgroups the pieces go to the library workspace (fhip_workspace_bytes counts them) and one more launch adds them in a
+ * fixed order instead of f32 atomic adds: the same call on the same inputs then returns the same bits on every run, for a
+ * few microseconds per matmul. Returns the policy before the call; any other value only queries. Process-wide, as
+ * fhip_matvec_precision; set it before sizing or reserving the workspace. */
 #define FHIP_BATCH_AUTO 0
 #define FHIP_BATCH_F32_MATVEC 1
+#define FHIP_BATCH_ORDERED 2
 int fhip_batch_policy(int policy);
 
 /* The library's workspace of a stream (NULL: the default stream): device memory the batched paths of fhip_matmul_q,

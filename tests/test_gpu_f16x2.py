@@ -272,3 +272,46 @@ def test_argument_checks(F):
     dn = F.QMatrix.from_bytes(synth_weights(Q6_K, 32, 256, 2), Q6_K, 32, 256)
     with pytest.raises(AssertionError, match="down in dim must equal n_ff"):
         F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256)).ffn_f16x2(q4, dn)
+
+
+# ---------------------------------------------------------------- FHIP_BATCH_ORDERED: the same kernels, partial sums added in order
+
+def test_ordered_policy_gives_the_same_bits_on_every_run(F, O):
+    # Under FHIP_BATCH_ORDERED (2) the drop-in calls keep the one-pass kernels, but a launch that cuts a group's K between
+    # workgroups writes the pieces to the library's workspace and adds them in a fixed order: run after run the same bits,
+    # and the same bars against the oracle as the default policy. Shapes: cut along K (few groups, long rows), not cut
+    # (one chunk), ragged rows, each activation-row class, Q8_0's ragged K; then the FFN block at the model's size, where
+    # the down projection (40 groups of 68 chunks) is cut many ways.
+    from ferric_amd.synth import synth_weights
+    lib = F._lib.load()
+    before = lib.fhip_batch_policy(2)
+    try:
+        assert lib.fhip_batch_policy(-1) == 2
+        cases = [(Q4_K, 4, 512, 8192), (Q4_K, 8, 5120, 5120), (Q6_K, 3, 130, 4096), (Q6_K, 12, 1000, 17408), (Q4_K, 20, 257, 2048),
+                 (Q4_K, 32, 64, 256), (Q8_0, 5, 300, 4128), (Q8_0, 16, 1024, 4096), (Q4_K, 40, 384, 6144)]
+        for i, (ty, t, n, k) in enumerate(cases):
+            w = synth_weights(ty, n, k, 700 + i)
+            x = np.random.default_rng(800 + i).standard_normal((t, k)).astype(np.float32)
+            qm = F.QMatrix.from_bytes(w, ty, n, k)
+            xt = F.Tensor.from_vec(x, x.shape)
+            y = xt.matmul_q(qm).to_vec().reshape(t, n)
+            y64, wn = O.matmul_f64(x, w, ty, n, k)
+            bound = TIGHT * wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None]
+            assert (np.abs(y - y64) <= bound + 1e-300).all(), (ty, t, n, k)
+            for _ in range(3):
+                assert np.array_equal(xt.matmul_q(qm).to_vec().reshape(t, n), y), (ty, t, n, k)
+        n_embd, n_ff, batch = 5120, 17408, 8
+        gu = synth_weights(Q4_K, 2 * n_ff, n_embd, 3)
+        dn = synth_weights(Q6_K, n_embd, n_ff, 4)
+        x = np.random.default_rng(5).standard_normal((batch, n_embd)).astype(np.float32)
+        wgu = F.QMatrix.from_bytes(gu, Q4_K, 2 * n_ff, n_embd)
+        wdn = F.QMatrix.from_bytes(dn, Q6_K, n_embd, n_ff)
+        xt = F.Tensor.from_vec(x, x.shape)
+        y = xt.ffn(wgu, wdn).to_vec()
+        for _ in range(3):
+            assert np.array_equal(xt.ffn(wgu, wdn).to_vec(), y)
+        lib.fhip_batch_policy(0)
+        y0 = xt.ffn(wgu, wdn).to_vec()                 # the default policy: atomic adds, the same sums in another order
+        assert np.abs(y - y0).max() <= 2e-6 * np.abs(y0).max()
+    finally:
+        lib.fhip_batch_policy(before)
