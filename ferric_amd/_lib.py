@@ -90,6 +90,8 @@ SYMBOLS = {
     "fhip_rmsnorm": (C.c_int, [_vp, _vp, _sz, _sz, C.c_float, _vp, _vp]),
     "fhip_add_rmsnorm": (C.c_int, [_vp, _vp, _vp, _sz, _sz, C.c_float, _vp, _vp, _vp]),
     "fhip_add": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
+    "fhip_mul_sigmoid": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
+    "fhip_geglu": (C.c_int, [_vp, _sz, _sz, _vp, _vp]),
     "fhip_rope": (C.c_int, [_vp, _sz, _sz, _sz, _sz, _sz, C.c_float, _vp, _u32, _vp, C.c_int, _vp, _vp]),
     "fhip_kv_append2": (C.c_int, [_vp, _vp, _sz, _sz, _vp, _u32, _vp, _vp, _sz, _vp]),
     "fhip_qkv_post": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_int, C.c_float, C.c_float, _vp, _vp, _vp,

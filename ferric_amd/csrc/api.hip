@@ -709,6 +709,22 @@ int fhip_add(const float* d_a, const float* d_b, size_t n, float* d_out, void* s
     return fhip::launch_add(d_a, d_b, n, d_out, (hipStream_t)stream);
 }
 
+int fhip_mul_sigmoid(const float* d_a, const float* d_g, size_t n, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (n == 0) return FHIP_OK;
+    if (!d_a || !d_g || !d_out) return set_error(FHIP_ERR_ARG, "fhip_mul_sigmoid: NULL pointer");
+    return fhip::launch_mul_sigmoid(d_a, d_g, n, d_out, (hipStream_t)stream);
+}
+
+int fhip_geglu(const float* d_gu, size_t t, size_t d, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (t * d == 0) return FHIP_OK;
+    if (!d_gu || !d_out) return set_error(FHIP_ERR_ARG, "fhip_geglu: NULL pointer");
+    return fhip::launch_geglu(d_gu, t, d, d_out, (hipStream_t)stream);
+}
+
 static int rope_checks(const char* who, size_t n_heads, size_t head_dim, size_t n_rot) {
     if (n_rot > head_dim || n_rot % 2 != 0) return set_error(FHIP_ERR_SHAPE, "n_rot must be even and <= head_dim");   // lib.rs:437
     if (n_heads > 0xFFFFu || head_dim > 0xFFFFu) return set_error(FHIP_ERR_SHAPE, "%s: n_heads / head_dim exceed 65535", who);

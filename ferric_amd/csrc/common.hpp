@@ -132,6 +132,8 @@ int launch_rmsnorm(const float* a, const float* b, const float* weight, size_t r
                    hipStream_t s);
 int launch_add(const float* a, const float* b, size_t n, float* out, hipStream_t s);
 int launch_u32_add(uint32_t* w, size_t n, uint32_t delta, hipStream_t s);
+int launch_mul_sigmoid(const float* a, const float* g, size_t n, float* out, hipStream_t s);   // out = a * sigmoid(g); out may be a
+int launch_geglu(const float* gu, size_t t, size_t d, float* out, hipStream_t s);              // rows [gate | up] -> gelu_tanh(gate) * up
 int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int hd, int n_rot, float base, const uint32_t* d_pos, uint32_t pos_off,
                 const float* freq_scale, int interleaved, float* out, hipStream_t s);
 int launch_qkv_post(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos, const float* freq_scale,

@@ -113,6 +113,25 @@ __global__ void add_kernel(const float* a, const float* __restrict__ b, size_t n
     if (i < n) out[i] = a[i] + b[i];
 }
 
+// out = a * sigmoid(g): the gate of a gated attention layer on the attention output (crates/ferric-llama/src/qwen3.rs:936-938;
+// sigmoid as crates/ferric-tensor/src/lib.rs:1915, 1 / (1 + exp(-v)))
+__global__ void mul_sigmoid_kernel(const float* a, const float* __restrict__ g, size_t n, float* out) {   // out may be a
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] * (1.0f / (1.0f + expf(-g[i])));
+}
+
+// out[r, j] = gelu_tanh(gu[r, j]) * gu[r, d + j] for rows [gate | up] of 2 d values: the GEGLU of qwen3.rs:953-958 with the
+// tanh-approximated GELU of lib.rs:1926, 0.5 v (1 + tanh(clamp(0.79788456 (v + 0.044715 v^3), -15, 15)))
+__global__ void geglu_kernel(const float* __restrict__ gu, size_t n, size_t d, float* __restrict__ out) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t r = i / d, j = i - r * d;
+    const float v = gu[r * 2 * d + j], u = gu[r * 2 * d + d + j];
+    float a = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+    a = fminf(fmaxf(a, -15.0f), 15.0f);
+    out[i] = 0.5f * v * (1.0f + tanhf(a)) * u;
+}
+
 // ---------------------------------------------------------------- rotary embedding
 // Pair c of a head rotates by angle pos * base^(-2c / n_rot) (times freq_scale[c]); partners are (c, c + n_rot/2) in the
 // split-half layout and (2c, 2c + 1) interleaved; dims >= n_rot pass through (lib.rs:2118-2162, 2094-2116). The inverse
@@ -533,6 +552,23 @@ int launch_add(const float* a, const float* b, size_t n, float* out, hipStream_t
     if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "add: too many elements for one launch");
     hipLaunchKernelGGL(add_kernel, dim3((unsigned)grid), dim3(256), 0, s, a, b, n, out);
     return check_hip(hipGetLastError(), "add launch");
+}
+
+int launch_mul_sigmoid(const float* a, const float* g, size_t n, float* out, hipStream_t s) {
+    if (n == 0) return FHIP_OK;
+    size_t grid = (n + 255) / 256;
+    if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "mul_sigmoid: too many elements for one launch");
+    hipLaunchKernelGGL(mul_sigmoid_kernel, dim3((unsigned)grid), dim3(256), 0, s, a, g, n, out);
+    return check_hip(hipGetLastError(), "mul_sigmoid launch");
+}
+
+int launch_geglu(const float* gu, size_t t, size_t d, float* out, hipStream_t s) {
+    const size_t n = t * d;
+    if (n == 0) return FHIP_OK;
+    size_t grid = (n + 255) / 256;
+    if (grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "geglu: too many elements for one launch");
+    hipLaunchKernelGGL(geglu_kernel, dim3((unsigned)grid), dim3(256), 0, s, gu, n, d, out);
+    return check_hip(hipGetLastError(), "geglu launch");
 }
 
 int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int hd, int n_rot, float base, const uint32_t* d_pos, uint32_t pos_off,

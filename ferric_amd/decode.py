@@ -1,9 +1,11 @@
 """Host mirror of the reference's decode-layer ops and of `Qwen3::apply_layer` for one new token.
 
 The ops are the reference's `Tensor::rmsnorm / add_rmsnorm / add / rope*` (crates/ferric-tensor/src/lib.rs:279-520),
-`append2` (lib.rs:1379) and `nn::decode_attention` (crates/ferric-tensor/src/nn.rs:140); `Qwen3Decoder` is the default
-(pre-norm, no post-norms, no window, no softcap) arm of `Qwen3::attn / ffn / apply_layer`
-(crates/ferric-llama/src/qwen3.rs:861-966, 979-1052). Everything runs through libferric_hip; there is no CPU path.
+`append2` (lib.rs:1379) and `nn::decode_attention` (crates/ferric-tensor/src/nn.rs:140); `Qwen3Decoder` is
+`Qwen3::attn / ffn / apply_layer` (crates/ferric-llama/src/qwen3.rs:861-966, 979-1052) for one new token on an f32 cache:
+the default pre-norm arm, and per layer or configuration a sliding window, a score softcap, no rotation (NoPE), a rope
+base of the layer's own, a sigmoid gate on the attention output, post-norms on both branch outputs, GEGLU.
+Everything runs through libferric_hip; there is no CPU path.
 """
 import ctypes as C
 
@@ -50,6 +52,23 @@ def add(a, b, stream=None):
     assert a.shape == b.shape, "add: shapes differ (no broadcasting on this path)"
     out = Tensor.empty(a.shape)
     _check(_lib.load().fhip_add(a.buf.ptr, b.buf.ptr, a.numel(), out.buf.ptr, _stream_handle(stream)))
+    return out
+
+
+def mul_sigmoid(a, g, stream=None):
+    """a * sigmoid(g), equal shapes -- the attention gate of qwen3.rs:936-938."""
+    assert a.shape == g.shape, "mul_sigmoid: shapes differ"
+    out = Tensor.empty(a.shape)
+    _check(_lib.load().fhip_mul_sigmoid(a.buf.ptr, g.buf.ptr, a.numel(), out.buf.ptr, _stream_handle(stream)))
+    return out
+
+
+def geglu(gu, stream=None):
+    """gelu_tanh(gate) * up for rows [gate | up] -- qwen3.rs:953-958 with lib.rs:304."""
+    assert gu.shape[-1] % 2 == 0, "geglu: rows hold gate | up"
+    d = gu.shape[-1] // 2
+    out = Tensor.empty(tuple(gu.shape[:-1]) + (d,))
+    _check(_lib.load().fhip_geglu(gu.buf.ptr, gu.numel() // (2 * d), d, out.buf.ptr, _stream_handle(stream)))
     return out
 
 
@@ -116,20 +135,31 @@ def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, 
 
 
 class Qwen3Cfg:
-    """The fields of the reference's Cfg this path reads (qwen3.rs: n_head, n_head_kv, head_dim, eps, rope pairing)."""
+    """The fields of the reference's Cfg this path reads (qwen3.rs:60-100: n_head, n_head_kv, head_dim, eps, rope pairing,
+    attn_softcap, post_norm_eps; geglu stands for is_gemma's FFN activation, qwen3.rs:953)."""
 
-    def __init__(self, d_model, n_head, n_head_kv, head_dim, n_ff, eps=1e-6, rope_base=1e6, rope_interleaved=False):
+    def __init__(self, d_model, n_head, n_head_kv, head_dim, n_ff, eps=1e-6, rope_base=1e6, rope_interleaved=False, attn_softcap=0.0,
+                 post_norm_eps=None, geglu=False):
         self.d_model, self.n_head, self.n_head_kv, self.head_dim, self.n_ff = d_model, n_head, n_head_kv, head_dim, n_ff
         self.eps, self.rope_base, self.rope_interleaved = float(eps), float(rope_base), bool(rope_interleaved)
+        self.attn_softcap = float(attn_softcap)
+        self.post_norm_eps = float(eps if post_norm_eps is None else post_norm_eps)
+        self.geglu = bool(geglu)
 
 
 class Qwen3Layer:
-    """qwen3.rs:230-253, the fields of the default arm: norms as f32 Tensors, projections as QMatrix (wqkv = q|k|v stacked,
-    ffn_gate_up = gate|up stacked)."""
+    """qwen3.rs:230-253: norms as f32 Tensors, projections as QMatrix (wqkv = q|k|v stacked, ffn_gate_up = gate|up stacked).
+    Beyond the default arm: window (> 0: a local layer attends to that many newest keys), rope (False: a NoPE layer, QK-norm
+    only), rope_base (None: the configuration's), attn_gate (QMatrix [n_head * head_dim, d_model]), post_attn_norm and
+    post_ffn_norm (both or neither)."""
 
-    def __init__(self, attn_norm, wqkv, wo, ffn_norm, ffn_gate_up, ffn_down, q_norm=None, k_norm=None, qkv_bias=None):
+    def __init__(self, attn_norm, wqkv, wo, ffn_norm, ffn_gate_up, ffn_down, q_norm=None, k_norm=None, qkv_bias=None, window=0,
+                 rope=True, rope_base=None, attn_gate=None, post_attn_norm=None, post_ffn_norm=None):
         self.attn_norm, self.wqkv, self.wo, self.ffn_norm = attn_norm, wqkv, wo, ffn_norm
         self.ffn_gate_up, self.ffn_down, self.q_norm, self.k_norm, self.qkv_bias = ffn_gate_up, ffn_down, q_norm, k_norm, qkv_bias
+        self.window, self.rope, self.rope_base, self.attn_gate = int(window), bool(rope), rope_base, attn_gate
+        assert (post_attn_norm is None) == (post_ffn_norm is None), "the two post-norms come together (qwen3.rs:567-568)"
+        self.post_attn_norm, self.post_ffn_norm = post_attn_norm, post_ffn_norm
 
 
 class Qwen3Decoder:
@@ -140,6 +170,8 @@ class Qwen3Decoder:
         f = swiglu(rmsnorm(x + o) Wgu^T)                  [again inside the mat-vec];  y = f Wdown^T
     With fuse_norm=False the norms run as their own launches (9 per layer), as the reference issues them. With fuse_attn=True
     (also what None, the default, means) the q/k norm + rope + cache append happen inside the attention launch, 6 launches per layer.
+    A gated layer adds two launches (the gate's mat-vec on the same normed input, the sigmoid product), post-norms two (the
+    RMSNorm of each branch output; the add happens inside the next mat-vec as before), GEGLU one (the activation on its own).
     """
 
     def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None, fuse_norm=True, fuse_attn=None):
@@ -162,6 +194,11 @@ class Qwen3Decoder:
         self.o = Tensor.empty((1, c.d_model))
         self.f = Tensor.empty((1, c.n_ff))
         self.y = Tensor.empty((1, c.d_model))
+        self.gate = Tensor.empty((1, self.q_out)) if any(l.attn_gate is not None for l in layers) else None
+        self.gu = Tensor.empty((1, 2 * c.n_ff)) if c.geglu else None
+        post = any(l.post_attn_norm is not None for l in layers)
+        self.on = Tensor.empty((1, c.d_model)) if post else None      # post-normed attention branch
+        self.yn = Tensor.empty((1, c.d_model)) if post else None      # post-normed FFN branch
         lib = _lib.load()
         need = lib.fhip_decode_attention_ws_bytes(c.n_head, c.n_head_kv, c.head_dim, self.max_len)
         self.ws = DeviceBuffer(need) if need else None
@@ -170,7 +207,7 @@ class Qwen3Decoder:
             # of its own up to 2048 keys (5.12 -> 5.06 ms/token there, 4.92 -> 4.84 at 128) and is level with it from 4096 on.
             self.fuse_attn = True
         self.fuse_attn = bool(self.fuse_attn)
-        self.launches_per_layer = (7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0)
+        self.launches_per_layer = (7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0)   # a default-arm layer
         self._graph = None
 
     # -- state ------------------------------------------------------------------------------------
@@ -208,30 +245,52 @@ class Qwen3Decoder:
         lib, c, s = _lib.load(), self.cfg, _stream_handle(self.stream)
         cur, alt = self.xa, self.xb
         other = lambda t: self.xb if t is self.xa else self.xa
+        pending = None                                   # the previous layer's FFN branch, not yet added to the residual
         for il, (l, kv) in enumerate(zip(self.layers, self.caches)):
-            cur = self._norm_matmul(l.wqkv, cur, alt, self.y if il else None, l.attn_norm, self.qkv, False)
+            cur = self._norm_matmul(l.wqkv, cur, alt, pending, l.attn_norm, self.qkv, False)
             alt = other(cur)
+            if l.attn_gate is not None:                  # the gate projects the same normed input (qwen3.rs:936-938)
+                if self.fuse_norm:
+                    self._norm_matmul(l.attn_gate, cur, alt, None, l.attn_norm, self.gate, False)
+                else:                                    # self.h still holds the normed input
+                    _check(lib.fhip_matmul_q(l.attn_gate.handle, self.h.buf.ptr, 1, self.gate.buf.ptr, s))
+            n_rot = c.head_dim if l.rope else 0          # NoPE: q/k norm only (qwen3.rs:857-863)
+            base = c.rope_base if l.rope_base is None else float(l.rope_base)
             bias = l.qkv_bias.buf.ptr if l.qkv_bias is not None else None
             qn = l.q_norm.buf.ptr if l.q_norm is not None else None
             kn = l.k_norm.buf.ptr if l.k_norm is not None else None
             ws = self.ws.ptr if self.ws is not None else None
             if self.fuse_attn:
                 _check(lib.fhip_qkv_post_attention(self.qkv.buf.ptr, bias, qn, kn, self.pos.buf.ptr, None, c.n_head, c.n_head_kv, c.head_dim,
-                                                   c.head_dim, int(c.rope_interleaved), c.eps, c.rope_base, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap,
-                                                   self.max_len, 0, 0.0, ws, self.att.buf.ptr, s))
+                                                   n_rot, int(c.rope_interleaved), c.eps, base, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap,
+                                                   self.max_len, l.window, c.attn_softcap, ws, self.att.buf.ptr, s))
             else:
-                _check(lib.fhip_qkv_post(self.qkv.buf.ptr, bias, qn, kn, self.pos.buf.ptr, None, 1, c.n_head, c.n_head_kv, c.head_dim, c.head_dim,
-                                         int(c.rope_interleaved), c.eps, c.rope_base, self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap, s))
-                _check(lib.fhip_decode_attention(self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, c.n_head, c.n_head_kv, c.head_dim, self.max_len,
-                                                 self.pos.buf.ptr, ws, self.att.buf.ptr, s))
+                _check(lib.fhip_qkv_post(self.qkv.buf.ptr, bias, qn, kn, self.pos.buf.ptr, None, 1, c.n_head, c.n_head_kv, c.head_dim, n_rot,
+                                         int(c.rope_interleaved), c.eps, base, self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap, s))
+                _check(lib.fhip_decode_attention_ex(self.q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, c.n_head, c.n_head_kv, c.head_dim, self.max_len,
+                                                    self.pos.buf.ptr, l.window, c.attn_softcap, ws, self.att.buf.ptr, s))
+            if l.attn_gate is not None:
+                _check(lib.fhip_mul_sigmoid(self.att.buf.ptr, self.gate.buf.ptr, self.q_out, self.att.buf.ptr, s))
             _check(lib.fhip_matmul_q(l.wo.handle, self.att.buf.ptr, 1, self.o.buf.ptr, s))
-            cur = self._norm_matmul(l.ffn_gate_up, cur, alt, self.o, l.ffn_norm, self.f, True)
+            branch = self.o
+            if l.post_attn_norm is not None:             # x + post_attn_norm(attn(..)), its own epsilon (qwen3.rs:1015-1018)
+                _check(lib.fhip_rmsnorm(self.o.buf.ptr, l.post_attn_norm.buf.ptr, 1, c.d_model, c.post_norm_eps, self.on.buf.ptr, s))
+                branch = self.on
+            if c.geglu:                                  # Gemma: gate|up unfused, gelu_tanh(gate) * up (qwen3.rs:953-958)
+                cur = self._norm_matmul(l.ffn_gate_up, cur, alt, branch, l.ffn_norm, self.gu, False)
+                _check(lib.fhip_geglu(self.gu.buf.ptr, 1, c.n_ff, self.f.buf.ptr, s))
+            else:
+                cur = self._norm_matmul(l.ffn_gate_up, cur, alt, branch, l.ffn_norm, self.f, True)
             alt = other(cur)
             _check(lib.fhip_matmul_q(l.ffn_down.handle, self.f.buf.ptr, 1, self.y.buf.ptr, s))
+            pending = self.y
+            if l.post_ffn_norm is not None:              # x1 + post_ffn_norm(ffn(..)) (qwen3.rs:1019-1020)
+                _check(lib.fhip_rmsnorm(self.y.buf.ptr, l.post_ffn_norm.buf.ptr, 1, c.d_model, c.post_norm_eps, self.yn.buf.ptr, s))
+                pending = self.yn
         if self.lm_head is not None:   # last residual add fused with the output norm, then the LM head
-            cur = self._norm_matmul(self.lm_head, cur, alt, self.y, self.output_norm, self.logits, False)
+            cur = self._norm_matmul(self.lm_head, cur, alt, pending, self.output_norm, self.logits, False)
         else:
-            _check(lib.fhip_add(cur.buf.ptr, self.y.buf.ptr, c.d_model, cur.buf.ptr, s))
+            _check(lib.fhip_add(cur.buf.ptr, pending.buf.ptr, c.d_model, cur.buf.ptr, s))
         self.x = cur
         _check(lib.fhip_u32_add(self.pos.buf.ptr, 1, 1, s))
 

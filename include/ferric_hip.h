@@ -245,6 +245,12 @@ int fhip_add_rmsnorm(const float* d_a, const float* d_b, const float* d_weight, 
 
 /* lib.rs:279 Tensor::add, same shapes: out = a + b, n elements. */
 int fhip_add(const float* d_a, const float* d_b, size_t n, float* d_out, void* stream);
+/* out = a * sigmoid(g), n values; d_out may be d_a. The gate of a gated-attention layer on the attention output,
+ * crates/ferric-llama/src/qwen3.rs:936-938 (`o.mul(&h.matmul_q(wg).sigmoid())`), sigmoid as lib.rs:299 / :1915. */
+int fhip_mul_sigmoid(const float* d_a, const float* d_g, size_t n, float* d_out, void* stream);
+/* out [t, d] = gelu_tanh(gate) * up for rows gu [t, 2 d] = [gate | up]: Gemma's GEGLU, qwen3.rs:953-958, with the
+ * tanh-approximated GELU of lib.rs:304 / :1926. The unfused counterpart of fhip_swiglu for that activation. */
+int fhip_geglu(const float* d_gu, size_t t, size_t d, float* d_out, void* stream);
 
 /* lib.rs:417 Tensor::rope / :409 rope_interleaved / :429 rope_partial / :465 rope_at / :489 rope_at_ex (kernels :2118,
  * :2094). x: t rows of n_heads * head_dim, row i at d_x + i * src_row_stride (a strided window such as a slice of the

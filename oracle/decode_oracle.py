@@ -102,22 +102,51 @@ def silu_mul(gu, n_ff):
     return g / (1.0 + np.exp(-g)) * u
 
 
+def sigmoid(x):
+    """crates/ferric-tensor/src/lib.rs:1915: 1 / (1 + exp(-v))."""
+    return 1.0 / (1.0 + np.exp(-np.asarray(x, np.float64)))
+
+
+def gelu_tanh(x):
+    """lib.rs:1926: 0.5 v (1 + tanh(clamp(0.7978845608028654 (v + 0.044715 v^3), -15, 15)))."""
+    v = np.asarray(x, np.float64)
+    a = np.clip(0.7978845608028654 * (v + 0.044715 * v * v * v), -15.0, 15.0)
+    return 0.5 * v * (1.0 + np.tanh(a))
+
+
+def gelu_mul(gu, n_ff):
+    """crates/ferric-llama/src/qwen3.rs:953-958: gelu_tanh(gate) * up of rows [gate | up]."""
+    return gelu_tanh(gu[..., :n_ff]) * gu[..., n_ff:]
+
+
 class Layer:
-    """Dequantized (f64) weights of one layer: attn_norm, wqkv [q+2kv, d], wo, ffn_norm, gate_up [2 n_ff, d], down, norms."""
+    """Dequantized (f64) weights of one layer: attn_norm, wqkv [q+2kv, d], wo, ffn_norm, gate_up [2 n_ff, d], down, norms.
+    Optional, for the other arms of the reference's layer: window (keys a local layer attends to), rope (False: a NoPE layer),
+    rope_base, attn_gate [q, d], post_attn_norm / post_ffn_norm [d]."""
 
     def __init__(self, **kw):
         self.__dict__.update(kw)
 
 
 def apply_layer(x, l, kc, vc, pos, cfg):
-    """qwen3.rs:1041-1047 (default arm) for one token at position pos; kc / vc are lists of earlier K / V rows (appended to)."""
+    """qwen3.rs:979-1047 for one token at position pos; kc / vc are lists of earlier K / V rows (appended to). The default
+    arm (:1041-1047) unless the layer or the configuration carries one of: a sliding window and a score softcap (:917-924),
+    no rotation (:857-863: QK-norm still applies), its own rope base, a sigmoid gate on the attention output projected from
+    the normed input (:936-938), post-norms on both branch outputs with their own epsilon (:1015-1020), GEGLU (:953-958)."""
+    opt = lambda o, name, default: getattr(o, name, default) if getattr(o, name, None) is not None else default
     h = rmsnorm(x, l.attn_norm, cfg.eps)
     qkv = h @ l.wqkv.T
+    n_rot = cfg.head_dim if opt(l, "rope", True) else 0
     q, k, v = qkv_post(qkv.reshape(1, -1), getattr(l, "qkv_bias", None), getattr(l, "q_norm", None), getattr(l, "k_norm", None), [pos],
-                       cfg.n_head, cfg.n_head_kv, cfg.head_dim, cfg.eps, cfg.rope_base, cfg.rope_interleaved)
+                       cfg.n_head, cfg.n_head_kv, cfg.head_dim, cfg.eps, opt(l, "rope_base", cfg.rope_base), cfg.rope_interleaved, n_rot)
     kc.append(k[0]); vc.append(v[0])
-    a = decode_attention(q[0], np.stack(kc), np.stack(vc), cfg.n_head, cfg.n_head_kv)
+    a = decode_attention(q[0], np.stack(kc), np.stack(vc), cfg.n_head, cfg.n_head_kv, opt(l, "window", 0), opt(cfg, "attn_softcap", 0.0))
+    if getattr(l, "attn_gate", None) is not None:
+        a = a * sigmoid(h @ l.attn_gate.T)
     y = a[0] @ l.wo.T
-    xy = x + y
-    f = silu_mul(rmsnorm(xy, l.ffn_norm, cfg.eps) @ l.gate_up.T, cfg.n_ff)
-    return xy + f @ l.down.T
+    post = getattr(l, "post_attn_norm", None) is not None
+    pe = opt(cfg, "post_norm_eps", cfg.eps)
+    xy = x + (rmsnorm(y, l.post_attn_norm, pe) if post else y)
+    gu = rmsnorm(xy, l.ffn_norm, cfg.eps) @ l.gate_up.T
+    f = (gelu_mul(gu, cfg.n_ff) if opt(cfg, "geglu", False) else silu_mul(gu, cfg.n_ff)) @ l.down.T
+    return xy + (rmsnorm(f, l.post_ffn_norm, pe) if post else f)

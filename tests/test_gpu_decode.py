@@ -416,3 +416,112 @@ def test_decoder_steps_match_the_oracle_layer_by_layer_and_replay_as_a_graph(F, 
     assert np.array_equal(bits(dec2.hidden()), bits(eager[0]))
     head = O.deq_raw(head_raw, 300 * d, Q6_K).reshape(300, d).astype(np.float64)
     assert close(dec2.logits.to_vec(stream), D.rmsnorm(want[0], onorm, 1e-6) @ head.T, dot_bar(20))
+
+
+# ---------------------------------------------------------------- the other arms of the layer (qwen3.rs:857-863, 917-938, 953-958, 1015-1020)
+
+def test_mul_sigmoid_and_geglu(F, X, D):
+    rng = np.random.default_rng(31)
+    T = lambda a: F.Tensor.from_vec(a, a.shape)
+    # magnitudes from 1e-3 to 40, both signs, the saturated ends, zero; sizes that do not fill a workgroup
+    for n in (1, 255, 5120, 12345):
+        a = (rng.standard_normal(n) * 3).astype(np.float32)
+        g = (rng.standard_normal(n) * rng.choice([1e-3, 1.0, 10.0, 40.0], n)).astype(np.float32)
+        g[:1] = 0.0
+        got = X.mul_sigmoid(T(a.reshape(1, n)), T(g.reshape(1, n))).to_vec()
+        want = a.astype(np.float64) * D.sigmoid(g)
+        # expf and the division are each good to an ulp or two: 1e-6 of the value
+        assert (np.abs(got.reshape(-1) - want) <= 1e-6 * np.abs(want) + 1e-37).all(), n
+    out_in_place = T(np.ones((1, 64), np.float32))
+    F._lib.check(F._lib.load().fhip_mul_sigmoid(out_in_place.buf.ptr, T(np.zeros((1, 64), np.float32)).buf.ptr, 64, out_in_place.buf.ptr, None))
+    assert np.array_equal(out_in_place.to_vec(), np.full(64, 0.5, np.float32))
+    for t, d in ((1, 1), (1, 17408), (3, 1000), (5, 7)):
+        gu = (rng.standard_normal((t, 2 * d)) * rng.choice([0.01, 1.0, 4.0, 30.0], (t, 2 * d))).astype(np.float32)
+        gu[0, 0] = 0.0
+        got = X.geglu(T(gu)).to_vec().reshape(t, d)
+        want = D.gelu_mul(gu.astype(np.float64), d)
+        # tanhf to a few ulp, and 1 + tanh cancels for very negative gates, where the value itself is below 1e-6 |v u|
+        assert (np.abs(got - want) <= 2e-6 * np.abs(gu[:, :d].astype(np.float64) * gu[:, d:]) + 1e-37).all(), (t, d)
+    lib = F._lib.load()
+    assert lib.fhip_geglu(None, 1, 8, None, None) != 0 and b"NULL" in lib.fhip_last_error()
+    assert lib.fhip_mul_sigmoid(None, None, 0, None, None) == 0          # nothing to do
+
+
+def _arm_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, arms):
+    """_tiny_model with the optional members of each layer: arms is a list (one per layer) of sets out of
+    {"gate", "post", "nope", "window", "base"}."""
+    from ferric_amd.synth import synth_weights
+    from oracle import decode_oracle as D
+    layers, olayers = _tiny_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, True)
+    T = lambda a: F.Tensor.from_vec(a, a.shape)
+    for il, (l, ol, arm) in enumerate(zip(layers, olayers, arms)):
+        if "gate" in arm:
+            b = synth_weights(Q4_K, nh * hd, d, 900 + il)
+            l.attn_gate = F.QMatrix.from_bytes(b, Q4_K, nh * hd, d)
+            ol.attn_gate = O.deq_raw(b, nh * hd * d, Q4_K).reshape(nh * hd, d).astype(np.float64)
+        if "post" in arm:
+            pa, pf = (rng.random(d) + 0.5).astype(np.float32), (rng.random(d) + 0.5).astype(np.float32)
+            l.post_attn_norm, l.post_ffn_norm, ol.post_attn_norm, ol.post_ffn_norm = T(pa), T(pf), pa, pf
+        if "nope" in arm:
+            l.rope = ol.rope = False
+        if "window" in arm:
+            l.window = ol.window = 3
+        if "base" in arm:
+            l.rope_base = ol.rope_base = 1e4
+    return layers, olayers
+
+
+POST = {"post_norm_eps": 1e-8}
+
+
+@pytest.mark.parametrize("name,arms,cfg_kw,without,fuse", [
+    ("gated attention", [{"gate"}, set(), {"gate"}], {}, ([set()] * 3, {}), True),
+    ("gated attention, launches apart", [{"gate"}, {"gate"}, set()], {}, ([set()] * 3, {}), False),
+    ("post-norms with their own epsilon", [{"post"}] * 3, POST, ([set()] * 3, {}), True),
+    ("post-norms, launches apart", [{"post"}] * 3, POST, ([set()] * 3, {}), False),
+    ("local and global layers, NoPE on the global ones", [{"window", "base", "post"}, {"nope", "post"}, {"window", "base", "post"}],
+     dict(POST, attn_softcap=30.0), ([{"post"}] * 3, POST), True),
+    ("the same, launches apart", [{"window", "base", "post"}, {"nope", "post"}, {"window", "base", "post"}],
+     dict(POST, attn_softcap=30.0), ([{"post"}] * 3, POST), False),
+    ("GEGLU on post-normed layers", [{"post"}] * 3, dict(POST, geglu=True), ([{"post"}] * 3, POST), True),
+    ("GEGLU, launches apart", [{"post"}] * 3, dict(POST, geglu=True), ([{"post"}] * 3, POST), False),
+    ("everything at once", [{"gate", "post", "window"}, {"gate", "post", "nope"}, {"post", "base"}],
+     dict(POST, geglu=True, attn_softcap=50.0), ([{"post"}] * 3, POST), True),
+])
+def test_decoder_arms_match_the_oracle_and_replay_as_a_graph(F, X, O, D, name, arms, cfg_kw, without, fuse, precision):
+    n_layer, d, nh, nkv, hd, n_ff, steps = 3, 1024, 8, 2, 128, 1536, 6
+    cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6, **cfg_kw)
+    rng = np.random.default_rng(8)
+    layers, olayers = _arm_model(F, X, O, rng, n_layer, d, nh, nkv, hd, n_ff, arms)
+    xs = (np.random.default_rng(9).standard_normal((steps, d)) * 0.5).astype(np.float32)
+
+    def oracle_steps(ols, c):
+        kcs, vcs = [[] for _ in ols], [[] for _ in ols]
+        out = []
+        for pos in range(steps):
+            x = xs[pos].astype(np.float64)
+            for l, kc, vc in zip(ols, kcs, vcs):
+                x = D.apply_layer(x, l, kc, vc, pos, c)
+            out.append(x)
+        return out
+    want = oracle_steps(olayers, cfg)
+    # as the default arm's test: <= 20 times the bar of one dot product, of the step's largest hidden value
+    bar = dot_bar(20)
+    # The bar tells the arm from its absence: the oracle without it (same weights and norms) lies five bars away or more at some step.
+    _, oplain = _arm_model(F, X, O, np.random.default_rng(8), n_layer, d, nh, nkv, hd, n_ff, without[0])
+    plain = oracle_steps(oplain, X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6, **without[1]))
+    assert max(np.abs(a - b).max() / np.abs(a).max() for a, b in zip(want, plain)) > 5 * bar, name
+    stream = F.Stream()
+    dec = X.Qwen3Decoder(cfg, layers, max_len=steps + 2, stream=stream, fuse_norm=fuse, fuse_attn=fuse)
+    eager = []
+    for pos in range(steps):
+        dec.set_input(xs[pos])
+        dec.step()
+        eager.append(dec.hidden())
+        assert close(eager[-1], want[pos], bar), (name, pos)
+    dec.set_pos(0)
+    dec.capture()
+    for pos in range(steps):
+        dec.set_input(xs[pos])
+        dec.step_graph()
+        assert np.array_equal(bits(dec.hidden()), bits(eager[pos])), (name, pos)

@@ -160,3 +160,106 @@ def test_apply_layer_reduces_to_the_residual_when_the_output_projections_vanish(
     xy = x + a[0] @ l.wo.T
     f = D.silu_mul(D.rmsnorm(xy, l.ffn_norm, 1e-6) @ l.gate_up.T, 6)
     assert np.allclose(y, xy + f @ l.down.T, rtol=1e-13)
+
+
+def test_sigmoid_and_gelu_tanh_against_library_routines():
+    from scipy.special import expit
+    import torch
+    x = np.concatenate([np.linspace(-30, 30, 2001), [0.0, 1e-8, -1e-8, 88.0, -88.0]])
+    assert np.allclose(D.sigmoid(x), expit(x), rtol=1e-14, atol=0)
+    assert D.sigmoid(0.0) == 0.5 and np.allclose(D.sigmoid(x) + D.sigmoid(-x), 1.0, rtol=1e-15)
+    g = torch.nn.functional.gelu(torch.from_numpy(x), approximate="tanh").numpy()      # f64 on the CPU
+    inside = np.abs(0.7978845608028654 * (x + 0.044715 * x ** 3)) < 15                  # where the reference's clamp is idle
+    # (1 + tanh(a) cancels for a << 0: an absolute 1e-14 on values of 1e-12)
+    assert np.allclose(D.gelu_tanh(x)[inside], g[inside], rtol=1e-13, atol=1e-14)
+    # beyond the clamp tanh(15) = 1 - 1.9e-13: the value is x (or 0) to that relative error, as the unclamped form's
+    assert np.allclose(D.gelu_tanh(x)[~inside], g[~inside], rtol=1e-12, atol=1e-10)
+    assert np.allclose(D.gelu_tanh(x) - D.gelu_tanh(-x), x, rtol=1e-13, atol=1e-15)    # odd part of x Phi(x) is x / 2 twice
+    gu = np.array([[1.0, -2.0, 0.5, 3.0]])
+    assert np.array_equal(D.gelu_mul(gu, 2), D.gelu_tanh(gu[:, :2]) * gu[:, 2:])
+
+
+def _arm_layer(rng, d, nh, nkv, hd, n_ff):
+    return D.Layer(attn_norm=rng.random(d) + 0.5, wqkv=rng.standard_normal(((nh + 2 * nkv) * hd, d)), wo=rng.standard_normal((d, nh * hd)),
+                   ffn_norm=rng.random(d) + 0.5, gate_up=rng.standard_normal((2 * n_ff, d)), down=rng.standard_normal((d, n_ff)))
+
+
+def test_the_other_arms_of_apply_layer_by_their_invariants():
+    rng = np.random.default_rng(6)
+
+    class Cfg:
+        n_head, n_head_kv, head_dim, n_ff, eps, rope_base, rope_interleaved = 4, 2, 8, 12, 1e-6, 1e4, False
+    d = 16
+    l = _arm_layer(rng, d, 4, 2, 8, 12)
+    xs = rng.standard_normal((4, d))
+
+    def run(layer, cfg, positions=(0, 1, 2, 3)):
+        kc, vc, out = [], [], []
+        for x, pos in zip(xs, positions):
+            out.append(D.apply_layer(x, layer, kc, vc, pos, cfg))
+        return np.stack(out)
+    base = run(l, Cfg)
+    # gate: a zero gate projection is sigmoid(0) = 1/2 on every attention output, i.e. the output projection halved; a gate
+    # saturated at +40 is the ungated layer
+    lg = D.Layer(**l.__dict__); lg.attn_gate = np.zeros((32, d))
+    lh = D.Layer(**l.__dict__); lh.wo = l.wo * 0.5
+    assert np.allclose(run(lg, Cfg), run(lh, Cfg), rtol=1e-13)
+    big = D.Layer(**l.__dict__); big.attn_norm = np.ones(d); big.attn_gate = np.ones((32, d)) * 1e3
+    ref = D.Layer(**l.__dict__); ref.attn_norm = np.ones(d)
+    xs_pos = np.abs(xs)                                          # a normed input of positive entries: every gate logit >> 40
+    kc1, vc1, kc2, vc2 = [], [], [], []
+    assert np.allclose(D.apply_layer(xs_pos[0], big, kc1, vc1, 0, Cfg), D.apply_layer(xs_pos[0], ref, kc2, vc2, 0, Cfg), rtol=1e-13)
+    # window: at least the history is no window; a window of 1 attends to the newest key only, whose softmax weight is 1:
+    # the attention output is the token's own value row, whatever the history
+    lw = D.Layer(**l.__dict__); lw.window = 4
+    assert np.array_equal(run(lw, Cfg), base)
+    l1 = D.Layer(**l.__dict__); l1.window = 1
+    w1 = run(l1, Cfg)
+    assert np.allclose(w1[0], base[0], rtol=1e-13) and not np.allclose(w1[3], base[3], rtol=1e-3)
+    kc, vc = [rng.standard_normal(16)] * 3, [rng.standard_normal(16)] * 3      # another history, same result under window 1
+    assert np.allclose(D.apply_layer(xs[3], l1, kc, vc, 3, Cfg), w1[3], rtol=1e-13)
+    # NoPE: no rotation, so the positions do not matter; a rotating layer agrees with it at position 0 only
+    ln = D.Layer(**l.__dict__); ln.rope = False
+    assert np.allclose(run(ln, Cfg), run(ln, Cfg, positions=(7, 3, 11, 2)), rtol=1e-13)
+    assert np.allclose(run(ln, Cfg)[0], base[0], rtol=1e-13) and not np.allclose(run(ln, Cfg)[2], base[2], rtol=1e-3)
+    # the layer's own rope base replaces the configuration's
+    lb = D.Layer(**l.__dict__); lb.rope_base = 5e5
+
+    class Cfg5(Cfg):
+        rope_base = 5e5
+    assert np.array_equal(run(lb, Cfg), run(l, Cfg5)) and not np.allclose(run(lb, Cfg)[3], base[3], rtol=1e-6)
+    # softcap: a huge cap is the identity on the scores
+    class CfgCap(Cfg):
+        attn_softcap = 1e9
+    assert np.allclose(run(l, CfgCap), base, rtol=1e-9)
+    # post-norms: each branch output is normalised before the add, so (with a negligible epsilon) scaling an output projection
+    # leaves the layer unchanged, and unit post-norm weights give the branch at RMS 1
+    class CfgPost(Cfg):
+        post_norm_eps = 1e-30
+    lp = D.Layer(**l.__dict__); lp.post_attn_norm = rng.random(d) + 0.5; lp.post_ffn_norm = rng.random(d) + 0.5
+    ls = D.Layer(**lp.__dict__); ls.wo = lp.wo * 7.0; ls.down = lp.down * 0.125
+    assert np.allclose(run(lp, CfgPost), run(ls, CfgPost), rtol=1e-12) and not np.allclose(run(lp, CfgPost), base, rtol=1e-3)
+    lu = D.Layer(**l.__dict__); lu.post_attn_norm = np.ones(d); lu.post_ffn_norm = np.ones(d); lu.down = np.zeros((d, 12))
+    kc, vc = [], []
+    y = D.apply_layer(xs[0], lu, kc, vc, 0, CfgPost)             # down = 0: the FFN branch is rmsnorm(0) = 0
+    assert math.isclose(np.sqrt(np.mean((y - xs[0]) ** 2)), 1.0, rel_tol=1e-12)
+    # the post-norm epsilon is the configuration's own: with a large one the branch shrinks
+    class CfgPostBig(Cfg):
+        post_norm_eps = 1e6
+    kc, vc = [], []
+    yb = D.apply_layer(xs[0], lu, kc, vc, 0, CfgPostBig)
+    assert np.sqrt(np.mean((yb - xs[0]) ** 2)) < 0.1
+    # GEGLU: the same chain with the gate through the library's tanh GELU
+    import torch
+
+    class CfgGe(Cfg):
+        geglu = True
+    kc, vc = [], []
+    yg = D.apply_layer(xs[0], l, kc, vc, 0, CfgGe)
+    kc2, vc2 = [], []
+    h = D.rmsnorm(xs[0], l.attn_norm, 1e-6)
+    q, k, v = D.qkv_post((h @ l.wqkv.T).reshape(1, -1), None, None, None, [0], 4, 2, 8, 1e-6, 1e4)
+    xy = xs[0] + D.decode_attention(q[0], k, v, 4, 2)[0] @ l.wo.T
+    gu = D.rmsnorm(xy, l.ffn_norm, 1e-6) @ l.gate_up.T
+    act = torch.nn.functional.gelu(torch.from_numpy(gu[:12]), approximate="tanh").numpy() * gu[12:]
+    assert np.allclose(yg, xy + act @ l.down.T, rtol=1e-12)
