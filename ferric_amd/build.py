@@ -3,8 +3,8 @@
     python -m ferric_amd.build
 
 Every translation unit is compiled for gfx950 with packed-FP32 instruction selection switched
-off; dequant.hip additionally with -ffp-contract=off, because its outputs must match the
-reference's separately-rounded f32 arithmetic bit for bit.
+off; dequant.hip and kvquant.hip additionally with -ffp-contract=off, because their outputs
+must match the reference's separately-rounded f32 arithmetic bit for bit.
 """
 import os
 import subprocess
@@ -21,6 +21,7 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-
 UNITS = {
     "api.hip": [],
     "dequant.hip": ["-ffp-contract=off"],
+    "kvquant.hip": ["-ffp-contract=off"],       # the reference multiplies, then adds: no fused multiply-add
     "gemv.hip": ["-DFHIP_GEMV_PLANES=2"],
     "gemv.hip@p3": ["-DFHIP_GEMV_PLANES=3"],   # the same source again: the 24-bit-activation copy of the streaming mat-vec
     "gemv_generic.hip": [],

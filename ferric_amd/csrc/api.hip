@@ -725,6 +725,48 @@ int fhip_geglu(const float* d_gu, size_t t, size_t d, float* d_out, void* stream
     return fhip::launch_geglu(d_gu, t, d, d_out, (hipStream_t)stream);
 }
 
+static int kvq_checks(const char* who, int fmt, size_t width) {
+    if (fmt != FHIP_KVQ_Q8_0 && fmt != FHIP_KVQ_Q4_0 && fmt != FHIP_KVQ_Q4_1) return set_error(FHIP_ERR_ARG, "%s: unknown format %d", who, fmt);
+    // crates/ferric-tensor/src/kvquant.rs:470
+    if (width % 32 != 0) return set_error(FHIP_ERR_SHAPE, "QKvCache row width %zu must be a multiple of 32", width);
+    return FHIP_OK;
+}
+
+int fhip_kvq_sizes(int fmt, size_t rows, size_t width, size_t* code_words, size_t* scale_words) {
+    int rc = kvq_checks("fhip_kvq_sizes", fmt, width);
+    if (rc) return rc;
+    const size_t nblk = rows * (width / 32);
+    if (code_words) *code_words = nblk * (fmt == FHIP_KVQ_Q8_0 ? 8 : 4);
+    if (scale_words) *scale_words = fmt == FHIP_KVQ_Q4_1 ? nblk : (nblk + 1) / 2;
+    return FHIP_OK;
+}
+
+int fhip_kvq_append(int fmt, const float* d_src, size_t src_row_stride, size_t t, size_t width, const uint32_t* d_positions, uint32_t pos_off,
+                    int src_at_pos, size_t cap, uint32_t* d_codes, uint32_t* d_scales, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = kvq_checks("fhip_kvq_append", fmt, width))) return rc;
+    if (t == 0 || width == 0) return FHIP_OK;
+    if (!d_src || !d_codes || !d_scales) return set_error(FHIP_ERR_ARG, "fhip_kvq_append: NULL pointer");
+    if (src_row_stride == 0) src_row_stride = width;
+    if (src_row_stride < width) return set_error(FHIP_ERR_SHAPE, "fhip_kvq_append: source row stride %zu below the width %zu", src_row_stride, width);
+    if (!d_positions && (size_t)pos_off + t > cap)
+        return set_error(FHIP_ERR_SHAPE, "fhip_kvq_append: rows %u + %zu exceed the capacity %zu", pos_off, t, cap);
+    return fhip::launch_kvq_append(fmt, d_src, src_row_stride, t, width, d_positions, pos_off, src_at_pos != 0, cap, d_codes, (uint16_t*)d_scales,
+                                   (hipStream_t)stream);
+}
+
+int fhip_kvq_dequantize_rows(int fmt, const uint32_t* d_codes, const uint32_t* d_scales, size_t row0, size_t rows, size_t width,
+                             const uint32_t* d_last_pos, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = kvq_checks("fhip_kvq_dequantize_rows", fmt, width))) return rc;
+    if (rows == 0 || width == 0) return FHIP_OK;
+    if (!d_codes || !d_scales || !d_out) return set_error(FHIP_ERR_ARG, "fhip_kvq_dequantize_rows: NULL pointer");
+    if (((uintptr_t)d_out & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_kvq_dequantize_rows: the output must be 16-byte aligned");
+    return fhip::launch_kvq_dequantize(fmt, d_codes, (const uint16_t*)d_scales, row0, rows, width, d_last_pos, d_out, (hipStream_t)stream);
+}
+
 static int rope_checks(const char* who, size_t n_heads, size_t head_dim, size_t n_rot) {
     if (n_rot > head_dim || n_rot % 2 != 0) return set_error(FHIP_ERR_SHAPE, "n_rot must be even and <= head_dim");   // lib.rs:437
     if (n_heads > 0xFFFFu || head_dim > 0xFFFFu) return set_error(FHIP_ERR_SHAPE, "%s: n_heads / head_dim exceed 65535", who);

@@ -132,6 +132,11 @@ int launch_rmsnorm(const float* a, const float* b, const float* weight, size_t r
                    hipStream_t s);
 int launch_add(const float* a, const float* b, size_t n, float* out, hipStream_t s);
 int launch_u32_add(uint32_t* w, size_t n, uint32_t delta, hipStream_t s);
+// block-quantized K / V cache (kvquant.hip); scales addressed as uint16 [block] (Q4_1: [block][2])
+int launch_kvq_append(int fmt, const float* src, size_t src_row_stride, size_t t, size_t width, const uint32_t* d_pos, uint32_t pos_off,
+                      bool src_at_pos, size_t cap, uint32_t* codes, uint16_t* scales, hipStream_t s);
+int launch_kvq_dequantize(int fmt, const uint32_t* codes, const uint16_t* scales, size_t row0, size_t rows, size_t width, const uint32_t* d_last_pos,
+                          float* out, hipStream_t s);
 int launch_mul_sigmoid(const float* a, const float* g, size_t n, float* out, hipStream_t s);   // out = a * sigmoid(g); out may be a
 int launch_geglu(const float* gu, size_t t, size_t d, float* out, hipStream_t s);              // rows [gate | up] -> gelu_tanh(gate) * up
 int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int hd, int n_rot, float base, const uint32_t* d_pos, uint32_t pos_off,

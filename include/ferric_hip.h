@@ -276,6 +276,31 @@ int fhip_qkv_post(const float* d_qkv, const float* d_bias, const float* d_q_norm
                   const float* d_freq_scale, size_t t, size_t n_head, size_t n_kv, size_t head_dim, size_t n_rot, int interleaved,
                   float eps, float base, float* d_q_out, float* d_k_cache, float* d_v_cache, size_t cap, void* stream);
 
+/* Block-quantized K / V cache, crates/ferric-tensor/src/kvquant.rs (KvqFmt :57-64): rows of `width` values (a multiple of
+ * 32, else FHIP_ERR_SHAPE with the reference's message, :470) stored as llama.cpp-layout blocks of 32 along the row, block
+ * b = row * (width / 32) + col / 32. d_codes: 8 (Q8_0) or 4 (Q4_0, Q4_1) u32 words per block; d_scales: f16 bit patterns,
+ * two blocks per u32 word for Q8_0 / Q4_0 (block b in half b % 2 of word b / 2), one word d | min << 16 per block for Q4_1:
+ * the reference's `codes` / `scales` buffers byte for byte, and its arithmetic operation for operation (`mod reference`,
+ * :943-1186: d = amax / 127 with roundf; d = extreme / -8 with floor(x + 8.5); d = (max - min) / 15 with floor(x + 0.5)), so
+ * codes, scales and dequantized values are bit-identical to the reference's. */
+#define FHIP_KVQ_Q8_0 0
+#define FHIP_KVQ_Q4_0 1
+#define FHIP_KVQ_Q4_1 2
+/* KvqFmt::code_words / scale_words (:66-81) for rows x width: u32 words of each array. */
+int fhip_kvq_sizes(int fmt, size_t rows, size_t width, size_t* code_words, size_t* scale_words);
+/* QKvCache::append (:464-517) without the growth (the caller owns arrays of `cap` rows): quantizes exactly the t rows handed
+ * over and writes their blocks at their flat offsets; nothing already stored is touched or read. Source row i is at
+ * d_src + i * src_row_stride (0 = packed; a window of a fused qkv row is read in place) and goes to cache row
+ * d_positions[i] (device u32) or pos_off + i. src_at_pos != 0: the source row index is the cache row too (the newest row of
+ * an f32 staging cache of full length), for a captured decode step whose position lives in a device word. */
+int fhip_kvq_append(int fmt, const float* d_src, size_t src_row_stride, size_t t, size_t width, const uint32_t* d_positions, uint32_t pos_off,
+                    int src_at_pos, size_t cap, uint32_t* d_codes, uint32_t* d_scales, void* stream);
+/* QKvCache::dequantize_rows (:621-650; dequantize :617 is row0 = 0, rows = len): cache rows row0 .. row0 + rows to f32
+ * d_out [rows, width]. d_last_pos (optional, device u32): rows past *d_last_pos are not written, so a captured step can pass
+ * the capacity as `rows` and the position word of the token being decoded. */
+int fhip_kvq_dequantize_rows(int fmt, const uint32_t* d_codes, const uint32_t* d_scales, size_t row0, size_t rows, size_t width,
+                             const uint32_t* d_last_pos, float* d_out, void* stream);
+
 /* crates/ferric-tensor/src/nn.rs:140 decode_attention -> lib.rs:762 fused_decode_attention (kernels :2675, :2740 ff.):
  * one query row q [n_head * head_dim] against the cache rows [0, len) of K and V [., n_kv * head_dim];
  * out[h] = softmax_j(q_h . K[j, h / g] / sqrt(head_dim)) @ V[:, h / g], g = n_head / n_kv (1..=8), head_dim 64 or 128.
