@@ -408,12 +408,28 @@ def decode_stack(F, lib, check, layers=64):
     return cfg, lay, small, head, weight_bytes_total, stacks
 
 
-def decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, room, stream, rng):
-    """A decoder over the stack with `ctx` earlier tokens' keys and values (synthetic) in every layer's cache and an input set."""
+def decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, room, stream, rng, kv_fmt=None):
+    """A decoder over the stack with `ctx` earlier tokens' keys and values (synthetic) in every layer's cache and an input set.
+    kv_fmt: block-quantized caches of that format instead of f32 ones."""
     from ferric_amd import decode as X
     nkv, hd, d = cfg.n_head_kv, cfg.head_dim, cfg.d_model
-    dec = X.Qwen3Decoder(cfg, lay, max_len=ctx + room + 2, stream=stream, output_norm=small, lm_head=head)
+    dec = X.Qwen3Decoder(cfg, lay, max_len=ctx + room + 2, stream=stream, output_norm=small, lm_head=head, kv_fmt=kv_fmt)
     kv_fill = (rng.standard_normal((ctx, nkv * hd)) * 0.5).astype(np.float32)
+    if kv_fmt is not None:
+        kq = dec.caches[0][0]                     # quantized once, the packed arrays copied on the device
+        kq.append(F.Tensor.from_vec(kv_fill, kv_fill.shape))
+        check(lib.fhip_stream_sync(None))
+        from ferric_amd import kvquant
+        cw, sw = kvquant.sizes(kv_fmt, ctx, nkv * hd)
+        for pair in dec.caches:
+            for c in pair:
+                if c is not kq:
+                    check(lib.fhip_memcpy_d2d(c.codes.ptr, kq.codes.ptr, cw * 4, None))
+                    check(lib.fhip_memcpy_d2d(c.scales.ptr, kq.scales.ptr, sw * 4, None))
+        check(lib.fhip_stream_sync(None))
+        dec.set_pos(ctx)
+        dec.set_input((rng.standard_normal(d) * 0.5).astype(np.float32))
+        return dec
     first = dec.caches[0]                         # uploaded once, copied on the device
     check(lib.fhip_memcpy_h2d(first.k.buf.ptr, kv_fill.ctypes.data_as(C.c_void_p), kv_fill.nbytes, None))
     check(lib.fhip_stream_sync(None))
@@ -446,8 +462,19 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
                          "kv_bytes_read": kv_bytes, "GBps_weights_plus_kv": (weight_bytes_total + kv_bytes) / (ms * 1e-3) / 1e9,
                          "logits_finite": bool(np.isfinite(logits).all())}
         del dec
+    # the same step on a Q8_0 block-quantized cache, attention reading the blocks in place (8.5 bits per cached value)
+    ctx = contexts[-1]
+    dec = decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, steps, stream, rng, kv_fmt=0)
+    dec.capture()
+    dec.step_graph()
+    ms = timer.time_ms(lambda: [dec.step_graph() for _ in range(steps)]) / steps
+    logits = dec.logits.to_vec(stream)
+    kv_bytes = 2 * (ctx + steps // 2) * (nkv * hd // 32) * 34 * layers
+    out[f"{ctx}_q8_0_cache"] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * dec.launches_per_layer + 2,
+                                "kv_bytes_read": kv_bytes, "logits_finite": bool(np.isfinite(logits).all())}
+    del dec
     out["weight_bytes"] = weight_bytes_total
-    out["model"] = "64 layers, d 5120, 40 query / 8 KV heads x 128, n_ff 17408, vocab 151936; Q4_K projections, Q6_K down and lm_head; f32 KV cache"
+    out["model"] = "64 layers, d 5120, 40 query / 8 KV heads x 128, n_ff 17408, vocab 151936; Q4_K projections, Q6_K down and lm_head; f32 KV cache (the _q8_0_cache entry: Q8_0 blocks)"
     return out
 
 

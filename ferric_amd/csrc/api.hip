@@ -808,6 +808,48 @@ int fhip_qkv_post(const float* d_qkv, const float* d_bias, const float* d_q_norm
                                  (int)n_rot, interleaved != 0, eps, base, d_q_out, d_k_cache, d_v_cache, cap, (hipStream_t)stream);
 }
 
+int fhip_qkv_post_packed(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_positions,
+                         const float* d_freq_scale, size_t t, size_t n_head, size_t n_kv, size_t head_dim, size_t n_rot, int interleaved,
+                         float eps, float base, float* d_q_out, float* d_k_out, float* d_v_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = rope_checks("fhip_qkv_post_packed", n_head + 2 * n_kv, head_dim, n_rot))) return rc;
+    if (t == 0 || head_dim == 0 || n_head + n_kv == 0) return FHIP_OK;
+    if (!d_qkv || !d_positions || !d_q_out || !d_k_out || !d_v_out) return set_error(FHIP_ERR_ARG, "fhip_qkv_post_packed: NULL pointer");
+    return fhip::launch_qkv_post(d_qkv, d_bias, d_q_norm, d_k_norm, d_positions, d_freq_scale, t, (int)n_head, (int)n_kv, (int)head_dim,
+                                 (int)n_rot, interleaved != 0, eps, base, d_q_out, d_k_out, d_v_out, 0, (hipStream_t)stream, true);
+}
+
+int fhip_kvq_append2(int fmt, const float* d_k, const float* d_v, size_t src_row_stride, size_t t, size_t width, const uint32_t* d_positions,
+                     uint32_t pos_off, size_t cap, uint32_t* d_k_codes, uint32_t* d_k_scales, uint32_t* d_v_codes, uint32_t* d_v_scales,
+                     void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = kvq_checks("fhip_kvq_append2", fmt, width))) return rc;
+    if (t == 0 || width == 0) return FHIP_OK;
+    if (!d_k || !d_v || !d_k_codes || !d_k_scales || !d_v_codes || !d_v_scales) return set_error(FHIP_ERR_ARG, "fhip_kvq_append2: NULL pointer");
+    if (src_row_stride == 0) src_row_stride = width;
+    if (src_row_stride < width) return set_error(FHIP_ERR_SHAPE, "fhip_kvq_append2: source row stride %zu below the width %zu", src_row_stride, width);
+    if (!d_positions && (size_t)pos_off + t > cap)
+        return set_error(FHIP_ERR_SHAPE, "fhip_kvq_append2: rows %u + %zu exceed the capacity %zu", pos_off, t, cap);
+    return fhip::launch_kvq_append(fmt, d_k, src_row_stride, t, width, d_positions, pos_off, false, cap, d_k_codes, (uint16_t*)d_k_scales,
+                                   (hipStream_t)stream, d_v, d_v_codes, (uint16_t*)d_v_scales);
+}
+
+int fhip_decode_attention_kvq(int fmt, const float* d_q, const uint32_t* d_k_codes, const uint32_t* d_k_scales, const uint32_t* d_v_codes,
+                              const uint32_t* d_v_scales, size_t n_head, size_t n_kv, size_t head_dim, size_t len, const uint32_t* d_last_pos,
+                              size_t window, float softcap, float* d_ws, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if ((rc = kvq_checks("fhip_decode_attention_kvq", fmt, n_kv * head_dim))) return rc;
+    if (n_head == 0 || head_dim == 0) return FHIP_OK;
+    if (!d_q || !d_k_codes || !d_k_scales || !d_v_codes || !d_v_scales || !d_out)
+        return set_error(FHIP_ERR_ARG, "fhip_decode_attention_kvq: NULL pointer");
+    if (n_head > 0x7FFFFFFFull || n_kv > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "fhip_decode_attention_kvq: too many heads");
+    return fhip::launch_decode_attention_kvq(fmt, d_q, d_k_codes, (const uint16_t*)d_k_scales, d_v_codes, (const uint16_t*)d_v_scales, (int)n_head,
+                                             (int)n_kv, (int)head_dim, len, d_last_pos, window, softcap, d_ws, d_out, (hipStream_t)stream);
+}
+
 size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_dim, size_t len) {
     if (g_device < 0 || n_kv == 0 || len == 0) return 0;
     int splits = fhip::attn_splits(len, (int)n_kv);

@@ -134,7 +134,11 @@ int launch_add(const float* a, const float* b, size_t n, float* out, hipStream_t
 int launch_u32_add(uint32_t* w, size_t n, uint32_t delta, hipStream_t s);
 // block-quantized K / V cache (kvquant.hip); scales addressed as uint16 [block] (Q4_1: [block][2])
 int launch_kvq_append(int fmt, const float* src, size_t src_row_stride, size_t t, size_t width, const uint32_t* d_pos, uint32_t pos_off,
-                      bool src_at_pos, size_t cap, uint32_t* codes, uint16_t* scales, hipStream_t s);
+                      bool src_at_pos, size_t cap, uint32_t* codes, uint16_t* scales, hipStream_t s, const float* src2 = nullptr,
+                      uint32_t* codes2 = nullptr, uint16_t* scales2 = nullptr);
+int launch_decode_attention_kvq(int fmt, const float* q, const uint32_t* k_codes, const uint16_t* k_scales, const uint32_t* v_codes,
+                                const uint16_t* v_scales, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len, size_t window,
+                                float softcap, float* ws, float* out, hipStream_t s);
 int launch_kvq_dequantize(int fmt, const uint32_t* codes, const uint16_t* scales, size_t row0, size_t rows, size_t width, const uint32_t* d_last_pos,
                           float* out, hipStream_t s);
 int launch_mul_sigmoid(const float* a, const float* g, size_t n, float* out, hipStream_t s);   // out = a * sigmoid(g); out may be a
@@ -143,7 +147,7 @@ int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int 
                 const float* freq_scale, int interleaved, float* out, hipStream_t s);
 int launch_qkv_post(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos, const float* freq_scale,
                     size_t t, int n_head, int n_kv, int hd, int n_rot, int interleaved, float eps, float base, float* q_out, float* k_cache,
-                    float* v_cache, size_t cap, hipStream_t s);
+                    float* v_cache, size_t cap, hipStream_t s, bool kv_packed = false);   // kv_packed: K / V rows to packed [t, n_kv * hd] outputs
 int launch_kv_append(const float* k, const float* v, size_t t, size_t width, const uint32_t* d_pos, uint32_t pos_off, size_t cap, float* kc,
                      float* vc, hipStream_t s);
 int attn_splits(size_t len, int n_kv);

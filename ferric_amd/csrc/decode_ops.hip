@@ -11,6 +11,8 @@
 // except attention, which streams the layer's K and V rows once (HBM-bound: 2 * len * n_kv * head_dim * 4 bytes).
 #include "common.hpp"
 
+#include <hip/hip_fp16.h>
+
 #include <math.h>
 #include <stdlib.h>
 
@@ -180,6 +182,7 @@ struct QkvPostParams {
     int t, n_head, n_kv, hd, n_rot, interleaved;
     uint32_t cap;
     float eps, base;
+    int kv_packed;           // != 0: k_cache / v_cache are packed [t, n_kv * hd] outputs, row i for token i (cap is not looked at)
 };
 
 __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
@@ -196,10 +199,11 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostParams p) {
     float* dst;
     const float* nw;
     bool rotate = true;
+    const size_t kv_row = p.kv_packed ? (size_t)i : (size_t)pos;
     if (h < p.n_head) { dst = p.q_out + ((size_t)i * p.n_head + h) * p.hd; nw = p.q_norm; }
-    else if (h < p.n_head + p.n_kv) { dst = p.k_cache + (size_t)pos * kvw + (size_t)(h - p.n_head) * p.hd; nw = p.k_norm; }
-    else { dst = p.v_cache + (size_t)pos * kvw + (size_t)(h - p.n_head - p.n_kv) * p.hd; nw = nullptr; rotate = false; }
-    if (h >= p.n_head && pos >= p.cap) return;   // a position past the cache is dropped, never written out of bounds
+    else if (h < p.n_head + p.n_kv) { dst = p.k_cache + kv_row * kvw + (size_t)(h - p.n_head) * p.hd; nw = p.k_norm; }
+    else { dst = p.v_cache + kv_row * kvw + (size_t)(h - p.n_head - p.n_kv) * p.hd; nw = nullptr; rotate = false; }
+    if (h >= p.n_head && !p.kv_packed && pos >= p.cap) return;   // a position past the cache is dropped, never written out of bounds
     if (!rotate) {
         for (int j = lane; j < p.hd; j += 64) dst[j] = bias ? x[j] + bias[j] : x[j];
         return;
@@ -265,6 +269,48 @@ __device__ __forceinline__ void load_dims(const float* p, float (&r)[DPL]) {   /
     }
 }
 
+// A block-quantized cache (kvquant.hip's layout) read in place: codes and f16 scales of the keys and of the values.
+struct QCache {
+    const uint32_t* k_codes; const uint16_t* k_scales;
+    const uint32_t* v_codes; const uint16_t* v_scales;
+};
+// DPL (4 or 8) consecutive dims of one row, starting at column `col` (a multiple of DPL) of block row `key`: the values the
+// dequantize kernel would write, by the same single operations (q * d; (q - 8) * d; q * d then + m, not fused), so attention
+// over the codes is attention over the dequantized rows, bit for bit.
+template <int FMT, int DPL>
+__device__ __forceinline__ void load_dims_q(const uint32_t* __restrict__ codes, const uint16_t* __restrict__ scales, size_t key, int nblk, int col,
+                                            float (&r)[DPL]) {
+#pragma clang fp contract(off)
+    const size_t b = key * (size_t)nblk + (size_t)(col >> 5);
+    const int j = col & 31;
+    if constexpr (FMT == FHIP_KVQ_Q8_0) {
+        const float d = __half2float(__ushort_as_half(scales[b]));
+#pragma unroll
+        for (int w = 0; w < DPL / 4; w++) {
+            const uint32_t word = codes[b * 8 + (j >> 2) + w];
+            r[4 * w] = (float)(int8_t)(word & 255u) * d;
+            r[4 * w + 1] = (float)(int8_t)((word >> 8) & 255u) * d;
+            r[4 * w + 2] = (float)(int8_t)((word >> 16) & 255u) * d;
+            r[4 * w + 3] = (float)(int8_t)(word >> 24) * d;
+        }
+    } else {
+        const int shift = j < 16 ? 0 : 4;
+        float d, m = 0.f;
+        if constexpr (FMT == FHIP_KVQ_Q4_0) d = __half2float(__ushort_as_half(scales[b]));
+        else { d = __half2float(__ushort_as_half(scales[2 * b])); m = __half2float(__ushort_as_half(scales[2 * b + 1])); }
+#pragma unroll
+        for (int w = 0; w < DPL / 4; w++) {
+            const uint32_t word = codes[b * 4 + ((j & 15) >> 2) + w] >> shift;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float n = (float)((word >> (8 * i)) & 15u);
+                if constexpr (FMT == FHIP_KVQ_Q4_0) r[4 * w + i] = (n - 8.0f) * d;
+                else { const float t = n * d; r[4 * w + i] = t + m; }
+            }
+        }
+    }
+}
+
 // FUSED: the query heads do not come from memory but are formed here from the raw QKV row of the newest token -- bias, per-head
 // RMSNorm, rotation, exactly qkv_post_kernel's arithmetic -- by every workgroup for its own G heads, into LDS; and the
 // workgroup whose key range holds the token's position also forms that token's K and V rows for its KV head and appends them
@@ -273,11 +319,13 @@ __device__ __forceinline__ void load_dims(const float* p, float (&r)[DPL]) {   /
 template <bool FUSED> struct CachePtr { typedef const float* __restrict__ type; };
 template <> struct CachePtr<true> { typedef const float* type; };   // the fused kernel also writes the cache: no promise of no alias
 
-template <int G, int DPL, bool FUSED>
+// QF: -1 for an f32 cache (K, V), else the FHIP_KVQ_* format of the block-quantized cache in qc (K and V are null then).
+template <int G, int DPL, bool FUSED, int QF = -1>
 __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typename CachePtr<FUSED>::type K, typename CachePtr<FUSED>::type V,
                                                 int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
                                                 uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out,
-                                                const QkvPostParams& fp) {
+                                                const QkvPostParams& fp, const QCache& qc = QCache{}) {
+    static_assert(!(FUSED && QF >= 0), "the fused post-processing appends f32 rows");
     constexpr int HD = 16 * DPL;
     __shared__ float sm_m[4][G], sm_l[4][G];
     __shared__ float sm_acc[4][G][HD];
@@ -311,8 +359,8 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
     const uint32_t per = (len - first + splits - 1) / splits;
     const uint32_t k0 = first + (uint32_t)split * per, k1 = min(len, k0 + per);
     const size_t stride = (size_t)n_kv * HD;
-    const float* Kb = K + (size_t)kvh * HD + sub * DPL;
-    const float* Vb = V + (size_t)kvh * HD + sub * DPL;
+    const float* Kb = QF >= 0 ? nullptr : K + (size_t)kvh * HD + sub * DPL;
+    const float* Vb = QF >= 0 ? nullptr : V + (size_t)kvh * HD + sub * DPL;
 
     if constexpr (FUSED) {
         const uint32_t pos = *len_dev;
@@ -375,8 +423,13 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
 #pragma unroll
         for (int j = 0; j < ATT_KB; j++) {
             const uint32_t key = min(kb + j, k1 - 1);   // a row past the split re-reads its last row and is masked below
-            load_dims<DPL>(Kb + key * stride, kr[j]);
-            load_dims<DPL>(Vb + key * stride, vr[j]);
+            if constexpr (QF >= 0) {
+                load_dims_q<QF, DPL>(qc.k_codes, qc.k_scales, key, n_kv * (HD / 32), kvh * HD + sub * DPL, kr[j]);
+                load_dims_q<QF, DPL>(qc.v_codes, qc.v_scales, key, n_kv * (HD / 32), kvh * HD + sub * DPL, vr[j]);
+            } else {
+                load_dims<DPL>(Kb + key * stride, kr[j]);
+                load_dims<DPL>(Vb + key * stride, vr[j]);
+            }
         }
 #pragma unroll
         for (int h = 0; h < G; h++) {
@@ -455,6 +508,13 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict
     attn_split_body<G, DPL, false>(q, K, V, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, QkvPostParams{});
 }
 
+template <int G, int DPL, int QF>
+__global__ __launch_bounds__(256) void attn_split_kvq_kernel(const float* __restrict__ q, QCache qc, int n_kv, uint32_t len_host,
+                                                             const uint32_t* __restrict__ len_dev, float scale, int splits, uint32_t window,
+                                                             float softcap, float* __restrict__ part, float* __restrict__ out) {
+    attn_split_body<G, DPL, false, QF>(q, nullptr, nullptr, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, QkvPostParams{}, qc);
+}
+
 template <int G, int DPL>
 __global__ __launch_bounds__(256) void attn_split_fused_kernel(QkvPostParams fp, int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev,
                                                                float scale, int splits, uint32_t window, float softcap, float* __restrict__ part,
@@ -507,6 +567,32 @@ int launch_attn_g(int hd, dim3 grid, hipStream_t s, const float* q, const float*
         default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     }
     return FHIP_OK;
+}
+
+template <int G, int QF>
+int launch_attn_kvq_g(int hd, dim3 grid, hipStream_t s, const float* q, const QCache& qc, int n_kv, uint32_t len, const uint32_t* d_len,
+                      float scale, int splits, uint32_t window, float softcap, float* part, float* out) {
+    switch (hd) {
+        case 64: hipLaunchKernelGGL((attn_split_kvq_kernel<G, 4, QF>), grid, dim3(256), 0, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        case 128: hipLaunchKernelGGL((attn_split_kvq_kernel<G, 8, QF>), grid, dim3(256), 0, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
+    }
+    return FHIP_OK;
+}
+template <int QF>
+int launch_attn_kvq(int g, int hd, dim3 grid, hipStream_t s, const float* q, const QCache& qc, int n_kv, uint32_t len, const uint32_t* d_len,
+                    float scale, int splits, uint32_t window, float softcap, float* part, float* out) {
+    switch (g) {
+        case 1: return launch_attn_kvq_g<1, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        case 2: return launch_attn_kvq_g<2, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        case 3: return launch_attn_kvq_g<3, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        case 4: return launch_attn_kvq_g<4, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        case 5: return launch_attn_kvq_g<5, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        case 6: return launch_attn_kvq_g<6, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        case 7: return launch_attn_kvq_g<7, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        case 8: return launch_attn_kvq_g<8, QF>(hd, grid, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out);
+        default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: %d query heads per KV head (1..=8 supported)", g);
+    }
 }
 
 template <int G>
@@ -584,13 +670,13 @@ int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int 
 
 int launch_qkv_post(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos, const float* freq_scale,
                     size_t t, int n_head, int n_kv, int hd, int n_rot, int interleaved, float eps, float base, float* q_out, float* k_cache,
-                    float* v_cache, size_t cap, hipStream_t s) {
+                    float* v_cache, size_t cap, hipStream_t s, bool kv_packed) {
     if (t == 0) return FHIP_OK;
     QkvPostParams p;
     p.qkv = qkv; p.bias = bias; p.q_norm = q_norm; p.k_norm = k_norm; p.pos = d_pos; p.freq_scale = freq_scale;
     p.q_out = q_out; p.k_cache = k_cache; p.v_cache = v_cache;
     p.t = (int)t; p.n_head = n_head; p.n_kv = n_kv; p.hd = hd; p.n_rot = n_rot; p.interleaved = interleaved;
-    p.cap = (uint32_t)cap; p.eps = eps; p.base = base;
+    p.cap = (uint32_t)cap; p.eps = eps; p.base = base; p.kv_packed = kv_packed ? 1 : 0;
     size_t waves = t * (size_t)(n_head + 2 * n_kv), grid = (waves + 3) / 4;
     if (t > 0x7FFFFFFFull || grid > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "qkv_post: too many rows for one launch");
     hipLaunchKernelGGL(qkv_post_kernel, dim3((unsigned)grid), dim3(256), 0, s, p);
@@ -653,6 +739,36 @@ int launch_decode_attention(const float* q, const float* K, const float* V, int 
     return rc;
 }
 
+int launch_decode_attention_kvq(int fmt, const float* q, const uint32_t* k_codes, const uint16_t* k_scales, const uint32_t* v_codes,
+                                const uint16_t* v_scales, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len, size_t window,
+                                float softcap, float* ws, float* out, hipStream_t s) {
+    if (n_head == 0 || hd == 0) return FHIP_OK;
+    if (len == 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: empty cache");
+    if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: n_heads must be a multiple of n_kv_heads");
+    if (hd != 64 && hd != 128) return set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
+    if (len > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "decode_attention: cache length exceeds 2^31");
+    const int g = n_head / n_kv, splits = attn_splits(len, n_kv);
+    if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
+    const float scale = 1.0f / sqrtf((float)hd);
+    const uint32_t win = window > 0x7FFFFFFFull ? 0u : (uint32_t)window;
+    const dim3 grid((unsigned)n_kv, (unsigned)splits);
+    const QCache qc{k_codes, k_scales, v_codes, v_scales};
+    int rc;
+    switch (fmt) {
+        case FHIP_KVQ_Q8_0: rc = launch_attn_kvq<FHIP_KVQ_Q8_0>(g, hd, grid, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case FHIP_KVQ_Q4_0: rc = launch_attn_kvq<FHIP_KVQ_Q4_0>(g, hd, grid, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        case FHIP_KVQ_Q4_1: rc = launch_attn_kvq<FHIP_KVQ_Q4_1>(g, hd, grid, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
+        default: return set_error(FHIP_ERR_ARG, "decode_attention: unknown KV format %d", fmt);
+    }
+    if (rc) return rc;
+    if ((rc = check_hip(hipGetLastError(), "decode_attention launch"))) return rc;
+    if (splits > 1) {
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)n_head), dim3(COMBINE_THREADS), 0, s, ws, hd, splits, out);
+        rc = check_hip(hipGetLastError(), "decode_attention combine launch");
+    }
+    return rc;
+}
+
 int launch_qkv_post_attention(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos,
                               const float* freq_scale, int n_head, int n_kv, int hd, int n_rot, bool interleaved, float eps, float base,
                               float* k_cache, float* v_cache, size_t cap, size_t len, size_t window, float softcap, float* ws, float* out,
@@ -668,7 +784,7 @@ int launch_qkv_post_attention(const float* qkv, const float* bias, const float* 
     fp.qkv = qkv; fp.bias = bias; fp.q_norm = q_norm; fp.k_norm = k_norm; fp.pos = d_pos; fp.freq_scale = freq_scale;
     fp.q_out = nullptr; fp.k_cache = k_cache; fp.v_cache = v_cache;
     fp.t = 1; fp.n_head = n_head; fp.n_kv = n_kv; fp.hd = hd; fp.n_rot = n_rot; fp.interleaved = interleaved ? 1 : 0;
-    fp.cap = (uint32_t)cap; fp.eps = eps; fp.base = base;
+    fp.cap = (uint32_t)cap; fp.eps = eps; fp.base = base; fp.kv_packed = 0;
     const float scale = 1.0f / sqrtf((float)hd);
     const uint32_t win = window > 0x7FFFFFFFull ? 0u : (uint32_t)window;
     dim3 grid((unsigned)n_kv, (unsigned)splits);

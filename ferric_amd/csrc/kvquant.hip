@@ -97,11 +97,19 @@ __device__ __forceinline__ void quantize_block(const float (&v)[QK], uint32_t* _
 }
 
 // One thread per block of t source rows. Row i goes to cache row pos[i] (or pos_off + i); src_at_pos: the source row sits at
-// that index too (the newest row of a full-length f32 staging cache), else at i.
+// that index too (the newest row of a full-length f32 staging cache), else at i. blockIdx.y picks one of up to two
+// (source, cache) pairs, so a token's K and V rows are stored by one launch.
+struct KvqTargets {
+    const float* src[2];
+    uint32_t* codes[2];
+    uint16_t* scales[2];
+};
 template <int FMT>
-__global__ __launch_bounds__(256) void kvq_quant_kernel(const float* __restrict__ src, size_t src_row_stride, int t, int nblk,
-                                                       const uint32_t* __restrict__ pos, uint32_t pos_off, int src_at_pos, uint32_t cap,
-                                                       uint32_t* __restrict__ codes, uint16_t* __restrict__ scales) {
+__global__ __launch_bounds__(256) void kvq_quant_kernel(KvqTargets tg, size_t src_row_stride, int t, int nblk,
+                                                       const uint32_t* __restrict__ pos, uint32_t pos_off, int src_at_pos, uint32_t cap) {
+    const float* __restrict__ src = tg.src[blockIdx.y];
+    uint32_t* __restrict__ codes = tg.codes[blockIdx.y];
+    uint16_t* __restrict__ scales = tg.scales[blockIdx.y];
     const size_t id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (id >= (size_t)t * nblk) return;
     const int i = (int)(id / nblk), cb = (int)(id % nblk);
@@ -162,17 +170,23 @@ __global__ __launch_bounds__(256) void kvq_dequant_kernel(const uint32_t* __rest
 
 namespace fhip {
 
+// src2 / codes2 / scales2: a second source and cache of the same shape stored by the same launch (null: one only)
 int launch_kvq_append(int fmt, const float* src, size_t src_row_stride, size_t t, size_t width, const uint32_t* d_pos, uint32_t pos_off,
-                      bool src_at_pos, size_t cap, uint32_t* codes, uint16_t* scales, hipStream_t s) {
+                      bool src_at_pos, size_t cap, uint32_t* codes, uint16_t* scales, hipStream_t s, const float* src2, uint32_t* codes2,
+                      uint16_t* scales2) {
     if (t == 0 || width == 0) return FHIP_OK;
     const size_t nblk = width / QK, n = t * nblk, grid = (n + 255) / 256;
     if (t > 0x7FFFFFFFull || nblk > 0x7FFFFFFFull || grid > 0x7FFFFFFFull || cap > 0xFFFFFFFFull)
         return set_error(FHIP_ERR_SHAPE, "kvq_append: too large for one launch");
-    const dim3 g((unsigned)grid), wg(256);
+    const dim3 g((unsigned)grid, src2 ? 2u : 1u), wg(256);
+    KvqTargets tg;
+    tg.src[0] = src; tg.codes[0] = codes; tg.scales[0] = scales;
+    tg.src[1] = src2; tg.codes[1] = codes2; tg.scales[1] = scales2;
+    const int at = src_at_pos ? 1 : 0;
     switch (fmt) {
-        case FHIP_KVQ_Q8_0: hipLaunchKernelGGL((kvq_quant_kernel<FHIP_KVQ_Q8_0>), g, wg, 0, s, src, src_row_stride, (int)t, (int)nblk, d_pos, pos_off, src_at_pos ? 1 : 0, (uint32_t)cap, codes, scales); break;
-        case FHIP_KVQ_Q4_0: hipLaunchKernelGGL((kvq_quant_kernel<FHIP_KVQ_Q4_0>), g, wg, 0, s, src, src_row_stride, (int)t, (int)nblk, d_pos, pos_off, src_at_pos ? 1 : 0, (uint32_t)cap, codes, scales); break;
-        case FHIP_KVQ_Q4_1: hipLaunchKernelGGL((kvq_quant_kernel<FHIP_KVQ_Q4_1>), g, wg, 0, s, src, src_row_stride, (int)t, (int)nblk, d_pos, pos_off, src_at_pos ? 1 : 0, (uint32_t)cap, codes, scales); break;
+        case FHIP_KVQ_Q8_0: hipLaunchKernelGGL((kvq_quant_kernel<FHIP_KVQ_Q8_0>), g, wg, 0, s, tg, src_row_stride, (int)t, (int)nblk, d_pos, pos_off, at, (uint32_t)cap); break;
+        case FHIP_KVQ_Q4_0: hipLaunchKernelGGL((kvq_quant_kernel<FHIP_KVQ_Q4_0>), g, wg, 0, s, tg, src_row_stride, (int)t, (int)nblk, d_pos, pos_off, at, (uint32_t)cap); break;
+        case FHIP_KVQ_Q4_1: hipLaunchKernelGGL((kvq_quant_kernel<FHIP_KVQ_Q4_1>), g, wg, 0, s, tg, src_row_stride, (int)t, (int)nblk, d_pos, pos_off, at, (uint32_t)cap); break;
         default: return set_error(FHIP_ERR_ARG, "kvq_append: unknown format %d", fmt);
     }
     return check_hip(hipGetLastError(), "kvq_append launch");

@@ -134,6 +134,28 @@ def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, 
     return out
 
 
+def decode_attention_kvq(q, kcache, vcache, n_heads, n_kv_heads, length=None, last_pos=None, ws=None, stream=None, window=0, softcap=0.0):
+    """decode_attention over a pair of block-quantized caches (kvquant.QKvCache) read in place -- the quantized arm of
+    qwen3.rs:906-924 without the dequantized copy of the history."""
+    assert len(q.shape) == 2 and q.shape[0] == 1, "decode_attention takes one query row"
+    dh = q.shape[1] // n_heads
+    length = kcache.len if length is None else length
+    assert kcache.fmt == vcache.fmt and kcache.width == vcache.width == n_kv_heads * dh
+    assert 1 <= length <= min(kcache.cap, vcache.cap), f"decode_attention: length {length} outside the caches"
+    lib = _lib.load()
+    need = lib.fhip_decode_attention_ws_bytes(n_heads, n_kv_heads, dh, length)
+    own = None
+    if need and ws is None:
+        own = ws = DeviceBuffer(need)
+    out = Tensor.empty((1, n_heads * dh))
+    _check(lib.fhip_decode_attention_kvq(kcache.fmt, q.buf.ptr, kcache.codes.ptr, kcache.scales.ptr, vcache.codes.ptr, vcache.scales.ptr,
+                                         n_heads, n_kv_heads, dh, length, last_pos.buf.ptr if last_pos is not None else None, window, softcap,
+                                         ws.ptr if ws is not None else None, out.buf.ptr, _stream_handle(stream)))
+    if own is not None:
+        _check(lib.fhip_stream_sync(_stream_handle(stream)))   # the scratch is freed on return
+    return out
+
+
 class Qwen3Cfg:
     """The fields of the reference's Cfg this path reads (qwen3.rs:60-100: n_head, n_head_kv, head_dim, eps, rope pairing,
     attn_softcap, post_norm_eps; geglu stands for is_gemma's FFN activation, qwen3.rs:953)."""
@@ -172,17 +194,26 @@ class Qwen3Decoder:
     (also what None, the default, means) the q/k norm + rope + cache append happen inside the attention launch, 6 launches per layer.
     A gated layer adds two launches (the gate's mat-vec on the same normed input, the sigmoid product), post-norms two (the
     RMSNorm of each branch output; the add happens inside the next mat-vec as before), GEGLU one (the activation on its own).
+    kv_fmt: the caches are block-quantized (kvquant.QKvCache pairs of fixed capacity): the token's K and V rows are quantized by
+    one launch and attention reads the blocks in place, 8 launches per layer; no f32 copy of the history exists.
     """
 
-    def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None, fuse_norm=True, fuse_attn=None):
+    def __init__(self, cfg, layers, max_len, stream=None, output_norm=None, lm_head=None, fuse_norm=True, fuse_attn=None, kv_fmt=None):
         self.cfg, self.layers, self.max_len, self.stream, self.fuse_norm = cfg, layers, int(max_len), stream, bool(fuse_norm)
         self.fuse_attn = fuse_attn
+        self.kv_fmt = kv_fmt                              # None: f32 caches; else kvquant.Q8_0 / Q4_0 / Q4_1 (Cache::with_kvq, qwen3.rs:303)
         self.output_norm, self.lm_head = output_norm, lm_head          # final norm + LM head: hidden -> logits in the same step
         assert (output_norm is None) == (lm_head is None), "output_norm and lm_head come together"
         self.logits = Tensor.empty((1, lm_head.rows())) if lm_head is not None else None
         c = cfg
         self.q_out, self.kv_out = c.n_head * c.head_dim, c.n_head_kv * c.head_dim
-        self.caches = [KvCache(max_len, self.kv_out) for _ in layers]
+        if kv_fmt is None:
+            self.caches = [KvCache(max_len, self.kv_out) for _ in layers]
+        else:
+            from .kvquant import QKvCache
+            self.caches = [(QKvCache(kv_fmt, max_len, self.kv_out), QKvCache(kv_fmt, max_len, self.kv_out)) for _ in layers]
+            self.k1, self.v1 = Tensor.empty((1, self.kv_out)), Tensor.empty((1, self.kv_out))     # the new token's rows before they are stored
+            fuse_attn = self.fuse_attn = False            # the rows are quantized by a launch of their own
         self.pos = _u32_tensor([0])                       # device word: the position of the token being decoded
         self.xa = Tensor.empty((1, c.d_model))            # residual stream: the step's input is written here ...
         self.xb = Tensor.empty((1, c.d_model))            # ... and the residual alternates between the two buffers
@@ -207,7 +238,7 @@ class Qwen3Decoder:
             # of its own up to 2048 keys (5.12 -> 5.06 ms/token there, 4.92 -> 4.84 at 128) and is level with it from 4096 on.
             self.fuse_attn = True
         self.fuse_attn = bool(self.fuse_attn)
-        self.launches_per_layer = (7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0)   # a default-arm layer
+        self.launches_per_layer = (7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0) + (1 if kv_fmt is not None else 0)   # a default-arm layer
         self._graph = None
 
     # -- state ------------------------------------------------------------------------------------
@@ -215,8 +246,11 @@ class Qwen3Decoder:
         a = np.array([pos], np.uint32)
         _check(_lib.load().fhip_memcpy_h2d(self.pos.buf.ptr, _vp(a), 4, _stream_handle(self.stream)))
         _check(_lib.load().fhip_stream_sync(_stream_handle(self.stream)))
-        for c in self.caches:
+        for c in self._all_caches():
             c.len = pos
+
+    def _all_caches(self):
+        return self.caches if self.kv_fmt is None else [c for pair in self.caches for c in pair]
 
     def set_input(self, x_host):
         a = np.ascontiguousarray(x_host, dtype=np.float32).reshape(-1)
@@ -260,7 +294,17 @@ class Qwen3Decoder:
             qn = l.q_norm.buf.ptr if l.q_norm is not None else None
             kn = l.k_norm.buf.ptr if l.k_norm is not None else None
             ws = self.ws.ptr if self.ws is not None else None
-            if self.fuse_attn:
+            if self.kv_fmt is not None:
+                # the quantized arm (qwen3.rs:906-912): post-process, store the token's rows as blocks, attend over the blocks
+                kq, vq = kv
+                _check(lib.fhip_qkv_post_packed(self.qkv.buf.ptr, bias, qn, kn, self.pos.buf.ptr, None, 1, c.n_head, c.n_head_kv, c.head_dim, n_rot,
+                                                int(c.rope_interleaved), c.eps, base, self.q.buf.ptr, self.k1.buf.ptr, self.v1.buf.ptr, s))
+                _check(lib.fhip_kvq_append2(self.kv_fmt, self.k1.buf.ptr, self.v1.buf.ptr, 0, 1, self.kv_out, self.pos.buf.ptr, 0, kq.cap,
+                                            kq.codes.ptr, kq.scales.ptr, vq.codes.ptr, vq.scales.ptr, s))
+                _check(lib.fhip_decode_attention_kvq(self.kv_fmt, self.q.buf.ptr, kq.codes.ptr, kq.scales.ptr, vq.codes.ptr, vq.scales.ptr, c.n_head,
+                                                     c.n_head_kv, c.head_dim, self.max_len, self.pos.buf.ptr, l.window, c.attn_softcap, ws,
+                                                     self.att.buf.ptr, s))
+            elif self.fuse_attn:
                 _check(lib.fhip_qkv_post_attention(self.qkv.buf.ptr, bias, qn, kn, self.pos.buf.ptr, None, c.n_head, c.n_head_kv, c.head_dim,
                                                    n_rot, int(c.rope_interleaved), c.eps, base, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap,
                                                    self.max_len, l.window, c.attn_softcap, ws, self.att.buf.ptr, s))
@@ -297,7 +341,7 @@ class Qwen3Decoder:
     def step(self):
         """Eager: enqueue one step and account for the appended row."""
         self._enqueue_step()
-        for c in self.caches:
+        for c in self._all_caches():
             c.len += 1
 
     def capture(self):
@@ -310,7 +354,7 @@ class Qwen3Decoder:
 
     def step_graph(self):
         self._graph.launch()
-        for c in self.caches:
+        for c in self._all_caches():
             c.len += 1
 
     def hidden(self):

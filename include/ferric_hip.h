@@ -301,6 +301,26 @@ int fhip_kvq_append(int fmt, const float* d_src, size_t src_row_stride, size_t t
 int fhip_kvq_dequantize_rows(int fmt, const uint32_t* d_codes, const uint32_t* d_scales, size_t row0, size_t rows, size_t width,
                              const uint32_t* d_last_pos, float* d_out, void* stream);
 
+/* K and V rows of the same tokens into their two caches in one launch (the quantized twin of fhip_kv_append2; the
+ * reference appends them apart, crates/ferric-llama/src/qwen3.rs:909-910). Both sources share the row stride. */
+int fhip_kvq_append2(int fmt, const float* d_k, const float* d_v, size_t src_row_stride, size_t t, size_t width, const uint32_t* d_positions,
+                     uint32_t pos_off, size_t cap, uint32_t* d_k_codes, uint32_t* d_k_scales, uint32_t* d_v_codes, uint32_t* d_v_scales,
+                     void* stream);
+/* fhip_decode_attention_ex over a block-quantized cache read in place: each key / value row is dequantized in registers as it
+ * is loaded (the use the reference chose the block layout for and left unbuilt, kvquant.rs:30-37, qwen3.rs:897-905: it
+ * materialises `dequantize()` of the whole history per layer and step and attends over that). The values that enter the
+ * softmax are exactly fhip_kvq_dequantize_rows', so the result has the bits of fhip_decode_attention_ex over the dequantized
+ * rows, at 8.5 / 4.5 / 5 bits per value of traffic instead of 32 + 32 written and read back. */
+int fhip_decode_attention_kvq(int fmt, const float* d_q, const uint32_t* d_k_codes, const uint32_t* d_k_scales, const uint32_t* d_v_codes,
+                              const uint32_t* d_v_scales, size_t n_head, size_t n_kv, size_t head_dim, size_t len, const uint32_t* d_last_pos,
+                              size_t window, float softcap, float* d_ws, float* d_out, void* stream);
+
+/* fhip_qkv_post with the key and value heads written to packed outputs [t, n_kv * head_dim] (row i for token i) instead of
+ * cache rows: for callers that store them themselves, as the quantized arm of qwen3.rs:906-912 does. */
+int fhip_qkv_post_packed(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_positions,
+                         const float* d_freq_scale, size_t t, size_t n_head, size_t n_kv, size_t head_dim, size_t n_rot, int interleaved,
+                         float eps, float base, float* d_q_out, float* d_k_out, float* d_v_out, void* stream);
+
 /* crates/ferric-tensor/src/nn.rs:140 decode_attention -> lib.rs:762 fused_decode_attention (kernels :2675, :2740 ff.):
  * one query row q [n_head * head_dim] against the cache rows [0, len) of K and V [., n_kv * head_dim];
  * out[h] = softmax_j(q_h . K[j, h / g] / sqrt(head_dim)) @ V[:, h / g], g = n_head / n_kv (1..=8), head_dim 64 or 128.

@@ -132,13 +132,20 @@ def apply_layer(x, l, kc, vc, pos, cfg):
     """qwen3.rs:979-1047 for one token at position pos; kc / vc are lists of earlier K / V rows (appended to). The default
     arm (:1041-1047) unless the layer or the configuration carries one of: a sliding window and a score softcap (:917-924),
     no rotation (:857-863: QK-norm still applies), its own rope base, a sigmoid gate on the attention output projected from
-    the normed input (:936-938), post-norms on both branch outputs with their own epsilon (:1015-1020), GEGLU (:953-958)."""
+    the normed input (:936-938), post-norms on both branch outputs with their own epsilon (:1015-1020), GEGLU (:953-958), a
+    block-quantized cache (cfg.kv_fmt, :906-912)."""
     opt = lambda o, name, default: getattr(o, name, default) if getattr(o, name, None) is not None else default
     h = rmsnorm(x, l.attn_norm, cfg.eps)
     qkv = h @ l.wqkv.T
     n_rot = cfg.head_dim if opt(l, "rope", True) else 0
     q, k, v = qkv_post(qkv.reshape(1, -1), getattr(l, "qkv_bias", None), getattr(l, "q_norm", None), getattr(l, "k_norm", None), [pos],
                        cfg.n_head, cfg.n_head_kv, cfg.head_dim, cfg.eps, opt(l, "rope_base", cfg.rope_base), cfg.rope_interleaved, n_rot)
+    kv_fmt = getattr(cfg, "kv_fmt", None)
+    if kv_fmt is not None:
+        # the quantized arm (:906-912): the rows are stored as blocks and attention reads what dequantize() gives back
+        from . import kvquant_oracle as KQ
+        k = KQ.roundtrip(k.astype(np.float32), 1, k.shape[1], kv_fmt).astype(np.float64)
+        v = KQ.roundtrip(v.astype(np.float32), 1, v.shape[1], kv_fmt).astype(np.float64)
     kc.append(k[0]); vc.append(v[0])
     a = decode_attention(q[0], np.stack(kc), np.stack(vc), cfg.n_head, cfg.n_head_kv, opt(l, "window", 0), opt(cfg, "attn_softcap", 0.0))
     if getattr(l, "attn_gate", None) is not None:

@@ -525,3 +525,53 @@ def test_decoder_arms_match_the_oracle_and_replay_as_a_graph(F, X, O, D, name, a
         dec.set_input(xs[pos])
         dec.step_graph()
         assert np.array_equal(bits(dec.hidden()), bits(eager[pos])), (name, pos)
+
+
+@pytest.mark.parametrize("kv_fmt,arms,cfg_kw", [(0, [set()] * 3, {}), (1, [set()] * 3, {}), (2, [set()] * 3, {}),
+                                                (0, [{"gate", "post", "window"}, {"gate", "post", "nope"}, {"post", "base"}],
+                                                 dict(POST, geglu=True, attn_softcap=50.0))])
+def test_decoder_on_a_block_quantized_cache(F, X, O, D, kv_fmt, arms, cfg_kw, precision):
+    """The quantized arm of the layer (qwen3.rs:906-912): K and V rows stored as Q8_0 / Q4_0 / Q4_1 blocks, attention over what
+    they dequantize to. The oracle quantizes its own f64 rows (rounded to f32) the same way. Same bar as the f32 cache; and the
+    quantized cache is live: what the device cache dequantizes to is the oracle's dequantized rows (the hidden state itself
+    moves by less than the bar between an f32 and a quantized cache on this model, so it cannot tell)."""
+    n_layer, d, nh, nkv, hd, n_ff, steps = 3, 1024, 8, 2, 128, 1536, 6
+    cfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6, **cfg_kw)
+    ocfg = X.Qwen3Cfg(d, nh, nkv, hd, n_ff, eps=1e-6, rope_base=1e6, **cfg_kw)
+    ocfg.kv_fmt = kv_fmt
+    layers, olayers = _arm_model(F, X, O, np.random.default_rng(8), n_layer, d, nh, nkv, hd, n_ff, arms)
+    xs = (np.random.default_rng(9).standard_normal((steps, d)) * 0.5).astype(np.float32)
+
+    def oracle_steps(c):
+        kcs, vcs = [[] for _ in olayers], [[] for _ in olayers]
+        out = []
+        for pos in range(steps):
+            x = xs[pos].astype(np.float64)
+            for l, kc, vc in zip(olayers, kcs, vcs):
+                x = D.apply_layer(x, l, kc, vc, pos, c)
+            out.append(x)
+        return out, kcs
+    want, kcs = oracle_steps(ocfg)
+    bar = dot_bar(20)
+    stream = F.Stream()
+    dec = X.Qwen3Decoder(cfg, layers, max_len=steps + 2, stream=stream, kv_fmt=kv_fmt)
+    eager = []
+    for pos in range(steps):
+        dec.set_input(xs[pos])
+        dec.step()
+        eager.append(dec.hidden())
+        assert close(eager[-1], want[pos], bar), (kv_fmt, pos)
+    # the first layer's key cache against the oracle's dequantized rows: the same blocks up to codes that sat near a rounding
+    # boundary (what is quantized differs between the mat-vec kernel and the f64 oracle by up to the dot-product bar, a few
+    # per cent of a Q8_0 step): never more than one step off, and few of them off at all
+    got = dec.caches[0][0].dequantize(stream).to_vec(stream).reshape(steps, nkv * hd)
+    ref = np.stack(kcs[0])
+    step = np.abs(ref).reshape(steps, -1, 32).max(axis=2) / (127 if kv_fmt == 0 else 7)
+    off = np.abs(got - ref).reshape(steps, -1, 32)
+    assert (off <= 1.01 * step[:, :, None] + 1e-6).all() and (off > 1e-4 * step[:, :, None] + 1e-6).mean() < 0.1
+    dec.set_pos(0)
+    dec.capture()
+    for pos in range(steps):
+        dec.set_input(xs[pos])
+        dec.step_graph()
+        assert np.array_equal(bits(dec.hidden()), bits(eager[pos])), (kv_fmt, pos)

@@ -169,3 +169,65 @@ def test_positions_on_the_device_and_argument_checks(F, Q, K):
         assert lib.fhip_kvq_sizes(f, 7, 96, C.byref(cw), C.byref(sw)) == 0 and (cw.value, sw.value) == K.sizes(7, 96, f)
     with pytest.raises(AssertionError, match="past len"):
         cache.dequantize_rows(0, 1)
+
+
+@pytest.mark.parametrize("fmt", [0, 1, 2])
+def test_attention_over_the_blocks_is_attention_over_the_dequantized_rows(F, Q, K, fmt):
+    """fhip_decode_attention_kvq dequantizes rows in registers by the dequantize kernel's own operations, so its output has the
+    bits of fhip_decode_attention_ex over dequantize(); and it is the oracle's attention over the oracle's dequantized rows to the
+    f32 attention's tolerance (1e-5 of the largest output)."""
+    from types import SimpleNamespace
+    from ferric_amd import decode as X
+    from oracle import decode_oracle as D
+    rng = np.random.default_rng(70 + fmt)
+    # (heads, kv heads, head dim, rows, window, softcap): one split and many, both head sizes, every group size class, a
+    # length that leaves the last split ragged, a window, a softcap
+    cases = [(8, 2, 128, 7, 0, 0.0), (40, 8, 128, 300, 0, 0.0), (8, 8, 64, 129, 0, 0.0), (6, 2, 64, 1000, 0, 0.0), (16, 2, 128, 2100, 512, 0.0),
+             (5, 1, 128, 260, 0, 30.0), (14, 2, 64, 33, 8, 50.0)]
+    for nh, nkv, hd, rows, window, cap in cases:
+        width = nkv * hd
+        k = (rng.standard_normal((rows, width)) * 2).astype(np.float32)
+        v = (rng.standard_t(3, (rows, width))).astype(np.float32)
+        q = rng.standard_normal((1, nh * hd)).astype(np.float32)
+        kq = Q.QKvCache.from_tensor(F.Tensor.from_vec(k, k.shape), fmt)
+        vq = Q.QKvCache.from_tensor(F.Tensor.from_vec(v, v.shape), fmt)
+        qt = F.Tensor.from_vec(q, q.shape)
+        got = X.decode_attention_kvq(qt, kq, vq, nh, nkv, window=window, softcap=cap).to_vec()
+        plain = SimpleNamespace(k=kq.dequantize(), v=vq.dequantize(), cap=rows, width=width, len=rows)
+        same = X.decode_attention(qt, plain, nh, nkv, window=window, softcap=cap).to_vec()
+        assert np.array_equal(bits(got), bits(same)), (nh, nkv, hd, rows)
+        want = D.decode_attention(q[0], K.roundtrip(k, rows, width, fmt), K.roundtrip(v, rows, width, fmt), nh, nkv, window, cap)
+        assert np.abs(got - want.reshape(-1)).max() <= 1e-5 * np.abs(want).max(), (nh, nkv, hd, rows)
+        # a shorter length, and the length read from a device word (what a captured step does)
+        n = max(1, rows // 3)
+        word = F.Tensor(F.DeviceBuffer(4), (1,), np.uint32)
+        last = np.array([n - 1], np.uint32)
+        F._lib.check(F._lib.load().fhip_memcpy_h2d(word.buf.ptr, last.ctypes.data, 4, None))
+        a = X.decode_attention_kvq(qt, kq, vq, nh, nkv, length=n, window=window, softcap=cap).to_vec()
+        b = X.decode_attention_kvq(qt, kq, vq, nh, nkv, length=rows, last_pos=word, window=window, softcap=cap).to_vec()
+        want = D.decode_attention(q[0], K.roundtrip(k[:n], n, width, fmt), K.roundtrip(v[:n], n, width, fmt), nh, nkv, window, cap).reshape(-1)
+        assert np.abs(a - want).max() <= 1e-5 * np.abs(want).max() and np.abs(b - want).max() <= 1e-5 * np.abs(want).max()
+    lib = F._lib.load()
+    assert lib.fhip_decode_attention_kvq(fmt, qt.buf.ptr, kq.codes.ptr, kq.scales.ptr, vq.codes.ptr, vq.scales.ptr, 14, 2, 48, 5, None, 0, 0.0, None,
+                                         qt.buf.ptr, None) != 0                      # 2 x 48 is a multiple of 32, the head size is not one the kernel takes
+    assert b"head_dim must be 64 or 128" in lib.fhip_last_error()
+
+
+def test_k_and_v_rows_stored_by_one_launch(F, Q, K):
+    rng = np.random.default_rng(80)
+    t, width, cap = 5, 256, 16
+    k, v = rng.standard_normal((t, width)).astype(np.float32), (rng.standard_normal((t, width)) * 7).astype(np.float32)
+    lib = F._lib.load()
+    for fmt in (0, 1, 2):
+        kq, vq = Q.QKvCache(fmt, cap, width), Q.QKvCache(fmt, cap, width)
+        pos = F.Tensor(F.DeviceBuffer(4 * t), (t,), np.uint32)
+        where = np.array([3, 0, 9, 15, 4], np.uint32)
+        F._lib.check(lib.fhip_memcpy_h2d(pos.buf.ptr, where.ctypes.data, 4 * t, None))
+        kt, vt = F.Tensor.from_vec(k, k.shape), F.Tensor.from_vec(v, v.shape)
+        F._lib.check(lib.fhip_kvq_append2(fmt, kt.buf.ptr, vt.buf.ptr, 0, t, width, pos.buf.ptr, 0, cap, kq.codes.ptr, kq.scales.ptr, vq.codes.ptr,
+                                          vq.scales.ptr, None))
+        kq.len = vq.len = cap
+        for cache, x in ((kq, k), (vq, v)):
+            got = cache.dequantize().to_vec().reshape(cap, width)
+            for i, r in enumerate(where):
+                assert np.array_equal(bits(got[r]), bits(K.roundtrip(x[i], 1, width, fmt)[0])), (fmt, i)
