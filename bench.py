@@ -653,6 +653,42 @@ def probe_decode(F, lib, check):
     check(lib.fhip_stream_sync(None))
 
 
+def probe_kvq(F, lib, check):
+    """Work for a kernel trace of attention over a long cache: 40 query / 8 KV heads x 128 at 32768 cached rows, four launches
+    each on four f32 caches (268 MB of rows per launch) and on four caches of every block format (71 / 38 / 42 MB), every
+    cache read for the first time by its launch; then one token's K and V rows appended to a quantized cache four times."""
+    from ferric_amd import decode as X
+    from ferric_amd import kvquant as Q
+    nh, nkv, hd, rows = 40, 8, 128, 32768
+    rng = np.random.default_rng(3)
+    fill = (rng.standard_normal((rows, nkv * hd)) * 0.5).astype(np.float32)
+    ft = F.Tensor.from_vec(fill, fill.shape)
+    q = F.Tensor.from_vec(rng.standard_normal(nh * hd).astype(np.float32), (1, nh * hd))
+    plain = []
+    for _ in range(4):
+        c = X.KvCache(rows, nkv * hd)
+        check(lib.fhip_memcpy_d2d(c.k.buf.ptr, ft.buf.ptr, fill.nbytes, None))
+        check(lib.fhip_memcpy_d2d(c.v.buf.ptr, ft.buf.ptr, fill.nbytes, None))
+        c.len = rows
+        plain.append(c)
+    packed = {fmt: [(Q.QKvCache.from_tensor(ft, fmt), Q.QKvCache.from_tensor(ft, fmt)) for _ in range(4)] for fmt in Q.ALL}
+    check(lib.fhip_stream_sync(None))
+    scrub_src, scrub_dst = F.DeviceBuffer(512 << 20), F.DeviceBuffer(512 << 20)
+    check(lib.fhip_memcpy_d2d(scrub_dst.ptr, scrub_src.ptr, 512 << 20, None))      # pushes what was just written out of the cache levels
+    check(lib.fhip_stream_sync(None))
+    for c in plain:
+        X.decode_attention(q, c, nh, nkv)
+    for fmt in Q.ALL:
+        for kq, vq in packed[fmt]:
+            X.decode_attention_kvq(q, kq, vq, nh, nkv)
+    row = F.Tensor.from_vec(fill[:1], (1, nkv * hd))
+    kq, vq = Q.QKvCache(Q.Q8_0, 64, nkv * hd), Q.QKvCache(Q.Q8_0, 64, nkv * hd)
+    for i in range(4):
+        check(lib.fhip_kvq_append2(Q.Q8_0, row.buf.ptr, row.buf.ptr, 0, 1, nkv * hd, None, i, 64, kq.codes.ptr, kq.scales.ptr, vq.codes.ptr,
+                                   vq.scales.ptr, None))
+    check(lib.fhip_stream_sync(None))
+
+
 def cpu_baseline(rows, cols, x_seed, budget_s=12.0):
     """The reference's CPU route for Q4_K (deq_raw then a sequential f32 dot per row, rows split in
     contiguous spans over threads), timed through the C oracle on this host's cores."""
@@ -699,6 +735,7 @@ def main():
                     help="counter probe for rocprofv3 --pmc: one 256 MiB device copy (calibration), then 16 cold Q4_K 5120x5120 "
                          "GEMVs, one fused gate|up 34816x5120 and one Q6_K 5120x17408 GEMV; prints nothing else")
     ap.add_argument("--probe-step", action="store_true", help="three eager decode steps at context 128 and 4096 (for a kernel trace)")
+    ap.add_argument("--probe-kvq", action="store_true", help="attention at 32768 rows on f32 and block-quantized caches (for a kernel trace)")
     ap.add_argument("--probe-decode", action="store_true",
                     help="profiler probe for the decode attention kernel: 8 launches each at 4096 and 128 cached rows; prints nothing else")
     ap.add_argument("--probe-prefill", action="store_true",
@@ -727,6 +764,9 @@ def main():
         return
     if args.probe_prefill:
         probe_prefill(F, lib, check)
+        return
+    if args.probe_kvq:
+        probe_kvq(F, lib, check)
         return
     if args.probe_decode:
         probe_decode(F, lib, check)

@@ -277,17 +277,41 @@ struct QCache {
 // DPL (4 or 8) consecutive dims of one row, starting at column `col` (a multiple of DPL) of block row `key`: the values the
 // dequantize kernel would write, by the same single operations (q * d; (q - 8) * d; q * d then + m, not fused), so attention
 // over the codes is attention over the dequantized rows, bit for bit.
+// What a lane holds of a row between the load and its use: the code words and scale halves as loaded (the next rows are
+// requested while the current ones are worked on, and packed they cost a third of the registers of their f32 values).
 template <int FMT, int DPL>
-__device__ __forceinline__ void load_dims_q(const uint32_t* __restrict__ codes, const uint16_t* __restrict__ scales, size_t key, int nblk, int col,
-                                            float (&r)[DPL]) {
-#pragma clang fp contract(off)
+struct RawDims {
+    uint32_t w[DPL / 4];
+    uint16_t d, m;
+};
+template <int FMT, int DPL>
+__device__ __forceinline__ RawDims<FMT, DPL> fetch_dims_q(const uint32_t* __restrict__ codes, const uint16_t* __restrict__ scales, size_t key,
+                                                         int nblk, int col) {
     const size_t b = key * (size_t)nblk + (size_t)(col >> 5);
     const int j = col & 31;
+    RawDims<FMT, DPL> r;
+    r.m = 0;
     if constexpr (FMT == FHIP_KVQ_Q8_0) {
-        const float d = __half2float(__ushort_as_half(scales[b]));
+        r.d = scales[b];
+#pragma unroll
+        for (int w = 0; w < DPL / 4; w++) r.w[w] = codes[b * 8 + (j >> 2) + w];
+    } else {
+        if constexpr (FMT == FHIP_KVQ_Q4_0) r.d = scales[b];
+        else { r.d = scales[2 * b]; r.m = scales[2 * b + 1]; }
+#pragma unroll
+        for (int w = 0; w < DPL / 4; w++) r.w[w] = codes[b * 4 + ((j & 15) >> 2) + w];
+    }
+    return r;
+}
+template <int FMT, int DPL>
+__device__ __forceinline__ void expand_dims_q(const RawDims<FMT, DPL>& raw, int col, float (&r)[DPL]) {
+#pragma clang fp contract(off)
+    const int j = col & 31;
+    if constexpr (FMT == FHIP_KVQ_Q8_0) {
+        const float d = __half2float(__ushort_as_half(raw.d));
 #pragma unroll
         for (int w = 0; w < DPL / 4; w++) {
-            const uint32_t word = codes[b * 8 + (j >> 2) + w];
+            const uint32_t word = raw.w[w];
             r[4 * w] = (float)(int8_t)(word & 255u) * d;
             r[4 * w + 1] = (float)(int8_t)((word >> 8) & 255u) * d;
             r[4 * w + 2] = (float)(int8_t)((word >> 16) & 255u) * d;
@@ -295,12 +319,10 @@ __device__ __forceinline__ void load_dims_q(const uint32_t* __restrict__ codes, 
         }
     } else {
         const int shift = j < 16 ? 0 : 4;
-        float d, m = 0.f;
-        if constexpr (FMT == FHIP_KVQ_Q4_0) d = __half2float(__ushort_as_half(scales[b]));
-        else { d = __half2float(__ushort_as_half(scales[2 * b])); m = __half2float(__ushort_as_half(scales[2 * b + 1])); }
+        const float d = __half2float(__ushort_as_half(raw.d)), m = __half2float(__ushort_as_half(raw.m));
 #pragma unroll
         for (int w = 0; w < DPL / 4; w++) {
-            const uint32_t word = codes[b * 4 + ((j & 15) >> 2) + w] >> shift;
+            const uint32_t word = raw.w[w] >> shift;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const float n = (float)((word >> (8 * i)) & 15u);
@@ -418,19 +440,40 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
 #pragma unroll
         for (int i = 0; i < DPL; i++) acc[h][i] = 0.f;
     }
+    // The rows of a step are requested one step ahead: a stream's steps depend on one another only through the running
+    // maximum, so without this every step paid a memory round trip before its arithmetic (32 in a row for a split of 1024 keys).
+    // A step past the split's end re-reads the split's last row (always a row of the cache) and is never used.
+    constexpr int QFMT = QF >= 0 ? QF : 0;
+    const int qcol = kvh * HD + sub * DPL, qnblk = n_kv * (HD / 32);
+    RawDims<QFMT, DPL> kq[QF >= 0 ? ATT_KB : 1], vq[QF >= 0 ? ATT_KB : 1];
+    float kf[QF >= 0 ? 1 : ATT_KB][DPL], vf[QF >= 0 ? 1 : ATT_KB][DPL];
+    auto request = [&](uint32_t at) {
+#pragma unroll
+        for (int j = 0; j < ATT_KB; j++) {
+            const uint32_t key = min(at + j, k1 - 1);   // a row past the split re-reads its last row and is masked below
+            if constexpr (QF >= 0) {
+                kq[j] = fetch_dims_q<QFMT, DPL>(qc.k_codes, qc.k_scales, key, qnblk, qcol);
+                vq[j] = fetch_dims_q<QFMT, DPL>(qc.v_codes, qc.v_scales, key, qnblk, qcol);
+            } else {
+                load_dims<DPL>(Kb + key * stride, kf[j]);
+                load_dims<DPL>(Vb + key * stride, vf[j]);
+            }
+        }
+    };
+    request(k0 + sid * ATT_KB);
     for (uint32_t kb = k0 + sid * ATT_KB; kb < k1; kb += ATT_STREAMS * ATT_KB) {
         float kr[ATT_KB][DPL], vr[ATT_KB][DPL];
 #pragma unroll
         for (int j = 0; j < ATT_KB; j++) {
-            const uint32_t key = min(kb + j, k1 - 1);   // a row past the split re-reads its last row and is masked below
             if constexpr (QF >= 0) {
-                load_dims_q<QF, DPL>(qc.k_codes, qc.k_scales, key, n_kv * (HD / 32), kvh * HD + sub * DPL, kr[j]);
-                load_dims_q<QF, DPL>(qc.v_codes, qc.v_scales, key, n_kv * (HD / 32), kvh * HD + sub * DPL, vr[j]);
+                expand_dims_q<QFMT, DPL>(kq[j], qcol, kr[j]);
+                expand_dims_q<QFMT, DPL>(vq[j], qcol, vr[j]);
             } else {
-                load_dims<DPL>(Kb + key * stride, kr[j]);
-                load_dims<DPL>(Vb + key * stride, vr[j]);
+#pragma unroll
+                for (int i = 0; i < DPL; i++) { kr[j][i] = kf[j][i]; vr[j][i] = vf[j][i]; }
             }
         }
+        request(kb + ATT_STREAMS * ATT_KB);
 #pragma unroll
         for (int h = 0; h < G; h++) {
             float sc[ATT_KB];
