@@ -528,6 +528,29 @@ def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
     return res
 
 
+def bench_prefill_attention(F, lib, check, stream, timer, reps=5):
+    """Causal attention of a prompt block (fhip_causal_attention, f32 matrix instructions): 40 query / 8 KV heads x 128, T rows
+    against a cache of S rows. FLOPs = 4 * head_dim * n_head * (query, key) pairs inside the causal mask."""
+    nh, nkv, hd = 40, 8, 128
+    rng = np.random.default_rng(1)
+    out = {}
+    for t, s in ((512, 512), (2048, 2048), (4096, 4096), (512, 8192)):
+        q = F.Tensor.from_vec(rng.standard_normal((t, nh * hd)).astype(np.float32), (t, nh * hd))
+        k = F.Tensor.from_vec(rng.standard_normal((s, nkv * hd)).astype(np.float32), (s, nkv * hd))
+        v = F.Tensor.from_vec(rng.standard_normal((s, nkv * hd)).astype(np.float32), (s, nkv * hd))
+        o = F.Tensor.empty((t, nh * hd))
+        g = F.Graph.begin(stream)
+        for _ in range(reps):
+            check(lib.fhip_causal_attention(q.buf.ptr, k.buf.ptr, v.buf.ptr, t, s, nh, nkv, hd, 0, 0.0, o.buf.ptr, stream.handle))
+        g.end()
+        g.launch()
+        ms = timer.time_ms(g.launch) / reps
+        pairs = t * (s - t) + t * (t + 1) / 2
+        tf = 4.0 * pairs * nh * hd / (ms * 1e-3) / 1e12
+        out[f"{t}x{s}"] = {"ms": ms, "TFLOPs": tf, "frac_of_f32_mfma_peak": tf / 157.3}
+    return out
+
+
 def probe(F, lib, check):
     """Work for a profiler run (kernel trace or hardware counters) of the mat-vec kernels, launched eagerly on the null stream:
     a copy of known size first (it calibrates FETCH_SIZE / WRITE_SIZE), then every weight shape of the decode sweep and the
@@ -653,6 +676,21 @@ def probe_decode(F, lib, check):
     check(lib.fhip_stream_sync(None))
 
 
+def probe_prefill_attn(F, lib, check):
+    """Work for a profiler run on the causal attention kernel: 40 query / 8 KV heads x 128, five launches each at 2048 rows
+    against 2048 (a stateless prefill), at 512 against 512 and at 512 against a cache of 8192 (a chunk of a long prompt)."""
+    from ferric_amd import decode as X
+    nh, nkv, hd = 40, 8, 128
+    rng = np.random.default_rng(1)
+    for t, s in ((2048, 2048), (512, 512), (512, 8192)):
+        q = F.Tensor.from_vec(rng.standard_normal((t, nh * hd)).astype(np.float32), (t, nh * hd))
+        k = F.Tensor.from_vec(rng.standard_normal((s, nkv * hd)).astype(np.float32), (s, nkv * hd))
+        v = F.Tensor.from_vec(rng.standard_normal((s, nkv * hd)).astype(np.float32), (s, nkv * hd))
+        for _ in range(5):
+            X.causal_attention(q, k, v, nh, nkv)
+    check(lib.fhip_stream_sync(None))
+
+
 def probe_kvq(F, lib, check):
     """Work for a kernel trace of attention over a long cache: 40 query / 8 KV heads x 128 at 32768 cached rows, four launches
     each on four f32 caches (268 MB of rows per launch) and on four caches of every block format (71 / 38 / 42 MB), every
@@ -735,6 +773,7 @@ def main():
                     help="counter probe for rocprofv3 --pmc: one 256 MiB device copy (calibration), then 16 cold Q4_K 5120x5120 "
                          "GEMVs, one fused gate|up 34816x5120 and one Q6_K 5120x17408 GEMV; prints nothing else")
     ap.add_argument("--probe-step", action="store_true", help="three eager decode steps at context 128 and 4096 (for a kernel trace)")
+    ap.add_argument("--probe-prefill-attn", action="store_true", help="causal attention at 2048 / 512 rows (for a profiler run)")
     ap.add_argument("--probe-kvq", action="store_true", help="attention at 32768 rows on f32 and block-quantized caches (for a kernel trace)")
     ap.add_argument("--probe-decode", action="store_true",
                     help="profiler probe for the decode attention kernel: 8 launches each at 4096 and 128 cached rows; prints nothing else")
@@ -767,6 +806,9 @@ def main():
         return
     if args.probe_kvq:
         probe_kvq(F, lib, check)
+        return
+    if args.probe_prefill_attn:
+        probe_prefill_attn(F, lib, check)
         return
     if args.probe_decode:
         probe_decode(F, lib, check)
@@ -819,6 +861,7 @@ def main():
     if not args.no_prefill:
         log("[bench] prefill dequant-GEMM, T = 128/512/2048 ...")
         line["prefill_q4k_bf16_mfma"] = bench_prefill(F, lib, check, stream, timer)
+        line["prefill_causal_attention_f32_mfma"] = bench_prefill_attention(F, lib, check, stream, timer)
     if not args.no_moe:
         log("[bench] routed-expert block of an MoE decode layer ...")
         line["moe_routed_experts_q4k_q6k"] = bench_moe(F, lib, check, stream, timer)

@@ -93,6 +93,7 @@ SYMBOLS = {
     "fhip_mul_sigmoid": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
     "fhip_kvq_sizes": (C.c_int, [C.c_int, _sz, _sz, C.POINTER(_sz), C.POINTER(_sz)]),
     "fhip_kvq_append": (C.c_int, [C.c_int, _vp, _sz, _sz, _sz, _vp, C.c_uint32, C.c_int, _sz, _vp, _vp, _vp]),
+    "fhip_causal_attention": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_float, _vp, _vp]),
     "fhip_kvq_append2": (C.c_int, [C.c_int, _vp, _vp, _sz, _sz, _sz, _vp, C.c_uint32, _sz, _vp, _vp, _vp, _vp, _vp]),
     "fhip_decode_attention_kvq": (C.c_int, [C.c_int, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, C.c_float, _vp, _vp, _vp]),
     "fhip_qkv_post_packed": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_int, C.c_float, C.c_float, _vp, _vp, _vp, _vp]),

@@ -30,6 +30,7 @@ UNITS = {
     "moe.hip": [],
     "probe.hip": [],
     "decode_ops.hip": [],
+    "prefill_attn.hip": [],
     "gguf.hip": [],
 }
 

@@ -850,6 +850,18 @@ int fhip_decode_attention_kvq(int fmt, const float* d_q, const uint32_t* d_k_cod
                                              (int)n_kv, (int)head_dim, len, d_last_pos, window, softcap, d_ws, d_out, (hipStream_t)stream);
 }
 
+int fhip_causal_attention(const float* d_q, const float* d_k, const float* d_v, size_t t, size_t s, size_t n_head, size_t n_kv, size_t head_dim,
+                          size_t window, float softcap, float* d_out, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (t == 0 || n_head == 0 || head_dim == 0) return FHIP_OK;
+    if (!d_q || !d_k || !d_v || !d_out) return set_error(FHIP_ERR_ARG, "fhip_causal_attention: NULL pointer");
+    if ((((uintptr_t)d_q | (uintptr_t)d_k | (uintptr_t)d_v | (uintptr_t)d_out) & 15) != 0)
+        return set_error(FHIP_ERR_ARG, "fhip_causal_attention: pointers must be 16-byte aligned");
+    if (n_head > 0x7FFFFFFFull || n_kv > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "fhip_causal_attention: too many heads");
+    return fhip::launch_causal_attention(d_q, d_k, d_v, t, s, (int)n_head, (int)n_kv, (int)head_dim, window, softcap, d_out, (hipStream_t)stream);
+}
+
 size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_dim, size_t len) {
     if (g_device < 0 || n_kv == 0 || len == 0) return 0;
     int splits = fhip::attn_splits(len, (int)n_kv);

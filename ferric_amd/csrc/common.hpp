@@ -141,6 +141,8 @@ int launch_decode_attention_kvq(int fmt, const float* q, const uint32_t* k_codes
                                 float softcap, float* ws, float* out, hipStream_t s);
 int launch_kvq_dequantize(int fmt, const uint32_t* codes, const uint16_t* scales, size_t row0, size_t rows, size_t width, const uint32_t* d_last_pos,
                           float* out, hipStream_t s);
+int launch_causal_attention(const float* q, const float* K, const float* V, size_t t, size_t s, int n_head, int n_kv, int hd, size_t window,
+                            float softcap, float* out, hipStream_t st);
 int launch_mul_sigmoid(const float* a, const float* g, size_t n, float* out, hipStream_t s);   // out = a * sigmoid(g); out may be a
 int launch_geglu(const float* gu, size_t t, size_t d, float* out, hipStream_t s);              // rows [gate | up] -> gelu_tanh(gate) * up
 int launch_rope(const float* x, size_t src_row_stride, size_t t, int heads, int hd, int n_rot, float base, const uint32_t* d_pos, uint32_t pos_off,

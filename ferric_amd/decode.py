@@ -134,6 +134,18 @@ def decode_attention(q, cache, n_heads, n_kv_heads, length=None, last_pos=None, 
     return out
 
 
+def causal_attention(q, k, v, n_heads, n_kv_heads, window=0, softcap=0.0, stream=None):
+    """nn.rs:40 causal_attention / :66 causal_attention_win / :239 chunked_attention: q [t, n_heads * dh] against k, v
+    [s, n_kv_heads * dh] with s >= t; query i at position s - t + i."""
+    t, s = q.shape[0], k.shape[0]
+    assert s >= t, f"cache ({s}) cannot be shorter than the query block ({t})"
+    assert k.shape == v.shape and k.shape[1] * n_heads == q.shape[1] * n_kv_heads
+    out = Tensor.empty(q.shape)
+    _check(_lib.load().fhip_causal_attention(q.buf.ptr, k.buf.ptr, v.buf.ptr, t, s, n_heads, n_kv_heads, q.shape[1] // n_heads, window, softcap,
+                                             out.buf.ptr, _stream_handle(stream)))
+    return out
+
+
 def decode_attention_kvq(q, kcache, vcache, n_heads, n_kv_heads, length=None, last_pos=None, ws=None, stream=None, window=0, softcap=0.0):
     """decode_attention over a pair of block-quantized caches (kvquant.QKvCache) read in place -- the quantized arm of
     qwen3.rs:906-924 without the dequantized copy of the history."""

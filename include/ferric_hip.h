@@ -315,6 +315,16 @@ int fhip_decode_attention_kvq(int fmt, const float* d_q, const uint32_t* d_k_cod
                               const uint32_t* d_v_scales, size_t n_head, size_t n_kv, size_t head_dim, size_t len, const uint32_t* d_last_pos,
                               size_t window, float softcap, float* d_ws, float* d_out, void* stream);
 
+/* Causal attention of t query rows q [t, n_head * head_dim] against the first s >= t rows of K and V [., n_kv * head_dim]:
+ * query i sits at absolute position (s - t) + i and attends to keys 0 ..= (s - t) + i, or only to the newest `window` of them
+ * when window > 0; softcap > 0 replaces each scaled score x by softcap * tanh(x / softcap). One entry point for
+ * crates/ferric-tensor/src/nn.rs:40 causal_attention (s == t), :66 causal_attention_win, :239 chunked_attention (prefix-cached
+ * and chunked prefill) and the flash prefill kernel crates/ferric-llama/src/qwen3.rs:925 picks when it can -- "all three are
+ * the same math". s < t -> FHIP_ERR_SHAPE with the reference's message (nn.rs:73). head_dim 64 or 128; f32 throughout (f32
+ * matrix instructions), out [t, n_head * head_dim]; pointers 16-byte aligned. */
+int fhip_causal_attention(const float* d_q, const float* d_k, const float* d_v, size_t t, size_t s, size_t n_head, size_t n_kv, size_t head_dim,
+                          size_t window, float softcap, float* d_out, void* stream);
+
 /* fhip_qkv_post with the key and value heads written to packed outputs [t, n_kv * head_dim] (row i for token i) instead of
  * cache rows: for callers that store them themselves, as the quantized arm of qwen3.rs:906-912 does. */
 int fhip_qkv_post_packed(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_positions,

@@ -79,6 +79,18 @@ def decode_attention(q, k, v, n_heads, n_kv_heads, window=0, softcap=0.0):
     return out.reshape(1, n_heads * dh)
 
 
+def causal_attention(q, k, v, n_heads, n_kv_heads, window=0, softcap=0.0):
+    """nn.rs:40-57, :66-88, :239-265: q [t, n_heads * dh] against k, v [s, n_kv_heads * dh], s >= t; query i sits at position
+    off + i, off = s - t, sees keys 0 ..= off + i and, with a window, only those with (off + i) - j < window (:128-133): row by
+    row the single-query attention over the keys up to the row's position."""
+    q = np.asarray(q, np.float64)
+    t, s = q.shape[0], np.asarray(k).shape[0]
+    assert s >= t
+    off = s - t
+    return np.concatenate([decode_attention(q[i], np.asarray(k)[:off + i + 1], np.asarray(v)[:off + i + 1], n_heads, n_kv_heads, window, softcap)
+                           for i in range(t)], axis=0)
+
+
 def qkv_post(qkv, bias, q_norm, k_norm, positions, n_head, n_kv, hd, eps, base, interleaved=False, n_rot=None, freq_scale=None):
     """crates/ferric-llama/src/qwen3.rs:848-905: + bias, per-head RMSNorm of q and k (when the norms exist), rope of both at
     the rows' positions; returns (q [t, n_head*hd], k [t, n_kv*hd], v [t, n_kv*hd])."""

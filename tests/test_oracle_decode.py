@@ -263,3 +263,31 @@ def test_the_other_arms_of_apply_layer_by_their_invariants():
     gu = D.rmsnorm(xy, l.ffn_norm, 1e-6) @ l.gate_up.T
     act = torch.nn.functional.gelu(torch.from_numpy(gu[:12]), approximate="tanh").numpy() * gu[12:]
     assert np.allclose(yg, xy + act @ l.down.T, rtol=1e-12)
+
+
+def test_causal_attention_against_the_masked_matrix_form():
+    """The reference's own formulation (nn.rs:40-57, :66-88, :239-265): all scores at once, an additive mask of -1e30 where
+    j > off + i or (off + i) - j >= window, softmax over the keys, times V -- against the row-by-row oracle."""
+    rng = np.random.default_rng(12)
+    for t, s, nh, nkv, dh, window, cap in [(5, 5, 4, 2, 8, 0, 0.0), (7, 19, 6, 2, 4, 0, 0.0), (9, 9, 2, 2, 8, 3, 0.0), (6, 14, 4, 1, 8, 5, 20.0),
+                                           (1, 11, 4, 2, 8, 0, 0.0)]:
+        q, k, v = rng.standard_normal((t, nh * dh)), rng.standard_normal((s, nkv * dh)), rng.standard_normal((s, nkv * dh))
+        got = D.causal_attention(q, k, v, nh, nkv, window, cap)
+        off, g = s - t, nh // nkv
+        qh = q.reshape(t, nh, dh).transpose(1, 0, 2)
+        kh = np.repeat(k.reshape(s, nkv, dh).transpose(1, 0, 2), g, axis=0)
+        vh = np.repeat(v.reshape(s, nkv, dh).transpose(1, 0, 2), g, axis=0)
+        sc = qh @ kh.transpose(0, 2, 1) * float(np.float32(1.0) / np.sqrt(np.float32(dh)))
+        if cap > 0:
+            sc = cap * np.tanh(sc / cap)
+        ii, jj = np.arange(t)[:, None] + off, np.arange(s)[None, :]
+        mask = np.where((jj > ii) | ((window > 0) & (ii - jj >= window)), -1e30, 0.0)
+        sc = sc + mask
+        p = np.exp(sc - sc.max(axis=2, keepdims=True))
+        want = ((p / p.sum(axis=2, keepdims=True)) @ vh).transpose(1, 0, 2).reshape(t, nh * dh)
+        assert np.allclose(got, want, rtol=1e-12, atol=1e-14), (t, s)
+    # one query row against the whole cache is the decode op; the first row of a stateless prefill returns its own value row
+    q, k, v = rng.standard_normal((1, 32)), rng.standard_normal((6, 16)), rng.standard_normal((6, 16))
+    assert np.array_equal(D.causal_attention(q, k, v, 4, 2), D.decode_attention(q[0], k, v, 4, 2))
+    q = rng.standard_normal((6, 32))
+    assert np.allclose(D.causal_attention(q, k, v, 4, 2)[0].reshape(4, 8), np.repeat(v[0].reshape(2, 8), 2, axis=0), rtol=1e-14)
