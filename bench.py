@@ -473,6 +473,22 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
     out[f"{ctx}_q8_0_cache"] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * dec.launches_per_layer + 2,
                                 "kv_bytes_read": kv_bytes, "logits_finite": bool(np.isfinite(logits).all())}
     del dec
+    # the same stack on a block of prompt rows: projections on the bf16 matrix cores, causal attention on the f32 ones
+    from ferric_amd import decode as X
+    import time
+    pre = {}
+    for t in (512, 2048):
+        dec = X.Qwen3Decoder(cfg, lay, max_len=t + 1, stream=stream)
+        xs = (rng.standard_normal((t, cfg.d_model)) * 0.5).astype(np.float32)
+        dec.prefill(xs[:64])                      # warm-up (first-use costs), then from an empty cache again
+        dec.set_pos(0)
+        check(lib.fhip_stream_sync(stream.handle))
+        t0 = time.perf_counter()
+        hid = dec.prefill(xs)                     # returns after the device has finished (it downloads the hidden rows)
+        ms = (time.perf_counter() - t0) * 1e3
+        pre[str(t)] = {"ms": ms, "tokens_per_s": t / (ms * 1e-3), "hidden_finite": bool(np.isfinite(hid).all())}
+        del dec
+    out["prefill_block"] = pre
     out["weight_bytes"] = weight_bytes_total
     out["model"] = "64 layers, d 5120, 40 query / 8 KV heads x 128, n_ff 17408, vocab 151936; Q4_K projections, Q6_K down and lm_head; f32 KV cache (the _q8_0_cache entry: Q8_0 blocks)"
     return out

@@ -350,6 +350,99 @@ class Qwen3Decoder:
         self.x = cur
         _check(lib.fhip_u32_add(self.pos.buf.ptr, 1, 1, s))
 
+    # -- a block of prompt rows -------------------------------------------------------------------
+    def prefill(self, x_host, precise=False):
+        """`forward_cached` for t > 1 rows (qwen3.rs:979-1052 with the attention arms of :917-930): hidden rows x [t, d_model] at
+        the positions behind what the caches hold; appends their K and V rows, leaves the position word behind them and returns
+        the rows' final hidden states [t, d_model] (host). Eager, with buffers of its own. The projections run on the bf16
+        matrix cores (fhip_matmul_q_coop / fhip_ffn_coop, the reference's coop route for prompt rows, dtype.rs:1818); precise=True
+        takes fhip_matmul_q / fhip_ffn instead, whose results have the f32 grade of the decode step. Attention is
+        fhip_causal_attention over the cache; on a quantized cache the rows are stored as blocks first and attention reads
+        what they dequantize to, as the reference does (qwen3.rs:906-912)."""
+        lib, c, s = _lib.load(), self.cfg, _stream_handle(self.stream)
+        x = np.ascontiguousarray(x_host, dtype=np.float32).reshape(-1, c.d_model)
+        t = x.shape[0]
+        pos0 = self._all_caches()[0].len
+        assert pos0 + t <= self.max_len, f"prefill: {pos0} + {t} rows exceed the capacity {self.max_len}"
+        E = Tensor.empty
+        X = Tensor.from_vec(x, x.shape, self.stream)
+        positions = _u32_tensor(np.arange(pos0, pos0 + t))
+        h, qkv, q, att = E((t, c.d_model)), E((t, self.q_out + 2 * self.kv_out)), E((t, self.q_out)), E((t, self.q_out))
+        o, x1, y = E((t, c.d_model)), E((t, c.d_model)), E((t, c.d_model))
+        normed = E((t, c.d_model)) if self.on is not None else None                   # a post-normed branch output
+        f, gu = E((t, c.n_ff)), (E((t, 2 * c.n_ff)) if c.geglu else None)
+        gate = E((t, self.q_out)) if self.gate is not None else None
+        ws16 = DeviceBuffer(2 * t * max(c.d_model, self.q_out, c.n_ff) + 256)          # bf16 copies of the coop matmuls' inputs
+        k1 = v1 = kd = vd = None
+        if self.kv_fmt is not None:
+            k1, v1 = E((t, self.kv_out)), E((t, self.kv_out))
+            kd, vd = E((pos0 + t, self.kv_out)), E((pos0 + t, self.kv_out))          # what the stored blocks dequantize to
+        wsf = [None]
+
+        def matmul(w, a, out):
+            if precise:
+                _check(lib.fhip_matmul_q(w.handle, a.buf.ptr, t, out.buf.ptr, s))
+            else:
+                _check(lib.fhip_matmul_q_coop(w.handle, a.buf.ptr, t, out.buf.ptr, ws16.ptr, s))
+
+        def ffn(l, a, out):
+            if c.geglu:
+                matmul(l.ffn_gate_up, a, gu)
+                _check(lib.fhip_geglu(gu.buf.ptr, t, c.n_ff, f.buf.ptr, s))
+                matmul(l.ffn_down, f, out)
+            elif precise:
+                _check(lib.fhip_ffn(l.ffn_gate_up.handle, l.ffn_down.handle, a.buf.ptr, t, out.buf.ptr, f.buf.ptr, s))
+            else:
+                need = lib.fhip_ffn_coop_ws_bytes(l.ffn_gate_up.handle, l.ffn_down.handle, t)
+                if wsf[0] is None or wsf[0].nbytes < need:
+                    wsf[0] = DeviceBuffer(max(need, 256))
+                _check(lib.fhip_ffn_coop(l.ffn_gate_up.handle, l.ffn_down.handle, a.buf.ptr, t, out.buf.ptr, wsf[0].ptr, s))
+
+        for l, kv in zip(self.layers, self.caches):
+            _check(lib.fhip_rmsnorm(X.buf.ptr, l.attn_norm.buf.ptr, t, c.d_model, c.eps, h.buf.ptr, s))
+            matmul(l.wqkv, h, qkv)
+            bias = l.qkv_bias.buf.ptr if l.qkv_bias is not None else None
+            qn = l.q_norm.buf.ptr if l.q_norm is not None else None
+            kn = l.k_norm.buf.ptr if l.k_norm is not None else None
+            n_rot = c.head_dim if l.rope else 0
+            base = c.rope_base if l.rope_base is None else float(l.rope_base)
+            if self.kv_fmt is None:
+                _check(lib.fhip_qkv_post(qkv.buf.ptr, bias, qn, kn, positions.buf.ptr, None, t, c.n_head, c.n_head_kv, c.head_dim, n_rot,
+                                         int(c.rope_interleaved), c.eps, base, q.buf.ptr, kv.k.buf.ptr, kv.v.buf.ptr, kv.cap, s))
+                kp, vp = kv.k.buf.ptr, kv.v.buf.ptr
+            else:
+                kq, vq = kv
+                _check(lib.fhip_qkv_post_packed(qkv.buf.ptr, bias, qn, kn, positions.buf.ptr, None, t, c.n_head, c.n_head_kv, c.head_dim, n_rot,
+                                                int(c.rope_interleaved), c.eps, base, q.buf.ptr, k1.buf.ptr, v1.buf.ptr, s))
+                _check(lib.fhip_kvq_append2(self.kv_fmt, k1.buf.ptr, v1.buf.ptr, 0, t, self.kv_out, positions.buf.ptr, 0, kq.cap, kq.codes.ptr,
+                                            kq.scales.ptr, vq.codes.ptr, vq.scales.ptr, s))
+                for cache, dst in ((kq, kd), (vq, vd)):
+                    _check(lib.fhip_kvq_dequantize_rows(self.kv_fmt, cache.codes.ptr, cache.scales.ptr, 0, pos0 + t, self.kv_out, None,
+                                                        dst.buf.ptr, s))
+                kp, vp = kd.buf.ptr, vd.buf.ptr
+            _check(lib.fhip_causal_attention(q.buf.ptr, kp, vp, t, pos0 + t, c.n_head, c.n_head_kv, c.head_dim, l.window, c.attn_softcap,
+                                             att.buf.ptr, s))
+            if l.attn_gate is not None:
+                matmul(l.attn_gate, h, gate)
+                _check(lib.fhip_mul_sigmoid(att.buf.ptr, gate.buf.ptr, t * self.q_out, att.buf.ptr, s))
+            matmul(l.wo, att, o)
+            branch = o
+            if l.post_attn_norm is not None:
+                _check(lib.fhip_rmsnorm(o.buf.ptr, l.post_attn_norm.buf.ptr, t, c.d_model, c.post_norm_eps, normed.buf.ptr, s))
+                branch = normed
+            _check(lib.fhip_add_rmsnorm(X.buf.ptr, branch.buf.ptr, l.ffn_norm.buf.ptr, t, c.d_model, c.eps, x1.buf.ptr, h.buf.ptr, s))
+            ffn(l, h, y)
+            branch = y
+            if l.post_ffn_norm is not None:
+                _check(lib.fhip_rmsnorm(y.buf.ptr, l.post_ffn_norm.buf.ptr, t, c.d_model, c.post_norm_eps, normed.buf.ptr, s))
+                branch = normed
+            _check(lib.fhip_add(x1.buf.ptr, branch.buf.ptr, t * c.d_model, X.buf.ptr, s))
+        _check(lib.fhip_u32_add(self.pos.buf.ptr, 1, t, s))
+        out = X.to_vec(self.stream).reshape(t, c.d_model)      # synchronises: the temporaries may go
+        for cache in self._all_caches():
+            cache.len += t
+        return out
+
     def step(self):
         """Eager: enqueue one step and account for the appended row."""
         self._enqueue_step()
