@@ -1120,13 +1120,33 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     // pipeline fill and drain), so the rows are dealt out in as few rounds as possible: one workgroup per
     // CU with up to RPG_MAX rows per row group, more rounds of equal size only beyond that. With a
     // partly filled single round the row groups are spread over all CUs.
-    constexpr int RPG_MAX = 256;
+    int RPG_MAX = 256;
     int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     if (p.sel.npairs > 1) cus = cus / p.sel.npairs > 0 ? cus / p.sel.npairs : 1;   // the pairs of an "_id" launch share the chip
     int Gcap = MAXW / WPR;
     if (Gcap < 1) Gcap = 1;
+    // Fewer waves per CU for the launches that live off the memory system's queue depth rather than off latency hiding.
+    // About 10 MB in flight fill this device's HBM pipe (6.5 TB/s times ~1.5 us), 40 KB per CU; 15 waves with two rows each
+    // hold 90 - 100 KB, and what is queued beyond the pipe's depth only reaches the DRAM pages in a worse order. Measured on
+    // cold weights, one activation row: Q6_K is fastest with 5 - 7 waves per workgroup at every size (5120 columns, 5120 /
+    // 20480 / 151936 rows: 8.65 -> 7.83, 19.7 -> 18.5, 118.5 -> 107.0 us; 128256 x 4096: 82.1 -> 73.7 us with six row groups),
+    // Q4_K with 8 - 10 waves once the weight has 28 MB or more (20480 x 5120 13.9 -> 12.6 us, fused gate|up 34816 x 5120
+    // 20.9 -> 20.2, 28672 x 4096 15.3 -> 14.6) and with all 15 - 16 below that (5120 x 5120: 5.95 us against 6.39).
+    if (M == 1 && p.sel.npairs <= 1) {
+        int want = Gcap;
+        if (F::TYPE == FHIP_Q6_K) want = 6 / WPR;
+        else if (F::TYPE == FHIP_Q4_K && (size_t)w->rows * w->row_bytes >= ((size_t)28 << 20)) want = ((WPR == 1 ? 8 : 10) + WPR - 1) / WPR;
+        if (want < 1) want = 1;
+        // the fused norm holds one 8-value piece of the row per thread
+        if (norm) { const int need = (int)((w->cols + (size_t)512 * WPR - 1) / ((size_t)512 * WPR)); if (want < need) want = need; }
+        if (want < Gcap) {
+            Gcap = want;
+            // one round for up to 1024 rows per row group where the partial sums still fit beside the staged row
+            if (lds_bytes<F, M, SWIGLU>(w->cols, p.NG, Gcap, 1024) + 512 <= fhip::device_lds_bytes()) RPG_MAX = 1024;
+        }
+    }
     const size_t slots = (size_t)cus * Gcap;
-    const size_t rounds = (out_rows + slots * RPG_MAX - 1) / (slots * RPG_MAX);
+    const size_t rounds = (out_rows + slots * (size_t)RPG_MAX - 1) / (slots * (size_t)RPG_MAX);
     int rpg = (int)((out_rows + slots * rounds - 1) / (slots * rounds));
     if (rpg < 1) rpg = 1;
     const size_t nrg = (out_rows + rpg - 1) / rpg;

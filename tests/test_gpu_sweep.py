@@ -14,8 +14,8 @@ import pytest
 from conftest import bits, dot_bar
 
 pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("precision")]
-Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q5_K: (256, 176), Q6_K: (256, 210)}
 
 
 def row_bytes(ty, cols):
@@ -63,10 +63,12 @@ def test_vocabulary_head_151936_x_5120_q6_k(F, O):
         assert np.array_equal(bits(xt.matmul_q(part).to_vec()), bits(y[r0:r0 + n])), r0
 
 
-@pytest.mark.parametrize("ty,cols,period", [(Q4_K, 5120, 4096), (Q8_0, 1024, 3000)])
+@pytest.mark.parametrize("ty,cols,period", [(Q4_K, 5120, 4096), (Q5_K, 5120, 4096), (Q8_0, 1024, 3000)])
 def test_more_rows_than_one_round_of_workgroups(F, O, ty, cols, period):
     """A vocabulary of 262144 rows (the Gemma-class callers of the same matmul_q, crates/ferric-llama/src/gemma4.rs:274-280)
-    is more than one workgroup per CU takes at 256 rows per row group: the launch goes over the rows in several rounds. The
+    is more than one workgroup per CU takes at 256 rows per row group: the launch goes over the rows in several rounds (Q5_K:
+    two rounds of three row groups per workgroup; Q4_K, with two row groups per workgroup for a weight this large, takes up
+    to 1024 rows per row group and stays at one round; Q8_0 rows this short fill one round of sixteen row groups). The
     weight repeats a block of `period` random rows, so every output has an oracle value and equal rows must give equal bits."""
     from ferric_amd.synth import synth_weights
     rows = 262144
