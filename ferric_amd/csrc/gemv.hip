@@ -723,7 +723,7 @@ __device__ __forceinline__ void quantize8(const float (&v)[8], uint32_t (&pl)[NP
     sum_out = scale * (float)qsum;
 }
 
-template <class F, int M, int U, bool SWIGLU, bool NORM>
+template <class F, int M, int U, bool SWIGLU, bool NORM, bool LATE>
 __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     fhip::apply_selection(p);
@@ -892,10 +892,17 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     for (int e = e0 + (XR + 1) * e_step; e < M * p.cols; e += e_step)      // rows beyond four passes
         stage(e, *(const float4*)(p.x + e), *(const float4*)(p.x + e + 4));
     if (!fused_norm && stager) __builtin_amdgcn_s_setprio(0);
-    // the rest of the prefetch: in flight while the workgroup meets at the barrier and copies its planes out of LDS
+    // The rest of the prefetch. Early: in flight while the workgroup meets at the barrier and copies its planes out of LDS
+    // (rows so long that the staging takes several passes, and the large weights, whose row loop should find its pipeline
+    // full). Late, behind the barrier: what is requested in front of the barrier stands in the memory pipe in front of the
+    // younger workgroups' activation loads, and a small weight is all latency: with one row per wave there instead of two
+    // the staged activations are ready sooner and the launch ends sooner (Q4_K 5120 x 5120 5.96 -> 5.53 us, 7168 x 5120
+    // 7.20 -> 6.96, Q6_K 5120 x 5120 7.84 -> 7.08 on cold weights; no row at all in front of the barrier: 6.59).
+    if constexpr (!LATE) {
 #pragma unroll
-    for (int j = 1; j < U; j++)
-        if (j < n_it) buf[j] = fetch(j);
+        for (int j = 1; j < U; j++)
+            if (j < n_it) buf[j] = fetch(j);
+    }
     __syncthreads();
 
     // The row scale the staged activations went without, for the threads that will write outputs: worked out here, under
@@ -966,6 +973,11 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams 
     // explicitly gives the compiler's wait-count tracking a clean state at the loop head; without it the
     // merge of the prologue's load order with the loop's makes every iteration wait for vmcnt(0).
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt/lgkmcnt untouched
+    if constexpr (LATE) {
+#pragma unroll
+        for (int j = 1; j < U; j++)
+            if (j < n_it) buf[j] = fetch(j);
+    }
 #pragma unroll 1
     for (; i0 + 2 * U <= n_full; i0 += U) {      // every row of this step and of the next one exists
 #pragma unroll
@@ -1095,16 +1107,13 @@ template <class F, int M, bool SWIGLU>
 int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr,
                const fhip::NormParams* norm = nullptr) {
     constexpr int U = rows_in_flight<F>(M);
-    void (*kernel)(GemvParams) = gemv_stream_kernel<F, M, U, SWIGLU, false>;
-    if constexpr (M == 1) {
-        if (norm) kernel = gemv_stream_kernel<F, M, U, SWIGLU, true>;
-    }
-    static bool lds_raised[2] = {false, false};
-    if (!lds_raised[norm ? 1 : 0]) {  // workgroups may use more than the default 64 KiB of the CU's 160 KiB
-        (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fhip::device_lds_bytes());
-        (void)hipGetLastError();
-        lds_raised[norm ? 1 : 0] = true;
-    }
+    // The prefetch of a wave's later rows waits behind the staging barrier for the small weights of the two formats the
+    // decode layers are made of (see the kernel); measured level or worse elsewhere: rows of 14336 columns and more, whose
+    // staging takes several passes (Q6_K 5120 x 17408 16.7 -> 17.3 us), and Q4_K from 28 MB on (10240 x 5120 8.13 -> 8.30).
+    constexpr bool HAS_LATE = M == 1 && U > 1 && (F::TYPE == FHIP_Q4_K || F::TYPE == FHIP_Q6_K);
+    const size_t wbytes = (size_t)w->rows * w->row_bytes;
+    const bool small = wbytes < ((size_t)28 << 20);
+    bool late = HAS_LATE && !sel && w->cols <= 8192 && (F::TYPE == FHIP_Q6_K || small);
     GemvParams p;
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
@@ -1131,11 +1140,13 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     // cold weights, one activation row: Q6_K is fastest with 5 - 7 waves per workgroup at every size (5120 columns, 5120 /
     // 20480 / 151936 rows: 8.65 -> 7.83, 19.7 -> 18.5, 118.5 -> 107.0 us; 128256 x 4096: 82.1 -> 73.7 us with six row groups),
     // Q4_K with 8 - 10 waves once the weight has 28 MB or more (20480 x 5120 13.9 -> 12.6 us, fused gate|up 34816 x 5120
-    // 20.9 -> 20.2, 28672 x 4096 15.3 -> 14.6) and with all 15 - 16 below that (5120 x 5120: 5.95 us against 6.39).
+    // 20.9 -> 20.2, 28672 x 4096 15.3 -> 14.6) and with all 15 - 16 below that (5120 x 5120: 5.95 us against 6.39). A small
+    // Q6_K weight whose later rows are requested behind the barrier keeps all its waves (5120 x 5120: 7.08 us against 7.98;
+    // twelve of the sixteen one-wave row groups of 4096 columns: 4096 x 4096 5.49 us against 5.98).
     if (M == 1 && p.sel.npairs <= 1) {
         int want = Gcap;
-        if (F::TYPE == FHIP_Q6_K) want = 6 / WPR;
-        else if (F::TYPE == FHIP_Q4_K && (size_t)w->rows * w->row_bytes >= ((size_t)28 << 20)) want = ((WPR == 1 ? 8 : 10) + WPR - 1) / WPR;
+        if (F::TYPE == FHIP_Q6_K) want = late && small ? (WPR == 1 ? 12 : Gcap) : 6 / WPR;
+        else if (F::TYPE == FHIP_Q4_K && !small) want = ((WPR == 1 ? 8 : 10) + WPR - 1) / WPR;
         if (want < 1) want = 1;
         // the fused norm holds one 8-value piece of the row per thread
         if (norm) { const int need = (int)((w->cols + (size_t)512 * WPR - 1) / ((size_t)512 * WPR)); if (want < need) want = need; }
@@ -1162,6 +1173,24 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
         if (rr_rpg <= (size_t)RPG_MAX) { p.rr = 1; p.nrg = (int)nrg_all; p.kfull = (int)kfull; p.rem = (int)rem; rpg = (int)rr_rpg; }
     }
     p.G = G; p.rpg = rpg;
+    // With one row per wave there is no later row to hold back and the two kernels do the same work; which of the two
+    // compilations is the faster one then was measured per format (Q4_K 4096 x 4096: 4.71 us early, 4.82 late; Q6_K
+    // 4096 x 4096: 6.38 early, 5.49 late).
+    if (F::TYPE != FHIP_Q6_K && rpg * (SWIGLU ? 2 : 1) <= p.RF) late = false;
+    void (*kernel)(GemvParams) = gemv_stream_kernel<F, M, U, SWIGLU, false, false>;
+    if constexpr (M == 1) {
+        if (norm) kernel = gemv_stream_kernel<F, M, U, SWIGLU, true, false>;
+    }
+    if constexpr (HAS_LATE) {
+        if (late) kernel = norm ? gemv_stream_kernel<F, M, U, SWIGLU, true, true> : gemv_stream_kernel<F, M, U, SWIGLU, false, true>;
+    }
+    static bool lds_raised[4] = {false, false, false, false};
+    const int variant = (norm ? 1 : 0) + (late ? 2 : 0);
+    if (!lds_raised[variant]) {  // workgroups may use more than the default 64 KiB of the CU's 160 KiB
+        (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)fhip::device_lds_bytes());
+        (void)hipGetLastError();
+        lds_raised[variant] = true;
+    }
     auto magic = [](int d) { return d > 1 ? (uint32_t)(((1ull << 32) + (unsigned)d - 1) / (unsigned)d) : 0u; };
     p.m_wpr = magic(WPR); p.m_ngf = magic(p.NG >> 2); p.m_rf = magic(p.RF); p.m_rpg = magic(rpg);
     const size_t per_wg = (size_t)G * rpg;
