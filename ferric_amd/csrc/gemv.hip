@@ -299,7 +299,7 @@ struct Q6K {
 
 struct Q80 {
     static constexpr uint32_t TYPE = FHIP_Q8_0;
-    static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 2;   // two rows in flight: 4096 x 4096 6.89 -> 6.57 us against four
     static constexpr bool RR = true;      // round-robin row dealing of large weights
     struct Lane { uint32_t off; };
     struct Data {
@@ -1107,10 +1107,11 @@ template <class F, int M, bool SWIGLU>
 int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr,
                const fhip::NormParams* norm = nullptr) {
     constexpr int U = rows_in_flight<F>(M);
-    // The prefetch of a wave's later rows waits behind the staging barrier for the small weights of the two formats the
-    // decode layers are made of (see the kernel); measured level or worse elsewhere: rows of 14336 columns and more, whose
-    // staging takes several passes (Q6_K 5120 x 17408 16.7 -> 17.3 us), and Q4_K from 28 MB on (10240 x 5120 8.13 -> 8.30).
-    constexpr bool HAS_LATE = M == 1 && U > 1 && (F::TYPE == FHIP_Q4_K || F::TYPE == FHIP_Q6_K);
+    // The prefetch of a wave's later rows waits behind the staging barrier for the small weights of the formats the
+    // decode layers are made of (see the kernel; also Q5_K 5120 x 5120 7.20 -> 6.47 us, Q8_0 4096 x 4096 6.78 -> 6.57);
+    // measured level or worse elsewhere: rows of 14336 columns and more, whose staging takes several passes (Q6_K
+    // 5120 x 17408 16.7 -> 17.3 us), Q4_K from 28 MB on (10240 x 5120 8.13 -> 8.30), the other 32-value formats.
+    constexpr bool HAS_LATE = M == 1 && U > 1 && (F::TYPE == FHIP_Q4_K || F::TYPE == FHIP_Q6_K || F::TYPE == FHIP_Q5_K || F::TYPE == FHIP_Q8_0);
     const size_t wbytes = (size_t)w->rows * w->row_bytes;
     const bool small = wbytes < ((size_t)28 << 20);
     bool late = HAS_LATE && !sel && w->cols <= 8192 && (F::TYPE == FHIP_Q6_K || small);
