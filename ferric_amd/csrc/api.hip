@@ -17,7 +17,7 @@ namespace {
 // current device's copy and keeps it per device.
 constexpr size_t WEIGHT_SLACK = 256;   // readable bytes every weight has behind its last block
 constexpr size_t NOALLOC_FLOATS = 131072;
-__device__ __align__(256) float scratch[NOALLOC_FLOATS];
+static __device__ __align__(256) float scratch[NOALLOC_FLOATS];
 constexpr int MAX_DEVICES = 64;
 float* g_scratch_ptr[MAX_DEVICES] = {};
 

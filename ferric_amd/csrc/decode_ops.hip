@@ -346,7 +346,7 @@ template <int G, int DPL, bool FUSED, int QF = -1>
 __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typename CachePtr<FUSED>::type K, typename CachePtr<FUSED>::type V,
                                                 int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
                                                 uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out,
-                                                const QkvPostParams& fp, const QCache& qc = QCache{}) {
+                                                const QkvPostParams& fp, int gq, const QCache& qc = QCache{}) {
     static_assert(!(FUSED && QF >= 0), "the fused post-processing appends f32 rows");
     constexpr int HD = 16 * DPL;
     __shared__ float sm_m[4][G], sm_l[4][G];
@@ -354,7 +354,9 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
     __shared__ float sm_q[FUSED ? G : 1][FUSED ? HD : 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane & 15;
     const int sid = wave * 4 + (lane >> 4);
-    const int kvh = blockIdx.x, split = blockIdx.y;
+    // Workgroup blockIdx.x takes the G query heads from head0 on; gq = query heads per KV head. gq == G: one workgroup per KV
+    // head and split. gq > G (short caches, G = 1): one workgroup per query head, the KV head's rows read by each of them.
+    const int head0 = blockIdx.x * G, kvh = head0 / gq, split = blockIdx.y;
     // FUSED: the raw values of every head this wave will post-process (job j = wave + 4 r: query head j of the group, then
     // the key and the value row) are requested before anything else, the length word with them, so that one memory round
     // trip covers what used to be three in a row (the length, the first round's rows, the second round's).
@@ -365,7 +367,7 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
         for (int r = 0; r < ROUNDS; r++) {
             const int j = wave + 4 * r;
             if (j < G + 2) {
-                const int src = j < G ? kvh * G + j : (j == G ? fp.n_head + kvh : fp.n_head + n_kv + kvh);
+                const int src = j < G ? head0 + j : (j == G ? fp.n_head + kvh : fp.n_head + n_kv + kvh);
                 const float* x = fp.qkv + (size_t)src * HD;
                 const float* bias = fp.bias ? fp.bias + (size_t)src * HD : nullptr;
 #pragma unroll
@@ -395,7 +397,7 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
         for (int r = 0; r < ROUNDS; r++) {                 // job j < G: query head j of the group; G: the K row; G + 1: the V row
             const int j = wave + 4 * r;
             if (j >= njobs) continue;
-            const int src = j < G ? kvh * G + j : (j == G ? fp.n_head + kvh : fp.n_head + n_kv + kvh);
+            const int src = j < G ? head0 + j : (j == G ? fp.n_head + kvh : fp.n_head + n_kv + kvh);
             const float* x = fp.qkv + (size_t)src * HD;
             const float* bias = fp.bias ? fp.bias + (size_t)src * HD : nullptr;
             const float* nw = j < G ? fp.q_norm : (j == G ? fp.k_norm : nullptr);
@@ -435,7 +437,7 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
 #pragma unroll
             for (int i = 0; i < DPL; i++) qr[h][i] = sm_q[FUSED ? h : 0][sub * DPL + i];
         } else {
-            load_dims<DPL>(q + ((size_t)kvh * G + h) * HD + sub * DPL, qr[h]);
+            load_dims<DPL>(q + ((size_t)head0 + h) * HD + sub * DPL, qr[h]);
         }
 #pragma unroll
         for (int i = 0; i < DPL; i++) acc[h][i] = 0.f;
@@ -533,7 +535,7 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
             L = fmaf(sm_l[w][h], f, L);
             A = fmaf(sm_acc[w][h][d], f, A);
         }
-        const int head = kvh * G + h;
+        const int head = head0 + h;
         if (splits == 1) {
             out[(size_t)head * HD + d] = A / L;
         } else {
@@ -547,22 +549,22 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
 template <int G, int DPL>
 __global__ __launch_bounds__(256) void attn_split_kernel(const float* __restrict__ q, const float* __restrict__ K, const float* __restrict__ V,
                                                          int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev, float scale, int splits,
-                                                         uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out) {
-    attn_split_body<G, DPL, false>(q, K, V, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, QkvPostParams{});
+                                                         uint32_t window, float softcap, float* __restrict__ part, float* __restrict__ out, int gq) {
+    attn_split_body<G, DPL, false>(q, K, V, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, QkvPostParams{}, gq);
 }
 
 template <int G, int DPL, int QF>
 __global__ __launch_bounds__(256) void attn_split_kvq_kernel(const float* __restrict__ q, QCache qc, int n_kv, uint32_t len_host,
                                                              const uint32_t* __restrict__ len_dev, float scale, int splits, uint32_t window,
-                                                             float softcap, float* __restrict__ part, float* __restrict__ out) {
-    attn_split_body<G, DPL, false, QF>(q, nullptr, nullptr, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, QkvPostParams{}, qc);
+                                                             float softcap, float* __restrict__ part, float* __restrict__ out, int gq) {
+    attn_split_body<G, DPL, false, QF>(q, nullptr, nullptr, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, QkvPostParams{}, gq, qc);
 }
 
 template <int G, int DPL>
 __global__ __launch_bounds__(256) void attn_split_fused_kernel(QkvPostParams fp, int n_kv, uint32_t len_host, const uint32_t* __restrict__ len_dev,
                                                                float scale, int splits, uint32_t window, float softcap, float* __restrict__ part,
-                                                               float* __restrict__ out) {
-    attn_split_body<G, DPL, true>(nullptr, fp.k_cache, fp.v_cache, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, fp);
+                                                               float* __restrict__ out, int gq) {
+    attn_split_body<G, DPL, true>(nullptr, fp.k_cache, fp.v_cache, n_kv, len_host, len_dev, scale, splits, window, softcap, part, out, fp, gq);
 }
 
 // One workgroup per query head: weights exp(m_s - max m) of the splits once (through LDS), then every output dim is a
@@ -603,10 +605,10 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_combine_kernel(const flo
 
 template <int G>
 int launch_attn_g(int hd, dim3 grid, hipStream_t s, const float* q, const float* K, const float* V, int n_kv, uint32_t len, const uint32_t* d_len,
-                  float scale, int splits, uint32_t window, float softcap, float* part, float* out) {
+                  float scale, int splits, uint32_t window, float softcap, float* part, float* out, int gq = G) {
     switch (hd) {
-        case 64: hipLaunchKernelGGL((attn_split_kernel<G, 4>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
-        case 128: hipLaunchKernelGGL((attn_split_kernel<G, 8>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        case 64: hipLaunchKernelGGL((attn_split_kernel<G, 4>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out, gq); break;
+        case 128: hipLaunchKernelGGL((attn_split_kernel<G, 8>), grid, dim3(256), 0, s, q, K, V, n_kv, len, d_len, scale, splits, window, softcap, part, out, gq); break;
         default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     }
     return FHIP_OK;
@@ -614,10 +616,10 @@ int launch_attn_g(int hd, dim3 grid, hipStream_t s, const float* q, const float*
 
 template <int G, int QF>
 int launch_attn_kvq_g(int hd, dim3 grid, hipStream_t s, const float* q, const QCache& qc, int n_kv, uint32_t len, const uint32_t* d_len,
-                      float scale, int splits, uint32_t window, float softcap, float* part, float* out) {
+                      float scale, int splits, uint32_t window, float softcap, float* part, float* out, int gq = G) {
     switch (hd) {
-        case 64: hipLaunchKernelGGL((attn_split_kvq_kernel<G, 4, QF>), grid, dim3(256), 0, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
-        case 128: hipLaunchKernelGGL((attn_split_kvq_kernel<G, 8, QF>), grid, dim3(256), 0, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        case 64: hipLaunchKernelGGL((attn_split_kvq_kernel<G, 4, QF>), grid, dim3(256), 0, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out, gq); break;
+        case 128: hipLaunchKernelGGL((attn_split_kvq_kernel<G, 8, QF>), grid, dim3(256), 0, s, q, qc, n_kv, len, d_len, scale, splits, window, softcap, part, out, gq); break;
         default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     }
     return FHIP_OK;
@@ -640,10 +642,10 @@ int launch_attn_kvq(int g, int hd, dim3 grid, hipStream_t s, const float* q, con
 
 template <int G>
 int launch_attn_fused_g(int hd, dim3 grid, hipStream_t s, const QkvPostParams& fp, int n_kv, uint32_t len, const uint32_t* d_len, float scale,
-                        int splits, uint32_t window, float softcap, float* part, float* out) {
+                        int splits, uint32_t window, float softcap, float* part, float* out, int gq = G) {
     switch (hd) {
-        case 64: hipLaunchKernelGGL((attn_split_fused_kernel<G, 4>), grid, dim3(256), 0, s, fp, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
-        case 128: hipLaunchKernelGGL((attn_split_fused_kernel<G, 8>), grid, dim3(256), 0, s, fp, n_kv, len, d_len, scale, splits, window, softcap, part, out); break;
+        case 64: hipLaunchKernelGGL((attn_split_fused_kernel<G, 4>), grid, dim3(256), 0, s, fp, n_kv, len, d_len, scale, splits, window, softcap, part, out, gq); break;
+        case 128: hipLaunchKernelGGL((attn_split_fused_kernel<G, 8>), grid, dim3(256), 0, s, fp, n_kv, len, d_len, scale, splits, window, softcap, part, out, gq); break;
         default: return fhip::set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     }
     return FHIP_OK;
@@ -737,6 +739,12 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
 
 // Splits of the key range: about two workgroups per CU over all KV heads, at least 64 keys each (two rounds of the
 // workgroup's 16 streams x 2 keys; 16 for caches of up to 256 rows), at most 256 (the combine kernel's LDS tables).
+// Caches of up to ATT_SHORT rows with several query heads per KV head: one workgroup per query head over the whole key range, no
+// splits, no combine launch. The rows of a KV head are read by each of its query heads' workgroups (a few hundred KB out of the
+// L2), which costs less than the second launch and the trip of the partial results through memory.
+constexpr size_t ATT_SHORT = 256;
+bool attn_per_query_head(size_t len, int n_head, int n_kv) { return n_kv > 0 && n_head > n_kv && len <= ATT_SHORT; }
+
 int attn_splits(size_t len, int n_kv) {
     if (n_kv <= 0 || len == 0) return 1;
     constexpr int keys = 64;
@@ -756,10 +764,16 @@ int launch_decode_attention(const float* q, const float* K, const float* V, int 
     if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: n_heads must be a multiple of n_kv_heads");
     if (hd != 64 && hd != 128) return set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     if (len > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "decode_attention: cache length exceeds 2^31");
-    const int g = n_head / n_kv, splits = attn_splits(len, n_kv);
-    if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
+    const int g = n_head / n_kv;
     const float scale = 1.0f / sqrtf((float)hd);
     const uint32_t win = window > 0x7FFFFFFFull ? 0u : (uint32_t)window;   // a window that large is no window
+    if (g > 8) return set_error(FHIP_ERR_SHAPE, "decode_attention: %d query heads per KV head (1..=8 supported)", g);
+    if (attn_per_query_head(len, n_head, n_kv)) {
+        int rc = launch_attn_g<1>(hd, dim3((unsigned)n_head, 1), s, q, K, V, n_kv, (uint32_t)len, d_len, scale, 1, win, softcap, ws, out, g);
+        return rc ? rc : check_hip(hipGetLastError(), "decode_attention launch");
+    }
+    const int splits = attn_splits(len, n_kv);
+    if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
     dim3 grid((unsigned)n_kv, (unsigned)splits);
     int rc;
     switch (g) {
@@ -790,13 +804,24 @@ int launch_decode_attention_kvq(int fmt, const float* q, const uint32_t* k_codes
     if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "decode_attention: n_heads must be a multiple of n_kv_heads");
     if (hd != 64 && hd != 128) return set_error(FHIP_ERR_SHAPE, "decode_attention: head_dim must be 64 or 128");
     if (len > 0x7FFFFFFFull) return set_error(FHIP_ERR_SHAPE, "decode_attention: cache length exceeds 2^31");
-    const int g = n_head / n_kv, splits = attn_splits(len, n_kv);
-    if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
+    const int g = n_head / n_kv;
     const float scale = 1.0f / sqrtf((float)hd);
     const uint32_t win = window > 0x7FFFFFFFull ? 0u : (uint32_t)window;
-    const dim3 grid((unsigned)n_kv, (unsigned)splits);
     const QCache qc{k_codes, k_scales, v_codes, v_scales};
     int rc;
+    if (g >= 1 && g <= 8 && attn_per_query_head(len, n_head, n_kv)) {   // as the f32 cache's launch: the same sums, the same bits
+        const dim3 per_head((unsigned)n_head, 1);
+        switch (fmt) {
+            case FHIP_KVQ_Q8_0: rc = launch_attn_kvq_g<1, FHIP_KVQ_Q8_0>(hd, per_head, s, q, qc, n_kv, (uint32_t)len, d_len, scale, 1, win, softcap, ws, out, g); break;
+            case FHIP_KVQ_Q4_0: rc = launch_attn_kvq_g<1, FHIP_KVQ_Q4_0>(hd, per_head, s, q, qc, n_kv, (uint32_t)len, d_len, scale, 1, win, softcap, ws, out, g); break;
+            case FHIP_KVQ_Q4_1: rc = launch_attn_kvq_g<1, FHIP_KVQ_Q4_1>(hd, per_head, s, q, qc, n_kv, (uint32_t)len, d_len, scale, 1, win, softcap, ws, out, g); break;
+            default: return set_error(FHIP_ERR_ARG, "decode_attention: unknown KV format %d", fmt);
+        }
+        return rc ? rc : check_hip(hipGetLastError(), "decode_attention launch");
+    }
+    const int splits = attn_splits(len, n_kv);
+    if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
+    const dim3 grid((unsigned)n_kv, (unsigned)splits);
     switch (fmt) {
         case FHIP_KVQ_Q8_0: rc = launch_attn_kvq<FHIP_KVQ_Q8_0>(g, hd, grid, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
         case FHIP_KVQ_Q4_0: rc = launch_attn_kvq<FHIP_KVQ_Q4_0>(g, hd, grid, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
@@ -821,7 +846,7 @@ int launch_qkv_post_attention(const float* qkv, const float* bias, const float* 
     if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: n_heads must be a multiple of n_kv_heads");
     if (hd != 64 && hd != 128) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: head_dim must be 64 or 128");
     if (len > 0x7FFFFFFFull || len > cap) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: length outside the cache");
-    const int g = n_head / n_kv, splits = attn_splits(len, n_kv);
+    const int g = n_head / n_kv, splits = attn_per_query_head(len, n_head, n_kv) ? 1 : attn_splits(len, n_kv);
     if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "qkv_post_attention: this cache length needs the workspace");
     QkvPostParams fp;
     fp.qkv = qkv; fp.bias = bias; fp.q_norm = q_norm; fp.k_norm = k_norm; fp.pos = d_pos; fp.freq_scale = freq_scale;
@@ -830,6 +855,13 @@ int launch_qkv_post_attention(const float* qkv, const float* bias, const float* 
     fp.cap = (uint32_t)cap; fp.eps = eps; fp.base = base; fp.kv_packed = 0;
     const float scale = 1.0f / sqrtf((float)hd);
     const uint32_t win = window > 0x7FFFFFFFull ? 0u : (uint32_t)window;
+    if (g > 8) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: %d query heads per KV head (1..=8 supported)", g);
+    if (attn_per_query_head(len, n_head, n_kv)) {
+        // every workgroup of a KV head forms the new token's K and V rows and stores them (the same bits from each) before
+        // it reads them back with the other keys
+        int rc = launch_attn_fused_g<1>(hd, dim3((unsigned)n_head, 1), s, fp, n_kv, (uint32_t)len, d_pos, scale, 1, win, softcap, ws, out, g);
+        return rc ? rc : check_hip(hipGetLastError(), "qkv_post_attention launch");
+    }
     dim3 grid((unsigned)n_kv, (unsigned)splits);
     int rc;
     switch (g) {
