@@ -386,6 +386,37 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
     const float* Kb = QF >= 0 ? nullptr : K + (size_t)kvh * HD + sub * DPL;
     const float* Vb = QF >= 0 ? nullptr : V + (size_t)kvh * HD + sub * DPL;
 
+    // The rows of a step are requested one step ahead: a stream's steps depend on one another only through the running
+    // maximum, so without this every step paid a memory round trip before its arithmetic (32 in a row for a split of 1024 keys).
+    // A step past the split's end re-reads the split's last row (always a row of the cache) and is never used.
+    constexpr int QFMT = QF >= 0 ? QF : 0;
+    const int qcol = kvh * HD + sub * DPL, qnblk = n_kv * (HD / 32);
+    RawDims<QFMT, DPL> kq[QF >= 0 ? ATT_KB : 1], vq[QF >= 0 ? ATT_KB : 1];
+    float kf[QF >= 0 ? 1 : ATT_KB][DPL], vf[QF >= 0 ? 1 : ATT_KB][DPL];
+    auto request = [&](uint32_t at) {
+#pragma unroll
+        for (int j = 0; j < ATT_KB; j++) {
+            const uint32_t key = min(at + j, k1 - 1);   // a row past the split re-reads its last row and is masked below
+            if constexpr (QF >= 0) {
+                kq[j] = fetch_dims_q<QFMT, DPL>(qc.k_codes, qc.k_scales, key, qnblk, qcol);
+                vq[j] = fetch_dims_q<QFMT, DPL>(qc.v_codes, qc.v_scales, key, qnblk, qcol);
+            } else {
+                load_dims<DPL>(Kb + key * stride, kf[j]);
+                load_dims<DPL>(Vb + key * stride, vf[j]);
+            }
+        }
+    };
+    // FUSED: the first step's rows are requested in front of the post-processing, so that their memory round trip runs under it,
+    // unless one of them could be the row this workgroup is about to append (then they are requested behind the barrier that
+    // follows the store; a step past the split's end re-reads row k1 - 1, which is why that row counts too).
+    bool requested = false;
+    if constexpr (FUSED) {
+        const uint32_t pos = *len_dev;
+        if (k0 < k1 && (pos >= k0 + ATT_STREAMS * ATT_KB || pos >= k1)) {
+            request(k0 + sid * ATT_KB);
+            requested = true;
+        }
+    }
     if constexpr (FUSED) {
         const uint32_t pos = *len_dev;
         // the rows are appended by the workgroup whose keys include them; a position past the rows attention looks at (but
@@ -442,27 +473,7 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
 #pragma unroll
         for (int i = 0; i < DPL; i++) acc[h][i] = 0.f;
     }
-    // The rows of a step are requested one step ahead: a stream's steps depend on one another only through the running
-    // maximum, so without this every step paid a memory round trip before its arithmetic (32 in a row for a split of 1024 keys).
-    // A step past the split's end re-reads the split's last row (always a row of the cache) and is never used.
-    constexpr int QFMT = QF >= 0 ? QF : 0;
-    const int qcol = kvh * HD + sub * DPL, qnblk = n_kv * (HD / 32);
-    RawDims<QFMT, DPL> kq[QF >= 0 ? ATT_KB : 1], vq[QF >= 0 ? ATT_KB : 1];
-    float kf[QF >= 0 ? 1 : ATT_KB][DPL], vf[QF >= 0 ? 1 : ATT_KB][DPL];
-    auto request = [&](uint32_t at) {
-#pragma unroll
-        for (int j = 0; j < ATT_KB; j++) {
-            const uint32_t key = min(at + j, k1 - 1);   // a row past the split re-reads its last row and is masked below
-            if constexpr (QF >= 0) {
-                kq[j] = fetch_dims_q<QFMT, DPL>(qc.k_codes, qc.k_scales, key, qnblk, qcol);
-                vq[j] = fetch_dims_q<QFMT, DPL>(qc.v_codes, qc.v_scales, key, qnblk, qcol);
-            } else {
-                load_dims<DPL>(Kb + key * stride, kf[j]);
-                load_dims<DPL>(Vb + key * stride, vf[j]);
-            }
-        }
-    };
-    request(k0 + sid * ATT_KB);
+    if (!requested) request(k0 + sid * ATT_KB);
     for (uint32_t kb = k0 + sid * ATT_KB; kb < k1; kb += ATT_STREAMS * ATT_KB) {
         float kr[ATT_KB][DPL], vr[ATT_KB][DPL];
 #pragma unroll
@@ -739,10 +750,10 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
 
 // Splits of the key range: about two workgroups per CU over all KV heads, at least 64 keys each (two rounds of the
 // workgroup's 16 streams x 2 keys; 16 for caches of up to 256 rows), at most 256 (the combine kernel's LDS tables).
-// Caches of up to ATT_SHORT rows with several query heads per KV head: one workgroup per query head over the whole key range, no
+// Caches of up to ATT_SHORT rows (a launch sized for that many) with several query heads per KV head: one workgroup per query head over the whole key range, no
 // splits, no combine launch. The rows of a KV head are read by each of its query heads' workgroups (a few hundred KB out of the
 // L2), which costs less than the second launch and the trip of the partial results through memory.
-constexpr size_t ATT_SHORT = 256;
+constexpr size_t ATT_SHORT = 384;   // chained 64-layer step, ms per token per-head | split: 180 keys 3.95 | 4.23, 248: 4.04 | 4.23, 370: 4.25 | 4.31, 500: 4.45 | 4.30
 bool attn_per_query_head(size_t len, int n_head, int n_kv) { return n_kv > 0 && n_head > n_kv && len <= ATT_SHORT; }
 
 int attn_splits(size_t len, int n_kv) {
