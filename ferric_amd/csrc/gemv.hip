@@ -1112,9 +1112,9 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     // measured level or worse elsewhere: rows of 14336 columns and more, whose staging takes several passes (Q6_K
     // 5120 x 17408 16.7 -> 17.3 us), Q4_K from 28 MB on (10240 x 5120 8.13 -> 8.30), the other 32-value formats.
     constexpr bool HAS_LATE = M == 1 && U > 1 && (F::TYPE == FHIP_Q4_K || F::TYPE == FHIP_Q6_K || F::TYPE == FHIP_Q5_K || F::TYPE == FHIP_Q8_0);
-    const size_t wbytes = (size_t)w->rows * w->row_bytes;
+    const size_t wbytes = out_rows * (SWIGLU ? 2 : 1) * w->row_bytes;   // of the rows this launch walks (one expert's, behind a selection)
     const bool small = wbytes < ((size_t)28 << 20);
-    bool late = HAS_LATE && !sel && w->cols <= 8192 && (F::TYPE == FHIP_Q6_K || small);
+    bool late = HAS_LATE && w->cols <= 8192 && (F::TYPE == FHIP_Q6_K || small);
     GemvParams p;
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
