@@ -108,7 +108,13 @@ __device__ __forceinline__ float slot_sum(float v) {
 template <int U>
 __device__ __forceinline__ float slot_sum_many(const float (&v)[U], bool bit0, bool bit1) {
     static_assert(U >= 1 && U <= 4, "one to four values");
-    if constexpr (U == 1) return slot_sum(v[0]);
+    if constexpr (U == 1) {   // the same tree of additions as below, so that a row's bits do not depend on U
+        float r = v[0] + dpp_f<DPP_XOR1>(v[0]);
+        r += dpp_f<DPP_XOR2>(r);
+        r += dpp_f<DPP_ROR4>(r);
+        r += dpp_f<DPP_ROR8>(r);
+        return r;
+    }
     float a, b;
     if constexpr (U == 2) {
         a = v[0] + dpp_f<DPP_XOR1>(v[0]);
@@ -1103,10 +1109,9 @@ size_t lds_bytes(size_t cols, int NG, int G, int rpg) {
     return M * cols * NP + 2 * M * (cols / F::RUN) * sizeof(float) + (size_t)G * rpg * (SWIGLU ? 2 : 1) * NG * M * sizeof(float);
 }
 
-template <class F, int M, bool SWIGLU>
-int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr,
-               const fhip::NormParams* norm = nullptr) {
-    constexpr int U = rows_in_flight<F>(M);
+template <class F, int M, bool SWIGLU, int U>
+int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel,
+                 const fhip::NormParams* norm) {
     // The prefetch of a wave's later rows waits behind the staging barrier for the small weights of the formats the
     // decode layers are made of (see the kernel; also Q5_K 5120 x 5120 7.20 -> 6.47 us, Q8_0 4096 x 4096 6.78 -> 6.57);
     // measured level or worse elsewhere: rows of 14336 columns and more, whose staging takes several passes (Q6_K
@@ -1216,6 +1221,19 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     const size_t launch_wgs = grid + ((norm && norm->x_out && grid < (size_t)cus) ? 1 : 0);
     hipLaunchKernelGGL(kernel, dim3((unsigned)launch_wgs, (unsigned)p.sel.npairs), dim3(64 * WPR * G), lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
+}
+
+template <class F, int M, bool SWIGLU>
+int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, hipStream_t s, const fhip::SelParams* sel = nullptr,
+               const fhip::NormParams* norm = nullptr) {
+    // Q6_K rows of more than 8192 columns (the down projection: nine waves per workgroup, early prefetch) stream with one row in
+    // flight per wave instead of two: 5120 x 17408 16.7 -> 16.35 us, 4096 x 14336 12.56 -> 12.41 on cold weights (Q4_K rows of
+    // that length lose 6 % the same way and keep two). The slot sums are the same tree of additions for every U, so the row's
+    // bits stay those of the batched launches.
+    if constexpr (M == 1 && F::TYPE == FHIP_Q6_K) {
+        if (w->cols > 8192 && !sel && !norm) return launch_one_u<F, M, SWIGLU, 1>(w, d_x, d_y, out_rows, s, sel, norm);
+    }
+    return launch_one_u<F, M, SWIGLU, rows_in_flight<F>(M)>(w, d_x, d_y, out_rows, s, sel, norm);
 }
 
 // Largest batch width (4, 2, 1, or 0 = shape not covered) whose workgroup fits the wave and LDS limits.
