@@ -1129,12 +1129,21 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
     p.NG = (p.units + 15) / 16;
     constexpr int MAXW = max_threads(M) / 64;
     p.RF = full_wave_replicas(p.NG, MAXW);
-    const int WPR = waves_per_row_group(p.NG, MAXW);
+    int WPR = waves_per_row_group(p.NG, MAXW);
     // Rows per row group (rpg) and row groups per workgroup (G). A CU holds Gcap row groups at once (one
     // workgroup of MAXW waves). Every workgroup pays a fixed few microseconds (activation quantisation,
     // pipeline fill and drain), so the rows are dealt out in as few rounds as possible: one workgroup per
     // CU with up to RPG_MAX rows per row group, more rounds of equal size only beyond that. With a
     // partly filled single round the row groups are spread over all CUs.
+    // A small late-prefetch weight whose rows leave one slot over (5120 columns: four full waves' worth and a tail slot) runs
+    // two replicas of the full-wave set per row group instead of four: row groups of three waves, five of them per workgroup,
+    // four rows each where 5120 rows meet 256 CUs -- every full wave gets exactly two rows and no CU stays empty (5120 x 5120
+    // Q4_K 5.53 -> 5.50 us, QKV 6.96 -> 6.86, Q6_K 5120 x 5120 7.09 -> 6.83, Q5_K 6.48 -> 6.33; the large weights lose 5 - 8 %
+    // that way and keep four).
+    if (late && small && M == 1 && p.RF == 4 && (p.NG & 3) == 1) {
+        p.RF = 2;
+        WPR = (p.NG >> 2) * 2 + 1;
+    }
     int RPG_MAX = 256;
     int cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     if (p.sel.npairs > 1) cus = cus / p.sel.npairs > 0 ? cus / p.sel.npairs : 1;   // the pairs of an "_id" launch share the chip
