@@ -1166,6 +1166,15 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
         // the fused norm holds one 8-value piece of the row per thread
         if (norm) { const int need = (int)((w->cols + (size_t)512 * WPR - 1) / ((size_t)512 * WPR)); if (want < need) want = need; }
         if (want < Gcap) {
+            // rows per CU after rounding up to whole row groups: one or two row groups fewer where that leaves a twentieth or
+            // more of the chip less idle (8192 rows on 256 CUs: five row groups of 7 rows fill 234 CUs, four of 8 fill all;
+            // 8192 x 8192 Q4_K 10.4 -> 9.4 us). More row groups for the same reason measured slower (22016 x 4096: 12.2 -> 12.6).
+            const int need = norm ? (int)((w->cols + (size_t)512 * WPR - 1) / ((size_t)512 * WPR)) : 1;
+            auto rows_per_cu = [&](int g) { return (size_t)g * ((out_rows + (size_t)cus * g - 1) / ((size_t)cus * g)); };
+            int best = want;
+            for (int g = want - 1; g >= want - 2 && g >= 1 && g >= need; g--)
+                if (rows_per_cu(g) * 20 <= rows_per_cu(best) * 19) best = g;
+            want = best;
             Gcap = want;
             // one round for up to 1024 rows per row group where the partial sums still fit beside the staged row
             if (lds_bytes<F, M, SWIGLU>(w->cols, p.NG, Gcap, 1024) + 512 <= fhip::device_lds_bytes()) RPG_MAX = 1024;
