@@ -1154,14 +1154,14 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
     // hold 90 - 100 KB, and what is queued beyond the pipe's depth only reaches the DRAM pages in a worse order. Measured on
     // cold weights, one activation row: Q6_K is fastest with 5 - 7 waves per workgroup at every size (5120 columns, 5120 /
     // 20480 / 151936 rows: 8.65 -> 7.83, 19.7 -> 18.5, 118.5 -> 107.0 us; 128256 x 4096: 82.1 -> 73.7 us with six row groups),
-    // Q4_K with 8 - 10 waves once the weight has 28 MB or more (20480 x 5120 13.9 -> 12.6 us, fused gate|up 34816 x 5120
+    // Q4_K with the fewest whole row groups that make 8 waves (8 - 14) once the weight has 28 MB or more (20480 x 5120 13.9 -> 12.6 us, fused gate|up 34816 x 5120
     // 20.9 -> 20.2, 28672 x 4096 15.3 -> 14.6) and with all 15 - 16 below that (5120 x 5120: 5.95 us against 6.39). A small
     // Q6_K weight whose later rows are requested behind the barrier keeps all its waves (5120 x 5120: 7.08 us against 7.98;
     // twelve of the sixteen one-wave row groups of 4096 columns: 4096 x 4096 5.49 us against 5.98).
     if (M == 1 && p.sel.npairs <= 1) {
         int want = Gcap;
         if (F::TYPE == FHIP_Q6_K) want = late && small ? (WPR == 1 ? 12 : Gcap) : 6 / WPR;
-        else if (F::TYPE == FHIP_Q4_K && !small) want = ((WPR == 1 ? 8 : 10) + WPR - 1) / WPR;
+        else if (F::TYPE == FHIP_Q4_K && !small) want = (8 + WPR - 1) / WPR;
         if (want < 1) want = 1;
         // the fused norm holds one 8-value piece of the row per thread
         if (norm) { const int need = (int)((w->cols + (size_t)512 * WPR - 1) / ((size_t)512 * WPR)); if (want < need) want = need; }
