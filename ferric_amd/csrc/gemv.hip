@@ -662,8 +662,10 @@ struct GemvParams {
     int row_wgs;         // workgroups that own rows; the launch may hold one more, which only stores x + resid
 };
 
-// Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 512 -> 256).
-constexpr int max_threads(int M) { return M == 1 ? 1024 : 512; }
+// Threads per workgroup allowed for M activation rows (register budget: 1024 -> 128 VGPRs, 640 -> 168, 512 -> 256).
+// Two Q4_K activation rows fit 168 registers, ten waves (5120 columns: two row groups per workgroup; cold, two rows: 5120 x 5120
+// 8.9 -> 8.0 us, fused gate|up 27.7 -> 23.2); Q6_K spills there (down 23.0 -> 28.9) and keeps eight.
+template <class F> constexpr int max_threads(int M) { return M == 1 ? 1024 : (F::TYPE == FHIP_Q4_K ? 640 : 512); }
 // Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit 128 VGPRs
 // at batch 1 (16 waves per CU).
 template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? F::U1 : 2; }
@@ -730,7 +732,7 @@ __device__ __forceinline__ void quantize8(const float (&v)[8], uint32_t (&pl)[NP
 }
 
 template <class F, int M, int U, bool SWIGLU, bool NORM, bool LATE>
-__global__ void __launch_bounds__(max_threads(M)) gemv_stream_kernel(GemvParams p) {
+__global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     fhip::apply_selection(p);
     constexpr int VPR = SWIGLU ? 2 : 1;       // weight rows walked per output row
@@ -1127,7 +1129,7 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
     p.sel = sel ? *sel : fhip::SelParams{nullptr, 0, 0, 0, 0, 0, 1};
     p.units = (int)(w->cols / F::WPL);
     p.NG = (p.units + 15) / 16;
-    constexpr int MAXW = max_threads(M) / 64;
+    constexpr int MAXW = max_threads<F>(M) / 64;
     p.RF = full_wave_replicas(p.NG, MAXW);
     int WPR = waves_per_row_group(p.NG, MAXW);
     // Rows per row group (rpg) and row groups per workgroup (G). A CU holds Gcap row groups at once (one
@@ -1259,11 +1261,11 @@ template <class F, bool SWIGLU>
 int max_batch(const fhip_weight* w, size_t left) {
     if (w->cols % F::WPL != 0 || g_force_generic) return 0;
     const int NG = (int)((w->cols / F::WPL + 15) / 16);
-    auto WPRm = [&](int m) { return waves_per_row_group(NG, max_threads(m) / 64); };
+    auto WPRm = [&](int m) { return waves_per_row_group(NG, max_threads<F>(m) / 64); };
     const size_t cap = fhip::device_lds_bytes();
-    if (left >= 4 && max_m<F>() >= 4 && WPRm(4) * 64 <= max_threads(4) && lds_bytes<F, 4, SWIGLU>(w->cols, NG, max_threads(4) / 64 / WPRm(4), 256) <= cap) return 4;
-    if (left >= 2 && WPRm(2) * 64 <= max_threads(2) && lds_bytes<F, 2, SWIGLU>(w->cols, NG, max_threads(2) / 64 / WPRm(2), 256) <= cap) return 2;
-    if (WPRm(1) * 64 <= max_threads(1) && lds_bytes<F, 1, SWIGLU>(w->cols, NG, max_threads(1) / 64 / WPRm(1), 256) <= cap) return 1;
+    if (left >= 4 && max_m<F>() >= 4 && WPRm(4) * 64 <= max_threads<F>(4) && lds_bytes<F, 4, SWIGLU>(w->cols, NG, max_threads<F>(4) / 64 / WPRm(4), 256) <= cap) return 4;
+    if (left >= 2 && WPRm(2) * 64 <= max_threads<F>(2) && lds_bytes<F, 2, SWIGLU>(w->cols, NG, max_threads<F>(2) / 64 / WPRm(2), 256) <= cap) return 2;
+    if (WPRm(1) * 64 <= max_threads<F>(1) && lds_bytes<F, 1, SWIGLU>(w->cols, NG, max_threads<F>(1) / 64 / WPRm(1), 256) <= cap) return 1;
     return 0;
 }
 
