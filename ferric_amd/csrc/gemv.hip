@@ -667,10 +667,13 @@ struct GemvParams {
 // 8.9 -> 8.0 us, fused gate|up 27.7 -> 23.2); Q6_K fits them with one weight row in flight per wave instead of two (156
 // registers; with two it spills: 5120 x 17408 at two rows 23.0 us in eight waves, 28.9 in ten with spills, 20.2 in ten with one
 // row in flight; 151936 x 5120 133 -> 120).
-template <class F> constexpr int max_threads(int M) { return M == 1 ? 1024 : (F::TYPE == FHIP_Q4_K || F::TYPE == FHIP_Q6_K ? 640 : 512); }
+// (With three activation planes both spill at 168 registers, 152 and 64 bytes a lane: that build keeps eight waves.)
+template <class F> constexpr int max_threads(int M) {
+    return M == 1 ? 1024 : (NP == 2 && (F::TYPE == FHIP_Q4_K || F::TYPE == FHIP_Q6_K) ? 640 : 512);
+}
 // Rows in flight per wave, sized so the prefetched rows plus the resident activation planes fit 128 VGPRs
 // at batch 1 (16 waves per CU).
-template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? F::U1 : (F::TYPE == FHIP_Q6_K ? 1 : 2); }
+template <class F> constexpr int rows_in_flight(int M) { return M == 1 ? F::U1 : (NP == 2 && F::TYPE == FHIP_Q6_K ? 1 : 2); }
 // Activation rows one pass can hold in registers.
 template <class F> constexpr int max_m() { return F::WPL == 64 ? 2 : 4; }
 
