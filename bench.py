@@ -458,7 +458,7 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
         ms = timer.time_ms(lambda: [dec.step_graph() for _ in range(steps)]) / steps
         logits = dec.logits.to_vec(stream)
         kv_bytes = 2 * (ctx + steps // 2) * nkv * hd * 4 * layers
-        out[str(ctx)] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * dec.launches_per_layer + 2,
+        out[str(ctx)] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * dec.launches_per_layer + dec.launches_per_token_extra,
                          "kv_bytes_read": kv_bytes, "GBps_weights_plus_kv": (weight_bytes_total + kv_bytes) / (ms * 1e-3) / 1e9,
                          "logits_finite": bool(np.isfinite(logits).all())}
         del dec
@@ -470,7 +470,7 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
     ms = timer.time_ms(lambda: [dec.step_graph() for _ in range(steps)]) / steps
     logits = dec.logits.to_vec(stream)
     kv_bytes = 2 * (ctx + steps // 2) * (nkv * hd // 32) * 34 * layers
-    out[f"{ctx}_q8_0_cache"] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * dec.launches_per_layer + 2,
+    out[f"{ctx}_q8_0_cache"] = {"ms_per_token": ms, "tokens_per_s": 1e3 / ms, "launches_per_token": layers * dec.launches_per_layer + dec.launches_per_token_extra,
                                 "kv_bytes_read": kv_bytes, "logits_finite": bool(np.isfinite(logits).all())}
     del dec
     # the same stack on a block of prompt rows: projections on the bf16 matrix cores, causal attention on the f32 ones

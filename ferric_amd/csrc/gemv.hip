@@ -1171,7 +1171,13 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
         else if (F::TYPE == FHIP_Q4_K && !small) want = (8 + WPR - 1) / WPR;
         if (want < 1) want = 1;
         // the fused norm holds one 8-value piece of the row per thread
-        if (norm) { const int need = (int)((w->cols + (size_t)512 * WPR - 1) / ((size_t)512 * WPR)); if (want < need) want = need; }
+        if (norm) {
+            const int need = (int)((w->cols + (size_t)512 * WPR - 1) / ((size_t)512 * WPR));
+            // a weight of 128 MB and more loses more to the extra waves than a norm launch of its own costs (vocabulary head
+            // 151936 x 5120: 119.2 us fused in two row groups, 107.7 + 3 apart): nothing is launched, the caller norms first
+            if (want < need && wbytes >= ((size_t)128 << 20)) return fhip::NORM_NOT_FUSED;
+            if (want < need) want = need;
+        }
         if (want < Gcap) {
             // rows per CU after rounding up to whole row groups: one or two row groups fewer where that leaves a twentieth or
             // more of the chip less idle (8192 rows on 256 CUs: five row groups of 7 rows fill 234 CUs, four of 8 fill all;

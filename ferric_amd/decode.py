@@ -254,6 +254,10 @@ class Qwen3Decoder:
         short = self.max_len <= 384 and c.n_head > c.n_head_kv
         self.launches_per_layer = ((7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0) + (1 if kv_fmt is not None else 0)
                                    - (1 if short else 0))
+        # per token beside the layers: the position word's increment and the head (final norm inside the head's mat-vec; a head of
+        # 128 MB and more takes the norm as a launch of its own, which costs less than the wider workgroups the fused norm needs)
+        big_head = lm_head is not None and lm_head.nbytes() >= (128 << 20)
+        self.launches_per_token_extra = 1 + ((1 if self.fuse_norm and not big_head else 2) if lm_head is not None else 0)
         self._graph = None
 
     # -- state ------------------------------------------------------------------------------------
