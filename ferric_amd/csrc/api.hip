@@ -864,7 +864,7 @@ int fhip_causal_attention(const float* d_q, const float* d_k, const float* d_v, 
 
 size_t fhip_decode_attention_ws_bytes(size_t n_head, size_t n_kv, size_t head_dim, size_t len) {
     if (g_device < 0 || n_kv == 0 || len == 0) return 0;
-    int splits = fhip::attn_splits(len, (int)n_kv);
+    int splits = fhip::attn_ws_splits(len, (int)n_head, (int)n_kv);
     return splits > 1 ? n_head * (size_t)splits * (head_dim + 2) * sizeof(float) : 0;
 }
 

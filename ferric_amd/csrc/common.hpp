@@ -153,6 +153,7 @@ int launch_qkv_post(const float* qkv, const float* bias, const float* q_norm, co
 int launch_kv_append(const float* k, const float* v, size_t t, size_t width, const uint32_t* d_pos, uint32_t pos_off, size_t cap, float* kc,
                      float* vc, hipStream_t s);
 int attn_splits(size_t len, int n_kv);
+int attn_ws_splits(size_t len, int n_head, int n_kv);
 int launch_qkv_post_attention(const float* qkv, const float* bias, const float* q_norm, const float* k_norm, const uint32_t* d_pos,
                               const float* freq_scale, int n_head, int n_kv, int hd, int n_rot, bool interleaved, float eps, float base,
                               float* k_cache, float* v_cache, size_t cap, size_t len, size_t window, float softcap, float* ws, float* out,

@@ -356,7 +356,16 @@ __device__ __forceinline__ void attn_split_body(const float* __restrict__ q, typ
     const int sid = wave * 4 + (lane >> 4);
     // Workgroup blockIdx.x takes the G query heads from head0 on; gq = query heads per KV head. gq == G: one workgroup per KV
     // head and split. gq > G (short caches, G = 1): one workgroup per query head, the KV head's rows read by each of them.
-    const int head0 = blockIdx.x * G, kvh = head0 / gq, split = blockIdx.y;
+    // gq < 0 (G = 1, a one-dimensional grid): one workgroup per (query head, split) for -gq query heads per KV head, dealt so
+    // that the workgroups of one KV head and split -- which read the same rows -- are consecutive slots of one XCD (workgroup
+    // L runs on XCD L % 8): slot i = L / 8 of XCD x = L % 8 is query head i % g of group (i / g) * 8 + x.
+    int head0 = blockIdx.x * G, kvh = gq > 0 ? head0 / gq : 0, split = blockIdx.y;
+    if (gq < 0) {
+        const int g = -gq, x = blockIdx.x & 7, i = blockIdx.x >> 3;
+        const int grp = (i / g) * 8 + x;
+        if (grp >= n_kv * splits) return;
+        kvh = grp % n_kv; split = grp / n_kv; head0 = kvh * g + i % g;
+    }
     // FUSED: the raw values of every head this wave will post-process (job j = wave + 4 r: query head j of the group, then
     // the key and the value row) are requested before anything else, the length word with them, so that one memory round
     // trip covers what used to be three in a row (the length, the first round's rows, the second round's).
@@ -756,6 +765,21 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
 constexpr size_t ATT_SHORT = 384;   // chained 64-layer step, ms per token per-head | split: 180 keys 3.95 | 4.23, 248: 4.04 | 4.23, 370: 4.25 | 4.31, 500: 4.45 | 4.30
 bool attn_per_query_head(size_t len, int n_head, int n_kv) { return n_kv > 0 && n_head > n_kv && len <= ATT_SHORT; }
 
+// Between ATT_SHORT and ATT_MID rows under grouped query heads: one workgroup per (query head, split of at least ATT_MID_KEYS
+// keys). The kernel that takes all query heads of a KV head at once holds 180 registers a lane (two waves per SIMD) and its
+// waves spend their time in the dependent arithmetic of five softmax chains; with one head a workgroup (107 registers, four
+// waves per SIMD) the same arithmetic is spread over five times the waves, and the rows they share come out of one XCD's L2
+// (see the kernel's workgroup numbering). Chained 64-layer step, ms per token, this shape | all heads of a KV head per
+// workgroup: 500 keys 3.99 | 4.24, 1000: 4.06 | 4.28, 2048: 4.22 | 4.56, 4096: 4.63 | 4.77, 6000: 4.97 | 4.90, 8000: 5.41 | 5.08.
+constexpr size_t ATT_MID = 5120, ATT_MID_KEYS = 128;
+bool attn_per_head_splits(size_t len, int n_head, int n_kv) { return n_kv > 0 && n_head > n_kv && len > ATT_SHORT && len <= ATT_MID; }
+// splits of at least ATT_MID_KEYS keys, at most about two and a half workgroups per CU over all query heads
+int attn_mid_splits(size_t len, int n_head) {
+    const int by_keys = (int)((len + ATT_MID_KEYS - 1) / ATT_MID_KEYS), cap = 5 * device_cus() / 2 / (n_head > 0 ? n_head : 1);
+    const int s = by_keys < cap ? by_keys : cap;
+    return s < 1 ? 1 : (s > 256 ? 256 : s);
+}
+
 int attn_splits(size_t len, int n_kv) {
     if (n_kv <= 0 || len == 0) return 1;
     constexpr int keys = 64;
@@ -766,6 +790,13 @@ int attn_splits(size_t len, int n_kv) {
     size_t by_keys = (len + per_split - 1) / per_split;
     int splits = (int)(by_keys < (size_t)want ? by_keys : (size_t)want);
     return splits < 1 ? 1 : (splits > 256 ? 256 : splits);
+}
+
+// the most splits any launch shape takes for this cache length: what the workspace has to hold
+int attn_ws_splits(size_t len, int n_head, int n_kv) {
+    const int a = attn_splits(len, n_kv);
+    const int b = attn_per_head_splits(len, n_head, n_kv) ? attn_mid_splits(len, n_head) : 1;
+    return a > b ? a : b;
 }
 
 int launch_decode_attention(const float* q, const float* K, const float* V, int n_head, int n_kv, int hd, size_t len, const uint32_t* d_len,
@@ -783,10 +814,15 @@ int launch_decode_attention(const float* q, const float* K, const float* V, int 
         int rc = launch_attn_g<1>(hd, dim3((unsigned)n_head, 1), s, q, K, V, n_kv, (uint32_t)len, d_len, scale, 1, win, softcap, ws, out, g);
         return rc ? rc : check_hip(hipGetLastError(), "decode_attention launch");
     }
-    const int splits = attn_splits(len, n_kv);
+    const bool mid = attn_per_head_splits(len, n_head, n_kv);
+    const int splits = mid ? attn_mid_splits(len, n_head) : attn_splits(len, n_kv);
     if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
     dim3 grid((unsigned)n_kv, (unsigned)splits);
     int rc;
+    if (mid) {
+        const unsigned wgs = (unsigned)((n_kv * splits + 7) / 8 * 8 * g);
+        rc = launch_attn_g<1>(hd, dim3(wgs, 1), s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out, -g);
+    } else
     switch (g) {
         case 1: rc = launch_attn_g<1>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
         case 2: rc = launch_attn_g<2>(hd, grid, s, q, K, V, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
@@ -830,9 +866,19 @@ int launch_decode_attention_kvq(int fmt, const float* q, const uint32_t* k_codes
         }
         return rc ? rc : check_hip(hipGetLastError(), "decode_attention launch");
     }
-    const int splits = attn_splits(len, n_kv);
+    const bool mid = g >= 1 && g <= 8 && attn_per_head_splits(len, n_head, n_kv);
+    const int splits = mid ? attn_mid_splits(len, n_head) : attn_splits(len, n_kv);
     if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "decode_attention: this cache length needs the workspace");
     const dim3 grid((unsigned)n_kv, (unsigned)splits);
+    if (mid) {
+        const dim3 lin((unsigned)((n_kv * splits + 7) / 8 * 8 * g), 1);
+        switch (fmt) {
+            case FHIP_KVQ_Q8_0: rc = launch_attn_kvq_g<1, FHIP_KVQ_Q8_0>(hd, lin, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out, -g); break;
+            case FHIP_KVQ_Q4_0: rc = launch_attn_kvq_g<1, FHIP_KVQ_Q4_0>(hd, lin, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out, -g); break;
+            case FHIP_KVQ_Q4_1: rc = launch_attn_kvq_g<1, FHIP_KVQ_Q4_1>(hd, lin, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out, -g); break;
+            default: return set_error(FHIP_ERR_ARG, "decode_attention: unknown KV format %d", fmt);
+        }
+    } else
     switch (fmt) {
         case FHIP_KVQ_Q8_0: rc = launch_attn_kvq<FHIP_KVQ_Q8_0>(g, hd, grid, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
         case FHIP_KVQ_Q4_0: rc = launch_attn_kvq<FHIP_KVQ_Q4_0>(g, hd, grid, s, q, qc, n_kv, (uint32_t)len, d_len, scale, splits, win, softcap, ws, out); break;
@@ -857,7 +903,9 @@ int launch_qkv_post_attention(const float* qkv, const float* bias, const float* 
     if (n_kv <= 0 || n_head % n_kv != 0) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: n_heads must be a multiple of n_kv_heads");
     if (hd != 64 && hd != 128) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: head_dim must be 64 or 128");
     if (len > 0x7FFFFFFFull || len > cap) return set_error(FHIP_ERR_SHAPE, "qkv_post_attention: length outside the cache");
-    const int g = n_head / n_kv, splits = attn_per_query_head(len, n_head, n_kv) ? 1 : attn_splits(len, n_kv);
+    const int g = n_head / n_kv;
+    const bool mid = g <= 8 && attn_per_head_splits(len, n_head, n_kv);
+    const int splits = attn_per_query_head(len, n_head, n_kv) ? 1 : (mid ? attn_mid_splits(len, n_head) : attn_splits(len, n_kv));
     if (splits > 1 && !ws) return set_error(FHIP_ERR_ARG, "qkv_post_attention: this cache length needs the workspace");
     QkvPostParams fp;
     fp.qkv = qkv; fp.bias = bias; fp.q_norm = q_norm; fp.k_norm = k_norm; fp.pos = d_pos; fp.freq_scale = freq_scale;
@@ -875,6 +923,10 @@ int launch_qkv_post_attention(const float* qkv, const float* bias, const float* 
     }
     dim3 grid((unsigned)n_kv, (unsigned)splits);
     int rc;
+    if (mid) {
+        const unsigned wgs = (unsigned)((n_kv * splits + 7) / 8 * 8 * g);
+        rc = launch_attn_fused_g<1>(hd, dim3(wgs, 1), s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out, -g);
+    } else
     switch (g) {
         case 1: rc = launch_attn_fused_g<1>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;
         case 2: rc = launch_attn_fused_g<2>(hd, grid, s, fp, n_kv, (uint32_t)len, d_pos, scale, splits, win, softcap, ws, out); break;

@@ -89,7 +89,7 @@ def test_kv_append2_and_decode_attention(F, X, D):
     rng = np.random.default_rng(2)
     # (14, 2, 64, [8192]): head_dim 64 with more than 64 splits of the key range (2 KV heads on 256 CUs), the case in which
     # the combine kernel's thread count and its loop stride have to agree
-    for nh, nkv, hd, lens in [(40, 8, 128, [1, 7, 64, 65, 383, 384, 385, 1000]), (8, 8, 64, [3, 257]), (16, 2, 128, [130]), (6, 2, 64, [33]), (5, 1, 128, [2049]),
+    for nh, nkv, hd, lens in [(40, 8, 128, [1, 7, 64, 65, 383, 384, 385, 1000, 5120, 5121]), (8, 8, 64, [3, 257]), (16, 2, 128, [130]), (6, 2, 64, [33]), (5, 1, 128, [2049]),
                               (64, 8, 128, [4097]), (14, 2, 64, [8192])]:
         cap = max(lens) + 3
         width = nkv * hd
