@@ -762,7 +762,7 @@ int launch_kv_append(const float* k, const float* v, size_t t, size_t width, con
 // Caches of up to ATT_SHORT rows (a launch sized for that many) with several query heads per KV head: one workgroup per query head over the whole key range, no
 // splits, no combine launch. The rows of a KV head are read by each of its query heads' workgroups (a few hundred KB out of the
 // L2), which costs less than the second launch and the trip of the partial results through memory.
-constexpr size_t ATT_SHORT = 384;   // chained 64-layer step, ms per token per-head | split: 180 keys 3.95 | 4.23, 248: 4.04 | 4.23, 370: 4.25 | 4.31, 500: 4.45 | 4.30
+constexpr size_t ATT_SHORT = 256;   // chained 64-layer step, ms per token, this shape | one workgroup per (query head, split): 180 keys 3.87 | 3.92, 248: 3.96 | 3.99, 300: 4.05 | 3.96, 370: 4.11 | 3.97
 bool attn_per_query_head(size_t len, int n_head, int n_kv) { return n_kv > 0 && n_head > n_kv && len <= ATT_SHORT; }
 
 // Between ATT_SHORT and ATT_MID rows under grouped query heads: one workgroup per (query head, split of at least ATT_MID_KEYS

@@ -250,8 +250,8 @@ class Qwen3Decoder:
             # of its own up to 2048 keys (5.12 -> 5.06 ms/token there, 4.92 -> 4.84 at 128) and is level with it from 4096 on.
             self.fuse_attn = True
         self.fuse_attn = bool(self.fuse_attn)
-        # a default-arm layer; caches of up to 384 rows under grouped query heads need no combine launch behind the attention
-        short = self.max_len <= 384 and c.n_head > c.n_head_kv
+        # a default-arm layer; caches of up to 256 rows under grouped query heads need no combine launch behind the attention
+        short = self.max_len <= 256 and c.n_head > c.n_head_kv
         self.launches_per_layer = ((7 if self.fuse_norm else 9) - (1 if self.fuse_attn else 0) + (1 if kv_fmt is not None else 0)
                                    - (1 if short else 0))
         # per token beside the layers: the position word's increment and the head (final norm inside the head's mat-vec; a head of

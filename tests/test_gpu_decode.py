@@ -89,7 +89,7 @@ def test_kv_append2_and_decode_attention(F, X, D):
     rng = np.random.default_rng(2)
     # (14, 2, 64, [8192]): head_dim 64 with more than 64 splits of the key range (2 KV heads on 256 CUs), the case in which
     # the combine kernel's thread count and its loop stride have to agree
-    for nh, nkv, hd, lens in [(40, 8, 128, [1, 7, 64, 65, 383, 384, 385, 1000, 5120, 5121]), (8, 8, 64, [3, 257]), (16, 2, 128, [130]), (6, 2, 64, [33]), (5, 1, 128, [2049]),
+    for nh, nkv, hd, lens in [(40, 8, 128, [1, 7, 64, 65, 255, 256, 257, 384, 1000, 5120, 5121]), (8, 8, 64, [3, 257]), (16, 2, 128, [130]), (6, 2, 64, [33]), (5, 1, 128, [2049]),
                               (64, 8, 128, [4097]), (14, 2, 64, [8192])]:
         cap = max(lens) + 3
         width = nkv * hd
@@ -247,11 +247,12 @@ def test_post_processing_inside_the_attention_launch(F, X, D):
              (4, 2, 64, 300, 120, False, True, False, 0, 0.0), (6, 3, 128, 2100, 2099, True, True, True, 0, 0.0),
              (8, 8, 64, 90, 89, False, False, False, 0, 0.0), (12, 4, 128, 1500, 1499, True, False, False, 256, 0.0),
              (10, 2, 128, 513, 512, True, True, False, 0, 30.0), (2, 1, 128, 1, 0, True, False, False, 0, 0.0),
-             # caches of up to 384 rows under grouped query heads: one workgroup per query head, each of a KV head's workgroups
+             # caches of up to 256 rows under grouped query heads: one workgroup per query head, each of a KV head's workgroups
              # appending the same rows; the first key step requested ahead of the post-processing (position past the first 32
              # rows) or behind the append (position among them); the first length past that launch shape
-             (40, 8, 128, 384, 383, True, True, False, 0, 0.0), (14, 2, 64, 300, 20, True, False, True, 0, 0.0),
-             (14, 2, 64, 300, 299, True, False, True, 64, 0.0), (40, 8, 128, 385, 384, True, False, False, 0, 0.0)]
+             (40, 8, 128, 256, 255, True, True, False, 0, 0.0), (14, 2, 64, 200, 20, True, False, True, 0, 0.0),
+             (14, 2, 64, 200, 199, True, False, True, 64, 0.0), (40, 8, 128, 257, 256, True, False, False, 0, 0.0),
+             (14, 2, 64, 300, 20, True, False, True, 0, 0.0), (40, 8, 128, 5120, 5119, True, False, False, 0, 0.0)]
     for nh, nkv, hd, cap, pos, use_norm, use_bias, inter, window, softcap in cases:
         width = (nh + 2 * nkv) * hd
         qkv = rng.standard_normal(width).astype(np.float32)
