@@ -349,8 +349,9 @@ int fhip_decode_attention_ex(const float* d_q, const float* d_k_cache, const flo
 
 /* fhip_qkv_post and fhip_decode_attention_ex for ONE new token in one launch (crates/ferric-llama/src/qwen3.rs:861-905 followed
  * by crates/ferric-tensor/src/nn.rs:140-166): every attention workgroup forms its own query heads from the raw QKV row
- * [(n_head + 2 n_kv) * head_dim] (bias, per-head RMSNorm, rotation at *d_pos), and the workgroup whose keys include position
- * *d_pos forms and appends that token's K and V rows before it reads them back. Attention is over rows [0, min(*d_pos + 1,
+ * [(n_head + 2 n_kv) * head_dim] (bias, per-head RMSNorm, rotation at *d_pos), and the workgroups whose keys include position
+ * *d_pos (one, or one per query head of the KV head) form and append that token's K and V rows, the same bits from each,
+ * before they read them back. Attention is over rows [0, min(*d_pos + 1,
  * len)) of the caches; `len` (at most cap) is the host-side upper bound that sizes the launch, as in fhip_decode_attention.
  * d_ws: fhip_decode_attention_ws_bytes(n_head, n_kv, head_dim, len) bytes. Same results as the two calls. */
 int fhip_qkv_post_attention(const float* d_qkv, const float* d_bias, const float* d_q_norm, const float* d_k_norm, const uint32_t* d_pos,
