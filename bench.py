@@ -34,12 +34,28 @@ Q8_0, Q4_K, Q6_K = 8, 12, 14
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "gemv_q4k_5120x5120_hbm_traffic.json")
 
 
+def kernel_source_sha():
+    """sha256 (first 16 hex digits) of the streaming mat-vec's source: counter summaries carry it, so a summary taken on other
+    code than the one that runs can be told."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in ("gemv.hip", "common.hpp", "deq_at.hpp"):
+        with open(os.path.join(ROOT, "ferric_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def headline_traffic():
+    """The counter summary of the headline kernel; `stale` says that the kernel's source has changed since it was taken."""
     try:
         with open(TRAFFIC_JSON) as f:
-            return json.load(f)
+            t = json.load(f)
     except (OSError, ValueError):
         return None
+    t["stale"] = t.get("kernel_source_sha16") != kernel_source_sha()
+    if t["stale"]:
+        log("[bench] WARNING: profiles/gemv_q4k_5120x5120_hbm_traffic.json was measured on other kernel source than this tree holds")
+    return t
 
 
 def log(*a):
@@ -115,12 +131,15 @@ def rotating_graphs(make, steps, ncopy):
     return [make(j * steps) for j in range(n)]
 
 
-def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed, x_seed, ncopy, cold_only=False, with_reader=False):
+def bench_gemv(F, lib, check, stream, timer, ty, rows, cols, steps, warmup, seed, x_seed, ncopy, cold_only=False, with_reader=False, bits=None):
     from ferric_amd.synth import synth_weights
     nbytes = weight_bytes(ty, rows, cols)
     host = synth_weights(ty, rows, cols, seed)
     buf = replicate(F, lib, check, host, ncopy)
     ws = [F.QMatrix.wrap_device(buf, nbytes, ty, rows, cols, offset=i * nbytes) for i in range(ncopy)]
+    if bits:                                                   # activation precision of these handles (a new handle has 24 bits)
+        for w in ws:
+            w.matvec_precision(bits)
     x = F.Tensor.from_vec(np.random.default_rng(x_seed).standard_normal(cols).astype(np.float32), (1, cols))
     y = F.Tensor.empty((1, rows))
     alg = nbytes + 4 * cols + 4 * rows
@@ -166,9 +185,9 @@ def bench_q80_batch(F, lib, check, stream, timer, rows=4096, cols=4096, batch=8,
     # the drop-in entry point takes the same kernels for this batch, out of the library's workspace
     check(lib.fhip_workspace_reserve(stream.handle, lib.fhip_workspace_bytes(ws[0].handle, None, batch)))
     drop_in = timed(lambda w: check(lib.fhip_matmul_q(w.handle, x.buf.ptr, batch, y.buf.ptr, stream.handle)))
-    before = lib.fhip_batch_policy(1)                  # FHIP_BATCH_F32_MATVEC
+    for w in ws:
+        w.batch_policy(1)                              # FHIP_BATCH_F32_MATVEC
     per_row = timed(lambda w: check(lib.fhip_matmul_q(w.handle, x.buf.ptr, batch, y.buf.ptr, stream.handle)))
-    lib.fhip_batch_policy(before)
     return {"batch": batch, "matmul_q_us": drop_in, "matmul_q_weight_GBps": nbytes / drop_in / 1e3, "f16x2_us": one_pass,
             "f32_matvec_policy_us": per_row}
 
@@ -222,11 +241,14 @@ def bench_ffn(F, lib, check, stream, timer, batches, reps=20, ncopy=4):
         f32 = lambda gu, dn: check(lib.fhip_ffn(gu.handle, dn.handle, x.buf.ptr, b, y.buf.ptr, ws.buf.ptr, stream.handle))
         res[str(b)] = entry(timed(f32, ncopy), b)
         res[str(b)]["warm_one_copy_ms"] = timed(f32, 1)
-        res[str(b)]["path"] = "streaming mat-vec" if b <= 2 else "one-pass f16 hi/lo matrix-core kernels"
+        res[str(b)]["path"] = "streaming mat-vec" if b <= 2 else "one-pass f16 hi/lo matrix-core kernels, cut rows added in a fixed order (FHIP_BATCH_ORDERED)"
         if b > 2:
-            before = lib.fhip_batch_policy(1)          # FHIP_BATCH_F32_MATVEC: two rows per pass over the weights
-            res[str(b)]["f32_matvec_policy"] = entry(timed(f32, ncopy), b)
-            lib.fhip_batch_policy(before)
+            for policy, key in ((0, "atomic_adds_policy"), (1, "f32_matvec_policy")):   # FHIP_BATCH_AUTO, FHIP_BATCH_F32_MATVEC
+                for w in gus + dns:
+                    w.batch_policy(policy)
+                res[str(b)][key] = entry(timed(f32, ncopy), b)
+            for w in gus + dns:
+                w.batch_policy(2)
         # the same block through the matrix-core entry point (bf16 operands, f32 accumulate): one pass over
         # the weights for the whole batch
         wsb = F.DeviceBuffer(max(256, lib.fhip_ffn_coop_ws_bytes(gus[0].handle, dns[0].handle, b)))
@@ -331,7 +353,10 @@ def bench_gguf(F, lib, check, n_tensors=8, rows=11008, cols=5120):
 
 def bench_sweep(F, lib, check, stream, timer, tokens=4, layers=64):
     """The decode weight sweep: per layer fused QKV 5120->7168, O 5120->5120, fused gate+up 5120->34816 (+SwiGLU), all Q4_K,
-    down 17408->5120 Q6_K; lm_head 5120->151936 Q6_K. One stream, one graph of layers*4+1 launches."""
+    down 17408->5120 Q6_K; lm_head 5120->151936 Q6_K. One stream, one graph of layers*4+1 launches. Measured three ways:
+    every op on a fixed activation vector with the handles at 16-bit activations (`ms_per_token`, as the headline) and at the
+    24 bits a handle has unless told otherwise (`ms_per_token_x24`), and as a true chain in which every op reads what the op before it wrote, held finite by the
+    RMS norms fused into the QKV and gate|up mat-vecs (`chained`)."""
     from ferric_amd.synth import synth_weights
     shapes = [("qkv", Q4_K, 7168, 5120), ("o", Q4_K, 5120, 5120), ("gate_up", Q4_K, 34816, 5120), ("down", Q6_K, 5120, 17408)]
     host = {n: synth_weights(ty, r, c, 40 + i) for i, (n, ty, r, c) in enumerate(shapes)}
@@ -350,35 +375,146 @@ def bench_sweep(F, lib, check, stream, timer, tokens=4, layers=64):
     for n, ty, r, c in shapes:
         nb = host[n].size
         W[n] = [F.QMatrix.wrap_device(stacks[n], nb, ty, r, c, offset=l * nb) for l in range(layers)]
-    g = F.Graph.begin(stream)
     s = stream.handle
-    for l in range(layers):
-        check(lib.fhip_matmul_q(W["qkv"][l].handle, x.buf.ptr, 1, y_qkv.buf.ptr, s))
-        check(lib.fhip_matmul_q(W["o"][l].handle, x.buf.ptr, 1, y_o.buf.ptr, s))
-        check(lib.fhip_matmul_q_swiglu(W["gate_up"][l].handle, x.buf.ptr, 1, y_ff.buf.ptr, s))
-        check(lib.fhip_matmul_q(W["down"][l].handle, h.buf.ptr, 1, y_dn.buf.ptr, s))
-    check(lib.fhip_matmul_q(head.handle, x.buf.ptr, 1, logits.buf.ptr, s))
-    g.end()
-    g.launch()
-    ts = sorted(timer.time_ms(lambda: [g.launch() for _ in range(tokens)]) / tokens for _ in range(5))
-    ms = ts[len(ts) // 2]
+
+    def timed(record):
+        g = F.Graph.begin(stream)
+        record()
+        g.end()
+        g.launch()
+        ts = sorted(timer.time_ms(lambda: [g.launch() for _ in range(tokens)]) / tokens for _ in range(5))
+        return ts[len(ts) // 2], ts
+
+    def fixed_inputs():
+        for l in range(layers):
+            check(lib.fhip_matmul_q(W["qkv"][l].handle, x.buf.ptr, 1, y_qkv.buf.ptr, s))
+            check(lib.fhip_matmul_q(W["o"][l].handle, x.buf.ptr, 1, y_o.buf.ptr, s))
+            check(lib.fhip_matmul_q_swiglu(W["gate_up"][l].handle, x.buf.ptr, 1, y_ff.buf.ptr, s))
+            check(lib.fhip_matmul_q(W["down"][l].handle, h.buf.ptr, 1, y_dn.buf.ptr, s))
+        check(lib.fhip_matmul_q(head.handle, x.buf.ptr, 1, logits.buf.ptr, s))
+
+    def set_bits(bits):
+        for ws in W.values():
+            for w in ws:
+                w.matvec_precision(bits)
+        head.matvec_precision(bits)
+
+    per_bits = {}
+    for bits in (24, 16):
+        set_bits(bits)
+        per_bits[bits] = timed(fixed_inputs)
+    ms, ts = per_bits[16]
+    # The chain: x -> norm+QKV -> O (on the first 5120 of the QKV row) -> norm+gate|up+SwiGLU -> down -> next layer; the
+    # head's norm is a launch of its own (a weight of that size is not fused). 16-bit activations, as ms_per_token.
+    norm_w = F.Tensor.from_vec(((rng.random(5120) + 0.5) * 0.01).astype(np.float32), (1, 5120))
+    scratch, dn2 = F.Tensor.empty((1, 5120)), [F.Tensor.empty((1, 5120)) for _ in range(2)]
+
+    def chained():
+        cur = x
+        for l in range(layers):
+            check(lib.fhip_norm_matmul_q(W["qkv"][l].handle, cur.buf.ptr, None, norm_w.buf.ptr, 1e-6, None, scratch.buf.ptr, 0, y_qkv.buf.ptr, s))
+            check(lib.fhip_matmul_q(W["o"][l].handle, y_qkv.buf.ptr, 1, y_o.buf.ptr, s))
+            check(lib.fhip_norm_matmul_q(W["gate_up"][l].handle, y_o.buf.ptr, None, norm_w.buf.ptr, 1e-6, None, scratch.buf.ptr, 1, y_ff.buf.ptr, s))
+            check(lib.fhip_matmul_q(W["down"][l].handle, y_ff.buf.ptr, 1, dn2[l % 2].buf.ptr, s))
+            cur = dn2[l % 2]
+        check(lib.fhip_norm_matmul_q(head.handle, cur.buf.ptr, None, norm_w.buf.ptr, 1e-6, None, scratch.buf.ptr, 0, logits.buf.ptr, s))
+    ms_chain, _ = timed(chained)
+    finite = bool(np.isfinite(logits.to_vec(stream)).all())
     # The same 257 launches with a kernel that only reads each weight's bytes (fhip_debug_read_probe): what this device gives
     # a sweep cut into these launches when no arithmetic, staging or reduction stands in the way.
     sink = F.DeviceBuffer(256)
-    gr = F.Graph.begin(stream)
-    for l in range(layers):
-        for n, _, _, _ in shapes:
-            check(lib.fhip_debug_read_probe(C.c_void_p(stacks[n].ptr.value + l * host[n].size), host[n].size, sink.ptr, s))
-    check(lib.fhip_debug_read_probe(head_buf.ptr, head_bytes, sink.ptr, s))
-    gr.end()
-    gr.launch()
-    tr = sorted(timer.time_ms(lambda: [gr.launch() for _ in range(tokens)]) / tokens for _ in range(5))
-    floor_ms = tr[len(tr) // 2]
-    return {"ms_per_token": ms, "ms_per_token_min_max": [ts[0], ts[-1]], "GBps": total / (ms * 1e-3) / 1e9, "frac_of_peak": total / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-            "reader_floor_ms": floor_ms, "reader_floor_GBps": total / (floor_ms * 1e-3) / 1e9, "frac_of_reader": floor_ms / ms,
+
+    def readers():
+        for l in range(layers):
+            for n, _, _, _ in shapes:
+                check(lib.fhip_debug_read_probe(C.c_void_p(stacks[n].ptr.value + l * host[n].size), host[n].size, sink.ptr, s))
+        check(lib.fhip_debug_read_probe(head_buf.ptr, head_bytes, sink.ptr, s))
+    floor_ms, _ = timed(readers)
+    gbps = lambda t: total / (t * 1e-3) / 1e9
+    return {"ms_per_token": ms, "ms_per_token_min_max": [ts[0], ts[-1]], "GBps": gbps(ms), "frac_of_peak": gbps(ms) / HBM_PEAK_GBPS, "activation_bits": 16,
+            "ms_per_token_x16": ms,
+            "ms_per_token_x24": per_bits[24][0], "GBps_x24": gbps(per_bits[24][0]), "frac_of_peak_x24": gbps(per_bits[24][0]) / HBM_PEAK_GBPS,
+            "chained": {"ms_per_token": ms_chain, "GBps": gbps(ms_chain), "launches_per_token": layers * 4 + 2, "logits_finite": finite,
+                        "what": "every op reads the op before it: x -> norm+QKV -> O -> norm+gate|up+SwiGLU -> down -> next layer; norm launch + lm_head"},
+            "reader_floor_ms": floor_ms, "reader_floor_GBps": gbps(floor_ms), "frac_of_reader": floor_ms / ms,
             "weight_bytes": total, "layers": layers, "launches_per_token": layers * 4 + 1,
-            "inputs": "fixed N(0,1) activations per op (outputs are not fed forward, so values stay finite); "
-                      "ops still execute in stream order"}
+            "inputs": "fixed N(0,1) activations per op for ms_per_token (outputs are not fed forward, so values stay finite); "
+                      "ops still execute in stream order; `chained` feeds every op the output of the one before"}
+
+
+def bench_marginal(F, lib, check, stream, timer, sizes=(5120, 20480, 81920, 327680), cols=5120):
+    """Time against bytes for Q4_K weights of `cols` columns, one activation row, cold: a least-squares line through the launch
+    times of four weight sizes gives what a launch costs whatever its size (`fixed_us`) and the rate at which every further
+    byte moves (`marginal_GBps`) -- the reference's own model of a mat-vec call (crates/ferric-tensor/examples/matvec_roofline.rs:37-41).
+    The same for the kernel that only reads. Every size rotates over copies that add up to 0.9 GB or more."""
+    from ferric_amd.synth import synth_weights
+    unit_rows = sizes[0]
+    unit = weight_bytes(Q4_K, unit_rows, cols)
+    ncopy = max(64, 2 * sizes[-1] // unit_rows)
+    buf = replicate(F, lib, check, synth_weights(Q4_K, unit_rows, cols, 1), ncopy)     # big weights are runs of the small one's rows
+    x = F.Tensor.from_vec(np.random.default_rng(2).standard_normal(cols).astype(np.float32), (1, cols))
+    y = F.Tensor.empty((1, sizes[-1]))
+    sink = F.DeviceBuffer(256)
+    pts = []
+    for rows in sizes:
+        per = rows // unit_rows
+        n = ncopy // per
+        ws = [F.QMatrix.wrap_device(buf, unit * per, Q4_K, rows, cols, offset=i * unit * per) for i in range(n)]
+        for w in ws:
+            w.matvec_precision(16)                                # as the headline
+        launches = max(n, 8)
+        g = F.Graph.begin(stream)
+        for i in range(launches):
+            check(lib.fhip_matmul_q(ws[i % n].handle, x.buf.ptr, 1, y.buf.ptr, stream.handle))
+        g = g.end()
+        gr = F.Graph.begin(stream)
+        for i in range(launches):
+            check(lib.fhip_debug_read_probe(C.c_void_p(buf.ptr.value + (i % n) * unit * per), unit * per, sink.ptr, stream.handle))
+        gr = gr.end()
+        t = time_per_launch(timer, [g], launches, min_launches=max(launches, 256 // per), batches=5) * 1e3
+        tr = time_per_launch(timer, [gr], launches, min_launches=max(launches, 256 // per), batches=5) * 1e3
+        pts.append({"rows": rows, "bytes": unit * per, "us": t, "reader_us": tr})
+        del ws
+
+    def fit(key):
+        bx = np.array([p["bytes"] for p in pts], np.float64)
+        ty = np.array([p[key] for p in pts], np.float64)
+        slope, icept = np.polyfit(bx, ty, 1)                      # us per byte, us
+        return {"fixed_us": float(icept), "marginal_GBps": float(1e-3 / slope), "marginal_frac_of_peak": float(1e-3 / slope / HBM_PEAK_GBPS)}
+    return {"points": pts, "mat_vec": fit("us"), "reader": fit("reader_us"), "activation_bits": 16,
+            "what": f"Q4_K, {cols} columns, batch 1, cold; time = fixed_us + bytes / marginal rate (least squares over the four sizes)"}
+
+
+def bench_other_shapes(F, lib, check, stream, timer):
+    """Cold launch times of the weight shapes of other models that the launch policy was tuned on (besides the benchmark's own):
+    a retune that helps one set and hurts the other shows here. `cold_us`: handles at 16-bit activations, as the headline;
+    `cold_us_x24`: as the library makes them."""
+    from ferric_amd.synth import synth_weights
+    shapes = [("q4_k 8192x8192", Q4_K, 8192, 8192, 0), ("q4_k 10240x8192", Q4_K, 10240, 8192, 0), ("q4_k gate|up 57344x8192", Q4_K, 57344, 8192, 1),
+              ("q4_k 28672x4096", Q4_K, 28672, 4096, 0), ("q4_k gate|up 22016x4096", Q4_K, 22016, 4096, 1), ("q4_k 4096x4096", Q4_K, 4096, 4096, 0),
+              ("q4_k 20480x5120", Q4_K, 20480, 5120, 0), ("q6_k 5120x5120", Q6_K, 5120, 5120, 0), ("q6_k 4096x4096", Q6_K, 4096, 4096, 0),
+              ("q6_k 4096x14336", Q6_K, 4096, 14336, 0), ("q6_k 8192x28672", Q6_K, 8192, 28672, 0), ("q6_k 128256x4096", Q6_K, 128256, 4096, 0),
+              ("q8_0 12288x4096", Q8_0, 12288, 4096, 0), ("q5_k 5120x5120", 13, 5120, 5120, 0)]
+    out = {}
+    for name, ty, rows, cols, swiglu in shapes:
+        nb = weight_bytes(ty, rows, cols)
+        ncopy = max(2, min(48, -(-(600 << 20) // nb)))
+        small = synth_weights(ty, min(rows, 2048), cols, 90)       # rows repeat: the values do not matter for timing
+        host = np.tile(small, -(-rows // min(rows, 2048)))[:nb]
+        buf = replicate(F, lib, check, host, ncopy)
+        ws = [F.QMatrix.wrap_device(buf, nb, ty, rows, cols, offset=i * nb) for i in range(ncopy)]
+        x = F.Tensor.from_vec(np.random.default_rng(2).standard_normal(cols).astype(np.float32), (1, cols))
+        y = F.Tensor.empty((1, rows))
+        launches = max(ncopy, 16)
+        g = gemv_graph(F, lib, check, stream, ws, x, y, launches, swiglu=bool(swiglu))
+        us24 = time_per_launch(timer, [g], launches, min_launches=128, batches=5) * 1e3
+        for w in ws:
+            w.matvec_precision(16)
+        g = gemv_graph(F, lib, check, stream, ws, x, y, launches, swiglu=bool(swiglu))
+        us = time_per_launch(timer, [g], launches, min_launches=128, batches=5) * 1e3
+        out[name] = {"cold_us": us, "weight_GBps": nb / us / 1e3, "cold_us_x24": us24}
+        del ws, buf
+    return out
 
 
 def decode_stack(F, lib, check, layers=64):
@@ -833,37 +969,53 @@ def main():
         probe_step(F, lib, check)
         return
     log("[bench] Q4_K GEMV 5120x5120 ...")
+    # `value`: handles switched to 16-bit activations (QMatrix.matvec_precision(16)): inside the benchmark's tolerance
+    # 1e-3 * ||w_row|| * ||x|| by three orders of magnitude, but not inside the 1e-5 of the reference's own examples. A handle as
+    # the library makes it computes at 24 bits (the f32 significand, which those examples pass): `value_x24` beside it.
     c2, alg, nbytes = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64,
-                                 cold_only=args.headline_only, with_reader=True)
+                                 cold_only=args.headline_only, with_reader=True, bits=16)
+    x24 = None
     if args.headline_only:
         args.no_q8 = args.no_ffn = args.no_prefill = args.no_moe = args.no_sweep = args.no_cpu = args.no_decode = True
         c2["warm"] = None
+    else:
+        x24, _, _ = bench_gemv(F, lib, check, stream, timer, Q4_K, rows, cols, args.steps, args.warmup, seed=1, x_seed=2, ncopy=64, bits=24)
     ms_step = c2["cold"]["ms_per_step"]
     value = c2["cold"]["GBps"]
     traffic = headline_traffic()
-    bits = lib.fhip_matvec_precision(0)
     line = {
         "metric": "Q4_K GEMV HBM GB/s (% of 8 TB/s) at batch 1; decode-step weight-sweep ms",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32 in / f32 out; weights Q4_K exact; activations inside the kernel: 16-bit block fixed point per 32 columns (opt-in; "
+                 "a new handle has 24-bit: value_x24), integer dot products per sub-block, f32 accumulation above it",
+        "data": "synthetic",
         "config": {"workload": "Q4_K GEMV batch 1, W 5120x5120 (14745600 B raw GGUF blocks), x f32[5120]; "
                                "64 distinct weight copies rotated (944 MB > 256 MB Infinity Cache) so each step reads HBM",
                    "rows": rows, "cols": cols, "batch": 1, "weight_copies": 64},
         "pct_of_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "value_x16": value, "us_x16": ms_step * 1e3,
+        "value_x24": x24["cold"]["GBps"] if x24 else None, "us_x24": x24["cold"]["ms_per_step"] * 1e3 if x24 else None,
         "warm_single_copy": c2["warm"],
         "roofline": {"bound": "hbm", "achieved": alg / (ms_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": alg / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                      "traffic": traffic.get("hbm_bytes_per_launch") if traffic else None, "traffic_source": traffic,
-                     "kernel": "gemv_stream_kernel<Q4K, M=1, plain>", "algorithmic_bytes_per_launch": alg,
+                     "kernel": "gemv_stream_kernel<Q4K, M=1, plain>, two activation planes (16-bit)", "algorithmic_bytes_per_launch": alg,
                      "launch_us": ms_step * 1e3,
                      # the same 14.7 MB through a kernel that only reads them (same rotation, same timing), and a launch
                      # that does nothing: what this box leaves a single cold launch of this size
                      "reader_floor_us": c2["reader_ms"] * 1e3, "frac_of_reader": c2["reader_ms"] / ms_step,
                      "empty_launch_us": launch_floor_us(F, lib, check, stream, timer)},
-        "activation_bits": bits,
+        "activation_bits": 16,
         "timing": "median of 9 batches; a batch = the K-step graph(s) replayed back to back until >= 1024 launches, one HIP event pair",
     }
+    if not args.headline_only:
+        log("[bench] time against bytes (fixed cost and marginal rate) ...")
+        fit = bench_marginal(F, lib, check, stream, timer)
+        line["roofline"]["marginal_GBps"] = fit["mat_vec"]["marginal_GBps"]
+        line["roofline"]["marginal_frac"] = fit["mat_vec"]["marginal_frac_of_peak"]
+        line["roofline"]["fixed_us"] = fit["mat_vec"]["fixed_us"]
+        line["roofline"]["time_vs_bytes"] = fit
     if not args.no_q8:
         log("[bench] Q8_0 GEMV 4096x4096 ...")
         c1, alg1, _ = bench_gemv(F, lib, check, stream, timer, Q8_0, 4096, 4096, args.steps, args.warmup, seed=0, x_seed=0, ncopy=56)
@@ -896,6 +1048,8 @@ def main():
     if not args.no_sweep:
         log("[bench] 64-layer decode weight sweep (14.0 GB) ...")
         line["decode_sweep"] = bench_sweep(F, lib, check, stream, timer)
+        log("[bench] weight shapes of other models ...")
+        line["other_model_shapes"] = bench_other_shapes(F, lib, check, stream, timer)
     if not args.no_decode:
         log("[bench] 64-layer decode step with attention (context 128 / 4096 / 32768) ...")
         line["decode_step_chained"] = bench_decode(F, lib, check, stream, timer)

@@ -112,6 +112,8 @@ SYMBOLS = {
     "fhip_debug_generic_matvec": (C.c_int, [C.c_int]),
     "fhip_debug_gemm_tile": (C.c_int, [C.c_int]),
     "fhip_matvec_precision": (C.c_int, [C.c_int]),
+    "fhip_weight_matvec_precision": (C.c_int, [_vp, C.c_int]),
+    "fhip_weight_batch_policy": (C.c_int, [_vp, C.c_int]),
     "fhip_ffn_noalloc": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _vp]),
     "fhip_batch_policy": (C.c_int, [C.c_int]),
     "fhip_workspace_bytes": (C.c_size_t, [_vp, _vp, C.c_size_t]),

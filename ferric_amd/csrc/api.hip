@@ -23,6 +23,9 @@ float* g_scratch_ptr[MAX_DEVICES] = {};
 
 thread_local char g_err[512] = "";
 int g_device = -1;
+// What a new weight handle starts with (fhip_matvec_precision, fhip_batch_policy); read when a handle is made, never at a launch.
+int g_default_planes = 3;
+int g_default_batch_policy = FHIP_BATCH_ORDERED;
 int g_cus = 0;
 size_t g_lds = 64 * 1024;
 
@@ -75,6 +78,7 @@ int make_weight(uint32_t ty, size_t nbytes, size_t rows, size_t cols, fhip_weigh
     if (nbytes != rows * row_bytes) return fhip::set_error(FHIP_ERR_SHAPE, "unexpected %s byte length", type_name(ty));
     if (rows > 0x7FFFFFFFull || cols > 0x7FFFFFFFull) return fhip::set_error(FHIP_ERR_SHAPE, "weight dimensions exceed 2^31");
     w.type = ty; w.rows = rows; w.cols = cols; w.row_bytes = row_bytes; w.nbytes = nbytes; w.d_raw = nullptr; w.owns = false;
+    w.planes = g_default_planes; w.batch_policy = g_default_batch_policy;
     return FHIP_OK;
 }
 
@@ -98,17 +102,15 @@ int check_hip(hipError_t e, const char* what) {
 int device_cus() { return g_cus; }
 size_t device_lds_bytes() { return g_lds; }
 
-// The streaming mat-vec exists in two copies, one per activation precision; these forward to the selected one.
-static int g_planes = 2;
-int matvec_planes() { return g_planes; }
+// The streaming mat-vec exists in two copies, one per activation precision; these forward to the one the weight names.
 int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s) {
-    return g_planes == 3 ? launch_gemv_p3(w, d_x, rows_x, d_y, n_ff, s) : launch_gemv_p2(w, d_x, rows_x, d_y, n_ff, s);
+    return w->planes == 3 ? launch_gemv_p3(w, d_x, rows_x, d_y, n_ff, s) : launch_gemv_p2(w, d_x, rows_x, d_y, n_ff, s);
 }
 int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s) {
-    return g_planes == 3 ? launch_gemv_norm_p3(w, d_x, d_y, n_ff, norm, s) : launch_gemv_norm_p2(w, d_x, d_y, n_ff, norm, s);
+    return w->planes == 3 ? launch_gemv_norm_p3(w, d_x, d_y, n_ff, norm, s) : launch_gemv_norm_p2(w, d_x, d_y, n_ff, norm, s);
 }
 int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu, const SelParams& sel, hipStream_t s) {
-    return g_planes == 3 ? launch_gemv_sel_p3(w, d_x, d_y, out_rows, swiglu, sel, s) : launch_gemv_sel_p2(w, d_x, d_y, out_rows, swiglu, sel, s);
+    return w->planes == 3 ? launch_gemv_sel_p3(w, d_x, d_y, out_rows, swiglu, sel, s) : launch_gemv_sel_p2(w, d_x, d_y, out_rows, swiglu, sel, s);
 }
 void gemv_force_generic(bool on) {
     gemv_force_generic_p2(on);
@@ -185,11 +187,10 @@ static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t,
 // (five for Q8_0) the f16 hi/lo matrix-core kernels read the weights once for up to 32 (Q8_0: 16) rows; longer batches are cut
 // into such groups. FHIP_BATCH_F32_MATVEC keeps every batch on the mat-vec kernel: a row then has the same bits whatever batch
 // it is part of.
-int g_batch_policy = FHIP_BATCH_AUTO;
 
 size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32; }
 bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
-    if (g_batch_policy == FHIP_BATCH_F32_MATVEC) return false;
+    if (w->batch_policy == FHIP_BATCH_F32_MATVEC) return false;
     if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0) return false;
     if (rows_x < (w->type == FHIP_Q8_0 ? 5u : 3u)) return false;
     return fhip::gemm_f16x2_supports(w, rows_x < f16x2_group(w) ? rows_x : f16x2_group(w));
@@ -198,18 +199,18 @@ bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
 // y [t, rows] = 0 on the stream, by the mat-vec launcher's fill kernel (what a weight without columns gives)
 int zero_outputs(size_t t, size_t rows, float* d_y, hipStream_t s) {
     fhip_weight z{};
-    z.type = FHIP_Q8_0; z.rows = rows; z.cols = 0;
+    z.type = FHIP_Q8_0; z.rows = rows; z.cols = 0; z.planes = 2;
     return fhip::launch_gemv(&z, d_y, t, d_y, 0, s);
 }
 
 // y [t, w->rows] = x [t, cols] W^T for t rows of one group; ws: f16x2_matmul_ws(w, t) bytes
 // (FHIP_BATCH_ORDERED: behind the prepared activations, the partial sums of the groups the launch cuts along K)
 size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) {
-    return align256(fhip::gemm_f16x2_xp_bytes(w, t)) + (g_batch_policy == FHIP_BATCH_ORDERED ? align256(fhip::gemm_f16x2_part_bytes_upto(w, t)) : 0);
+    return align256(fhip::gemm_f16x2_xp_bytes(w, t)) + (w->batch_policy == FHIP_BATCH_ORDERED ? align256(fhip::gemm_f16x2_part_bytes_upto(w, t)) : 0);
 }
 int f16x2_matmul(const fhip_weight* w, const float* d_x, size_t t, bool swiglu_in, float* d_y, void* d_ws, hipStream_t s) {
     uint16_t* xp = (uint16_t*)d_ws;
-    const bool ordered = g_batch_policy == FHIP_BATCH_ORDERED;
+    const bool ordered = w->batch_policy == FHIP_BATCH_ORDERED;
     float* part = ordered && fhip::gemm_f16x2_part_bytes(w, t) ? (float*)((uint8_t*)d_ws + align256(fhip::gemm_f16x2_xp_bytes(w, t))) : nullptr;
     const bool clr = !part && fhip::gemm_f16x2_adds_into_y(w, t);   // then the split clears y on the side
     int rc = fhip::launch_xsplit_f16(w, d_x, t, swiglu_in, xp, s, clr ? d_y : nullptr, clr ? t * w->rows : 0);
@@ -638,9 +639,27 @@ int fhip_ffn_noalloc(const fhip_weight* gu, const fhip_weight* down, const float
     return fhip::launch_gemv(down, h, rows_x, d_y, 0, s);
 }
 
+static bool known_policy(int policy) { return policy == FHIP_BATCH_AUTO || policy == FHIP_BATCH_F32_MATVEC || policy == FHIP_BATCH_ORDERED; }
+
 int fhip_batch_policy(int policy) {
-    const int before = g_batch_policy;
-    if (policy == FHIP_BATCH_AUTO || policy == FHIP_BATCH_F32_MATVEC || policy == FHIP_BATCH_ORDERED) g_batch_policy = policy;
+    const int before = g_default_batch_policy;
+    if (known_policy(policy)) g_default_batch_policy = policy;
+    return before;
+}
+
+int fhip_weight_batch_policy(fhip_weight* w, int policy) {
+    if (!w) return set_error(FHIP_ERR_ARG, "fhip_weight_batch_policy: NULL weight");
+    const int before = w->batch_policy;
+    if (known_policy(policy)) w->batch_policy = policy;
+    return before;
+}
+
+int fhip_weight_matvec_precision(fhip_weight* w, int bits) {
+    if (!w) return set_error(FHIP_ERR_ARG, "fhip_weight_matvec_precision: NULL weight");
+    const int before = w->planes == 3 ? 24 : 16;
+    if (bits == 0) return before;
+    if (bits != 16 && bits != 24) return set_error(FHIP_ERR_ARG, "fhip_weight_matvec_precision: 16 or 24 bits (0 to query), not %d", bits);
+    w->planes = bits == 24 ? 3 : 2;
     return before;
 }
 
@@ -958,10 +977,10 @@ int fhip_debug_matmul_q_loop(const fhip_weight* const* ws, size_t n_weights, siz
 }
 
 int fhip_matvec_precision(int bits) {
-    const int before = fhip::g_planes == 3 ? 24 : 16;
+    const int before = g_default_planes == 3 ? 24 : 16;
     if (bits == 0) return before;
     if (bits != 16 && bits != 24) return set_error(FHIP_ERR_ARG, "fhip_matvec_precision: 16 or 24 bits (0 to query), not %d", bits);
-    fhip::g_planes = bits == 24 ? 3 : 2;
+    g_default_planes = bits == 24 ? 3 : 2;
     return before;
 }
 

@@ -14,6 +14,10 @@ struct fhip_weight {
     size_t nbytes;      // rows * row_bytes
     const uint8_t* d_raw;  // raw GGUF block stream in HBM
     bool owns;          // allocated by fhip_weight_create (freed on destroy)
+    // How launches on this weight compute, fixed when the handle is made (from the process defaults of that moment) and
+    // changed only through the handle's own setters: launches on other handles never see it.
+    int planes;         // activation planes of its streaming mat-vec: 3 = 24-bit (the f32 significand), 2 = 16-bit
+    int batch_policy;   // FHIP_BATCH_*: which kernels its batches of three rows and more take
 };
 
 namespace fhip {
@@ -70,9 +74,8 @@ int launch_dequant(uint32_t type, const uint8_t* d_raw, size_t nblocks, float* d
 // y[rows_x, n_ff] = silu(gate.x) * (up.x).
 int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 // gemv.hip is built once per activation precision (two or three byte planes per run: a 16- or 24-bit significand at the run
-// maximum); launch_gemv, launch_gemv_norm, launch_gemv_sel and gemv_force_generic (api.hip) forward to the copy
-// matvec_planes() names.
-int matvec_planes();
+// maximum); launch_gemv, launch_gemv_norm, launch_gemv_sel and gemv_force_generic (api.hip) forward to the copy the weight's
+// `planes` names.
 #define FHIP_GEMV_COPY(sfx)                                                                                                         \
     int launch_gemv##sfx(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);            \
     int launch_gemv_norm##sfx(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const struct NormParams& norm,        \

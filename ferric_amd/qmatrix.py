@@ -21,6 +21,7 @@ from . import _lib
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 Q4_0, Q4_1, Q5_0, Q5_1, Q5_K = 2, 3, 6, 7, 13   # further formats: unpackers, mat-vec / small batch, "_id" variants
 IQ4_NL, IQ4_XS, MXFP4 = 20, 23, 39             # codebook / microscaling formats, same coverage
+BATCH_AUTO, BATCH_F32_MATVEC, BATCH_ORDERED = 0, 1, 2   # QMatrix.batch_policy
 F32, F16, BF16 = 0, 1, 30                      # unquantized tensor types: type_size and deq_raw only (lib.rs:473-475, 499-501)
 
 
@@ -482,6 +483,19 @@ class QMatrix:
 
     def n_shards(self):
         return 1  # one HBM allocation holds any size; the reference shards only for WebGPU binding limits
+
+    def matvec_precision(self, bits=0):
+        """Activation bits of this weight's streaming mat-vec: 24 (what a new weight has: the f32 significand, the reference
+        examples' 1e-5 bar) or 16 (faster, about 1e-4); 0 only queries. Returns the setting before the call."""
+        rc = _lib.load().fhip_weight_matvec_precision(self.handle, bits)
+        if rc < 0:
+            _lib.check(rc)
+        return rc
+
+    def batch_policy(self, policy=-1):
+        """Which kernels this weight's batches of three rows and more take (BATCH_ORDERED, what a new weight has, BATCH_AUTO or
+        BATCH_F32_MATVEC); any other value only queries. Returns the policy before the call."""
+        return _lib.load().fhip_weight_batch_policy(self.handle, policy)
 
     def dequant_rows(self, row0, nrows, stream=None):
         """Rows [row0, row0+nrows) dequantized on the GPU, bit-exact with deq_raw."""

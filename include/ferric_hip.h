@@ -377,18 +377,25 @@ int fhip_norm_matmul_q(const fhip_weight* w, const float* d_x, const float* d_re
  * calls that overlap in time on one GPU (two streams, two threads) race on it. It has no counterpart in the reference. */
 int fhip_ffn_noalloc(const fhip_weight* gate_up, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y, void* stream);
 
-/* Which kernel fhip_matmul_q, fhip_matmul_q_swiglu and fhip_ffn give a batch of three rows or more. FHIP_BATCH_AUTO (the
- * default): the one-pass matrix-core kernels as described at fhip_matmul_q. FHIP_BATCH_F32_MATVEC: the streaming mat-vec, two
- * rows per pass over the weights; an output row then has the same bits whatever batch it was part of (the guarantee the
- * reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200), at the price of rows_x / 2 passes.
- * FHIP_BATCH_ORDERED: the one-pass kernels of FHIP_BATCH_AUTO, but where a launch cuts a weight row's columns between
- * workgroups the pieces go to the library workspace (fhip_workspace_bytes counts them) and one more launch adds them in a
- * fixed order instead of f32 atomic adds: the same call on the same inputs then returns the same bits on every run, for a
- * few microseconds per matmul. Returns the policy before the call; any other value only queries. Process-wide, as
- * fhip_matvec_precision; set it before sizing or reserving the workspace. */
+/* Which kernels a weight's batches of three rows or more take in fhip_matmul_q, fhip_matmul_q_swiglu and fhip_ffn. It is a
+ * property of the weight handle (the reference's QMatrix is immutable after from_bytes, crates/ferric-tensor/src/dtype.rs:865-931;
+ * so is this handle as far as launches go: nothing process-wide is read when a launch is enqueued).
+ * FHIP_BATCH_ORDERED (what a new handle starts with): the one-pass matrix-core kernels described at fhip_matmul_q; where a
+ * launch cuts a weight row's columns between workgroups the pieces go to the library workspace (fhip_workspace_bytes counts
+ * them) and one more launch adds them in a fixed order, so the same call on the same inputs returns the same bits on every run.
+ * FHIP_BATCH_AUTO: the same kernels with the pieces added by f32 atomics instead: a few microseconds per matmul faster, the
+ * last bits vary from run to run (within 2e-6 of the largest output).
+ * FHIP_BATCH_F32_MATVEC: the streaming mat-vec, up to four rows per pass over the weights; an output row then has the same
+ * bits whatever batch it was part of (the guarantee the reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200),
+ * at the price of rows_x / 4 (Q6_K: / 2) passes.
+ * fhip_weight_batch_policy sets one handle's policy and returns the one before; any value that is no policy only queries. Set it
+ * before sizing or reserving the workspace and not while another thread launches on the handle.
+ * fhip_batch_policy sets what handles made AFTERWARDS start with (existing handles keep theirs) and returns the previous
+ * default. */
 #define FHIP_BATCH_AUTO 0
 #define FHIP_BATCH_F32_MATVEC 1
 #define FHIP_BATCH_ORDERED 2
+int fhip_weight_batch_policy(fhip_weight* w, int policy);
 int fhip_batch_policy(int policy);
 
 /* The library's workspace of a stream (NULL: the default stream): device memory the batched paths of fhip_matmul_q,
@@ -430,11 +437,16 @@ int fhip_debug_matmul_q_loop(const fhip_weight* const* ws, size_t n_weights, siz
 /* Precision of the activations inside the streaming mat-vec kernels (fhip_matmul_q, _swiglu, fhip_ffn, the "_id" entry points,
  * fhip_norm_matmul_q): per run of 32 (16 for Q6_K) columns the activations are held as block fixed point with a `bits`-bit
  * significand at the run's largest magnitude, the weights exactly, the sums exactly, and everything above the sub-block in
- * f32. bits = 16 (the default): dot products within about 1e-4 of the largest output, three orders of magnitude inside
- * 1e-3 * ||w_row|| * ||x||. bits = 24: the significand of f32 itself, results within 1e-5 of the largest output (the bar of
- * the reference's scalar kernels, crates/ferric-tensor/examples/q4_k.rs:54), 1-6 % slower. bits = 0 only queries. Returns the
- * setting before the call (16 or 24), or FHIP_ERR_ARG. Process-wide; takes effect for launches enqueued afterwards, so do
- * not change it while another thread enqueues. The reference has no such switch: its kernels multiply f32 by f32. */
+ * f32. A property of the weight handle, like the batch policy.
+ * bits = 24 (what a new handle starts with): the significand of f32 itself, results within 1e-5 of the largest output -- the
+ * bar the reference's own examples hold its scalar kernels to (crates/ferric-tensor/examples/q4_k.rs:54, q6_k.rs:33,
+ * q8_0.rs:21), so a handle left alone passes them.
+ * bits = 16 (opt-in): dot products within about 1e-4 of the largest output, still three orders of magnitude inside
+ * 1e-3 * ||w_row|| * ||x||, but NOT inside the 1e-5 of those examples; 1-6 % faster.
+ * fhip_weight_matvec_precision sets one handle (bits = 0 only queries) and returns its setting before the call (16 or 24), or
+ * FHIP_ERR_ARG; not while another thread launches on the handle. fhip_matvec_precision sets what handles made AFTERWARDS start
+ * with and returns the previous default. The reference has no such switch: its kernels multiply f32 by f32. */
+int fhip_weight_matvec_precision(fhip_weight* w, int bits);
 int fhip_matvec_precision(int bits);
 
 /* words[i] += delta for n device u32 words: advances the position word(s) at the end of a captured decode step. */

@@ -39,12 +39,13 @@ def bits(a):
     return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
 
 
-# ---- precision of the streaming mat-vec's activations (fhip_matvec_precision): the tests of the mat-vec entry points run
-# once per setting. At 24 bits the dot products are held to the bar the reference's examples use for its scalar kernels
-# (1e-5 of the largest output, crates/ferric-tensor/examples/q4_k.rs:54); at 16 bits (the default) to 2e-4: a 16-bit
-# significand at the run maximum is 1.5e-5 of that maximum per activation, and the sum over a row measures 2e-5 .. 7e-5
-# of the largest output on these inputs. The north-star bound 1e-3 * ||w_row|| * ||x|| is asserted at both.
-_PRECISION = {"bits": 16}
+# ---- precision of the streaming mat-vec's activations (a property of the weight handle; fhip_matvec_precision sets what new
+# handles start with): the tests of the mat-vec entry points run once per setting, making their weights under it. At 24
+# bits (what a handle has unless told otherwise) the dot products are held to the bar the reference's examples use for its
+# scalar kernels (1e-5 of the largest output, crates/ferric-tensor/examples/q4_k.rs:54); at 16 bits (opt-in) to 2e-4: a
+# 16-bit significand at the run maximum is 1.5e-5 of that maximum per activation, and the sum over a row measures 2e-5 ..
+# 7e-5 of the largest output on these inputs. The north-star bound 1e-3 * ||w_row|| * ||x|| is asserted at both.
+_PRECISION = {"bits": 24}
 
 
 def dot_bar(scale=1.0):
@@ -64,8 +65,9 @@ def precision(request, F):
 
 @pytest.fixture
 def precision24(F):
-    """For tests that use the streaming mat-vec as the f32-grade side of a comparison: 24-bit activations, and every batch
-    on that kernel (by default a batch of three rows or more goes to the one-pass matrix-core kernels)."""
+    """For tests that use the streaming mat-vec as the f32-grade side of a comparison: the weights they make have 24-bit
+    activations, and every batch on that kernel (otherwise a batch of three rows or more goes to the one-pass matrix-core
+    kernels)."""
     lib = F._lib.load()
     before = lib.fhip_matvec_precision(24)
     policy = lib.fhip_batch_policy(1)

@@ -277,7 +277,7 @@ def test_argument_checks(F):
 # ---------------------------------------------------------------- FHIP_BATCH_ORDERED: the same kernels, partial sums added in order
 
 def test_ordered_policy_gives_the_same_bits_on_every_run(F, O):
-    # Under FHIP_BATCH_ORDERED (2) the drop-in calls keep the one-pass kernels, but a launch that cuts a group's K between
+    # Under FHIP_BATCH_ORDERED (2, what a new weight has) the drop-in calls keep the one-pass kernels, but a launch that cuts a group's K between
     # workgroups writes the pieces to the library's workspace and adds them in a fixed order: run after run the same bits,
     # and the same bars against the oracle as the default policy. Shapes: cut along K (few groups, long rows), not cut
     # (one chunk), ragged rows, each activation-row class, Q8_0's ragged K; then the FFN block at the model's size, where
@@ -310,8 +310,8 @@ def test_ordered_policy_gives_the_same_bits_on_every_run(F, O):
         y = xt.ffn(wgu, wdn).to_vec()
         for _ in range(3):
             assert np.array_equal(xt.ffn(wgu, wdn).to_vec(), y)
-        lib.fhip_batch_policy(0)
-        y0 = xt.ffn(wgu, wdn).to_vec()                 # the default policy: atomic adds, the same sums in another order
+        wgu.batch_policy(0), wdn.batch_policy(0)
+        y0 = xt.ffn(wgu, wdn).to_vec()                 # FHIP_BATCH_AUTO: atomic adds, the same sums in another order
         assert np.abs(y - y0).max() <= 2e-6 * np.abs(y0).max()
     finally:
         lib.fhip_batch_policy(before)

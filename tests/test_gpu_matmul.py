@@ -218,24 +218,23 @@ def test_config3_ffn_block(F, O, batch):
         assert np.array_equal(bits(y2), bits(y))
     else:
         assert np.abs(y2 - y).max() <= 2e-6 * np.abs(y).max()
-        lib = F._lib.load()
-        before = lib.fhip_batch_policy(1)            # FHIP_BATCH_F32_MATVEC: every batch on the mat-vec kernel
-        try:
-            h1 = xt.try_matmul_swiglu(wgu)
-            y1 = h1.matmul_q(wdn).to_vec().reshape(batch, n_embd)
-            assert np.array_equal(bits(xt.ffn(wgu, wdn).to_vec().reshape(batch, n_embd)), bits(y1))
-            assert np.abs(y1 - y64).max() / np.abs(y64).max() < 2 * dot_bar()
-        finally:
-            lib.fhip_batch_policy(before)
+        # the one-pass kernels add a cut row's pieces in a fixed order (what a new weight does): the same bits on every run
+        assert np.array_equal(bits(xt.ffn(wgu, wdn).to_vec().reshape(batch, n_embd)), bits(y2))
+        assert wgu.batch_policy(F.BATCH_F32_MATVEC) == F.BATCH_ORDERED and wdn.batch_policy(F.BATCH_F32_MATVEC) == F.BATCH_ORDERED
+        h1 = xt.try_matmul_swiglu(wgu)               # every batch on the mat-vec kernel
+        y1 = h1.matmul_q(wdn).to_vec().reshape(batch, n_embd)
+        assert np.array_equal(bits(xt.ffn(wgu, wdn).to_vec().reshape(batch, n_embd)), bits(y1))
+        assert np.abs(y1 - y64).max() / np.abs(y64).max() < 2 * dot_bar()
 
 
 # ---------------------------------------------------------------- invariants
 
 @pytest.mark.parametrize("ty,rows,cols", [(Q4_K, 96, 5120), (Q6_K, 70, 2048), (Q8_0, 130, 1024), (Q6_K, 40, 17408)])
 def test_batch_rows_are_independent(F, O, ty, rows, cols):
-    # On the mat-vec kernel row r of a batch-m result is bit-identical to the batch-1 result for x_r: always under
-    # FHIP_BATCH_F32_MATVEC, and for the one- and two-row batches that take that kernel by default. Wider batches go to the
-    # one-pass matrix-core kernels by default: the same values to the accuracy of the two paths.
+    # On the mat-vec kernel row r of a batch-m result is bit-identical to the batch-1 result for x_r: always when the weight's
+    # policy is FHIP_BATCH_F32_MATVEC, and for the one- and two-row batches that take that kernel anyway. Wider batches go to the
+    # one-pass matrix-core kernels unless told otherwise: the same values to the accuracy of the two paths, and (the policy a
+    # new weight has adds a cut row's pieces in a fixed order) the same bits on every run.
     from ferric_amd.synth import synth_weights
     lib = F._lib.load()
     w = synth_weights(ty, rows, cols, 7)
@@ -249,12 +248,21 @@ def test_batch_rows_are_independent(F, O, ty, rows, cols):
             assert np.array_equal(bits(y), bits(singles[:m])), m
         else:
             assert np.abs(y - singles[:m]).max() <= dot_bar() * np.abs(singles).max(), m
-    before = lib.fhip_batch_policy(1)
+    for m in (3, 8, 33):                            # run to run: the same bits
+        xt = F.Tensor.from_vec(x[:m], (m, cols))
+        assert np.array_equal(bits(xt.matmul_q(qm).to_vec()), bits(xt.matmul_q(qm).to_vec())), m
+    # the policy is the handle's own: another handle on the same bytes keeps what it was made with
+    other = F.QMatrix.from_bytes(w, ty, rows, cols)
+    assert qm.batch_policy(F.BATCH_F32_MATVEC) == F.BATCH_ORDERED and qm.batch_policy(7) == F.BATCH_F32_MATVEC   # an unknown value only queries
+    assert other.batch_policy() == F.BATCH_ORDERED
+    for m in (3, 8, 11):
+        xt = F.Tensor.from_vec(x[:m], (m, cols))
+        assert np.array_equal(bits(xt.matmul_q(qm).to_vec().reshape(m, rows)), bits(singles[:m])), m
+    # and what new handles start with can be set for the process; existing handles do not follow
+    before = lib.fhip_batch_policy(F.BATCH_F32_MATVEC)
     try:
-        assert before == 0 and lib.fhip_batch_policy(7) == 1           # an unknown value only queries
-        for m in (3, 8, 11):
-            y = check_matmul(F, O, w, ty, rows, cols, x[:m], f"batch {m}, mat-vec policy")
-            assert np.array_equal(bits(y), bits(singles[:m])), m
+        assert before == F.BATCH_ORDERED and other.batch_policy() == F.BATCH_ORDERED
+        assert F.QMatrix.from_bytes(w, ty, rows, cols).batch_policy() == F.BATCH_F32_MATVEC
     finally:
         lib.fhip_batch_policy(before)
 
@@ -404,7 +412,7 @@ def test_non_finite_and_tiny_activations_give_what_the_f32_dot_gives(F, O, ty):
     lib = F._lib.load()
     wide = 5 if ty == Q8_0 else 3                      # from this many rows on a batch takes the one-pass matrix-core kernels
     for policy in (0, 1):
-        before = lib.fhip_batch_policy(policy)
+        before = qm.batch_policy(policy)
         try:
             for sl in (slice(0, 6), slice(0, 1), slice(1, 3), slice(2, 6)):      # batches of 6, 1, 2, 4 rows: every pass width
                 xs = x[sl]
@@ -424,7 +432,7 @@ def test_non_finite_and_tiny_activations_give_what_the_f32_dot_gives(F, O, ty):
                     assert np.array_equal(np.isposinf(y[i]), np.isposinf(w_[i])) and np.array_equal(np.isneginf(y[i]), np.isneginf(w_[i])), (ty, r)
                     assert (np.abs(y[i] - y_[i])[fin] <= bound[i][fin] + 1e-30).all(), (ty, r)
         finally:
-            lib.fhip_batch_policy(before)
+            qm.batch_policy(before)
     assert np.isnan(want[0]).all() and not np.isfinite(want[1]).any() and np.isfinite(want[3:6]).all()
 
 
