@@ -76,9 +76,11 @@ pub struct HipQMatrix {
     rows: usize,
     cols: usize,
 }
-// The handle is immutable after creation and the library's launches only read it.
+// The handle may move between threads. It is not `Sync`: every method enqueues on the default stream, and the batched paths
+// of one stream share that stream's library workspace across the several launches of a call, so two threads enqueueing
+// through one handle (or on one stream) at once could interleave those launches. One thread drives one stream, as in the
+// reference (its pipeline cache and batch recorder are thread-local, crates/ferric-tensor/src/lib.rs:1515-1532).
 unsafe impl Send for HipQMatrix {}
-unsafe impl Sync for HipQMatrix {}
 
 impl HipQMatrix {
     /// `QMatrix::from_bytes` (dtype.rs:893): `Err` for a type without a native matmul, panic on `cols % block` or a wrong
@@ -92,6 +94,14 @@ impl HipQMatrix {
     pub fn cols(&self) -> usize { self.cols }
     pub fn n_shards(&self) -> usize { 1 }
     pub fn nbytes(&self) -> usize { unsafe { ffi::fhip_weight_nbytes(self.h) } }
+    /// Activation bits of this weight's streaming mat-vec: 24 as created (the f32 significand; the reference examples' 1e-5
+    /// bar), 16 for the faster opt-in. Returns the setting before the call.
+    pub fn set_matvec_precision(&mut self, bits: i32) -> Result<i32, String> {
+        let rc = unsafe { ffi::fhip_weight_matvec_precision(self.h, bits) };
+        if rc < 0 { Err(last_error()) } else { Ok(rc) }
+    }
+    /// Which kernels batches of three rows and more take (`ffi::FHIP_BATCH_*`; `FHIP_BATCH_ORDERED` as created).
+    pub fn set_batch_policy(&mut self, policy: i32) -> i32 { unsafe { ffi::fhip_weight_batch_policy(self.h, policy) } }
 
     /// `Tensor::matmul_q` (dtype.rs:935): y [rows_x, rows] = x [rows_x, cols] * W^T.
     pub fn matmul_q(&self, x: &DeviceF32, rows_x: usize) -> Result<DeviceF32, String> {
@@ -103,6 +113,7 @@ impl HipQMatrix {
 
     /// `Tensor::try_matmul_swiglu` (dtype.rs:949): `None` where the reference has no fused kernel (Q8_0).
     pub fn try_matmul_swiglu(&self, x: &DeviceF32, rows_x: usize) -> Option<DeviceF32> {
+        assert_eq!(x.len(), rows_x * self.cols, "matmul_swiglu: inner dim");
         let mut y = DeviceF32::zeros(rows_x * self.rows / 2).ok()?;
         match unsafe { ffi::fhip_matmul_q_swiglu(self.h, x.as_ptr(), rows_x, y.as_mut_ptr(), ptr::null_mut()) } {
             ffi::FHIP_OK => Some(y),
@@ -114,6 +125,7 @@ impl HipQMatrix {
 
     /// The FFN block of crates/ferric-llama/src/qwen3.rs:944-964: down(swiglu(gate_up(x))).
     pub fn ffn(gate_up: &HipQMatrix, down: &HipQMatrix, x: &DeviceF32, rows_x: usize) -> Result<DeviceF32, String> {
+        assert_eq!(x.len(), rows_x * gate_up.cols, "ffn: inner dim");
         let mut ws = DeviceF32::zeros(rows_x * gate_up.rows / 2)?;
         let mut y = DeviceF32::zeros(rows_x * down.rows)?;
         check(unsafe { ffi::fhip_ffn(gate_up.h, down.h, x.as_ptr(), rows_x, y.as_mut_ptr(), ws.as_mut_ptr(), ptr::null_mut()) })?;

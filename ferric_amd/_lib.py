@@ -59,6 +59,7 @@ SYMBOLS = {
     "fhip_gemm_q_bf16": (C.c_int, [_vp, _vp, _sz, _vp, _vp]),
     "fhip_moe_topk": (C.c_int, [_vp, _vp, _sz, _sz, _sz, C.c_int, C.c_float, C.c_int, _vp, _vp]),
     "fhip_matmul_q_swiglu_id": (C.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _vp, _vp]),
+    "fhip_matmul_q_relu2_id": (C.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _vp, _vp]),
     "fhip_matmul_q_id": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _vp, _vp]),
     "fhip_matmul_q_id_wsum": (C.c_int, [_vp, _vp, _sz, _vp, _sz, _sz, _vp, _vp, _vp]),
     "fhip_gguf_parse": (C.c_int, [_vp, _sz, _vp]),

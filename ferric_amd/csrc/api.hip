@@ -1028,6 +1028,19 @@ int fhip_matmul_q_swiglu_id(const fhip_weight* w, const float* d_x, size_t t, co
     return fhip::launch_gemv_sel(w, d_x, d_y, eff, true, sel, (hipStream_t)stream);
 }
 
+int fhip_matmul_q_relu2_id(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t eff, float* d_y,
+                           void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    fhip::SelParams sel{};
+    if ((rc = sel_checks("matmul_q_relu2_id", w, k, eff, &sel))) return rc;
+    if (t == 0) return FHIP_OK;
+    if (!d_x || !d_selw || !d_y) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_relu2_id: NULL pointer");
+    if (((uintptr_t)d_x & 15) != 0 || (w->cols * 4) % 16 != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_relu2_id: x rows must be 16-byte aligned");
+    sel.selw = d_selw; sel.x_per_pair = 0; sel.y_stride = eff; sel.npairs = (int)(t * k); sel.relu2 = 1;
+    return fhip::launch_gemv_sel(w, d_x, d_y, eff, false, sel, (hipStream_t)stream);
+}
+
 int fhip_matmul_q_id(const fhip_weight* w, const float* d_x, const float* d_selw, size_t k, size_t out_pe, float* d_y, void* stream) {
     int rc = need_init();
     if (rc) return rc;

@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/ferric_hip.h"
+#include "../../include/ferric_hip_debug.h"
 
 struct fhip_weight {
     uint32_t type;      // ggml id: 2 / 3 / 6 / 7 / 8 / 12 / 13 / 14 / 20 / 23 / 39
@@ -34,6 +35,7 @@ struct SelParams {
     int x_per_pair;
     size_t y_stride;
     int npairs;
+    int relu2;   // the pair's outputs leave as max(v, 0)^2 (the squared-ReLU expert MLP, dtype.rs:1703-1729)
 };
 // applied at the top of a kernel: moves the three base pointers to this y-slice's expert / row / output
 template <class P>

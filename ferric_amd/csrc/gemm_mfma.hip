@@ -2,7 +2,7 @@
 // X bf16 [T, K], W raw GGUF blocks [N, K], Y f32 [T, N], f32 accumulate.
 //
 // Stands for the reference's cooperative-matrix prefill kernels (crates/ferric-tensor/src/dtype.rs:2059-2096
-// Q4_K, :1217-1257 Q6_K, :1333-1370 Q8_0), which dequantize an 8x8 weight tile into shared memory and
+// Q4_K, :1217-1257 Q6_K, :1333-1370 Q8_0, :1074-1131 Q5_K), which dequantize an 8x8 weight tile into shared memory and
 // feed an 8x8 f32 matrix unit. Here the unit is v_mfma_f32_32x32x16_bf16.
 //
 // Shape of the kernel. The reference found this path bound by the unpack arithmetic, not the matrix
@@ -127,6 +127,58 @@ struct Q4K {
         const uint8_t* nb = row + (size_t)nc * BLOCK;
         r.q[G] = *(const u32x4*)(nb + 16 + 32 * G + 16 * h);
         if (G == 1) r.hdn = *(const u32x4*)nb;
+    }
+};
+
+// Q5_K is Q4_K with a fifth bit per quant (the reference's matmul_q5_k_coop, crates/ferric-tensor/src/dtype.rs:1074-1131):
+// 176 B = [f16 d][f16 dmin][scales 12 B][qh 32 B][qs 128 B]; bit s of qh[l] is the fifth bit of element l of sub-block s
+// (crates/ferric-gguf/src/lib.rs:692-716), q = nibble + 16 * bit in 0..31, y = (d*sc)*q - dmin*m. A lane half h works on
+// elements 16h + [0, 16) of every sub-block, so it holds the same 16 bytes qh[16h, 16h + 16) for the whole chunk; slice T of
+// step G takes bit 2G + (T >> 1) of them. The high nibbles are shifted down (with the fifth bit on top they do not fit a
+// byte in place), so both sub-block scales are plain d * sc.
+struct Q5K {
+    static constexpr int BLOCK = 176;
+    static constexpr float UNPACK_US = 1.8f;
+    static constexpr bool PARTIAL = false;
+    static __host__ __device__ int chunks(int K) { return K / 256; }
+    struct Raw { u32x4 hd, hdn, qh, qhn, q[4]; };
+    struct Ctx { float d0, o0, d1, o1; };
+    static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int h, int) {
+        const uint8_t* blk = row + (size_t)c * BLOCK;
+        r.hd = *(const u32x4*)blk;
+        r.hdn = r.hd;
+        r.qh = *(const u32x4*)(blk + 16 + 16 * h);
+        r.qhn = r.qh;
+#pragma unroll
+        for (int g = 0; g < 4; g++) r.q[g] = *(const u32x4*)(blk + 48 + 32 * g + 16 * h);
+    }
+    template <int G>
+    static __device__ __forceinline__ void begin(Raw& r, int, int, int, Ctx& x) {
+        if (G == 0) { r.hd = r.hdn; r.qh = r.qhn; }
+        const float d = f16_bits(r.hd[0] & 0xFFFFu), dmin = f16_bits(r.hd[0] >> 16);
+        float s0, m0, s1, m1;
+        Q4K::sc_min(r.hd, 2 * G, s0, m0);
+        Q4K::sc_min(r.hd, 2 * G + 1, s1, m1);
+        // every product is exact in f32 (11-bit d, 6-bit scale, 5-bit quant), so the fused form rounds as the reference's
+        x.d0 = d * s0; x.o0 = -(dmin * m0); x.d1 = d * s1; x.o1 = -(dmin * m1);
+    }
+    template <int G, int T>
+    static __device__ __forceinline__ bf16x8 frag(const Raw& r, const Ctx& x) {
+        constexpr int w = 2 * (T & 1), s = 2 * G + (T >> 1);
+        uint32_t v[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t nib = T < 2 ? r.q[G][w + i] & 0x0F0F0F0Fu : (r.q[G][w + i] >> 4) & 0x0F0F0F0Fu;
+            const uint32_t bit = (s >= 4 ? r.qh[w + i] >> (s - 4) : r.qh[w + i] << (4 - s)) & 0x10101010u;
+            v[i] = nib | bit;
+        }
+        return frag8(v[0], v[1], T < 2 ? x.d0 : x.d1, T < 2 ? x.o0 : x.o1);
+    }
+    template <int G>
+    static __device__ __forceinline__ void refill(Raw& r, const uint8_t* row, int nc, int h, int) {
+        const uint8_t* nb = row + (size_t)nc * BLOCK;
+        r.q[G] = *(const u32x4*)(nb + 48 + 32 * G + 16 * h);
+        if (G == 1) { r.hdn = *(const u32x4*)nb; r.qhn = *(const u32x4*)(nb + 16 + 16 * h); }
     }
 };
 
@@ -1089,6 +1141,7 @@ size_t gemm_bf16_ws_bytes(const fhip_weight* w, size_t t) {
         case FHIP_Q4_K: return ws_bytes_fmt<Q4K>(w, t);
         case FHIP_Q6_K: return ws_bytes_fmt<Q6K>(w, t);
         case FHIP_Q8_0: return ws_bytes_fmt<Q80>(w, t);
+        case FHIP_Q5_K: return ws_bytes_fmt<Q5K>(w, t);
         default: return 0;
     }
 }
@@ -1102,6 +1155,7 @@ int launch_gemm_bf16(const fhip_weight* w, const uint16_t* d_x, size_t t, float*
         case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_x, t, d_y, s, d_ws, ws_bytes);
         case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_x, t, d_y, s, d_ws, ws_bytes);
         case FHIP_Q8_0: return launch_fmt<Q80>(w, d_x, t, d_y, s, d_ws, ws_bytes);
+        case FHIP_Q5_K: return launch_fmt<Q5K>(w, d_x, t, d_y, s, d_ws, ws_bytes);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "QMatrix: no native matmul for ggml type %u", w->type);
     }
 }

@@ -572,6 +572,7 @@ __global__ void __launch_bounds__(max_threads(M)) gemv_kernel(GemvParams p) {
             // silu(g) * u, crates/ferric-tensor/src/dtype.rs:2408
             a = (a / (1.0f + expf(-a))) * b;
         }
+        if (p.sel.relu2) { a = fmaxf(a, 0.f); a *= a; }   // max(v, 0)^2, crates/ferric-tensor/src/dtype.rs:3755-3756
         p.y[(size_t)m * p.out_rows + r] = a;
     }
 }
@@ -582,7 +583,7 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
     p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
     p.pair_bytes = SWIGLU ? out_rows * w->row_bytes : 0;
-    p.sel = sel ? *sel : fhip::SelParams{nullptr, 0, 0, 0, 0, 0, 1};
+    p.sel = sel ? *sel : fhip::SelParams{nullptr, 0, 0, 0, 0, 0, 1, 0};
     const int units = (int)(w->cols / 32);
     p.S = (units + 63) / 64;
     constexpr int MAXW = max_threads(M) / 64;

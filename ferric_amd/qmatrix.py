@@ -295,6 +295,21 @@ class Tensor:
         assert w.ggml_type == Q8_0
         return self.matmul_q_swiglu_id(w, selw, k, eff, stream)
 
+    def matmul_q_relu2_id(self, w, selw, k, eff, stream=None):
+        """Any format's selected-expert up projection with max(v, 0)^2 applied: [T, in] -> [T, k, eff]."""
+        t, inn = self._rows_inner()
+        assert 1 <= k <= 8, "k must be 1..=8"
+        assert inn == w.cols(), f"inner dim mismatch: x[..,{inn}] vs W[..,{w.cols()}]"
+        out = Tensor.empty((t, k, eff))
+        _lib.check(_lib.load().fhip_matmul_q_relu2_id(w.handle, self.buf.ptr, t, selw.buf.ptr, k, eff, out.buf.ptr, _stream_handle(stream)))
+        return out
+
+    def matmul_q5_0_relu2_id(self, w, selw, k, eff, stream=None):
+        """The squared-ReLU expert MLP's up projection on a Q5_0 slab -- dtype.rs:1711."""
+        assert w.ggml_type == Q5_0
+        assert self._rows_inner()[1] % 32 == 0, "Q5_0 inner dim must be a multiple of 32"
+        return self.matmul_q_relu2_id(w, selw, k, eff, stream)
+
     def matmul_q6_k_id(self, w, selw, out_pe, stream=None):
         """Selected experts' down projection, one row per slot: [k, in] -> [k, out_pe] -- dtype.rs:1640."""
         k, inn = self._rows_inner()
@@ -348,7 +363,7 @@ class Tensor:
         return out
 
     def matmul_q_coop(self, w, stream=None):
-        """f32 x [rows, in] @ W^T on the matrix cores -- dtype.rs:1818 matmul_q4_k_coop / :1199 / :1316."""
+        """f32 x [rows, in] @ W^T on the matrix cores -- dtype.rs:1818 matmul_q4_k_coop / :1199 / :1316 / :1074 (Q5_K)."""
         assert self.dtype == np.float32, "matmul_q_coop expects f32 activations"
         rows, inn = self._rows_inner()
         assert inn == w.cols(), "inner dim mismatch"
@@ -372,6 +387,10 @@ class Tensor:
 
     def matmul_q8_0_coop(self, w, stream=None):
         assert w.ggml_type == 8
+        return self.matmul_q_coop(w, stream)
+
+    def matmul_q5_k_coop(self, w, stream=None):  # dtype.rs:1074
+        assert w.ggml_type == 13
         return self.matmul_q_coop(w, stream)
 
     def matmul_q_f16x2(self, w, stream=None):

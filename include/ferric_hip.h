@@ -220,6 +220,13 @@ int fhip_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t n
 int fhip_matmul_q_swiglu_id(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t eff, float* d_y,
                             void* stream);
 
+/* dtype.rs:1703-1729 matmul_q5_0_relu2_id (kernel :3714-3758): the selected-expert UP projection of a squared-ReLU expert
+ * MLP (no gate slab). x [t, cols], w packs all experts' up rows expert-major (rows = n_expert * eff), selw the [t, 2k]
+ * moe_topk output; y [t, k, eff] = max(up_e . x_t, 0)^2 for every (token, selected expert), the activation applied as the
+ * dot product leaves the kernel. The reference has it for Q5_0; any format with a native mat-vec is taken. */
+int fhip_matmul_q_relu2_id(const fhip_weight* w, const float* d_x, size_t t, const float* d_selw, size_t k, size_t eff, float* d_y,
+                           void* stream);
+
 /* dtype.rs:1640 matmul_q6_k_id (kernel :2509): x [k, cols] (row s = slot s's SwiGLU output), w packs all experts' down
  * rows expert-major (rows = n_expert * out_pe), selw one moe_topk row [2k]; y [k, out_pe]. Any of the three formats. */
 int fhip_matmul_q_id(const fhip_weight* w, const float* d_x, const float* d_selw, size_t k, size_t out_pe, float* d_y, void* stream);
@@ -297,7 +304,9 @@ int fhip_kvq_append(int fmt, const float* d_src, size_t src_row_stride, size_t t
                     int src_at_pos, size_t cap, uint32_t* d_codes, uint32_t* d_scales, void* stream);
 /* QKvCache::dequantize_rows (:621-650; dequantize :617 is row0 = 0, rows = len): cache rows row0 .. row0 + rows to f32
  * d_out [rows, width]. d_last_pos (optional, device u32): rows past *d_last_pos are not written, so a captured step can pass
- * the capacity as `rows` and the position word of the token being decoded. */
+ * the capacity as `rows` and the position word of the token being decoded. The arrays carry no length: row0 + rows (and, with
+ * d_last_pos, *d_last_pos + 1) must not exceed the `rows` the caller sized them for with fhip_kvq_sizes -- an unchecked
+ * precondition, as for every other device pointer of this header. */
 int fhip_kvq_dequantize_rows(int fmt, const uint32_t* d_codes, const uint32_t* d_scales, size_t row0, size_t rows, size_t width,
                              const uint32_t* d_last_pos, float* d_out, void* stream);
 
@@ -411,28 +420,6 @@ size_t fhip_workspace_bytes(const fhip_weight* w, const fhip_weight* down, size_
 size_t fhip_workspace_bytes_coop(const fhip_weight* w, const fhip_weight* down, size_t rows_x);
 int fhip_workspace_reserve(void* stream, size_t nbytes);
 void fhip_workspace_release(void* stream);
-
-/* Debugging and tests: on != 0 sends every mat-vec to the shape-complete f32 kernel instead of the streaming one (process-wide,
- * not thread-safe against concurrent launches). No counterpart in the reference. */
-int fhip_debug_generic_matvec(int on);
-
-/* Debugging and tests: pins the workgroup tile of the matrix-core GEMM (fhip_gemm_q_bf16, fhip_matmul_q_coop, fhip_ffn_coop)
- * for launches of more than 32 rows: 0, 1, 2 = 64, 128, 256 activation rows x 256 outputs, 3 = 256 x 160; -1 (the default)
- * lets the cost estimate choose. Returns the value before the call. Process-wide, not thread-safe against concurrent
- * launches; fhip_workspace_bytes_coop follows it. No counterpart in the reference. */
-int fhip_debug_gemm_tile(int tile);
-
-/* Measurement aid: one launch that reads nbytes at d_src (16-byte loads over the whole chip) and does nothing else; d_sink is
- * one device word that is practically never written. Timed beside a mat-vec of the same size it gives the time a perfect reader
- * needs for those bytes on this device. No counterpart in the reference (its matvec_roofline example prints bytes / time of the
- * kernel itself, crates/ferric-tensor/examples/matvec_roofline.rs:85-100). */
-int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, void* stream);
-
-/* Measurement aid: `launches` one-row calls of fhip_matmul_q (swiglu != 0: fhip_matmul_q_swiglu) enqueued back to back from
- * native code, launch i on weight ws[i % n_weights], all with the same x and y. A profiler run that cannot replay graphs gets
- * the same steady stream of launches from it that a captured graph gives. No counterpart in the reference. */
-int fhip_debug_matmul_q_loop(const fhip_weight* const* ws, size_t n_weights, size_t launches, const float* d_x, int swiglu, float* d_y,
-                             void* stream);
 
 /* Precision of the activations inside the streaming mat-vec kernels (fhip_matmul_q, _swiglu, fhip_ffn, the "_id" entry points,
  * fhip_norm_matmul_q): per run of 32 (16 for Q6_K) columns the activations are held as block fixed point with a `bits`-bit

@@ -274,6 +274,28 @@ def matmul_swiglu_id_f64(x, w, ty, selw, k, eff, cols):
     return out
 
 
+def matmul_relu2_id_f64(x, w, ty, selw, k, eff, cols):
+    """MATMUL_Q5_0_RELU2_ID_WGSL (crates/ferric-tensor/src/dtype.rs:3714-3758) in f64 on the dequantized expert slab
+    [n_expert * eff, cols]: out[ti, s, o] = max(acc, 0)^2 with acc the dot of token ti's row with row e * eff + o,
+    e = selw[ti, k + s] (the index half of the moe_topk row). Also returns the rows' norms for the tolerance bound."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, cols)
+    w, _ = _u8(w)
+    rows = w.size // (cols // BLOCK[ty][0] * BLOCK[ty][1])
+    wd = deq_raw(w, rows * cols, ty).reshape(rows, cols).astype(np.float64)
+    selw = np.asarray(selw, dtype=np.float32).reshape(x.shape[0], 2 * k)
+    out = np.zeros((x.shape[0], k, eff))
+    acc = np.zeros((x.shape[0], k, eff))
+    wn = np.zeros((x.shape[0], k, eff))
+    for ti in range(x.shape[0]):
+        for s in range(k):
+            blk = wd[int(selw[ti, k + s]) * eff:][:eff]
+            acc[ti, s] = blk @ x[ti].astype(np.float64)
+            wn[ti, s] = np.linalg.norm(blk, axis=1)
+            a = np.maximum(acc[ti, s], 0.0)
+            out[ti, s] = a * a
+    return out, acc, wn
+
+
 def matmul_id_f64(x, w, ty, selw, k, out_pe, cols):
     """MATMUL_Q6_K_ID_WGSL (dtype.rs:2509-2536) in f64: out[s, o] = x[s] . W[e_s*out_pe + o], plus the weight norms."""
     x = np.ascontiguousarray(x, dtype=np.float32).reshape(k, cols)

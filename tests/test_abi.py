@@ -9,10 +9,22 @@ import pytest
 from conftest import ROOT
 
 
-def _declared():
-    text = open(os.path.join(ROOT, "include", "ferric_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(fhip_[a-z0-9_]+)\s*\(", text)))
+HEADERS = ("ferric_hip.h", "ferric_hip_debug.h")   # the interface a caller binds, and the measurement / test aids of the same library
+
+
+def _header_text(names=HEADERS):
+    text = "".join(open(os.path.join(ROOT, "include", n)).read() for n in names)
+    return re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+
+
+def _declared(names=HEADERS):
+    return sorted(set(re.findall(r"\b(fhip_[a-z0-9_]+)\s*\(", _header_text(names))))
+
+
+def test_debug_entry_points_stay_out_of_the_product_header():
+    product, aids = _declared(("ferric_hip.h",)), _declared(("ferric_hip_debug.h",))
+    assert not [n for n in product if n.startswith("fhip_debug_")]
+    assert aids and all(n.startswith("fhip_debug_") for n in aids)
 
 
 def test_library_exports_every_declared_symbol():
@@ -36,8 +48,7 @@ def test_no_undeclared_fhip_exports():
 def test_the_rust_binding_declares_the_same_entry_points():
     # crates/ferric-hip/src/ffi.rs is the binding a maintainer links: one `pub fn` per entry point of the header, with as many
     # arguments as the C prototype has
-    text = open(os.path.join(ROOT, "include", "ferric_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = _header_text()
     c_args = {}
     for name, args in re.findall(r"\b(fhip_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
         args = " ".join(args.split())

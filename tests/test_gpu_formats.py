@@ -113,10 +113,13 @@ def test_id_variants_on_the_other_formats(F, O):
 
 
 def test_matrix_core_entry_points_refuse_the_other_formats(F):
+    # the matrix-core prefill takes the formats the reference has coop kernels for (Q4_K, Q5_K, Q6_K, Q8_0), no other
     from ferric_amd.synth import synth_weights
-    w = F.QMatrix.from_bytes(synth_weights(Q5_K, 32, 256, 1), Q5_K, 32, 256)
-    with pytest.raises(ValueError, match="no native matmul for ggml type 13"):
-        F.Tensor.from_bf16_bits(np.zeros(256, np.uint16), (1, 256)).gemm_q_bf16(w)
+    for ty in (Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4):
+        cols = GEOM[ty][0] * (8 if GEOM[ty][0] == 32 else 1)
+        w = F.QMatrix.from_bytes(synth_weights(ty, 32, cols, 1), ty, 32, cols)
+        with pytest.raises(ValueError, match=f"no native matmul for ggml type {ty}"):
+            F.Tensor.from_bf16_bits(np.zeros(cols, np.uint16), (1, cols)).gemm_q_bf16(w)
 
 
 def test_these_formats_load_from_a_gguf_file(F, O, tmp_path):

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q6_K, Q5_K = 8, 12, 14, 13
 
 
 def bf16_round(a):
@@ -42,19 +42,19 @@ def run_case(F, O, ty, t, n, k, seed, gen=None):
     return y
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0, Q5_K])
 def test_small_and_ragged_shapes(F, O, ty):
     for i, (t, n, k) in enumerate([(1, 32, 256), (8, 256, 256), (33, 100, 512), (64, 96, 768), (100, 300, 1024), (130, 257, 2048)]):
         run_case(F, O, ty, t, n, k, 10 + i)
 
 
 def test_seeded_random_shapes(F, O):
-    # 36 shapes drawn with a fixed seed: any row count on either side of the 32-row kernel switch, output widths that are
+    # 48 shapes drawn with a fixed seed: any row count on either side of the 32-row kernel switch, output widths that are
     # no multiple of a tile (or of 4: the ordered sum of K-split tiles then stores element by element), 1 to 9 chunks of
     # K -- whatever way the launch is cut, every output meets the oracle
     rng = np.random.default_rng(20240607)
-    for i in range(36):
-        ty = (Q4_K, Q6_K, Q8_0)[i % 3]
+    for i in range(48):
+        ty = (Q4_K, Q6_K, Q8_0, Q5_K)[i % 4] if i >= 36 else (Q4_K, Q6_K, Q8_0)[i % 3]
         t = int(rng.integers(1, 300)) if i % 4 else int(rng.integers(1, 33))
         n = int(rng.integers(1, 700))
         k = int(rng.integers(1, 10)) * 256 if ty != Q8_0 else int(rng.integers(1, 73)) * 32
@@ -70,7 +70,7 @@ def test_every_tile_on_ragged_shapes(F, O, tile):
     before = lib.fhip_debug_gemm_tile(tile)
     try:
         shapes = [(Q4_K, 33, 100, 512), (Q4_K, 300, 4001, 1024), (Q6_K, 130, 257, 2048), (Q8_0, 70, 1283, 1184), (Q4_K, 520, 7000, 768),
-                  (Q6_K, 257, 161, 256), (Q8_0, 1025, 330, 96)]
+                  (Q6_K, 257, 161, 256), (Q8_0, 1025, 330, 96), (Q5_K, 300, 1283, 1024), (Q5_K, 70, 161, 2048)]
         for i, (ty, t, n, k) in enumerate(shapes):
             run_case(F, O, ty, t, n, k, 300 + 10 * tile + i)
     finally:
@@ -114,6 +114,7 @@ def test_the_layer_s_large_projections_on_sampled_outputs(F, O, ty, t, n, k):
 
 
 def test_prefill_other_formats_at_size(F, O):
+    run_case(F, O, Q5_K, 512, 5120, 5120, 24)
     run_case(F, O, Q6_K, 256, 5120, 5120, 22)
     run_case(F, O, Q8_0, 256, 4096, 4096, 23)
 
@@ -137,7 +138,8 @@ def test_rows_are_independent_of_the_batch(F, O):
 
 @pytest.mark.parametrize("ty,t,n,k", [(Q4_K, 128, 5120, 5120), (Q4_K, 512, 5120, 5120), (Q4_K, 2048, 9216, 5120),
                                       (Q6_K, 300, 1000, 4096), (Q8_0, 200, 1300, 2080), (Q4_K, 70, 3000, 8192),
-                                      (Q4_K, 8, 5120, 5120), (Q6_K, 20, 1000, 4096), (Q8_0, 3, 1300, 2080), (Q4_K, 32, 1024, 5120)])
+                                      (Q4_K, 8, 5120, 5120), (Q6_K, 20, 1000, 4096), (Q8_0, 3, 1300, 2080), (Q4_K, 32, 1024, 5120),
+                                      (Q5_K, 256, 5120, 5120), (Q5_K, 9, 3000, 2048)])
 def test_two_runs_give_identical_bits(F, O, ty, t, n, k):
     # Launches with fewer whole tiles than the chip has workgroups cut tiles along K (every shape here does; 2048 x 9216
     # has a cut remainder behind whole tiles; up to 32 rows it is groups of 128 outputs that are cut). The partial tiles are
@@ -171,7 +173,8 @@ def test_coop_entry_takes_f32_activations(F, O):
     # (equal up to the order in which K slices are added when the launch splits K).
     from ferric_amd.synth import synth_weights
     for ty, name, (t, n, k) in [(Q4_K, "matmul_q4_k_coop", (8, 512, 1024)), (Q6_K, "matmul_q6_k_coop", (4, 256, 512)),
-                                (Q8_0, "matmul_q8_0_coop", (21, 264, 416)), (Q4_K, "matmul_q4_k_coop", (150, 384, 768))]:
+                                (Q8_0, "matmul_q8_0_coop", (21, 264, 416)), (Q4_K, "matmul_q4_k_coop", (150, 384, 768)),
+                                (Q5_K, "matmul_q5_k_coop", (12, 256, 1024)), (Q5_K, "matmul_q5_k_coop", (150, 384, 768))]:
         w = synth_weights(ty, n, k, 60)
         qm = F.QMatrix.from_bytes(w, ty, n, k)
         x = (np.random.default_rng(61).standard_normal((t, k)) * 3).astype(np.float32)

@@ -82,6 +82,37 @@ def test_swiglu_id(F, O, ty, name, cols, eff):
                 assert np.array_equal(one.to_vec().view(np.uint32), got[ti, s].view(np.uint32)), (ti, s)
 
 
+# the squared-ReLU expert MLP's up projection (dtype.rs:1703-1729): Q5_0 as in the reference, streaming (cols a multiple of
+# 512) and shape-complete kernels, and two other formats through the type-generic entry point
+@pytest.mark.parametrize("ty,cols,eff", [(6, 1024, 72), (6, 160, 24), (6, 2688, 58), (Q4_K, 2048, 40), (Q8_0, 512, 33)])
+def test_relu2_id(F, O, ty, cols, eff):
+    from ferric_amd.synth import synth_weights
+    rng = np.random.default_rng(25)
+    n_expert, t, k = 6, 3, 4
+    raw = synth_weights(ty, n_expert * eff, cols, 9)
+    w = F.QMatrix.from_bytes(raw, ty, n_expert * eff, cols)
+    x = rng.standard_normal((t, cols)).astype(np.float32)
+    sel = selection(rng, t, k, n_expert)
+    st = F.Tensor.from_vec(sel.reshape(-1), (t, 2 * k))
+    xt = F.Tensor.from_vec(x.reshape(-1), (t, cols))
+    got = (xt.matmul_q5_0_relu2_id(w, st, k, eff) if ty == 6 else xt.matmul_q_relu2_id(w, st, k, eff)).to_vec().reshape(t, k, eff)
+    want, acc, wn = O.matmul_relu2_id_f64(x, raw, ty, sel, k, eff, cols)
+    # the dot to the north-star bound, carried through v -> max(v, 0)^2 (slope 2|v|), and to the bar of the scalar kernels
+    bound = 1e-3 * wn * np.linalg.norm(x.astype(np.float64), axis=1)[:, None, None]
+    assert (np.abs(got - want) <= 2 * np.abs(acc) * bound + bound ** 2 + 1e-30).all()
+    assert np.abs(got - want).max() <= 3 * dot_bar() * np.abs(want).max()
+    assert (got >= 0).all() and (got[acc < -1e-3 * np.abs(acc).max()] == 0).all()
+    rb = raw.size // (n_expert * eff)
+    for ti in range(t):          # the plain mat-vec on the selected expert's slice, then the activation: the same bits
+        for s in range(k):
+            e = int(sel[ti, k + s])
+            one = F.Tensor.from_vec(x[ti], (1, cols)).matmul_q(F.QMatrix.from_bytes(raw[e * eff * rb:(e + 1) * eff * rb], ty, eff, cols)).to_vec()
+            a = np.maximum(one, np.float32(0))
+            assert np.array_equal((a * a).view(np.uint32), got[ti, s].view(np.uint32)), (ti, s)
+    with pytest.raises(AssertionError, match="k must be"):
+        xt.matmul_q_relu2_id(w, st, 9, eff)
+
+
 def test_matmul_q6_k_id(F, O):
     rng = np.random.default_rng(22)
     for cols, out_pe in [(1024, 72), (768, 130)]:

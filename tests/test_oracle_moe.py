@@ -70,3 +70,43 @@ def test_asserts(O):
         O.moe_topk(np.zeros((1, 16), np.float32), None, 9, False, 1.0)
     with pytest.raises(AssertionError, match="n_expert"):
         O.moe_topk(np.zeros((1, 1025), np.float32), None, 2, False, 1.0)
+
+
+def test_relu2_id_against_the_reference_kernel_s_element_formulation(O):
+    # oracle.matmul_relu2_id_f64 (dequantize the slab, dot, max(v, 0)^2) against the kernel's own arithmetic restated word by
+    # word (crates/ferric-tensor/src/dtype.rs:3735-3756: nibble | fifth bit from qh, minus 16, times d; expert ids from the
+    # second half of the moe_topk row), and against what one-hot activations fix: out = max(c * w, 0)^2, 0 for a negative dot.
+    from ferric_amd.synth import synth_weights
+    Q5_0 = 6
+    n_expert, eff, cols, t, k = 5, 7, 96, 3, 2
+    raw = synth_weights(Q5_0, n_expert * eff, cols, 31)
+    rng = np.random.default_rng(32)
+    x = rng.standard_normal((t, cols)).astype(np.float32)
+    sel = np.zeros((t, 2 * k), np.float32)
+    for ti in range(t):
+        sel[ti, :k] = rng.random(k)
+        sel[ti, k:] = rng.choice(n_expert, size=k, replace=False)
+    got, acc, wn = O.matmul_relu2_id_f64(x, raw, Q5_0, sel, k, eff, cols)
+    blocks = raw.reshape(n_expert * eff, cols // 32, 22)
+    for ti in range(t):
+        for s in range(k):
+            e = int(sel[ti, k + s])
+            for o in range(eff):
+                a = 0.0
+                for b in range(cols // 32):
+                    blk = blocks[e * eff + o, b]
+                    d = float(blk[0:2].view(np.float16)[0])
+                    qh = int(blk[2:6].view(np.uint32)[0])
+                    for j in range(16):
+                        lo = ((int(blk[6 + j]) & 15) | (((qh >> j) & 1) << 4)) - 16
+                        hi = ((int(blk[6 + j]) >> 4) | (((qh >> (j + 16)) & 1) << 4)) - 16
+                        a += (float(x[ti, 32 * b + j]) * lo + float(x[ti, 32 * b + 16 + j]) * hi) * d
+                assert abs(a - acc[ti, s, o]) <= 1e-9 * (1 + abs(a))
+                assert abs(max(a, 0.0) ** 2 - got[ti, s, o]) <= 1e-9 * (1 + a * a)
+    assert (got >= 0).all() and (got[acc < 0] == 0).all() and (acc < 0).any() and (acc > 0).any()
+    wd = O.deq_raw(raw, n_expert * eff * cols, Q5_0).reshape(n_expert * eff, cols)
+    hot = np.zeros((1, cols), np.float32)
+    hot[0, 37] = 3.0
+    one = np.array([[1.0, 4.0]], np.float32)                              # k = 1: weight, expert 4
+    g1, _, _ = O.matmul_relu2_id_f64(hot, raw, Q5_0, one, 1, eff, cols)
+    assert np.allclose(g1[0, 0], np.maximum(3.0 * wd[4 * eff:5 * eff, 37].astype(np.float64), 0) ** 2, rtol=1e-12)
