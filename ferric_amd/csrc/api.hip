@@ -191,7 +191,7 @@ static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t,
 size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32; }
 bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
     if (w->batch_policy == FHIP_BATCH_F32_MATVEC) return false;
-    if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0) return false;
+    if (w->type != FHIP_Q4_K && w->type != FHIP_Q5_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0) return false;
     if (rows_x < (w->type == FHIP_Q8_0 ? 5u : 3u)) return false;
     return fhip::gemm_f16x2_supports(w, rows_x < f16x2_group(w) ? rows_x : f16x2_group(w));
 }
@@ -1122,8 +1122,8 @@ size_t fhip_matmul_q_f16x2_ws_bytes(const fhip_weight* w, size_t rows_x) {
 
 static int f16x2_checks(const char* who, const fhip_weight* w, size_t rows_x) {
     if (rows_x > 32) return set_error(FHIP_ERR_SHAPE, "%s: at most 32 activation rows (got %zu)", who, rows_x);
-    if (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0)
-        return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "%s: no kernel for ggml type %u (Q4_K, Q6_K and Q8_0 only)", who, w->type);
+    if (w->type != FHIP_Q4_K && w->type != FHIP_Q5_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0)
+        return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "%s: no kernel for ggml type %u (Q4_K, Q5_K, Q6_K and Q8_0 only)", who, w->type);
     if (w->type == FHIP_Q8_0 && rows_x > 16) return set_error(FHIP_ERR_SHAPE, "%s: at most 16 activation rows for Q8_0 (got %zu)", who, rows_x);
     if (rows_x && w->rows && !fhip::gemm_f16x2_supports(w, rows_x))
         return set_error(FHIP_ERR_SHAPE, "%s: weight rows of %zu columns are outside what the kernels take", who, w->cols);

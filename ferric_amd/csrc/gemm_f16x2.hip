@@ -109,7 +109,7 @@ struct Q4K {
     }
     struct Raw { u32x4 hd, q0, q1; };
     struct Head { u32x4 hd; };
-    struct Ctx { uint32_t s0, c0, s1, c1; float d, dm; };
+    struct Ctx { uint32_t s0, c0, s1, c1; float d, dm; int sh; };   // sh: Q5_K's shift to its fifth-bit planes
     static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int g4) {
         const uint8_t* blk = row + (size_t)c * BLOCK;
         r.hd = *(const u32x4*)blk;
@@ -178,6 +178,80 @@ struct Q4K {
         o[3] = hadd2(__builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u), HNEG1024);
         if (g4 != 0) o = (u32x4){0u, 0u, 0u, 0u};
         return __builtin_bit_cast(f16x8, o);
+    }
+};
+
+// Q5_K (crates/ferric-gguf/src/lib.rs:687-716): Q4_K's header and nibbles with 32 bytes in between that hold a fifth bit
+// for every weight: bit 2 g4 of qh[l] belongs to the low nibble of qs[32 g4 + l], bit 2 g4 + 1 to its high nibble. The
+// operand order, the scales and the minima are Q4_K's; codes up to 31 times scales up to 63 are still exact in f16.
+struct Q5K {
+    static constexpr int BLOCK = 176;
+    static constexpr bool HAS_MIN = true;
+    static __host__ __device__ constexpr int occupancy(int nt) { return nt == 1 ? 3 : 2; }
+    static __host__ __device__ constexpr int src_k(int pos) { return Q4K::src_k(pos); }
+    static __host__ __device__ constexpr int pos_of(int k) { return Q4K::pos_of(k); }
+    struct Raw { u32x4 hd, h0, h1, q0, q1; };
+    struct Head { u32x4 hd; };
+    typedef Q4K::Ctx Ctx;
+    static __device__ __forceinline__ void prime(Raw& r, const uint8_t* row, int c, int g4) {
+        const uint8_t* blk = row + (size_t)c * BLOCK;
+        r.hd = *(const u32x4*)blk;
+        r.h0 = *(const u32x4*)(blk + 16);
+        r.h1 = *(const u32x4*)(blk + 32);
+        r.q0 = *(const u32x4*)(blk + 48 + 32 * g4);
+        r.q1 = *(const u32x4*)(blk + 64 + 32 * g4);
+    }
+    static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) { h.hd = *(const u32x4*)(row + (size_t)c * BLOCK); }
+    static constexpr int PARTS = 11, LROW = 176, TAILS = 0, ROWS_OCCUPANCY = 3;   // 40 KB of LDS a workgroup
+    static constexpr bool ROWS_AT_16 = false;
+    static constexpr bool ROW_PER_LANE = true, SLICE_SCALE = false;
+    static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return *(const u32x4*)p; }
+    static __device__ __forceinline__ uint32_t piece_off(int ck, int part, int) { return (uint32_t)(ck * BLOCK + 16 * part); }
+    static __device__ __forceinline__ int piece_lds(int part) { return 16 * part; }
+    static __device__ __forceinline__ uint32_t tail_off(int, int, int, bool& live) { live = false; return 0; }
+    static __device__ __forceinline__ int tail_lds(int) { return 0; }
+    static __device__ __forceinline__ void from_lds(Raw& r, const uint8_t* row, int g4) {
+        r.hd = *(const u32x4*)row;
+        r.h0 = *(const u32x4*)(row + 16);
+        r.h1 = *(const u32x4*)(row + 32);
+        r.q0 = *(const u32x4*)(row + 48 + 32 * g4);
+        r.q1 = *(const u32x4*)(row + 64 + 32 * g4);
+    }
+    static __device__ __forceinline__ void take(Raw& r, const Head& h) { r.hd = h.hd; }
+    template <int I>
+    static __device__ __forceinline__ void refill(Raw& r, const uint8_t* row, int nc, int g4) {
+        const uint8_t* blk = row + (size_t)nc * BLOCK;
+        if (I == 3) { r.h0 = *(const u32x4*)(blk + 16); r.q0 = *(const u32x4*)(blk + 48 + 32 * g4); }
+        if (I == 7) { r.h1 = *(const u32x4*)(blk + 32); r.q1 = *(const u32x4*)(blk + 64 + 32 * g4); }
+    }
+    template <int I>
+    static __device__ __forceinline__ void pre(const Raw& r, int g4, Ctx& x) {
+        if (I != 0) return;
+        const uint32_t scw = Q4K::sc_bytes(r.hd, g4 >= 2) >> (16 * (g4 & 1));
+        const uint32_t s0 = splat_h((_Float16)(unsigned short)(scw & 0xFFu)), s1 = splat_h((_Float16)(unsigned short)((scw >> 8) & 0xFFu));
+        x.s0 = s0; x.c0 = hmul2(s0, HNEG1024);
+        x.s1 = hmul2(s1, H16TH); x.c1 = hmul2(s1, HNEG64);
+        x.d = f16_bits(r.hd[0] & 0xFFFFu);
+        x.dm = -64.0f * f16_bits(r.hd[0] >> 16);
+        // the two fifth-bit planes of this lane's sub-blocks, moved to bits 0 and 1 of every byte once for the chunk
+        x.sh = 2 * g4;
+    }
+    // the fifth bit is worth 16: mantissa bit 4 beside a low nibble (step 1), bit 8 beside a high nibble in place (step 1/16)
+    template <int I>
+    static __device__ __forceinline__ f16x8 frag(const Raw& r, const Ctx& x) {
+        const uint32_t w = I < 4 ? r.q0[I & 3] : r.q1[I & 3], w8 = w >> 8;
+        const uint32_t hb = (I < 4 ? r.h0[I & 3] : r.h1[I & 3]) >> x.sh;
+        u32x4 o;
+        o[0] = hfma2(and_or(w, 0x000F000Fu, H1024) | ((hb << 4) & 0x00100010u), x.s0, x.c0);
+        o[1] = hfma2(and_or(w8, 0x000F000Fu, H1024) | ((hb >> 4) & 0x00100010u), x.s0, x.c0);
+        o[2] = hfma2(and_or(w, 0x00F000F0u, H1024) | ((hb << 7) & 0x01000100u), x.s1, x.c1);
+        o[3] = hfma2(and_or(w8, 0x00F000F0u, H1024) | ((hb >> 1) & 0x01000100u), x.s1, x.c1);
+        return __builtin_bit_cast(f16x8, o);
+    }
+    static __device__ __forceinline__ f16x8 mins(const Raw& r, int g4) {
+        Q4K::Raw q;
+        q.hd = r.hd;
+        return Q4K::mins(q, g4);
     }
 };
 
@@ -816,7 +890,8 @@ Plan make_plan(const fhip_weight* w, size_t t) {
     const long long groups = ((long long)w->rows + 127) / 128;
     q.units = groups * q.nchunks;
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    const long long wgs = cus * (w->type == FHIP_Q6_K ? slots<Q6K>(q.nt) : w->type == FHIP_Q8_0 ? slots<Q80>(q.nt) : slots<Q4K>(q.nt));
+    const long long wgs = cus * (w->type == FHIP_Q6_K ? slots<Q6K>(q.nt) : w->type == FHIP_Q8_0 ? slots<Q80>(q.nt) :
+                                 w->type == FHIP_Q5_K ? slots<Q5K>(q.nt) : slots<Q4K>(q.nt));
     // one workgroup per resident slot, each with the same share of the units (a grid of 2.66 workgroups per CU leaves
     // two thirds of the CUs with half as much again to do as the rest); shares of three quarters of a group's chunks or
     // more are rounded to whole groups, which store instead of adding
@@ -876,7 +951,7 @@ namespace fhip {
 bool gemm_f16x2_supports(const fhip_weight* w, size_t t) {
     if (!w || t < 1 || w->cols == 0 || w->cols > (size_t)MAXW * 1024) return false;
     if (w->type == FHIP_Q8_0) return t <= 16 && w->cols % 32 == 0;   // rows of any whole number of blocks
-    return (w->type == FHIP_Q4_K || w->type == FHIP_Q6_K) && t <= 32 && w->cols % CHUNK == 0;
+    return (w->type == FHIP_Q4_K || w->type == FHIP_Q5_K || w->type == FHIP_Q6_K) && t <= 32 && w->cols % CHUNK == 0;
 }
 
 size_t gemm_f16x2_xp_bytes(const fhip_weight* w, size_t t) {
@@ -902,6 +977,7 @@ int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swi
     const Plan q = make_plan(w, t);
     switch (w->type) {
         case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
+        case FHIP_Q5_K: return launch_xsplit_fmt<Q5K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
         case FHIP_Q6_K: return launch_xsplit_fmt<Q6K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
         case FHIP_Q8_0: return launch_xsplit_fmt<Q80>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
@@ -911,6 +987,7 @@ int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swi
 int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_part) {
     switch (w->type) {
         case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, t, d_y, s, y_cleared, d_part);
+        case FHIP_Q5_K: return launch_fmt<Q5K>(w, d_xp, t, d_y, s, y_cleared, d_part);
         case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, t, d_y, s, y_cleared, d_part);
         case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, t, d_y, s, y_cleared, d_part);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);

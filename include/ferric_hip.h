@@ -170,7 +170,7 @@ int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ggml_ty
  * :1172 matmul_q6_k): y[rows_x, rows] = x[rows_x, cols] * W^T, f32 in, f32 accumulate, f32 out.
  * rows_x = 1 is the decode GEMV; any rows_x >= 1 is accepted.
  * Which kernel a batch takes (fhip_batch_policy): one or two rows go through the streaming mat-vec; from three rows on (five
- * for Q8_0) Q4_K / Q6_K / Q8_0 weights are read once per group of up to 32 (Q8_0: 16) rows by the f16 hi/lo matrix-core
+ * for Q8_0) Q4_K / Q5_K / Q6_K / Q8_0 weights are read once per group of up to 32 (Q8_0: 16) rows by the f16 hi/lo matrix-core
  * kernels (see fhip_matmul_q_f16x2: f32-grade, 22-bit activations), longer batches group by group. That path keeps its
  * prepared activations in a workspace the library owns per stream (fhip_workspace_reserve); inside a graph capture the
  * workspace cannot grow, and the call then fails with FHIP_ERR_ARG and says how many bytes to reserve beforehand.
@@ -461,8 +461,8 @@ int fhip_ffn_coop(const fhip_weight* gate_up, const fhip_weight* down, const flo
 
 /* crates/ferric-tensor/src/dtype.rs:935-944 Tensor::matmul_q for 1..32 activation rows in ONE pass over the weights
  * with f32-grade results (the reference's kernels, :2995-3051 and :3423-3469, walk the weight row once per activation
- * row): x f32 [rows_x, cols] -> y f32 [rows_x, rows]. Q4_K and Q6_K (cols a multiple of 256, as the formats require),
- * and Q8_0 (:2948-2990; cols a multiple of 32) for up to 16 rows.
+ * row): x f32 [rows_x, cols] -> y f32 [rows_x, rows]. Q4_K, Q5_K and Q6_K (cols a multiple of 256, as the formats
+ * require), and Q8_0 (:2948-2990; cols a multiple of 32) for up to 16 rows.
  * Each 256-column chunk of an activation row is scaled by a power of two and split into two f16 operand rows (22
  * significant bits at the chunk's largest magnitude), the
  * weights enter the f16 matrix cores as exact integers (sub-block scale x quant; the int8 quant for Q8_0) and the f32

@@ -15,7 +15,7 @@ import pytest
 
 # the f32 mat-vec path is the other side of most comparisons here: it runs with 24-bit activations
 pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("precision24")]
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 TIGHT = 2.5e-7
 
 
@@ -33,7 +33,7 @@ def run_case(F, O, ty, t, n, k, seed, x=None, w=None, tol=TIGHT):
     return y, y64
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K, Q8_0])
 def test_small_and_ragged_shapes(F, O, ty):
     # every activation-row count class (1..8 -> one group of operand rows, 9..16 -> two, 17..32 -> four), weight rows that
     # do not fill a 16-row set, a 128-row group or a workgroup's share, one chunk and many
@@ -47,16 +47,16 @@ def test_small_and_ragged_shapes(F, O, ty):
         run_case(F, O, ty, t, n, k, 100 + i)
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
 def test_a_chunk_of_small_values_keeps_its_bits_beside_a_large_one(F, O, ty):
     # The scale is per 256-column chunk. Weights whose first super-block has scale 0 ignore the first chunk of x, so a
     # first chunk 2^60 times larger than the rest must not cost the rest its precision: the outputs are held to the bound
     # taken over the other chunks' activations only (with one scale per row their 22 bits would all lie above those values).
     from ferric_amd.synth import synth_weights
     t, n, k = 6, 160, 1280
-    blk = {Q4_K: 144, Q6_K: 210}[ty]
+    blk = {Q4_K: 144, Q5_K: 176, Q6_K: 210}[ty]
     w = synth_weights(ty, n, k, 61).copy().reshape(n, k // 256, blk)
-    if ty == Q4_K:
+    if ty in (Q4_K, Q5_K):
         w[:, 0, 0:4] = 0          # d and dmin of the first super-block of every row
     else:
         w[:, 0, 208:210] = 0      # d
@@ -72,7 +72,7 @@ def test_a_chunk_of_small_values_keeps_its_bits_beside_a_large_one(F, O, ty):
     assert (np.abs(y - y64) <= bound).all(), float(np.max(np.abs(y - y64) / bound))
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K, Q8_0])
 def test_rows_of_very_different_magnitude(F, O, ty):
     # each chunk of a row is scaled by its own power of two: tiny, huge, zero and outlier rows side by side keep the per-row bound
     t, n, k = 8, 96, 1024
@@ -118,6 +118,23 @@ def test_q6_k_products_beyond_the_exact_f16_range(F, O):
     run_case(F, O, Q6_K, t, n, k, 13, w=w.reshape(-1))
 
 
+def test_q5_k_every_code_and_the_largest_scales(F, O):
+    # all 32 codes (both nibbles, the fifth bit set and clear) under 6-bit scales and minima at their ends: the largest
+    # product, 63 * 31 = 1953, is still an exact f16 integer
+    n, k, t = 64, 1024, 8
+    rng = np.random.default_rng(16)
+    w = np.zeros((n, k // 256, 176), np.uint8)
+    d = rng.choice(np.array([0.01, -0.02, 0.5, 3e-4], np.float16), size=(n, k // 256, 2))
+    w[:, :, 0:4] = d.view(np.uint8).reshape(n, k // 256, 4)
+    w[:, :, 4:16] = rng.choice(np.array([0xFF, 0x3F, 0xC0, 0x00, 0x7E, 0xA5], np.uint8), size=(n, k // 256, 12))
+    w[:, :, 16:48] = rng.choice(np.array([0x00, 0xFF, 0xAA, 0x55, 0x81], np.uint8), size=(n, k // 256, 32))
+    w[:, :, 48:] = rng.choice(np.array([0x00, 0xFF, 0x0F, 0xF0, 0x1E, 0xE1], np.uint8), size=(n, k // 256, 128))
+    w[0, 0, 16:48] = np.arange(32, dtype=np.uint8) * 8 + 1
+    w[0, 0, 48:] = np.arange(128, dtype=np.uint8) * 2 + 1
+    run_case(F, O, Q5_K, t, n, k, 17, w=w.reshape(-1))
+    run_case(F, O, Q5_K, 20, n, k, 18, w=w.reshape(-1))
+
+
 def test_q8_0_every_int8_value_and_scale_signs(F, O):
     # quants over all 256 byte values (-128 included), scales of both signs, zero and the largest finite f16 magnitude class
     n, k, t = 48, 512, 4
@@ -131,7 +148,7 @@ def test_q8_0_every_int8_value_and_scale_signs(F, O):
     run_case(F, O, Q8_0, t, n, k, 15, w=w.reshape(-1))
 
 
-@pytest.mark.parametrize("ty,n,k", [(Q4_K, 512, 2048), (Q6_K, 384, 1024), (Q8_0, 640, 1120)])
+@pytest.mark.parametrize("ty,n,k", [(Q4_K, 512, 2048), (Q5_K, 400, 1536), (Q6_K, 384, 1024), (Q8_0, 640, 1120)])
 def test_agrees_with_the_f32_matvec_path_and_rows_are_independent(F, O, ty, n, k):
     from ferric_amd.synth import synth_weights
     w = synth_weights(ty, n, k, 20)
@@ -191,7 +208,7 @@ def test_ffn_block_with_q8_0_weights(F, O, tg, td):
         assert np.abs(y - y32).max() / np.abs(y32).max() < 2e-6
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K, Q8_0])
 def test_random_shapes_against_the_f32_path(F, O, ty):
     # 24 seeded random (rows of x, rows of W, columns) triples: every branch of the launch plan (whole groups, dealt runs,
     # runs that cross group boundaries, weights shorter than a workgroup's share) against the exact f32 mat-vec path
@@ -256,7 +273,7 @@ def test_argument_checks(F):
         F.Tensor.from_vec(np.zeros((33, 256), np.float32), (33, 256)).matmul_q_f16x2(q4)
     with pytest.raises(AssertionError, match="at most 16 activation rows for Q8_0"):
         F.Tensor.from_vec(np.zeros((17, 256), np.float32), (17, 256)).matmul_q_f16x2(q8)
-    with pytest.raises(ValueError, match="Q4_K, Q6_K and Q8_0 only"):
+    with pytest.raises(ValueError, match="Q4_K, Q5_K, Q6_K and Q8_0 only"):
         F.Tensor.from_vec(np.zeros((2, 256), np.float32), (2, 256)).matmul_q_f16x2(q40)
     with pytest.raises(AssertionError, match="inner dim mismatch"):
         F.Tensor.from_vec(np.zeros((2, 512), np.float32), (2, 512)).matmul_q_f16x2(q4)
@@ -288,7 +305,8 @@ def test_ordered_policy_gives_the_same_bits_on_every_run(F, O):
     try:
         assert lib.fhip_batch_policy(-1) == 2
         cases = [(Q4_K, 4, 512, 8192), (Q4_K, 8, 5120, 5120), (Q6_K, 3, 130, 4096), (Q6_K, 12, 1000, 17408), (Q4_K, 20, 257, 2048),
-                 (Q4_K, 32, 64, 256), (Q8_0, 5, 300, 4128), (Q8_0, 16, 1024, 4096), (Q4_K, 40, 384, 6144)]
+                 (Q4_K, 32, 64, 256), (Q8_0, 5, 300, 4128), (Q8_0, 16, 1024, 4096), (Q4_K, 40, 384, 6144),
+                 (Q5_K, 6, 256, 8192), (Q5_K, 24, 1000, 2048)]
         for i, (ty, t, n, k) in enumerate(cases):
             w = synth_weights(ty, n, k, 700 + i)
             x = np.random.default_rng(800 + i).standard_normal((t, k)).astype(np.float32)

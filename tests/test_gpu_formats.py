@@ -54,9 +54,13 @@ def test_matmul_small_batch(F, O, ty):
         y64, wn = O.matmul_f64(x, raw, ty, rows, cols)
         assert (np.abs(y - y64) <= 1e-3 * wn[None, :] * np.linalg.norm(x.astype(np.float64), axis=1)[:, None]).all(), (rows, cols, b)
         assert np.abs(y - y64).max() <= dot_bar() * max(1e-3, np.abs(y64).max()), (rows, cols, b)
-        # a row of a batch is bit-identical to the same row alone
+        # a row of a batch is bit-identical to the same row alone; Q5_K batches of three rows and more take the one-pass
+        # matrix-core kernels, as Q4_K's do, and agree with the mat-vec to the bar both are held to
         y1 = F.Tensor.from_vec(x[b - 1], (1, cols)).matmul_q(w).to_vec()
-        assert np.array_equal(bits(y1), bits(y[b - 1]))
+        if ty == Q5_K and b >= 3:
+            assert np.abs(y1 - y[b - 1]).max() <= 2 * dot_bar() * np.abs(y64).max()
+        else:
+            assert np.array_equal(bits(y1), bits(y[b - 1]))
     name = {Q4_0: "matmul_q4_0", Q4_1: "matmul_q4_1", Q5_0: "matmul_q5_0", Q5_1: "matmul_q5_1", Q5_K: "matmul_q5_k",
             IQ4_NL: "matmul_iq4_nl", IQ4_XS: "matmul_iq4_xs", MXFP4: "matmul_mxfp4"}[ty]
     assert np.array_equal(bits(getattr(F.Tensor.from_vec(x[0], (1, cols)), name)(w).to_vec()), bits(y[0]))

@@ -420,7 +420,7 @@ def test_non_finite_and_tiny_activations_give_what_the_f32_dot_gives(F, O, ty):
                 w_, y_ = want[sl], y64[sl]
                 with np.errstate(all="ignore"):
                     bound = 1e-3 * wn[None, :] * np.linalg.norm(xs.astype(np.float64), axis=1)[:, None]
-                one_pass = policy == 0 and xs.shape[0] >= wide and ty in (Q8_0, Q4_K, Q6_K)
+                one_pass = policy == 0 and xs.shape[0] >= wide and ty in (Q8_0, Q4_K, Q6_K, 13)
                 for i, r in enumerate(range(sl.start, sl.stop)):
                     fin = np.isfinite(w_[i])
                     if one_pass and not np.isfinite(xs[i]).all():
