@@ -677,6 +677,27 @@ def bench_prefill(F, lib, check, stream, timer, ts=(128, 512, 2048), reps=10):
                 ms0 = timer.time_ms(g.launch) / reps
                 out[str(t)]["ms_on_zero_activations"] = ms0
         res[name] = out
+    # What the matrix pipe gives with nothing else to do (register-resident operands, random mantissas), in graphs of ten
+    # launches like the GEMMs above, at two launch lengths: about the 5120 x 5120 T = 2048 launch and about the large one.
+    # The clock under sustained matrix work is set by the power limit, so this, not the 2.5 PFLOP/s at 2.4 GHz, is what
+    # 100 % reads in wall-clock terms on this box.
+    sink = F.DeviceBuffer(256)
+    ceil = {}
+    for label, iters in (("launch_of_130us", 900), ("launch_of_700us", 5000)):
+        fl = C.c_double()
+        g = F.Graph.begin(stream)
+        for _ in range(reps):
+            check(lib.fhip_debug_mfma_probe(iters, sink.ptr, C.byref(fl), stream.handle))
+        g.end()
+        g.launch()
+        ms = timer.time_ms(g.launch) / reps
+        ceil[label] = {"ms": ms, "TFLOPs": fl.value / (ms * 1e-3) / 1e12}
+    res["mfma_only_ceiling_TFLOPs"] = ceil["launch_of_700us"]["TFLOPs"]
+    res["mfma_only_ceiling"] = ceil
+    big = res["34816x5120"][str(max(ts))]
+    big["frac_of_mfma_only_ceiling"] = big["TFLOPs"] / ceil["launch_of_700us"]["TFLOPs"]
+    small = res["5120x5120"][str(max(ts))]
+    small["frac_of_mfma_only_ceiling"] = small["TFLOPs"] / ceil["launch_of_130us"]["TFLOPs"]
     return res
 
 

@@ -122,6 +122,7 @@ SYMBOLS = {
     "fhip_workspace_reserve": (C.c_int, [_vp, C.c_size_t]),
     "fhip_workspace_release": (None, [_vp]),
     "fhip_debug_read_probe": (C.c_int, [_vp, _sz, _vp, _vp]),
+    "fhip_debug_mfma_probe": (C.c_int, [C.c_int, _vp, C.POINTER(C.c_double), _vp]),
     "fhip_debug_matmul_q_loop": (C.c_int, [_vp, _sz, _sz, _vp, C.c_int, _vp, _vp]),
     "fhip_u32_add": (C.c_int, [_vp, _sz, _u32, _vp]),
     "fhip_matvec_q8_0_host": (C.c_int, [_vp, _vp, _sz, _sz, _sz, _vp]),

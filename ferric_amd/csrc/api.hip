@@ -963,6 +963,13 @@ int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, vo
     return fhip::launch_read_probe(d_src, nbytes, d_sink, (hipStream_t)stream);
 }
 
+int fhip_debug_mfma_probe(int iters, float* d_sink, double* flops, void* stream) {
+    int rc = need_init();
+    if (rc) return rc;
+    if (iters < 1 || !d_sink) return set_error(FHIP_ERR_ARG, "fhip_debug_mfma_probe: iters >= 1 and a sink are needed");
+    return fhip::launch_mfma_probe(iters, d_sink, (hipStream_t)stream, flops);
+}
+
 int fhip_debug_matmul_q_loop(const fhip_weight* const* ws, size_t n_weights, size_t launches, const float* d_x, int swiglu, float* d_y,
                              void* stream) {
     int rc = need_init();

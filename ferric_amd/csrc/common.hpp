@@ -102,6 +102,7 @@ int launch_gemv_generic_sel(const fhip_weight* w, const float* d_x, float* d_y, 
 
 // probe.hip: reads nbytes (a multiple of 16 is read) and stores nothing to speak of
 int launch_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, hipStream_t s);
+int launch_mfma_probe(int iters, float* d_sink, hipStream_t s, double* flops);
 
 // moe.hip
 int launch_moe_topk(const float* d_logits, const float* d_bias, size_t t, size_t ne, int k, int sigmoid, float scale, int norm,

@@ -718,8 +718,10 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
   }
 }
 
-// Rows 16 * blockIdx.y .. + 15 of left-over tile `blockIdx.x` (BM x BN outputs, BN <= 256 a multiple of 4), if more than one
-// run contributed to it: Y = slot 0 + slot 1 + ... in that order. A thread owns four adjacent columns of one row per pass.
+// Left-over tile `blockIdx.x` (BM x BN outputs, BN a multiple of 4), if more than one run contributed to it: Y = slot 0 +
+// slot 1 + ... in that order. A thread owns four adjacent columns of one row (item blockIdx.y * 256 + threadIdx.x of the
+// tile's BM * BN / 4) and asks for up to eight slots at once: the launch is a few dependent trips to memory long, so it
+// is cut as finely as that allows (a thread per 16 rows took 7.6 us for the 40 tiles of 5120 x 5120 at T = 128).
 __global__ void __launch_bounds__(256) sum_split_tiles_kernel(float* __restrict__ Y, const float* __restrict__ ws, int T, int N, int BM, int BN,
                                                             int tiles_n, int nchunks, int per, int kmax, int first_tile) {
     const int rt = blockIdx.x, tile = first_tile + rt;
@@ -727,32 +729,29 @@ __global__ void __launch_bounds__(256) sum_split_tiles_kernel(float* __restrict_
     const int nk = (int)((u0 + nchunks - 1) / per) - (int)(u0 / per) + 1;
     if (nk == 1) return;                          // one run covered the whole K of this tile and stored it
     const int tile_y = tile / tiles_n, tile_x = tile - tile_y * tiles_n;
-    const int c4 = (threadIdx.x & 63) * 4, col = tile_x * BN + c4;
-    if (c4 >= BN) return;
+    const int item = blockIdx.y * 256 + threadIdx.x, bn4 = BN >> 2;
+    const int lt = item / bn4, c4 = (item - lt * bn4) * 4;
+    const int t = tile_y * BM + lt, col = tile_x * BN + c4;
+    if (lt >= BM || t >= T || col >= N) return;
     const size_t slot = (size_t)BM * BN;
-    const float* base = ws + (size_t)rt * kmax * slot + c4;
+    const float* q = ws + (size_t)rt * kmax * slot + (size_t)lt * BN + c4;
+    float4 a = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < nk; k0 += 8) {
+        float4 v[8];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int lt = blockIdx.y * 16 + i * 4 + (threadIdx.x >> 6), t = tile_y * BM + lt;
-        if (t >= T || col >= N) continue;
-        const float* q = base + (size_t)lt * BN;
-        float4 a = *(const float4*)q;
-        for (int k0 = 1; k0 < nk; k0 += 4) {          // four slots requested at a time, added in slot order
-            float4 v[4];
+        for (int j = 0; j < 8; j++) v[j] = *(const float4*)(q + (size_t)(k0 + j < nk ? k0 + j : 0) * slot);
+        if (k0 == 0) a = v[0];
 #pragma unroll
-            for (int j = 0; j < 4; j++) v[j] = *(const float4*)(q + (size_t)(k0 + j < nk ? k0 + j : 0) * slot);
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                if (k0 + j < nk) { a.x += v[j].x; a.y += v[j].y; a.z += v[j].z; a.w += v[j].w; }
-        }
-        float* y = Y + (size_t)t * N + col;
-        if ((N & 3) == 0) *(float4*)y = a;
-        else {
-            y[0] = a.x;
-            if (col + 1 < N) y[1] = a.y;
-            if (col + 2 < N) y[2] = a.z;
-            if (col + 3 < N) y[3] = a.w;
-        }
+        for (int j = 0; j < 8; j++)
+            if (k0 + j > 0 && k0 + j < nk) { a.x += v[j].x; a.y += v[j].y; a.z += v[j].z; a.w += v[j].w; }
+    }
+    float* y = Y + (size_t)t * N + col;
+    if ((N & 3) == 0) *(float4*)y = a;
+    else {
+        y[0] = a.x;
+        if (col + 1 < N) y[1] = a.y;
+        if (col + 2 < N) y[2] = a.z;
+        if (col + 3 < N) y[3] = a.w;
     }
 }
 
@@ -1039,7 +1038,7 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     if constexpr (BN == 256) hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(q.grid), dim3(512), 0, s, p);
     else hipLaunchKernelGGL((gemm_q_bf16_n160_kernel<F>), dim3(q.grid), dim3(512), 0, s, p);
     if (q.split_wgs > 0)
-        hipLaunchKernelGGL(sum_split_tiles_kernel, dim3((unsigned)q.left, (unsigned)(64 * MI / 16)), dim3(256), 0, s, d_y, (const float*)d_ws, p.T, p.N, 64 * MI,
+        hipLaunchKernelGGL(sum_split_tiles_kernel, dim3((unsigned)q.left, (unsigned)((64 * MI * BN / 4 + 255) / 256)), dim3(256), 0, s, d_y, (const float*)d_ws, p.T, p.N, 64 * MI,
                            BN, p.tiles_n, p.nchunks, p.per, p.kmax, (int)(p.whole_rounds * cus));
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }

@@ -25,6 +25,13 @@ int fhip_debug_gemm_tile(int tile);
  * kernel itself, crates/ferric-tensor/examples/matvec_roofline.rs:85-100). */
 int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, void* stream);
 
+/* Measurement aid: one launch of matrix instructions only (v_mfma_f32_32x32x16_bf16 on register-resident operands with random
+ * mantissas; one workgroup of eight waves per CU, `iters` rounds of four instructions per wave). *flops (may be NULL) receives
+ * the floating-point operations of the launch: 2 * 32 * 32 * 16 per instruction. Timed, it is what the matrix pipe gives on this
+ * device at the clock its power limit allows, the ceiling the dequant-GEMM is priced against. d_sink is one device float that
+ * is practically never written. No counterpart in the reference. */
+int fhip_debug_mfma_probe(int iters, float* d_sink, double* flops, void* stream);
+
 /* Measurement aid: `launches` one-row calls of fhip_matmul_q (swiglu != 0: fhip_matmul_q_swiglu) enqueued back to back from
  * native code, launch i on weight ws[i % n_weights], all with the same x and y. A profiler run that cannot replay graphs gets
  * the same steady stream of launches from it that a captured graph gives. No counterpart in the reference. */
