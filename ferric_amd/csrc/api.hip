@@ -208,14 +208,16 @@ int zero_outputs(size_t t, size_t rows, float* d_y, hipStream_t s) {
 size_t f16x2_matmul_ws(const fhip_weight* w, size_t t) {
     return align256(fhip::gemm_f16x2_xp_bytes(w, t)) + (w->batch_policy == FHIP_BATCH_ORDERED ? align256(fhip::gemm_f16x2_part_bytes_upto(w, t)) : 0);
 }
-int f16x2_matmul(const fhip_weight* w, const float* d_x, size_t t, bool swiglu_in, float* d_y, void* d_ws, hipStream_t s) {
+// deferred: the ordered sum of K-split groups is left to the reader of y, which gets *deferred as its `src`
+int f16x2_matmul(const fhip_weight* w, const float* d_x, size_t t, bool swiglu_in, float* d_y, void* d_ws, hipStream_t s,
+                 fhip::F16Parts* deferred = nullptr, const fhip::F16Parts* src = nullptr) {
     uint16_t* xp = (uint16_t*)d_ws;
     const bool ordered = w->batch_policy == FHIP_BATCH_ORDERED;
     float* part = ordered && fhip::gemm_f16x2_part_bytes(w, t) ? (float*)((uint8_t*)d_ws + align256(fhip::gemm_f16x2_xp_bytes(w, t))) : nullptr;
     const bool clr = !part && fhip::gemm_f16x2_adds_into_y(w, t);   // then the split clears y on the side
-    int rc = fhip::launch_xsplit_f16(w, d_x, t, swiglu_in, xp, s, clr ? d_y : nullptr, clr ? t * w->rows : 0);
+    int rc = fhip::launch_xsplit_f16(w, d_x, t, swiglu_in, xp, s, clr ? d_y : nullptr, clr ? t * w->rows : 0, src);
     if (rc) return rc;
-    return fhip::launch_gemm_f16x2(w, xp, t, d_y, s, clr, part);
+    return fhip::launch_gemm_f16x2(w, xp, t, d_y, s, clr, part, deferred);
 }
 
 }  // namespace
@@ -609,8 +611,11 @@ int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, s
         if (!takes_f16x2(gu, t) || !takes_f16x2(down, t)) {
             if ((rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, d_ws + m0 * n_ff, n_ff, s))) return rc;
             rc = fhip::launch_gemv(down, d_ws + m0 * n_ff, t, d_y + m0 * down->rows, 0, s);
-        } else if (!(rc = f16x2_matmul(gu, d_x + m0 * gu->cols, t, false, g, ws, s))) {
-            rc = f16x2_matmul(down, g, t, true, d_y + m0 * down->rows, ws2, s);
+        } else {
+            // under the ordered policy gate|up's K-split groups stay partial sums; the split for the down projection adds them
+            fhip::F16Parts parts{nullptr, 0, 0, 0, 0};
+            if (!(rc = f16x2_matmul(gu, d_x + m0 * gu->cols, t, false, g, ws, s, &parts)))
+                rc = f16x2_matmul(down, g, t, true, d_y + m0 * down->rows, ws2, s, nullptr, &parts);
         }
         if (rc) return rc;
     }

@@ -124,12 +124,22 @@ size_t gemm_f16x2_xp_bytes(const fhip_weight* w, size_t t);       // prepared-ac
 bool gemm_f16x2_adds_into_y(const fhip_weight* w, size_t t);      // true: the launch adds into y, a cleared y saves it a launch
 // splits the rows of x [t, cols] (swiglu: of silu(gate) * up of x [t, 2 cols]) chunk by chunk into scaled f16 hi / lo
 // operand rows, each carrying the factor that takes its scale out again
+// Where the K-split groups of a matmul's output still lie as partial sums, one slot per (128-output group, contributor):
+// output n of activation row t is slot 0 + slot 1 + ... of its group in that order (one contributor: the value in y itself).
+struct F16Parts {
+    const float* part;    // null: every output is in y
+    int kmax, nchunks, grid;
+    long long units;
+};
+// src: x is the output of a matmul whose ordered sum was left to this launch (launch_gemm_f16x2 with `deferred`)
 int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero = nullptr,
-                      size_t zero_n = 0);
+                      size_t zero_n = 0, const F16Parts* src = nullptr);
 // d_part: null, or gemm_f16x2_part_bytes(w, t) bytes: partial sums of K-split groups go there and are added in a fixed
 // order by a launch behind the matmul (y then needs no clearing) instead of being added into y atomically
+// deferred: with d_part, the launch that adds the partial sums is left out and *deferred says where they lie; the reader of y
+// (launch_xsplit_f16 with `src`) adds them in the same order
 int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared = false,
-                      float* d_part = nullptr);
+                      float* d_part = nullptr, F16Parts* deferred = nullptr);
 size_t gemm_f16x2_part_bytes(const fhip_weight* w, size_t t);
 size_t gemm_f16x2_part_bytes_upto(const fhip_weight* w, size_t t);   // the largest over batches of 1..t rows
 

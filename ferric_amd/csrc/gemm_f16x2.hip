@@ -416,19 +416,39 @@ struct Q80 {
 // ------------------------------------------------------------------------------------------------
 constexpr int MAXW = 64;   // rows of up to 65 536 columns
 
+// Workgroup b of G takes units [b U / G, (b + 1) U / G): the workgroup that holds unit u
+__device__ __host__ __forceinline__ int holder_of(long long u, long long G, long long U) { return (int)(((u + 1) * G - 1) / U); }
+
+// element n of row t of the matrix the split reads: as stored, or, where the producing matmul left a K-split group's
+// partial sums to this launch, slot 0 + slot 1 + ... of that group (the order sum_split_kernel adds them in)
+__device__ __forceinline__ float x_at(const float* __restrict__ x, int t, size_t n, const fhip::F16Parts& src) {
+    if (src.part) {
+        const int grp = (int)(n >> 7);
+        const int first = holder_of((long long)grp * src.nchunks, src.grid, src.units);
+        const int nk = holder_of((long long)(grp + 1) * src.nchunks - 1, src.grid, src.units) - first + 1;
+        if (nk > 1) {
+            const float* q = src.part + ((size_t)grp * src.kmax * 32 + t) * 128 + (n & 127);
+            float a = q[0];
+            for (int k = 1; k < nk; k++) a += q[(size_t)k * (32 * 128)];
+            return a;
+        }
+    }
+    return x[n];
+}
+
 template <bool SWIGLU>
-__device__ __forceinline__ float act(const float* __restrict__ x, int K, int k) {
+__device__ __forceinline__ float act(const float* __restrict__ x, int t, int K, int k, const fhip::F16Parts& src) {
     if (SWIGLU) {
-        const float g = x[k], u = x[(size_t)K + k];
+        const float g = x_at(x, t, k, src), u = x_at(x, t, (size_t)K + k, src);
         return (g / (1.0f + expf(-g))) * u;
     }
-    return x[k];
+    return x_at(x, t, k, src);
 }
 
 // one workgroup per (chunk, operand row of a group of 8): thread k of it converts column k of the chunk
 template <class F, bool SWIGLU>
 __global__ void __launch_bounds__(256) xsplit_f16_kernel(const float* __restrict__ X, int T, int K, int NT, uint16_t* __restrict__ Xp,
-                                                       float* __restrict__ zero, size_t zero_n) {
+                                                       float* __restrict__ zero, size_t zero_n, fhip::F16Parts src) {
     __shared__ float red[4];
     const int tid = threadIdx.x, lane = tid & 63;
     const size_t nwg = (size_t)gridDim.x * gridDim.y;
@@ -437,7 +457,7 @@ __global__ void __launch_bounds__(256) xsplit_f16_kernel(const float* __restrict
     const bool live = t < T;
     const int k = ck * CHUNK + tid;
     const float* x = X + (size_t)(live ? t : 0) * (SWIGLU ? 2 * (size_t)K : (size_t)K);
-    const float raw = (live && k < K) ? act<SWIGLU>(x, K, k) : 0.f;
+    const float raw = (live && k < K) ? act<SWIGLU>(x, live ? t : 0, K, k, src) : 0.f;
     // the chunk's largest magnitude (a NaN is not one: it reaches the operands as it is and makes the output row NaN)
     float m = fabsf(raw);
 #pragma unroll
@@ -490,8 +510,6 @@ struct F16Params {
     int kmax;
 };
 
-// Workgroup b of G takes units [b U / G, (b + 1) U / G): the workgroup that holds unit u
-__device__ __host__ __forceinline__ int holder_of(long long u, long long G, long long U) { return (int)(((u + 1) * G - 1) / U); }
 // where a partial output (activation row t, output n of group grp) goes in ordered mode
 __device__ __forceinline__ float* part_slot(const F16Params& p, int grp, int t, int n) {
     const int k = (int)blockIdx.x - holder_of((long long)grp * p.nchunks, gridDim.x, p.units);
@@ -910,15 +928,15 @@ Plan make_plan(const fhip_weight* w, size_t t) {
 
 template <class F>
 int launch_xsplit_fmt(const float* d_x, size_t t, size_t k, bool swiglu, const Plan& q, uint16_t* d_xp, hipStream_t s, float* zero,
-                      size_t zero_n) {
+                      size_t zero_n, const fhip::F16Parts& src) {
     const dim3 grid((unsigned)q.nchunks, (unsigned)(8 * q.nt)), wg(256);
-    if (swiglu) hipLaunchKernelGGL((xsplit_f16_kernel<F, true>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_xp, zero, zero_n);
-    else hipLaunchKernelGGL((xsplit_f16_kernel<F, false>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_xp, zero, zero_n);
+    if (swiglu) hipLaunchKernelGGL((xsplit_f16_kernel<F, true>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_xp, zero, zero_n, src);
+    else hipLaunchKernelGGL((xsplit_f16_kernel<F, false>), grid, wg, 0, s, d_x, (int)t, (int)k, q.nt, d_xp, zero, zero_n, src);
     return fhip::check_hip(hipGetLastError(), "xsplit_f16 launch");
 }
 
 template <class F>
-int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_part) {
+int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_part, fhip::F16Parts* deferred) {
     const Plan q = make_plan(w, t);
     F16Params p;
     p.W = w->d_raw; p.Xp = d_xp; p.Y = d_y;
@@ -938,7 +956,8 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y,
     } else {
         return fhip::set_error(FHIP_ERR_SHAPE, "f16x2 matmul: this format takes at most 16 activation rows, got %zu", t);
     }
-    if (p.part)
+    if (deferred) *deferred = fhip::F16Parts{p.part, p.kmax, p.nchunks, (int)q.grid, p.units};
+    if (p.part && !deferred)
         hipLaunchKernelGGL(sum_split_kernel, dim3((unsigned)q.groups, (unsigned)((t + 1) / 2)), dim3(256), 0, s, d_y, (const float*)d_part, p.T, p.N,
                            p.nchunks, p.units, (int)q.grid, p.kmax);
     return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
@@ -973,23 +992,26 @@ size_t gemm_f16x2_part_bytes_upto(const fhip_weight* w, size_t t) {
     return m;
 }
 
-int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero, size_t zero_n) {
+int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero, size_t zero_n,
+                      const F16Parts* src_in) {
     const Plan q = make_plan(w, t);
+    const F16Parts src = src_in ? *src_in : F16Parts{nullptr, 0, 0, 0, 0};
     switch (w->type) {
-        case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
-        case FHIP_Q5_K: return launch_xsplit_fmt<Q5K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
-        case FHIP_Q6_K: return launch_xsplit_fmt<Q6K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
-        case FHIP_Q8_0: return launch_xsplit_fmt<Q80>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n);
+        case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n, src);
+        case FHIP_Q5_K: return launch_xsplit_fmt<Q5K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n, src);
+        case FHIP_Q6_K: return launch_xsplit_fmt<Q6K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n, src);
+        case FHIP_Q8_0: return launch_xsplit_fmt<Q80>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n, src);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
     }
 }
 
-int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_part) {
+int launch_gemm_f16x2(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y, hipStream_t s, bool y_cleared, float* d_part,
+                      F16Parts* deferred) {
     switch (w->type) {
-        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, t, d_y, s, y_cleared, d_part);
-        case FHIP_Q5_K: return launch_fmt<Q5K>(w, d_xp, t, d_y, s, y_cleared, d_part);
-        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, t, d_y, s, y_cleared, d_part);
-        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, t, d_y, s, y_cleared, d_part);
+        case FHIP_Q4_K: return launch_fmt<Q4K>(w, d_xp, t, d_y, s, y_cleared, d_part, deferred);
+        case FHIP_Q5_K: return launch_fmt<Q5K>(w, d_xp, t, d_y, s, y_cleared, d_part, deferred);
+        case FHIP_Q6_K: return launch_fmt<Q6K>(w, d_xp, t, d_y, s, y_cleared, d_part, deferred);
+        case FHIP_Q8_0: return launch_fmt<Q80>(w, d_xp, t, d_y, s, y_cleared, d_part, deferred);
         default: return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "f16x2 matmul: no kernel for ggml type %u", w->type);
     }
 }

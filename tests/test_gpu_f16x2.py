@@ -328,8 +328,18 @@ def test_ordered_policy_gives_the_same_bits_on_every_run(F, O):
         y = xt.ffn(wgu, wdn).to_vec()
         for _ in range(3):
             assert np.array_equal(xt.ffn(wgu, wdn).to_vec(), y)
+        # the block leaves gate|up's partial sums to the launch that prepares the down projection's activations; the three
+        # calls it stands for add them in a launch of their own, in the same order: the same bits
+        steps = xt.try_matmul_swiglu(wgu).matmul_q(wdn).to_vec()
+        assert np.array_equal(steps, y)
         wgu.batch_policy(0), wdn.batch_policy(0)
         y0 = xt.ffn(wgu, wdn).to_vec()                 # FHIP_BATCH_AUTO: atomic adds, the same sums in another order
         assert np.abs(y - y0).max() <= 2e-6 * np.abs(y0).max()
+        # a ragged block (hidden width not a multiple of 128, three rows) in one call and in three
+        n_embd, n_ff, batch = 768, 1280 + 256, 3
+        wgu = F.QMatrix.from_bytes(synth_weights(Q4_K, 2 * n_ff, n_embd, 33), Q4_K, 2 * n_ff, n_embd)
+        wdn = F.QMatrix.from_bytes(synth_weights(Q6_K, n_embd - 1, n_ff, 34), Q6_K, n_embd - 1, n_ff)
+        xt = F.Tensor.from_vec(np.random.default_rng(35).standard_normal((batch, n_embd)).astype(np.float32), (batch, n_embd))
+        assert np.array_equal(xt.try_matmul_swiglu(wgu).matmul_q(wdn).to_vec(), xt.ffn(wgu, wdn).to_vec())
     finally:
         lib.fhip_batch_policy(before)
