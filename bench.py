@@ -731,7 +731,8 @@ def probe(F, lib, check):
     reads HBM: 512 launches of the headline Q4_K 5120 x 5120 (the O projection's shape too) over 64 copies, 256 of the fused
     QKV 7168 x 5120 over 40, 64 of gate|up 34816 x 5120 with SwiGLU over 8, 64 of down 5120 x 17408 Q6_K over 10, 512 of Q8_0
     4096 x 4096 over 56 and 8 of the vocabulary head 151936 x 5120 Q6_K over 2. The launches of a shape are enqueued back to
-    back from native code (fhip_debug_matmul_q_loop), so the device sees the steady stream a captured graph would give it."""
+    back from native code (fhip_debug_matmul_q_loop), so the device sees the steady stream a captured graph would give it.
+    Every shape runs twice: with 16-bit activations (what `value` is quoted on), then with 24-bit ones (what a new handle has)."""
     from ferric_amd.synth import synth_weights
     n = 256 << 20
     src, dst = F.DeviceBuffer(n), F.DeviceBuffer(n)
@@ -750,8 +751,11 @@ def probe(F, lib, check):
         buf = replicate(F, lib, check, host, ncopy)
         ws = [F.QMatrix.wrap_device(buf, host.size, ty, rows, cols, offset=i * host.size) for i in range(ncopy)]
         handles = (C.c_void_p * ncopy)(*[w.handle for w in ws])
-        check(lib.fhip_debug_matmul_q_loop(handles, ncopy, launches, xin.buf.ptr, 1 if swiglu else 0, y.buf.ptr, None))
-        check(lib.fhip_stream_sync(None))
+        for bits in (16, 24):       # the kernels carry the precision in their names: ..._p2 (16-bit activations), ..._p3 (24)
+            for w in ws:
+                w.matvec_precision(bits)
+            check(lib.fhip_debug_matmul_q_loop(handles, ncopy, launches, xin.buf.ptr, 1 if swiglu else 0, y.buf.ptr, None))
+            check(lib.fhip_stream_sync(None))
         del ws, buf
 
 

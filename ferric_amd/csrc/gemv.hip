@@ -48,7 +48,8 @@
 #include <type_traits>
 
 // This file is compiled twice, once per activation precision (FHIP_GEMV_PLANES = 2 and 3); the two copies export their
-// launchers under different names and fhip_matvec_precision() picks between them at run time.
+// launchers under different names and the precision of the weight handle picks between them at every launch. The kernel
+// carries the suffix too, so that a profiler's trace says which copy ran.
 #ifndef FHIP_GEMV_PLANES
 #define FHIP_GEMV_PLANES 2
 #endif
@@ -57,6 +58,7 @@
 #else
 #define GEMV_EXPORT(name) name##_p3
 #endif
+#define gemv_stream_kernel GEMV_EXPORT(gemv_stream_kernel)
 
 namespace {
 
