@@ -598,6 +598,23 @@ def bench_decode(F, lib, check, stream, timer, contexts=(128, 4096, 32768), laye
                          "kv_bytes_read": kv_bytes, "GBps_weights_plus_kv": (weight_bytes_total + kv_bytes) / (ms * 1e-3) / 1e9,
                          "logits_finite": bool(np.isfinite(logits).all())}
         del dec
+    # the figures above are on weight handles as the library makes them (24-bit activations in the mat-vecs); the same step
+    # with the handles switched to 16-bit activations, the precision `value` is quoted on
+    def set_bits(bits):
+        for L in lay:
+            for w in (L.wqkv, L.wo, L.ffn_gate_up, L.ffn_down):
+                w.matvec_precision(bits)
+        head.matvec_precision(bits)
+    set_bits(16)
+    for ctx in contexts[:2]:
+        dec = decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, steps, stream, rng)
+        dec.capture()
+        dec.step_graph()
+        ms = timer.time_ms(lambda: [dec.step_graph() for _ in range(steps)]) / steps
+        out[str(ctx)]["ms_per_token_x16"] = ms
+        del dec
+    set_bits(24)
+    out["activation_bits"] = 24
     # the same step on a Q8_0 block-quantized cache, attention reading the blocks in place (8.5 bits per cached value)
     ctx = contexts[-1]
     dec = decoder_at_context(F, lib, check, cfg, lay, small, head, ctx, steps, stream, rng, kv_fmt=0)
@@ -783,8 +800,8 @@ def probe_prefill(F, lib, check):
 
 def probe_f16x2(F, lib, check, ncopy=4):
     """Work for a profiler run of the small-batch f16 matrix-core path at 8 activation rows: fhip_matmul_q_f16x2 on the
-    gate|up (34816 x 5120 Q4_K) and down (5120 x 17408 Q6_K) weights, then the whole block through fhip_ffn_f16x2, 12
-    launches each, eagerly on the null stream, rotating over 4 copies of each weight (694 MB in all, more than the
+    gate|up (34816 x 5120 Q4_K) and down (5120 x 17408 Q6_K) weights, then the whole block through fhip_ffn_f16x2 and through
+    fhip_ffn (ordered sums), 12 launches each, eagerly on the null stream, rotating over 4 copies of each weight (694 MB in all, more than the
     Infinity Cache holds) so that every launch reads HBM. Last, 32 launches of fhip_matmul_q_f16x2 over 32 copies of a
     4096 x 4096 Q8_0 weight (571 MB) and 16 over 16 copies of a 12288 x 4096 one (857 MB), 8 rows each."""
     from ferric_amd.synth import synth_weights
@@ -807,6 +824,12 @@ def probe_f16x2(F, lib, check, ncopy=4):
     ws = F.DeviceBuffer(lib.fhip_ffn_f16x2_ws_bytes(gus[0].handle, dns[0].handle, t))
     for i in range(12):
         check(lib.fhip_ffn_f16x2(gus[i % ncopy].handle, dns[i % ncopy].handle, x.buf.ptr, t, y.buf.ptr, ws.ptr, None))
+    check(lib.fhip_stream_sync(None))
+    # the drop-in call on the same weights: handles as the library makes them add the partial sums of cut rows in a fixed
+    # order (FHIP_BATCH_ORDERED) instead of atomically, gate|up's inside the split for the down projection
+    hws = F.Tensor.empty((t, n_ff))
+    for i in range(12):
+        check(lib.fhip_ffn(gus[i % ncopy].handle, dns[i % ncopy].handle, x.buf.ptr, t, y.buf.ptr, hws.buf.ptr, None))
     check(lib.fhip_stream_sync(None))
     del gus, dns, gbuf, dbuf
     for rows, nc in ((4096, 32), (12288, 16)):
