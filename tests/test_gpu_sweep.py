@@ -140,6 +140,64 @@ def test_layers_of_the_sweep_chained_in_one_graph(F, O):
     check_rows(O, logits.to_vec(stream), x, head_raw, Q6_K, 5120, [(0, 3001)], "head")
 
 
+def test_layers_chained_output_to_input_in_one_graph(F, O):
+    """Two layers of the same four projections with every launch reading the launch before it, as the benchmark's chained
+    sweep does: x -> rmsnorm + QKV -> O (on the first 5120 of the QKV row) -> rmsnorm + gate|up + SwiGLU -> down -> next layer,
+    the norms fused into the mat-vecs that consume them (fhip_norm_matmul_q), one captured graph replayed twice. The oracle
+    walks the same chain in f64 from the device's own input of each step, so every step is held to the mat-vec's bar by itself,
+    and the end of the chain to the product of the steps."""
+    from ferric_amd.synth import synth_weights
+    lib = F._lib.load()
+    check = F._lib.check
+    shapes = [("qkv", Q4_K, 7168, 5120, 0), ("o", Q4_K, 5120, 5120, 0), ("gate_up", Q4_K, 34816, 5120, 1), ("down", Q6_K, 5120, 17408, 0)]
+    layers, eps = 2, 1e-6
+    rng = np.random.default_rng(71)
+    x0 = rng.standard_normal(5120).astype(np.float32)
+    nw = ((rng.random(5120) + 0.5) * 0.01).astype(np.float32)      # small norm weights keep the chain inside the f32 range
+    raws, ws = {}, {}
+    for l in range(layers):
+        for i, (name, ty, r, c, sw) in enumerate(shapes):
+            raws[l, name] = synth_weights(ty, r, c, 300 + 10 * l + i)
+            ws[l, name] = F.QMatrix.from_bytes(raws[l, name], ty, r, c)
+    T = lambda n: F.Tensor.empty((1, n))
+    xt, nwt, scratch = F.Tensor.from_vec(x0, (1, 5120)), F.Tensor.from_vec(nw, (1, 5120)), T(5120)
+    bufs = {(l, name): T(r // 2 if sw else r) for l in range(layers) for name, ty, r, c, sw in shapes}
+    stream = F.Stream()
+    g = F.Graph.begin(stream)
+    cur = xt
+    for l in range(layers):
+        check(lib.fhip_norm_matmul_q(ws[l, "qkv"].handle, cur.buf.ptr, None, nwt.buf.ptr, eps, None, scratch.buf.ptr, 0, bufs[l, "qkv"].buf.ptr, stream.handle))
+        check(lib.fhip_matmul_q(ws[l, "o"].handle, bufs[l, "qkv"].buf.ptr, 1, bufs[l, "o"].buf.ptr, stream.handle))
+        check(lib.fhip_norm_matmul_q(ws[l, "gate_up"].handle, bufs[l, "o"].buf.ptr, None, nwt.buf.ptr, eps, None, scratch.buf.ptr, 1, bufs[l, "gate_up"].buf.ptr, stream.handle))
+        check(lib.fhip_matmul_q(ws[l, "down"].handle, bufs[l, "gate_up"].buf.ptr, 1, bufs[l, "down"].buf.ptr, stream.handle))
+        cur = bufs[l, "down"]
+    g.end()
+    for replay in range(2):
+        g.launch()
+        stream.synchronize()
+
+    def norm64(v):
+        v = v.astype(np.float64)
+        return v / np.sqrt((v * v).mean() + eps) * nw.astype(np.float64)
+
+    got = {k: b.to_vec(stream).astype(np.float32) for k, b in bufs.items()}
+    prev = x0
+    for l in range(layers):
+        for name, ty, r, c, sw in shapes:
+            xin = norm64(prev) if name in ("qkv", "gate_up") else prev[:c].astype(np.float64)
+            y64, wn = O.matmul_f64(xin.astype(np.float32)[None, :], raws[l, name], ty, r, c)
+            # the oracle's input is rounded to f32 where the device's staged row is f32 too; the bound covers the difference
+            if sw:
+                gate, up = y64[0, :r // 2], y64[0, r // 2:]
+                want = gate / (1.0 + np.exp(-gate)) * up
+            else:
+                want = y64[0]
+            err = np.abs(got[l, name] - want)
+            assert err.max() <= 2 * dot_bar() * np.abs(want).max(), (l, name, float(err.max() / np.abs(want).max()))
+            prev = got[l, name]            # the next step starts from what the device produced
+    assert np.isfinite(got[layers - 1, "down"]).all() and np.abs(got[layers - 1, "down"]).max() > 0
+
+
 @pytest.mark.parametrize("ty,rows,cols,swiglu", [(Q4_K, 12301, 5120, False), (Q4_K, 2 * 12303, 5120, True), (Q6_K, 4099, 17408, False),
                                                  (Q8_0, 33001, 1024, False)])
 def test_large_weights_whose_rows_are_dealt_in_chunks_of_four(F, O, ty, rows, cols, swiglu):
