@@ -45,6 +45,7 @@
 
 #include <hip/hip_fp16.h>
 
+#include <cstddef>
 #include <type_traits>
 
 // This file is compiled twice, once per activation precision (FHIP_GEMV_PLANES = 2 and 3); the two copies export their
@@ -636,7 +637,7 @@ struct GemvParams {
     float* y;            // [M, out_rows]
     int out_rows;        // rows of y (n_ff when fused SwiGLU)
     int cols;
-    size_t row_bytes;
+    uint32_t row_bytes;  // below 2^32 (rows of at most ~40 000 columns): a row's address is one 32 x 32 -> 64 bit product
     size_t pair_bytes;   // fused SwiGLU: byte distance from gate row r to up row r (= n_ff * row_bytes)
     int NG;              // 16-lane slots per row = ceil(units / 16)
     int units;           // units per row = cols / WPL; the last slot may be partly filled
@@ -647,7 +648,12 @@ struct GemvParams {
     // ceil(2^32 / d) for the three divisors of the kernel's index arithmetic (waves per row group, full waves per row, RF), 0
     // for d = 1: floor(n / d) = mulhi(n, magic) for n < 65 536, 2 <= d <= 1024; a hardware-less integer division costs ~35
     // dependent instructions, and four of them stood in front of the first load
-    uint32_t m_wpr, m_ngf, m_rf, m_rpg;
+    uint32_t m_rf, m_rpg;
+    // What wave w of a workgroup is, worked out by the launcher once instead of by every wave in front of its first load
+    // (wave_word): bits 0-3 its row group in the workgroup, 4-7 the first virtual row it takes, 8 set for the tail wave of a
+    // row group, 9-10 the slots the tail holds (NG % 4), 11-18 the first slot of its four, 19-20 log2 of the rows a tail wave
+    // works on at once.
+    uint32_t wtab[16];
     // Dealing of rows to row groups. rr == 0: row group g owns the rpg consecutive rows from g * rpg. rr == 1 (large weights):
     // the rows are dealt in chunks of 4, chunk c to row group c % nrg, so that at any moment the whole chip reads one dense
     // window of the weight that moves through it (measured 3 - 5 % faster than 768 separate streams on the FFN shapes);
@@ -752,19 +758,32 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
     // every phase): up to four 8-value pieces per thread, all requested here so that they arrive under one memory round
     // trip. The other waves go straight to their weight rows and meet the stagers at the barrier.
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // What this wave is (wtab), wave-uniform: one scalar load straight from the kernel-argument segment (the struct is the kernel's only argument, so
+    // its fields lie at their offsets there; indexing the by-value copy with a run-time index would move all of it to scratch)
+    typedef const uint32_t __attribute__((address_space(4))) karg_word;
+    const uint32_t ww = ((karg_word*)__builtin_amdgcn_kernarg_segment_ptr())[offsetof(GemvParams, wtab) / 4 + wave];
     const bool stager = wave < p.S;
     const int e0 = stager ? tid * 8 : M * p.cols, e_step = p.S * 512;
-    float4 xa0 = {0, 0, 0, 0}, xb0 = {0, 0, 0, 0};
-    if (e0 < M * p.cols) { xa0 = *(const float4*)(p.x + e0); xb0 = *(const float4*)(p.x + e0 + 4); }
-    constexpr int XR = 3;
-    float4 xar[XR], xbr[XR];
-#pragma unroll
-    for (int k = 0; k < XR; k++) {
-        const int e = e0 + (k + 1) * e_step;
-        xar[k] = xbr[k] = float4{0, 0, 0, 0};
-        if (e < M * p.cols) { xar[k] = *(const float4*)(p.x + e); xbr[k] = *(const float4*)(p.x + e + 4); }
-    }
+    // A staging wave asks for its pieces unconditionally, from a clamped address: a piece past the end is loaded from a
+    // place inside the row instead and never used (under a condition each piece cost eight register clears and a branch
+    // in front of the wave's first weight request). A wave that does not stage skips them in one branch and leaves the
+    // registers as they are: nothing reads them (every wave re-reading the one last line: 5120 x 5120 5.37 -> 5.94 us).
     constexpr bool fused_norm = NORM && M == 1;   // a separate instantiation: the plain kernel carries none of this
+    constexpr int XR = 3;
+    float4 xa0, xb0, xar[XR], xbr[XR];
+    if (stager) {
+        const int e_last = M * p.cols - 8, e_own = e0 < e_last ? e0 : e_last;
+        // (a later piece past the end re-reads the thread's own first piece, not the row's last: many threads on one line wait)
+        auto piece = [&](int e) { return p.x + (e <= e_last ? e : e_own); };
+        xa0 = *(const float4*)(p.x + e_own); xb0 = *(const float4*)(p.x + e_own + 4);
+        if constexpr (!fused_norm) {               // under the fused norm a thread holds at most one piece of the row
+#pragma unroll
+            for (int k = 0; k < XR; k++) {
+                const float* src = piece(e0 + (k + 1) * e_step);
+                xar[k] = *(const float4*)src; xbr[k] = *(const float4*)(src + 4);
+            }
+        }
+    }
     float4 nwa = {1, 1, 1, 1}, nwb = {1, 1, 1, 1}, rsa = {0, 0, 0, 0}, rsb = {0, 0, 0, 0};
     if (fused_norm && e0 < p.cols) {              // the norm's weights and the residual ride with the activations
         nwa = *(const float4*)(p.norm_w + e0); nwb = *(const float4*)(p.norm_w + e0 + 4);
@@ -782,14 +801,13 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
         }
         return;
     }
-    const int NGF = p.NG >> 2, NT = p.NG & 3, NFW = NGF * p.RF, WPR = NFW + (NT ? 1 : 0);
-    const int rg = (int)div_magic((uint32_t)wave, p.m_wpr), wr = wave - rg * WPR;   // row group within workgroup, wave within row group
-    const int wq = (int)div_magic((uint32_t)wr, p.m_ngf), wm = wr - wq * NGF;       // wr / NGF, wr % NGF (NGF = 0: never used)
-    const bool tail = wr == NFW;                         // wave-uniform
-    const int RTL = tail ? (NT == 1 ? 2 : NT == 2 ? 1 : 0) : 0;   // log2 of the rows this wave works on at once
+    const int rg = (int)(ww & 15u);                       // row group within the workgroup
+    const bool tail = ((ww >> 8) & 1u) != 0;
+    const int NT = (int)((ww >> 9) & 3u), gbase = (int)((ww >> 11) & 255u);
+    const int RTL = (int)((ww >> 19) & 3u);               // log2 of the rows this wave works on at once (0 unless tail)
     const int RT = 1 << RTL;
     // iteration i of this wave works on virtual row v_start + i * v_step (+ row_off per lane in a tail wave)
-    const int v_start = tail ? 0 : wq, v_step = tail ? RT : p.RF;
+    const int v_start = (int)((ww >> 4) & 15u), v_step = tail ? RT : p.RF;
 
     // LDS: activation planes | scales [M][NRUN][units] | sums [M][NRUN][units] | partials. The planes are laid out for the
     // readers: the 16-byte piece c of plane pp of run j of unit u (of activation row m) sits at
@@ -806,9 +824,9 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
     const int slot = lane >> 4, l16 = lane & 15;
     int group, row_off;
     bool lane_ok = true;
-    if (!tail) { group = 4 * wm + slot; row_off = 0; }
-    else if (NT == 3) { lane_ok = slot < 3; group = 4 * NGF + (lane_ok ? slot : 0); row_off = 0; }
-    else { group = 4 * NGF + (NT == 2 ? (slot & 1) : 0); row_off = NT == 2 ? (slot >> 1) : slot; }
+    if (!tail) { group = gbase + slot; row_off = 0; }
+    else if (NT == 3) { lane_ok = slot < 3; group = gbase + (lane_ok ? slot : 0); row_off = 0; }
+    else { group = gbase + (NT == 2 ? (slot & 1) : 0); row_off = NT == 2 ? (slot >> 1) : slot; }
     typename F::Lane L;
     int run[NRUN];
     // a lane past the row's last unit (rows whose length does not fill the last slot) works on unit 0 and contributes 0
@@ -818,7 +836,44 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
 
     const int rgid = blockIdx.x * p.G + rg;
     const bool dealt = F::RR && p.rr != 0;             // rows dealt round-robin in chunks of 4
-    const int r0 = dealt ? 0 : rgid * p.rpg;              // rr: the row group's rows are spread over the weight, see row_base
+    // Address of iteration `it`: a wave-uniform row base (scalar registers) plus a 32-bit lane offset. A tail
+    // wave's lanes sit row_off rows further (v_start + it*v_step is a multiple of RT there, so with fused
+    // SwiGLU the gate/up split of row_off is fixed); lanes past the last row read the uniform row instead
+    // and are masked when the partial is written.
+    const uint32_t lane_extra = SWIGLU ? (uint32_t)((size_t)(row_off >> 1) * p.row_bytes + (size_t)(row_off & 1) * p.pair_bytes)
+                                       : (uint32_t)((size_t)row_off * p.row_bytes);
+    // row l of the row group is row l of its span, or, dealt (rr): row l % 4 of the row group's chunk l / 4, which is chunk
+    // (l / 4) * nrg + rgid of the weight. A tail wave's RT rows start at a multiple of RT <= 4, so they lie in one chunk and
+    // lane_extra holds as it stands.
+    auto weight_row = [&](int l) { return dealt ? ((((l >> 2) * p.nrg + rgid) << 2) + (l & 3)) : rgid * p.rpg + l; };
+
+    // ---- The activation loads went out first; now the weight bytes of the wave's first row, UNCONDITIONALLY and from an
+    // address that needs as little arithmetic as possible: the row the wave would start on, clamped to the weight's last
+    // row (a wave or a lane without a share loads a row that exists and drops it). How many rows the wave owns, how many
+    // iterations that makes and where the later rows lie is worked out behind this load, under its latency: a CU has one
+    // scalar unit, a SIMD's four waves get one scalar instruction in 16 cycles each while they all run this prologue, and
+    // every instruction in front of the first weight request is paid by the whole launch (5120 x 5120: with the
+    // launch geometry as compile-time constants, 95 instructions fewer in front of the load, 5.51 -> 5.26 us).
+    // Loads return in issue order, so the wait for the activations is a counted one only if the compiler knows how many
+    // loads follow them; behind a conditional load it has to drain the queue, and the quantisation below then waits for
+    // every prefetched row of the wave. The rest of the prefetch goes out behind the quantisation.
+    typename F::Data buf[U];
+    // One row in flight per wave (the long Q6_K rows, whose staging takes four passes and is what the launch waits for): the
+    // first row is requested behind the share arithmetic as before, so that it does not stand in front of the younger
+    // workgroups' activation loads any earlier (5120 x 17408: 16.5 us; requested early 16.7).
+    constexpr bool EARLY = U > 1;
+    if constexpr (EARLY) {
+        const int l0 = SWIGLU ? v_start >> 1 : v_start;
+        const int last = p.out_rows - 1;
+        int row = weight_row(l0);
+        const bool lane_row_ok = row + (SWIGLU ? row_off >> 1 : row_off) <= last;
+        row = row < last ? row : last;
+        const uint8_t* first = p.W + (size_t)(uint32_t)row * p.row_bytes + (SWIGLU && (v_start & 1) ? p.pair_bytes : (size_t)0);
+        buf[0] = F::load(first, L, lane_row_ok ? lane_extra : 0u);
+    }
+    asm volatile("" ::: "memory");
+
+    const int r0 = dealt ? 0 : rgid * p.rpg;              // rr: the row group's rows are spread over the weight, see weight_row
     int nrows = p.out_rows - r0;
     if (dealt) {                                         // kfull whole chunks and what the last round leaves this row group
         int last = p.rem - rgid * 4;
@@ -827,38 +882,25 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
     }
     nrows = nrows < 0 ? 0 : (nrows > p.rpg ? p.rpg : nrows);
     const int nv = nrows * VPR;                          // virtual rows: v -> the row group's row v/VPR (+ pair for odd v)
-    const uint8_t* base = p.W + (size_t)(nrows > 0 ? r0 : 0) * p.row_bytes;   // a row group past the end points at row 0
     // (nv - v_start + v_step - 1) / v_step with v_step = 4, 2, 1 (tail wave) or RF
     const uint32_t n_num = (uint32_t)(nv - v_start + v_step - 1);
     const int n_it = nv > v_start ? (int)(tail ? n_num >> RTL : div_magic(n_num, p.m_rf)) : 0;
     // iterations all of whose rows exist (a tail wave's last iteration may hold fewer than RT)
     const int n_full = tail ? nv >> RTL : n_it;
-    // Address of iteration `it`: a wave-uniform row base (scalar registers) plus a 32-bit lane offset. A tail
-    // wave's lanes sit row_off rows further (v_start + it*v_step is a multiple of RT there, so with fused
-    // SwiGLU the gate/up split of row_off is fixed); lanes past the last row read the uniform row instead
-    // and are masked when the partial is written.
-    const uint32_t lane_extra = SWIGLU ? (uint32_t)((size_t)(row_off >> 1) * p.row_bytes + (size_t)(row_off & 1) * p.pair_bytes)
-                                       : (uint32_t)((size_t)row_off * p.row_bytes);
+    const uint8_t* base = p.W + (size_t)(uint32_t)(nrows > 0 ? r0 : 0) * p.row_bytes;   // a row group past the end points at row 0
     auto row_base = [&](int it) -> const uint8_t* {
         const int v = v_start + it * v_step;             // wave-uniform
         int l = SWIGLU ? v >> 1 : v;                     // row of the row group
-        // rr: row l is row l % 4 of the row group's chunk l / 4, which is chunk (l / 4) * nrg + rgid of the weight. A tail
-        // wave's RT rows start at a multiple of RT <= 4, so they lie in one chunk and lane_extra holds as it stands.
-        if (dealt) l = (((l >> 2) * p.nrg + rgid) << 2) + (l & 3);
-        return SWIGLU ? base + (size_t)l * p.row_bytes + (size_t)(v & 1) * p.pair_bytes : base + (size_t)l * p.row_bytes;
+        if (dealt) l = (((l >> 2) * p.nrg + rgid) << 2) + (l & 3);   // as weight_row, from row 0 (r0 = 0)
+        return SWIGLU ? base + (size_t)(uint32_t)l * p.row_bytes + (size_t)(v & 1) * p.pair_bytes : base + (size_t)(uint32_t)l * p.row_bytes;
     };
     auto lane_eo = [&](int it) { return (v_start + it * v_step + row_off < nv) ? lane_extra : 0u; };
     auto fetch = [&](int it) { return F::load(row_base(it), L, lane_eo(it)); };
     auto fetch_full = [&](int it) { return F::load(row_base(it), L, lane_extra); };   // it < n_full: every lane's row exists
-
-    // ---- the activation loads went out first; now the weight bytes of the wave's first row, UNCONDITIONALLY (a wave
-    // without rows reads the weight's row 0 and drops it). Loads return in issue order, so the wait for the activations
-    // is a counted one only if the compiler knows how many loads follow them; behind a conditional load it has to drain
-    // the queue, and the quantisation below then waits for every prefetched row of the wave (seconds of microseconds on
-    // the large shapes, during which the memory pipe runs dry). The rest of the prefetch goes out behind the quantisation.
-    typename F::Data buf[U];
-    buf[0] = F::load(n_it > 0 ? row_base(0) : p.W, L, n_it > 0 ? lane_eo(0) : 0u);
-    asm volatile("" ::: "memory");
+    if constexpr (!EARLY) {
+        buf[0] = F::load(n_it > 0 ? row_base(0) : p.W, L, n_it > 0 ? lane_eo(0) : 0u);
+        asm volatile("" ::: "memory");
+    }
 
     if (fused_norm) {
         // x <- rmsnorm(x + resid) * norm_w (crates/ferric-tensor/src/lib.rs:2057-2074): each thread holds at most one
@@ -874,6 +916,7 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
         }
         float ss = fmaf(xa0.x, xa0.x, fmaf(xa0.y, xa0.y, fmaf(xa0.z, xa0.z, xa0.w * xa0.w)))
                  + fmaf(xb0.x, xb0.x, fmaf(xb0.y, xb0.y, fmaf(xb0.z, xb0.z, xb0.w * xb0.w)));
+        if (e0 >= p.cols) ss = 0.f;                           // a thread past the row holds a copy of the last piece
         ss = slot_sum(ss);                                    // four 16-lane sums per wave, no trip through LDS to combine them
         float* red = (float*)(smem + p.red_off);
         if ((lane & 15) == 0) red[wave * 4 + (lane >> 4)] = ss;
@@ -899,13 +942,15 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
         if (within == 0) { scales[mj * p.units + u] = scale; sums[mj * p.units + u] = qsum; }
     };
     if (e0 < M * p.cols) stage(e0, xa0, xb0);
+    if constexpr (!fused_norm) {
 #pragma unroll
-    for (int k = 0; k < XR; k++) {
-        const int e = e0 + (k + 1) * e_step;
-        if (e < M * p.cols) stage(e, xar[k], xbr[k]);
+        for (int k = 0; k < XR; k++) {
+            const int e = e0 + (k + 1) * e_step;
+            if (e < M * p.cols) stage(e, xar[k], xbr[k]);
+        }
+        for (int e = e0 + (XR + 1) * e_step; e < M * p.cols; e += e_step)      // rows beyond four passes
+            stage(e, *(const float4*)(p.x + e), *(const float4*)(p.x + e + 4));
     }
-    for (int e = e0 + (XR + 1) * e_step; e < M * p.cols; e += e_step)      // rows beyond four passes
-        stage(e, *(const float4*)(p.x + e), *(const float4*)(p.x + e + 4));
     if (!fused_norm && stager) __builtin_amdgcn_s_setprio(0);
     // The rest of the prefetch. Early: in flight while the workgroup meets at the barrier and copies its planes out of LDS
     // (rows so long that the staging takes several passes, and the large weights, whose row loop should find its pipeline
@@ -1112,6 +1157,18 @@ int full_wave_replicas(int NG, int maxw) {
     while (rf > 1 && NGF * rf + 1 > maxw) rf /= 2;
     return rf;
 }
+// What wave `wave` of a workgroup is (GemvParams::wtab): a row group is NG / 4 full waves (four slots of one row each),
+// replicated RF times with replica q taking every RF-th row from row q, and, when NG % 4 slots are left over, a tail wave that
+// holds them for 4 (one slot), 2 (two) or 1 (three) rows at once.
+uint32_t wave_word(int wave, int NG, int RF, int WPR) {
+    const int NGF = NG >> 2, NT = NG & 3, NFW = NGF * RF;
+    const int rg = wave / WPR, wr = wave - rg * WPR;
+    const bool tail = wr == NFW;
+    const int wq = NGF ? wr / NGF : 0, wm = NGF ? wr - wq * NGF : 0;
+    const int rtl = tail ? (NT == 1 ? 2 : NT == 2 ? 1 : 0) : 0;
+    const int v_start = tail ? 0 : wq, gbase = tail ? 4 * NGF : 4 * wm;
+    return (uint32_t)rg | (uint32_t)v_start << 4 | (tail ? 1u : 0u) << 8 | (uint32_t)NT << 9 | (uint32_t)gbase << 11 | (uint32_t)rtl << 19;
+}
 int waves_per_row_group(int NG, int maxw) { return (NG / 4) * full_wave_replicas(NG, maxw) + (NG % 4 ? 1 : 0); }
 
 template <class F, int M, bool SWIGLU>
@@ -1132,7 +1189,7 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
     bool late = HAS_LATE && w->cols <= 8192 && (F::TYPE == FHIP_Q6_K || small);
     GemvParams p;
     p.W = w->d_raw; p.x = d_x; p.y = d_y;
-    p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = w->row_bytes;
+    p.out_rows = (int)out_rows; p.cols = (int)w->cols; p.row_bytes = (uint32_t)w->row_bytes;
     p.pair_bytes = SWIGLU ? out_rows * w->row_bytes : 0;
     p.sel = sel ? *sel : fhip::SelParams{nullptr, 0, 0, 0, 0, 0, 1, 0};
     p.units = (int)(w->cols / F::WPL);
@@ -1232,7 +1289,8 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
         lds_raised[variant] = true;
     }
     auto magic = [](int d) { return d > 1 ? (uint32_t)(((1ull << 32) + (unsigned)d - 1) / (unsigned)d) : 0u; };
-    p.m_wpr = magic(WPR); p.m_ngf = magic(p.NG >> 2); p.m_rf = magic(p.RF); p.m_rpg = magic(rpg);
+    p.m_rf = magic(p.RF); p.m_rpg = magic(rpg);
+    for (int wv = 0; wv < 16; wv++) p.wtab[wv] = wv < WPR * G ? wave_word(wv, p.NG, p.RF, WPR) : 0u;
     const size_t per_wg = (size_t)G * rpg;
     const size_t grid = p.rr ? (size_t)p.nrg / G : (out_rows + per_wg - 1) / per_wg;
     size_t lds = lds_bytes<F, M, SWIGLU>(w->cols, p.NG, G, rpg);
