@@ -25,7 +25,7 @@ namespace fhip {
 
 // Expert selection for the mixture-of-experts "_id" matmuls (crates/ferric-tensor/src/dtype.rs:2463-2700).
 // The weight is a slab of n_expert experts of `expert_rows` rows each. The launch is replicated over `npairs`
-// (token, slot) pairs along grid.y; pair p = ti * k + s uses expert e = selw[ti*2k + k + s] (the index half of a
+// (token, slot) pairs, slot s along grid.y and token ti along grid.z (sel_grid); pair p = ti * k + s uses expert e = selw[ti*2k + k + s] (the index half of a
 // moe_topk row, stored as f32), activation row (x_per_pair ? p : ti) and writes at y + p * y_stride.
 // selw == nullptr: a plain launch.
 struct SelParams {
@@ -37,11 +37,16 @@ struct SelParams {
     int npairs;
     int relu2;   // the pair's outputs leave as max(v, 0)^2 (the squared-ReLU expert MLP, dtype.rs:1703-1729)
 };
+// grid of a launch of `wgs` workgroups per pair
+inline dim3 sel_grid(unsigned wgs, const SelParams& sel) {
+    const unsigned k = sel.selw && sel.k > 0 ? (unsigned)sel.k : 1u;
+    return dim3(wgs, k, sel.selw ? (unsigned)sel.npairs / k : 1u);
+}
 // applied at the top of a kernel: moves the three base pointers to this y-slice's expert / row / output
 template <class P>
 __device__ __forceinline__ void apply_selection(P& p) {
     if (p.sel.selw) {
-        const int pair = blockIdx.y, ti = pair / p.sel.k, s = pair - ti * p.sel.k;
+        const int s = blockIdx.y, ti = blockIdx.z, pair = ti * p.sel.k + s;   // grid (workgroups, k, tokens): no division
         int e = (int)p.sel.selw[(size_t)ti * 2 * p.sel.k + p.sel.k + s];
         e = e < 0 ? 0 : (e >= p.sel.n_expert ? p.sel.n_expert - 1 : e);   // a corrupt index must not leave the slab
         e = __builtin_amdgcn_readfirstlane(e);

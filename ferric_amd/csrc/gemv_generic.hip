@@ -608,7 +608,7 @@ int launch_one(const fhip_weight* w, const float* d_x, float* d_y, size_t out_ro
     if (lds > 64 * 1024) return fhip::set_error(FHIP_ERR_SHAPE, "matmul_q: LDS budget exceeded (%zu B)", lds);
     dim3 block(64 * p.S * G);
     constexpr int U = rows_in_flight(M);
-    const dim3 g3((unsigned)grid, (unsigned)p.sel.npairs);
+    const dim3 g3 = fhip::sel_grid((unsigned)grid, p.sel);
     hipLaunchKernelGGL((gemv_kernel<F, M, U, SWIGLU>), g3, block, lds, s, p);
     return fhip::check_hip(hipGetLastError(), "gemv launch");
 }
