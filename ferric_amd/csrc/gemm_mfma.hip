@@ -81,7 +81,9 @@ __device__ __forceinline__ constexpr int kcol(int t, int h) { return 32 * (t >> 
 
 struct Q4K {
     static constexpr int BLOCK = 144;
-    static constexpr float UNPACK_US = 1.4f;   // unpack of a 256 x 256 chunk by one workgroup (fitted, see plan_cost_us)
+    static constexpr float UNPACK_US = 1.4f;   // unpack of a 256 x 256 chunk by one workgroup
+    // one chunk of a workgroup tile of 64 x 256, 128 x 256, 256 x 256, 256 x 160, 128 x 128, 64 x 128, in us (fitted, see plan_cost_us)
+    static constexpr float CHUNK_US[6] = {3.49f, 4.69f, 8.03f, 5.10f, 2.79f, 1.96f};
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 hd, hdn, q[4]; };
@@ -139,6 +141,7 @@ struct Q4K {
 struct Q5K {
     static constexpr int BLOCK = 176;
     static constexpr float UNPACK_US = 1.8f;
+    static constexpr float CHUNK_US[6] = {3.63f, 5.03f, 9.14f, 5.86f, 3.07f, 2.19f};
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 hd, hdn, qh, qhn, q[4]; };
@@ -188,6 +191,7 @@ struct Q6K {
     // whose scale is sc[8hf + 2g + h]  (crates/ferric-gguf/src/lib.rs:833-851).
     static constexpr int BLOCK = 210;
     static constexpr float UNPACK_US = 2.3f;
+    static constexpr float CHUNK_US[6] = {5.83f, 6.71f, 9.68f, 6.18f, 4.62f, 3.93f};
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 ql[2][2], qh[2], sc, scn; uint32_t d, dn; };
@@ -253,6 +257,7 @@ struct Q80 {
     // read from the last valid block's address and given scale 0 (their activations are staged as 0 too).
     static constexpr int BLOCK = 34;
     static constexpr float UNPACK_US = 5.1f;
+    static constexpr float CHUNK_US[6] = {9.31f, 9.74f, 11.58f, 6.67f, 7.04f, 6.64f};
     static constexpr bool PARTIAL = true;   // a row may end inside a chunk
     static __host__ __device__ int chunks(int K) { return (K + 255) / 256; }
     struct Raw { u32x4 q[4][2]; uint32_t d[4][2]; };
@@ -334,13 +339,17 @@ __device__ __forceinline__ void static_for(Fn&& f) {
 // the runs that touch the tile, and sum_split_tiles_kernel adds a tile's slots in that order afterwards: the result does not
 // depend on which workgroup finishes first (f32 atomics into Y, which this replaced, gave run-to-run differences in the
 // last bits wherever a tile had three contributors or more).
-template <class F, int MI>
+//
+// NI = 1 is the same layout at half the width, a workgroup tile of (64*MI) x 128 for short prompts: a T-pair then needs one
+// block of 32 weight rows, both waves carry its raw bytes and each unpacks two of a step's four slices, so that at 128
+// activation rows (MI = 2) every weight is unpacked once (the 64 x 256 tile unpacks it twice, once per tile row) with the
+// same partial-tile bytes per workgroup.
+template <class F, int MI, int NI>
 __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
-    constexpr int NI = 2;
-    constexpr int BM = 64 * MI;
+    constexpr int BM = 64 * MI, BN = 128 * NI;
     constexpr int FRAG = 512;                                   // bf16 per published fragment (64 lanes x 8)
     __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_ROW];
-    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][32 * FRAG];   // [n-block 0..7][slice 0..3]
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[2][16 * NI * FRAG];   // [n-block 0..4 NI - 1][slice 0..3]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave & 3, wm = wave >> 2;
     const int h = lane >> 5, c = lane & 31;
@@ -364,18 +373,19 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
     const bool whole = c_begin == 0 && c_end == nchunks;
     const int tile_y = tile / p.tiles_n, tile_x = tile - tile_y * p.tiles_n;
     const int t0 = tile_y * BM + wm * (32 * MI);
-    const int n0 = tile_x * 256 + wn * 64;
+    const int n0 = tile_x * BN + wn * (32 * NI);
     const int c_last = c_end - 1;
 
-    // the weight row this lane unpacks: n-block 2*wn + wm of the workgroup tile (clamped: rows past N are
-    // computed but not stored)
+    // the weight row this lane unpacks: n-block 2*wn + wm of the workgroup tile (NI = 1: n-block wn, of which this wave
+    // unpacks slices 2*wm and 2*wm + 1); clamped: rows past N are computed but not stored
     const uint8_t* wrow;
     {
-        int n = n0 + 32 * wm + c;
+        int n = n0 + (NI == 2 ? 32 * wm : 0) + c;
         wrow = p.W + (size_t)(n < p.N ? n : p.N - 1) * p.row_bytes;
     }
-    const int b_wr = ((2 * wn + wm) * 4) * FRAG + lane * 8;    // + t * FRAG
-    const int b_rd = ((2 * wn) * 4) * FRAG + lane * 8;         // + (4 * j + t) * FRAG
+    const int b_wr = ((NI == 2 ? 2 * wn + wm : wn) * 4) * FRAG + lane * 8;    // + t * FRAG
+    const int b_rd = ((NI * wn) * 4) * FRAG + lane * 8;                        // + (4 * j + t) * FRAG
+    auto mine = [&](int t) { return NI == 2 || (t >> 1) == wm; };             // does this wave unpack slice t (wave-uniform)
 
     f32x16 acc[MI][NI];
 #pragma unroll
@@ -426,7 +436,7 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
         typename F::Ctx x;
         F::template begin<0>(raw, c_begin, h, p.nblk, x);
         static_for<0, 4>([&](auto T) {
-            *(bf16x8*)(&Bs[0][b_wr + T.value * FRAG]) = F::template frag<0, T.value>(raw, x);
+            if (mine(T.value)) *(bf16x8*)(&Bs[0][b_wr + T.value * FRAG]) = F::template frag<0, T.value>(raw, x);
         });
         F::template refill<0>(raw, wrow, nc, h, p.nblk);
     }
@@ -466,7 +476,7 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
 #pragma unroll
                 for (int j = 0; j < NI; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t & 1][i], b[t & 1][j], acc[i][j], 0, 0, 0);
-            *(bf16x8*)(&Bs[buf ^ 1][b_wr + t * FRAG]) = F::template frag<GN, t>(raw, ctx);
+            if (mine(t)) *(bf16x8*)(&Bs[buf ^ 1][b_wr + t * FRAG]) = F::template frag<GN, t>(raw, ctx);
             if constexpr (t < 3) __builtin_amdgcn_sched_group_barrier(0x100, MI + NI, 0);
 #pragma unroll
             for (int u = 0; u < MI * NI; u++) {
@@ -495,7 +505,7 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
     if (!whole) {
         const int rt = tile - p.whole_rounds * (int)gridDim.x;
         const int k = (int)blockIdx.x - (int)(((long long)rt * nchunks) / p.per);
-        part = p.ws + ((size_t)rt * p.kmax + k) * (size_t)(BM * 256);
+        part = p.ws + ((size_t)rt * p.kmax + k) * (size_t)(BM * BN);
     }
     // D layout of the 32x32 MFMA: register r of lane (h, c) is row 8*(r/4) + 4*h + (r%4), column c
 #pragma unroll
@@ -509,7 +519,7 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
                 const int t = t0 + 32 * i + 8 * (r >> 2) + 4 * h + (r & 3);
                 if (t < p.T) {
                     if (whole) p.Y[(size_t)t * p.N + n] = acc[i][j][r];
-                    else part[(size_t)(t - tile_y * BM) * 256 + (n - tile_x * 256)] = acc[i][j][r];
+                    else part[(size_t)(t - tile_y * BM) * BN + (n - tile_x * BN)] = acc[i][j][r];
                 }
             }
         }
@@ -970,6 +980,7 @@ struct TilePlan {
     long long left, units, split_wgs;   // left-over tiles, their chunks, workgroups whose run ends in partial tiles
     int kmax;                           // most runs that touch one left-over tile
     long long slots;                    // partial tiles the launch writes: over the left-over tiles cut along K, the runs that touch each
+    float extra_starts;                 // tiles a run touches beyond its first, on average (a run that ends in the next tile starts twice)
     unsigned grid;
 };
 
@@ -990,29 +1001,39 @@ static TilePlan plan_tiles(long long tiles_n, int nchunks, size_t t, int mi, lon
     q.split_wgs = (q.left > 0 && per % nchunks != 0) ? runs : 0;
     q.kmax = 1;
     q.slots = 0;
+    long long segs = 0;
     for (long long rt = 0; rt < q.left && q.split_wgs > 0; rt++) {
         const long long u0 = rt * nchunks;
         const int k = (int)((u0 + nchunks - 1) / per - u0 / per) + 1;
         if (k > q.kmax) q.kmax = k;
         if (k > 1) q.slots += k;
+        segs += k;
     }
+    q.extra_starts = q.split_wgs > 0 ? (float)segs / (float)runs - 1.f : 0.f;
     return q;
 }
 
-// Estimated duration of a plan in us: 1.5 per tile or run a workgroup starts, chunks per workgroup x the cost of a chunk, and,
-// when tiles are cut along K, the fix-up: 10.5 for the summing launch and 5 x mi per 256 partial tiles of 256 columns written
-// (and read back; a run that starts inside one tile and ends inside the next writes two). A chunk of a 256-column tile costs
-// the format's unpack time + 0.7 + 1.64 x mi (Q4_K: 3.7 / 5.4 / 8.6 us at 64 / 128 / 256 rows); a chunk of the 256 x 160 tile
-// 5.75 + 0.23 x the unpack time (its pace is set by the MFMAs and the operand reads; five of eight waves share the
-// unpacking). Constants fitted to forced-tile builds on 14 shapes of the three formats (53 launches, 7 % rms): the choice
-// is the fastest tile on all of them (candidates within 2 % of each other: the lower tile).
+// Estimated duration of a plan in us: 4.3 for the launch, 1.5 per tile or run a workgroup starts (3.7 more per further tile a
+// run reaches into), chunks per workgroup x the cost of a chunk of that tile and format (F::CHUNK_US), and, when tiles are cut
+// along K, the partial tiles and the launch that sums them: 8.1 per 256 partial tiles of 64 x 256 written and read back, plus a
+// constant per tile shape. A linear model fitted (relative least squares, 7 % rms) to 520 forced-tile launches: ten weights of
+// the four formats (5120 x 5120, 34816 x 5120, 7168 x 5120, 10240 x 5120, 4096 x 4096 Q4_K; 5120 x 17408, 5120 x 5120 Q6_K;
+// 4096 x 4096, 12288 x 4096 Q8_0; 5120 x 5120 Q5_K) at 48 ... 2048 rows, every tile. On those the tile it picks is 0.7 % slower
+// than the measured best on average (worst: 16 %, 5120 x 5120 at 256 rows); the constants it replaced, fitted before the
+// 128-column tiles and the finer summing launch, picked tiles up to 23 % off.
+constexpr float FIXUP_US[6] = {0.8f, -2.9f, -14.2f, -5.7f, -1.2f, 1.5f};
+static int tile_index(const TilePlan& q) { return q.bn == 256 ? (q.mi == 1 ? 0 : q.mi == 2 ? 1 : 2) : q.bn == 160 ? 3 : (q.mi == 2 ? 4 : 5); }
 template <class F>
 static float plan_cost_us(const TilePlan& q, int nchunks, long long cus) {
-    const float width = (float)q.bn / 256.f;
-    const float chunk_us = q.bn == 256 ? F::UNPACK_US + 0.68f + 1.64f * (float)q.mi : 5.75f + 0.23f * F::UNPACK_US;
+    const int ti = tile_index(q);
     const float chunks = (float)q.whole_rounds * (float)nchunks + (q.left > 0 ? (float)q.per : 0.f);
     const float starts = (float)q.whole_rounds + (q.left > 0 ? 1.f : 0.f);
-    return 1.5f * starts + chunks * chunk_us + (q.split_wgs > 0 ? 10.5f + 4.96f * (float)q.mi * width * (float)q.slots / (float)cus : 0.f);
+    float fix = 0.f;
+    if (q.split_wgs > 0) {
+        fix = FIXUP_US[ti] + 8.07f * (float)q.mi * ((float)q.bn / 256.f) * (float)q.slots / (float)cus;
+        fix = fix > 0.f ? fix : 0.f;
+    }
+    return 4.33f + 1.5f * starts + 3.74f * q.extra_starts + chunks * F::CHUNK_US[ti] + fix;
 }
 
 static size_t plan_ws_bytes(const TilePlan& q) {
@@ -1035,7 +1056,8 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     p.ws = d_ws; p.kmax = q.kmax;
     if (q.split_wgs > 0 && (!d_ws || ws_bytes < plan_ws_bytes(q)))
         return fhip::set_error(FHIP_ERR_ARG, "gemm_q_bf16: the launch cuts tiles along K and needs %zu bytes of workspace", plan_ws_bytes(q));
-    if constexpr (BN == 256) hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI>), dim3(q.grid), dim3(512), 0, s, p);
+    if constexpr (BN == 256) hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI, 2>), dim3(q.grid), dim3(512), 0, s, p);
+    else if constexpr (BN == 128) hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI, 1>), dim3(q.grid), dim3(512), 0, s, p);
     else hipLaunchKernelGGL((gemm_q_bf16_n160_kernel<F>), dim3(q.grid), dim3(512), 0, s, p);
     if (q.split_wgs > 0)
         hipLaunchKernelGGL(sum_split_tiles_kernel, dim3((unsigned)q.left, (unsigned)((64 * MI * BN / 4 + 255) / 256)), dim3(256), 0, s, d_y, (const float*)d_ws, p.T, p.N, 64 * MI,
@@ -1043,7 +1065,7 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
-int g_force_tile = -1;   // tests: 0..3 = 64, 128, 256 rows x 256 columns, 256 x 160; anything else: the estimate decides
+int g_force_tile = -1;   // tests: 0..3 = 64, 128, 256 rows x 256 columns, 256 x 160; 4, 5 = 128, 64 rows x 128 columns; anything else: the estimate decides
 
 // the tile the estimate picks for this launch (256 columns by 256, 128 or 64 rows, or 160 columns by 256 rows) with its plan
 template <class F>
@@ -1051,9 +1073,9 @@ static void choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     const int nchunks = F::chunks((int)w->cols);
     float best_cost = 0.f;
-    for (int i = 0; i < 4; i++) {                 // 64, 128, 256 rows x 256 columns, then 256 x 160
-        const int mi = i < 3 ? 1 << i : 4, bn = i < 3 ? 256 : 160;
-        if (g_force_tile >= 0 && g_force_tile <= 3 && i != g_force_tile) continue;
+    for (int i = 0; i < 6; i++) {                 // 64, 128, 256 rows x 256 columns, 256 x 160, then 128 and 64 rows x 128 columns
+        const int mi = i < 3 ? 1 << i : (i == 3 ? 4 : (i == 4 ? 2 : 1)), bn = i < 3 ? 256 : (i == 3 ? 160 : 128);
+        if (g_force_tile >= 0 && g_force_tile <= 5 && i != g_force_tile) continue;
         const TilePlan q = plan_tiles((long long)((w->rows + bn - 1) / bn), nchunks, t, mi, cus, bn);
         const float c = plan_cost_us<F>(q, nchunks, cus);
         if (best_cost == 0.f || c < 0.98f * best_cost) { best_cost = c; out = q; }
@@ -1073,15 +1095,19 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     if (t <= 32) return launch_skinny<F>(w, d_x, t, d_y, s, d_ws, ws_bytes);
     // Which tile. The 256 x 256 tile unpacks each weight once per 256 activation rows, but when there is no whole round of
     // such tiles for the chip every tile is cut along K, each workgroup writes a whole partial tile for a few chunks of
-    // work, and a lower tile (twice the tiles, half the fix-up, longer runs) or the 256 x 160 tile (whose count divides the
-    // chip for output widths like 5120 and 4096) can win: the estimate decides (measured, us at 256 / 128 / 64 rows x 256 and
-    // 256 x 160; Q4_K 5120 x 5120: T = 2048 176 / 162 / 207 / 128, T = 512 57 / 60 / 66 / 50, T = 128 43 / 33 / 30 / 45;
-    // Q6_K 5120 x 17408 T = 2048 458 / 511 / 788 / 426; Q8_0 4096 x 4096 T = 2048 131 / 156 / 278 / 111; Q4_K 34816 x 5120
-    // T = 512 219 / 247 / 326 / 233).
+    // work, and a lower tile (twice the tiles, half the fix-up, longer runs), the 256 x 160 tile (whose count divides the
+    // chip for output widths like 5120 and 4096) or, for short prompts, a 128-column tile (half the partial-tile bytes a
+    // workgroup writes, every weight unpacked once at 128 rows) can win: the estimate decides. Measured, us at 64 / 128 / 256
+    // rows x 256, 256 x 160, 128 / 64 rows x 128: Q4_K 5120 x 5120 T = 64 21 / 25 / 32 / 34 / 21 / 18, T = 128 25 / 27 / 35 / 36 /
+    // 22 / 27, T = 512 67 / 56 / 53 / 47 / 54 / 62; Q4_K 34816 x 5120 T = 64 57 / 68 / 102 / 96 / 68 / 55, T = 256 157 / 113 / 119 /
+    // 100 / 132 / 187; Q6_K 5120 x 17408 T = 128 80 / 62 / 77 / 73 / 67 / 103, T = 512 254 / 157 / 133 / 116 / 209 / 327; Q8_0
+    // 4096 x 4096 T = 128 35 / 33 / 37 / 32 / 31 / 40.
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     TilePlan q;
     choose_plan<F>(w, t, q);
     if (q.bn == 160) return launch_cfg<F, 4, 160>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    if (q.bn == 128) return q.mi == 2 ? launch_cfg<F, 2, 128>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes)
+                                      : launch_cfg<F, 1, 128>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
     if (q.mi == 4) return launch_cfg<F, 4, 256>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
     if (q.mi == 2) return launch_cfg<F, 2, 256>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
     return launch_cfg<F, 1, 256>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
