@@ -23,9 +23,9 @@
 // One k-step is 64 columns = 4 MFMA slices; a chunk is 4 steps = one K-quant super-block or 8 Q8_0 blocks.
 // Dequantized values are exactly the f32 the CPU dequantizer produces, rounded to bf16 (RNE) by
 // v_cvt_pk_bf16_f32.
-// Three kernels: the tiled one (64, 128 or 256 activation rows x 256 outputs per workgroup), its 256 x 160 variant for
-// output widths that 160 deals to the chip's workgroups exactly, and one for up to 32 rows; the launcher picks by a cost
-// estimate. A launch that cuts output tiles along K sums the partial tiles in a fixed order: the same inputs give the
+// Three kernels: the tiled one (64, 128 or 256 activation rows x 256 or 128 outputs per workgroup), its 160-column variant
+// (256 or 128 rows) for output widths that 160 deals to the chip's workgroups exactly, and one for up to 32 rows; the
+// launcher picks by a cost estimate. A launch that cuts output tiles along K sums the partial tiles in a fixed order: the same inputs give the
 // same bits on every run.
 #include "common.hpp"
 #include "loads.hpp"
@@ -82,8 +82,8 @@ __device__ __forceinline__ constexpr int kcol(int t, int h) { return 32 * (t >> 
 struct Q4K {
     static constexpr int BLOCK = 144;
     static constexpr float UNPACK_US = 1.4f;   // unpack of a 256 x 256 chunk by one workgroup
-    // one chunk of a workgroup tile of 64 x 256, 128 x 256, 256 x 256, 256 x 160, 128 x 128, 64 x 128, in us (fitted, see plan_cost_us)
-    static constexpr float CHUNK_US[6] = {3.49f, 4.69f, 8.03f, 5.10f, 2.79f, 1.96f};
+    // one chunk of a workgroup tile of 64 x 256, 128 x 256, 256 x 256, 256 x 160, 128 x 128, 64 x 128, 128 x 160, in us (fitted, see plan_cost_us)
+    static constexpr float CHUNK_US[7] = {3.43f, 4.76f, 8.15f, 5.19f, 2.84f, 2.00f, 3.29f};
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 hd, hdn, q[4]; };
@@ -141,7 +141,7 @@ struct Q4K {
 struct Q5K {
     static constexpr int BLOCK = 176;
     static constexpr float UNPACK_US = 1.8f;
-    static constexpr float CHUNK_US[6] = {3.63f, 5.03f, 9.14f, 5.86f, 3.07f, 2.19f};
+    static constexpr float CHUNK_US[7] = {3.83f, 5.16f, 9.41f, 6.12f, 3.17f, 2.26f, 3.78f};
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 hd, hdn, qh, qhn, q[4]; };
@@ -191,7 +191,7 @@ struct Q6K {
     // whose scale is sc[8hf + 2g + h]  (crates/ferric-gguf/src/lib.rs:833-851).
     static constexpr int BLOCK = 210;
     static constexpr float UNPACK_US = 2.3f;
-    static constexpr float CHUNK_US[6] = {5.83f, 6.71f, 9.68f, 6.18f, 4.62f, 3.93f};
+    static constexpr float CHUNK_US[7] = {5.93f, 6.83f, 9.84f, 6.27f, 4.68f, 3.95f, 4.35f};
     static constexpr bool PARTIAL = false;
     static __host__ __device__ int chunks(int K) { return K / 256; }
     struct Raw { u32x4 ql[2][2], qh[2], sc, scn; uint32_t d, dn; };
@@ -257,7 +257,7 @@ struct Q80 {
     // read from the last valid block's address and given scale 0 (their activations are staged as 0 too).
     static constexpr int BLOCK = 34;
     static constexpr float UNPACK_US = 5.1f;
-    static constexpr float CHUNK_US[6] = {9.31f, 9.74f, 11.58f, 6.67f, 7.04f, 6.64f};
+    static constexpr float CHUNK_US[7] = {9.51f, 9.88f, 11.93f, 6.86f, 7.16f, 6.65f, 5.76f};
     static constexpr bool PARTIAL = true;   // a row may end inside a chunk
     static __host__ __device__ int chunks(int K) { return (K + 255) / 256; }
     struct Raw { u32x4 q[4][2]; uint32_t d[4][2]; };
@@ -536,17 +536,27 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_kernel(GemmParams p) {
 // 4..7, one slice each, so that every SIMD carries the same unpack arithmetic, was slower: 130 -> 141 us at T = 2048 --
 // four more waves fetch raw bytes and derive scales every step.) Work distribution and K-split slots are the tall
 // kernel's at MI = 4.
+// MI = 2 is the tile at 128 rows, for prompts of 96 ... 256 rows, where the 256-row tile multiplies rows that do not exist
+// or is cut along K more finely: four waves along T, and the five column blocks dealt to two wave groups, three to waves
+// 0..3 and two to waves 4..7 -- wave w and wave w + 4 share a SIMD, so every SIMD still carries five blocks of MFMAs per
+// slice. Measured against the best other tile, us: Q4_K 5120 x 5120 at 256 rows 36.1 -> 32.9, 34816 x 5120 at 128 rows
+// 75.7 -> 68.9, Q6_K 5120 x 17408 at 128 rows 64.6 -> 59.0, Q8_0 12288 x 4096 at 128 rows 57.8 -> 52.3; at 512 rows of
+// 5120 x 5120 (128 tiles cut in two instead of 64 cut in four) it is level, 49.2 against 48.0.
 // ------------------------------------------------------------------------------------------------
-template <class F>
+template <class F, int MI>
 __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
-    constexpr int MI = 4, NB = 5;
+    constexpr int NB = 5;
     constexpr int BM = 64 * MI, BN = 32 * NB;
+    constexpr int TW = BM / 32, NBW = TW == 8 ? NB : 3;         // waves along T; column blocks a wave holds at most
     constexpr int FRAG = 512;
     __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_ROW];
     __shared__ __attribute__((aligned(16))) uint16_t Bs[2][NB * 4 * FRAG];   // [n-block 0..4][slice 0..3]
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = lane >> 5, c = lane & 31;
     const bool unpacker = wave < NB;                            // wave-uniform
+    const int tw = TW == 8 ? wave : (wave & 3);                 // the wave's 32 activation rows of the tile
+    const int j0 = TW == 8 ? 0 : (wave < 4 ? 0 : 3);            // its first column block ...
+    const int nj = TW == 8 ? NB : (wave < 4 ? 3 : 2);           // ... and how many it holds (wave-uniform)
     const int nchunks = p.nchunks;
     long long u = (long long)blockIdx.x * p.per;
     const long long u_end = u + p.per < p.units ? u + p.per : p.units;
@@ -566,7 +576,7 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
     }
     const bool whole = c_begin == 0 && c_end == nchunks;
     const int tile_y = tile / p.tiles_n, tile_x = tile - tile_y * p.tiles_n;
-    const int t0 = tile_y * BM + 32 * wave;
+    const int t0 = tile_y * BM + 32 * tw;
     const int n0 = tile_x * BN;
     const int c_last = c_end - 1;
 
@@ -578,11 +588,11 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
         wrow = p.W + (size_t)(n < p.N ? n : p.N - 1) * p.row_bytes;
     }
     const int b_wr = (wave * 4) * FRAG + lane * 8;              // + t * FRAG (unpackers)
-    const int b_rd = lane * 8;                                  // + (4 * j + t) * FRAG
+    const int b_rd = (4 * j0) * FRAG + lane * 8;                // + (4 * j + t) * FRAG
 
-    f32x16 acc[NB];
+    f32x16 acc[NBW];
 #pragma unroll
-    for (int j = 0; j < NB; j++)
+    for (int j = 0; j < NBW; j++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
@@ -593,10 +603,11 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
     // (sl & 7) of rows (sl >> 3) + 24 q, q < 11 (the eleventh round holds 16 rows, for the first two of the three waves) --
     // which takes 20 of some 190 instructions a step off the waves that set the pace (Q8_0 5120 x 4096 at T = 2048 150 ->
     // 133 us, Q6_K 5120 x 17408 444 -> 432 us; Q4_K 5120 x 5120 131 -> 135 us, so it keeps the even split).
+    // (at 128 rows: six rounds, the sixth holds 8 rows, for the first of the three waves)
     constexpr bool SPLIT = F::UNPACK_US > 2.f;
-    constexpr int NQ = SPLIT ? 11 : MI, RSTEP = SPLIT ? 24 : 64;
+    constexpr int NQ = SPLIT ? (MI == 4 ? 11 : 6) : MI, RSTEP = SPLIT ? 24 : 64;
     const bool stager = SPLIT ? !unpacker : true;               // wave-uniform
-    const bool qlast = SPLIT ? wave < NB + 2 : true;            // wave-uniform: the wave has a piece in the last round
+    const bool qlast = SPLIT ? wave < NB + (MI == 4 ? 2 : 1) : true;   // wave-uniform: the wave has a piece in the last round
     const int sl = SPLIT ? (wave - NB) * 64 + lane : tid;
     const int a_col = (sl & 7) * 8;
     uint32_t a_src[NQ];
@@ -632,7 +643,7 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
         for (int q = 0; q < NQ; q++)
             if (q < NQ - 1 || qlast) *(u32x4*)(&As[buf][a_dst + RSTEP * q * LDS_ROW]) = stage[q];
     };
-    const int a_rd = (32 * wave + c) * LDS_ROW + 16 * h;        // + kcol(t, 0)
+    const int a_rd = (32 * tw + c) * LDS_ROW + 16 * h;          // + kcol(t, 0)
     typename F::Raw raw;
     if (stager) load_a(4 * c_begin);
     if (unpacker) {
@@ -649,20 +660,22 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
     __syncthreads();
 
     // one k-step, as in the tall kernel; UNPACK: the wave produces its block's fragments, one behind each slice's MFMAs
-    auto step = [&](auto Gc, auto Uc, int ck) {
+    // (NJ: the column blocks the wave holds, a constant of the loop it runs)
+    auto step = [&](auto Gc, auto Uc, auto Jc, int ck) {
         constexpr int G = decltype(Gc)::value;
         constexpr bool UNPACK = decltype(Uc)::value;
+        constexpr int NJ = decltype(Jc)::value;
         constexpr int GN = (G + 1) & 3;
         constexpr int buf = G & 1;
-        constexpr int VPM = (26 + NB - 1) / NB;
+        constexpr int VPM = (26 + NJ - 1) / NJ;
         const int pc = G == 3 ? (ck + 1 < c_last ? ck + 1 : c_last) : ck;
         const int nc = pc + 1 < c_last ? pc + 1 : c_last;
         typename F::Ctx ctx;
-        bf16x8 a[2], b[2][NB];
-        auto read_ops = [&](int t, bf16x8& da, bf16x8 (&db)[NB]) {
+        bf16x8 a[2], b[2][NJ];
+        auto read_ops = [&](int t, bf16x8& da, bf16x8 (&db)[NJ]) {
             da = *(const bf16x8*)(&As[buf][a_rd + kcol(t, 0)]);
 #pragma unroll
-            for (int j = 0; j < NB; j++) db[j] = *(const bf16x8*)(&Bs[buf][b_rd + (4 * j + t) * FRAG]);
+            for (int j = 0; j < NJ; j++) db[j] = *(const bf16x8*)(&Bs[buf][b_rd + (4 * j + t) * FRAG]);
         };
         read_ops(0, a[0], b[0]);
         if constexpr (!(UNPACK && SPLIT)) load_a(4 * ck + G + 1);
@@ -672,11 +685,11 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
             constexpr int t = decltype(S)::value;
             if constexpr (t < 3) read_ops(t + 1, a[(t + 1) & 1], b[(t + 1) & 1]);
 #pragma unroll
-            for (int j = 0; j < NB; j++) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t & 1], b[t & 1][j], acc[j], 0, 0, 0);
+            for (int j = 0; j < NJ; j++) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t & 1], b[t & 1][j], acc[j], 0, 0, 0);
             if constexpr (UNPACK) *(bf16x8*)(&Bs[buf ^ 1][b_wr + t * FRAG]) = F::template frag<GN, t>(raw, ctx);
-            if constexpr (t < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1 + NB, 0);
+            if constexpr (t < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1 + NJ, 0);
 #pragma unroll
-            for (int m = 0; m < NB; m++) {
+            for (int m = 0; m < NJ; m++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if constexpr (UNPACK) __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);
             }
@@ -689,20 +702,21 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    if (unpacker) {
+    auto run = [&](auto Uc, auto Jc) {
         for (int ck = c_begin; ck < c_end; ck++) {
-            step(std::integral_constant<int, 0>{}, std::true_type{}, ck);
-            step(std::integral_constant<int, 1>{}, std::true_type{}, ck);
-            step(std::integral_constant<int, 2>{}, std::true_type{}, ck);
-            step(std::integral_constant<int, 3>{}, std::true_type{}, ck);
+            step(std::integral_constant<int, 0>{}, Uc, Jc, ck);
+            step(std::integral_constant<int, 1>{}, Uc, Jc, ck);
+            step(std::integral_constant<int, 2>{}, Uc, Jc, ck);
+            step(std::integral_constant<int, 3>{}, Uc, Jc, ck);
         }
+    };
+    if constexpr (TW == 8) {
+        if (unpacker) run(std::true_type{}, std::integral_constant<int, NB>{});
+        else run(std::false_type{}, std::integral_constant<int, NB>{});
     } else {
-        for (int ck = c_begin; ck < c_end; ck++) {
-            step(std::integral_constant<int, 0>{}, std::false_type{}, ck);
-            step(std::integral_constant<int, 1>{}, std::false_type{}, ck);
-            step(std::integral_constant<int, 2>{}, std::false_type{}, ck);
-            step(std::integral_constant<int, 3>{}, std::false_type{}, ck);
-        }
+        if (wave < 4) run(std::true_type{}, std::integral_constant<int, 3>{});
+        else if (unpacker) run(std::true_type{}, std::integral_constant<int, 2>{});
+        else run(std::false_type{}, std::integral_constant<int, 2>{});
     }
 
     float* part = nullptr;
@@ -713,9 +727,9 @@ __global__ void __launch_bounds__(512) gemm_q_bf16_n160_kernel(GemmParams p) {
     }
     // D layout of the 32x32 MFMA: register r of lane (h, c) is row 8*(r/4) + 4*h + (r%4), column c
 #pragma unroll
-    for (int j = 0; j < NB; j++) {
-        const int n = n0 + 32 * j + c;
-        if (n >= p.N) continue;
+    for (int j = 0; j < NBW; j++) {
+        const int n = n0 + 32 * (j0 + j) + c;
+        if (j >= nj || n >= p.N) continue;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int t = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
@@ -975,7 +989,7 @@ int launch_skinny(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_
 // How a launch of the tiled kernel with tile height 64 * mi is dealt to the chip: `whole_rounds` whole tiles per workgroup,
 // then the left-over tiles cut along K into runs of `per` chunks.
 struct TilePlan {
-    int mi, bn;                         // tile of 64 * mi activation rows x bn outputs (256, or 160 with mi = 4)
+    int mi, bn;                         // tile of 64 * mi activation rows x bn outputs (256, 128, or 160 with mi = 4 or 2)
     int whole_rounds, per;
     long long left, units, split_wgs;   // left-over tiles, their chunks, workgroups whose run ends in partial tiles
     int kmax;                           // most runs that touch one left-over tile
@@ -1013,16 +1027,15 @@ static TilePlan plan_tiles(long long tiles_n, int nchunks, size_t t, int mi, lon
     return q;
 }
 
-// Estimated duration of a plan in us: 4.3 for the launch, 1.5 per tile or run a workgroup starts (3.7 more per further tile a
+// Estimated duration of a plan in us: 4.3 for the launch, 1.5 per tile or run a workgroup starts (4.0 more per further tile a
 // run reaches into), chunks per workgroup x the cost of a chunk of that tile and format (F::CHUNK_US), and, when tiles are cut
-// along K, the partial tiles and the launch that sums them: 8.1 per 256 partial tiles of 64 x 256 written and read back, plus a
-// constant per tile shape. A linear model fitted (relative least squares, 7 % rms) to 520 forced-tile launches: ten weights of
+// along K, the partial tiles and the launch that sums them: 7.8 per 256 partial tiles of 64 x 256 written and read back, plus a
+// constant per tile shape. A linear model fitted (relative least squares, 7 % rms) to 620 forced-tile launches: ten weights of
 // the four formats (5120 x 5120, 34816 x 5120, 7168 x 5120, 10240 x 5120, 4096 x 4096 Q4_K; 5120 x 17408, 5120 x 5120 Q6_K;
-// 4096 x 4096, 12288 x 4096 Q8_0; 5120 x 5120 Q5_K) at 48 ... 2048 rows, every tile. On those the tile it picks is 0.7 % slower
-// than the measured best on average (worst: 16 %, 5120 x 5120 at 256 rows); the constants it replaced, fitted before the
-// 128-column tiles and the finer summing launch, picked tiles up to 23 % off.
-constexpr float FIXUP_US[6] = {0.8f, -2.9f, -14.2f, -5.7f, -1.2f, 1.5f};
-static int tile_index(const TilePlan& q) { return q.bn == 256 ? (q.mi == 1 ? 0 : q.mi == 2 ? 1 : 2) : q.bn == 160 ? 3 : (q.mi == 2 ? 4 : 5); }
+// 4096 x 4096, 12288 x 4096 Q8_0; 5120 x 5120 Q5_K) at 48 ... 2048 rows, every tile. On those the tile it picks is 1.0 % slower
+// than the measured best on average (worst: 17 %, Q6_K 5120 x 5120 at 256 rows).
+constexpr float FIXUP_US[7] = {0.9f, -2.3f, -13.2f, -5.2f, -1.0f, 1.5f, 0.4f};
+static int tile_index(const TilePlan& q) { return q.bn == 256 ? (q.mi == 1 ? 0 : q.mi == 2 ? 1 : 2) : q.bn == 160 ? (q.mi == 4 ? 3 : 6) : (q.mi == 2 ? 4 : 5); }
 template <class F>
 static float plan_cost_us(const TilePlan& q, int nchunks, long long cus) {
     const int ti = tile_index(q);
@@ -1030,10 +1043,10 @@ static float plan_cost_us(const TilePlan& q, int nchunks, long long cus) {
     const float starts = (float)q.whole_rounds + (q.left > 0 ? 1.f : 0.f);
     float fix = 0.f;
     if (q.split_wgs > 0) {
-        fix = FIXUP_US[ti] + 8.07f * (float)q.mi * ((float)q.bn / 256.f) * (float)q.slots / (float)cus;
+        fix = FIXUP_US[ti] + 7.77f * (float)q.mi * ((float)q.bn / 256.f) * (float)q.slots / (float)cus;
         fix = fix > 0.f ? fix : 0.f;
     }
-    return 4.33f + 1.5f * starts + 3.74f * q.extra_starts + chunks * F::CHUNK_US[ti] + fix;
+    return 4.29f + 1.5f * starts + 3.96f * q.extra_starts + chunks * F::CHUNK_US[ti] + fix;
 }
 
 static size_t plan_ws_bytes(const TilePlan& q) {
@@ -1058,24 +1071,25 @@ int launch_cfg(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
         return fhip::set_error(FHIP_ERR_ARG, "gemm_q_bf16: the launch cuts tiles along K and needs %zu bytes of workspace", plan_ws_bytes(q));
     if constexpr (BN == 256) hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI, 2>), dim3(q.grid), dim3(512), 0, s, p);
     else if constexpr (BN == 128) hipLaunchKernelGGL((gemm_q_bf16_kernel<F, MI, 1>), dim3(q.grid), dim3(512), 0, s, p);
-    else hipLaunchKernelGGL((gemm_q_bf16_n160_kernel<F>), dim3(q.grid), dim3(512), 0, s, p);
+    else hipLaunchKernelGGL((gemm_q_bf16_n160_kernel<F, MI>), dim3(q.grid), dim3(512), 0, s, p);
     if (q.split_wgs > 0)
         hipLaunchKernelGGL(sum_split_tiles_kernel, dim3((unsigned)q.left, (unsigned)((64 * MI * BN / 4 + 255) / 256)), dim3(256), 0, s, d_y, (const float*)d_ws, p.T, p.N, 64 * MI,
                            BN, p.tiles_n, p.nchunks, p.per, p.kmax, (int)(p.whole_rounds * cus));
     return fhip::check_hip(hipGetLastError(), "gemm_q_bf16 launch");
 }
 
-int g_force_tile = -1;   // tests: 0..3 = 64, 128, 256 rows x 256 columns, 256 x 160; 4, 5 = 128, 64 rows x 128 columns; anything else: the estimate decides
+int g_force_tile = -1;   // tests: 0..3 = 64, 128, 256 rows x 256 columns, 256 x 160; 4, 5 = 128, 64 rows x 128 columns; 6 = 128 x 160; anything else: the estimate decides
 
-// the tile the estimate picks for this launch (256 columns by 256, 128 or 64 rows, or 160 columns by 256 rows) with its plan
+// the tile the estimate picks for this launch (one of the seven the loop lists) with its plan
 template <class F>
 static void choose_plan(const fhip_weight* w, size_t t, TilePlan& out) {
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     const int nchunks = F::chunks((int)w->cols);
     float best_cost = 0.f;
-    for (int i = 0; i < 6; i++) {                 // 64, 128, 256 rows x 256 columns, 256 x 160, then 128 and 64 rows x 128 columns
-        const int mi = i < 3 ? 1 << i : (i == 3 ? 4 : (i == 4 ? 2 : 1)), bn = i < 3 ? 256 : (i == 3 ? 160 : 128);
-        if (g_force_tile >= 0 && g_force_tile <= 5 && i != g_force_tile) continue;
+    for (int i = 0; i < 7; i++) {                 // 64, 128, 256 rows x 256 columns, 256 x 160, 128 and 64 rows x 128 columns, 128 x 160
+        constexpr int MI_OF[7] = {1, 2, 4, 4, 2, 1, 2}, BN_OF[7] = {256, 256, 256, 160, 128, 128, 160};
+        const int mi = MI_OF[i], bn = BN_OF[i];
+        if (g_force_tile >= 0 && g_force_tile <= 6 && i != g_force_tile) continue;
         const TilePlan q = plan_tiles((long long)((w->rows + bn - 1) / bn), nchunks, t, mi, cus, bn);
         const float c = plan_cost_us<F>(q, nchunks, cus);
         if (best_cost == 0.f || c < 0.98f * best_cost) { best_cost = c; out = q; }
@@ -1105,7 +1119,8 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_x, size_t t, float* d_y, 
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
     TilePlan q;
     choose_plan<F>(w, t, q);
-    if (q.bn == 160) return launch_cfg<F, 4, 160>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
+    if (q.bn == 160) return q.mi == 4 ? launch_cfg<F, 4, 160>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes)
+                                      : launch_cfg<F, 2, 160>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
     if (q.bn == 128) return q.mi == 2 ? launch_cfg<F, 2, 128>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes)
                                       : launch_cfg<F, 1, 128>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);
     if (q.mi == 4) return launch_cfg<F, 4, 256>(w, d_x, t, d_y, s, q, cus, d_ws, ws_bytes);

@@ -15,8 +15,7 @@ int fhip_debug_generic_matvec(int on);
 
 /* Debugging and tests: pins the workgroup tile of the matrix-core GEMM (fhip_gemm_q_bf16, fhip_matmul_q_coop, fhip_ffn_coop)
  * for launches of more than 32 rows: 0, 1, 2 = 64, 128, 256 activation rows x 256 outputs, 3 = 256 x 160, 4, 5 = 128, 64 rows x
- * 128 outputs; -1 (the default)
- * lets the cost estimate choose. Returns the value before the call. Process-wide, not thread-safe against concurrent
+ * 128 outputs, 6 = 128 x 160; -1 (the default) lets the cost estimate choose. Returns the value before the call. Process-wide, not thread-safe against concurrent
  * launches; fhip_workspace_bytes_coop follows it. No counterpart in the reference. */
 int fhip_debug_gemm_tile(int tile);
 

@@ -61,10 +61,10 @@ def test_seeded_random_shapes(F, O):
         run_case(F, O, ty, t, n, k, 1000 + i)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
 def test_every_tile_on_ragged_shapes(F, O, tile):
-    # The launcher picks one of six workgroup tiles by estimate; here each is pinned in turn (64 / 128 / 256 rows x 256
-    # outputs, 256 x 160, 128 / 64 rows x 128) and run on shapes that fill no tile: rows and outputs that end inside a tile, outputs that are no
+    # The launcher picks one of seven workgroup tiles by estimate; here each is pinned in turn (64 / 128 / 256 rows x 256
+    # outputs, 256 x 160, 128 / 64 rows x 128, 128 x 160) and run on shapes that fill no tile: rows and outputs that end inside a tile, outputs that are no
     # multiple of 4, launches with whole rounds of tiles and a cut remainder, launches where every tile is cut along K.
     lib = F._lib.load()
     before = lib.fhip_debug_gemm_tile(tile)
