@@ -111,6 +111,7 @@ SYMBOLS = {
     "fhip_decode_attention_ex": (C.c_int, [_vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, C.c_float, _vp, _vp, _vp]),
     "fhip_norm_matmul_q": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, _vp, C.c_int, _vp, _vp]),
     "fhip_debug_generic_matvec": (C.c_int, [C.c_int]),
+    "fhip_debug_quad_matvec": (C.c_int, [C.c_int]),
     "fhip_debug_gemm_tile": (C.c_int, [C.c_int]),
     "fhip_matvec_precision": (C.c_int, [C.c_int]),
     "fhip_weight_matvec_precision": (C.c_int, [_vp, C.c_int]),

@@ -24,6 +24,8 @@ UNITS = {
     "kvquant.hip": ["-ffp-contract=off"],       # the reference multiplies, then adds: no fused multiply-add
     "gemv.hip": ["-DFHIP_GEMV_PLANES=2"],
     "gemv.hip@p3": ["-DFHIP_GEMV_PLANES=3"],   # the same source again: the 24-bit-activation copy of the streaming mat-vec
+    "gemv_quad.hip": ["-DFHIP_GEMV_PLANES=2"],
+    "gemv_quad.hip@p3": ["-DFHIP_GEMV_PLANES=3"],
     "gemv_generic.hip": [],
     "gemm_mfma.hip": [],
     "gemm_f16x2.hip": [],

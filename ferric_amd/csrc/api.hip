@@ -103,8 +103,33 @@ int device_cus() { return g_cus; }
 size_t device_lds_bytes() { return g_lds; }
 
 // The streaming mat-vec exists in two copies, one per activation precision; these forward to the one the weight names.
+// From three rows on, Q4_K and Q6_K batches go four rows at a time through the kernel that multiplies on the 4 x 4 x 4 int8
+// matrix instruction (gemv_quad.hip: the same arithmetic and the same bits per row, one pass over the weight for four rows);
+// what is left of a batch, one or two rows, and every other format take the dot-product kernel.
+bool g_quad_matvec = true, g_generic_forced = false;
 int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s) {
-    return w->planes == 3 ? launch_gemv_p3(w, d_x, rows_x, d_y, n_ff, s) : launch_gemv_p2(w, d_x, rows_x, d_y, n_ff, s);
+    const bool p3 = w->planes == 3;
+    if (rows_x >= 3 && g_quad_matvec && !g_generic_forced && d_x && d_y &&
+        (p3 ? gemv_quad_supports_p3(w, 4, n_ff) : gemv_quad_supports_p2(w, 4, n_ff))) {
+        const size_t out_rows = n_ff ? n_ff : w->rows;
+        for (size_t m0 = 0; m0 < rows_x;) {
+            const size_t t = rows_x - m0 < 4 ? rows_x - m0 : 4;
+            const float* x = d_x + m0 * w->cols;
+            float* y = d_y + m0 * out_rows;
+            int rc;
+            if (t >= 3) rc = p3 ? launch_gemv_quad_p3(w, x, t, y, n_ff, s) : launch_gemv_quad_p2(w, x, t, y, n_ff, s);
+            else rc = p3 ? launch_gemv_p3(w, x, t, y, n_ff, s) : launch_gemv_p2(w, x, t, y, n_ff, s);
+            if (rc) return rc;
+            m0 += t;
+        }
+        return FHIP_OK;
+    }
+    return p3 ? launch_gemv_p3(w, d_x, rows_x, d_y, n_ff, s) : launch_gemv_p2(w, d_x, rows_x, d_y, n_ff, s);
+}
+bool gemv_quad_matvec(bool on) {
+    const bool before = g_quad_matvec;
+    g_quad_matvec = on;
+    return before;
 }
 int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s) {
     return w->planes == 3 ? launch_gemv_norm_p3(w, d_x, d_y, n_ff, norm, s) : launch_gemv_norm_p2(w, d_x, d_y, n_ff, norm, s);
@@ -113,6 +138,7 @@ int launch_gemv_sel(const fhip_weight* w, const float* d_x, float* d_y, size_t o
     return w->planes == 3 ? launch_gemv_sel_p3(w, d_x, d_y, out_rows, swiglu, sel, s) : launch_gemv_sel_p2(w, d_x, d_y, out_rows, swiglu, sel, s);
 }
 void gemv_force_generic(bool on) {
+    g_generic_forced = on;
     gemv_force_generic_p2(on);
     gemv_force_generic_p3(on);
 }
@@ -185,8 +211,9 @@ static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t,
 // ---- which kernel a batch takes ---------------------------------------------------------------------------------------------
 // One or two activation rows go through the streaming mat-vec (one pass over the weights serves two rows). From three rows on
 // (five for Q8_0) the f16 hi/lo matrix-core kernels read the weights once for up to 32 (Q8_0: 16) rows; longer batches are cut
-// into such groups. FHIP_BATCH_F32_MATVEC keeps every batch on the mat-vec kernel: a row then has the same bits whatever batch
-// it is part of.
+// into such groups. FHIP_BATCH_F32_MATVEC keeps every batch on the mat-vec's arithmetic (launch_gemv: four rows a pass on the
+// int8 matrix instruction for Q4_K / Q6_K, the dot-product kernel otherwise): a row then has the same bits whatever batch it
+// is part of.
 
 size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32; }
 bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
@@ -194,6 +221,14 @@ bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
     if (w->type != FHIP_Q4_K && w->type != FHIP_Q5_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0) return false;
     if (rows_x < (w->type == FHIP_Q8_0 ? 5u : 3u)) return false;
     return fhip::gemm_f16x2_supports(w, rows_x < f16x2_group(w) ? rows_x : f16x2_group(w));
+}
+
+// Fused gate|up + SwiGLU at three or four rows: one pass of the int8 matrix-instruction mat-vec (gemv_quad.hip, 31 us on
+// 34816 x 5120) is faster than the one-pass f16 kernel plus the SwiGLU launch behind it (34 + 4), and its rows carry the bits
+// they have in a batch of one. The plain matmuls of such batches stay on the f16 kernels (down 5120 x 17408: 27 us against 42).
+bool swiglu_takes_quad(const fhip_weight* gu, size_t t) {
+    if (t < 3 || t > 4 || gu->rows % 2 != 0) return false;
+    return gu->planes == 3 ? fhip::gemv_quad_supports_p3(gu, t, gu->rows / 2) : fhip::gemv_quad_supports_p2(gu, t, gu->rows / 2);
 }
 
 // y [t, rows] = 0 on the stream, by the mat-vec launcher's fill kernel (what a weight without columns gives)
@@ -552,7 +587,7 @@ int fhip_matmul_q_swiglu(const fhip_weight* gu, const float* d_x, size_t rows_x,
     if (((uintptr_t)d_x & 15) != 0) return set_error(FHIP_ERR_ARG, "fhip_matmul_q_swiglu: x must be 16-byte aligned");
     hipStream_t s = (hipStream_t)stream;
     const size_t n_ff = gu->rows / 2;
-    if (!takes_f16x2(gu, rows_x)) return fhip::launch_gemv(gu, d_x, rows_x, d_y, n_ff, s);
+    if (!takes_f16x2(gu, rows_x) || swiglu_takes_quad(gu, rows_x)) return fhip::launch_gemv(gu, d_x, rows_x, d_y, n_ff, s);
     // gate|up for the group in one pass into the workspace, then the reference's un-fused SwiGLU over it
     const size_t grp = f16x2_group(gu), t0 = rows_x < grp ? rows_x : grp;
     const size_t mm = f16x2_matmul_ws(gu, t0);
@@ -561,7 +596,7 @@ int fhip_matmul_q_swiglu(const fhip_weight* gu, const float* d_x, size_t rows_x,
     float* g = (float*)((uint8_t*)ws + mm);
     for (size_t m0 = 0; m0 < rows_x; m0 += grp) {
         const size_t t = rows_x - m0 < grp ? rows_x - m0 : grp;
-        if (!takes_f16x2(gu, t)) { rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, d_y + m0 * n_ff, n_ff, s); }
+        if (!takes_f16x2(gu, t) || swiglu_takes_quad(gu, t)) { rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, d_y + m0 * n_ff, n_ff, s); }
         else if (!(rc = f16x2_matmul(gu, d_x + m0 * gu->cols, t, false, g, ws, s))) rc = fhip::launch_swiglu(g, t, n_ff, d_y + m0 * n_ff, s);
         if (rc) return rc;
     }
@@ -611,6 +646,10 @@ int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, s
         if (!takes_f16x2(gu, t) || !takes_f16x2(down, t)) {
             if ((rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, d_ws + m0 * n_ff, n_ff, s))) return rc;
             rc = fhip::launch_gemv(down, d_ws + m0 * n_ff, t, d_y + m0 * down->rows, 0, s);
+        } else if (swiglu_takes_quad(gu, t)) {
+            // three or four rows: silu(gate) * up straight out of the mat-vec, then the down projection's one pass over it
+            if (!(rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, g, n_ff, s)))
+                rc = f16x2_matmul(down, g, t, false, d_y + m0 * down->rows, ws2, s);
         } else {
             // under the ordered policy gate|up's K-split groups stay partial sums; the split for the down projection adds them
             fhip::F16Parts parts{nullptr, 0, 0, 0, 0};
@@ -959,6 +998,8 @@ int fhip_debug_generic_matvec(int on) {
 }
 
 int fhip_debug_gemm_tile(int tile) { return fhip::gemm_bf16_force_tile(tile); }
+
+int fhip_debug_quad_matvec(int on) { return fhip::gemv_quad_matvec(on != 0) ? 1 : 0; }
 
 int fhip_debug_read_probe(const void* d_src, size_t nbytes, uint32_t* d_sink, void* stream) {
     int rc = need_init();

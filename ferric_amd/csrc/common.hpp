@@ -89,7 +89,9 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
                               hipStream_t s);                                                                                       \
     int launch_gemv_sel##sfx(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu,                      \
                              const struct SelParams& sel, hipStream_t s);                                                           \
-    void gemv_force_generic##sfx(bool on);
+    void gemv_force_generic##sfx(bool on);                                                                                         \
+    bool gemv_quad_supports##sfx(const fhip_weight* w, size_t rows_x, size_t n_ff);                                                 \
+    int launch_gemv_quad##sfx(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 FHIP_GEMV_COPY(_p2)
 FHIP_GEMV_COPY(_p3)
 #undef FHIP_GEMV_COPY
@@ -97,6 +99,7 @@ FHIP_GEMV_COPY(_p3)
 int launch_gemv_generic(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 int launch_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, hipStream_t s);
 void gemv_force_generic(bool on);   // debugging / tests: every mat-vec through gemv_generic.hip
+bool gemv_quad_matvec(bool on);     // debugging / tests: off keeps batches of three and more off gemv_quad.hip; returns the setting before
 // One batch-1 GEMV per (token, slot) pair on the selected expert's `out_rows` rows (fused SwiGLU over its
 // gate|up halves when swiglu: then expert_rows = 2 * out_rows). Both files provide it, same contract as above.
 int launch_gemv_norm(const fhip_weight* w, const float* d_x, float* d_y, size_t n_ff, const NormParams& norm, hipStream_t s);

@@ -394,9 +394,11 @@ int fhip_ffn_noalloc(const fhip_weight* gate_up, const fhip_weight* down, const 
  * them) and one more launch adds them in a fixed order, so the same call on the same inputs returns the same bits on every run.
  * FHIP_BATCH_AUTO: the same kernels with the pieces added by f32 atomics instead: a few microseconds per matmul faster, the
  * last bits vary from run to run (within 2e-6 of the largest output).
- * FHIP_BATCH_F32_MATVEC: the streaming mat-vec, up to four rows per pass over the weights; an output row then has the same
- * bits whatever batch it was part of (the guarantee the reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200),
- * at the price of rows_x / 4 (Q6_K: / 2) passes.
+ * FHIP_BATCH_F32_MATVEC: the streaming mat-vec's arithmetic for every row; an output row then has the same bits whatever
+ * batch it was part of (the guarantee the reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200), at the
+ * price of one pass over the weights per four rows (Q4_K and Q6_K: the products of four rows at a time go through the
+ * 4 x 4 x 4 int8 matrix instruction, three quarters of the time of two dot-product passes; other formats: two to four rows
+ * a pass on the dot-product kernel).
  * fhip_weight_batch_policy sets one handle's policy and returns the one before; any value that is no policy only queries. Set it
  * before sizing or reserving the workspace and not while another thread launches on the handle.
  * fhip_batch_policy sets what handles made AFTERWARDS start with (existing handles keep theirs) and returns the previous

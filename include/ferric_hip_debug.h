@@ -19,6 +19,12 @@ int fhip_debug_generic_matvec(int on);
  * launches; fhip_workspace_bytes_coop follows it. No counterpart in the reference. */
 int fhip_debug_gemm_tile(int tile);
 
+/* Debugging and tests: on == 0 keeps Q4_K / Q6_K batches of three and more rows off the kernel that multiplies on the
+ * 4 x 4 x 4 int8 matrix instruction, so that the mat-vec entry points run them on the dot-product kernel two rows at a time
+ * (the two give the same bits; the tests compare them this way). Returns the setting before the call (1 = on, the default).
+ * Process-wide, not thread-safe against concurrent launches. No counterpart in the reference. */
+int fhip_debug_quad_matvec(int on);
+
 /* Measurement aid: one launch that reads nbytes at d_src (16-byte loads over the whole chip) and does nothing else; d_sink is
  * one device word that is practically never written. Timed beside a mat-vec of the same size it gives the time a perfect reader
  * needs for those bytes on this device. No counterpart in the reference (its matvec_roofline example prints bytes / time of the

@@ -114,7 +114,9 @@ def test_fused_projections_from_a_gguf_file(F, O, tmp_path, precision):
         want = g64[:, :n_ff] / (1.0 + np.exp(-g64[:, :n_ff])) * g64[:, n_ff:]
         assert np.abs(got - want).max() <= dot_bar() * np.abs(want).max()
         unfused = p.matmul(xt).swiglu(n_ff).to_vec().reshape(3, n_ff)
-        assert np.abs(got - unfused).max() <= 2e-6 * np.abs(unfused).max()
+        # (three rows: the fused K-quant kernel is the mat-vec, block fixed point activations at the precision under test; the plain
+        # matmul of the unfused steps takes the one-pass f16 kernels. The Q8_0 pair runs the same kernel both ways.)
+        assert np.abs(got - unfused).max() <= (2e-6 if ty == Q8_0 else dot_bar()) * np.abs(unfused).max()
 
 
 def test_cat_of_tensors(F):
