@@ -249,7 +249,9 @@ def bench_ffn(F, lib, check, stream, timer, batches, reps=20, ncopy=4):
         f32 = lambda gu, dn: check(lib.fhip_ffn(gu.handle, dn.handle, x.buf.ptr, b, y.buf.ptr, ws.buf.ptr, stream.handle))
         res[str(b)] = entry(timed(f32, ncopy), b)
         res[str(b)]["warm_one_copy_ms"] = timed(f32, 1)
-        res[str(b)]["path"] = "streaming mat-vec" if b <= 2 else "one-pass f16 hi/lo matrix-core kernels, cut rows added in a fixed order (FHIP_BATCH_ORDERED)"
+        res[str(b)]["path"] = ("streaming mat-vec" if b <= 2 else
+                               "gate|up + SwiGLU on the four-row int8 matrix-instruction mat-vec, down on the one-pass f16 hi/lo kernels, cut rows added in a fixed order (FHIP_BATCH_ORDERED)" if b <= 4 else
+                               "one-pass f16 hi/lo matrix-core kernels, cut rows added in a fixed order (FHIP_BATCH_ORDERED)")
         if b > 2:
             for policy, key in ((0, "atomic_adds_policy"), (1, "f32_matvec_policy")):   # FHIP_BATCH_AUTO, FHIP_BATCH_F32_MATVEC
                 for w in gus + dns:

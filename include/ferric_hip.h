@@ -182,8 +182,10 @@ int fhip_matmul_q(const fhip_weight* w, const float* d_x, size_t rows_x, float* 
  * matmul_q6_k_swiglu: `gate_up` stacks gate rows [0, n_ff) then up rows [n_ff, 2 n_ff);
  * y[rows_x, n_ff] = silu(x*gate^T) * (x*up^T), silu(g) = g / (1 + exp(-g)).
  * Errors: odd row count -> FHIP_ERR_SHAPE; Q8_0 -> FHIP_ERR_UNSUPPORTED_TYPE (reference: None,
- * the caller then runs matmul_q + swiglu). Batches of three rows and more: as fhip_matmul_q, then the un-fused
- * SwiGLU of crates/ferric-tensor/src/lib.rs:2603-2618 over the [rows, 2 n_ff] intermediate in the library's workspace. */
+ * the caller then runs matmul_q + swiglu). Batches of three and four rows (Q4_K, Q6_K): one pass of the mat-vec's
+ * arithmetic for four rows at a time (the int8 matrix instruction; every row has the bits it has in a batch of one, no
+ * workspace). Other batches of three rows and more: as fhip_matmul_q, then the un-fused SwiGLU of
+ * crates/ferric-tensor/src/lib.rs:2603-2618 over the [rows, 2 n_ff] intermediate in the library's workspace. */
 int fhip_matmul_q_swiglu(const fhip_weight* gate_up, const float* d_x, size_t rows_x, float* d_y, void* stream);
 
 /* crates/ferric-tensor/src/lib.rs:728 Tensor::swiglu(d): gu is [t, 2d] = [gate | up] per row,
@@ -192,7 +194,9 @@ int fhip_swiglu(const float* d_gu, size_t t, size_t d, float* d_out, void* strea
 
 /* The FFN block of crates/ferric-llama/src/qwen3.rs:944-964: y = down( swiglu( gate_up(x) ) ).
  * d_ws is caller-provided scratch of at least rows_x * n_ff f32 (n_ff = gate_up rows / 2). Batches of three rows and more
- * run as fhip_ffn_f16x2 does (one pass over each weight per group of up to 32 rows) out of the library's workspace. */
+ * run as fhip_ffn_f16x2 does (one pass over each weight per group of up to 32 rows) out of the library's workspace; in a
+ * group of three or four rows gate|up + SwiGLU is the call fhip_matmul_q_swiglu makes for such a batch, and the block gives
+ * the bits of that call followed by fhip_matmul_q on the down projection. */
 int fhip_ffn(const fhip_weight* gate_up, const fhip_weight* down, const float* d_x, size_t rows_x, float* d_y,
              float* d_ws, void* stream);
 
