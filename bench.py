@@ -814,7 +814,9 @@ def probe_f16x2(F, lib, check, ncopy=4):
     gate|up (34816 x 5120 Q4_K) and down (5120 x 17408 Q6_K) weights, then the whole block through fhip_ffn_f16x2 and through
     fhip_ffn (ordered sums), 12 launches each, eagerly on the null stream, rotating over 4 copies of each weight (694 MB in all, more than the
     Infinity Cache holds) so that every launch reads HBM. Last, 32 launches of fhip_matmul_q_f16x2 over 32 copies of a
-    4096 x 4096 Q8_0 weight (571 MB) and 16 over 16 copies of a 12288 x 4096 one (857 MB), 8 rows each."""
+    4096 x 4096 Q8_0 weight (571 MB) and 16 over 16 copies of a 12288 x 4096 one (857 MB), 8 rows each. Between the two: 12
+    launches of fhip_ffn at 4 rows (gate|up + SwiGLU on the four-row mat-vec, down on the f16 kernels) and 12 with the weights
+    set to FHIP_BATCH_F32_MATVEC (both on the four-row mat-vec)."""
     from ferric_amd.synth import synth_weights
     n_embd, n_ff, t = 5120, 17408, 8
     gbuf = replicate(F, lib, check, synth_weights(Q4_K, 2 * n_ff, n_embd, 3), ncopy)
@@ -842,6 +844,16 @@ def probe_f16x2(F, lib, check, ncopy=4):
     for i in range(12):
         check(lib.fhip_ffn(gus[i % ncopy].handle, dns[i % ncopy].handle, x.buf.ptr, t, y.buf.ptr, hws.buf.ptr, None))
     check(lib.fhip_stream_sync(None))
+    # four rows: fhip_ffn runs gate|up + SwiGLU on the four-row mat-vec (the int8 4 x 4 x 4 matrix instruction) and the down
+    # projection on the f16 kernels; then the same call with every row on the mat-vec's arithmetic (FHIP_BATCH_F32_MATVEC)
+    x4 = F.Tensor.from_vec(np.random.default_rng(6).standard_normal((4, n_embd)).astype(np.float32), (4, n_embd))
+    y4 = F.Tensor.empty((4, n_embd))
+    for policy in (2, 1):
+        for w in gus + dns:
+            w.batch_policy(policy)
+        for i in range(12):
+            check(lib.fhip_ffn(gus[i % ncopy].handle, dns[i % ncopy].handle, x4.buf.ptr, 4, y4.buf.ptr, hws.buf.ptr, None))
+        check(lib.fhip_stream_sync(None))
     del gus, dns, gbuf, dbuf
     for rows, nc in ((4096, 32), (12288, 16)):
         nb = weight_bytes(Q8_0, rows, 4096)
