@@ -846,7 +846,7 @@ def probe_f16x2(F, lib, check, ncopy=4):
     check(lib.fhip_stream_sync(None))
     # four rows: fhip_ffn runs gate|up + SwiGLU on the four-row mat-vec (the int8 4 x 4 x 4 matrix instruction) and the down
     # projection on the f16 kernels; then the same call with every row on the mat-vec's arithmetic (FHIP_BATCH_F32_MATVEC)
-    x4 = F.Tensor.from_vec(np.random.default_rng(6).standard_normal((4, n_embd)).astype(np.float32), (4, n_embd))
+    x4 = F.Tensor.from_vec(np.random.default_rng(5).standard_normal((4, n_embd)).astype(np.float32), (4, n_embd))   # (bench_ffn's rows)
     y4 = F.Tensor.empty((4, n_embd))
     for policy in (2, 1):
         for w in gus + dns:
