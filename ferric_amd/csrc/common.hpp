@@ -90,6 +90,7 @@ int launch_gemv(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
     int launch_gemv_sel##sfx(const fhip_weight* w, const float* d_x, float* d_y, size_t out_rows, bool swiglu,                      \
                              const struct SelParams& sel, hipStream_t s);                                                           \
     void gemv_force_generic##sfx(bool on);                                                                                         \
+    bool gemv_streams##sfx(const fhip_weight* w, size_t n_ff);                                                                      \
     bool gemv_quad_supports##sfx(const fhip_weight* w, size_t rows_x, size_t n_ff);                                                 \
     int launch_gemv_quad##sfx(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_y, size_t n_ff, hipStream_t s);
 FHIP_GEMV_COPY(_p2)

@@ -633,8 +633,9 @@ bool QUAD_EXPORT(gemv_quad_supports)(const fhip_weight* w, size_t rows_x, size_t
     const size_t out_rows = n_ff ? n_ff : w->rows;
     // 32-bit byte offsets inside a workgroup's span and to the up row of a pair
     if (w->row_bytes > 0xFFFFu * 4 || out_rows * w->row_bytes > 0xF0000000ull) return false;
-    const size_t ng = (w->cols / 64 + 15) / 16;
-    return ng <= 40 && ((uintptr_t)w->d_raw & 15) == 0;
+    // only where one or two rows would take the streaming kernel: its bits are what this kernel promises (the longest rows go to
+    // the shape-complete f32 kernel instead)
+    return w->cols <= 32768 && ((uintptr_t)w->d_raw & 15) == 0 && QUAD_EXPORT(gemv_streams)(w, n_ff);
 }
 
 // y [rows_x, out_rows] = x [rows_x, cols] W^T (n_ff != 0: silu(gate) * up over the fused [gate | up] rows), rows_x <= 4

@@ -24,9 +24,11 @@ def both(F, fn):
 
 
 # rows x cols: one group of units and several, a last group that is partly filled (2304 = 36 units), rows that end inside a
-# quad and inside a workgroup's share, fewer rows than the chip has workgroups, rows long enough for a second pass (17408 columns)
+# quad and inside a workgroup's share, fewer rows than the chip has workgroups, rows long enough for a second pass (17408 columns),
+# for three and four passes (28672, 31488 with a partly filled last group, 32768: the longest rows the mat-vec entry points take)
 SHAPES = [(Q4_K, 96, 5120), (Q4_K, 1023, 256), (Q4_K, 7, 2304), (Q4_K, 2050, 1024), (Q4_K, 300, 17408), (Q4_K, 5120, 5120),
-          (Q6_K, 70, 2048), (Q6_K, 40, 17408), (Q6_K, 1, 256), (Q6_K, 1500, 2304), (Q6_K, 5120, 5120), (Q6_K, 515, 11264)]
+          (Q6_K, 70, 2048), (Q6_K, 40, 17408), (Q6_K, 1, 256), (Q6_K, 1500, 2304), (Q6_K, 5120, 5120), (Q6_K, 515, 11264),
+          (Q4_K, 37, 28672), (Q4_K, 12, 31488), (Q6_K, 9, 32768), (Q6_K, 261, 28672)]
 
 
 @pytest.mark.parametrize("ty,rows,cols", SHAPES)
@@ -42,8 +44,9 @@ def test_same_bits_as_the_dot_product_kernel(F, O, ty, rows, cols):
     for m in (3, 4, 7, 8, 9):
         xt = F.Tensor.from_vec(x[:m], (m, cols))
         on, off = both(F, lambda: xt.matmul_q(qm).to_vec().reshape(m, rows))
-        assert np.array_equal(bits(on), bits(off)), (m, "quad against pairs")
         assert np.array_equal(bits(on), bits(singles[:m])), (m, "quad against single rows")
+        if cols <= 17408:       # (two rows of longer columns do not fit the streaming kernel's LDS: pairs then take the f32 kernel)
+            assert np.array_equal(bits(on), bits(off)), (m, "quad against pairs")
     # against f64 on the exactly dequantised weights: the north-star bound everywhere, the bar of the precision under test
     # where a row is long enough for it to be about sums (a single 256-column row at 16 bits is about one run's rounding)
     y64, wn = O.matmul_f64(x[:4], w, ty, rows, cols)
