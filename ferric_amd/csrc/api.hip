@@ -216,10 +216,20 @@ static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t,
 // is part of.
 
 size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32; }
+// Three and four rows of a Q4_K / Q6_K weight whose rows the four-row mat-vec (gemv_quad.hip) covers in one pass (up to 10240
+// columns) take that kernel under every policy: one launch, no workspace, the bits of a batch of one, and faster than the f16
+// kernels with their split and sum launches (cold, ordered sums: 5120 x 5120 17.7 -> 12.5 us, 7168 x 5120 19.9 -> 14.1, Q6_K
+// 151936 x 5120 178 -> 164; with atomic sums 12.6 / 14.5 / 178). Longer rows take two passes and lose (5120 x 17408: 36.6 against
+// 43.8), so they stay on the f16 kernels.
+bool matmul_takes_quad(const fhip_weight* w, size_t t) {
+    if (t < 3 || t > 4 || w->cols > 10240) return false;
+    return w->planes == 3 ? fhip::gemv_quad_supports_p3(w, t, 0) : fhip::gemv_quad_supports_p2(w, t, 0);
+}
 bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
     if (w->batch_policy == FHIP_BATCH_F32_MATVEC) return false;
     if (w->type != FHIP_Q4_K && w->type != FHIP_Q5_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0) return false;
     if (rows_x < (w->type == FHIP_Q8_0 ? 5u : 3u)) return false;
+    if (matmul_takes_quad(w, rows_x)) return false;
     return fhip::gemm_f16x2_supports(w, rows_x < f16x2_group(w) ? rows_x : f16x2_group(w));
 }
 
@@ -227,8 +237,14 @@ bool takes_f16x2(const fhip_weight* w, size_t rows_x) {
 // 34816 x 5120) is faster than the one-pass f16 kernel plus the SwiGLU launch behind it (34 + 4), and its rows carry the bits
 // they have in a batch of one. The plain matmuls of such batches stay on the f16 kernels (down 5120 x 17408: 27 us against 42).
 bool swiglu_takes_quad(const fhip_weight* gu, size_t t) {
-    if (t < 3 || t > 4 || gu->rows % 2 != 0) return false;
+    if (t < 3 || t > 4 || gu->rows % 2 != 0 || gu->cols > 10240) return false;   // (one pass of the kernel, as matmul_takes_quad)
     return gu->planes == 3 ? fhip::gemv_quad_supports_p3(gu, t, gu->rows / 2) : fhip::gemv_quad_supports_p2(gu, t, gu->rows / 2);
+}
+
+// fhip_ffn on a group of t rows needs no library workspace when the down projection does not take the f16 kernels, or when
+// gate|up takes neither them nor the four-row mat-vec: both matmuls then go through the mat-vec launcher.
+bool ffn_direct(const fhip_weight* gu, const fhip_weight* down, size_t t) {
+    return !takes_f16x2(down, t) || (!takes_f16x2(gu, t) && !swiglu_takes_quad(gu, t));
 }
 
 // y [t, rows] = 0 on the stream, by the mat-vec launcher's fill kernel (what a weight without columns gives)
@@ -628,14 +644,14 @@ int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, s
         return set_error(FHIP_ERR_UNSUPPORTED_TYPE, "fhip_ffn: gate_up must be Q4_K or Q6_K");
     }
     hipStream_t s = (hipStream_t)stream;
-    if (!takes_f16x2(gu, rows_x) || !takes_f16x2(down, rows_x)) {
+    size_t grp = f16x2_group(gu) < f16x2_group(down) ? f16x2_group(gu) : f16x2_group(down);
+    const size_t t0 = rows_x < grp ? rows_x : grp;
+    if (ffn_direct(gu, down, t0)) {
         if ((rc = fhip::launch_gemv(gu, d_x, rows_x, d_ws, n_ff, s))) return rc;
         return fhip::launch_gemv(down, d_ws, rows_x, d_y, 0, s);
     }
     // groups of up to 32 rows, each one pass over gate|up and one over down; SwiGLU happens while the rows are prepared
     // for the down projection. The intermediates live in the library's workspace; d_ws is left alone.
-    size_t grp = f16x2_group(gu) < f16x2_group(down) ? f16x2_group(gu) : f16x2_group(down);
-    const size_t t0 = rows_x < grp ? rows_x : grp;
     const size_t mm1 = f16x2_matmul_ws(gu, t0), gb = align256(t0 * gu->rows * sizeof(float));
     void* ws = nullptr;
     if ((rc = lib_workspace(s, mm1 + gb + f16x2_matmul_ws(down, t0), &ws, "fhip_ffn"))) return rc;
@@ -643,7 +659,7 @@ int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, s
     void* ws2 = (uint8_t*)ws + mm1 + gb;
     for (size_t m0 = 0; m0 < rows_x; m0 += grp) {
         const size_t t = rows_x - m0 < grp ? rows_x - m0 : grp;
-        if (!takes_f16x2(gu, t) || !takes_f16x2(down, t)) {
+        if (ffn_direct(gu, down, t)) {
             if ((rc = fhip::launch_gemv(gu, d_x + m0 * gu->cols, t, d_ws + m0 * n_ff, n_ff, s))) return rc;
             rc = fhip::launch_gemv(down, d_ws + m0 * n_ff, t, d_y + m0 * down->rows, 0, s);
         } else if (swiglu_takes_quad(gu, t)) {
@@ -718,10 +734,15 @@ size_t fhip_workspace_bytes(const fhip_weight* gu, const fhip_weight* down, size
     // what fhip_matmul_q (down == NULL), fhip_matmul_q_swiglu (down == NULL) or fhip_ffn asks of the workspace: the largest
     size_t need = 0;
     if (!gu || rows_x == 0) return 0;
+    if (down) {      // fhip_ffn: [gate|up's workspace][the t0 x 2 n_ff intermediate][down's workspace], t0 the widest group
+        const size_t grp = f16x2_group(gu) < f16x2_group(down) ? f16x2_group(gu) : f16x2_group(down);
+        const size_t t0 = rows_x < grp ? rows_x : grp;
+        if (ffn_direct(gu, down, t0)) return 0;
+        return f16x2_matmul_ws(gu, t0) + align256(t0 * gu->rows * sizeof(float)) + f16x2_matmul_ws(down, t0);
+    }
     if (takes_f16x2(gu, rows_x)) {
         const size_t t0 = rows_x < f16x2_group(gu) ? rows_x : f16x2_group(gu);
         need = f16x2_matmul_ws(gu, t0) + align256(t0 * gu->rows * sizeof(float));
-        if (down && takes_f16x2(down, rows_x)) need += f16x2_matmul_ws(down, t0 < f16x2_group(down) ? t0 : f16x2_group(down));
     }
     return need;
 }
