@@ -351,6 +351,8 @@ struct QuadParams {
     int WPS, QS, GPW;    // waves that share a quad of rows (one group each per pass); quads in flight per workgroup; passes
     int rows_wg;         // output rows per workgroup (rows_wg * VPR is a multiple of 4)
     int pieces;          // 8-column pieces of a pass's activations a thread stages
+    uint32_t magic_S;    // ceil(2^32 / (128 WPS)): thread index -> activation row of its first piece
+    int step_m, step_slot;   // threads / (128 WPS), threads % (128 WPS): from one piece of a thread to its next
     uint32_t scales_off, sums_off, ctr_off, part_off;   // byte offsets in LDS: run scales, run sums, quad counters, group sums [virtual row][NG][4]
 };
 
@@ -418,20 +420,28 @@ __global__ void __launch_bounds__(640) gemv_quad_kernel(QuadParams p) {
         // quantiser's lane exchanges all the same).
         if (pass > 0) __syncthreads();                               // the planes of the pass before are still being read
         if (tid < p.WPS) next_quad[tid] = p.QS;                      // quads 0 .. QS-1 are the waves' first; the others are taken as the waves go
-        const int cols_pass = 64 * UP, col_lo = 64 * u_lo, e_step = (int)blockDim.x * 8;
+        // Piece id of a thread's k-th piece: tid + k * threads; id -> activation row m = id / S and 8-column slot id % S of the
+        // pass's columns, S = 128 WPS. Worked out once by a multiplication and carried along by additions (a division and the
+        // address products per piece were as many instructions as the quantiser itself).
+        const int col_lo = 64 * u_lo, S = 128 * p.WPS;
+        const uint32_t UP16 = (uint32_t)UP * 16u, row_stride = (uint32_t)(NRUN * NP * RC) * UP16;
+        int pm = (int)__umulhi((uint32_t)tid, p.magic_S), pslot = tid - pm * S;
         typename F::Data buf[U];
 #pragma unroll 1
         for (int k0 = 0; k0 < p.pieces; k0 += QUAD_PIECES) {         // rounds of QUAD_PIECES pieces a thread: one trip to memory each
             float4 xa[QUAD_PIECES], xb[QUAD_PIECES];
+            int ms[QUAD_PIECES], slots[QUAD_PIECES];
 #pragma unroll
             for (int k = 0; k < QUAD_PIECES; k++) {
-                const int e = tid * 8 + (k0 + k) * e_step;
-                const int m = e / cols_pass, col = col_lo + (e - m * cols_pass);
+                ms[k] = pm; slots[k] = pslot;
+                const int col = col_lo + 8 * pslot;
                 xa[k] = float4{0.f, 0.f, 0.f, 0.f}; xb[k] = xa[k];
-                if (k0 + k < p.pieces && m < p.rows_x && col < p.cols) {
-                    const float* src = p.x + (size_t)m * p.cols + col;
+                if (k0 + k < p.pieces && pm < p.rows_x && col < p.cols) {
+                    const float* src = p.x + ((uint32_t)__umul24(pm, p.cols) + (uint32_t)col);
                     xa[k] = *(const float4*)src; xb[k] = *(const float4*)(src + 4);
                 }
+                pm += p.step_m; pslot += p.step_slot;
+                if (pslot >= S) { pslot -= S; pm++; }
             }
             if (k0 == 0) {                                           // the wave's first quad goes out behind the first activations
                 asm volatile("" ::: "memory");
@@ -440,22 +450,20 @@ __global__ void __launch_bounds__(640) gemv_quad_kernel(QuadParams p) {
             }
 #pragma unroll
             for (int k = 0; k < QUAD_PIECES; k++) {
-                const int e = tid * 8 + (k0 + k) * e_step;
-                if (k0 + k < p.pieces && e < 4 * cols_pass) {        // whole waves: 4 cols_pass / 8 is a multiple of 64
-                    const int m = e / cols_pass, cl = e - m * cols_pass, col = col_lo + cl;
+                if (k0 + k < p.pieces && ms[k] < 4) {                // whole waves: an activation row's 128 WPS pieces are a multiple of 64
+                    const int m = ms[k], cl = 8 * slots[k], col = col_lo + cl;
                     const float v[8] = {xa[k].x, xa[k].y, xa[k].z, xa[k].w, xb[k].x, xb[k].y, xb[k].z, xb[k].w};
                     uint32_t pl[NP][2];
                     float scale, qsum;
                     quantize8<RUN>(v, pl, scale, qsum);
-                    const int within = cl % RUN;
+                    const int within = cl & (RUN - 1);
                     int gu, j;                                       // the unit that uses the run, and which of its runs it is
                     F::owner(col / RUN, gu, j);
                     const int ul = gu - u_lo;
-                    const int mj = m * NRUN + j;
+                    uint8_t* dst = planes + (__umul24(m, row_stride) + __umul24(j * (NP * RC) + (within >> 4), UP16) + (uint32_t)(ul * 16 + (within & 15)));
 #pragma unroll
-                    for (int pp = 0; pp < NP; pp++)
-                        *(u32x2*)(planes + ((size_t)((mj * NP + pp) * RC + (within >> 4)) * UP + ul) * 16 + (within & 15)) = u32x2{pl[pp][0], pl[pp][1]};
-                    if (within == 0) { scales[ul * (4 * NRUN) + mj] = scale; sums[ul * (4 * NRUN) + mj] = qsum; }
+                    for (int pp = 0; pp < NP; pp++) *(u32x2*)(dst + pp * (RC * UP16)) = u32x2{pl[pp][0], pl[pp][1]};
+                    if (within == 0) { scales[ul * (4 * NRUN) + m * NRUN + j] = scale; sums[ul * (4 * NRUN) + m * NRUN + j] = qsum; }
                 }
             }
         }
@@ -611,6 +619,9 @@ int launch_quad(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
     const unsigned threads = 64u * (unsigned)(p.WPS * p.QS);
     // 8-column pieces of a pass (4 rows x 1024 WPS columns) per thread
     p.pieces = (int)((4 * 128 * (size_t)p.WPS + threads - 1) / threads);
+    const unsigned S = 128u * (unsigned)p.WPS;
+    p.magic_S = (uint32_t)(((1ull << 32) + S - 1) / S);
+    p.step_m = (int)(threads / S); p.step_slot = (int)(threads % S);
     const size_t lds = stage + (size_t)rows_wg * VPR * p.NG * 16;
     static bool lds_raised = false;
     if (!lds_raised) {  // workgroups may use more than the default 64 KiB of the CU's 160 KiB
