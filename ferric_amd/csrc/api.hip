@@ -103,7 +103,7 @@ int device_cus() { return g_cus; }
 size_t device_lds_bytes() { return g_lds; }
 
 // The streaming mat-vec exists in two copies, one per activation precision; these forward to the one the weight names.
-// From three rows on, Q4_K and Q6_K batches go four rows at a time through the kernel that multiplies on the 4 x 4 x 4 int8
+// From three rows on, Q4_K, Q5_K and Q6_K batches go four rows at a time through the kernel that multiplies on the 4 x 4 x 4 int8
 // matrix instruction (gemv_quad.hip: the same arithmetic and the same bits per row, one pass over the weight for four rows);
 // what is left of a batch, one or two rows, and every other format take the dot-product kernel.
 bool g_quad_matvec = true, g_generic_forced = false;
@@ -212,11 +212,11 @@ static int gemm_bf16_lib_ws(const fhip_weight* w, const uint16_t* d_x, size_t t,
 // One or two activation rows go through the streaming mat-vec (one pass over the weights serves two rows). From three rows on
 // (five for Q8_0) the f16 hi/lo matrix-core kernels read the weights once for up to 32 (Q8_0: 16) rows; longer batches are cut
 // into such groups. FHIP_BATCH_F32_MATVEC keeps every batch on the mat-vec's arithmetic (launch_gemv: four rows a pass on the
-// int8 matrix instruction for Q4_K / Q6_K, the dot-product kernel otherwise): a row then has the same bits whatever batch it
+// int8 matrix instruction for Q4_K / Q5_K / Q6_K, the dot-product kernel otherwise): a row then has the same bits whatever batch it
 // is part of.
 
 size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32; }
-// Three and four rows of a Q4_K / Q6_K weight whose rows the four-row mat-vec (gemv_quad.hip) covers in one pass (up to 10240
+// Three and four rows of a Q4_K / Q5_K / Q6_K weight whose rows the four-row mat-vec (gemv_quad.hip) covers in one pass (up to 10240
 // columns) take that kernel under every policy: one launch, no workspace, the bits of a batch of one, and faster than the f16
 // kernels with their split and sum launches (cold, ordered sums: 5120 x 5120 17.7 -> 12.5 us, 7168 x 5120 19.9 -> 14.1, Q6_K
 // 151936 x 5120 178 -> 164; with atomic sums 12.6 / 14.5 / 178). Longer rows take two passes and lose (5120 x 17408: 36.6 against

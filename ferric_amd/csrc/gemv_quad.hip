@@ -1,4 +1,4 @@
-// Mat-vec for three or four activation rows in one pass over a Q4_K or Q6_K weight (the reference's matmul_q4_k /
+// Mat-vec for three or four activation rows in one pass over a Q4_K, Q5_K or Q6_K weight (the reference's matmul_q4_k /
 // matmul_q6_k / matmul_q4_k_swiglu at small M, crates/ferric-tensor/src/dtype.rs:954-1003, and the CPU row loop
 // crates/ferric-tensor/src/cpu_simd.rs:175-200 whose result for a row does not depend on the rows beside it).
 //
@@ -177,6 +177,85 @@ struct Q4K {
             // sum x * nibble = (sum x * 16 (nibble - 8)) / 16 + 8 sum x
             const float f1 = fmaf(xs(m, 1) * 0.0625f, planes_f32(a1), 8.0f * xq1);
             // sum_l x_l (d*sc*q_l - dmin*m) = d * (sc0 f0 + sc1 f1) - dmin * (m0 sum0 + m1 sum1)
+            outs[m] = d * fmaf(s1, f1, s0 * f0) - dmin * fmaf(n1, xq1, n0 * xq0);
+        }
+    }
+};
+
+// Q5_K: 176 B = [f16 d][f16 dmin][12 B 6-bit scales/mins][qh 32 B][qs 128 B] -- Q4_K plus bit s of qh[l] as the fifth bit of
+// element l of sub-block s (crates/ferric-gguf/src/lib.rs:692-716). Unit = group g of block b (sub-blocks 2g, 2g+1): its 32
+// quant bytes and the whole 32 bytes of high bits; codes 0..31.
+struct Q5K {
+    static constexpr uint32_t TYPE = FHIP_Q5_K;
+    // (weight quads in flight: a unit is 20 registers, and with three activation planes two of them spill)
+    static constexpr int RUN = 32, NRUN = 2, NS = 6, DEPTH = NP == 3 ? 1 : 2;
+    struct Lane { uint32_t off_h, off_q, sh, g2, m1, m2, m3; };
+    struct Data {
+        u32x4 h, b0, b1, q0, q1;
+        __device__ __forceinline__ void pin_all() { pin(h); pin(b0); pin(b1); pin(q0); pin(q1); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        const int b = u >> 2, g = u & 3;
+        L.off_h = b * 176;
+        L.off_q = b * 176 + 48 + 32 * g;
+        L.sh = 16 * (g & 1);
+        L.g2 = 2 * g;
+        L.m1 = g >= 2 ? 0u : 0x3F3Fu;
+        L.m2 = g >= 2 ? 0x0F0Fu : 0u;
+        L.m3 = g >= 2 ? 0x3030u : 0u;
+        run[0] = 2 * u;
+        run[1] = 2 * u + 1;
+    }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r >> 1; j = r & 1; }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+        Data d;
+        d.h = *(const u32x4*)(row + L.off_h);
+        d.b0 = *(const u32x4*)(row + L.off_h + 16);
+        d.b1 = *(const u32x4*)(row + L.off_h + 32);
+        d.q0 = *(const u32x4*)(row + L.off_q);
+        d.q1 = *(const u32x4*)(row + L.off_q + 16);
+        return d;
+    }
+    template <class PL, class XS, class XQ>
+    static __device__ __forceinline__ void unit_sums(const Data& D, const Lane& L, PL plane, XS xs, XQ xq, float (&outs)[4]) {
+        i32x4 acc[NRUN][NP];
+#pragma unroll
+        for (int j = 0; j < NRUN; j++)
+#pragma unroll
+            for (int p = 0; p < NP; p++) acc[j][p] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            uint32_t lo[4], hi[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t w = c == 0 ? D.q0[k] : D.q1[k];
+                const uint32_t hb = (c == 0 ? D.b0[k] : D.b1[k]) >> L.g2;   // bit 0: sub-block 2g, bit 1: sub-block 2g+1
+                lo[k] = (w & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4);
+                hi[k] = ((w >> 4) & 0x0F0F0F0Fu) | ((hb & 0x02020202u) << 3);
+            }
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const u32x4 x0 = plane(0, p, c), x1 = plane(1, p, c);
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    acc[0][p] = mma(x0[k], lo[k], acc[0][p]);
+                    acc[1][p] = mma(x1[k], hi[k], acc[1][p]);
+                }
+            }
+        }
+        const uint32_t a = D.h[1] >> L.sh, b = D.h[2] >> L.sh, c = D.h[3] >> L.sh;
+        const uint32_t scp = (a & L.m1) | (c & L.m2) | ((a >> 2) & L.m3);
+        const uint32_t mp = (b & L.m1) | ((c >> 4) & L.m2) | ((b >> 2) & L.m3);
+        const float d = f16_bits(D.h[0] & 0xFFFFu), dmin = f16_bits(D.h[0] >> 16);
+        const float s0 = ub(scp, 0), s1 = ub(scp, 1), n0 = ub(mp, 0), n1 = ub(mp, 1);
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            int a0[NP], a1[NP];
+#pragma unroll
+            for (int p = 0; p < NP; p++) { a0[p] = acc[0][p][m]; a1[p] = acc[1][p][m]; }
+            const float xq0 = xq(m, 0), xq1 = xq(m, 1);
+            const float f0 = xs(m, 0) * planes_f32(a0);
+            const float f1 = xs(m, 1) * planes_f32(a1);
             outs[m] = d * fmaf(s1, f1, s0 * f0) - dmin * fmaf(n1, xq1, n0 * xq0);
         }
     }
@@ -638,7 +717,7 @@ int launch_quad(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
 namespace fhip {
 
 bool QUAD_EXPORT(gemv_quad_supports)(const fhip_weight* w, size_t rows_x, size_t n_ff) {
-    if (!w || (w->type != FHIP_Q4_K && w->type != FHIP_Q6_K)) return false;
+    if (!w || (w->type != FHIP_Q4_K && w->type != FHIP_Q5_K && w->type != FHIP_Q6_K)) return false;
     if (rows_x < 1 || rows_x > 4 || w->cols == 0 || w->cols % 256 != 0 || w->rows == 0) return false;
     if (n_ff ? w->rows != 2 * n_ff : false) return false;
     const size_t out_rows = n_ff ? n_ff : w->rows;
@@ -654,6 +733,7 @@ int QUAD_EXPORT(launch_gemv_quad)(const fhip_weight* w, const float* d_x, size_t
     if (!QUAD_EXPORT(gemv_quad_supports)(w, rows_x, n_ff)) return set_error(FHIP_ERR_ARG, "gemv_quad: unsupported weight or batch");
     const size_t out_rows = n_ff ? n_ff : w->rows;
     if (w->type == FHIP_Q4_K) return n_ff ? launch_quad<Q4K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_quad<Q4K, false>(w, d_x, rows_x, d_y, out_rows, s);
+    if (w->type == FHIP_Q5_K) return n_ff ? launch_quad<Q5K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_quad<Q5K, false>(w, d_x, rows_x, d_y, out_rows, s);
     return n_ff ? launch_quad<Q6K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_quad<Q6K, false>(w, d_x, rows_x, d_y, out_rows, s);
 }
 

@@ -8,7 +8,7 @@ import pytest
 from conftest import bits, dot_bar
 
 pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("precision")]
-Q4_K, Q6_K = 12, 14
+Q4_K, Q5_K, Q6_K = 12, 13, 14
 
 
 def both(F, fn):
@@ -28,7 +28,8 @@ def both(F, fn):
 # for three and four passes (28672, 31488 with a partly filled last group, 32768: the longest rows the mat-vec entry points take)
 SHAPES = [(Q4_K, 96, 5120), (Q4_K, 1023, 256), (Q4_K, 7, 2304), (Q4_K, 2050, 1024), (Q4_K, 300, 17408), (Q4_K, 5120, 5120),
           (Q6_K, 70, 2048), (Q6_K, 40, 17408), (Q6_K, 1, 256), (Q6_K, 1500, 2304), (Q6_K, 5120, 5120), (Q6_K, 515, 11264),
-          (Q4_K, 37, 28672), (Q4_K, 12, 31488), (Q6_K, 9, 32768), (Q6_K, 261, 28672)]
+          (Q4_K, 37, 28672), (Q4_K, 12, 31488), (Q6_K, 9, 32768), (Q6_K, 261, 28672),
+          (Q5_K, 96, 5120), (Q5_K, 7, 2304), (Q5_K, 5120, 5120), (Q5_K, 130, 17408), (Q5_K, 1023, 256)]
 
 
 @pytest.mark.parametrize("ty,rows,cols", SHAPES)
@@ -56,7 +57,7 @@ def test_same_bits_as_the_dot_product_kernel(F, O, ty, rows, cols):
         assert np.abs(y - y64).max() / max(1e-3, np.abs(y64).max()) < dot_bar()
 
 
-@pytest.mark.parametrize("ty,n_ff,cols", [(Q4_K, 1024, 1024), (Q4_K, 333, 2304), (Q6_K, 96, 512), (Q4_K, 17408, 5120)])
+@pytest.mark.parametrize("ty,n_ff,cols", [(Q4_K, 1024, 1024), (Q4_K, 333, 2304), (Q6_K, 96, 512), (Q4_K, 17408, 5120), (Q5_K, 500, 1536)])
 def test_fused_swiglu_same_bits(F, O, ty, n_ff, cols):
     from ferric_amd.synth import synth_weights
     gu = synth_weights(ty, 2 * n_ff, cols, 5)
@@ -70,7 +71,7 @@ def test_fused_swiglu_same_bits(F, O, ty, n_ff, cols):
         assert np.array_equal(bits(on), bits(off)) and np.array_equal(bits(on), bits(singles[:m])), m
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
 def test_runs_block_fixed_point_cannot_hold(F, O, ty):
     """Non-finite activations and runs at the ends of the f32 range take the element-by-element pass: the same bits as on
     the dot-product kernel there too, NaN for NaN."""
