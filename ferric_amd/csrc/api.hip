@@ -222,7 +222,7 @@ size_t f16x2_group(const fhip_weight* w) { return w->type == FHIP_Q8_0 ? 16 : 32
 // 151936 x 5120 178 -> 164; with atomic sums 12.6 / 14.5 / 178). Longer rows take two passes and lose (5120 x 17408: 36.6 against
 // 43.8), so they stay on the f16 kernels.
 bool matmul_takes_quad(const fhip_weight* w, size_t t) {
-    if (t < 3 || t > 4 || w->cols > 10240) return false;
+    if (t < 3 || t > 4 || w->cols > 10240) return false;      // (Q8_0: 5120, gemv_quad_supports)
     return w->planes == 3 ? fhip::gemv_quad_supports_p3(w, t, 0) : fhip::gemv_quad_supports_p2(w, t, 0);
 }
 bool takes_f16x2(const fhip_weight* w, size_t rows_x) {

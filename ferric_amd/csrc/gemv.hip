@@ -1399,12 +1399,13 @@ int GEMV_EXPORT(launch_gemv)(const fhip_weight* w, const float* d_x, size_t rows
     }
 }
 
-// Whether launch_gemv runs this Q4_K / Q5_K / Q6_K weight on the streaming kernel (and not on the shape-complete f32 kernel, whose
+// Whether launch_gemv runs this Q4_K / Q5_K / Q6_K / Q8_0 weight on the streaming kernel (and not on the shape-complete f32 kernel, whose
 // sums round differently): the four-row mat-vec, which promises the streaming kernel's bits, takes a weight only then.
 bool GEMV_EXPORT(gemv_streams)(const fhip_weight* w, size_t n_ff) {
     if (w->type == FHIP_Q4_K) return (n_ff ? max_batch<Q4K, true>(w, 1) : max_batch<Q4K, false>(w, 1)) > 0;
     if (w->type == FHIP_Q6_K) return (n_ff ? max_batch<Q6K, true>(w, 1) : max_batch<Q6K, false>(w, 1)) > 0;
     if (w->type == FHIP_Q5_K) return (n_ff ? max_batch<Q5K, true>(w, 1) : max_batch<Q5K, false>(w, 1)) > 0;
+    if (w->type == FHIP_Q8_0) return !n_ff && max_batch<Q80, false>(w, 1) > 0;
     return false;
 }
 

@@ -1,4 +1,4 @@
-// Mat-vec for three or four activation rows in one pass over a Q4_K, Q5_K or Q6_K weight (the reference's matmul_q4_k /
+// Mat-vec for three or four activation rows in one pass over a Q4_K, Q5_K, Q6_K or Q8_0 weight (the reference's matmul_q4_k /
 // matmul_q6_k / matmul_q4_k_swiglu at small M, crates/ferric-tensor/src/dtype.rs:954-1003, and the CPU row loop
 // crates/ferric-tensor/src/cpu_simd.rs:175-200 whose result for a row does not depend on the rows beside it).
 //
@@ -6,7 +6,7 @@
 // or 32 columns, two or three signed byte planes), exact integer dot products per run, the same f32 operations in the same
 // order above them, the same trees for the sums over a row's units. What differs is who multiplies. Here the integer
 // products go through v_mfma_i32_4x4x4_16b_i8: sixteen independent 4 x 4 x 4 products per wave. A wave's lane l = 4 u + r
-// holds unit u (64 weights) of WEIGHT row r of a quad of four rows as the B operand (four bytes of it are four consecutive
+// holds unit u (64 weights; a block of 32 for Q8_0) of WEIGHT row r of a quad of four rows as the B operand (four bytes of it are four consecutive
 // columns: one column of B) and the planes of unit u of ACTIVATION row r as the A operand (one row of A). Block u of the
 // instruction then gives all 16 (activation row, weight row) dot products of the unit's four columns, and lane 4 u + r ends
 // up with its own weight row's sums against the four activation rows in its four accumulator registers -- next to that
@@ -87,7 +87,7 @@ __device__ __forceinline__ float planes_f32(const int (&a)[NP]) {
 __device__ __forceinline__ i32x4 mma(uint32_t a, uint32_t b, i32x4 c) { return __builtin_amdgcn_mfma_i32_4x4x4i8((int)a, (int)b, c, 0, 0, 0); }
 
 // ------------------------------------------------------------------------------------------------
-// Per-format lane work. A unit is 64 weights of one row, read as the streaming mat-vec reads it; a lane needs NRUN activation
+// Per-format lane work. A unit is WPL weights of one row, read as the streaming mat-vec reads it; a lane needs NRUN activation
 // runs of RUN columns, run j being columns [run[j] * RUN, run[j] * RUN + RUN).
 //   products() : the unit's integer products with the lane's activation planes, one accumulator quad per (run, plane);
 //                element m of a quad is the lane's weight row against activation row m
@@ -97,7 +97,7 @@ __device__ __forceinline__ i32x4 mma(uint32_t a, uint32_t b, i32x4 c) { return _
 // ------------------------------------------------------------------------------------------------
 struct Q4K {
     static constexpr uint32_t TYPE = FHIP_Q4_K;
-    static constexpr int RUN = 32, NRUN = 2, NS = 6, DEPTH = 2;
+    static constexpr int WPL = 64, RUN = 32, NRUN = 2, NS = 6, DEPTH = 2;
     struct Lane { uint32_t off_h, off_q, sh, m1, m2, m3; };
     struct Data {
         u32x4 h, q0, q1;
@@ -188,7 +188,7 @@ struct Q4K {
 struct Q5K {
     static constexpr uint32_t TYPE = FHIP_Q5_K;
     // (weight quads in flight: a unit is 20 registers, and with three activation planes two of them spill)
-    static constexpr int RUN = 32, NRUN = 2, NS = 6, DEPTH = NP == 3 ? 1 : 2;
+    static constexpr int WPL = 64, RUN = 32, NRUN = 2, NS = 6, DEPTH = NP == 3 ? 1 : 2;
     struct Lane { uint32_t off_h, off_q, sh, g2, m1, m2, m3; };
     struct Data {
         u32x4 h, b0, b1, q0, q1;
@@ -265,7 +265,7 @@ struct Q6K {
     static constexpr uint32_t TYPE = FHIP_Q6_K;
     // (weight quads a wave has in flight: with three activation planes a second one spills 20 registers, and the down
     // projection 5120 x 17408 at four rows takes 58 us with it against 44 without)
-    static constexpr int RUN = 16, NRUN = 4, NS = 5, DEPTH = NP == 3 ? 1 : 2;
+    static constexpr int WPL = 64, RUN = 16, NRUN = 4, NS = 5, DEPTH = NP == 3 ? 1 : 2;
     struct Lane { uint32_t off_a, off_h, off_s, off_d, ssh; };
     struct Data {
         u32x4 a, b, h; u32x2 s; uint32_t d;
@@ -417,6 +417,53 @@ __device__ __forceinline__ void quantize8(const float (&v)[8], uint32_t (&pl)[NP
     sum_out = scale * (float)qsum;
 }
 
+// Q8_0: 34 B = [f16 d][32 int8] (crates/ferric-gguf/src/lib.rs:608-615). Unit = one block: the quants are the B operand as they
+// lie in memory.
+struct Q80 {
+    static constexpr uint32_t TYPE = FHIP_Q8_0;
+    static constexpr int WPL = 32, RUN = 32, NRUN = 1, NS = 1, DEPTH = 2;
+    struct Lane { uint32_t off; };
+    struct Data {
+        u32x4 q0, q1; uint32_t d;
+        __device__ __forceinline__ void pin_all() { pin(q0); pin(q1); pin(d); }
+    };
+    static __device__ __forceinline__ void setup(int u, Lane& L, int (&run)[NRUN]) {
+        L.off = u * 34;
+        run[0] = u;
+    }
+    static __device__ __forceinline__ void owner(int r, int& u, int& j) { u = r; j = 0; }
+    static __device__ __forceinline__ Data load(const uint8_t* row, const Lane& L) {
+        Data d;
+        d.d = *(const uint16_t*)(row + L.off);
+        d.q0 = ((const U4A2*)(row + L.off + 2))->v;
+        d.q1 = ((const U4A2*)(row + L.off + 18))->v;
+        return d;
+    }
+    template <class PL, class XS, class XQ>
+    static __device__ __forceinline__ void unit_sums(const Data& D, const Lane&, PL plane, XS xs, XQ, float (&outs)[4]) {
+        i32x4 acc[NP];
+#pragma unroll
+        for (int p = 0; p < NP; p++) acc[p] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const u32x4 x = plane(0, p, c);
+#pragma unroll
+                for (int k = 0; k < 4; k++) acc[p] = mma(x[k], c == 0 ? D.q0[k] : D.q1[k], acc[p]);
+            }
+        const float d = f16_bits(D.d);
+        // per block: part = sum x*q, then part*d -- crates/ferric-tensor/src/cpu_simd.rs:66-70
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            int a[NP];
+#pragma unroll
+            for (int p = 0; p < NP; p++) a[p] = acc[p][m];
+            outs[m] = (xs(m, 0) * planes_f32(a)) * d;
+        }
+    }
+};
+
 struct QuadParams {
     const uint8_t* W;
     const float* x;      // [rows_x, cols]
@@ -426,12 +473,12 @@ struct QuadParams {
     int cols;
     uint32_t row_bytes;
     uint32_t pair_bytes; // fused SwiGLU: byte distance from gate row r to up row r
-    int units, NG;       // 64-weight units per row; 16-unit groups per row
+    int units, NG;       // units (F::WPL weights) per row; 16-unit groups per row
     int WPS, QS, GPW;    // waves that share a quad of rows (one group each per pass); quads in flight per workgroup; passes
     int rows_wg;         // output rows per workgroup (rows_wg * VPR is a multiple of 4)
     int pieces;          // 8-column pieces of a pass's activations a thread stages
-    uint32_t magic_S;    // ceil(2^32 / (128 WPS)): thread index -> activation row of its first piece
-    int step_m, step_slot;   // threads / (128 WPS), threads % (128 WPS): from one piece of a thread to its next
+    uint32_t magic_S;    // ceil(2^32 / S), S = 2 WPL WPS the pieces of one activation row of a pass: thread index -> activation row of its first piece
+    int step_m, step_slot;   // threads / S, threads % S: from one piece of a thread to its next
     uint32_t scales_off, sums_off, ctr_off, part_off;   // byte offsets in LDS: run scales, run sums, quad counters, group sums [virtual row][NG][4]
 };
 
@@ -493,16 +540,16 @@ __global__ void __launch_bounds__(640) gemv_quad_kernel(QuadParams p) {
         };
 
         // ---- the pass's activations -> block fixed point, once per workgroup, through LDS: thread t takes the eight columns
-        // from 8 t of the pass's 4 x (64 UP) values, then 8 (t + threads), ...; all of a thread's pieces are requested before the
+        // from 8 t of the pass's 4 x (WPL UP) values, then 8 (t + threads), ...; all of a thread's pieces are requested before the
         // first is used, so that they cost one trip to memory, and the first weight quads go out right behind them. A piece
         // past the row's end or of an activation row the batch does not have is staged as zeros (its lanes take part in the
         // quantiser's lane exchanges all the same).
         if (pass > 0) __syncthreads();                               // the planes of the pass before are still being read
         if (tid < p.WPS) next_quad[tid] = p.QS;                      // quads 0 .. QS-1 are the waves' first; the others are taken as the waves go
         // Piece id of a thread's k-th piece: tid + k * threads; id -> activation row m = id / S and 8-column slot id % S of the
-        // pass's columns, S = 128 WPS. Worked out once by a multiplication and carried along by additions (a division and the
+        // pass's columns, S = 2 WPL WPS. Worked out once by a multiplication and carried along by additions (a division and the
         // address products per piece were as many instructions as the quantiser itself).
-        const int col_lo = 64 * u_lo, S = 128 * p.WPS;
+        const int col_lo = F::WPL * u_lo, S = (F::WPL / 8) * 16 * p.WPS;
         const uint32_t UP16 = (uint32_t)UP * 16u, row_stride = (uint32_t)(NRUN * NP * RC) * UP16;
         int pm = (int)__umulhi((uint32_t)tid, p.magic_S), pslot = tid - pm * S;
         typename F::Data buf[U];
@@ -529,7 +576,7 @@ __global__ void __launch_bounds__(640) gemv_quad_kernel(QuadParams p) {
             }
 #pragma unroll
             for (int k = 0; k < QUAD_PIECES; k++) {
-                if (k0 + k < p.pieces && ms[k] < 4) {                // whole waves: an activation row's 128 WPS pieces are a multiple of 64
+                if (k0 + k < p.pieces && ms[k] < 4) {                // whole waves: an activation row's S pieces are a multiple of 64
                     const int m = ms[k], cl = 8 * slots[k], col = col_lo + cl;
                     const float v[8] = {xa[k].x, xa[k].y, xa[k].z, xa[k].w, xb[k].x, xb[k].y, xb[k].z, xb[k].w};
                     uint32_t pl[NP][2];
@@ -669,14 +716,14 @@ int launch_quad(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
     p.rows_x = (int)rows_x; p.out_rows = (int)out_rows; p.cols = (int)w->cols;
     p.row_bytes = (uint32_t)w->row_bytes;
     p.pair_bytes = (uint32_t)(out_rows * w->row_bytes);
-    p.units = (int)(w->cols / 64);
+    p.units = (int)(w->cols / F::WPL);
     p.NG = (p.units + 15) / 16;
     p.GPW = (p.NG + MAXW - 1) / MAXW;
     p.WPS = (p.NG + p.GPW - 1) / p.GPW;
     p.QS = MAXW / p.WPS;
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    // LDS: a pass's staged activations (4 rows x 1024 WPS columns: planes, run scales, run sums), then the group sums
-    const size_t plane_bytes = (size_t)4 * 1024 * p.WPS * NP, sc_bytes = (size_t)16 * p.WPS * 4 * F::NRUN * sizeof(float);
+    // LDS: a pass's staged activations (4 rows x 16 WPL WPS columns: planes, run scales, run sums), then the group sums
+    const size_t plane_bytes = (size_t)4 * (16 * F::WPL) * p.WPS * NP, sc_bytes = (size_t)16 * p.WPS * 4 * F::NRUN * sizeof(float);
     p.scales_off = (uint32_t)plane_bytes;
     p.sums_off = p.scales_off + (uint32_t)sc_bytes;
     p.ctr_off = p.sums_off + (uint32_t)sc_bytes;
@@ -696,9 +743,9 @@ int launch_quad(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
     if (p.QS > quads) p.QS = quads;                      // no wave without a quad
     const unsigned grid = (unsigned)((out_rows + rows_wg - 1) / rows_wg);
     const unsigned threads = 64u * (unsigned)(p.WPS * p.QS);
-    // 8-column pieces of a pass (4 rows x 1024 WPS columns) per thread
-    p.pieces = (int)((4 * 128 * (size_t)p.WPS + threads - 1) / threads);
-    const unsigned S = 128u * (unsigned)p.WPS;
+    // 8-column pieces of a pass (4 rows x 16 WPL WPS columns) per thread
+    const unsigned S = (unsigned)(F::WPL / 8) * 16u * (unsigned)p.WPS;
+    p.pieces = (int)((4 * (size_t)S + threads - 1) / threads);
     p.magic_S = (uint32_t)(((1ull << 32) + S - 1) / S);
     p.step_m = (int)(threads / S); p.step_slot = (int)(threads % S);
     const size_t lds = stage + (size_t)rows_wg * VPR * p.NG * 16;
@@ -717,8 +764,11 @@ int launch_quad(const fhip_weight* w, const float* d_x, size_t rows_x, float* d_
 namespace fhip {
 
 bool QUAD_EXPORT(gemv_quad_supports)(const fhip_weight* w, size_t rows_x, size_t n_ff) {
-    if (!w || (w->type != FHIP_Q4_K && w->type != FHIP_Q5_K && w->type != FHIP_Q6_K)) return false;
-    if (rows_x < 1 || rows_x > 4 || w->cols == 0 || w->cols % 256 != 0 || w->rows == 0) return false;
+    if (!w || (w->type != FHIP_Q4_K && w->type != FHIP_Q5_K && w->type != FHIP_Q6_K && w->type != FHIP_Q8_0)) return false;
+    if (rows_x < 1 || rows_x > 4 || w->cols == 0 || w->rows == 0) return false;
+    // Q8_0: no fused SwiGLU (the reference has none), and rows the kernel covers in one pass (ten groups of 16 blocks): longer
+    // rows have the four-row dot-product kernel, one pass whatever their length
+    if (w->type == FHIP_Q8_0 ? (n_ff != 0 || w->cols % 32 != 0 || w->cols > 5120) : w->cols % 256 != 0) return false;
     if (n_ff ? w->rows != 2 * n_ff : false) return false;
     const size_t out_rows = n_ff ? n_ff : w->rows;
     // 32-bit byte offsets inside a workgroup's span and to the up row of a pair
@@ -733,6 +783,7 @@ int QUAD_EXPORT(launch_gemv_quad)(const fhip_weight* w, const float* d_x, size_t
     if (!QUAD_EXPORT(gemv_quad_supports)(w, rows_x, n_ff)) return set_error(FHIP_ERR_ARG, "gemv_quad: unsupported weight or batch");
     const size_t out_rows = n_ff ? n_ff : w->rows;
     if (w->type == FHIP_Q4_K) return n_ff ? launch_quad<Q4K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_quad<Q4K, false>(w, d_x, rows_x, d_y, out_rows, s);
+    if (w->type == FHIP_Q8_0) return launch_quad<Q80, false>(w, d_x, rows_x, d_y, out_rows, s);
     if (w->type == FHIP_Q5_K) return n_ff ? launch_quad<Q5K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_quad<Q5K, false>(w, d_x, rows_x, d_y, out_rows, s);
     return n_ff ? launch_quad<Q6K, true>(w, d_x, rows_x, d_y, out_rows, s) : launch_quad<Q6K, false>(w, d_x, rows_x, d_y, out_rows, s);
 }

@@ -170,7 +170,7 @@ int fhip_deq_raw(const uint8_t* h_raw, size_t nbytes, size_t n, uint32_t ggml_ty
  * :1172 matmul_q6_k): y[rows_x, rows] = x[rows_x, cols] * W^T, f32 in, f32 accumulate, f32 out.
  * rows_x = 1 is the decode GEMV; any rows_x >= 1 is accepted.
  * Which kernel a batch takes (fhip_batch_policy): one or two rows go through the streaming mat-vec; three and four rows of a
- * Q4_K / Q5_K / Q6_K weight with rows of up to 10240 columns through its four-row form (the same arithmetic on the int8 matrix
+ * Q4_K / Q5_K / Q6_K weight with rows of up to 10240 columns (Q8_0: 5120) through its four-row form (the same arithmetic on the int8 matrix
  * instruction: every row has the bits it has in a batch of one; one launch, no workspace); otherwise, from three rows on (five
  * for Q8_0) Q4_K / Q5_K / Q6_K / Q8_0 weights are read once per group of up to 32 (Q8_0: 16) rows by the f16 hi/lo matrix-core
  * kernels (see fhip_matmul_q_f16x2: f32-grade, 22-bit activations), longer batches group by group. That path keeps its
@@ -402,7 +402,7 @@ int fhip_ffn_noalloc(const fhip_weight* gate_up, const fhip_weight* down, const 
  * last bits vary from run to run (within 2e-6 of the largest output).
  * FHIP_BATCH_F32_MATVEC: the streaming mat-vec's arithmetic for every row; an output row then has the same bits whatever
  * batch it was part of (the guarantee the reference's CPU path gives, crates/ferric-tensor/src/cpu_simd.rs:175-200), at the
- * price of one pass over the weights per four rows (Q4_K, Q5_K and Q6_K: the products of four rows at a time go through the
+ * price of one pass over the weights per four rows (Q4_K, Q5_K, Q6_K and short-row Q8_0: the products of four rows at a time go through the
  * 4 x 4 x 4 int8 matrix instruction, three quarters of the time of two dot-product passes; other formats: two to four rows
  * a pass on the dot-product kernel).
  * fhip_weight_batch_policy sets one handle's policy and returns the one before; any value that is no policy only queries. Set it

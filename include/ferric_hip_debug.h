@@ -19,7 +19,7 @@ int fhip_debug_generic_matvec(int on);
  * launches; fhip_workspace_bytes_coop follows it. No counterpart in the reference. */
 int fhip_debug_gemm_tile(int tile);
 
-/* Debugging and tests: on == 0 keeps Q4_K / Q5_K / Q6_K batches of three and more rows off the kernel that multiplies on the
+/* Debugging and tests: on == 0 keeps Q4_K / Q5_K / Q6_K / Q8_0 batches of three and more rows off the kernel that multiplies on the
  * 4 x 4 x 4 int8 matrix instruction, so that the mat-vec entry points run them on the dot-product kernel two rows at a time
  * (the two give the same bits; the tests compare them this way). Returns the setting before the call (1 = on, the default).
  * Process-wide, not thread-safe against concurrent launches. No counterpart in the reference. */

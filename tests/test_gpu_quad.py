@@ -8,7 +8,7 @@ import pytest
 from conftest import bits, dot_bar
 
 pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("precision")]
-Q4_K, Q5_K, Q6_K = 12, 13, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 
 
 def both(F, fn):
@@ -29,7 +29,8 @@ def both(F, fn):
 SHAPES = [(Q4_K, 96, 5120), (Q4_K, 1023, 256), (Q4_K, 7, 2304), (Q4_K, 2050, 1024), (Q4_K, 300, 17408), (Q4_K, 5120, 5120),
           (Q6_K, 70, 2048), (Q6_K, 40, 17408), (Q6_K, 1, 256), (Q6_K, 1500, 2304), (Q6_K, 5120, 5120), (Q6_K, 515, 11264),
           (Q4_K, 37, 28672), (Q4_K, 12, 31488), (Q6_K, 9, 32768), (Q6_K, 261, 28672),
-          (Q5_K, 96, 5120), (Q5_K, 7, 2304), (Q5_K, 5120, 5120), (Q5_K, 130, 17408), (Q5_K, 1023, 256)]
+          (Q5_K, 96, 5120), (Q5_K, 7, 2304), (Q5_K, 5120, 5120), (Q5_K, 130, 17408), (Q5_K, 1023, 256),
+          (Q8_0, 4096, 4096), (Q8_0, 130, 1024), (Q8_0, 33, 96), (Q8_0, 12288, 4096), (Q8_0, 1000, 5120), (Q8_0, 77, 32)]
 
 
 @pytest.mark.parametrize("ty,rows,cols", SHAPES)
@@ -71,7 +72,7 @@ def test_fused_swiglu_same_bits(F, O, ty, n_ff, cols):
         assert np.array_equal(bits(on), bits(off)) and np.array_equal(bits(on), bits(singles[:m])), m
 
 
-@pytest.mark.parametrize("ty", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("ty", [Q8_0, Q4_K, Q5_K, Q6_K])
 def test_runs_block_fixed_point_cannot_hold(F, O, ty):
     """Non-finite activations and runs at the ends of the f32 range take the element-by-element pass: the same bits as on
     the dot-product kernel there too, NaN for NaN."""
