@@ -6,8 +6,8 @@
 // or 32 columns, two or three signed byte planes), exact integer dot products per run, the same f32 operations in the same
 // order above them, the same trees for the sums over a row's units. What differs is who multiplies. Here the integer
 // products go through v_mfma_i32_4x4x4_16b_i8: sixteen independent 4 x 4 x 4 products per wave. A wave's lane l = 4 u + r
-// holds unit u (64 weights; a block of 32 for Q8_0) of WEIGHT row r of a quad of four rows as the B operand (four bytes of it are four consecutive
-// columns: one column of B) and the planes of unit u of ACTIVATION row r as the A operand (one row of A). Block u of the
+// holds unit u (64 weights; a block of 32 for Q8_0) of WEIGHT row r of a quad of four rows as the B operand (four bytes of it
+// are four consecutive columns: one column of B) and the planes of unit u of ACTIVATION row r as the A operand (one row of A). Block u of the
 // instruction then gives all 16 (activation row, weight row) dot products of the unit's four columns, and lane 4 u + r ends
 // up with its own weight row's sums against the four activation rows in its four accumulator registers -- next to that
 // row's scales, which the same lane unpacked. No transposition, no LDS between the weight stream and the instruction: the
@@ -21,10 +21,11 @@
 // What it costs: a quad of rows x one group is 48 matrix instructions (32 with two planes) at 4.1 ns a SIMD, which do not
 // overlap with vector instructions of other waves on this chip (measured: 1 MFMA + 4 VALU = 9.4 ns, 4.1 + 4 x 1.35), beside
 // some 200 vector instructions: about 0.5 us a SIMD, and a CU's 170 of them on the fused gate|up weight 34816 x 5120 take
-// 23 us; the staging of four activation rows takes the first 5 us of the launch (one row: 2.3). Four rows: gate|up 33 us,
-// down 5120 x 17408 44 us at three planes (30 / 43 at two), against 20 / 17 for one row and 2 x 28 / 2 x 29 for four rows as
-// two passes of the dot-product kernel: this kernel serves the batches that are promised the mat-vec's bits, in three
-// quarters of the time; the one-pass f16 kernels (gemm_f16x2.hip) stay the faster way through a batch that is not.
+// 23 us; the staging of four activation rows takes the first 5 us of the launch (one row: 2.3). Four rows, cold, at three
+// planes (two): gate|up + SwiGLU 31 us (28), O 5120 x 5120 12.2 (10.8), down 5120 x 17408, two passes, 42 (39), against 20.1 /
+// 5.9 / 17.2 for one row and twice 28 / 8 / 29 for four rows as two passes of the dot-product kernel. Against the one-pass f16
+// kernels (gemm_f16x2.hip) with their split and sum launches it wins wherever it needs one pass and loses where it needs
+// two, which is how the entry points choose (api.hip).
 //
 // Built once per activation precision like gemv.hip (FHIP_GEMV_PLANES = 2 or 3).
 #include "common.hpp"
