@@ -702,9 +702,8 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
     u32x4 G[NW];
     constexpr int NTL = (32 * F::TAILS + 63) / 64;   // 2-byte tail pieces per lane
     uint32_t gt[NTL ? NTL : 1];
-    // requests the bytes of unit `v` = (128-row group, chunk); rows past the end of the weight repeat its last row
-    auto load_w = [&](long long v) {
-        const int grp = (int)(v / nchunks), ck = (int)(v - (long long)grp * nchunks);
+    // requests the bytes of unit (128-row group, chunk); rows past the end of the weight repeat its last row
+    auto load_w = [&](int grp, int ck) {
         const int row0 = grp * 128 + wave * 32 < p.N ? grp * 128 + wave * 32 : p.N - 1;
         const int rmax = p.N - 1 - row0;
         const uint8_t* b = p.W + (size_t)row0 * p.row_bytes;
@@ -741,18 +740,25 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
 
     // The workgroup's run of units is one stream: the chunk after a group's last is the next group's first, fetched and
     // parked like any other, so a run that crosses a group boundary pays no second start-up.
+    // (group, chunk) of the unit being worked on and of the next one to request: carried along by additions -- a 64-bit
+    // division per unit is some hundred scalar instructions, as many cycles of a wave as the unit's arithmetic
     const long long u_begin = u;
-    load_w(u);
-    load_x((int)(u % nchunks));
+    int grp = (int)(u / nchunks), ck = (int)(u - (long long)grp * nchunks);
+    int lgrp = grp, lck = ck;
+    auto request_next = [&]() {
+        load_w(lgrp, lck);
+        if (++lck == nchunks) { lck = 0; lgrp++; }
+    };
+    request_next();
+    load_x(ck);
     store_x(0);
     park_w();
-    if (u + 1 < u_end) load_w(u + 1);
+    if (u + 1 < u_end) request_next();
     __syncthreads();
 
     f32x4 total[2][NT];
     for (int it = 0; u < u_end; u++, it++) {
         const int buf = it & 1;
-        const int grp = (int)(u / nchunks), ck = (int)(u - (long long)grp * nchunks);
         const bool more = u + 1 < u_end;
         if (more) load_x(ck + 1 < nchunks ? ck + 1 : 0);
         if (u == u_begin || ck == 0) {
@@ -833,12 +839,13 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
         }
         if (more) {
             park_w();                             // unit u + 1 over unit u, which this wave has finished reading
-            if (u + 2 < u_end) load_w(u + 2);     // in flight through all of the next unit's arithmetic
+            if (u + 2 < u_end) request_next();    // in flight through all of the next unit's arithmetic
             store_x(buf ^ 1);
         }
         if (!more || ck == nchunks - 1) {
             // this group's share is complete: whole iff the run held all of its chunks
             const bool whole = (long long)grp * nchunks >= u_begin && (long long)(grp + 1) * nchunks <= u_end;
+            float* const slot0 = (!whole && p.part) ? part_slot(p, grp, 0, grp * 128) : nullptr;   // (one division, once per group share)
 #pragma unroll
             for (int s = 0; s < 2; s++)
 #pragma unroll
@@ -851,12 +858,13 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
                     if (g4 < 2 && t < p.T && n < p.N) {
                         float* y = p.Y + (size_t)t * p.N + n;
                         if (whole) *y = v;
-                        else if (p.part) *part_slot(p, grp, t, n) = v;
+                        else if (p.part) slot0[t * 128 + (n - grp * 128)] = v;
                         else unsafeAtomicAdd(y, v);
                     }
                 }
         }
         __syncthreads();
+        if (++ck == nchunks) { ck = 0; grp++; }
     }
 }
 
