@@ -641,6 +641,7 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
         // D layout of the 16x16 MFMA: register r of lane (g4, c) is operand row 4 g4 + r, column c. Operand rows 0..7
         // are the hi parts of activation rows 8 q + [0, 8), rows 8..15 their lo parts: lanes g4 and g4 ^ 2 hold the
         // two parts of the same output.
+        float* const slot0 = (!whole && p.part) ? part_slot(p, grp, 0, grp * 128) : nullptr;   // (its division once, not per store)
 #pragma unroll
         for (int s = 0; s < 2; s++)
 #pragma unroll
@@ -653,7 +654,7 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
                     if (g4 < 2 && t < p.T && n[s] < p.N) {
                         float* y = p.Y + (size_t)t * p.N + n[s];
                         if (whole) *y = v;
-                        else if (p.part) *part_slot(p, grp, t, n[s]) = v;
+                        else if (p.part) slot0[t * 128 + (n[s] - grp * 128)] = v;
                         else unsafeAtomicAdd(y, v);
                     }
                 }
