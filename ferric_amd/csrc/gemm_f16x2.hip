@@ -427,9 +427,17 @@ __device__ __forceinline__ float x_at(const float* __restrict__ x, int t, size_t
         const int first = holder_of((long long)grp * src.nchunks, src.grid, src.units);
         const int nk = holder_of((long long)(grp + 1) * src.nchunks - 1, src.grid, src.units) - first + 1;
         if (nk > 1) {
+            // (eight slots requested at a time: one trip to memory for the usual three or four contributors instead of one each)
             const float* q = src.part + ((size_t)grp * src.kmax * 32 + t) * 128 + (n & 127);
             float a = q[0];
-            for (int k = 1; k < nk; k++) a += q[(size_t)k * (32 * 128)];
+            for (int k0 = 1; k0 < nk; k0 += 8) {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = q[(size_t)(k0 + j < nk ? k0 + j : 0) * (32 * 128)];
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (k0 + j < nk) a += v[j];
+            }
             return a;
         }
     }
@@ -881,13 +889,14 @@ __global__ void __launch_bounds__(256) sum_split_kernel(float* __restrict__ Y, c
     if (n >= N || t >= T) return;
     const size_t slot = 32 * 128;
     const float* q = part + (size_t)grp * kmax * slot + t * 128 + col;
+    // (24 slots requested at a time: the down projection's 19 - 20 contributors in one trip to memory instead of three)
     float a = q[0];
-    for (int k0 = 1; k0 < nk; k0 += 8) {
-        float v[8];
+    for (int k0 = 1; k0 < nk; k0 += 24) {
+        float v[24];
 #pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = q[(size_t)(k0 + j < nk ? k0 + j : 0) * slot];
+        for (int j = 0; j < 24; j++) v[j] = q[(size_t)(k0 + j < nk ? k0 + j : 0) * slot];
 #pragma unroll
-        for (int j = 0; j < 8; j++)
+        for (int j = 0; j < 24; j++)
             if (k0 + j < nk) a += v[j];
     }
     Y[(size_t)t * N + n] = a;
