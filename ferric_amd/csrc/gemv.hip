@@ -835,8 +835,12 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
     const int my_unit = unit_ok ? group * 16 + l16 : 0;
     F::setup(my_unit, L, run);
 
-    const int rgid = blockIdx.x * p.G + rg;
     const bool dealt = F::RR && p.rr != 0;             // rows dealt round-robin in chunks of 4
+    // Dealt, the row groups are numbered across the workgroups (row group rg of workgroup b is number rg * row_wgs + b): the chunks
+    // of a last, partly filled round then go to the workgroups in turn. Numbered b * G + rg, the first workgroups got a chunk more
+    // in every one of their row groups and the last ones none (fused gate|up 34816 x 5120, two row groups a workgroup: 72 rows
+    // in workgroups 0 - 127, 64 in the others, whose row loops ended 1.3 us sooner).
+    const int rgid = dealt ? rg * p.row_wgs + (int)blockIdx.x : (int)blockIdx.x * p.G + rg;
     // Address of iteration `it`: a wave-uniform row base (scalar registers) plus a 32-bit lane offset. A tail
     // wave's lanes sit row_off rows further (v_start + it*v_step is a multiple of RT there, so with fused
     // SwiGLU the gate/up split of row_off is fixed); lanes past the last row read the uniform row instead
@@ -1114,7 +1118,7 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
             int r = row0 + rr;
             if (dealt) {                                 // local row -> (row group, row in it) -> row of the weight
                 const int g = (int)div_magic((uint32_t)rr, p.m_rpg), l = rr - g * p.rpg;
-                r = (((l >> 2) * p.nrg + blockIdx.x * p.G + g) << 2) + (l & 3);
+                r = (((l >> 2) * p.nrg + g * p.row_wgs + (int)blockIdx.x) << 2) + (l & 3);
                 if (r >= p.out_rows) continue;
             } else if (r >= p.out_rows) break;
             const float* q = part + ((size_t)rr * VPR * p.NG) * M + m;
