@@ -164,7 +164,7 @@ __device__ __forceinline__ float planes_f32(const int (&a)[NP]) {
 struct Q4K {
     static constexpr uint32_t TYPE = FHIP_Q4_K;
     static constexpr int WPL = 64, RUN = 32, NRUN = 2, U1 = 2;
-    static constexpr bool RR = true;      // round-robin row dealing of large weights
+    static constexpr bool RR = true, RR_ONE_ROW = true;      // round-robin row dealing of large weights
     struct Lane { uint32_t off_h, off_q, sh, m1, m2, m3; };
     struct Data {
         u32x4 h, q0, q1;
@@ -235,7 +235,9 @@ struct Q4K {
 struct Q6K {
     static constexpr uint32_t TYPE = FHIP_Q6_K;
     static constexpr int WPL = 64, RUN = 16, NRUN = 4, U1 = 2;
-    static constexpr bool RR = NP == 2;   // round-robin row dealing (with three planes its index arithmetic spills)
+    // round-robin row dealing: with three planes and two rows in flight its index arithmetic spills 8 registers (the vocabulary head
+    // 151936 x 5120 at 24 bits 118.7 -> 122.6 us dealt); with one row in flight it fits (down 5120 x 17408: 17.86 -> 17.39 us)
+    static constexpr bool RR = NP == 2, RR_ONE_ROW = true;
     struct Lane { uint32_t off_a, off_h, off_s, off_d, ssh; };
     struct Data {
         u32x4 a, b, h; u32x2 s; uint32_t d;
@@ -309,7 +311,7 @@ struct Q6K {
 struct Q80 {
     static constexpr uint32_t TYPE = FHIP_Q8_0;
     static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 2;   // two rows in flight: 4096 x 4096 6.89 -> 6.57 us against four
-    static constexpr bool RR = true;      // round-robin row dealing of large weights
+    static constexpr bool RR = true, RR_ONE_ROW = true;      // round-robin row dealing of large weights
     struct Lane { uint32_t off; };
     struct Data {
         u32x4 q0, q1; uint32_t d;
@@ -356,7 +358,7 @@ struct Q80 {
 struct Q5K {
     static constexpr uint32_t TYPE = FHIP_Q5_K;
     static constexpr int WPL = 64, RUN = 32, NRUN = 2, U1 = 2;
-    static constexpr bool RR = NP == 2;   // (three planes: the index arithmetic spills)
+    static constexpr bool RR = NP == 2, RR_ONE_ROW = NP == 2;   // (three planes: the index arithmetic spills)
     struct Lane { uint32_t off_h, off_q, sh, g2, m1, m2, m3; };
     struct Data {
         u32x4 h, b0, b1, q0, q1;
@@ -429,7 +431,7 @@ template <uint32_t TY, int BYTES, bool HAS_M, bool HAS_QH, int OFF>
 struct LegS {
     static constexpr uint32_t TYPE = TY;
     static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
-    static constexpr bool RR = true;      // round-robin row dealing of large weights
+    static constexpr bool RR = true, RR_ONE_ROW = true;      // round-robin row dealing of large weights
     static constexpr int QH = HAS_M ? 4 : 2, QS = QH + (HAS_QH ? 4 : 0);
     struct Lane { uint32_t off; };
     struct Data {
@@ -499,7 +501,7 @@ template <bool XS>
 struct IQ4S {
     static constexpr uint32_t TYPE = XS ? FHIP_IQ4_XS : FHIP_IQ4_NL;
     static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
-    static constexpr bool RR = true;      // round-robin row dealing of large weights
+    static constexpr bool RR = true, RR_ONE_ROW = true;      // round-robin row dealing of large weights
     struct Lane { uint32_t off_h, off_q, ib; };
     struct Data {
         u32x4 q; uint32_t h0, h1;
@@ -566,7 +568,7 @@ struct __attribute__((packed, aligned(1))) U4A1 { u32x4 v; };
 struct MXF4S {
     static constexpr uint32_t TYPE = FHIP_MXFP4;
     static constexpr int WPL = 32, RUN = 32, NRUN = 1, U1 = 4;
-    static constexpr bool RR = true;      // round-robin row dealing of large weights
+    static constexpr bool RR = true, RR_ONE_ROW = true;      // round-robin row dealing of large weights
     struct Lane { uint32_t off; };
     struct Data {
         u32x4 q; uint32_t e;
@@ -835,7 +837,7 @@ __global__ void __launch_bounds__(max_threads<F>(M)) gemv_stream_kernel(GemvPara
     const int my_unit = unit_ok ? group * 16 + l16 : 0;
     F::setup(my_unit, L, run);
 
-    const bool dealt = F::RR && p.rr != 0;             // rows dealt round-robin in chunks of 4
+    const bool dealt = (F::RR || (F::RR_ONE_ROW && U == 1)) && p.rr != 0;   // rows dealt round-robin in chunks of 4
     // Dealt, the row groups are numbered across the workgroups (row group rg of workgroup b is number rg * row_wgs + b): the chunks
     // of a last, partly filled round then go to the workgroups in turn. Numbered b * G + rg, the first workgroups got a chunk more
     // in every one of their row groups and the last ones none (fused gate|up 34816 x 5120, two row groups a workgroup: 72 rows
@@ -1268,7 +1270,7 @@ int launch_one_u(const fhip_weight* w, const float* d_x, float* d_y, size_t out_
     // all CUs (one CU is left to the workgroup that stores x + resid when the fused norm asks for that).
     p.rr = 0; p.nrg = 0; p.kfull = 0; p.rem = 0;
     const bool spare = norm && norm->x_out && cus > 1;
-    if (F::RR && rpg >= 16 && rounds == 1 && p.sel.npairs <= 1) {
+    if ((F::RR || (F::RR_ONE_ROW && U == 1)) && rpg >= 16 && rounds == 1 && p.sel.npairs <= 1) {
         const size_t nrg_all = (size_t)(cus - (spare ? 1 : 0)) * G, S = nrg_all * 4;
         const size_t kfull = out_rows / S, rem = out_rows % S;
         const size_t rr_rpg = (kfull + (rem ? 1 : 0)) * 4;
