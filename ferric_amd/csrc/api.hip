@@ -668,7 +668,7 @@ int fhip_ffn(const fhip_weight* gu, const fhip_weight* down, const float* d_x, s
                 rc = f16x2_matmul(down, g, t, false, d_y + m0 * down->rows, ws2, s);
         } else {
             // under the ordered policy gate|up's K-split groups stay partial sums; the split for the down projection adds them
-            fhip::F16Parts parts{nullptr, 0, 0, 0, 0};
+            fhip::F16Parts parts{nullptr, 0, 0, 0, 0, 128};
             if (!(rc = f16x2_matmul(gu, d_x + m0 * gu->cols, t, false, g, ws, s, &parts)))
                 rc = f16x2_matmul(down, g, t, true, d_y + m0 * down->rows, ws2, s, nullptr, &parts);
         }

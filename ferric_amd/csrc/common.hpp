@@ -139,6 +139,7 @@ struct F16Parts {
     const float* part;    // null: every output is in y
     int kmax, nchunks, grid;
     long long units;
+    int group;            // outputs of a group: 128, or 256 where the eight-wave row-streaming kernel made the sums
 };
 // src: x is the output of a matmul whose ordered sum was left to this launch (launch_gemm_f16x2 with `deferred`)
 int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero = nullptr,

@@ -26,8 +26,8 @@
 //     order the nibbles come out (xsplit_f16_kernel does that once per call).
 //
 // Lane (g4 = lane / 16, c = lane % 16) of a wave works on weight row c of a 16-row set and on k-group g4 of each
-// 32-wide MFMA slice; a wave carries two row sets (32 weight rows), a workgroup four waves (128 rows). The
-// (128-row group, 256-column chunk) units are dealt to the workgroups in equal contiguous runs; a run that covers its
+// 32-wide MFMA slice; a wave carries two row sets (32 weight rows), a workgroup four waves (128 rows; the row-streaming
+// kernel for up to 8 activation rows: eight waves, 256 rows). The (row group, 256-column chunk) units are dealt to the workgroups in equal contiguous runs; a run that covers its
 // group's whole K stores, any other adds atomically into a Y cleared beforehand (or, when the caller asks for ordered sums, stores
 // into a slot of its own that sum_split_kernel adds in contributor order).
 #include "common.hpp"
@@ -118,7 +118,7 @@ struct Q4K {
     }
     static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) { h.hd = *(const u32x4*)(row + (size_t)c * BLOCK); }
     // row-streaming kernel: a block is PARTS 16-byte pieces in global memory and a row of LROW bytes in the wave's LDS image
-    static constexpr int PARTS = 9, LROW = 144, TAILS = 0, ROWS_OCCUPANCY = 3;   // 120 VGPRs, 36 KB of LDS (four per CU ran slower: 36.7 vs 34.0 us)
+    static constexpr int PARTS = 9, LROW = 144, TAILS = 0, ROWS_OCCUPANCY = 3;   // (workgroups of the four-wave row-streaming kernel per CU)
     static constexpr bool ROWS_AT_16 = false;   // 9..16 rows, cold weights: 44.9 us against 42.0 us for the one-row-per-lane kernel
     static constexpr bool ROW_PER_LANE = true, SLICE_SCALE = false;
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return *(const u32x4*)p; }
@@ -202,7 +202,7 @@ struct Q5K {
         r.q1 = *(const u32x4*)(blk + 64 + 32 * g4);
     }
     static __device__ __forceinline__ void head(Head& h, const uint8_t* row, int c) { h.hd = *(const u32x4*)(row + (size_t)c * BLOCK); }
-    static constexpr int PARTS = 11, LROW = 176, TAILS = 0, ROWS_OCCUPANCY = 3;   // 40 KB of LDS a workgroup
+    static constexpr int PARTS = 11, LROW = 176, TAILS = 0, ROWS_OCCUPANCY = 3;   // (workgroups of the four-wave row-streaming kernel per CU)
     static constexpr bool ROWS_AT_16 = false;
     static constexpr bool ROW_PER_LANE = true, SLICE_SCALE = false;
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return *(const u32x4*)p; }
@@ -285,7 +285,7 @@ struct Q6K {
     // row-streaming kernel: 13 16-byte pieces + the 2-byte d; LDS rows of 240 bytes (a multiple of 16 whose dword count,
     // 60, puts the 16 rows of a read instruction into different banks). Contiguous lanes read contiguous bytes here, which
     // the 2-byte alignment of the blocks does not slow down.
-    static constexpr int PARTS = 13, LROW = 240, TAILS = 1, ROWS_OCCUPANCY = 3;   // 134 VGPRs, 49 KB of LDS
+    static constexpr int PARTS = 13, LROW = 240, TAILS = 1, ROWS_OCCUPANCY = 3;   // (workgroups of the four-wave row-streaming kernel per CU)
     static constexpr bool ROWS_AT_16 = true;    // 9..16 rows, cold weights: 33.2 us against 41.2 us
     static constexpr bool ROW_PER_LANE = true, SLICE_SCALE = false;
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return ((const U4A2*)p)->v; }
@@ -368,7 +368,7 @@ struct Q80 {
     static __host__ __device__ constexpr int occupancy(int) { return 2; }
     static __host__ __device__ constexpr int src_k(int pos) { return pos; }   // slice I is block I, in order
     static __host__ __device__ constexpr int pos_of(int k) { return k; }
-    static constexpr int PARTS = 16, LROW = 272, TAILS = 8, ROWS_OCCUPANCY = 3;
+    static constexpr int PARTS = 16, LROW = 272, TAILS = 8, ROWS_OCCUPANCY = 3;   // (workgroups of the four-wave row-streaming kernel per CU)
     static constexpr bool ROWS_AT_16 = true;
     static constexpr bool ROW_PER_LANE = false, SLICE_SCALE = true;
     static __device__ __forceinline__ u32x4 ldg(const uint8_t* p) { return ((const U4A2*)p)->v; }
@@ -423,17 +423,18 @@ __device__ __host__ __forceinline__ int holder_of(long long u, long long G, long
 // partial sums to this launch, slot 0 + slot 1 + ... of that group (the order sum_split_kernel adds them in)
 __device__ __forceinline__ float x_at(const float* __restrict__ x, int t, size_t n, const fhip::F16Parts& src) {
     if (src.part) {
-        const int grp = (int)(n >> 7);
+        const int gsh = src.group == 256 ? 8 : 7;   // (groups of 128 or 256 outputs)
+        const int grp = (int)(n >> gsh);
         const int first = holder_of((long long)grp * src.nchunks, src.grid, src.units);
         const int nk = holder_of((long long)(grp + 1) * src.nchunks - 1, src.grid, src.units) - first + 1;
         if (nk > 1) {
             // (eight slots requested at a time: one trip to memory for the usual three or four contributors instead of one each)
-            const float* q = src.part + ((size_t)grp * src.kmax * 32 + t) * 128 + (n & 127);
+            const float* q = src.part + ((size_t)grp * src.kmax * 32 + t) * src.group + (n & (size_t)(src.group - 1));
             float a = q[0];
             for (int k0 = 1; k0 < nk; k0 += 8) {
                 float v[8];
 #pragma unroll
-                for (int j = 0; j < 8; j++) v[j] = q[(size_t)(k0 + j < nk ? k0 + j : 0) * (32 * 128)];
+                for (int j = 0; j < 8; j++) v[j] = q[(size_t)(k0 + j < nk ? k0 + j : 0) * (32 * (size_t)src.group)];
 #pragma unroll
                 for (int j = 0; j < 8; j++)
                     if (k0 + j < nk) a += v[j];
@@ -512,16 +513,17 @@ struct F16Params {
     int T, N, nchunks;
     int nblk;             // Q8_0: blocks in a weight row (the last chunk may hold fewer than 8)
     size_t row_bytes;
-    long long units;      // 128-row groups * nchunks, chunk fastest
+    long long units;      // row groups * nchunks, chunk fastest
+    int group;            // rows of a group: 128, or 256 for the eight-wave row-streaming kernel
     float* part;          // null: a run that holds part of a group's K adds into Y atomically. Else it stores its partial sums
-                          // into slot (group, contributor) of [groups][kmax][32][128] floats, and sum_split_kernel adds them in order
+                          // into slot (group, contributor) of [groups][kmax][32][group] floats, and sum_split_kernel adds them in order
     int kmax;
 };
 
 // where a partial output (activation row t, output n of group grp) goes in ordered mode
 __device__ __forceinline__ float* part_slot(const F16Params& p, int grp, int t, int n) {
     const int k = (int)blockIdx.x - holder_of((long long)grp * p.nchunks, gridDim.x, p.units);
-    return p.part + (((size_t)grp * p.kmax + k) * 32 + t) * 128 + (n - grp * 128);
+    return p.part + (((size_t)grp * p.kmax + k) * 32 + t) * p.group + (n - grp * p.group);
 }
 
 template <class F, int NT>
@@ -649,7 +651,7 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
         // D layout of the 16x16 MFMA: register r of lane (g4, c) is operand row 4 g4 + r, column c. Operand rows 0..7
         // are the hi parts of activation rows 8 q + [0, 8), rows 8..15 their lo parts: lanes g4 and g4 ^ 2 hold the
         // two parts of the same output.
-        float* const slot0 = (!whole && p.part) ? part_slot(p, grp, 0, grp * 128) : nullptr;   // (its division once, not per store)
+        float* const slot0 = (!whole && p.part) ? part_slot(p, grp, 0, grp * 128) : nullptr;   // (its division once, not per store; p.group = 128 here)
 #pragma unroll
         for (int s = 0; s < 2; s++)
 #pragma unroll
@@ -678,12 +680,20 @@ __global__ void __launch_bounds__(256, F::occupancy(NT)) gemm_q_f16x2_kernel(F16
 // on bytes it has not seen) this takes 34 us for a 34816 x 5120 Q4_K weight and 27 us for 5120 x 17408 Q6_K, the kernel
 // above 39 and 35.5 us: its one-row-per-lane loads ask for every cache line two or three times, 16 bytes at a time.
 // ------------------------------------------------------------------------------------------------
-template <class F, int NT>
-__global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f16x2_rows_kernel(F16Params p) {
-    constexpr int PIECES = 16 * NT * XR / 8, NP = (PIECES + 255) / 256;
+template <class F, int NT, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : (NT == 1 ? F::ROWS_OCCUPANCY : 2)) gemm_q_f16x2_rows_kernel(F16Params p) {
+    // WAVES = 8 (up to 8 activation rows on the large K-split weights of the FFN block): ONE workgroup of eight waves (256 weight
+    // rows) per CU. Three workgroups of four waves, each with its own staged activations, ended far apart -- the younger a workgroup on its CU the later (ends of the first / second / third
+    // a CU received 24.2 / 26.0 / 28.8 us on the fused gate|up weight, 17.5 / 21.3 / 24.3 on the down projection), the last
+    // one at 32.5 / 27.6 us; eight waves of one age share one staging and one barrier: whole calls 37.4 -> 35.2 and 31.6 -> 30.0 us
+    // (twelve waves 35.7 - 36.8 / 30.7, ten 36.4 / 31.2, six 45.3 / 32.0, two workgroups of eight 36.2 / 35.0, of six 37.9 / 35.1).
+    // Small weights and weights whose groups are not cut along K keep the four-wave workgroups (at 8 rows, ordered sums, eight waves
+    // against four: 4096 x 4096 14.6 against 14.0 us, Q8_0 12288 x 4096 29.0 / 26.6, the vocabulary head 199 / 177).
+    constexpr int NTHR = 64 * WAVES, GROUP = 32 * WAVES;
+    constexpr int PIECES = 16 * NT * XR / 8, NP = (PIECES + NTHR - 1) / NTHR;
     constexpr int WP = 32 * F::PARTS, NW = (WP + 63) / 64;
     __shared__ __attribute__((aligned(16))) uint16_t Xs[2][16 * NT * XR];
-    __shared__ __attribute__((aligned(16))) uint8_t Wl[4][32 * F::LROW];
+    __shared__ __attribute__((aligned(16))) uint8_t Wl[WAVES][32 * F::LROW];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g4 = lane >> 4, c = lane & 15;
     const int nchunks = p.nchunks;
@@ -696,12 +706,12 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
         const u32x4* src = (const u32x4*)(p.Xp + (size_t)ck * 16 * NT * XR);
 #pragma unroll
         for (int q = 0; q < NP; q++)
-            if (tid + 256 * q < PIECES) stage[q] = src[tid + 256 * q];
+            if (tid + NTHR * q < PIECES) stage[q] = src[tid + NTHR * q];
     };
     auto store_x = [&](int buf) {
 #pragma unroll
         for (int q = 0; q < NP; q++)
-            if (tid + 256 * q < PIECES) ((u32x4*)Xs[buf])[tid + 256 * q] = stage[q];
+            if (tid + NTHR * q < PIECES) ((u32x4*)Xs[buf])[tid + NTHR * q] = stage[q];
     };
     const int a_rd = c * XR + 8 * g4;
     const int m_rd = c * XR + CHUNK + (g4 ? 8 : 0);
@@ -711,9 +721,9 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
     u32x4 G[NW];
     constexpr int NTL = (32 * F::TAILS + 63) / 64;   // 2-byte tail pieces per lane
     uint32_t gt[NTL ? NTL : 1];
-    // requests the bytes of unit (128-row group, chunk); rows past the end of the weight repeat its last row
+    // requests the bytes of unit (row group, chunk); rows past the end of the weight repeat its last row
     auto load_w = [&](int grp, int ck) {
-        const int row0 = grp * 128 + wave * 32 < p.N ? grp * 128 + wave * 32 : p.N - 1;
+        const int row0 = grp * GROUP + wave * 32 < p.N ? grp * GROUP + wave * 32 : p.N - 1;
         const int rmax = p.N - 1 - row0;
         const uint8_t* b = p.W + (size_t)row0 * p.row_bytes;
 #pragma unroll
@@ -854,20 +864,20 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
         if (!more || ck == nchunks - 1) {
             // this group's share is complete: whole iff the run held all of its chunks
             const bool whole = (long long)grp * nchunks >= u_begin && (long long)(grp + 1) * nchunks <= u_end;
-            float* const slot0 = (!whole && p.part) ? part_slot(p, grp, 0, grp * 128) : nullptr;   // (one division, once per group share)
+            float* const slot0 = (!whole && p.part) ? part_slot(p, grp, 0, grp * GROUP) : nullptr;   // (one division, once per group share)
 #pragma unroll
             for (int s = 0; s < 2; s++)
 #pragma unroll
               for (int q = 0; q < NT; q++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    const int t = 8 * q + 4 * (g4 & 1) + r, n = grp * 128 + wave * 32 + 16 * s + c;
+                    const int t = 8 * q + 4 * (g4 & 1) + r, n = grp * GROUP + wave * 32 + 16 * s + c;
                     float v = total[s][q][r];
                     v += __shfl_xor(v, 32);
                     if (g4 < 2 && t < p.T && n < p.N) {
                         float* y = p.Y + (size_t)t * p.N + n;
                         if (whole) *y = v;
-                        else if (p.part) slot0[t * 128 + (n - grp * 128)] = v;
+                        else if (p.part) slot0[t * GROUP + (n - grp * GROUP)] = v;
                         else unsafeAtomicAdd(y, v);
                     }
                 }
@@ -877,18 +887,18 @@ __global__ void __launch_bounds__(256, NT == 1 ? F::ROWS_OCCUPANCY : 2) gemm_q_f
     }
 }
 
-// Ordered mode: group `blockIdx.x` of 128 outputs, if more than one workgroup held part of its K: Y = slot 0 + slot 1 + ...
+// Ordered mode: group `blockIdx.x` of `group` (128 or 256) outputs, if more than one workgroup held part of its K: Y = slot 0 + slot 1 + ...
 // in that order. Thread = output column (threadIdx.x & 127) of activation row 2 * blockIdx.y + (threadIdx.x >> 7).
 __global__ void __launch_bounds__(256) sum_split_kernel(float* __restrict__ Y, const float* __restrict__ part, int T, int N, int nchunks,
-                                                      long long units, int grid, int kmax) {
+                                                      long long units, int grid, int kmax, int group) {
     const int grp = blockIdx.x;
     const int first = holder_of((long long)grp * nchunks, grid, units), last = holder_of((long long)(grp + 1) * nchunks - 1, grid, units);
     const int nk = last - first + 1;
     if (nk == 1) return;
-    const int col = threadIdx.x & 127, n = grp * 128 + col, t = 2 * blockIdx.y + (threadIdx.x >> 7);
+    const int per = 256 / group, trow = (int)threadIdx.x / group, col = (int)threadIdx.x - trow * group, n = grp * group + col, t = per * blockIdx.y + trow;
     if (n >= N || t >= T) return;
-    const size_t slot = 32 * 128;
-    const float* q = part + (size_t)grp * kmax * slot + t * 128 + col;
+    const size_t slot = 32 * (size_t)group;
+    const float* q = part + (size_t)grp * kmax * slot + t * group + col;
     // (24 slots requested at a time: the down projection's 19 - 20 contributors in one trip to memory instead of three)
     float a = q[0];
     for (int k0 = 1; k0 < nk; k0 += 24) {
@@ -913,6 +923,7 @@ struct Plan {
     unsigned grid;
     bool split;
     int kmax;             // most workgroups that hold part of one group's K
+    int group;            // rows of a group: 256 for up to 8 activation rows (the eight-wave kernel), else 128
 };
 
 // workgroups of the kernel that serves `nt` operand row sets that fit on a CU together
@@ -923,10 +934,17 @@ Plan make_plan(const fhip_weight* w, size_t t) {
     Plan q;
     q.nt = t <= 8 ? 1 : (t <= 16 ? 2 : 4);
     q.nchunks = (int)((w->cols + CHUNK - 1) / CHUNK);
-    const long long groups = ((long long)w->rows + 127) / 128;
-    q.units = groups * q.nchunks;
     const long long cus = fhip::device_cus() > 0 ? fhip::device_cus() : 256;
-    const long long wgs = cus * (w->type == FHIP_Q6_K ? slots<Q6K>(q.nt) : w->type == FHIP_Q8_0 ? slots<Q80>(q.nt) :
+    // the eight-wave kernel (groups of 256 rows, one workgroup per CU): up to 8 rows on a K-quant weight of 48 MB and more whose
+    // groups it cuts along K with every CU holding one share
+    q.group = 128;
+    if (q.nt == 1 && (w->type == FHIP_Q4_K || w->type == FHIP_Q5_K || w->type == FHIP_Q6_K) && w->nbytes >= ((size_t)48 << 20)) {
+        const long long g8 = ((long long)w->rows + 255) / 256, u8 = g8 * q.nchunks, per8 = (u8 + cus - 1) / cus;
+        if (u8 >= cus && per8 * 4 < (long long)q.nchunks * 3) q.group = 256;
+    }
+    const long long groups = ((long long)w->rows + q.group - 1) / q.group;
+    q.units = groups * q.nchunks;
+    const long long wgs = q.group == 256 ? cus : cus * (w->type == FHIP_Q6_K ? slots<Q6K>(q.nt) : w->type == FHIP_Q8_0 ? slots<Q80>(q.nt) :
                                  w->type == FHIP_Q5_K ? slots<Q5K>(q.nt) : slots<Q4K>(q.nt));
     // one workgroup per resident slot, each with the same share of the units (a grid of 2.66 workgroups per CU leaves
     // two thirds of the CUs with half as much again to do as the rest); shares of three quarters of a group's chunks or
@@ -961,23 +979,25 @@ int launch_fmt(const fhip_weight* w, const uint16_t* d_xp, size_t t, float* d_y,
     p.part = q.split ? d_part : nullptr; p.kmax = q.kmax;
     p.T = (int)t; p.N = (int)w->rows; p.nchunks = q.nchunks; p.row_bytes = w->row_bytes;
     p.nblk = (int)(w->cols / 32);
-    p.units = q.units;
+    p.units = q.units; p.group = q.group;
     if (q.split && !y_cleared && !d_part) {
         const size_t n = t * w->rows;
         hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, d_y, n);
     }
-    if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 1>), dim3(q.grid), dim3(256), 0, s, p);
-    else if (q.nt == 2 && F::ROWS_AT_16) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
+    if (q.nt == 1 && q.group == 256) {
+        if constexpr (F::ROW_PER_LANE) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 1, 8>), dim3(q.grid), dim3(512), 0, s, p);
+    } else if (q.nt == 1) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 1, 4>), dim3(q.grid), dim3(256), 0, s, p);
+    else if (q.nt == 2 && F::ROWS_AT_16) hipLaunchKernelGGL((gemm_q_f16x2_rows_kernel<F, 2, 4>), dim3(q.grid), dim3(256), 0, s, p);
     else if constexpr (F::ROW_PER_LANE) {
         if (q.nt == 2) hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 2>), dim3(q.grid), dim3(256), 0, s, p);
         else hipLaunchKernelGGL((gemm_q_f16x2_kernel<F, 4>), dim3(q.grid), dim3(256), 0, s, p);
     } else {
         return fhip::set_error(FHIP_ERR_SHAPE, "f16x2 matmul: this format takes at most 16 activation rows, got %zu", t);
     }
-    if (deferred) *deferred = fhip::F16Parts{p.part, p.kmax, p.nchunks, (int)q.grid, p.units};
+    if (deferred) *deferred = fhip::F16Parts{p.part, p.kmax, p.nchunks, (int)q.grid, p.units, q.group};
     if (p.part && !deferred)
-        hipLaunchKernelGGL(sum_split_kernel, dim3((unsigned)q.groups, (unsigned)((t + 1) / 2)), dim3(256), 0, s, d_y, (const float*)d_part, p.T, p.N,
-                           p.nchunks, p.units, (int)q.grid, p.kmax);
+        hipLaunchKernelGGL(sum_split_kernel, dim3((unsigned)q.groups, (unsigned)((t * q.group + 255) / 256)), dim3(256), 0, s, d_y, (const float*)d_part, p.T, p.N,
+                           p.nchunks, p.units, (int)q.grid, p.kmax, q.group);
     return fhip::check_hip(hipGetLastError(), "gemm_q_f16x2 launch");
 }
 
@@ -1000,7 +1020,7 @@ bool gemm_f16x2_adds_into_y(const fhip_weight* w, size_t t) { return make_plan(w
 
 size_t gemm_f16x2_part_bytes(const fhip_weight* w, size_t t) {
     const Plan q = make_plan(w, t);
-    return q.split ? (size_t)q.groups * q.kmax * 32 * 128 * sizeof(float) : 0;
+    return q.split ? (size_t)q.groups * q.kmax * 32 * q.group * sizeof(float) : 0;
 }
 // the most any batch of up to t rows needs (fewer rows can mean more resident workgroups, and so more contributors)
 size_t gemm_f16x2_part_bytes_upto(const fhip_weight* w, size_t t) {
@@ -1013,7 +1033,7 @@ size_t gemm_f16x2_part_bytes_upto(const fhip_weight* w, size_t t) {
 int launch_xsplit_f16(const fhip_weight* w, const float* d_x, size_t t, bool swiglu, uint16_t* d_xp, hipStream_t s, float* zero, size_t zero_n,
                       const F16Parts* src_in) {
     const Plan q = make_plan(w, t);
-    const F16Parts src = src_in ? *src_in : F16Parts{nullptr, 0, 0, 0, 0};
+    const F16Parts src = src_in ? *src_in : F16Parts{nullptr, 0, 0, 0, 0, 128};
     switch (w->type) {
         case FHIP_Q4_K: return launch_xsplit_fmt<Q4K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n, src);
         case FHIP_Q5_K: return launch_xsplit_fmt<Q5K>(d_x, t, w->cols, swiglu, q, d_xp, s, zero, zero_n, src);
